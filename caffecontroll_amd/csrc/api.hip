@@ -1,0 +1,168 @@
+// Process state, memory management and timing entry points of the driver library.
+#include <cstdarg>
+#include <cstring>
+#include <mutex>
+
+#include "cct_common.h"
+
+namespace cct {
+
+static Context g_ctx;
+static std::mutex g_mu;
+static thread_local char g_err[512] = "";
+
+Context &ctx() { return g_ctx; }
+
+int set_error(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static int init_locked(int device_id) {
+  int count = 0;
+  CCT_HIP_CHECK(hipGetDeviceCount(&count));
+  CCT_REQUIRE(device_id >= 0 && device_id < count, "device %d not present (%d devices)", device_id,
+              count);
+  CCT_HIP_CHECK(hipSetDevice(device_id));
+  if (g_ctx.device != device_id) {
+    hipDeviceProp_t prop;
+    CCT_HIP_CHECK(hipGetDeviceProperties(&prop, device_id));
+    CCT_REQUIRE(strncmp(prop.gcnArchName, "gfx950", 6) == 0,
+                "this library holds gfx950 code only; device %d is %s", device_id, prop.gcnArchName);
+    g_ctx.device = device_id;
+    g_ctx.compute_units = prop.multiProcessorCount;
+    g_ctx.workspace = nullptr;
+    g_ctx.workspace_bytes = 0;
+  }
+  return 0;
+}
+
+// Called at the top of every entry point: the reference creates a fresh std::thread per
+// forward/backward call (src/bridges/PhysicalStratum.h:52-64), so the device must be
+// re-selected on whichever thread arrives.
+int ensure_init() {
+  if (g_ctx.device < 0) {
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (g_ctx.device < 0) return init_locked(0);
+    return 0;
+  }
+  CCT_HIP_CHECK(hipSetDevice(g_ctx.device));
+  return 0;
+}
+
+int get_workspace(size_t bytes, void **out) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (bytes > g_ctx.workspace_bytes) {
+    if (g_ctx.workspace) {
+      CCT_HIP_CHECK(hipStreamSynchronize(g_ctx.stream));
+      CCT_HIP_CHECK(hipFree(g_ctx.workspace));
+      g_ctx.workspace = nullptr;
+      g_ctx.workspace_bytes = 0;
+    }
+    const size_t want = (bytes + (1u << 20) - 1) & ~(size_t)((1u << 20) - 1);
+    CCT_HIP_CHECK(hipMalloc(&g_ctx.workspace, want));
+    g_ctx.workspace_bytes = want;
+  }
+  *out = g_ctx.workspace;
+  return 0;
+}
+
+struct Timer {
+  hipEvent_t start, stop;
+};
+
+}  // namespace cct
+
+using namespace cct;
+
+extern "C" {
+
+int cct_hip_init(int device_id) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  return init_locked(device_id);
+}
+
+int cct_hip_set_stream(void *hip_stream) {
+  CCT_ENSURE_INIT();
+  ctx().stream = (hipStream_t)hip_stream;
+  return 0;
+}
+
+int cct_hip_device_sync(void) {
+  CCT_ENSURE_INIT();
+  CCT_HIP_CHECK(hipStreamSynchronize(ctx().stream));
+  return 0;
+}
+
+const char *cct_hip_last_error(void) { return g_err; }
+
+int cct_hip_compute_units(void) { return ctx().compute_units; }
+
+int cct_hip_malloc(void **dev_ptr, size_t size_in_byte) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(dev_ptr != nullptr, "malloc: null result pointer");
+  *dev_ptr = nullptr;
+  if (size_in_byte == 0) return 0;
+  CCT_HIP_CHECK(hipMalloc(dev_ptr, size_in_byte));
+  return 0;
+}
+
+int cct_hip_free(void *dev_ptr) {
+  CCT_ENSURE_INIT();
+  if (dev_ptr) CCT_HIP_CHECK(hipFree(dev_ptr));
+  return 0;
+}
+
+int cct_hip_memcpy(void *dst, const void *src, size_t size_in_byte, int kind) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(kind >= 0 && kind <= 2, "memcpy: kind %d not in {0,1,2}", kind);
+  if (size_in_byte == 0) return 0;
+  const hipMemcpyKind k =
+      kind == 0 ? hipMemcpyHostToDevice : kind == 1 ? hipMemcpyDeviceToHost : hipMemcpyDeviceToDevice;
+  CCT_HIP_CHECK(hipMemcpyAsync(dst, src, size_in_byte, k, ctx().stream));
+  if (kind != 2) CCT_HIP_CHECK(hipStreamSynchronize(ctx().stream));
+  return 0;
+}
+
+int cct_hip_timer_create(void **timer) {
+  CCT_ENSURE_INIT();
+  Timer *t = new Timer;
+  CCT_HIP_CHECK(hipEventCreate(&t->start));
+  CCT_HIP_CHECK(hipEventCreate(&t->stop));
+  *timer = t;
+  return 0;
+}
+
+int cct_hip_timer_destroy(void *timer) {
+  Timer *t = (Timer *)timer;
+  if (!t) return 0;
+  (void)hipEventDestroy(t->start);
+  (void)hipEventDestroy(t->stop);
+  delete t;
+  return 0;
+}
+
+int cct_hip_timer_start(void *timer) {
+  CCT_ENSURE_INIT();
+  CCT_HIP_CHECK(hipEventRecord(((Timer *)timer)->start, ctx().stream));
+  return 0;
+}
+
+int cct_hip_timer_stop(void *timer) {
+  CCT_ENSURE_INIT();
+  CCT_HIP_CHECK(hipEventRecord(((Timer *)timer)->stop, ctx().stream));
+  return 0;
+}
+
+int cct_hip_timer_elapsed_ms(void *timer, float *ms) {
+  CCT_ENSURE_INIT();
+  Timer *t = (Timer *)timer;
+  CCT_HIP_CHECK(hipEventSynchronize(t->stop));
+  CCT_HIP_CHECK(hipEventElapsedTime(ms, t->start, t->stop));
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,631 @@
+// HBM-bound helper kernels of the driver: slice remap, bias add, ReLU, max pooling, LRN, dropout,
+// softmax loss, BLAS-1 / SGD update, fills and gemv.  One pass over the data each; 16-byte
+// vector accesses where the element count and alignment allow it.
+#include <cfloat>
+#include <cstring>
+
+#include "cct_common.h"
+
+namespace cct {
+
+constexpr int TPB = 256;
+
+static inline uint32_t blocks_for(size_t n, int per_block = TPB) {
+  return (uint32_t)((n + per_block - 1) / per_block);
+}
+
+__device__ __forceinline__ float wave_sum_f(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max_f(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_down(v, off, 64));
+  return v;
+}
+
+// Reduction of one value per lane over a 256-lane workgroup; result valid on every lane.
+template <bool MAX>
+__device__ __forceinline__ float block_reduce(float v, float *scratch /* >= 5 floats */) {
+  v = MAX ? wave_max_f(v) : wave_sum_f(v);
+  const int tid = threadIdx.x;
+  __syncthreads();
+  if ((tid & 63) == 0) scratch[tid >> 6] = v;
+  __syncthreads();
+  if (tid == 0) {
+    float t = scratch[0];
+    for (int w = 1; w < TPB / 64; ++w) t = MAX ? fmaxf(t, scratch[w]) : t + scratch[w];
+    scratch[4] = t;
+  }
+  __syncthreads();
+  return scratch[4];
+}
+
+// ---- fills --------------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void fill_f32_kernel(float *__restrict__ p, size_t n, float v) {
+  const size_t stride = (size_t)gridDim.x * TPB;
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+__global__ __launch_bounds__(TPB) void fill_u8_kernel(unsigned char *__restrict__ p, size_t n,
+                                                      unsigned char v) {
+  const size_t stride = (size_t)gridDim.x * TPB;
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+
+// ---- slice remap: dst slice (j / sB) + (j % sB) * sD  <-  src slice j --------------------------
+__global__ __launch_bounds__(TPB) void remap_kernel(float *__restrict__ dst, const float *__restrict__ src,
+                                                    uint32_t rc, uint32_t sD, FastDiv div_b) {
+  const uint32_t j = blockIdx.x;  // source slice
+  const uint32_t reald = fdiv(j, div_b);
+  const uint32_t realb = j - reald * div_b.div;
+  const float *s = src + (size_t)j * rc;
+  float *d = dst + ((size_t)reald + (size_t)realb * sD) * rc;
+  for (uint32_t i = blockIdx.y * TPB + threadIdx.x; i < rc; i += gridDim.y * TPB) d[i] = s[i];
+}
+
+// ---- bias forward: out[slice][i] += bias[slice % depth] ----------------------------------------
+__global__ __launch_bounds__(TPB) void bias_forward_kernel(float *__restrict__ out,
+                                                           const float *__restrict__ bias, uint32_t fmap,
+                                                           FastDiv div_depth) {
+  const uint32_t sl = blockIdx.x;
+  const uint32_t q = fdiv(sl, div_depth);
+  const float bv = bias[sl - q * div_depth.div];
+  float *o = out + (size_t)sl * fmap;
+  for (uint32_t i = blockIdx.y * TPB + threadIdx.x; i < fmap; i += gridDim.y * TPB) o[i] += bv;
+}
+
+// ---- FC bias gradient: bias[d] = sum_b out[b][d] ------------------------------------------------
+__global__ __launch_bounds__(TPB) void bias_backward_fc_kernel(float *__restrict__ bias,
+                                                               const float *__restrict__ og, int D, int B) {
+  const int d = blockIdx.x * TPB + threadIdx.x;
+  if (d >= D) return;
+  float s = 0.0f;
+  for (int b = 0; b < B; ++b) s += og[(size_t)b * D + d];
+  bias[d] = s;
+}
+
+// ---- ReLU ----------------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void relu_fwd_kernel(float *__restrict__ out, const float *__restrict__ in,
+                                                       size_t n) {
+  const size_t stride = (size_t)gridDim.x * TPB;
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) {
+    const float x = in[i];
+    out[i] = x > 0.0f ? x : 0.0f;
+  }
+}
+__global__ __launch_bounds__(TPB) void relu_bwd_kernel(float *__restrict__ ig, const float *__restrict__ og,
+                                                       const float *__restrict__ x, size_t n) {
+  const size_t stride = (size_t)gridDim.x * TPB;
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride)
+    ig[i] = og[i] * (x[i] > 0.0f ? 1.0f : 0.0f);
+}
+
+// ---- max pooling -----------------------------------------------------------------------------
+// forward: one lane per output element; window scanned row-major with strict '>' so that the
+// first maximum wins, index stored as h*iC + w (int), as CPUDriver::maxpool_forward does
+__global__ __launch_bounds__(TPB) void maxpool_fwd_kernel(float *__restrict__ out, int *__restrict__ idx,
+                                                          const float *__restrict__ in, cct_pool_args a,
+                                                          uint32_t total, FastDiv div_oc, FastDiv div_or) {
+  const uint32_t e = blockIdx.x * TPB + threadIdx.x;
+  if (e >= total) return;
+  const uint32_t t1 = fdiv(e, div_oc);
+  const int pw = e - t1 * a.oC;
+  const uint32_t plane = fdiv(t1, div_or);
+  const int ph = t1 - plane * a.oR;
+  const float *src = in + (size_t)plane * a.iR * a.iC;
+  const int h0 = ph * a.stride, w0 = pw * a.stride;
+  const int h1 = min(h0 + a.kernel_size, a.iR), w1 = min(w0 + a.kernel_size, a.iC);
+  float best = -FLT_MAX;
+  int besti = 0;
+  for (int h = h0; h < h1; ++h)
+    for (int w = w0; w < w1; ++w) {
+      const float v = src[h * a.iC + w];
+      if (v > best) {
+        best = v;
+        besti = h * a.iC + w;
+      }
+    }
+  out[e] = best;
+  idx[e] = besti;
+}
+
+// backward as a gather: one lane per input element sums the output gradients whose argmax is this
+// element, scanning candidate windows in (ph, pw) ascending order = the order of the
+// reference's scatter loop, so sums with several contributors are bit-identical
+__global__ __launch_bounds__(TPB) void maxpool_bwd_kernel(float *__restrict__ ig, const float *__restrict__ og,
+                                                          const int *__restrict__ idx, cct_pool_args a,
+                                                          uint32_t total, FastDiv div_ic, FastDiv div_ir) {
+  const uint32_t e = blockIdx.x * TPB + threadIdx.x;
+  if (e >= total) return;
+  const uint32_t t1 = fdiv(e, div_ic);
+  const int w = e - t1 * a.iC;
+  const uint32_t plane = fdiv(t1, div_ir);
+  const int h = t1 - plane * a.iR;
+  const int k = a.kernel_size, s = a.stride;
+  const int ph_lo = h < k ? 0 : (h - k) / s + 1, ph_hi = min(h / s, a.oR - 1);
+  const int pw_lo = w < k ? 0 : (w - k) / s + 1, pw_hi = min(w / s, a.oC - 1);
+  const int me = h * a.iC + w;
+  const size_t obase = (size_t)plane * a.oR * a.oC;
+  float acc = 0.0f;
+  for (int ph = ph_lo; ph <= ph_hi; ++ph)
+    for (int pw = pw_lo; pw <= pw_hi; ++pw) {
+      const size_t o = obase + ph * a.oC + pw;
+      if (idx[o] == me) acc += og[o];
+    }
+  ig[e] = acc;
+}
+
+// ---- LRN (across channels) -----------------------------------------------------------------------
+// forward: one lane per (image, pixel) walks the depth with the running window of
+// _f_lrn_forward (copy previous, subtract leaving square, add entering square), then applies
+// scale = 1 + alpha/size * sum and out = in / scale^beta.  denoms keeps scale.
+__global__ __launch_bounds__(TPB) void lrn_fwd_kernel(float *__restrict__ out, float *__restrict__ denoms,
+                                                      const float *__restrict__ in, int rc, int D,
+                                                      uint32_t total, int w, float aos, float beta,
+                                                      FastDiv div_rc) {
+  const uint32_t e = blockIdx.x * TPB + threadIdx.x;
+  if (e >= total) return;
+  const uint32_t ib = fdiv(e, div_rc);
+  const uint32_t q = e - ib * rc;
+  const size_t base = (size_t)ib * D * rc + q;
+  float sum = 0.0f;
+  for (int i = 0; i <= w; ++i)
+    if (i < D) {
+      const float x = in[base + (size_t)i * rc];
+      sum += x * x;
+    }
+  for (int d = 0; d < D; ++d) {
+    if (d > 0) {
+      if (d - w - 1 >= 0) {
+        const float x = in[base + (size_t)(d - w - 1) * rc];
+        sum -= x * x;
+      }
+      if (d + w < D) {
+        const float x = in[base + (size_t)(d + w) * rc];
+        sum += x * x;
+      }
+    }
+    const float scale = aos * sum + 1.0f;
+    denoms[base + (size_t)d * rc] = scale;
+    out[base + (size_t)d * rc] = in[base + (size_t)d * rc] / powf(scale, beta);
+  }
+}
+
+// backward as a gather over the window: in_grad[ch] = sum over od in [ch-w, ch+w] (ascending, the
+// order in which _f_lrn_backward's od loop touches channel ch) of g(od,ch) * out_grad[od]
+__global__ __launch_bounds__(TPB) void lrn_bwd_kernel(float *__restrict__ ig, const float *__restrict__ og,
+                                                      const float *__restrict__ x, const float *__restrict__ den,
+                                                      int rc, int D, uint32_t total, int w, float aos,
+                                                      float beta, FastDiv div_rc, FastDiv div_d) {
+  const uint32_t e = blockIdx.x * TPB + threadIdx.x;
+  if (e >= total) return;
+  // e = (ib*D + ch)*rc + q
+  const uint32_t t1 = fdiv(e, div_rc);
+  const uint32_t q = e - t1 * rc;
+  const uint32_t ib = fdiv(t1, div_d);
+  const int ch = t1 - ib * D;
+  const size_t base = (size_t)ib * D * rc + q;
+  const float xv = x[base + (size_t)ch * rc];
+  float acc = 0.0f;
+  for (int od = max(0, ch - w); od <= min(D - 1, ch + w); ++od) {
+    const size_t o = base + (size_t)od * rc;
+    const float dne = den[o];
+    const float denom = powf(dne, beta);
+    const float denom_n1 = (float)(1.0 / (double)(denom * dne));
+    const float wd = x[o];
+    const float g2 = beta * denom_n1 * aos * 2 * wd;
+    float gv;
+    if (od == ch) gv = (float)(1.0 / (double)denom - (double)(g2 * xv));
+    else gv = -g2 * xv;
+    acc += gv * og[o];
+  }
+  ig[e] = acc;
+}
+
+// ---- dropout -------------------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void dropout_kernel(float *__restrict__ out, const float *__restrict__ in,
+                                                      const unsigned int *__restrict__ mask, float scale,
+                                                      unsigned int thr, size_t n) {
+  const size_t stride = (size_t)gridDim.x * TPB;
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride)
+    out[i] = in[i] * (mask[i] > thr ? 1.0f : 0.0f) * scale;
+}
+
+// counter-based uint32 stream (splitmix64 finaliser over seed, call number and word index)
+__global__ __launch_bounds__(TPB) void rand_uint_kernel(unsigned int *__restrict__ buf, size_t n,
+                                                        uint64_t seed, uint64_t call) {
+  const size_t stride = (size_t)gridDim.x * TPB;
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) {
+    uint64_t z = seed * 0x9E3779B97F4A7C15ull + call * 0xD1B54A32D192ED03ull + i + 0x632BE59BD9B4E019ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    buf[i] = (unsigned int)(z >> 16);
+  }
+}
+
+// ---- softmax loss: one workgroup per image ----------------------------------------------------------
+__global__ __launch_bounds__(TPB) void softmax_fwd_kernel(float *__restrict__ prob, const float *__restrict__ in,
+                                                          const float *__restrict__ labels,
+                                                          float *__restrict__ loss_per_image, int len) {
+  __shared__ float scratch[8];
+  const int ib = blockIdx.x, tid = threadIdx.x;
+  const float *x = in + (size_t)ib * len;
+  float *y = prob + (size_t)ib * len;
+  float mx = -FLT_MAX;
+  for (int i = tid; i < len; i += TPB) mx = fmaxf(mx, x[i]);
+  mx = block_reduce<true>(mx, scratch);
+  float s = 0.0f;
+  for (int i = tid; i < len; i += TPB) s += expf(x[i] - mx);
+  s = block_reduce<false>(s, scratch);
+  for (int i = tid; i < len; i += TPB) y[i] = expf(x[i] - mx) / s;
+  __syncthreads();
+  if (tid == 0) {
+    const float pl = y[(int)labels[ib]];
+    loss_per_image[ib] = -logf(fmaxf(pl, FLT_MIN));
+  }
+}
+// batch sum in ascending image order (the order the reference accumulates its scalar loss)
+__global__ void softmax_loss_sum_kernel(float *__restrict__ loss_sum, const float *__restrict__ per_image,
+                                        int batch) {
+  if (threadIdx.x == 0 && blockIdx.x == 0) {
+    float s = 0.0f;
+    for (int i = 0; i < batch; ++i) s += per_image[i];
+    *loss_sum = s;
+  }
+}
+__global__ __launch_bounds__(TPB) void softmax_bwd_kernel(float *__restrict__ ig, const float *__restrict__ prob,
+                                                          const float *__restrict__ labels, int len,
+                                                          uint32_t total, double factor, FastDiv div_len) {
+  const uint32_t e = blockIdx.x * TPB + threadIdx.x;
+  if (e >= total) return;
+  const uint32_t ib = fdiv(e, div_len);
+  const int i = e - ib * len;
+  float v = prob[e];
+  if (i == (int)labels[ib]) v -= 1.0f;
+  ig[e] = (float)((double)v * factor);
+}
+
+// ---- BLAS-1 / SGD ----------------------------------------------------------------------------------
+__global__ __launch_bounds__(TPB) void saxpby_kernel(size_t n, float a, const float *__restrict__ x, float b,
+                                                     float *__restrict__ y, int has_b) {
+  const size_t stride = (size_t)gridDim.x * TPB;
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride)
+    y[i] = has_b ? a * x[i] + b * y[i] : a * x[i] + y[i];
+}
+__global__ __launch_bounds__(TPB) void l1_update_kernel(int n, float *__restrict__ g, float lambda,
+                                                        const float *__restrict__ w) {
+  const int i = blockIdx.x * TPB + threadIdx.x;
+  if (i < n) g[i] += lambda * (w[i] > 0 ? 1.0f : -1.0f);
+}
+// one pass: the three BLAS-1 calls of SGDGradientUpdater::update applied per element in the same
+// order, each product/sum rounded to fp32 as the separate calls would
+__global__ __launch_bounds__(TPB) void sgd_kernel(size_t n, float *__restrict__ w, float *__restrict__ g,
+                                                  float *__restrict__ h, float step, float mom, float lambda,
+                                                  int l1) {
+  const size_t stride = (size_t)gridDim.x * TPB;
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) {
+    const float wi = w[i];
+    float gi = g[i];
+    if (lambda != 0.0f) {
+      gi = l1 ? gi + lambda * (wi > 0 ? 1.0f : -1.0f) : __fadd_rn(__fmul_rn(lambda, wi), gi);
+      g[i] = gi;
+    }
+    const float hi = __fadd_rn(__fmul_rn(step, gi), __fmul_rn(mom, h[i]));
+    h[i] = hi;
+    w[i] = __fadd_rn(__fmul_rn(-1.0f, hi), wi);
+  }
+}
+
+// ---- gemv (row-major M x N, lda = N) -------------------------------------------------------------------
+// NoTrans: one workgroup per output row; Trans: one lane per output column
+__global__ __launch_bounds__(TPB) void gemv_n_kernel(int M, int N, float alpha, const float *__restrict__ A,
+                                                     const float *__restrict__ x, float beta,
+                                                     float *__restrict__ y) {
+  __shared__ float scratch[8];
+  const int row = blockIdx.x;
+  float s = 0.0f;
+  for (int j = threadIdx.x; j < N; j += TPB) s += A[(size_t)row * N + j] * x[j];
+  s = block_reduce<false>(s, scratch);
+  if (threadIdx.x == 0) y[row] = (beta == 0.0f) ? alpha * s : alpha * s + beta * y[row];
+}
+__global__ __launch_bounds__(TPB) void gemv_t_kernel(int M, int N, float alpha, const float *__restrict__ A,
+                                                     const float *__restrict__ x, float beta,
+                                                     float *__restrict__ y) {
+  const int col = blockIdx.x * TPB + threadIdx.x;
+  if (col >= N) return;
+  float s = 0.0f;
+  for (int i = 0; i < M; ++i) s += A[(size_t)i * N + col] * x[i];
+  y[col] = (beta == 0.0f) ? alpha * s : alpha * s + beta * y[col];
+}
+
+static inline uint32_t grid_stride_blocks(size_t n) {
+  const size_t want = (n + TPB - 1) / TPB;
+  const size_t cap = 256 * 32;  // 32 workgroups per compute unit
+  return (uint32_t)(want < cap ? (want ? want : 1) : cap);
+}
+
+}  // namespace cct
+
+using namespace cct;
+
+extern "C" {
+
+int cct_hip_memset(void *dev_ptr, int value, size_t size_in_byte) {
+  CCT_ENSURE_INIT();
+  if (size_in_byte == 0) return 0;
+  CCT_REQUIRE(dev_ptr, "memset: null pointer");
+  const unsigned char b = (unsigned char)value;
+  if ((uintptr_t)dev_ptr % 4 == 0 && size_in_byte % 4 == 0) {
+    const uint32_t w = b * 0x01010101u;
+    float f;
+    memcpy(&f, &w, 4);
+    const size_t n = size_in_byte / 4;
+    hipLaunchKernelGGL(fill_f32_kernel, dim3(grid_stride_blocks(n)), dim3(TPB), 0, ctx().stream,
+                       (float *)dev_ptr, n, f);
+  } else {
+    hipLaunchKernelGGL(fill_u8_kernel, dim3(grid_stride_blocks(size_in_byte)), dim3(TPB), 0, ctx().stream,
+                       (unsigned char *)dev_ptr, size_in_byte, b);
+  }
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_sconstant_initialize(float *arr, size_t n, float value) {
+  CCT_ENSURE_INIT();
+  if (n == 0) return 0;
+  CCT_REQUIRE(arr, "sconstant_initialize: null pointer");
+  hipLaunchKernelGGL(fill_f32_kernel, dim3(grid_stride_blocks(n)), dim3(TPB), 0, ctx().stream, arr, n, value);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_remap(float *dst, const float *src, const cct_pmap_helper *a) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(dst && src && a, "remap: null argument");
+  const size_t rc = a->sR * a->sC, slices = a->sD * a->sB;
+  if (rc == 0 || slices == 0) return 0;
+  CCT_REQUIRE(slices < (1ull << 31) && rc < (1ull << 31), "remap: too many slices");
+  const char *d0 = (const char *)dst, *s0 = (const char *)src;
+  const size_t bytes = rc * slices * 4;
+  CCT_REQUIRE(d0 + bytes <= s0 || s0 + bytes <= d0, "remap: dst and src overlap");
+  uint32_t gy = (uint32_t)((rc + TPB - 1) / TPB);
+  if (gy > 64) gy = 64;
+  hipLaunchKernelGGL(remap_kernel, dim3((uint32_t)slices, gy), dim3(TPB), 0, ctx().stream, dst, src,
+                     (uint32_t)rc, (uint32_t)a->sD, make_fastdiv((uint32_t)a->sB));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_forward_bias(const float *bias, float *out, int fmap_size, int depth, int batch_size) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(bias && out, "forward_bias: null argument");
+  CCT_REQUIRE(fmap_size > 0 && depth > 0 && batch_size >= 0, "forward_bias: bad sizes");
+  if (batch_size == 0) return 0;
+  const size_t slices = (size_t)depth * batch_size;
+  CCT_REQUIRE(slices < (1ull << 31), "forward_bias: too many slices");
+  uint32_t gy = (uint32_t)((fmap_size + TPB - 1) / TPB);
+  if (gy > 64) gy = 64;
+  hipLaunchKernelGGL(bias_forward_kernel, dim3((uint32_t)slices, gy), dim3(TPB), 0, ctx().stream, out, bias,
+                     (uint32_t)fmap_size, make_fastdiv((uint32_t)depth));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_backward_bias_fc(float *bias_grad, const float *out_grad, int D, int B) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(bias_grad && out_grad && D > 0 && B >= 0, "backward_bias_fc: bad argument");
+  hipLaunchKernelGGL(bias_backward_fc_kernel, dim3(blocks_for(D)), dim3(TPB), 0, ctx().stream, bias_grad,
+                     out_grad, D, B);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_relu_forward(float *out, const float *in, size_t n) {
+  CCT_ENSURE_INIT();
+  if (n == 0) return 0;
+  CCT_REQUIRE(out && in, "relu_forward: null argument");
+  hipLaunchKernelGGL(relu_fwd_kernel, dim3(grid_stride_blocks(n)), dim3(TPB), 0, ctx().stream, out, in, n);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_relu_backward(float *in_grad, const float *out_grad, const float *in_data, size_t n) {
+  CCT_ENSURE_INIT();
+  if (n == 0) return 0;
+  CCT_REQUIRE(in_grad && out_grad && in_data, "relu_backward: null argument");
+  hipLaunchKernelGGL(relu_bwd_kernel, dim3(grid_stride_blocks(n)), dim3(TPB), 0, ctx().stream, in_grad,
+                     out_grad, in_data, n);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+static int check_pool(const cct_pool_args *a, const char *who) {
+  CCT_REQUIRE(a && a->max_index, "%s: null argument", who);
+  CCT_REQUIRE(a->stride >= 1 && a->kernel_size >= 1 && a->iR >= 1 && a->iC >= 1 && a->oR >= 1 && a->oC >= 1 &&
+                  a->D >= 0 && a->B >= 0,
+              "%s: bad sizes", who);
+  // every window must start inside the input, as the reference's floor-based output size guarantees
+  CCT_REQUIRE((a->oR - 1) * a->stride < a->iR && (a->oC - 1) * a->stride < a->iC,
+              "%s: output %dx%d does not fit input %dx%d", who, a->oR, a->oC, a->iR, a->iC);
+  CCT_REQUIRE((size_t)a->D * a->B * a->iR * a->iC < (1ull << 31), "%s: tensor too large", who);
+  return 0;
+}
+
+int cct_hip_maxpool_forward(float *out, const float *in, const cct_pool_args *a) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(out && in, "maxpool_forward: null argument");
+  int rc = check_pool(a, "maxpool_forward");
+  if (rc) return rc;
+  const size_t total = (size_t)a->D * a->B * a->oR * a->oC;
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, out,
+                     a->max_index, in, *a, (uint32_t)total, make_fastdiv(a->oC), make_fastdiv(a->oR));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_pool_args *a) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(in_grad && out_grad, "maxpool_backward: null argument");
+  int rc = check_pool(a, "maxpool_backward");
+  if (rc) return rc;
+  const size_t total = (size_t)a->D * a->B * a->iR * a->iC;
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad,
+                     out_grad, a->max_index, *a, (uint32_t)total, make_fastdiv(a->iC), make_fastdiv(a->iR));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args *a,
+                        const cct_lrn_forward_normalize_args *a2) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(out && in && a && a2 && a->denoms, "lrn_forward: null argument");
+  CCT_REQUIRE(a->iR > 0 && a->iC > 0 && a->iD > 0 && a->iB >= 0 && a->norm_window >= 0, "lrn_forward: bad sizes");
+  const size_t total = (size_t)a->iB * a->iR * a->iC;
+  CCT_REQUIRE(total * a->iD < (1ull << 31), "lrn_forward: tensor too large");
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(lrn_fwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, out,
+                     (float *)a->denoms, in, a->iR * a->iC, a->iD, (uint32_t)total, a->norm_window,
+                     a2->alpha_over_size, a2->beta, make_fastdiv(a->iR * a->iC));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_lrn_backward(float *in_grad, const float *out_grad, const cct_lrn_backward_args *a) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(in_grad && out_grad && a && a->denoms && a->input_data, "lrn_backward: null argument");
+  CCT_REQUIRE(a->oR > 0 && a->oC > 0 && a->oD > 0 && a->oB >= 0 && a->norm_window >= 0, "lrn_backward: bad sizes");
+  const size_t total = (size_t)a->oB * a->oD * a->oR * a->oC;
+  CCT_REQUIRE(total < (1ull << 31), "lrn_backward: tensor too large");
+  if (total == 0) return 0;
+  hipLaunchKernelGGL(lrn_bwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad, out_grad,
+                     (const float *)a->input_data, (const float *)a->denoms, a->oR * a->oC, a->oD,
+                     (uint32_t)total, a->norm_window, a->alpha_over_size, a->beta,
+                     make_fastdiv(a->oR * a->oC), make_fastdiv(a->oD));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_dropout_forward_train(float *out, const float *in, const unsigned int *mask, float scale,
+                                  unsigned int threshold, size_t n) {
+  CCT_ENSURE_INIT();
+  if (n == 0) return 0;
+  CCT_REQUIRE(out && in && mask, "dropout_forward_train: null argument");
+  hipLaunchKernelGGL(dropout_kernel, dim3(grid_stride_blocks(n)), dim3(TPB), 0, ctx().stream, out, in, mask,
+                     scale, threshold, n);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_init_rng(int random_seed) {
+  CCT_ENSURE_INIT();
+  ctx().rng_seed = (uint64_t)(int64_t)random_seed;
+  ctx().rng_calls = 0;
+  return 0;
+}
+
+int cct_hip_rand_uint_initialize(unsigned int *buf, int n) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(n >= 0, "rand_uint_initialize: negative count");
+  if (n == 0) return 0;
+  CCT_REQUIRE(buf, "rand_uint_initialize: null buffer");
+  hipLaunchKernelGGL(rand_uint_kernel, dim3(grid_stride_blocks((size_t)n)), dim3(TPB), 0, ctx().stream, buf,
+                     (size_t)n, ctx().rng_seed, ctx().rng_calls);
+  CCT_LAUNCH_CHECK();
+  ctx().rng_calls++;
+  return 0;
+}
+
+int cct_hip_softmax_loss_forward(float *prob, const float *in, const float *labels, float *loss_sum,
+                                 int len_per_image, int batch) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(prob && in && labels && loss_sum, "softmax_loss_forward: null argument");
+  CCT_REQUIRE(len_per_image > 0 && batch >= 0, "softmax_loss_forward: bad sizes");
+  void *ws = nullptr;
+  int rc = get_workspace((size_t)(batch > 0 ? batch : 1) * sizeof(float), &ws);
+  if (rc) return rc;
+  if (batch > 0) {
+    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(batch), dim3(TPB), 0, ctx().stream, prob, in, labels,
+                       (float *)ws, len_per_image);
+    CCT_LAUNCH_CHECK();
+  }
+  hipLaunchKernelGGL(softmax_loss_sum_kernel, dim3(1), dim3(64), 0, ctx().stream, loss_sum, (const float *)ws,
+                     batch);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_softmax_loss_backward(float *in_grad, const float *prob, const float *labels, int len_per_image,
+                                  int batch, int spatial) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(in_grad && prob && labels, "softmax_loss_backward: null argument");
+  CCT_REQUIRE(len_per_image > 0 && batch > 0 && spatial > 0, "softmax_loss_backward: bad sizes");
+  const size_t total = (size_t)len_per_image * batch;
+  CCT_REQUIRE(total < (1ull << 31), "softmax_loss_backward: tensor too large");
+  const double factor = 1. / (double)batch / (double)spatial;
+  hipLaunchKernelGGL(softmax_bwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad, prob,
+                     labels, len_per_image, (uint32_t)total, factor, make_fastdiv(len_per_image));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_math_saxpby(size_t n, float alpha, const float *x, float beta, float *y) {
+  CCT_ENSURE_INIT();
+  if (n == 0) return 0;
+  CCT_REQUIRE(x && y, "math_saxpby: null argument");
+  hipLaunchKernelGGL(saxpby_kernel, dim3(grid_stride_blocks(n)), dim3(TPB), 0, ctx().stream, n, alpha, x, beta,
+                     y, 1);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_math_saxpy(size_t n, float alpha, const float *x, float *y) {
+  CCT_ENSURE_INIT();
+  if (n == 0) return 0;
+  CCT_REQUIRE(x && y, "math_saxpy: null argument");
+  hipLaunchKernelGGL(saxpby_kernel, dim3(grid_stride_blocks(n)), dim3(TPB), 0, ctx().stream, n, alpha, x, 1.0f,
+                     y, 0);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_L1_update(int n, float *gradient, float lambda, const float *model) {
+  CCT_ENSURE_INIT();
+  if (n <= 0) return 0;
+  CCT_REQUIRE(gradient && model, "L1_update: null argument");
+  hipLaunchKernelGGL(l1_update_kernel, dim3(blocks_for(n)), dim3(TPB), 0, ctx().stream, n, gradient, lambda,
+                     model);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_sgd_update(size_t n, float *model, float *gradient, float *history, float stepsize, float momentum,
+                       float lambda, int l1) {
+  CCT_ENSURE_INIT();
+  if (n == 0) return 0;
+  CCT_REQUIRE(model && gradient && history, "sgd_update: null argument");
+  hipLaunchKernelGGL(sgd_kernel, dim3(grid_stride_blocks(n)), dim3(TPB), 0, ctx().stream, n, model, gradient,
+                     history, stepsize, momentum, lambda, l1);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_sgemv(int TA, int M, int N, float alpha, const float *A, const float *x, float beta, float *y) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(TA == CCT_NO_TRANS || TA == CCT_TRANS, "sgemv: bad transpose flag %d", TA);
+  CCT_REQUIRE(M >= 0 && N >= 0, "sgemv: negative dimension");
+  if (M == 0 || N == 0) return 0;
+  CCT_REQUIRE(A && x && y, "sgemv: null argument");
+  if (TA == CCT_NO_TRANS)
+    hipLaunchKernelGGL(gemv_n_kernel, dim3(M), dim3(TPB), 0, ctx().stream, M, N, alpha, A, x, beta, y);
+  else
+    hipLaunchKernelGGL(gemv_t_kernel, dim3(blocks_for(N)), dim3(TPB), 0, ctx().stream, M, N, alpha, A, x, beta,
+                       y);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // extern "C"

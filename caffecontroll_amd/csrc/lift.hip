@@ -1,0 +1,200 @@
+// Inverse lowering (col2im lifting) for gfx950, gather formulation, optionally in one launch
+// with the bias-gradient reduction.
+//
+//   dst[ib][id][y][x] = sum over (kr ascending, kc ascending) with cr*s + kr - p == y,
+//                       cc*s + kc - p == x, 0 <= cr,cc < m of
+//                       src[((id*k + kr)*k + kc) * iB*m*m + ib*m*m + cr*m + cc]
+//
+// One lane owns one destination pixel and adds its (at most ceil(k/s)^2) contributions in the
+// order the reference's scatter loop delivers them (src/sched/DeviceDriver_CPU.cpp:322-345), so
+// the result is bit-identical to that loop run on a zero-filled destination.  Every source
+// element is read exactly once; lanes of a wave read consecutive addresses of one (kr,kc) plane.
+//
+// HBM traffic per launch: reads iD*k*k*iB*m*m*4, writes iB*iD*iR*iC*4.  Bound: HBM read bandwidth.
+//
+// Bias gradient (fused variant): workgroups past the lift range each own one output channel and
+// reduce out_grad[b][o][fmap] over b and fmap with per-lane partial sums, a wavefront
+// (cross-lane) reduction and a final pass over the workgroup's wave sums.
+#include "cct_common.h"
+
+namespace cct {
+
+struct LiftParams {
+  int m;  // output rows == cols (the reference indexes with oh*cr + cc)
+  int k, s, p;
+  int iR, iC, iD, iB;
+  uint32_t npix;      // iB*iD*iR*iC
+  uint32_t nblocks;   // lift workgroups
+  size_t plane;       // iB*m*m
+  FastDiv div_c, div_r, div_d;
+  // bias part
+  const float *out_grad;
+  float *bias_grad;
+  int fmap, depth, batch;
+};
+
+constexpr int LIFT_THREADS = 256;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+  return v;
+}
+
+__device__ void bias_backward_block(const LiftParams &P, int o) {
+  __shared__ float wave_part[LIFT_THREADS / 64];
+  const int tid = threadIdx.x;
+  // four images at a time with independent partial sums keeps several loads in flight per lane
+  float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
+  const size_t img = (size_t)P.depth * P.fmap;
+  int bi = 0;
+  for (; bi + 4 <= P.batch; bi += 4) {
+    const float *g = P.out_grad + ((size_t)bi * P.depth + o) * P.fmap;
+    for (int i = tid; i < P.fmap; i += LIFT_THREADS) {
+      const float v0 = g[i], v1 = g[img + i], v2 = g[2 * img + i], v3 = g[3 * img + i];
+      a0 += v0; a1 += v1; a2 += v2; a3 += v3;
+    }
+  }
+  for (; bi < P.batch; ++bi) {
+    const float *g = P.out_grad + ((size_t)bi * P.depth + o) * P.fmap;
+    for (int i = tid; i < P.fmap; i += LIFT_THREADS) a0 += g[i];
+  }
+  float acc = wave_sum((a0 + a1) + (a2 + a3));
+  if ((tid & 63) == 0) wave_part[tid >> 6] = acc;
+  __syncthreads();
+  if (tid == 0) {
+    float t = 0.0f;
+#pragma unroll
+    for (int w = 0; w < LIFT_THREADS / 64; ++w) t += wave_part[w];
+    P.bias_grad[o] = t;
+  }
+}
+
+// KT/ST: compile-time kernel size / stride (0 = read from P at run time)
+template <int KT, int ST>
+__global__ __launch_bounds__(LIFT_THREADS) void lift_kernel(float *__restrict__ dst,
+                                                            const float *__restrict__ src,
+                                                            const LiftParams P) {
+  if (blockIdx.x >= P.nblocks) {
+    bias_backward_block(P, (int)(blockIdx.x - P.nblocks));
+    return;
+  }
+  const int k = KT ? KT : P.k;
+  const int s = ST ? ST : P.s;
+  const uint32_t pix = blockIdx.x * LIFT_THREADS + threadIdx.x;
+  if (pix >= P.npix) return;
+  // pix = ((ib*iD + id)*iR + y)*iC + x
+  const uint32_t t1 = fdiv(pix, P.div_c);
+  const int x = pix - t1 * P.iC;
+  const uint32_t t2 = fdiv(t1, P.div_r);
+  const int y = t1 - t2 * P.iR;
+  const uint32_t ib = fdiv(t2, P.div_d);
+  const int id = t2 - ib * P.iD;
+
+  const int m = P.m;
+  const float *base = src + (size_t)id * k * k * P.plane + (size_t)ib * m * m;
+  float acc = 0.0f;
+  const int yp = y + P.p, xp = x + P.p;
+  if (ST == 1) {
+    // every (kr,kc) is a candidate; out-of-range ones contribute an exact +0
+#pragma unroll
+    for (int kr = 0; kr < k; ++kr) {
+      const int cr = yp - kr;
+      const bool rok = (cr >= 0) && (cr < m);
+#pragma unroll
+      for (int kc = 0; kc < k; ++kc) {
+        const int cc = xp - kc;
+        const bool ok = rok && (cc >= 0) && (cc < m);
+        const size_t off = (size_t)(kr * k + kc) * P.plane + (size_t)(ok ? cr * m + cc : 0);
+        const float v = ok ? base[off] : 0.0f;
+        acc += v;
+      }
+    }
+  } else {
+    for (int kr = yp % s; kr < k; kr += s) {
+      const int cr = (yp - kr) / s;
+      if (yp < kr) break;
+      if (cr >= m) continue;
+      for (int kc = xp % s; kc < k; kc += s) {
+        const int cc = (xp - kc) / s;
+        if (xp < kc) break;
+        if (cc >= m) continue;
+        acc += base[(size_t)(kr * k + kc) * P.plane + (size_t)(cr * m + cc)];
+      }
+    }
+  }
+  dst[pix] = acc;
+}
+
+static int launch_lift(float *dst, const float *src, const cct_inverse_lower_cube_args *a,
+                       float *bias_grad, const float *out_grad, int fmap, int depth, int batch) {
+  CCT_REQUIRE(dst && src && a, "inverse_lower_cube: null argument");
+  CCT_REQUIRE(a->data_output_width == a->data_output_height,
+              "inverse_lower_cube: output must be square (%zu x %zu)", a->data_output_width,
+              a->data_output_height);
+  CCT_REQUIRE(a->stride >= 1 && a->kernel_size >= 1, "inverse_lower_cube: bad kernel/stride");
+  const size_t npix = a->iB * a->iD * a->iR * a->iC;
+  const size_t m = a->data_output_width;
+  CCT_REQUIRE(npix < (1ull << 31) && a->iB * m * m < (1ull << 31),
+              "inverse_lower_cube: tensor too large for 31-bit position arithmetic");
+  LiftParams P;
+  P.m = (int)m; P.k = (int)a->kernel_size; P.s = (int)a->stride; P.p = (int)a->padding;
+  P.iR = (int)a->iR; P.iC = (int)a->iC; P.iD = (int)a->iD; P.iB = (int)a->iB;
+  P.npix = (uint32_t)npix;
+  P.nblocks = (uint32_t)((npix + LIFT_THREADS - 1) / LIFT_THREADS);
+  P.plane = a->iB * m * m;
+  P.div_c = make_fastdiv(P.iC); P.div_r = make_fastdiv(P.iR); P.div_d = make_fastdiv(P.iD);
+  P.out_grad = out_grad; P.bias_grad = bias_grad; P.fmap = fmap; P.depth = depth; P.batch = batch;
+  const uint32_t extra = bias_grad ? (uint32_t)depth : 0;
+  const uint32_t grid = P.nblocks + extra;
+  if (grid == 0) return 0;
+  hipStream_t st = ctx().stream;
+  if (P.k == 5 && P.s == 1)
+    hipLaunchKernelGGL((lift_kernel<5, 1>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
+  else if (P.k == 3 && P.s == 1)
+    hipLaunchKernelGGL((lift_kernel<3, 1>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
+  else if (P.k == 11 && P.s == 4)
+    hipLaunchKernelGGL((lift_kernel<11, 4>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
+  else
+    hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+}  // namespace cct
+
+using namespace cct;
+
+extern "C" int cct_hip_inverse_lower_cube(float *dst, const float *src,
+                                          const cct_inverse_lower_cube_args *args) {
+  CCT_ENSURE_INIT();
+  return launch_lift(dst, src, args, nullptr, nullptr, 0, 0, 0);
+}
+
+extern "C" int cct_hip_inverse_lower_cube_bias_backward(float *dst, const float *src,
+                                                        const cct_inverse_lower_cube_args *args,
+                                                        float *bias_grad, const float *out_grad,
+                                                        int fmap_size, int depth, int batch_size) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(bias_grad && out_grad, "inverse_lower_cube_bias_backward: null bias argument");
+  CCT_REQUIRE(fmap_size > 0 && depth > 0 && batch_size > 0,
+              "inverse_lower_cube_bias_backward: fmap/depth/batch must be positive");
+  return launch_lift(dst, src, args, bias_grad, out_grad, fmap_size, depth, batch_size);
+}
+
+extern "C" int cct_hip_backward_bias(float *bias_grad, const float *out_grad, int fmap_size,
+                                     int depth, int batch_size) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(bias_grad && out_grad, "backward_bias: null argument");
+  CCT_REQUIRE(fmap_size > 0 && depth > 0 && batch_size > 0,
+              "backward_bias: fmap/depth/batch must be positive");
+  // the same kernel with zero lift blocks
+  LiftParams P = {};
+  P.nblocks = 0;
+  P.out_grad = out_grad; P.bias_grad = bias_grad; P.fmap = fmap_size; P.depth = depth;
+  P.batch = batch_size;
+  hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(depth), dim3(LIFT_THREADS), 0, ctx().stream,
+                     (float *)nullptr, (const float *)nullptr, P);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,199 @@
+// Type-1 lowering (im2col) for gfx950, whole batch per launch.
+//
+//   dst[(bi*m*m + r*m + c) * k*k*d + dd*k*k + kr*k + kc] = src[bi][dd][r*s-p+kr][c*s-p+kc]  (0 outside)
+//
+// One workgroup owns (image bi, band of RB output rows, slab of DS input channels).  It stages
+// the zero-padded input window of that band in LDS with coalesced row reads, then streams out
+// the lowered rows: consecutive lanes write consecutive addresses of one lowered row, each
+// lowered element is written exactly once, padding zeros come from the LDS tile so the store
+// loop has no bounds tests.  The per-row-position LDS offsets (the (dd,kr,kc) decomposition)
+// are tabulated once per workgroup.
+//
+// HBM traffic per launch: reads b*d*n*n*4 (plus band halo re-reads, served by L2), writes
+// b*m*m*k*k*d*4.  Bound: HBM write bandwidth.
+#include "cct_common.h"
+
+namespace cct {
+
+struct LowerParams {
+  int n, d, k, s, p, b, m;
+  int RB;      // output rows per band
+  int DS;      // channels per slab
+  int TH, TW;  // staged tile rows / cols per channel
+  int seglen;  // DS*k*k floats written per output position by one workgroup
+  int rowlen;  // k*k*d
+  int nbands, nslabs;
+  uint32_t nblocks;
+  FastDiv div_kk, div_k, div_tw, div_th, div_seg;
+};
+
+constexpr int LOWER_THREADS = 256;
+
+// dynamic LDS: [DS*TH*TW floats tile][seglen uint16 offsets]
+template <bool VEC4>
+__global__ __launch_bounds__(LOWER_THREADS) void lower_kernel(float *__restrict__ dst,
+                                                              const float *__restrict__ src,
+                                                              const LowerParams P) {
+  extern __shared__ float lds[];
+  const int tile_elems = P.DS * P.TH * P.TW;
+  float *tile = lds;
+  uint16_t *offs = reinterpret_cast<uint16_t *>(lds + tile_elems);
+
+  // logical block id -> (bi, band, slab); bands of one image stay on one XCD
+  uint32_t id = xcd_remap(blockIdx.x, P.nblocks);
+  const int slab = id % P.nslabs;
+  id /= P.nslabs;
+  const int band = id % P.nbands;
+  const int bi = id / P.nbands;
+
+  const int tid = threadIdx.x;
+  const int r0 = band * P.RB;
+  const int rb = min(P.RB, P.m - r0);
+  const int dd0 = slab * P.DS;
+  const int ds = min(P.DS, P.d - dd0);
+  const int seg = ds * P.k * P.k;
+
+  // (1) offset table: j = dl*k*k + kr*k + kc  ->  (dl*TH + kr)*TW + kc
+  for (int j = tid; j < seg; j += LOWER_THREADS) {
+    const uint32_t dl = fdiv(j, P.div_kk);
+    const uint32_t rem = j - dl * P.k * P.k;
+    const uint32_t kr = fdiv(rem, P.div_k);
+    const uint32_t kc = rem - kr * P.k;
+    offs[j] = (uint16_t)((dl * P.TH + kr) * P.TW + kc);
+  }
+
+  // (2) stage the padded window: tile[dl][ty][tx] = src[bi][dd0+dl][r0*s-p+ty][-p+tx]
+  {
+    const int y0 = r0 * P.s - P.p;
+    const int th_used = (rb - 1) * P.s + P.k;
+    const float *img = src + ((size_t)bi * P.d + dd0) * P.n * P.n;
+    const int total = ds * P.TH * P.TW;
+    for (int e = tid; e < total; e += LOWER_THREADS) {
+      const uint32_t row = fdiv(e, P.div_tw);  // dl*TH + ty
+      const int tx = e - row * P.TW;
+      const uint32_t dl = fdiv(row, P.div_th);
+      const int ty = row - dl * P.TH;
+      const int y = y0 + ty, x = tx - P.p;
+      float v = 0.0f;
+      if (ty < th_used && y >= 0 && y < P.n && x >= 0 && x < P.n)
+        v = img[((size_t)dl * P.n + y) * P.n + x];
+      tile[e] = v;
+    }
+  }
+  __syncthreads();
+
+  // (3) stream the lowered rows
+  float *out_band = dst + ((size_t)bi * P.m + r0) * P.m * P.rowlen + (size_t)dd0 * P.k * P.k;
+  if (VEC4) {
+    // seg % 4 == 0 and every segment start is 16-byte aligned: a lane owns 4 consecutive row
+    // positions and walks over the output positions of the band
+    const int nq = seg >> 2;
+    for (int q = tid; q < nq; q += LOWER_THREADS) {
+      const int o0 = offs[4 * q], o1 = offs[4 * q + 1], o2 = offs[4 * q + 2], o3 = offs[4 * q + 3];
+      float *outq = out_band + 4 * q;
+      for (int rl = 0; rl < rb; ++rl) {
+        const float *trow = tile + rl * P.s * P.TW;
+        float *orow = outq + (size_t)rl * P.m * P.rowlen;
+#pragma unroll 4
+        for (int c = 0; c < P.m; ++c) {
+          const float *t = trow + c * P.s;
+          float4 v = make_float4(t[o0], t[o1], t[o2], t[o3]);
+          *reinterpret_cast<float4 *>(orow + (size_t)c * P.rowlen) = v;
+        }
+      }
+    }
+  } else {
+    // general shapes: flat index over (c, j) of one band row; lanes write consecutive floats
+    const uint32_t per_row = (uint32_t)P.m * seg;
+    const bool contiguous = (ds == P.d);
+    for (int rl = 0; rl < rb; ++rl) {
+      const float *trow = tile + rl * P.s * P.TW;
+      float *orow = out_band + (size_t)rl * P.m * P.rowlen;
+      for (uint32_t e = tid; e < per_row; e += LOWER_THREADS) {
+        const uint32_t c = (seg == P.seglen) ? fdiv(e, P.div_seg) : e / (uint32_t)seg;
+        const uint32_t j = e - c * seg;
+        const float v = trow[c * P.s + offs[j]];
+        if (contiguous)
+          orow[e] = v;
+        else
+          orow[(size_t)c * P.rowlen + j] = v;
+      }
+    }
+  }
+}
+
+}  // namespace cct
+
+using namespace cct;
+
+extern "C" int cct_hip_lower_cube(float *dst, const float *src, const cct_pmap_helper *a) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(dst && src && a, "lower_cube: null argument");
+  // same preconditions as CPUDriver::lower_cube (src/sched/DeviceDriver_CPU.cpp:137-140)
+  CCT_REQUIRE(a->sR == a->sC, "lower_cube: input must be square (sR=%zu sC=%zu)", a->sR, a->sC);
+  CCT_REQUIRE(a->kR == a->kC, "lower_cube: kernel must be square (kR=%zu kC=%zu)", a->kR, a->kC);
+  CCT_REQUIRE(a->stride >= 1, "lower_cube: stride must be >= 1");
+  CCT_REQUIRE(a->kR >= 1 && a->sR + 2 * a->padding >= a->kR, "lower_cube: kernel larger than padded input");
+  if (a->sB == 0 || a->sD == 0) return 0;
+
+  LowerParams P;
+  P.n = (int)a->sR; P.d = (int)a->sD; P.k = (int)a->kR; P.s = (int)a->stride;
+  P.p = (int)a->padding; P.b = (int)a->sB;
+  P.m = (P.n + 2 * P.p - P.k) / P.s + 1;
+  P.rowlen = P.k * P.k * P.d;
+  const size_t out_elems = (size_t)P.b * P.m * P.m * P.rowlen;
+  CCT_REQUIRE((size_t)P.b * P.d * P.n * P.n < (1ull << 31) && out_elems / P.rowlen < (1ull << 31),
+              "lower_cube: tensor too large for 31-bit position arithmetic");
+
+  // Tile sizing: keep the staged window within 78 KB so two workgroups share a CU's 160 KB LDS,
+  // keep the uint16 offset table valid (< 65536 tile elements), prefer whole rows (DS = d).
+  const size_t lds_budget = 78 * 1024;
+  P.TW = (P.m - 1) * P.s + P.k;
+  P.RB = 1;
+  P.DS = P.d;
+  auto lds_need = [&](int RB, int DS) {
+    const size_t th = (size_t)(RB - 1) * P.s + P.k;
+    return (size_t)DS * th * P.TW * 4 + (((size_t)DS * P.k * P.k * 2 + 3) & ~(size_t)3);
+  };
+  while (P.DS > 1 && (lds_need(1, P.DS) > lds_budget || (size_t)P.DS * P.k * P.TW >= 65536))
+    P.DS = (P.DS + 1) / 2;
+  CCT_REQUIRE(lds_need(1, P.DS) <= 150 * 1024 && (size_t)P.DS * P.k * P.TW < 65536,
+              "lower_cube: one channel window (%d x %d floats) does not fit in LDS", P.k, P.TW);
+  // With strided kernels a one-row band re-reads k/s times the input; widen the band while it fits.
+  if (P.s < P.k) {
+    while (P.RB < P.m && P.RB < 8 && lds_need(P.RB * 2, P.DS) <= lds_budget &&
+           (size_t)P.DS * ((size_t)(P.RB * 2 - 1) * P.s + P.k) * P.TW < 65536 &&
+           (size_t)P.b * ((P.m + P.RB * 2 - 1) / (P.RB * 2)) >= 2048)
+      P.RB *= 2;
+  }
+  P.TH = (P.RB - 1) * P.s + P.k;
+  P.seglen = P.DS * P.k * P.k;
+  P.nbands = (P.m + P.RB - 1) / P.RB;
+  P.nslabs = (P.d + P.DS - 1) / P.DS;
+  const size_t nblocks = (size_t)P.b * P.nbands * P.nslabs;
+  CCT_REQUIRE(nblocks < (1ull << 31), "lower_cube: too many workgroups");
+  P.nblocks = (uint32_t)nblocks;
+  P.div_kk = make_fastdiv(P.k * P.k);
+  P.div_k = make_fastdiv(P.k);
+  P.div_tw = make_fastdiv(P.TW);
+  P.div_th = make_fastdiv(P.TH);
+  P.div_seg = make_fastdiv(P.seglen);
+
+  const size_t lds_bytes = lds_need(P.RB, P.DS);
+  // float4 stores need every (position, slab) segment to start 16-byte aligned and to hold a
+  // whole number of float4: k*k*DS % 4 == 0 covers both when dst itself is aligned.
+  const bool vec4 = ((uintptr_t)dst % 16 == 0) && (P.rowlen % 4 == 0) && ((P.DS * P.k * P.k) % 4 == 0) &&
+                    (P.d % P.DS == 0);
+  hipStream_t st = ctx().stream;
+  if (vec4) {
+    CCT_HIP_CHECK(hipFuncSetAttribute((const void *)lower_kernel<true>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    hipLaunchKernelGGL(lower_kernel<true>, dim3(P.nblocks), dim3(LOWER_THREADS), lds_bytes, st, dst, src, P);
+  } else {
+    CCT_HIP_CHECK(hipFuncSetAttribute((const void *)lower_kernel<false>,
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
+    hipLaunchKernelGGL(lower_kernel<false>, dim3(P.nblocks), dim3(LOWER_THREADS), lds_bytes, st, dst, src, P);
+  }
+  CCT_LAUNCH_CHECK();
+  return 0;
+}

@@ -1,0 +1,217 @@
+/*
+ * cct_hip.h -- C ABI of the MI355X (gfx950) device driver for CaffeConTroll's lowering-based
+ * convolution training path.
+ *
+ * Every entry point is what a `HIPDriver : DeviceDriver` placed next to the reference's CPUDriver
+ * binds for one DeviceDriver member; the member it stands for is cited on each declaration
+ * (paths relative to the CaffeConTroll tree).  Pointers named dst/src/A/B/C/x/y are DEVICE
+ * pointers unless the comment says otherwise; argument structs are HOST structs passed by
+ * pointer and copied by value into kernel arguments.  Tensors are dense fp32 in the
+ * reference's Layout_CRDB (index = c + r*C + d*R*C + b*R*C*D, src/LogicalCube_impl.hxx:216-220).
+ *
+ * Error convention: the reference's drivers return void and assert(false) on error
+ * (src/sched/DeviceDriver.h:48-51).  Here every function returns 0 on success or a non-zero
+ * code (a hipError_t value, or CCT_HIP_EINVAL for rejected arguments); the C++ HIPDriver
+ * wrapper turns non-zero into message + abort to keep the reference behaviour.
+ * cct_hip_last_error() describes the most recent failure on the calling thread.
+ *
+ * Streams: all work is enqueued on one stream per process (the null stream until
+ * cct_hip_set_stream is called).  Calls are asynchronous with respect to the host unless
+ * stated; cct_hip_device_sync() waits for the stream.
+ */
+#ifndef CCT_HIP_H
+#define CCT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CCT_HIP_EINVAL 100001
+
+/* CBLAS enum values as used by the reference's cblas.h consumers. */
+enum { CCT_ROW_MAJOR = 101, CCT_COL_MAJOR = 102, CCT_NO_TRANS = 111, CCT_TRANS = 112 };
+
+/* struct PMapHelper, src/sched/DeviceHeader.h:25-35 -- identical field order. */
+typedef struct cct_pmap_helper {
+  size_t dR, dC, dD, dB; /* dst RCDB */
+  size_t sR, sC, sD, sB; /* src RCDB */
+  size_t dBR, dBC;       /* dst block */
+  size_t sBR, sBC;       /* src block */
+  size_t kR, kC, kD, kB; /* kernel RCDB */
+  size_t stride;
+  size_t padding;
+} cct_pmap_helper;
+
+/* struct _inverse_lower_cube_arg_helper, src/kernels/lowering.h:22-32 -- identical field order. */
+typedef struct cct_inverse_lower_cube_args {
+  size_t data_output_width;
+  size_t data_output_height;
+  size_t kernel_size;
+  size_t stride;
+  size_t padding;
+  size_t iR, iC, iD, iB;
+} cct_inverse_lower_cube_args;
+
+/* struct _pool_forward_arg_helper / _pool_backward_arg_helper, src/kernels/pool.h:7-29
+ * (the two reference structs have the same fields in the same order). max_index: device. */
+typedef struct cct_pool_args {
+  int stride;
+  int kernel_size;
+  int iR, iC, oR, oC, D, B;
+  int *max_index;
+} cct_pool_args;
+
+/* struct _lrn_forward_arg_helper, src/kernels/lrn.h:7-15. denoms: device. */
+typedef struct cct_lrn_forward_args {
+  int iR, iC, iD, iB;
+  int norm_window;
+  int local_size;
+  char *denoms;
+} cct_lrn_forward_args;
+
+/* struct _lrn_forward_normalize_arg_helper, src/kernels/lrn.h:17-21. */
+typedef struct cct_lrn_forward_normalize_args {
+  float alpha_over_size;
+  float beta;
+  char *denoms;
+} cct_lrn_forward_normalize_args;
+
+/* struct _lrn_backward_arg_helper, src/kernels/lrn.h:23-35. Pointers: device. */
+typedef struct cct_lrn_backward_args {
+  int oR, oC, oD, oB;
+  float alpha_over_size;
+  float beta;
+  int norm_window;
+  int local_size;
+  char *denoms;
+  char *input_data;
+  char *output_data;
+} cct_lrn_backward_args;
+
+/* ---- process / device state --------------------------------------------------------- */
+/* DeviceDriver::set_device_id + init_thread (src/sched/DeviceDriver.h:269-272): selects the
+ * device for the calling thread and creates the library state on first use. */
+int cct_hip_init(int device_id);
+/* Use an existing hipStream_t (passed as void*) for all later work; NULL = null stream. */
+int cct_hip_set_stream(void *hip_stream);
+/* DeviceDriver::device_sync, src/sched/DeviceDriver.h:267. */
+int cct_hip_device_sync(void);
+const char *cct_hip_last_error(void);
+/* Number of compute units of the selected device (0 before init). */
+int cct_hip_compute_units(void);
+
+/* ---- memory: DeviceDriver::malloc/free/memcpy/memset, src/sched/DeviceDriver.h:83-86 ---- */
+int cct_hip_malloc(void **dev_ptr, size_t size_in_byte);
+int cct_hip_free(void *dev_ptr);
+/* kind: 0 host->device, 1 device->host, 2 device->device. Synchronous for kinds 0 and 1. */
+int cct_hip_memcpy(void *dst, const void *src, size_t size_in_byte, int kind);
+int cct_hip_memset(void *dev_ptr, int value, size_t size_in_byte);
+
+/* ---- lowering / lifting / remap ------------------------------------------------------ */
+/* DeviceDriver::lower_cube<_fpmap_id,_fmap_lower> (src/sched/DeviceDriver.h:108-112; CPU
+ * semantics src/sched/DeviceDriver_CPU.cpp:124-301).  src [sB][sD][sR][sC] ->
+ * dst [sB*m*m][kR*kR*sD], whole batch in one launch, zero padding written explicitly. */
+int cct_hip_lower_cube(float *dst, const float *src, const cct_pmap_helper *args);
+/* DeviceDriver::inverse_lower_cube (src/sched/DeviceDriver.h:119-122; CPU semantics
+ * src/sched/DeviceDriver_CPU.cpp:306-346).  src [iD*k*k][iB][oh*ow] -> dst [iB][iD][iR][iC].
+ * Gather formulation: dst is overwritten (no prior zero fill needed) with the same per-pixel
+ * summation order (kr ascending, kc ascending) as the reference's scatter loop. */
+int cct_hip_inverse_lower_cube(float *dst, const float *src,
+                               const cct_inverse_lower_cube_args *args);
+/* inverse_lower_cube and backward_bias in ONE launch: the lift blocks gather dst from src while
+ * extra blocks reduce out_grad [batch][depth][fmap] into bias_grad [depth] with wavefront
+ * reductions.  Replaces the pair Connector::inverse_lower_cube
+ * (src/Connector_impl_Lowering_type1.hxx:130-183) + bias gradient
+ * (src/bridges/ConvolutionBridge_impl.hxx:575-599). */
+int cct_hip_inverse_lower_cube_bias_backward(float *dst, const float *src,
+                                             const cct_inverse_lower_cube_args *args,
+                                             float *bias_grad, const float *out_grad,
+                                             int fmap_size, int depth, int batch_size);
+/* DeviceDriver::pmap2d_read_coalesce<_fpmap_id,_fmap_remap> (src/sched/DeviceDriver.h:100-104,
+ * src/kernels/lowering.hxx:241-258): slice j of src (sR*sC floats, j < sD*sB) goes to slice
+ * (j / sB) + (j % sB) * sD of dst.  dst and src must not overlap. */
+int cct_hip_remap(float *dst, const float *src, const cct_pmap_helper *args);
+
+/* ---- BLAS-shaped ----------------------------------------------------------------------- */
+/* DeviceDriver::sgemm (src/sched/DeviceDriver.h:206-208), cblas_sgemm contract. fp32 MFMA. */
+int cct_hip_sgemm(int order, int TA, int TB, int M, int N, int K, float alpha, const float *A,
+                  int lda, const float *B, int ldb, float beta, float *C, int ldc);
+/* DeviceDriver::sgemm_new (src/sched/DeviceDriver.h:211-213): row-major,
+ * lda = (TA==N ? K : M), ldb = (TB==N ? N : K), ldc = N. */
+int cct_hip_sgemm_new(int TA, int TB, int M, int N, int K, float alpha, const float *A,
+                      const float *B, float beta, float *C);
+/* Forward-convolution GEMM with the output permutation and bias of
+ * ConvolutionBridge::forward (src/bridges/ConvolutionBridge_impl.hxx:328-364) folded into the
+ * epilogue: out[b][o][fmap] = model[o x K] * lowered[b*fmap x K]^T + bias[o] (bias may be NULL). */
+int cct_hip_sgemm_conv_forward(int o, int batch, int fmap, int K, const float *model,
+                               const float *lowered, const float *bias, float *out);
+/* DeviceDriver::sgemv (src/sched/DeviceDriver.h:214-215): row-major M x N, lda = N. */
+int cct_hip_sgemv(int TA, int M, int N, float alpha, const float *A, const float *x, float beta,
+                  float *y);
+/* DeviceDriver::math_saxpy / math_saxpby (src/sched/DeviceDriver.h:197,204): y = a*x (+ b*y). */
+int cct_hip_math_saxpy(size_t n, float alpha, const float *x, float *y);
+int cct_hip_math_saxpby(size_t n, float alpha, const float *x, float beta, float *y);
+/* DeviceDriver::L1_update (src/sched/DeviceDriver.h:114-117). */
+int cct_hip_L1_update(int n, float *gradient, float lambda, const float *model);
+/* SGDGradientUpdater::update (src/algorithms/GradientUpdater.h:154-193) in one kernel:
+ * g += lambda*w (or lambda*sign(w) when l1), h = stepsize*g + momentum*h, w -= h. */
+int cct_hip_sgd_update(size_t n, float *model, float *gradient, float *history, float stepsize,
+                       float momentum, float lambda, int l1);
+/* DeviceDriver::sconstant_initialize (src/sched/DeviceDriver.h:258-260). */
+int cct_hip_sconstant_initialize(float *arr, size_t n, float value);
+/* DeviceDriver::rand_uint_initialize (src/sched/DeviceDriver.h:250-252) after init_rng(seed):
+ * counter-based generator, word i of call c depends only on (seed, c, i). */
+int cct_hip_init_rng(int random_seed);
+int cct_hip_rand_uint_initialize(unsigned int *buf, int n);
+
+/* ---- convolution / FC bias --------------------------------------------------------------- */
+/* DeviceDriver::forward_bias (src/sched/DeviceDriver.h:124-127): out[b][d][fmap] += bias[d]. */
+int cct_hip_forward_bias(const float *bias, float *out, int fmap_size, int depth, int batch_size);
+/* DeviceDriver::backward_bias (src/sched/DeviceDriver.h:129-133): bias_grad[d] = sum_b sum_fmap. */
+int cct_hip_backward_bias(float *bias_grad, const float *out_grad, int fmap_size, int depth,
+                          int batch_size);
+/* DeviceDriver::backward_bias_fc (src/sched/DeviceDriver.h:135-138): bias[d] = sum_b out[b][d]. */
+int cct_hip_backward_bias_fc(float *bias_grad, const float *out_grad, int D, int B);
+
+/* ---- elementwise / pooling / loss (the closed set of parallel_map UDF pairs the reference
+ *      instantiates, src/sched/DeviceDriver_CPU.cpp:725-784, as named kernels) ------------- */
+/* parallel_map<_f_src_to_dst_relu_forward,_f_relu_forward>, src/kernels/relu.hxx:10-28. */
+int cct_hip_relu_forward(float *out, const float *in, size_t n);
+/* parallel_map<_f_src_to_dst_relu_backward,_f_relu_backward>, src/kernels/relu.hxx:30-45. */
+int cct_hip_relu_backward(float *in_grad, const float *out_grad, const float *in_data, size_t n);
+/* DeviceDriver::maxpool_forward/backward, src/sched/DeviceDriver.h:149-156. dst is overwritten
+ * (no -FLT_MAX pre-fill needed); backward overwrites in_grad (no zero fill needed). */
+int cct_hip_maxpool_forward(float *out, const float *in, const cct_pool_args *args);
+int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_pool_args *args);
+/* DeviceDriver::lrn_forward/lrn_backward, src/sched/DeviceDriver.h:140-147. */
+int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args *args,
+                        const cct_lrn_forward_normalize_args *args2);
+int cct_hip_lrn_backward(float *in_grad, const float *out_grad, const cct_lrn_backward_args *args);
+/* parallel_map<_f_src_to_dst_dropout_forward,_f_dropout_forward_train>,
+ * src/kernels/dropout.hxx:20-32: out = in * (mask > threshold) * scale (in place allowed). */
+int cct_hip_dropout_forward_train(float *out, const float *in, const unsigned int *mask,
+                                  float scale, unsigned int threshold, size_t n);
+/* parallel_map<_f_src_to_dst_softmax_forward,_f_softmax_forward>, src/kernels/softmax.hxx:19-60.
+ * labels: device floats, one per image. loss_sum: device float, overwritten with the batch sum. */
+int cct_hip_softmax_loss_forward(float *prob, const float *in, const float *labels,
+                                 float *loss_sum, int len_per_image, int batch);
+/* parallel_map<_f_src_to_dst_softmax_backward,_f_softmax_backward>, src/kernels/softmax.hxx:62-81:
+ * in_grad = (prob - onehot(label)) / batch / spatial. */
+int cct_hip_softmax_loss_backward(float *in_grad, const float *prob, const float *labels,
+                                  int len_per_image, int batch, int spatial);
+
+/* ---- timing on the library's stream (used by the harness; hipEvent based) ---------------- */
+int cct_hip_timer_create(void **timer);
+int cct_hip_timer_destroy(void *timer);
+int cct_hip_timer_start(void *timer);
+int cct_hip_timer_stop(void *timer);
+/* Waits for the stop event; milliseconds between start and stop. */
+int cct_hip_timer_elapsed_ms(void *timer, float *ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CCT_HIP_H */

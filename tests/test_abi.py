@@ -1,0 +1,51 @@
+"""CPU-side checks of the drop-in boundary: the shared library loads without a GPU and exports
+every symbol that include/cct_hip.h declares; argument structs have the reference's layout."""
+import ctypes as C
+import os
+import re
+
+from conftest import ROOT
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "cct_hip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cct_hip_[a-zA-Z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from caffecontroll_amd import _lib
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 40
+    for n in names:
+        assert hasattr(lib, n), "missing export: " + n
+    # the ctypes prototype table covers the header, nothing more, nothing less
+    assert sorted(_lib.PROTOTYPES) == names
+
+
+def test_struct_layouts_match_reference_headers():
+    from caffecontroll_amd import _lib
+    # struct PMapHelper: 18 size_t (src/sched/DeviceHeader.h:25-35)
+    assert C.sizeof(_lib.PMapHelper) == 18 * 8
+    assert [f[0] for f in _lib.PMapHelper._fields_][:8] == ["dR", "dC", "dD", "dB", "sR", "sC", "sD", "sB"]
+    assert _lib.PMapHelper.stride.offset == 16 * 8 and _lib.PMapHelper.padding.offset == 17 * 8
+    # struct _inverse_lower_cube_arg_helper: 9 size_t (src/kernels/lowering.h:22-32)
+    assert C.sizeof(_lib.InverseLowerCubeArgs) == 9 * 8
+    # struct _pool_forward_arg_helper: 8 int + pointer (src/kernels/pool.h:7-17)
+    assert C.sizeof(_lib.PoolArgs) == 8 * 4 + 8 and _lib.PoolArgs.max_index.offset == 32
+    # lrn helpers (src/kernels/lrn.h:7-35)
+    assert C.sizeof(_lib.LrnForwardArgs) == 6 * 4 + 8
+    assert C.sizeof(_lib.LrnForwardNormalizeArgs) == 16
+    assert C.sizeof(_lib.LrnBackwardArgs) == 8 * 4 + 3 * 8
+
+
+def test_host_helpers_fill_structs_like_the_connector():
+    from caffecontroll_amd.driver import conv_pmap, lift_args, remap_pmap
+    a = conv_pmap(256, 96, 27, 5, 1, 2)
+    assert (a.dR, a.dC, a.sR, a.sC, a.sD, a.sB) == (2400, 186624, 27, 27, 96, 256)
+    assert (a.kR, a.kC, a.kD, a.kB, a.stride, a.padding, a.sBR) == (5, 5, 96, 1, 1, 2, 16)
+    l = lift_args(256, 3, 227, 11, 4, 0)
+    assert (l.data_output_width, l.kernel_size, l.stride, l.iR, l.iD, l.iB) == (55, 11, 4, 227, 3, 256)
+    r = remap_pmap(27, 27, 256, 8)
+    assert (r.sD, r.sB, r.sBR) == (256, 8, 16)
