@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Benchmark of the convolution training hot path on one MI355X.
+
+Workload (BASELINE.json configs[1]): AlexNet conv2 shape, ungrouped -- batch 256, input 96x27x27
+N(0,1), 256 filters 5x5, stride 1, pad 2, weights N(0,0.01), bias 0.1, output gradient N(0,1).
+One step = ConvolutionBridge forward + backward (lower, forward GEMM with remap+bias epilogue,
+out-grad remap, data-gradient GEMM, lift + bias gradient, weight-gradient GEMM) on tensors that
+are already resident in HBM.  Prints ONE JSON line.
+
+    python bench.py --gpus 1 --steps 20 --warmup 5
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+CONFIGS = {
+    # name: (b, d, n, k, s, p, o)
+    "lenet_conv1": (64, 1, 28, 5, 1, 0, 20),
+    "alexnet_conv2": (256, 96, 27, 5, 1, 2, 256),
+    "alexnet_conv1": (256, 3, 227, 11, 4, 0, 96),
+}
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def synth(cfg, seed, torch):
+    """Seeded synthetic tensors of BASELINE.json's configs, generated on the host and uploaded."""
+    import numpy as np
+    b, d, n, k, s, p, o = CONFIGS[cfg]
+    m = (n + 2 * p - k) // s + 1
+    rng = np.random.default_rng(seed)
+    if cfg == "alexnet_conv1":
+        x = rng.uniform(0, 255, (b, d, n, n)).astype(np.float32)
+        x -= np.array([104, 117, 123], np.float32)[None, :, None, None]
+        bias = np.zeros(o, np.float32)
+    elif cfg == "lenet_conv1":
+        x = rng.uniform(0, 1, (b, d, n, n)).astype(np.float32)
+        bias = np.zeros(o, np.float32)
+    else:
+        x = rng.standard_normal((b, d, n, n), dtype=np.float32)
+        bias = np.full(o, 0.1, np.float32)
+    w = (rng.standard_normal((o, d, k, k), dtype=np.float32) * np.float32(0.01))
+    og = rng.standard_normal((b, o, m, m), dtype=np.float32)
+    return x, w, bias, og
+
+
+def cpu_baseline(cfg, seed):
+    """The CPU oracle (a port of CcT's CPUDriver path, GEMMs through OpenBLAS when found) timed on
+    this host with CcT's own threading policy: P = min(2^floor(log2 cores), b) batch partitions,
+    one BLAS thread each (src/DeepNet.h:716-725, 1102-1105)."""
+    from concurrent.futures import ThreadPoolExecutor
+    import numpy as np
+    from oracle import cct_oracle as O
+    b, d, n, k, s, p, o = CONFIGS[cfg]
+    cores = os.cpu_count() or 1
+    try:
+        cores = min(cores, len(os.sched_getaffinity(0)))
+    except Exception:
+        pass
+    if os.environ.get("OMP_NUM_THREADS", "").isdigit():
+        cores = min(cores, int(os.environ["OMP_NUM_THREADS"]))
+    P = min(2 ** int(math.floor(math.log2(max(cores, 1)))), b)
+    blas = O.bind_openblas(1)
+    x, w, bias, og = synth(cfg, seed, None)
+    bounds = [(i * b // P, (i + 1) * b // P) for i in range(P)]
+
+    def part(lohi):
+        lo, hi = lohi
+        _, low = O.conv_forward(x[lo:hi], w, bias, k, s, p)
+        O.conv_backward((hi - lo, d, n, n), w, og[lo:hi], low, k, s, p)
+
+    def run():
+        t0 = time.perf_counter()
+        with ThreadPoolExecutor(P) as ex:
+            list(ex.map(part, bounds))
+        return time.perf_counter() - t0
+
+    warm = run()
+    reps = max(1, min(3, int(20.0 / max(warm, 1e-3))))
+    times = sorted(run() for _ in range(reps))
+    med = times[len(times) // 2]
+    O.unbind_openblas()
+    return {
+        "value": b / med, "unit": "images/sec", "cores": P, "kind": "port",
+        "sample": "full %s workload (b=%d), 1 warm-up + %d timed passes, median; %d batch partitions x 1 BLAS "
+                  "thread; sgemm=%s" % (cfg, b, reps, P, "OpenBLAS (scipy bundle)" if blas else "plain loops"),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="alexnet_conv2", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--unfused", action="store_true", help="staged forward (GEMM, remap, bias) and separate bias gradient")
+    ap.add_argument("--no-data-grad", action="store_true", help="first-layer mode: skip data-gradient GEMM and lift")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (batch sharding over several GPUs is a design note, "
+              "not built); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from caffecontroll_amd import HIPDriver, load
+    from caffecontroll_amd.bridges import ConvolutionLayer
+
+    load()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    cfg = args.workload
+    b, d, n, k, s, p, o = CONFIGS[cfg]
+    m = (n + 2 * p - k) // s + 1
+    seed = 1234 + sorted(CONFIGS).index(cfg)
+    drv = HIPDriver(0)
+    drv.set_stream(torch.cuda.current_stream().cuda_stream)
+
+    x, w, bias, og = synth(cfg, seed, torch)
+    in_data = torch.from_numpy(x).cuda()
+    in_grad = torch.empty_like(in_data)
+    out_data = torch.empty((b, o, m, m), device="cuda")
+    out_grad = torch.from_numpy(og).cuda()
+    layer = ConvolutionLayer(b, d, n, k, s, p, o, in_data, in_grad, out_data, out_grad)
+    drv.memcpy(layer.model_ptr(), w.ctypes.data, w.nbytes, 0)
+    drv.memcpy(layer.bias_ptr(), bias.ctypes.data, bias.nbytes, 0)
+    need_dgrad = not args.no_data_grad
+    layer.set_options(fused=not args.unfused, profile=True, needs_backward_grad=need_dgrad)
+
+    def step():
+        layer.forward()
+        layer.backward(with_update=False)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    stage_sum = {}
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+        # reading the stage events waits for the step's last kernel (one host sync per step,
+        # as a training loop that reads its loss does)
+        for name, ms in layer.stage_ms().items():
+            stage_sum[name] = stage_sum.get(name, 0.0) + ms
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    stages = {name: v / args.steps for name, v in stage_sum.items() if v > 0}
+
+    # algorithmic work per launch
+    lower_bytes = 4.0 * (b * d * n * n + b * m * m * k * k * d)
+    gemm_flop = 2.0 * o * (b * m * m) * (k * k * d)
+    per_stage = {}
+    for name, ms in stages.items():
+        ent = {"ms": round(ms, 4)}
+        if name in ("GEMM", "GEMM Data", "GEMM Wghts"):
+            ent["tflops"] = round(gemm_flop / ms / 1e9, 2)
+            ent["frac_fp32_mfma_peak"] = round(gemm_flop / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)
+        elif name in ("Lower Cube", "Inverse Lwr"):
+            ent["gbs"] = round(lower_bytes / ms / 1e6, 1)
+            ent["frac_hbm_peak"] = round(lower_bytes / ms / 1e6 / PEAK_HBM_GBS, 4)
+        per_stage[name] = ent
+    # dominant kernel = the GEMM instance with the longest average launch
+    gemm_names = [g for g in ("GEMM", "GEMM Data", "GEMM Wghts") if g in stages]
+    dom = max(gemm_names, key=lambda g: stages[g])
+    kernel_of = {"GEMM": "gemm_kernel<256x128x16, A k-contig, B k-contig> (forward, conv epilogue)",
+                 "GEMM Data": "gemm_kernel<256x128x16, A m-contig, B n-contig> (data gradient)",
+                 "GEMM Wghts": "gemm_kernel<256x128x16, A k-contig, B n-contig> split-K (weight gradient)"}
+    achieved = gemm_flop / stages[dom] / 1e9
+    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                "kernel": kernel_of[dom], "stage": dom, "flop_per_launch": gemm_flop,
+                "avg_launch_ms": round(stages[dom], 4)}
+
+    result = {
+        "metric": "images/sec conv fwd+bwd (1 GPU)", "value": round(b * args.steps / elapsed, 1),
+        "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "%s: conv fwd+bwd b=%d d=%d n=%d k=%d s=%d p=%d o=%d%s%s" % (
+            cfg, b, d, n, k, s, p, o, "" if need_dgrad else " (no data gradient)",
+            " (staged forward)" if args.unfused else "")},
+        "roofline": roofline, "stages": per_stage,
+    }
+    if not args.no_cpu_baseline:
+        layer.close()
+        del in_data, in_grad, out_data, out_grad
+        result["cpu_baseline"] = cpu_baseline(cfg, seed)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

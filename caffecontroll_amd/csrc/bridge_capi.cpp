@@ -1,0 +1,114 @@
+// C entry points over the C++ host layer (see include/cct_bridge.h).
+#include <string>
+
+#include "../../include/cct_bridge.h"
+#include "host/ConvolutionBridge.h"
+#include "host/ParallelizedBridge.h"
+
+using namespace cct;
+
+namespace {
+
+void fill_solver(cnn::SolverParameter &s, const cct_solver_param *p) {
+  if (!p) return;
+  s.base_lr_ = p->base_lr; s.momentum_ = p->momentum; s.gamma_ = p->gamma; s.power_ = p->power;
+  s.weight_decay_ = p->weight_decay; s.stepsize_ = p->stepsize; s.max_iter_ = p->max_iter;
+  s.random_seed_ = p->random_seed;
+  if (p->lr_policy) s.lr_policy_ = p->lr_policy;
+  if (p->regularization_type) s.regularization_type_ = p->regularization_type;
+}
+
+}  // namespace
+
+struct cct_conv_bridge {
+  HIPDriver driver;
+  cnn::LayerParameter layer_param;
+  cnn::SolverParameter solver_param;
+  Layer<float> *in_layer = nullptr, *out_layer = nullptr;
+  ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *pbridge = nullptr;
+};
+
+extern "C" {
+
+int cct_conv_bridge_create(cct_conv_bridge **out, int b, int d, int n, const cct_conv_param *conv,
+                           const cct_solver_param *solver, float *in_data, float *in_grad, float *out_data,
+                           float *out_grad) {
+  if (!out || !conv || b <= 0 || d <= 0 || n <= 0 || conv->kernel_size <= 0 || conv->stride <= 0 ||
+      conv->num_output <= 0 || n + 2 * conv->pad < conv->kernel_size || !in_data || !out_data)
+    return CCT_HIP_EINVAL;
+  cct_conv_bridge *h = new cct_conv_bridge;
+  const int k = conv->kernel_size, s = conv->stride, p = conv->pad, o = conv->num_output;
+  const int m = (n + 2 * p - k) / s + 1;
+  cnn::ConvolutionParameter &cp = h->layer_param.convolution_param_;
+  cp.num_output_ = o; cp.kernel_size_ = k; cp.stride_ = s; cp.pad_ = p; cp.bias_term_ = conv->bias_term != 0;
+  h->layer_param.blobs_lr_[0] = conv->lr_mult_weights; h->layer_param.blobs_lr_[1] = conv->lr_mult_bias;
+  h->layer_param.weight_decay_[0] = conv->decay_mult_weights; h->layer_param.weight_decay_[1] = conv->decay_mult_bias;
+  fill_solver(h->solver_param, solver);
+  h->in_layer = new Layer<float>(new LogicalCube<float>(in_data, n, n, d, b),
+                                 new LogicalCube<float>(in_grad, n, n, d, b));
+  h->out_layer = new Layer<float>(new LogicalCube<float>(out_data, m, m, o, b),
+                                  new LogicalCube<float>(out_grad, m, m, o, b));
+  h->pbridge = new ParallelizedBridge<float, ConvolutionBridge, HIPDriver>(
+      h->in_layer, h->out_layer, &h->layer_param, &h->solver_param, &h->driver, 1, 1);
+  *out = h;
+  return 0;
+}
+
+int cct_conv_bridge_destroy(cct_conv_bridge *h) {
+  if (!h) return 0;
+  delete h->pbridge;
+  delete h->in_layer;
+  delete h->out_layer;
+  delete h;
+  return 0;
+}
+
+int cct_conv_bridge_set_options(cct_conv_bridge *h, int fused, int profile, int needs_backward_grad) {
+  if (!h) return CCT_HIP_EINVAL;
+  h->pbridge->sub_bridge()->set_fused(fused != 0);
+  h->pbridge->sub_bridge()->set_stage_profiling(profile != 0);
+  h->pbridge->needs_to_calc_backward_grad = needs_backward_grad != 0;
+  h->pbridge->sub_bridge()->needs_to_calc_backward_grad = needs_backward_grad != 0;
+  return 0;
+}
+
+float *cct_conv_bridge_model(cct_conv_bridge *h) { return h->pbridge->p_model_cube->get_p_data(); }
+float *cct_conv_bridge_bias(cct_conv_bridge *h) {
+  return h->pbridge->p_bias_cube ? h->pbridge->p_bias_cube->get_p_data() : nullptr;
+}
+float *cct_conv_bridge_model_grad(cct_conv_bridge *h) { return h->pbridge->p_model_grad->get_p_data(); }
+float *cct_conv_bridge_bias_grad(cct_conv_bridge *h) {
+  return h->pbridge->p_bias_grad ? h->pbridge->p_bias_grad->get_p_data() : nullptr;
+}
+float *cct_conv_bridge_lowered(cct_conv_bridge *h) {
+  return h->pbridge->sub_bridge()->get_lowered_cube()->get_p_data();
+}
+float *cct_conv_bridge_history(cct_conv_bridge *h) {
+  return h->pbridge->get_grad_updater()->get_p_history_updates_cube()->get_p_data();
+}
+
+int cct_conv_bridge_forward(cct_conv_bridge *h) {
+  if (!h) return CCT_HIP_EINVAL;
+  h->pbridge->forward();
+  return 0;
+}
+
+int cct_conv_bridge_backward(cct_conv_bridge *h, int with_update) {
+  if (!h) return CCT_HIP_EINVAL;
+  if (with_update) {
+    h->pbridge->backward();
+  } else {
+    h->pbridge->sub_bridge()->needs_to_calc_backward_grad = h->pbridge->needs_to_calc_backward_grad;
+    h->pbridge->sub_bridge()->backward();
+  }
+  return 0;
+}
+
+int cct_conv_bridge_stage_ms(cct_conv_bridge *h, float ms[CCT_CONV_STAGE_COUNT]) {
+  if (!h || !ms) return CCT_HIP_EINVAL;
+  static_assert(CCT_CONV_STAGE_COUNT == STAGE_COUNT, "stage tables out of sync");
+  for (int i = 0; i < STAGE_COUNT; ++i) ms[i] = h->pbridge->sub_bridge()->stage_ms(i);
+  return 0;
+}
+
+}  // extern "C"

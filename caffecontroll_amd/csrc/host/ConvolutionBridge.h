@@ -1,0 +1,266 @@
+// Convolution operator for the HIP driver: lowering -> GEMM -> (remap, bias) forward;
+// bias gradient, data-gradient GEMM -> lifting, weight-gradient GEMM backward.
+//
+// Counterpart of ConvolutionBridge<float, Layout_CRDB, float, Layout_CRDB, DriverClass>
+// (src/bridges/ConvolutionBridge.h:74-215, _impl.hxx:13-226, 284-520, 541-796).  It follows the
+// reference's *batched* branch (the one CPUDriver takes, _impl.hxx:294-373 and 551-628): the
+// whole batch is lowered once into a (k*k*d) x (m*m*b) buffer that the backward pass reuses,
+// rather than the per-image loop the reference runs for non-CPU drivers (:375-520, 630-796).
+// Deliberate departures, none of which changes a result:
+//   * the output-gradient cube is permuted into a scratch cube, not in place (:604);
+//   * by default the forward GEMM writes [b][o][m*m] and adds the bias in its epilogue instead
+//     of running remap_output and the bias map as separate passes (set_fused(false) restores
+//     the staged sequence);
+//   * the bias gradient is reduced in the same launch as the lifting kernel.
+#pragma once
+#include <cstdio>
+#include <cstdlib>
+#include <string>
+
+#include "AbstractBridge.h"
+#include "Connector.h"
+#include "Kernel.h"
+
+namespace cct {
+
+// Stage labels of the reference's detailed profiling output (_impl.hxx:325-366, 601-623).
+enum ConvStage {
+  STAGE_LOWER = 0, STAGE_GEMM, STAGE_REMAP, STAGE_BIAS,            // forward
+  STAGE_BW_BIAS, STAGE_BW_REMAP, STAGE_GEMM_DATA, STAGE_INVERSE_LOWER, STAGE_GEMM_WEIGHTS,  // backward
+  STAGE_COUNT
+};
+
+template <typename DataType, typename DriverClass>
+class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
+  typedef AbstractBridge<DataType, DriverClass> Base;
+
+ public:
+  using Base::iR; using Base::iC; using Base::iD; using Base::iB;
+  using Base::oR; using Base::oC; using Base::oD; using Base::oB;
+  using Base::needs_to_calc_backward_grad;
+  using Base::layer_param; using Base::solver_param; using Base::p_driver;
+  using Base::p_input_layer; using Base::p_output_layer;
+  using Base::report_forward_history; using Base::report_backward_updateweight_history;
+  typedef Layer<DataType> InputLayerType;
+  typedef Layer<DataType> OutputLayerType;
+  typedef LogicalCube<DataType> LogicalCubeType;
+
+  const size_t K;
+  const size_t num_output_features;
+  const size_t stride;
+  const size_t padding;
+  const bool bias_term;
+  const cnn::FillerParameter weight_filler;
+  const cnn::FillerParameter bias_filler;
+
+  LogicalCubeType *p_model_cube;  // [o][d][k][k] == GEMM matrix [o x k*k*d]
+  LogicalCubeType *p_bias_cube;   // [o]
+
+  ConvolutionBridge(InputLayerType *const _p_input_layer, OutputLayerType *const _p_output_layer,
+                    const cnn::LayerParameter *const _layer_param,
+                    const cnn::SolverParameter *const _solver_param, DriverClass *const _p_driver)
+      : Base(_p_input_layer, _p_output_layer, _layer_param, _solver_param, _p_driver),
+        K(_layer_param->convolution_param().kernel_size()), num_output_features(_p_output_layer->dD),
+        stride(_layer_param->convolution_param().stride()), padding(_layer_param->convolution_param().pad()),
+        bias_term(_layer_param->convolution_param().bias_term()),
+        weight_filler(_layer_param->convolution_param().weight_filler()),
+        bias_filler(_layer_param->convolution_param().bias_filler()), p_model_cube(nullptr),
+        p_bias_cube(nullptr), p_bias_gradient_cube(nullptr) {
+    if (oR != (iR + 2 * padding - K) / stride + 1 || oC != (iC + 2 * padding - K) / stride + 1 || iB != oB ||
+        num_output_features != oD || iR != iC) {
+      std::fprintf(stderr, "ConvolutionBridge: inconsistent layer shapes\n");
+      std::abort();
+    }
+    // cubes read outside the bridge (model / gradients), device resident
+    p_model_cube = new LogicalCubeType(K, K, iD, num_output_features, p_driver);
+    initialize_logical_cube(p_model_cube, weight_filler);
+    p_model_gradient_cube = new LogicalCubeType(K, K, iD, num_output_features, p_driver);
+    DeviceMemoryPointer mg = p_model_gradient_cube->get_device_pointer(p_driver);
+    p_driver->sconstant_initialize(&mg, DataType(0.));
+    if (bias_term) {
+      p_bias_cube = new LogicalCubeType(1, 1, num_output_features, 1, p_driver);
+      initialize_logical_cube(p_bias_cube, bias_filler);
+      p_bias_gradient_cube = new LogicalCubeType(1, 1, num_output_features, 1, p_driver);
+      DeviceMemoryPointer bg = p_bias_gradient_cube->get_device_pointer(p_driver);
+      p_driver->sconstant_initialize(&bg, DataType(0.));
+    }
+    // cubes used inside the bridge only; sized for the whole batch
+    p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
+    p_backward_inputgrad = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
+    p_staging_cube = new LogicalCubeType(oR, oC, oD, oB, p_driver);  // [o][b][m*m] view of output / out-grad
+
+    LogicalCubeType lowered_forward_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
+    LogicalCubeType lowered_forward_output(p_staging_cube->get_p_data(), num_output_features, oR * oC * iB, 1, 1);
+    LogicalCubeType dummy_data_cube(nullptr, iR, iC, iD, iB);
+    p_forward_lower_connector =
+        new Connector<DataType, DriverClass>(&dummy_data_cube, p_forward_lowered_data, K, padding, stride, p_driver);
+    p_forward_gemm_kernel = new Kernel<DataType, KernelConfig_GEMM_NOTRANS_TRANS_NO_DIM_FLIP, DriverClass>(
+        &lowered_forward_model, p_forward_lowered_data, &lowered_forward_output, p_driver);
+    p_backward_gemm_updateweight_kernel = new Kernel<DataType, KernelConfig_GEMM_NOTRANS_NOTRANS_DIM_FLIP, DriverClass>(
+        &lowered_forward_output, p_forward_lowered_data, &lowered_forward_model, p_driver);
+    p_backward_gemm_updategrad_kernel = new Kernel<DataType, KernelConfig_GEMM_TRANS_NOTRANS, DriverClass>(
+        &lowered_forward_model, &lowered_forward_output, p_backward_inputgrad, p_driver);
+    for (int i = 0; i < STAGE_COUNT; ++i) { timers_[i] = nullptr; stage_ms_[i] = 0.f; }
+  }
+
+  ~ConvolutionBridge() {
+    for (int i = 0; i < STAGE_COUNT; ++i)
+      if (timers_[i]) cct_hip_timer_destroy(timers_[i]);
+    delete p_model_cube;
+    delete p_model_gradient_cube;
+    delete p_bias_cube;
+    delete p_bias_gradient_cube;
+    delete p_forward_lowered_data;
+    delete p_backward_inputgrad;
+    delete p_staging_cube;
+    delete p_forward_lower_connector;
+    delete p_forward_gemm_kernel;
+    delete p_backward_gemm_updateweight_kernel;
+    delete p_backward_gemm_updategrad_kernel;
+  }
+
+  LogicalCubeType *get_model_cube() override { return p_model_cube; }
+  LogicalCubeType *get_bias_cube() override { return p_bias_cube; }
+  LogicalCubeType *get_model_grad_cube() override { return p_model_gradient_cube; }
+  LogicalCubeType *get_bias_grad_cube() override { return p_bias_gradient_cube; }
+  LogicalCubeType *get_lowered_cube() { return p_forward_lowered_data; }
+
+  void set_fused(bool on) { fused_ = on; }
+  // per-stage hipEvent timing (the reference's -D_DETAILED_PROFILING stage prints)
+  void set_stage_profiling(bool on) { profile_ = on; }
+  float stage_ms(int stage) {
+    float ms = 0.f;
+    if (timers_[stage] && stage_ran_[stage]) cct_hip_timer_elapsed_ms(timers_[stage], &ms);
+    return ms;
+  }
+
+  // (1) input --lowering--> lowered  (2) model x lowered^T --> output  (3) remap + bias
+  void forward() override {
+    report_forward_history.reset();
+    for (int i = STAGE_LOWER; i <= STAGE_BIAS; ++i) stage_ran_[i] = false;
+    LogicalCubeType *input_d_cube = p_input_layer->p_data_cube;
+    LogicalCubeType *output_d_cube = p_output_layer->p_data_cube;
+    LogicalCubeType lowered_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
+
+    begin(STAGE_LOWER);
+    p_forward_lower_connector->lower_cube(input_d_cube, p_forward_lowered_data);
+    end(STAGE_LOWER);
+    if (fused_) {
+      begin(STAGE_GEMM);
+      p_driver->sgemm_conv_forward((int)num_output_features, (int)iB, (int)(oR * oC), (int)(K * K * iD),
+                                   p_model_cube->get_p_data(), p_forward_lowered_data->get_p_data(),
+                                   bias_term ? p_bias_cube->get_p_data() : nullptr, output_d_cube->get_p_data());
+      end(STAGE_GEMM);
+    } else {
+      LogicalCubeType lowered_output(p_staging_cube->get_p_data(), num_output_features, oR * oC * iB, 1, 1);
+      begin(STAGE_GEMM);
+      p_forward_gemm_kernel->compute(&lowered_model, p_forward_lowered_data, &lowered_output);
+      end(STAGE_GEMM);
+      begin(STAGE_REMAP);
+      p_forward_lower_connector->remap_output(*output_d_cube, *p_staging_cube, num_output_features, iB);
+      end(STAGE_REMAP);
+      if (bias_term) {
+        begin(STAGE_BIAS);
+        DeviceMemoryPointer output = output_d_cube->get_device_pointer(p_driver);
+        DeviceMemoryPointer bias = p_bias_cube->get_device_pointer(p_driver);
+        p_driver->forward_bias(&bias, &output, (int)(oR * oC), (int)oD, (int)iB);
+        end(STAGE_BIAS);
+      }
+    }
+    report_forward_history.end();
+  }
+
+  // bias gradient; remap of the output gradient; data-gradient GEMM + lifting (if needed);
+  // weight-gradient GEMM against the lowered data kept from forward()
+  void backward() override {
+    report_backward_updateweight_history.reset();
+    for (int i = STAGE_BW_BIAS; i < STAGE_COUNT; ++i) stage_ran_[i] = false;
+    LogicalCubeType *output_g_cube = p_output_layer->p_gradient_cube;
+    LogicalCubeType *input_g_cube = p_input_layer->p_gradient_cube;
+    LogicalCubeType lowered_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
+    LogicalCubeType lowered_model_grad(p_model_gradient_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
+    LogicalCubeType lowered_outputgrad(p_staging_cube->get_p_data(), num_output_features, oR * oC * iB, 1, 1);
+    DeviceMemoryPointer og = output_g_cube->get_device_pointer(p_driver);
+
+    const bool fuse_bias_into_lift = bias_term && needs_to_calc_backward_grad && fused_;
+    if (bias_term && !fuse_bias_into_lift) {
+      begin(STAGE_BW_BIAS);
+      DeviceMemoryPointer bias = p_bias_gradient_cube->get_device_pointer(p_driver);
+      p_driver->backward_bias(&bias, &og, (int)(oR * oC), (int)oD, (int)iB);
+      end(STAGE_BW_BIAS);
+    }
+    begin(STAGE_BW_REMAP);
+    p_forward_lower_connector->remap_output(*p_staging_cube, *output_g_cube, oB, num_output_features);
+    end(STAGE_BW_REMAP);
+    if (needs_to_calc_backward_grad) {
+      begin(STAGE_GEMM_DATA);
+      p_backward_gemm_updategrad_kernel->compute(&lowered_model, &lowered_outputgrad, p_backward_inputgrad);
+      end(STAGE_GEMM_DATA);
+      begin(STAGE_INVERSE_LOWER);
+      if (fuse_bias_into_lift) {
+        DeviceMemoryPointer input = input_g_cube->get_device_pointer(p_driver);
+        DeviceMemoryPointer lowered_grad = p_backward_inputgrad->get_device_pointer(p_driver);
+        DeviceMemoryPointer bias = p_bias_gradient_cube->get_device_pointer(p_driver);
+        p_driver->inverse_lower_cube_bias_backward(&input, &lowered_grad, p_forward_lower_connector->inverse_args(),
+                                                   &bias, &og, (int)(oR * oC), (int)oD, (int)iB);
+      } else {
+        p_forward_lower_connector->inverse_lower_cube(p_backward_inputgrad, input_g_cube);
+      }
+      end(STAGE_INVERSE_LOWER);
+    }
+    begin(STAGE_GEMM_WEIGHTS);
+    p_backward_gemm_updateweight_kernel->alpha = 1.0;
+    p_backward_gemm_updateweight_kernel->beta = 0.0;
+    p_backward_gemm_updateweight_kernel->compute(&lowered_outputgrad, p_forward_lowered_data, &lowered_model_grad);
+    end(STAGE_GEMM_WEIGHTS);
+    report_backward_updateweight_history.end();
+  }
+
+ protected:
+  LogicalCubeType *p_model_gradient_cube;
+  LogicalCubeType *p_bias_gradient_cube;
+  LogicalCubeType *p_forward_lowered_data;
+  LogicalCubeType *p_backward_inputgrad;
+  LogicalCubeType *p_staging_cube;
+  Connector<DataType, DriverClass> *p_forward_lower_connector;
+  Kernel<DataType, KernelConfig_GEMM_NOTRANS_TRANS_NO_DIM_FLIP, DriverClass> *p_forward_gemm_kernel;
+  Kernel<DataType, KernelConfig_GEMM_NOTRANS_NOTRANS_DIM_FLIP, DriverClass> *p_backward_gemm_updateweight_kernel;
+  Kernel<DataType, KernelConfig_GEMM_TRANS_NOTRANS, DriverClass> *p_backward_gemm_updategrad_kernel;
+
+  // Fillers, src/bridges/ConvolutionBridge_impl.hxx:250-267.
+  void initialize_logical_cube(const LogicalCubeType *cube, const cnn::FillerParameter &filler_param) {
+    DeviceMemoryPointer data = cube->get_device_pointer(p_driver);
+    const std::string &type = filler_param.type();
+    if (type == "constant") {
+      p_driver->sconstant_initialize(&data, (DataType)filler_param.value());
+    } else if (type == "xavier") {
+      p_driver->sinitialize_xavier(&data, cube->B, solver_param->random_seed());
+    } else if (type == "bernoulli") {
+      p_driver->sbernoulli_initialize(&data, (DataType)filler_param.value(), solver_param->random_seed());
+    } else if (type == "gaussian") {
+      p_driver->sgaussian_initialize(&data, (DataType)filler_param.mean(), (DataType)filler_param.std(),
+                                     solver_param->random_seed());
+    } else {
+      std::fprintf(stderr, "ERROR! INITIALIZATION TYPE NOT SUPPORTED: %s\n", type.c_str());
+      std::abort();
+    }
+  }
+
+ private:
+  bool fused_ = true, profile_ = false;
+  void *timers_[STAGE_COUNT];
+  bool stage_ran_[STAGE_COUNT] = {};
+  float stage_ms_[STAGE_COUNT];
+  void begin(int s) {
+    if (!profile_) return;
+    if (!timers_[s]) cct_hip_timer_create(&timers_[s]);
+    cct_hip_timer_start(timers_[s]);
+  }
+  void end(int s) {
+    if (!profile_) return;
+    cct_hip_timer_stop(timers_[s]);
+    stage_ran_[s] = true;
+  }
+};
+
+}  // namespace cct

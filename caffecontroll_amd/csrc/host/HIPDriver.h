@@ -1,0 +1,240 @@
+// HIPDriver: the MI355X counterpart of the reference's CPUDriver / GPUDriver
+// (src/sched/DeviceDriver.h:56-274, src/sched/DeviceDriver_CPU.h:24-111).  Same member names
+// and argument meaning; every member forwards to the C ABI in include/cct_hip.h.
+//
+// Error behaviour follows src/sched/DeviceDriver.h:48-51: members return void; on error the
+// message is printed and the process aborts (the reference asserts).
+//
+// The reference selects kernels with C function pointers as template arguments
+// (parallel_map<idx,func>).  The closed set of pairs it instantiates
+// (src/sched/DeviceDriver_CPU.cpp:725-784) is provided here as named members instead, one per
+// pair, so no device-side function pointers are needed.
+#pragma once
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <random>
+#include <vector>
+
+#include "../../../include/cct_hip.h"
+#include "DeviceMemoryPointer.h"
+
+namespace cct {
+
+typedef cct_pmap_helper PMapHelper;
+typedef cct_inverse_lower_cube_args _inverse_lower_cube_arg_helper;
+typedef cct_pool_args _pool_forward_arg_helper;
+typedef cct_pool_args _pool_backward_arg_helper;
+typedef cct_lrn_forward_args _lrn_forward_arg_helper;
+typedef cct_lrn_forward_normalize_args _lrn_forward_normalize_arg_helper;
+typedef cct_lrn_backward_args _lrn_backward_arg_helper;
+
+enum CBLAS_ORDER { CblasRowMajor = CCT_ROW_MAJOR, CblasColMajor = CCT_COL_MAJOR };
+enum CBLAS_TRANSPOSE { CblasNoTrans = CCT_NO_TRANS, CblasTrans = CCT_TRANS };
+
+class HIPDriver {
+ public:
+  explicit HIPDriver(int device_id = 0) { ok(cct_hip_init(device_id), "init"); }
+
+  // ---- pointers / memory (DeviceDriver.h:76-86) ----
+  void *choose_ptr(void *host, void *device) { (void)host; return device; }
+  DeviceMemoryPointer get_device_pointer(void *ptr, size_t size_in_byte) {
+    return DeviceMemoryPointer_Local_GPURAM(ptr, size_in_byte);
+  }
+  void malloc(DeviceMemoryPointer *dst) { ok(cct_hip_malloc(&dst->ptr, dst->size_in_byte), "malloc"); }
+  void free(DeviceMemoryPointer *dst) { ok(cct_hip_free(dst->ptr), "free"); dst->ptr = nullptr; }
+  // direction is taken from the two pointer types, as GPUDriver::memcpy does
+  void memcpy(DeviceMemoryPointer *dst, DeviceMemoryPointer *src) {
+    const bool dd = dst->type == DEVICEMEMORY_LOCAL_GPURAM, sd = src->type == DEVICEMEMORY_LOCAL_GPURAM;
+    if (!dd && !sd) { std::fprintf(stderr, "HIPDriver::memcpy: host to host copy\n"); std::abort(); }
+    const int kind = (dd && sd) ? 2 : dd ? 0 : 1;
+    ok(cct_hip_memcpy(dst->ptr, src->ptr, dst->size_in_byte, kind), "memcpy");
+  }
+  void memset(DeviceMemoryPointer *dst, const char value) {
+    ok(cct_hip_memset(dst->ptr, value, dst->size_in_byte), "memset");
+  }
+
+  // ---- lowering / lifting (DeviceDriver.h:100-122) ----
+  void lower_cube(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const PMapHelper args) {
+    ok(cct_hip_lower_cube((float *)dst->ptr, (const float *)src->ptr, &args), "lower_cube");
+  }
+  // pmap2d_read_coalesce<_fpmap_id,_fmap_remap>
+  void pmap2d_read_coalesce_remap(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const PMapHelper args) {
+    ok(cct_hip_remap((float *)dst->ptr, (const float *)src->ptr, &args), "remap");
+  }
+  void inverse_lower_cube(DeviceMemoryPointer *dst, DeviceMemoryPointer *src,
+                          const _inverse_lower_cube_arg_helper args) {
+    ok(cct_hip_inverse_lower_cube((float *)dst->ptr, (const float *)src->ptr, &args), "inverse_lower_cube");
+  }
+  void inverse_lower_cube_bias_backward(DeviceMemoryPointer *dst, DeviceMemoryPointer *src,
+                                        const _inverse_lower_cube_arg_helper args, DeviceMemoryPointer *bias,
+                                        DeviceMemoryPointer *out_grad, int fmap_size, int depth, int batch_size) {
+    ok(cct_hip_inverse_lower_cube_bias_backward((float *)dst->ptr, (const float *)src->ptr, &args,
+                                                (float *)bias->ptr, (const float *)out_grad->ptr, fmap_size,
+                                                depth, batch_size),
+       "inverse_lower_cube_bias_backward");
+  }
+
+  // ---- bias (DeviceDriver.h:124-138) ----
+  void forward_bias(DeviceMemoryPointer *bias, DeviceMemoryPointer *output, const int fmap_size,
+                    const int depth, const int batch_size) {
+    ok(cct_hip_forward_bias((const float *)bias->ptr, (float *)output->ptr, fmap_size, depth, batch_size),
+       "forward_bias");
+  }
+  void backward_bias(DeviceMemoryPointer *bias, DeviceMemoryPointer *output, const int fmap_size,
+                     const int depth, const int batch_size, const float *const device_ones = nullptr) {
+    (void)device_ones;  // the reference's gemv-with-ones vector is not needed
+    ok(cct_hip_backward_bias((float *)bias->ptr, (const float *)output->ptr, fmap_size, depth, batch_size),
+       "backward_bias");
+  }
+  void backward_bias_fc(DeviceMemoryPointer *bias, DeviceMemoryPointer *output, const int D, const int B,
+                        const float *const device_ones = nullptr) {
+    (void)device_ones;
+    ok(cct_hip_backward_bias_fc((float *)bias->ptr, (const float *)output->ptr, D, B), "backward_bias_fc");
+  }
+
+  // ---- pooling / LRN (DeviceDriver.h:140-156) ----
+  void lrn_forward(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const _lrn_forward_arg_helper args,
+                   const _lrn_forward_normalize_arg_helper args2) {
+    // argument order as the reference's call site: (input, output) -- LRNBridge_impl.hxx:103
+    ok(cct_hip_lrn_forward((float *)src->ptr, (const float *)dst->ptr, &args, &args2), "lrn_forward");
+  }
+  void lrn_backward(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const _lrn_backward_arg_helper args) {
+    // (input_grad, output_grad) -- LRNBridge_impl.hxx:168
+    ok(cct_hip_lrn_backward((float *)dst->ptr, (const float *)src->ptr, &args), "lrn_backward");
+  }
+  void maxpool_forward(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const _pool_forward_arg_helper args) {
+    ok(cct_hip_maxpool_forward((float *)dst->ptr, (const float *)src->ptr, &args), "maxpool_forward");
+  }
+  void maxpool_backward(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const _pool_backward_arg_helper args) {
+    // (output_grad, input_grad) -- CPUDriver::maxpool_backward reads dst and writes src
+    ok(cct_hip_maxpool_backward((float *)src->ptr, (const float *)dst->ptr, &args), "maxpool_backward");
+  }
+
+  // ---- the parallel_map pairs of the reference, by name ----
+  void relu_forward(DeviceMemoryPointer *dst, DeviceMemoryPointer *src) {
+    ok(cct_hip_relu_forward((float *)dst->ptr, (const float *)src->ptr, src->size_in_byte / sizeof(float)),
+       "relu_forward");
+  }
+  void relu_backward(DeviceMemoryPointer *in_grad, DeviceMemoryPointer *out_grad, const float *input_data) {
+    ok(cct_hip_relu_backward((float *)in_grad->ptr, (const float *)out_grad->ptr, input_data,
+                             out_grad->size_in_byte / sizeof(float)),
+       "relu_backward");
+  }
+  void dropout_forward_train(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const unsigned int *mask,
+                             float scale, unsigned int threshold) {
+    ok(cct_hip_dropout_forward_train((float *)dst->ptr, (const float *)src->ptr, mask, scale, threshold,
+                                     src->size_in_byte / sizeof(float)),
+       "dropout_forward_train");
+  }
+  void softmax_loss_forward(float *prob, const float *in, const float *labels, float *loss_sum,
+                            int len_per_image, int batch) {
+    ok(cct_hip_softmax_loss_forward(prob, in, labels, loss_sum, len_per_image, batch), "softmax_loss_forward");
+  }
+  void softmax_loss_backward(float *in_grad, const float *prob, const float *labels, int len_per_image,
+                             int batch, int spatial) {
+    ok(cct_hip_softmax_loss_backward(in_grad, prob, labels, len_per_image, batch, spatial),
+       "softmax_loss_backward");
+  }
+
+  // ---- single precision BLAS-shaped members (DeviceDriver.h:197-215) ----
+  void math_saxpy(const float alpha, DeviceMemoryPointer *X, DeviceMemoryPointer *Y) const {
+    ok(cct_hip_math_saxpy(X->size_in_byte / sizeof(float), alpha, (const float *)X->ptr, (float *)Y->ptr),
+       "math_saxpy");
+  }
+  void math_saxpy(const int nItems, const float alpha, float *X, float *Y) const {
+    ok(cct_hip_math_saxpy((size_t)nItems, alpha, X, Y), "math_saxpy");
+  }
+  void math_saxpby(const float alpha, DeviceMemoryPointer *X, const float beta, DeviceMemoryPointer *Y) const {
+    ok(cct_hip_math_saxpby(X->size_in_byte / sizeof(float), alpha, (const float *)X->ptr, beta, (float *)Y->ptr),
+       "math_saxpby");
+  }
+  void math_saxpby(const int N, const float alpha, const float *X, const float beta, float *Y) const {
+    ok(cct_hip_math_saxpby((size_t)N, alpha, X, beta, Y), "math_saxpby");
+  }
+  void L1_update(const int n_elements, float *const p_gradient, const float lambda, const float *const p_model) {
+    ok(cct_hip_L1_update(n_elements, p_gradient, lambda, p_model), "L1_update");
+  }
+  void sgd_update(size_t n, float *model, float *gradient, float *history, float stepsize, float momentum,
+                  float lambda, bool l1) {
+    ok(cct_hip_sgd_update(n, model, gradient, history, stepsize, momentum, lambda, l1 ? 1 : 0), "sgd_update");
+  }
+  void set_num_threads(const int) {}
+  void sgemm(const enum CBLAS_ORDER order, CBLAS_TRANSPOSE TA, CBLAS_TRANSPOSE TB, int M, int N, int K,
+             float alpha, float *pA, int LDA, float *pB, int LDB, float beta, float *pC, int LDC) {
+    ok(cct_hip_sgemm(order, TA, TB, M, N, K, alpha, pA, LDA, pB, LDB, beta, pC, LDC), "sgemm");
+  }
+  void sgemm_new(const CBLAS_TRANSPOSE TA, const CBLAS_TRANSPOSE TB, const int M, const int N, const int K,
+                 const float alpha, const float *pA, const float *pB, const float beta, float *pC) {
+    ok(cct_hip_sgemm_new(TA, TB, M, N, K, alpha, pA, pB, beta, pC), "sgemm_new");
+  }
+  void sgemm_conv_forward(int o, int batch, int fmap, int K, const float *model, const float *lowered,
+                          const float *bias, float *out) {
+    ok(cct_hip_sgemm_conv_forward(o, batch, fmap, K, model, lowered, bias, out), "sgemm_conv_forward");
+  }
+  void sgemv(const CBLAS_TRANSPOSE TA, const int M, const int N, const float alpha, const float *pA,
+             const float *px, const float beta, float *py) {
+    ok(cct_hip_sgemv(TA, M, N, alpha, pA, px, beta, py), "sgemv");
+  }
+
+  // ---- fillers / rng (DeviceDriver.h:238-260) ----
+  void init_rng(const int random_seed) { ok(cct_hip_init_rng(random_seed), "init_rng"); }
+  void rand_uint_initialize(unsigned int *buf, const int n) {
+    ok(cct_hip_rand_uint_initialize(buf, n), "rand_uint_initialize");
+  }
+  // Random fillers draw on the host from std::mt19937 with the same distributions and call
+  // order as CPUDriver (src/sched/DeviceDriver_CPU.cpp:661-699), then copy to the device.
+  void sinitialize_xavier(DeviceMemoryPointer *arr, const size_t n_batch, const int random_seed = -1) {
+    const size_t n = arr->size_in_byte / sizeof(float);
+    const size_t fan_in = n / n_batch;
+    const float scale = std::sqrt(3.0 / fan_in);
+    std::mt19937 gen(seed_or_random(random_seed));
+    std::uniform_real_distribution<float> uni(-scale, scale);
+    std::vector<float> tmp(n);
+    for (size_t i = 0; i < n; ++i) tmp[i] = uni(gen);
+    ok(cct_hip_memcpy(arr->ptr, tmp.data(), arr->size_in_byte, 0), "sinitialize_xavier");
+  }
+  void sbernoulli_initialize(DeviceMemoryPointer *arr, const float p, const int random_seed = -1) {
+    const size_t n = arr->size_in_byte / sizeof(float);
+    std::mt19937 gen(seed_or_random(random_seed));
+    std::bernoulli_distribution bern(p);
+    std::vector<float> tmp(n);
+    for (size_t i = 0; i < n; ++i) tmp[i] = bern(gen);
+    ok(cct_hip_memcpy(arr->ptr, tmp.data(), arr->size_in_byte, 0), "sbernoulli_initialize");
+  }
+  void sgaussian_initialize(DeviceMemoryPointer *arr, const float mean, const float std_dev,
+                            const int random_seed = -1) {
+    const size_t n = arr->size_in_byte / sizeof(float);
+    std::mt19937 gen(seed_or_random(random_seed));
+    std::normal_distribution<float> gaussian(mean, std_dev);
+    std::vector<float> tmp(n);
+    for (size_t i = 0; i < n; ++i) tmp[i] = gaussian(gen);
+    ok(cct_hip_memcpy(arr->ptr, tmp.data(), arr->size_in_byte, 0), "sgaussian_initialize");
+  }
+  void sconstant_initialize(DeviceMemoryPointer *arr, const float value) {
+    ok(cct_hip_sconstant_initialize((float *)arr->ptr, arr->size_in_byte / sizeof(float), value),
+       "sconstant_initialize");
+  }
+
+  // ---- hooks (DeviceDriver.h:266-272) ----
+  void device_sync() { ok(cct_hip_device_sync(), "device_sync"); }
+  void init_thread() { ok(cct_hip_init(device_id_), "init_thread"); }
+  void destroy_thread() {}
+  void set_device_id(int id) { device_id_ = id; ok(cct_hip_init(id), "set_device_id"); }
+
+ private:
+  int device_id_ = 0;
+  static unsigned seed_or_random(int random_seed) {
+    if (random_seed != -1) return (unsigned)random_seed;
+    std::random_device rd;
+    return rd();
+  }
+  static void ok(int rc, const char *what) {
+    if (rc != 0) {
+      std::fprintf(stderr, "HIPDriver::%s failed (%d): %s\n", what, rc, cct_hip_last_error());
+      std::abort();
+    }
+  }
+};
+
+}  // namespace cct

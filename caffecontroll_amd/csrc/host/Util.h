@@ -1,0 +1,37 @@
+// Device-independent helpers (src/util.h:66-93).
+#pragma once
+#include <cassert>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <string>
+
+namespace cct {
+
+struct Util {
+  // Learning-rate schedule, same policies and float/double steps as Util::get_learning_rate.
+  static inline float get_learning_rate(const std::string &lr_policy, float base_lr, float gamma, float iter,
+                                        float caffe_stepsize, float power, float max_iter) {
+    float rate;
+    if (lr_policy == "fixed") {
+      rate = base_lr;
+    } else if (lr_policy == "step") {
+      const float current_step = (float)(int)(iter / caffe_stepsize);
+      rate = base_lr * std::pow(gamma, current_step);
+    } else if (lr_policy == "exp") {
+      rate = base_lr * std::pow(gamma, iter);
+    } else if (lr_policy == "inv") {
+      rate = (float)(base_lr * std::pow(1.0 + gamma * iter, -power));
+    } else if (lr_policy == "poly") {
+      rate = (float)(base_lr * std::pow(1.0 - (iter / max_iter), power));
+    } else if (lr_policy == "sigmoid") {
+      rate = (float)(base_lr * (1.0 / (1.0 + std::exp(-gamma * (iter - caffe_stepsize)))));
+    } else {
+      std::fprintf(stderr, "Unknown or unsupported learning rate policy: %s\n", lr_policy.c_str());
+      std::abort();
+    }
+    return rate;
+  }
+};
+
+}  // namespace cct

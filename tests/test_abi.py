@@ -7,10 +7,10 @@ import re
 from conftest import ROOT
 
 
-def _declared_symbols():
-    text = open(os.path.join(ROOT, "include", "cct_hip.h")).read()
+def _declared_symbols(header="cct_hip.h", prefix="cct_hip_"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(cct_hip_[a-zA-Z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(%s[a-zA-Z0-9_]+)\s*\(" % prefix, text)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -22,6 +22,13 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), "missing export: " + n
     # the ctypes prototype table covers the header, nothing more, nothing less
     assert sorted(_lib.PROTOTYPES) == names
+    # operator-level entry points
+    from caffecontroll_amd import bridges
+    bnames = _declared_symbols("cct_bridge.h", "cct_conv_bridge_")
+    assert len(bnames) >= 12
+    for n in bnames:
+        assert hasattr(lib, n), "missing export: " + n
+    assert sorted(bridges.BRIDGE_PROTOTYPES) == bnames
 
 
 def test_struct_layouts_match_reference_headers():

@@ -1,0 +1,136 @@
+"""GPU parity at operator level: ParallelizedBridge<ConvolutionBridge> on the HIP driver against
+the reference's golden files (the same scenario as tests/test_parallelized_convolution.cpp:123-270
+and ..._large_CPU.cpp) and against the CPU oracle on seeded tensors."""
+import numpy as np
+import pytest
+
+from conftest import load_fixture
+from gpu_util import dev, driver, empty, host, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def _copy_to(ptr, arr):
+    a = np.ascontiguousarray(arr, np.float32)
+    driver().memcpy(ptr, a.ctypes.data, a.nbytes, 0)
+
+
+def _read(ptr, shape):
+    out = np.empty(shape, np.float32)
+    driver().memcpy(out.ctypes.data, ptr, out.nbytes, 1)
+    return out
+
+
+FIX = {
+    "small": dict(b=4, d=3, n=20, k=5, s=4, p=2, o=10, sfx=""),
+    "large": dict(b=4, d=3, n=127, k=11, s=4, p=2, o=8, sfx="_large"),
+}
+
+
+@pytest.mark.parametrize("case", ["small", "large"])
+@pytest.mark.parametrize("fused", [True, False])
+def test_pbridge_reference_scenario(case, fused):
+    from caffecontroll_amd.bridges import ConvolutionLayer, solver_param
+    c = FIX[case]
+    b, d, n, k, s, p, o, sfx = (c[x] for x in ("b", "d", "n", "k", "s", "p", "o", "sfx"))
+    m = (n + 2 * p - k) // s + 1
+    driver()
+    x = load_fixture("input", f"conv_forward_in{sfx}.txt").reshape(b, d, n, n)
+    in_data, in_grad = dev(x), empty((b, d, n, n), fill=0.0)
+    out_data, out_grad = empty((b, o, m, m), fill=0.0), empty((b, o, m, m), fill=0.0)
+    # solver of the reference test: lr 0.01, momentum 0, policy "step" with stepsize 10000
+    layer = ConvolutionLayer(b, d, n, k, s, p, o, in_data, in_grad, out_data, out_grad,
+                             solver=solver_param(base_lr=0.01, momentum=0.0, lr_policy="step", stepsize=10000))
+    layer.set_options(fused=fused)
+    # TestForward
+    _copy_to(layer.model_ptr(), load_fixture("input", f"conv_model{sfx}.txt"))
+    _copy_to(layer.bias_ptr(), load_fixture("input", f"conv_bias_in{sfx}.txt"))
+    layer.forward()
+    exp = load_fixture("output", f"conv_forward{sfx}.txt")
+    np.testing.assert_allclose(host(out_data).reshape(-1), exp, rtol=2e-5, atol=1e-3)
+    # TestBackward
+    _copy_to(layer.model_ptr(), load_fixture("input", f"conv_backward_model{sfx}.txt"))
+    og = (np.arange(b * o * m * m, dtype=np.float64) * 0.1).astype(np.float32)
+    out_grad.copy_(dev(og).reshape(out_grad.shape))
+    og_before = host(out_grad).copy()
+    layer.forward()
+    layer.backward(with_update=True)
+    exp_dx = load_fixture("output", f"conv_backward{sfx}.txt")
+    np.testing.assert_allclose(host(in_grad).reshape(-1)[:exp_dx.size], exp_dx, rtol=1e-4, atol=1e-3)
+    np.testing.assert_allclose(_read(layer.model_ptr(), (o * d * k * k,)),
+                               load_fixture("output", f"conv_weights{sfx}.txt"), rtol=1e-4, atol=1e-3)
+    np.testing.assert_allclose(_read(layer.bias_ptr(), (o,)),
+                               load_fixture("output", f"conv_bias{sfx}.txt"), rtol=1e-4, atol=1e-3)
+    # the caller's output-gradient cube is left as it was (the HIP bridge permutes into scratch)
+    np.testing.assert_array_equal(host(out_grad), og_before)
+    layer.close()
+
+
+@pytest.mark.parametrize("shape", [(8, 96, 27, 5, 1, 2, 256), (64, 1, 28, 5, 1, 0, 20), (4, 3, 227, 11, 4, 0, 96)],
+                         ids=lambda s: "b%d_d%d_n%d_k%d_s%d_p%d_o%d" % s)
+def test_pbridge_vs_oracle_with_momentum(oracle, shape):
+    """Two iterations with momentum and weight decay: gradients, history and weights track the
+    oracle's ConvolutionBridge + SGDGradientUpdater restatement."""
+    from caffecontroll_amd.bridges import ConvolutionLayer, solver_param
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
+    rng = np.random.default_rng(1234 + sum(shape))
+    x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+    w = (rng.standard_normal((o, d, k, k)) * 0.01).astype(np.float32)
+    bias = np.full(o, 0.1, np.float32)
+    driver()
+    in_data, in_grad = dev(x), empty((b, d, n, n))
+    out_data, out_grad = empty((b, o, m, m)), empty((b, o, m, m), fill=0.0)
+    lr, mom, wd = 0.01, 0.9, 0.0005
+    layer = ConvolutionLayer(b, d, n, k, s, p, o, in_data, in_grad, out_data, out_grad,
+                             solver=solver_param(base_lr=lr, momentum=mom, weight_decay=wd),
+                             lr_mult=(1.0, 2.0), decay_mult=(1.0, 0.0))
+    _copy_to(layer.model_ptr(), w)
+    _copy_to(layer.bias_ptr(), bias)
+    rw, rb = w.copy(), bias.copy()
+    hw, hb = np.zeros(w.size, np.float32), np.zeros(o, np.float32)
+    bound = oracle.bind_openblas(8)
+    try:
+        for it in range(2):
+            og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+            out_grad.copy_(dev(og))
+            layer.forward()
+            layer.backward(with_update=True)
+            ref_out, rlow = oracle.conv_forward(x, rw, rb, k, s, p)
+            rdx, rdw, rdb = oracle.conv_backward(x.shape, rw, og, rlow, k, s, p)
+            assert rel_err(host(out_data), ref_out) <= TOL
+            assert rel_err(host(in_grad), rdx) <= TOL
+            rw_flat = rw.reshape(-1)
+            oracle.sgd_update(rw_flat, rdw.reshape(-1), hw, lr * 1.0, mom, wd * 1.0)
+            oracle.sgd_update(rb, rdb, hb, lr * 2.0, mom, 0.0)
+            rw = rw_flat.reshape(w.shape)
+            assert rel_err(_read(layer.model_ptr(), w.shape), rw) <= TOL
+            assert rel_err(_read(layer.bias_ptr(), (o,)), rb) <= TOL
+            assert rel_err(_read(layer.history_ptr(), (w.size,)), hw) <= TOL
+    finally:
+        if bound:
+            oracle.unbind_openblas()
+    layer.close()
+
+
+def test_stage_profile_and_first_layer_mode():
+    from caffecontroll_amd.bridges import STAGE_NAMES, ConvolutionLayer
+    b, d, n, k, s, p, o = 4, 8, 12, 3, 1, 1, 16
+    driver()
+    in_data, in_grad = empty((b, d, n, n), fill=1.0), empty((b, d, n, n), fill=-5.0)
+    out_data, out_grad = empty((b, o, n, n)), empty((b, o, n, n), fill=1.0)
+    layer = ConvolutionLayer(b, d, n, k, s, p, o, in_data, in_grad, out_data, out_grad)
+    layer.set_options(fused=False, profile=True, needs_backward_grad=False)
+    layer.forward()
+    layer.backward()
+    ms = layer.stage_ms()
+    assert set(ms) == set(STAGE_NAMES)
+    assert ms["Lower Cube"] > 0 and ms["GEMM"] > 0 and ms["Remap"] > 0 and ms["Bias"] > 0 and ms["GEMM Wghts"] > 0
+    assert ms["GEMM Data"] == 0 and ms["Inverse Lwr"] == 0      # skipped for a first layer
+    assert (host(in_grad) == -5.0).all()                          # and the input gradient is untouched
+    # bias gradient of an all-ones output gradient = b * m * m
+    bg = np.empty(o, np.float32)
+    driver().memcpy(bg.ctypes.data, layer.bias_grad_ptr(), bg.nbytes, 1)
+    assert (bg == b * n * n).all()
+    layer.close()
