@@ -137,7 +137,7 @@ __device__ __forceinline__ void load_frags(float (&f)[NT][4], const float *__res
 }
 
 template <class T, bool A_KC, bool B_KC>
-__global__ __launch_bounds__(T::THREADS) void gemm_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
   using LA = OperandLayout<T, A_KC, T::BM>;
   using LB = OperandLayout<T, B_KC, T::BN>;
   __shared__ __attribute__((aligned(16))) float smem[2 * (LA::SIZE + LB::SIZE)];

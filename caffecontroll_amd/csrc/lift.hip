@@ -25,6 +25,8 @@ struct LiftParams {
   int iR, iC, iD, iB;
   uint32_t npix;      // iB*iD*iR*iC
   uint32_t nblocks;   // lift workgroups
+  uint32_t nbias;     // bias-gradient workgroups; they take the FIRST block ids so that their long
+                      // serial reductions start at once and overlap the lift blocks
   size_t plane;       // iB*m*m
   FastDiv div_c, div_r, div_d;
   // bias part
@@ -75,13 +77,13 @@ template <int KT, int ST>
 __global__ __launch_bounds__(LIFT_THREADS) void lift_kernel(float *__restrict__ dst,
                                                             const float *__restrict__ src,
                                                             const LiftParams P) {
-  if (blockIdx.x >= P.nblocks) {
-    bias_backward_block(P, (int)(blockIdx.x - P.nblocks));
+  if (blockIdx.x < P.nbias) {
+    bias_backward_block(P, (int)blockIdx.x);
     return;
   }
   const int k = KT ? KT : P.k;
   const int s = ST ? ST : P.s;
-  const uint32_t pix = blockIdx.x * LIFT_THREADS + threadIdx.x;
+  const uint32_t pix = (blockIdx.x - P.nbias) * LIFT_THREADS + threadIdx.x;
   if (pix >= P.npix) return;
   // pix = ((ib*iD + id)*iR + y)*iC + x
   const uint32_t t1 = fdiv(pix, P.div_c);
@@ -145,8 +147,8 @@ static int launch_lift(float *dst, const float *src, const cct_inverse_lower_cub
   P.plane = a->iB * m * m;
   P.div_c = make_fastdiv(P.iC); P.div_r = make_fastdiv(P.iR); P.div_d = make_fastdiv(P.iD);
   P.out_grad = out_grad; P.bias_grad = bias_grad; P.fmap = fmap; P.depth = depth; P.batch = batch;
-  const uint32_t extra = bias_grad ? (uint32_t)depth : 0;
-  const uint32_t grid = P.nblocks + extra;
+  P.nbias = bias_grad ? (uint32_t)depth : 0;
+  const uint32_t grid = P.nblocks + P.nbias;
   if (grid == 0) return 0;
   hipStream_t st = ctx().stream;
   if (P.k == 5 && P.s == 1)
@@ -191,6 +193,7 @@ extern "C" int cct_hip_backward_bias(float *bias_grad, const float *out_grad, in
   // the same kernel with zero lift blocks
   LiftParams P = {};
   P.nblocks = 0;
+  P.nbias = (uint32_t)depth;
   P.out_grad = out_grad; P.bias_grad = bias_grad; P.fmap = fmap_size; P.depth = depth;
   P.batch = batch_size;
   hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(depth), dim3(LIFT_THREADS), 0, ctx().stream,

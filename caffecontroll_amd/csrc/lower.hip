@@ -24,20 +24,22 @@ struct LowerParams {
   int rowlen;  // k*k*d
   int nbands, nslabs;
   uint32_t nblocks;
-  FastDiv div_kk, div_k, div_tw, div_th, div_seg;
+  int chunk_full;  // staged floats per channel for an interior band: ((RB-1)*s + k) * n
+  FastDiv div_kk, div_k, div_seg, div_n, div_chunk;
 };
 
-constexpr int LOWER_THREADS = 256;
+constexpr int LOWER_MAX_THREADS = 512;  // block size is chosen per launch (multiple of 64)
 
 // dynamic LDS: [DS*TH*TW floats tile][seglen uint16 offsets]
 template <bool VEC4>
-__global__ __launch_bounds__(LOWER_THREADS) void lower_kernel(float *__restrict__ dst,
+__global__ __launch_bounds__(LOWER_MAX_THREADS) void lower_kernel(float *__restrict__ dst,
                                                               const float *__restrict__ src,
                                                               const LowerParams P) {
   extern __shared__ float lds[];
   const int tile_elems = P.DS * P.TH * P.TW;
   float *tile = lds;
-  uint16_t *offs = reinterpret_cast<uint16_t *>(lds + tile_elems);
+  // the table starts on the next 16-byte boundary so that the float4 clear of the tile cannot touch it
+  uint16_t *offs = reinterpret_cast<uint16_t *>(lds + ((tile_elems + 3) & ~3));
 
   // logical block id -> (bi, band, slab); bands of one image stay on one XCD
   uint32_t id = xcd_remap(blockIdx.x, P.nblocks);
@@ -47,6 +49,7 @@ __global__ __launch_bounds__(LOWER_THREADS) void lower_kernel(float *__restrict_
   const int bi = id / P.nbands;
 
   const int tid = threadIdx.x;
+  const int T = blockDim.x;
   const int r0 = band * P.RB;
   const int rb = min(P.RB, P.m - r0);
   const int dd0 = slab * P.DS;
@@ -54,7 +57,7 @@ __global__ __launch_bounds__(LOWER_THREADS) void lower_kernel(float *__restrict_
   const int seg = ds * P.k * P.k;
 
   // (1) offset table: j = dl*k*k + kr*k + kc  ->  (dl*TH + kr)*TW + kc
-  for (int j = tid; j < seg; j += LOWER_THREADS) {
+  for (int j = tid; j < seg; j += T) {
     const uint32_t dl = fdiv(j, P.div_kk);
     const uint32_t rem = j - dl * P.k * P.k;
     const uint32_t kr = fdiv(rem, P.div_k);
@@ -62,22 +65,45 @@ __global__ __launch_bounds__(LOWER_THREADS) void lower_kernel(float *__restrict_
     offs[j] = (uint16_t)((dl * P.TH + kr) * P.TW + kc);
   }
 
-  // (2) stage the padded window: tile[dl][ty][tx] = src[bi][dd0+dl][r0*s-p+ty][-p+tx]
+  // (2) stage the padded window: tile[dl][ty][tx] = src[bi][dd0+dl][r0*s-p+ty][-p+tx].
+  // The tile is cleared first (that is the zero padding); then the in-image rows of every channel,
+  // which are one contiguous run of nrows*n floats in HBM, are copied with eight independent
+  // loads in flight per lane.
+  {
+    const int nz4 = (tile_elems + 3) >> 2;
+    float4 *t4 = reinterpret_cast<float4 *>(tile);
+    for (int e = tid; e < nz4; e += T) t4[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  __syncthreads();
   {
     const int y0 = r0 * P.s - P.p;
     const int th_used = (rb - 1) * P.s + P.k;
-    const float *img = src + ((size_t)bi * P.d + dd0) * P.n * P.n;
-    const int total = ds * P.TH * P.TW;
-    for (int e = tid; e < total; e += LOWER_THREADS) {
-      const uint32_t row = fdiv(e, P.div_tw);  // dl*TH + ty
-      const int tx = e - row * P.TW;
-      const uint32_t dl = fdiv(row, P.div_th);
-      const int ty = row - dl * P.TH;
-      const int y = y0 + ty, x = tx - P.p;
-      float v = 0.0f;
-      if (ty < th_used && y >= 0 && y < P.n && x >= 0 && x < P.n)
-        v = img[((size_t)dl * P.n + y) * P.n + x];
-      tile[e] = v;
+    const int ylo = max(y0, 0), yhi = min(y0 + th_used, P.n);
+    const int chunk = (yhi - ylo) * P.n;
+    const int total = ds * chunk;
+    const int nn = P.n * P.n;
+    const float *img = src + ((size_t)bi * P.d + dd0) * nn + ylo * P.n;
+    const int trow0 = ylo - y0;
+    const bool fast = (chunk == P.chunk_full);
+    for (int base = 0; base < total; base += T * 8) {
+      float v[8];
+      int dst_i[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int e = base + j * T + tid;
+        const bool ok = e < total;
+        const uint32_t ec = ok ? e : 0;
+        const uint32_t dl = fast ? fdiv(ec, P.div_chunk) : ec / (uint32_t)chunk;
+        const uint32_t i = ec - dl * chunk;
+        const uint32_t row = fdiv(i, P.div_n);
+        const uint32_t x = i - row * P.n;
+        v[j] = img[(size_t)dl * nn + i];
+        // columns past the last window (strided layers) have no place in the tile
+        dst_i[j] = (ok && (int)x + P.p < P.TW) ? (int)((dl * P.TH + trow0 + row) * P.TW + P.p + x) : -1;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if (dst_i[j] >= 0) tile[dst_i[j]] = v[j];
     }
   }
   __syncthreads();
@@ -88,7 +114,7 @@ __global__ __launch_bounds__(LOWER_THREADS) void lower_kernel(float *__restrict_
     // seg % 4 == 0 and every segment start is 16-byte aligned: a lane owns 4 consecutive row
     // positions and walks over the output positions of the band
     const int nq = seg >> 2;
-    for (int q = tid; q < nq; q += LOWER_THREADS) {
+    for (int q = tid; q < nq; q += T) {
       const int o0 = offs[4 * q], o1 = offs[4 * q + 1], o2 = offs[4 * q + 2], o3 = offs[4 * q + 3];
       float *outq = out_band + 4 * q;
       for (int rl = 0; rl < rb; ++rl) {
@@ -109,7 +135,7 @@ __global__ __launch_bounds__(LOWER_THREADS) void lower_kernel(float *__restrict_
     for (int rl = 0; rl < rb; ++rl) {
       const float *trow = tile + rl * P.s * P.TW;
       float *orow = out_band + (size_t)rl * P.m * P.rowlen;
-      for (uint32_t e = tid; e < per_row; e += LOWER_THREADS) {
+      for (uint32_t e = tid; e < per_row; e += T) {
         const uint32_t c = (seg == P.seglen) ? fdiv(e, P.div_seg) : e / (uint32_t)seg;
         const uint32_t j = e - c * seg;
         const float v = trow[c * P.s + offs[j]];
@@ -153,7 +179,7 @@ extern "C" int cct_hip_lower_cube(float *dst, const float *src, const cct_pmap_h
   P.DS = P.d;
   auto lds_need = [&](int RB, int DS) {
     const size_t th = (size_t)(RB - 1) * P.s + P.k;
-    return (size_t)DS * th * P.TW * 4 + (((size_t)DS * P.k * P.k * 2 + 3) & ~(size_t)3);
+    return ((((size_t)DS * th * P.TW) + 3) & ~(size_t)3) * 4 + (((size_t)DS * P.k * P.k * 2 + 3) & ~(size_t)3);
   };
   while (P.DS > 1 && (lds_need(1, P.DS) > lds_budget || (size_t)P.DS * P.k * P.TW >= 65536))
     P.DS = (P.DS + 1) / 2;
@@ -173,26 +199,38 @@ extern "C" int cct_hip_lower_cube(float *dst, const float *src, const cct_pmap_h
   const size_t nblocks = (size_t)P.b * P.nbands * P.nslabs;
   CCT_REQUIRE(nblocks < (1ull << 31), "lower_cube: too many workgroups");
   P.nblocks = (uint32_t)nblocks;
+  P.chunk_full = P.TH * P.n;
   P.div_kk = make_fastdiv(P.k * P.k);
   P.div_k = make_fastdiv(P.k);
-  P.div_tw = make_fastdiv(P.TW);
-  P.div_th = make_fastdiv(P.TH);
   P.div_seg = make_fastdiv(P.seglen);
+  P.div_n = make_fastdiv(P.n);
+  P.div_chunk = make_fastdiv(P.chunk_full);
 
   const size_t lds_bytes = lds_need(P.RB, P.DS);
   // float4 stores need every (position, slab) segment to start 16-byte aligned and to hold a
   // whole number of float4: k*k*DS % 4 == 0 covers both when dst itself is aligned.
   const bool vec4 = ((uintptr_t)dst % 16 == 0) && (P.rowlen % 4 == 0) && ((P.DS * P.k * P.k) % 4 == 0) &&
                     (P.d % P.DS == 0);
+  // block size: the multiple of 64 that wastes the fewest lanes in the store loop
+  const long units = vec4 ? P.seglen / 4 : (long)P.m * P.seglen;
+  int threads = 256;
+  double best = 1e30;
+  for (int t = 128; t <= LOWER_MAX_THREADS; t += 64) {
+    const double waste = (double)((units + t - 1) / t * t) / (double)units;
+    if (waste < best - 1e-9 || (waste < best + 1e-9 && t <= 320)) {
+      best = waste;
+      threads = t;
+    }
+  }
   hipStream_t st = ctx().stream;
   if (vec4) {
     CCT_HIP_CHECK(hipFuncSetAttribute((const void *)lower_kernel<true>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    hipLaunchKernelGGL(lower_kernel<true>, dim3(P.nblocks), dim3(LOWER_THREADS), lds_bytes, st, dst, src, P);
+    hipLaunchKernelGGL(lower_kernel<true>, dim3(P.nblocks), dim3(threads), lds_bytes, st, dst, src, P);
   } else {
     CCT_HIP_CHECK(hipFuncSetAttribute((const void *)lower_kernel<false>,
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    hipLaunchKernelGGL(lower_kernel<false>, dim3(P.nblocks), dim3(LOWER_THREADS), lds_bytes, st, dst, src, P);
+    hipLaunchKernelGGL(lower_kernel<false>, dim3(P.nblocks), dim3(threads), lds_bytes, st, dst, src, P);
   }
   CCT_LAUNCH_CHECK();
   return 0;
