@@ -102,6 +102,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="staged forward (GEMM, remap, bias) and separate bias gradient")
     ap.add_argument("--no-data-grad", action="store_true", help="first-layer mode: skip data-gradient GEMM and lift")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run 5 device-to-device copies of 1 GiB (a plain copy kernel of known size, used "
+                         "to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters) and exit")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU (batch sharding over several GPUs is a design note, "
@@ -117,6 +120,17 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(3)
+    if args.copy_calibration:
+        drv = HIPDriver(0)
+        nbytes = 1 << 30
+        src = torch.ones(nbytes // 4, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            drv.memcpy(dst, src, nbytes, 2)
+        drv.device_sync()
+        print(json.dumps({"copy_calibration_bytes_read": nbytes, "copy_calibration_bytes_written": nbytes,
+                          "copies": 5}))
+        return
     cfg = args.workload
     b, d, n, k, s, p, o = CONFIGS[cfg]
     m = (n + 2 * p - k) // s + 1

@@ -18,11 +18,15 @@
 //     writes [b][o][fmap] directly and adds the bias.
 //
 // Bound: fp32 MFMA rate (256 FLOP/clk/CU).  Algorithmic work 2*M*N*K FLOP per call.
+#include <cstdlib>
+
 #include "cct_common.h"
 
 namespace cct {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
+// native 4-float vector: stays in registers where HIP's f4 struct (a union) can end up in scratch
+typedef float f4 __attribute__((ext_vector_type(4)));
 
 enum EpilogueMode { EPI_ALPHA_BETA = 0, EPI_SPLITK_PARTIAL = 1, EPI_CONV_FORWARD = 2 };
 
@@ -42,15 +46,18 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   uint32_t ntiles;
   int a_vec, b_vec;  // operand allows aligned 16-byte global loads
+  int splits;        // K slices; grid = ntiles * splits workgroups
+  uint32_t nblocks;
+  int nt_store;      // stream the output with non-temporal stores (large outputs that are not re-read)
 };
 
-__device__ __forceinline__ float4 ldg4(const float *__restrict__ base, int major, int minor,
+__device__ __forceinline__ f4 ldg4(const float *__restrict__ base, int major, int minor,
                                        int major_lim, int minor_lim, int ld, int vec) {
-  float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+  f4 v = f4{0.f, 0.f, 0.f, 0.f};
   if (major < major_lim) {
     const float *p = base + (size_t)major * ld + minor;
     if (vec && minor + 3 < minor_lim) {
-      v = *reinterpret_cast<const float4 *>(p);
+      v = *reinterpret_cast<const f4 *>(p);
     } else {
       if (minor + 0 < minor_lim) v.x = p[0];
       if (minor + 1 < minor_lim) v.y = p[1];
@@ -78,12 +85,12 @@ template <class T, bool KC, int ROWS>
 struct OperandLayout {
   // floats per LDS stage
   static constexpr int SIZE = KC ? ROWS * (T::BK + T::PK) : T::BK * (ROWS + T::PR);
-  static constexpr int NV = ROWS * T::BK / 4 / T::THREADS;  // float4 per lane per stage
+  static constexpr int NV = ROWS * T::BK / 4 / T::THREADS;  // f4 per lane per stage
 };
 
 // global -> registers for one operand tile (rows x BK) starting at (row0, k0)
 template <class T, bool KC, int ROWS>
-__device__ __forceinline__ void load_tile(float4 *__restrict__ r,
+__device__ __forceinline__ void load_tile(f4 *__restrict__ r,
                                           const float *__restrict__ g, int ld, int row0, int k0,
                                           int row_lim, int k_lim, int vec, int tid) {
   constexpr int NV = OperandLayout<T, KC, ROWS>::NV;
@@ -101,7 +108,7 @@ __device__ __forceinline__ void load_tile(float4 *__restrict__ r,
 }
 
 template <class T, bool KC, int ROWS>
-__device__ __forceinline__ void store_tile(float *__restrict__ lds, const float4 *__restrict__ r,
+__device__ __forceinline__ void store_tile(float *__restrict__ lds, const f4 *__restrict__ r,
                                            int tid) {
   constexpr int NV = OperandLayout<T, KC, ROWS>::NV;
 #pragma unroll
@@ -109,31 +116,164 @@ __device__ __forceinline__ void store_tile(float *__restrict__ lds, const float4
     const int f = tid + i * T::THREADS;
     if (KC) {
       const int row = f / (T::BK / 4), kq = f % (T::BK / 4);
-      *reinterpret_cast<float4 *>(lds + row * (T::BK + T::PK) + kq * 4) = r[i];
+      *reinterpret_cast<f4 *>(lds + row * (T::BK + T::PK) + kq * 4) = r[i];
     } else {
       const int kk = f / (ROWS / 4), rq = f % (ROWS / 4);
-      *reinterpret_cast<float4 *>(lds + kk * (ROWS + T::PR) + rq * 4) = r[i];
+      *reinterpret_cast<f4 *>(lds + kk * (ROWS + T::PR) + rq * 4) = r[i];
     }
   }
 }
 
-// fragments of k-group kg for NT 32-row tiles starting at row0: f[t][i], i = MFMA index in group
+// fragments of k-group kg for NT 32-row tiles starting at row0: component i of f[t] feeds MFMA i
+// of the group
 template <class T, bool KC, int ROWS, int NT>
-__device__ __forceinline__ void load_frags(float (&f)[NT][4], const float *__restrict__ lds,
-                                           int row0, int kg, int lane) {
+__device__ __forceinline__ void load_frags(f4 (&f)[NT], const float *__restrict__ lds, int row0, int kg,
+                                           int lane) {
   const int r = lane & 31, h = lane >> 5;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     if (KC) {
-      const float4 v = *reinterpret_cast<const float4 *>(lds + (row0 + t * 32 + r) * (T::BK + T::PK) +
-                                                         kg * 8 + h * 4);
-      f[t][0] = v.x; f[t][1] = v.y; f[t][2] = v.z; f[t][3] = v.w;
+      f[t] = *reinterpret_cast<const f4 *>(lds + (row0 + t * 32 + r) * (T::BK + T::PK) + kg * 8 + h * 4);
     } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        f[t][i] = lds[(kg * 8 + h * 4 + i) * (ROWS + T::PR) + row0 + t * 32 + r];
+      const float *p = lds + (kg * 8 + h * 4) * (ROWS + T::PR) + row0 + t * 32 + r;
+      f[t].x = p[0];
+      f[t].y = p[ROWS + T::PR];
+      f[t].z = p[2 * (ROWS + T::PR)];
+      f[t].w = p[3 * (ROWS + T::PR)];
     }
   }
+}
+
+template <int I>
+__device__ __forceinline__ float comp(const f4 &v) {
+  return I == 0 ? v.x : I == 1 ? v.y : I == 2 ? v.z : v.w;
+}
+
+template <int I, int TM, int TN>
+__device__ __forceinline__ void mfma_step(v16f (&acc)[TM][TN], const f4 (&fa)[TM], const f4 (&fb)[TN]) {
+#pragma unroll
+  for (int a = 0; a < TM; ++a)
+#pragma unroll
+    for (int b = 0; b < TN; ++b)
+      acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(comp<I>(fa[a]), comp<I>(fb[b]), acc[a][b], 0, 0, 0);
+}
+
+template <int TM, int TN>
+__device__ __forceinline__ void mfma_group(v16f (&acc)[TM][TN], const f4 (&fa)[TM], const f4 (&fb)[TN]) {
+  mfma_step<0>(acc, fa, fb);
+  mfma_step<1>(acc, fa, fb);
+  mfma_step<2>(acc, fa, fb);
+  mfma_step<3>(acc, fa, fb);
+}
+
+// Unguarded loader state for interior tiles: one 16-byte pointer per f4 a lane fetches,
+// advanced by one K step per tile.
+template <class T, bool KC, int ROWS>
+struct FastLoader {
+  static constexpr int NV = OperandLayout<T, KC, ROWS>::NV;
+  const f4 *p[NV];
+  size_t step;  // f4 units per K step
+  __device__ __forceinline__ void init(const float *g, int ld, int row0, int k0, int tid) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int f = tid + i * T::THREADS;
+      if (KC) {
+        const int row = f / (T::BK / 4), kq = f % (T::BK / 4);
+        p[i] = reinterpret_cast<const f4 *>(g + (size_t)(row0 + row) * ld + k0 + kq * 4);
+      } else {
+        const int kk = f / (ROWS / 4), rq = f % (ROWS / 4);
+        p[i] = reinterpret_cast<const f4 *>(g + (size_t)(k0 + kk) * ld + row0 + rq * 4);
+      }
+    }
+    step = KC ? (size_t)(T::BK / 4) : (size_t)T::BK * ld / 4;
+  }
+  __device__ __forceinline__ void load(f4 *__restrict__ r) {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      r[i] = *p[i];
+      p[i] += step;
+    }
+  }
+};
+
+// Main K loop of one macro tile.  GUARD = false: the tile lies inside the matrices, K steps are
+// whole and both operands allow aligned 16-byte loads, so the loaders carry no bounds tests.
+//
+// Software pipeline (BK = 16 = two k-groups of 8, two LDS stages, ONE barrier per K step):
+//   step t, first half : MFMAs of k-group 0 of stage t (fragments fetched during step t-1);
+//                        meanwhile the global data of tile t+1 (requested during step t-1) is
+//                        written to stage t+1 and the loads of tile t+2 are issued
+//   barrier            : stage t+1 is complete, nobody reads stage t any more
+//   step t, second half: fragments of k-group 0 of stage t+1 are requested, MFMAs of k-group 1
+//                        of stage t run, then the fragments of k-group 1 of stage t+1 are requested
+// so LDS and HBM latencies are covered by 32 MFMAs (2048 matrix-pipe cycles) each.
+template <class T, bool A_KC, bool B_KC, bool GUARD>
+__device__ __forceinline__ void gemm_mainloop(const GemmArgs &g, float *smem, v16f (&acc)[T::TM][T::TN], int m0,
+                                              int n0, int kbeg, int kend, int nk, int tid, int lane, int wm0,
+                                              int wn0) {
+  using LA = OperandLayout<T, A_KC, T::BM>;
+  using LB = OperandLayout<T, B_KC, T::BN>;
+  constexpr int STAGE = LA::SIZE + LB::SIZE;  // stage s: A at smem + s*STAGE, B right after it
+  static_assert(T::BK == 16, "the pipeline below is written for two k-groups per K step");
+  f4 ra[LA::NV], rb[LB::NV];
+  FastLoader<T, A_KC, T::BM> la;
+  FastLoader<T, B_KC, T::BN> lb;
+  if (!GUARD) {
+    la.init(g.A, g.lda, m0, kbeg, tid);
+    lb.init(g.B, g.ldb, n0, kbeg, tid);
+  }
+// global -> registers for K step t
+#define CCT_FETCH(t)                                                                         \
+  do {                                                                                       \
+    if (GUARD) {                                                                             \
+      const int k0_ = kbeg + (t) * T::BK;                                                    \
+      load_tile<T, A_KC, T::BM>(ra, g.A, g.lda, m0, k0_, g.M, kend, g.a_vec, tid);           \
+      load_tile<T, B_KC, T::BN>(rb, g.B, g.ldb, n0, k0_, g.N, kend, g.b_vec, tid);           \
+    } else {                                                                                 \
+      la.load(ra);                                                                           \
+      lb.load(rb);                                                                           \
+    }                                                                                        \
+  } while (0)
+// registers -> LDS stage
+#define CCT_STASH(stage)                                                                     \
+  do {                                                                                       \
+    store_tile<T, A_KC, T::BM>(smem + (stage) * STAGE, ra, tid);                             \
+    store_tile<T, B_KC, T::BN>(smem + (stage) * STAGE + LA::SIZE, rb, tid);                  \
+  } while (0)
+// LDS stage, k-group -> MFMA fragments
+#define CCT_FRAGS(stage, kg, fa, fb)                                                         \
+  do {                                                                                       \
+    load_frags<T, A_KC, T::BM, T::TM>(fa, smem + (stage) * STAGE, wm0, kg, lane);            \
+    load_frags<T, B_KC, T::BN, T::TN>(fb, smem + (stage) * STAGE + LA::SIZE, wn0, kg, lane); \
+  } while (0)
+
+  f4 fa0[T::TM], fb0[T::TN], fa1[T::TM], fb1[T::TN];
+  if (nk <= 0) return;
+  CCT_FETCH(0);
+  CCT_STASH(0);
+  if (nk > 1) CCT_FETCH(1);
+  __syncthreads();
+  CCT_FRAGS(0, 0, fa0, fb0);
+  CCT_FRAGS(0, 1, fa1, fb1);
+  for (int t = 0; t < nk; ++t) {
+    const int cur = t & 1;
+    const bool more = (t + 1 < nk);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_group<T::TM, T::TN>(acc, fa0, fb0);
+    if (more) {
+      CCT_STASH(cur ^ 1);
+      if (t + 2 < nk) CCT_FETCH(t + 2);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
+    if (more) CCT_FRAGS(cur ^ 1, 0, fa0, fb0);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_group<T::TM, T::TN>(acc, fa1, fb1);
+    if (more) CCT_FRAGS(cur ^ 1, 1, fa1, fb1);
+  }
+#undef CCT_FETCH
+#undef CCT_STASH
+#undef CCT_FRAGS
 }
 
 template <class T, bool A_KC, bool B_KC>
@@ -141,15 +281,17 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
   using LA = OperandLayout<T, A_KC, T::BM>;
   using LB = OperandLayout<T, B_KC, T::BN>;
   __shared__ __attribute__((aligned(16))) float smem[2 * (LA::SIZE + LB::SIZE)];
-  constexpr int STAGE = LA::SIZE + LB::SIZE;  // stage s: A at smem + s*STAGE, B right after it
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int wm0 = (wave / T::WGN) * T::WM, wn0 = (wave % T::WGN) * T::WN;
 
-  // tile id: the dimension with fewer tiles runs fastest so that neighbouring workgroups on one
-  // XCD share the larger operand tile in L2
-  const uint32_t id = xcd_remap(blockIdx.x, g.ntiles);
+  // One flat grid over (K slice, tile) with the tile index fastest: the workgroups that share an
+  // operand panel (same K slice, neighbouring tiles) get consecutive ids on one XCD and run
+  // together.  Within a K slice the dimension with fewer tiles runs fastest.
+  const uint32_t flat = xcd_remap(blockIdx.x, g.nblocks);
+  const uint32_t kslice = flat / g.ntiles;
+  const uint32_t id = flat - kslice * g.ntiles;
   int tm, tn;
   if (g.tiles_m <= g.tiles_n) {
     tm = id % g.tiles_m; tn = id / g.tiles_m;
@@ -157,7 +299,7 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
     tn = id % g.tiles_n; tm = id / g.tiles_n;
   }
   const int m0 = tm * T::BM, n0 = tn * T::BN;
-  const int kbeg = blockIdx.y * g.kchunk;
+  const int kbeg = kslice * g.kchunk;
   const int kend = min(g.K, kbeg + g.kchunk);
   const int nk = (kend - kbeg + T::BK - 1) / T::BK;
 
@@ -169,44 +311,12 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  float4 ra[LA::NV], rb[LB::NV];
-  if (nk > 0) {
-    load_tile<T, A_KC, T::BM>(ra, g.A, g.lda, m0, kbeg, g.M, kend, g.a_vec, tid);
-    load_tile<T, B_KC, T::BN>(rb, g.B, g.ldb, n0, kbeg, g.N, kend, g.b_vec, tid);
-    store_tile<T, A_KC, T::BM>(smem, ra, tid);
-    store_tile<T, B_KC, T::BN>(smem + LA::SIZE, rb, tid);
-  }
-  __syncthreads();
-
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    const bool more = (kt + 1 < nk);
-    if (more) {
-      const int k0 = kbeg + (kt + 1) * T::BK;
-      load_tile<T, A_KC, T::BM>(ra, g.A, g.lda, m0, k0, g.M, kend, g.a_vec, tid);
-      load_tile<T, B_KC, T::BN>(rb, g.B, g.ldb, n0, k0, g.N, kend, g.b_vec, tid);
-    }
-    const float *as = smem + cur * STAGE;
-    const float *bs = as + LA::SIZE;
-#pragma unroll
-    for (int kg = 0; kg < T::BK / 8; ++kg) {
-      float fa[T::TM][4], fb[T::TN][4];
-      load_frags<T, A_KC, T::BM, T::TM>(fa, as, wm0, kg, lane);
-      load_frags<T, B_KC, T::BN, T::TN>(fb, bs, wn0, kg, lane);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int a = 0; a < T::TM; ++a)
-#pragma unroll
-          for (int b = 0; b < T::TN; ++b)
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[a][i], fb[b][i], acc[a][b], 0, 0, 0);
-    }
-    if (more) {
-      store_tile<T, A_KC, T::BM>(smem + (cur ^ 1) * STAGE, ra, tid);
-      store_tile<T, B_KC, T::BN>(smem + (cur ^ 1) * STAGE + LA::SIZE, rb, tid);
-    }
-    __syncthreads();
-  }
+  const bool interior = g.a_vec && g.b_vec && (m0 + T::BM <= g.M) && (n0 + T::BN <= g.N) &&
+                        ((kend - kbeg) % T::BK == 0);
+  if (interior)
+    gemm_mainloop<T, A_KC, B_KC, false>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
+  else
+    gemm_mainloop<T, A_KC, B_KC, true>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
 
   // epilogue: accumulator register v of lane (r,h) is C[8*(v/4) + 4*h + v%4][r] of its 32x32 tile
   const int r = lane & 31, h = lane >> 5;
@@ -230,11 +340,15 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
         const float x = acc[a][b][v];
         if (g.epi == EPI_ALPHA_BETA) {
           float *c = g.C + (size_t)row * g.ldc + col_off;
-          *c = (g.beta == 0.0f) ? g.alpha * x : g.alpha * x + g.beta * (*c);
+          const float y = (g.beta == 0.0f) ? g.alpha * x : g.alpha * x + g.beta * (*c);
+          if (g.nt_store) __builtin_nontemporal_store(y, c);
+          else *c = y;
         } else if (g.epi == EPI_SPLITK_PARTIAL) {
-          g.ws[((size_t)blockIdx.y * g.M + row) * g.N + col_off] = x;
+          g.ws[((size_t)kslice * g.M + row) * g.N + col_off] = x;
         } else {
-          g.C[(size_t)row * g.fmap + col_off] = g.bias ? x + g.bias[row] : x;
+          const float y = g.bias ? x + g.bias[row] : x;
+          if (g.nt_store) __builtin_nontemporal_store(y, g.C + (size_t)row * g.fmap + col_off);
+          else g.C[(size_t)row * g.fmap + col_off] = y;
         }
       }
     }
@@ -266,7 +380,11 @@ static int launch_cfg(GemmArgs &g, bool a_kc, bool b_kc, int splits, hipStream_t
   g.tiles_m = (g.M + T::BM - 1) / T::BM;
   g.tiles_n = (g.N + T::BN - 1) / T::BN;
   g.ntiles = (uint32_t)g.tiles_m * g.tiles_n;
-  dim3 grid(g.ntiles, splits), block(T::THREADS);
+  g.splits = splits;
+  const size_t nblocks = (size_t)g.ntiles * splits;
+  if (nblocks >= (1ull << 31)) return set_error(CCT_HIP_EINVAL, "sgemm: too many workgroups");
+  g.nblocks = (uint32_t)nblocks;
+  dim3 grid(g.nblocks), block(T::THREADS);
   if (a_kc && b_kc) hipLaunchKernelGGL((gemm_kernel<T, true, true>), grid, block, 0, st, g);
   else if (a_kc && !b_kc) hipLaunchKernelGGL((gemm_kernel<T, true, false>), grid, block, 0, st, g);
   else if (!a_kc && b_kc) hipLaunchKernelGGL((gemm_kernel<T, false, true>), grid, block, 0, st, g);
@@ -288,6 +406,10 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   g.div_fmap = make_fastdiv((uint32_t)g.fmap); g.bias = bias; g.ws = nullptr;
   g.a_vec = ((uintptr_t)A % 16 == 0) && (lda % 4 == 0);
   g.b_vec = ((uintptr_t)B % 16 == 0) && (ldb % 4 == 0);
+  {
+    const char *e = getenv("CCT_HIP_GEMM_NT");
+    g.nt_store = e ? atoi(e) : 0;
+  }
   if (K <= 0) g.K = 0;  // degenerate: C = beta*C through the normal epilogue with zero accumulators
 
   // tile choice: largest macro tile that still yields at least one workgroup per compute unit
