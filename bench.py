@@ -93,12 +93,82 @@ def cpu_baseline(cfg, seed):
     }
 
 
+def net_iteration(args, torch, np):
+    """BASELINE.json configs[3] / configs[4]: one step = forward + backward + SGD update of every layer,
+    synthetic images and labels already on the device."""
+    from caffecontroll_amd import HIPDriver, nets
+    drv = HIPDriver(0)
+    drv.set_stream(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(1234 + (4 if args.workload == "lenet" else 5))
+    if args.workload == "lenet":
+        B, D, S, classes = 64, 1, 28, 10
+        layers = nets.lenet_layers()
+        x = rng.uniform(0, 1, (B, D, S, S)).astype(np.float32)
+        solver = nets.solver_param(base_lr=0.01, momentum=0.9, weight_decay=0.0005, lr_policy="inv",
+                                   gamma=0.0001, power=0.75)
+    else:
+        B, D, S, classes = 256, 3, 227, 1000
+        layers = nets.caffenet_layers(groups=True)
+        x = rng.uniform(0, 255, (B, D, S, S)).astype(np.float32)
+        x -= np.array([104, 117, 123], np.float32)[None, :, None, None]
+        solver = nets.solver_param(base_lr=0.01, momentum=0.9, weight_decay=0.0005, lr_policy="step",
+                                   gamma=0.1, stepsize=100000)
+    labels = rng.integers(0, classes, B).astype(np.float32)
+    net = nets.Net(B, D, S, layers, solver)
+    # fillers of the reference's prototxts: gaussian weights (std 0.01; 0.005 for fc6/fc7), constant bias
+    n_fc = 0
+    for li, L in enumerate(layers):
+        for gi in range(max(L.group, 1)):
+            wp, wn = net.tensor(li, nets.MODEL, gi)
+            if not wp:
+                continue
+            std = 0.01
+            if L.type == nets.FC and args.workload == "caffenet":
+                n_fc += 1
+                std = 0.005 if n_fc <= 2 else 0.01
+            if args.workload == "lenet":
+                std = float(np.sqrt(1.0 / (wn / L.num_output)))  # xavier-sized
+            w = (rng.standard_normal(wn, dtype=np.float32) * np.float32(std))
+            drv.memcpy(wp, w.ctypes.data, w.nbytes, 0)
+            bp, bn = net.tensor(li, nets.BIAS, gi)
+            bias = np.full(bn, 0.1 if args.workload == "caffenet" else 0.0, np.float32)
+            drv.memcpy(bp, bias.ctypes.data, bias.nbytes, 0)
+    drv.memcpy(net.input_ptr(), x.ctypes.data, x.nbytes, 0)
+    drv.memcpy(net.labels_ptr(), labels.ctypes.data, labels.nbytes, 0)
+
+    def step():
+        net.forward()
+        net.backward()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    loss = net.loss() / B
+    ms = elapsed * 1e3 / args.steps
+    return {
+        "metric": "ms per %s train iteration (1 GPU)" % ("LeNet" if args.workload == "lenet" else "AlexNet-shaped"),
+        "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic", "images_per_sec": round(B * 1e3 / ms, 1),
+        "config": {"workload": "%s: fwd+bwd+SGD, batch %d, %dx%dx%d inputs, %d classes%s" % (
+            args.workload, B, D, S, S, classes, ", conv2/4/5 in 2 groups" if args.workload == "caffenet" else "")},
+        "final_loss_per_image": round(float(loss), 5),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="alexnet_conv2", choices=sorted(CONFIGS))
+    ap.add_argument("--workload", default="alexnet_conv2", choices=sorted(CONFIGS) + ["lenet", "caffenet"],
+                    help="a single conv layer (default: AlexNet conv2, the headline config) or a whole training "
+                         "iteration of LeNet (b=64) / CaffeNet (b=256, grouped conv2/4/5)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="staged forward (GEMM, remap, bias) and separate bias gradient")
     ap.add_argument("--no-data-grad", action="store_true", help="first-layer mode: skip data-gradient GEMM and lift")
@@ -130,6 +200,9 @@ def main():
         drv.device_sync()
         print(json.dumps({"copy_calibration_bytes_read": nbytes, "copy_calibration_bytes_written": nbytes,
                           "copies": 5}))
+        return
+    if args.workload in ("lenet", "caffenet"):
+        print(json.dumps(net_iteration(args, torch, np)))
         return
     cfg = args.workload
     b, d, n, k, s, p, o = CONFIGS[cfg]

@@ -3,6 +3,7 @@
 
 #include "../../include/cct_bridge.h"
 #include "host/ConvolutionBridge.h"
+#include "host/Network.h"
 #include "host/ParallelizedBridge.h"
 
 using namespace cct;
@@ -108,6 +109,97 @@ int cct_conv_bridge_stage_ms(cct_conv_bridge *h, float ms[CCT_CONV_STAGE_COUNT])
   if (!h || !ms) return CCT_HIP_EINVAL;
   static_assert(CCT_CONV_STAGE_COUNT == STAGE_COUNT, "stage tables out of sync");
   for (int i = 0; i < STAGE_COUNT; ++i) ms[i] = h->pbridge->sub_bridge()->stage_ms(i);
+  return 0;
+}
+
+struct cct_net {
+  Network *net;
+};
+
+int cct_net_create(cct_net **out, int batch, int depth, int size, const cct_layer_spec *layers, int n_layers,
+                   const cct_solver_param *solver) {
+  if (!out || !layers || batch <= 0 || depth <= 0 || size <= 0 || n_layers <= 0) return CCT_HIP_EINVAL;
+  cct_net *h = new cct_net;
+  h->net = new Network(batch, depth, size, layers, n_layers, solver);
+  *out = h;
+  return 0;
+}
+
+int cct_net_destroy(cct_net *h) {
+  if (!h) return 0;
+  delete h->net;
+  delete h;
+  return 0;
+}
+
+float *cct_net_input(cct_net *h) { return h->net->input(); }
+float *cct_net_labels(cct_net *h) { return h->net->labels(); }
+int cct_net_num_layers(cct_net *h) { return h->net->num_layers(); }
+
+void *cct_net_tensor(cct_net *h, int layer, int group, int which, size_t *n) {
+  if (n) *n = 0;
+  if (!h || layer < 0 || layer >= h->net->num_layers()) return nullptr;
+  Network::Node &nd = h->net->node(layer);
+  if (group < 0 || group >= (int)nd.bridges.size()) return nullptr;
+  Network::BridgeT *b = nd.bridges[group];
+  LogicalCube<float> *c = nullptr;
+  switch (which) {
+    case 0: c = b->get_model_cube(); break;
+    case 1: c = b->get_bias_cube(); break;
+    case 2: c = b->get_model_grad_cube(); break;
+    case 3: c = b->get_bias_grad_cube(); break;
+    case 4: c = nd.out->p_data_cube; break;
+    case 5: c = nd.in->p_gradient_cube; break;
+    case 6:
+      if (nd.spec.type == CCT_LAYER_DROPOUT) {
+        auto *m = static_cast<DropoutBridge<float, HIPDriver> *>(b)->get_mask_cube();
+        if (n) *n = m->n_elements;
+        return m->get_p_data();
+      }
+      if (nd.spec.type == CCT_LAYER_MAXPOOL) {
+        auto *m = static_cast<MaxPoolingBridge<float, HIPDriver> *>(b)->get_max_index_cube();
+        if (n) *n = m->n_elements;
+        return m->get_p_data();
+      }
+      return nullptr;
+    default: return nullptr;
+  }
+  if (!c) return nullptr;
+  if (n) *n = c->n_elements;
+  return c->get_p_data();
+}
+
+int cct_net_set_train(cct_net *h, int train) {
+  if (!h) return CCT_HIP_EINVAL;
+  h->net->set_train(train != 0);
+  return 0;
+}
+
+int cct_net_freeze_dropout_masks(cct_net *h, int freeze) {
+  if (!h) return CCT_HIP_EINVAL;
+  for (int i = 0; i < h->net->num_layers(); ++i) {
+    Network::Node &nd = h->net->node(i);
+    if (nd.spec.type == CCT_LAYER_DROPOUT)
+      static_cast<DropoutBridge<float, HIPDriver> *>(nd.bridges[0])->generate_mask = (freeze == 0);
+  }
+  return 0;
+}
+
+int cct_net_forward(cct_net *h) {
+  if (!h) return CCT_HIP_EINVAL;
+  h->net->forward();
+  return 0;
+}
+
+int cct_net_backward(cct_net *h) {
+  if (!h) return CCT_HIP_EINVAL;
+  h->net->backward();
+  return 0;
+}
+
+int cct_net_loss(cct_net *h, float *loss_sum) {
+  if (!h || !loss_sum) return CCT_HIP_EINVAL;
+  *loss_sum = h->net->loss();
   return 0;
 }
 

@@ -64,6 +64,19 @@ __global__ __launch_bounds__(TPB) void remap_kernel(float *__restrict__ dst, con
   for (uint32_t i = blockIdx.y * TPB + threadIdx.x; i < rc; i += gridDim.y * TPB) d[i] = s[i];
 }
 
+// ---- depth-slice copy: part [B][dc][rc] <-> channels [d_off, d_off+dc) of whole [B][D][rc] ----------
+__global__ __launch_bounds__(TPB) void depth_slice_kernel(float *__restrict__ part, float *__restrict__ whole,
+                                                          uint32_t per_image, uint32_t whole_stride,
+                                                          uint32_t whole_off, int gather) {
+  const uint32_t b = blockIdx.y;
+  float *p = part + (size_t)b * per_image;
+  float *w = whole + (size_t)b * whole_stride + whole_off;
+  for (uint32_t i = blockIdx.x * TPB + threadIdx.x; i < per_image; i += gridDim.x * TPB) {
+    if (gather) p[i] = w[i];
+    else w[i] = p[i];
+  }
+}
+
 // ---- bias forward: out[slice][i] += bias[slice % depth] ----------------------------------------
 __global__ __launch_bounds__(TPB) void bias_forward_kernel(float *__restrict__ out,
                                                            const float *__restrict__ bias, uint32_t fmap,
@@ -394,6 +407,23 @@ int cct_hip_remap(float *dst, const float *src, const cct_pmap_helper *a) {
   if (gy > 64) gy = 64;
   hipLaunchKernelGGL(remap_kernel, dim3((uint32_t)slices, gy), dim3(TPB), 0, ctx().stream, dst, src,
                      (uint32_t)rc, (uint32_t)a->sD, make_fastdiv((uint32_t)a->sB));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_copy_depth_slice(float *part, float *whole, int B, int d_total, int d_off, int d_count, size_t rc,
+                             int gather) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(part && whole, "copy_depth_slice: null argument");
+  CCT_REQUIRE(B >= 0 && d_total > 0 && d_off >= 0 && d_count > 0 && d_off + d_count <= d_total && rc > 0,
+              "copy_depth_slice: bad slice [%d, %d) of %d", d_off, d_off + d_count, d_total);
+  CCT_REQUIRE((size_t)d_total * rc < (1ull << 31) && B <= 65535, "copy_depth_slice: tensor too large");
+  if (B == 0) return 0;
+  const uint32_t per_image = (uint32_t)(d_count * rc);
+  uint32_t gx = (per_image + TPB - 1) / TPB;
+  if (gx > 1024) gx = 1024;
+  hipLaunchKernelGGL(depth_slice_kernel, dim3(gx, B), dim3(TPB), 0, ctx().stream, part, whole, per_image,
+                     (uint32_t)(d_total * rc), (uint32_t)(d_off * rc), gather);
   CCT_LAUNCH_CHECK();
   return 0;
 }

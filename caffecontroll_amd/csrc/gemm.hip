@@ -372,6 +372,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *__restrict__ 
 }
 
 typedef Tile<256, 128, 16, 2, 2> TileL;
+typedef Tile<128, 256, 16, 2, 2> TileLT;  // same wave work as TileL with the long side along N
 typedef Tile<128, 128, 16, 2, 2> TileM;
 typedef Tile<64, 64, 16, 2, 2> TileS;
 
@@ -412,14 +413,21 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   }
   if (K <= 0) g.K = 0;  // degenerate: C = beta*C through the normal epilogue with zero accumulators
 
-  // tile choice: largest macro tile that still yields at least one workgroup per compute unit
+  // tile choice: the big tiles (256x128 or 128x256, whichever pads M x N less) when the problem is
+  // large enough to fill the device with them, else 128x128, else 64x64
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
   auto ntiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-  int cfg;  // 0 = L, 1 = M, 2 = S
-  if (M > 128 && N >= 128 && (M % 256 == 0 || M > 512)) cfg = 0;
-  else if (M > 64 && N > 64) cfg = 1;
-  else cfg = 2;
-  const int bm = cfg == 0 ? 256 : cfg == 1 ? 128 : 64, bn = cfg == 2 ? 64 : 128, bk = 16;
+  auto padded = [&](int bm, int bn) { return (double)ntiles(bm, bn) * bm * bn; };
+  int cfg;  // 0 = L (256x128), 1 = M (128x128), 2 = S (64x64), 3 = LT (128x256)
+  if (M > 128 && N > 128 && padded(256, 128) <= 1.15 * padded(128, 128) && padded(256, 128) <= padded(128, 256))
+    cfg = 0;
+  else if (M > 64 && N > 128 && padded(128, 256) <= 1.15 * padded(128, 128))
+    cfg = 3;
+  else if (M > 64 && N > 64)
+    cfg = 1;
+  else
+    cfg = 2;
+  const int bm = cfg == 0 ? 256 : cfg == 2 ? 64 : 128, bn = cfg == 3 ? 256 : cfg == 2 ? 64 : 128, bk = 16;
   const long tiles = ntiles(bm, bn);
 
   // split-K only for the plain epilogue when the tile grid cannot fill the device
@@ -445,6 +453,7 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
     g.epi = EPI_SPLITK_PARTIAL;
   }
   int rc = cfg == 0   ? launch_cfg<TileL>(g, a_kc, b_kc, splits, st)
+           : cfg == 3 ? launch_cfg<TileLT>(g, a_kc, b_kc, splits, st)
            : cfg == 1 ? launch_cfg<TileM>(g, a_kc, b_kc, splits, st)
                       : launch_cfg<TileS>(g, a_kc, b_kc, splits, st);
   if (rc) return rc;

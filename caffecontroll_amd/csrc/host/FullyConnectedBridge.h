@@ -1,0 +1,135 @@
+// Fully connected operator for the HIP driver: three sgemm_new calls, no lowering.
+// Counterpart of FullyConnectedBridge (src/bridges/FullyConnectedBridge_impl.hxx:13-110 ctor,
+// 169-234 forward, 255-326 backward).  The model cube is [oD][iD][K][K] with K = iR, i.e. the
+// GEMM matrix [O x I] with I = iR*iC*iD.
+#pragma once
+#include <cstdio>
+#include <cstdlib>
+
+#include "AbstractBridge.h"
+
+namespace cct {
+
+template <typename DataType, typename DriverClass>
+class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
+  typedef AbstractBridge<DataType, DriverClass> Base;
+
+ public:
+  using Base::iR; using Base::iC; using Base::iD; using Base::iB;
+  using Base::oR; using Base::oC; using Base::oD; using Base::oB;
+  using Base::needs_to_calc_backward_grad;
+  using Base::layer_param; using Base::solver_param; using Base::p_driver;
+  using Base::p_input_layer; using Base::p_output_layer;
+  typedef Layer<DataType> LayerType;
+  typedef LogicalCube<DataType> LogicalCubeType;
+
+  const size_t K;
+  const size_t num_output_features;
+  const bool bias_term;
+  LogicalCubeType *p_model_cube;
+  LogicalCubeType *p_bias_cube;
+
+  FullyConnectedBridge(LayerType *const _p_input_layer, LayerType *const _p_output_layer,
+                       const cnn::LayerParameter *const _layer_param,
+                       const cnn::SolverParameter *const _solver_param, DriverClass *const _p_driver)
+      : Base(_p_input_layer, _p_output_layer, _layer_param, _solver_param, _p_driver), K(_p_input_layer->dR),
+        num_output_features(_layer_param->inner_product_param().num_output()),
+        bias_term(_layer_param->inner_product_param().bias_term()), p_model_cube(nullptr), p_bias_cube(nullptr),
+        p_bias_gradient_cube(nullptr) {
+    if (oR != 1 || oC != 1 || iB != oB || oD != num_output_features || iR != iC) {
+      std::fprintf(stderr, "FullyConnectedBridge: inconsistent layer shapes\n");
+      std::abort();
+    }
+    p_model_cube = new LogicalCubeType(K, K, iD, oD, p_driver);
+    initialize_logical_cube(p_model_cube, _layer_param->inner_product_param().weight_filler());
+    p_model_gradient_cube = new LogicalCubeType(K, K, iD, oD, p_driver);
+    DeviceMemoryPointer mg = p_model_gradient_cube->get_device_pointer(p_driver);
+    p_driver->sconstant_initialize(&mg, DataType(0.));
+    if (bias_term) {
+      p_bias_cube = new LogicalCubeType(1, 1, oD, 1, p_driver);
+      initialize_logical_cube(p_bias_cube, _layer_param->inner_product_param().bias_filler());
+      p_bias_gradient_cube = new LogicalCubeType(1, 1, oD, 1, p_driver);
+      DeviceMemoryPointer bg = p_bias_gradient_cube->get_device_pointer(p_driver);
+      p_driver->sconstant_initialize(&bg, DataType(0.));
+    }
+    // GEMM dimensions, named as in the reference
+    data_R = (int)iB;                 // rows of the data matrix (batch)
+    data_C = (int)(iR * iC * iD);     // its columns (features in)
+    model_R = (int)oD;                // rows of the model matrix (features out)
+    model_C = data_C;
+  }
+
+  ~FullyConnectedBridge() {
+    delete p_model_cube;
+    delete p_model_gradient_cube;
+    delete p_bias_cube;
+    delete p_bias_gradient_cube;
+  }
+
+  LogicalCubeType *get_model_cube() override { return p_model_cube; }
+  LogicalCubeType *get_bias_cube() override { return p_bias_cube; }
+  LogicalCubeType *get_model_grad_cube() override { return p_model_gradient_cube; }
+  LogicalCubeType *get_bias_grad_cube() override { return p_bias_gradient_cube; }
+
+  // Y[B x O] = X[B x I] * W^T, then the bias through forward_bias with a 1x1 feature map
+  // (the non-CPU branch of the reference, :224-228)
+  void forward() override {
+    this->report_forward_history.reset();
+    LogicalCubeType *input_d_cube = p_input_layer->p_data_cube;
+    LogicalCubeType *output_d_cube = p_output_layer->p_data_cube;
+    p_driver->sgemm_new(CblasNoTrans, CblasTrans, data_R, model_R, model_C, 1.f, input_d_cube->get_p_data(),
+                        p_model_cube->get_p_data(), 0.f, output_d_cube->get_p_data());
+    if (bias_term) {
+      DeviceMemoryPointer output = output_d_cube->get_device_pointer(p_driver);
+      DeviceMemoryPointer bias = p_bias_cube->get_device_pointer(p_driver);
+      p_driver->forward_bias(&bias, &output, 1, (int)oD, (int)iB);
+    }
+    this->report_forward_history.end();
+  }
+
+  // db = dY^T * ones;  dX[B x I] = dY * W;  dW[O x I] = dY^T * X
+  void backward() override {
+    this->report_backward_updateweight_history.reset();
+    LogicalCubeType *output_g_cube = p_output_layer->p_gradient_cube;
+    LogicalCubeType *input_g_cube = p_input_layer->p_gradient_cube;
+    LogicalCubeType *input_d_cube = p_input_layer->p_data_cube;
+    if (bias_term) {
+      DeviceMemoryPointer output = output_g_cube->get_device_pointer(p_driver);
+      DeviceMemoryPointer bias = p_bias_gradient_cube->get_device_pointer(p_driver);
+      p_driver->backward_bias_fc(&bias, &output, (int)oD, (int)iB);
+    }
+    // the reference always computes the data gradient here (:306-308); it is skipped when the
+    // caller says the layer below does not need it
+    if (needs_to_calc_backward_grad)
+      p_driver->sgemm_new(CblasNoTrans, CblasNoTrans, data_R, model_C, model_R, 1.f, output_g_cube->get_p_data(),
+                          p_model_cube->get_p_data(), 0.f, input_g_cube->get_p_data());
+    p_driver->sgemm_new(CblasTrans, CblasNoTrans, model_R, model_C, data_R, 1.f, output_g_cube->get_p_data(),
+                        input_d_cube->get_p_data(), 0.f, p_model_gradient_cube->get_p_data());
+    this->report_backward_updateweight_history.end();
+  }
+
+ protected:
+  LogicalCubeType *p_model_gradient_cube;
+  LogicalCubeType *p_bias_gradient_cube;
+  int data_R, data_C, model_R, model_C;
+
+  void initialize_logical_cube(const LogicalCubeType *cube, const cnn::FillerParameter &filler_param) {
+    DeviceMemoryPointer data = cube->get_device_pointer(p_driver);
+    const std::string &type = filler_param.type();
+    if (type == "constant") {
+      p_driver->sconstant_initialize(&data, (DataType)filler_param.value());
+    } else if (type == "xavier") {
+      p_driver->sinitialize_xavier(&data, cube->B, solver_param->random_seed());
+    } else if (type == "bernoulli") {
+      p_driver->sbernoulli_initialize(&data, (DataType)filler_param.value(), solver_param->random_seed());
+    } else if (type == "gaussian") {
+      p_driver->sgaussian_initialize(&data, (DataType)filler_param.mean(), (DataType)filler_param.std(),
+                                     solver_param->random_seed());
+    } else {
+      std::fprintf(stderr, "ERROR! INITIALIZATION TYPE NOT SUPPORTED: %s\n", type.c_str());
+      std::abort();
+    }
+  }
+};
+
+}  // namespace cct

@@ -1,0 +1,234 @@
+// A linear chain of bridges on the HIP driver, each wrapped in a one-partition ParallelizedBridge:
+// the device-resident equivalent of what DeepNet::construct_network builds from a prototxt
+// (src/DeepNet.h:968-2030) and of run_forward_pass / run_backward_pass (src/DeepNet.h:171-266),
+// for nets that are a plain sequence of layers (LeNet, CaffeNet).  Layer descriptions come as a C
+// array instead of a parsed prototxt.
+//
+// Placement rules kept from the reference:
+//   * output sizes: conv (R+2p-K)/s+1 (:112-115), pooling floor((R-K)/s)+1 unpadded (:1374-1376);
+//   * the first weight layer does not compute a data gradient (:1108-1110);
+//   * ReLU and dropout run in place on their input layer (the reference shares the layers on the
+//     GPU: ParallelizedBridge.h:183-198);
+//   * `group` > 1 is realised as `group` independent convolutions on channel slices whose outputs
+//     are concatenated along depth (the reference's two-tower Split/Concat arrangement,
+//     src/DeepNet.h:1700-1757); slices are moved with a strided device copy.
+#pragma once
+#include <memory>
+#include <vector>
+
+#include "../../../include/cct_bridge.h"
+#include "ConvolutionBridge.h"
+#include "FullyConnectedBridge.h"
+#include "ParallelizedBridge.h"
+#include "SimpleBridges.h"
+
+namespace cct {
+
+class Network {
+ public:
+  typedef Layer<float> LayerT;
+  typedef LogicalCube<float> CubeT;
+  typedef AbstractBridge<float, HIPDriver> BridgeT;
+
+  struct Node {
+    cct_layer_spec spec;
+    LayerT *in = nullptr;   // not owned here (owned through layers_)
+    LayerT *out = nullptr;
+    std::vector<BridgeT *> bridges;              // one per group (1 for everything but grouped conv)
+    std::vector<LayerT *> group_in, group_out;   // per-group contiguous layers (grouped conv only)
+    std::vector<cnn::LayerParameter *> params;
+  };
+
+  Network(int batch, int depth, int size, const cct_layer_spec *specs, int n_specs, const cct_solver_param *sp)
+      : batch_(batch) {
+    if (sp) {
+      solver_.base_lr_ = sp->base_lr; solver_.momentum_ = sp->momentum; solver_.gamma_ = sp->gamma;
+      solver_.power_ = sp->power; solver_.weight_decay_ = sp->weight_decay; solver_.stepsize_ = sp->stepsize;
+      solver_.max_iter_ = sp->max_iter; solver_.random_seed_ = sp->random_seed;
+      if (sp->lr_policy) solver_.lr_policy_ = sp->lr_policy;
+      if (sp->regularization_type) solver_.regularization_type_ = sp->regularization_type;
+    }
+    labels_ = new CubeT(1, 1, 1, batch, &driver_);
+    LayerT *cur = new_layer(size, size, depth);
+    bool first_weight_layer = true;
+    for (int i = 0; i < n_specs; ++i) {
+      Node nd;
+      nd.spec = specs[i];
+      nd.in = cur;
+      const cct_layer_spec &s = specs[i];
+      const size_t R = cur->dR, D = cur->dD;
+      switch (s.type) {
+        case CCT_LAYER_CONV: {
+          const int g = s.group > 1 ? s.group : 1;
+          if (D % g || s.num_output % g) fail("group must divide input depth and num_output");
+          const size_t m = (R + 2 * s.pad - s.kernel_size) / s.stride + 1;
+          nd.out = new_layer(m, m, s.num_output);
+          for (int gi = 0; gi < g; ++gi) {
+            cnn::LayerParameter *lp = new_param(s);
+            lp->convolution_param_.num_output_ = s.num_output / g;
+            lp->convolution_param_.kernel_size_ = s.kernel_size;
+            lp->convolution_param_.stride_ = s.stride;
+            lp->convolution_param_.pad_ = s.pad;
+            lp->convolution_param_.bias_term_ = s.bias_term != 0;
+            nd.params.push_back(lp);
+            LayerT *gin = cur, *gout = nd.out;
+            if (g > 1) {
+              gin = new_layer(R, R, D / g);
+              gout = new_layer(m, m, s.num_output / g);
+              nd.group_in.push_back(gin);
+              nd.group_out.push_back(gout);
+            }
+            auto *b = new ParallelizedBridge<float, ConvolutionBridge, HIPDriver>(gin, gout, lp, &solver_, &driver_);
+            b->needs_to_calc_backward_grad = !first_weight_layer;
+            nd.bridges.push_back(b);
+          }
+          first_weight_layer = false;
+          break;
+        }
+        case CCT_LAYER_FC: {
+          nd.out = new_layer(1, 1, s.num_output);
+          cnn::LayerParameter *lp = new_param(s);
+          lp->inner_product_param_.num_output_ = s.num_output;
+          lp->inner_product_param_.bias_term_ = s.bias_term != 0;
+          nd.params.push_back(lp);
+          auto *b = new ParallelizedBridge<float, FullyConnectedBridge, HIPDriver>(cur, nd.out, lp, &solver_, &driver_);
+          b->needs_to_calc_backward_grad = !first_weight_layer;
+          first_weight_layer = false;
+          nd.bridges.push_back(b);
+          break;
+        }
+        case CCT_LAYER_RELU: {
+          nd.out = cur;  // in place
+          nd.params.push_back(new_param(s));
+          nd.bridges.push_back(new ReLUBridge<float, HIPDriver>(cur, cur, nd.params[0], &solver_, &driver_));
+          break;
+        }
+        case CCT_LAYER_DROPOUT: {
+          nd.out = cur;  // in place
+          cnn::LayerParameter *lp = new_param(s);
+          lp->dropout_param_.dropout_ratio_ = s.dropout_ratio;
+          nd.params.push_back(lp);
+          nd.bridges.push_back(new DropoutBridge<float, HIPDriver>(cur, cur, lp, &solver_, &driver_));
+          break;
+        }
+        case CCT_LAYER_MAXPOOL: {
+          const size_t m = (R - s.kernel_size) / s.stride + 1;
+          nd.out = new_layer(m, m, D);
+          cnn::LayerParameter *lp = new_param(s);
+          lp->pooling_param_.kernel_size_ = s.kernel_size;
+          lp->pooling_param_.stride_ = s.stride;
+          nd.params.push_back(lp);
+          nd.bridges.push_back(new MaxPoolingBridge<float, HIPDriver>(cur, nd.out, lp, &solver_, &driver_));
+          break;
+        }
+        case CCT_LAYER_LRN: {
+          nd.out = new_layer(R, R, D);
+          cnn::LayerParameter *lp = new_param(s);
+          lp->lrn_param_.local_size_ = s.lrn_local_size;
+          lp->lrn_param_.alpha_ = s.lrn_alpha;
+          lp->lrn_param_.beta_ = s.lrn_beta;
+          nd.params.push_back(lp);
+          nd.bridges.push_back(new LRNBridge<float, HIPDriver>(cur, nd.out, lp, &solver_, &driver_));
+          break;
+        }
+        case CCT_LAYER_SOFTMAXLOSS: {
+          nd.out = new_layer(R, R, D);
+          nd.params.push_back(new_param(s));
+          softmax_ = new SoftmaxLossBridge<float, HIPDriver>(cur, nd.out, nd.params[0], &solver_, &driver_, labels_);
+          nd.bridges.push_back(softmax_);
+          break;
+        }
+        default:
+          fail("unknown layer type");
+      }
+      cur = nd.out;
+      nodes_.push_back(nd);
+    }
+  }
+
+  ~Network() {
+    for (Node &nd : nodes_) {
+      for (BridgeT *b : nd.bridges) delete b;
+      for (cnn::LayerParameter *p : nd.params) delete p;
+    }
+    for (LayerT *l : layers_) delete l;
+    delete labels_;
+  }
+  Network(const Network &) = delete;
+  Network &operator=(const Network &) = delete;
+
+  float *input() { return layers_[0]->p_data_cube->get_p_data(); }
+  float *labels() { return labels_->get_p_data(); }
+  int num_layers() const { return (int)nodes_.size(); }
+  Node &node(int i) { return nodes_[i]; }
+  HIPDriver &driver() { return driver_; }
+
+  void set_train(bool train) {
+    for (Node &nd : nodes_)
+      if (nd.spec.type == CCT_LAYER_DROPOUT)
+        static_cast<DropoutBridge<float, HIPDriver> *>(nd.bridges[0])->train = train;
+  }
+
+  // DeepNet::run_forward_pass: every bridge in order
+  void forward() {
+    for (Node &nd : nodes_) {
+      const size_t g = nd.group_in.size();
+      for (size_t gi = 0; gi < g; ++gi)
+        slice_copy(nd.group_in[gi]->p_data_cube, nd.in->p_data_cube, gi, /*gather=*/true);
+      for (BridgeT *b : nd.bridges) b->forward();
+      for (size_t gi = 0; gi < g; ++gi)
+        slice_copy(nd.group_out[gi]->p_data_cube, nd.out->p_data_cube, gi, /*gather=*/false);
+    }
+  }
+
+  // DeepNet::run_backward_pass: every bridge in reverse order; ParallelizedBridge::backward applies
+  // the SGD update of its layer
+  void backward() {
+    for (int i = (int)nodes_.size() - 1; i >= 0; --i) {
+      Node &nd = nodes_[i];
+      const size_t g = nd.group_in.size();
+      for (size_t gi = 0; gi < g; ++gi)
+        slice_copy(nd.group_out[gi]->p_gradient_cube, nd.out->p_gradient_cube, gi, /*gather=*/true);
+      for (BridgeT *b : nd.bridges) b->backward();
+      if (nd.bridges[0]->needs_to_calc_backward_grad)
+        for (size_t gi = 0; gi < g; ++gi)
+          slice_copy(nd.group_in[gi]->p_gradient_cube, nd.in->p_gradient_cube, gi, /*gather=*/false);
+    }
+  }
+
+  float loss() { return softmax_ ? softmax_->get_loss() : 0.f; }
+
+ private:
+  HIPDriver driver_;
+  cnn::SolverParameter solver_;
+  int batch_;
+  CubeT *labels_;
+  std::vector<LayerT *> layers_;
+  std::vector<Node> nodes_;
+  SoftmaxLossBridge<float, HIPDriver> *softmax_ = nullptr;
+
+  static void fail(const char *msg) {
+    std::fprintf(stderr, "Network: %s\n", msg);
+    std::abort();
+  }
+  LayerT *new_layer(size_t R, size_t C, size_t D) {
+    LayerT *l = new LayerT(new CubeT(R, C, D, batch_, &driver_), new CubeT(R, C, D, batch_, &driver_));
+    layers_.push_back(l);
+    return l;
+  }
+  static cnn::LayerParameter *new_param(const cct_layer_spec &s) {
+    cnn::LayerParameter *lp = new cnn::LayerParameter;
+    lp->blobs_lr_[0] = s.lr_mult[0]; lp->blobs_lr_[1] = s.lr_mult[1];
+    lp->weight_decay_[0] = s.decay_mult[0]; lp->weight_decay_[1] = s.decay_mult[1];
+    return lp;
+  }
+  // part: [B][D/g][R][C] contiguous; whole: [B][D][R][C]; moves channel group gi
+  void slice_copy(CubeT *part, CubeT *whole, size_t gi, bool gather) {
+    const size_t rc = part->R * part->C;
+    int rc_ = cct_hip_copy_depth_slice(part->get_p_data(), whole->get_p_data(), (int)part->B, (int)whole->D,
+                                       (int)(gi * part->D), (int)part->D, rc, gather ? 1 : 0);
+    if (rc_) fail(cct_hip_last_error());
+  }
+};
+
+}  // namespace cct

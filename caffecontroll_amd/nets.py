@@ -1,0 +1,162 @@
+"""Layer chains on the device (``cct_net_*`` of ``include/cct_bridge.h``) and the two networks of
+the benchmark configurations: LeNet and CaffeNet/AlexNet."""
+import ctypes as C
+
+from . import _lib
+from ._lib import check
+from .bridges import SolverParam, solver_param  # noqa: F401
+
+CONV, FC, RELU, MAXPOOL, LRN, DROPOUT, SOFTMAXLOSS = 1, 2, 3, 4, 5, 6, 7
+
+
+class LayerSpec(C.Structure):
+    _fields_ = [("type", C.c_int), ("num_output", C.c_int), ("kernel_size", C.c_int), ("stride", C.c_int),
+                ("pad", C.c_int), ("group", C.c_int), ("bias_term", C.c_int), ("lrn_local_size", C.c_int),
+                ("lrn_alpha", C.c_float), ("lrn_beta", C.c_float), ("dropout_ratio", C.c_float),
+                ("lr_mult", C.c_float * 2), ("decay_mult", C.c_float * 2)]
+
+
+def _spec(t, **kw):
+    s = LayerSpec()
+    s.type, s.stride, s.group, s.bias_term = t, 1, 1, 1
+    s.lr_mult[0], s.lr_mult[1], s.decay_mult[0], s.decay_mult[1] = 1.0, 2.0, 1.0, 0.0
+    for k, v in kw.items():
+        if k in ("lr_mult", "decay_mult"):
+            getattr(s, k)[0], getattr(s, k)[1] = v
+        else:
+            setattr(s, k, v)
+    return s
+
+
+def conv(num_output, kernel_size, stride=1, pad=0, group=1, **kw):
+    return _spec(CONV, num_output=num_output, kernel_size=kernel_size, stride=stride, pad=pad, group=group, **kw)
+
+
+def fc(num_output, **kw):
+    return _spec(FC, num_output=num_output, **kw)
+
+
+def relu():
+    return _spec(RELU)
+
+
+def maxpool(kernel_size, stride):
+    return _spec(MAXPOOL, kernel_size=kernel_size, stride=stride)
+
+
+def lrn(local_size=5, alpha=1e-4, beta=0.75):
+    return _spec(LRN, lrn_local_size=local_size, lrn_alpha=alpha, lrn_beta=beta)
+
+
+def dropout(ratio=0.5):
+    return _spec(DROPOUT, dropout_ratio=ratio)
+
+
+def softmax_loss():
+    return _spec(SOFTMAXLOSS)
+
+
+def lenet_layers():
+    """tests/lenet_train/lenet_train_test.prototxt of the reference: conv(20,5)-pool2-conv(50,5)-pool2-
+    ip500-relu-ip10-softmax loss; lr_mult 1 (weights) / 2 (bias)."""
+    return [conv(20, 5), maxpool(2, 2), conv(50, 5), maxpool(2, 2), fc(500), relu(), fc(10), softmax_loss()]
+
+
+def caffenet_layers(groups=True, num_classes=1000):
+    """tests/imagenet_train/train_val/alexnet_train_val_1GPU.prototxt of the reference (layer order
+    conv-relu-pool-norm).  ``groups=True`` runs conv2/4/5 as two channel groups, as the original
+    network defines them; the reference itself ignores `group` (src/DeepNet.h:1075-1077)."""
+    g = 2 if groups else 1
+    return [conv(96, 11, stride=4), relu(), maxpool(3, 2), lrn(),
+            conv(256, 5, pad=2, group=g), relu(), maxpool(3, 2), lrn(),
+            conv(384, 3, pad=1), relu(),
+            conv(384, 3, pad=1, group=g), relu(),
+            conv(256, 3, pad=1, group=g), relu(), maxpool(3, 2),
+            fc(4096), relu(), dropout(0.5), fc(4096), relu(), dropout(0.5), fc(num_classes), softmax_loss()]
+
+
+_P, _I = C.c_void_p, C.c_int
+NET_PROTOTYPES = {
+    "cct_net_create": ([C.POINTER(_P), _I, _I, _I, C.POINTER(LayerSpec), _I, C.POINTER(SolverParam)], _I),
+    "cct_net_destroy": ([_P], _I),
+    "cct_net_input": ([_P], _P),
+    "cct_net_labels": ([_P], _P),
+    "cct_net_num_layers": ([_P], _I),
+    "cct_net_tensor": ([_P, _I, _I, _I, C.POINTER(C.c_size_t)], _P),
+    "cct_net_set_train": ([_P, _I], _I),
+    "cct_net_freeze_dropout_masks": ([_P, _I], _I),
+    "cct_net_forward": ([_P], _I),
+    "cct_net_backward": ([_P], _I),
+    "cct_net_loss": ([_P, C.POINTER(C.c_float)], _I),
+}
+_bound = False
+
+
+def _bind():
+    global _bound
+    lib = _lib.load()
+    if not _bound:
+        for name, (argtypes, restype) in NET_PROTOTYPES.items():
+            fn = getattr(lib, name)
+            fn.argtypes, fn.restype = argtypes, restype
+        _bound = True
+    return lib
+
+
+MODEL, BIAS, MODEL_GRAD, BIAS_GRAD, OUTPUT, INPUT_GRAD, AUX = range(7)
+
+
+class Net:
+    """A chain of layers resident on the device; one ``forward()`` + ``backward()`` is one training
+    iteration (gradients and SGD update of every layer)."""
+
+    def __init__(self, batch, depth, size, layers, solver=None):
+        self.lib = _bind()
+        self.layers = list(layers)
+        arr = (LayerSpec * len(self.layers))(*self.layers)
+        self._solver = solver or solver_param()
+        h = C.c_void_p()
+        check(self.lib.cct_net_create(C.byref(h), batch, depth, size, arr, len(self.layers),
+                                      C.byref(self._solver)), "net_create")
+        self.h = h
+        self.batch, self.depth, self.size = batch, depth, size
+
+    def input_ptr(self):
+        return self.lib.cct_net_input(self.h)
+
+    def labels_ptr(self):
+        return self.lib.cct_net_labels(self.h)
+
+    def tensor(self, layer, which, group=0):
+        """(device address, element count) or (None, 0)."""
+        n = C.c_size_t()
+        p = self.lib.cct_net_tensor(self.h, layer, group, which, C.byref(n))
+        return p, n.value
+
+    def set_train(self, train):
+        check(self.lib.cct_net_set_train(self.h, int(train)), "net_set_train")
+
+    def freeze_dropout_masks(self, freeze=True):
+        check(self.lib.cct_net_freeze_dropout_masks(self.h, int(freeze)), "net_freeze_dropout_masks")
+
+    def forward(self):
+        check(self.lib.cct_net_forward(self.h), "net_forward")
+
+    def backward(self):
+        check(self.lib.cct_net_backward(self.h), "net_backward")
+
+    def loss(self):
+        v = C.c_float()
+        check(self.lib.cct_net_loss(self.h, C.byref(v)), "net_loss")
+        return v.value
+
+    def close(self):
+        if self.h:
+            self.lib.cct_net_destroy(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -67,6 +67,49 @@ int cct_conv_bridge_forward(cct_conv_bridge *h);
 int cct_conv_bridge_backward(cct_conv_bridge *h, int with_update);
 int cct_conv_bridge_stage_ms(cct_conv_bridge *h, float ms[CCT_CONV_STAGE_COUNT]);
 
+/* ---- a chain of layers (LeNet / CaffeNet style) --------------------------------------------
+ * Stands for DeepNet::construct_network + run_forward_pass / run_backward_pass
+ * (src/DeepNet.h:968-2030, 171-266) for nets that are a plain sequence of layers, with every
+ * layer wrapped in a one-partition ParallelizedBridge on the device. */
+enum cct_layer_type {
+  CCT_LAYER_CONV = 1, CCT_LAYER_FC = 2, CCT_LAYER_RELU = 3, CCT_LAYER_MAXPOOL = 4, CCT_LAYER_LRN = 5,
+  CCT_LAYER_DROPOUT = 6, CCT_LAYER_SOFTMAXLOSS = 7
+};
+
+/* The fields of cnn::LayerParameter this path reads; unused ones are ignored per type. */
+typedef struct cct_layer_spec {
+  int type;                 /* enum cct_layer_type */
+  int num_output;           /* conv, fc */
+  int kernel_size, stride, pad; /* conv, pooling */
+  int group;                /* conv: independent channel groups (<= 1: none) */
+  int bias_term;            /* conv, fc */
+  int lrn_local_size;
+  float lrn_alpha, lrn_beta;
+  float dropout_ratio;
+  float lr_mult[2];         /* weights, bias */
+  float decay_mult[2];
+} cct_layer_spec;
+
+typedef struct cct_net cct_net;
+
+int cct_net_create(cct_net **out, int batch, int depth, int size, const cct_layer_spec *layers, int n_layers,
+                   const cct_solver_param *solver);
+int cct_net_destroy(cct_net *net);
+float *cct_net_input(cct_net *net);   /* device [batch][depth][size][size] */
+float *cct_net_labels(cct_net *net);  /* device, one float per image */
+int cct_net_num_layers(cct_net *net);
+/* Device pointer + element count of a tensor of layer `layer`, channel group `group`:
+ * which = 0 model, 1 bias, 2 model gradient, 3 bias gradient, 4 output data of the layer,
+ * 5 gradient w.r.t. the layer's input, 6 dropout mask (uint32) / max-pool argmax (int32).
+ * Returns NULL (and *n = 0) when the layer has no such tensor. */
+void *cct_net_tensor(cct_net *net, int layer, int group, int which, size_t *n);
+int cct_net_set_train(cct_net *net, int train);
+/* Keep the dropout masks as they are instead of drawing new ones (for parity tests). */
+int cct_net_freeze_dropout_masks(cct_net *net, int freeze);
+int cct_net_forward(cct_net *net);
+int cct_net_backward(cct_net *net);   /* gradients + SGD update of every layer */
+int cct_net_loss(cct_net *net, float *loss_sum); /* batch-summed loss of the last forward (syncs) */
+
 #ifdef __cplusplus
 }
 #endif

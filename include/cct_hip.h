@@ -135,6 +135,13 @@ int cct_hip_inverse_lower_cube_bias_backward(float *dst, const float *src,
  * (j / sB) + (j % sB) * sD of dst.  dst and src must not overlap. */
 int cct_hip_remap(float *dst, const float *src, const cct_pmap_helper *args);
 
+/* Depth-slice copy between a contiguous cube part [B][d_count][rc] and channels
+ * [d_off, d_off + d_count) of whole [B][d_total][rc]; gather != 0: whole -> part, else part -> whole.
+ * Stands for the host loops of the reference's Split / Concat bridges used for grouped layers
+ * (src/DeepNet.h:1700-1757, 1924-2028). */
+int cct_hip_copy_depth_slice(float *part, float *whole, int B, int d_total, int d_off, int d_count,
+                             size_t rc, int gather);
+
 /* ---- BLAS-shaped ----------------------------------------------------------------------- */
 /* DeviceDriver::sgemm (src/sched/DeviceDriver.h:206-208), cblas_sgemm contract. fp32 MFMA. */
 int cct_hip_sgemm(int order, int TA, int TB, int M, int N, int K, float alpha, const float *A,

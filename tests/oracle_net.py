@@ -1,0 +1,142 @@
+"""CPU reference of a layer chain, composed from the oracle's per-layer functions in the order
+DeepNet::run_forward_pass / run_backward_pass visit the bridges (src/DeepNet.h:171-266): ReLU and
+dropout in place, the first weight layer without a data gradient, grouped convolutions as
+independent convolutions on channel slices, one SGD update per weight layer per iteration."""
+import numpy as np
+
+CONV, FC, RELU, MAXPOOL, LRN, DROPOUT, SOFTMAXLOSS = 1, 2, 3, 4, 5, 6, 7
+
+
+class OracleNet:
+    def __init__(self, O, layers, batch, depth, size, solver):
+        """solver: dict(base_lr, momentum, weight_decay); fixed learning-rate policy."""
+        self.O, self.layers, self.solver = O, layers, solver
+        self.params = {}   # (layer, group) -> dict(w, b, hw, hb)
+        self.shapes = []
+        d, n = depth, size
+        first = True
+        self.first_weight = None
+        for i, L in enumerate(layers):
+            if L.type == CONV:
+                g = max(L.group, 1)
+                for gi in range(g):
+                    self.params[(i, gi)] = dict(
+                        w=np.zeros((L.num_output // g, d // g, L.kernel_size, L.kernel_size), np.float32),
+                        b=np.zeros(L.num_output // g, np.float32))
+                n = (n + 2 * L.pad - L.kernel_size) // L.stride + 1
+                d = L.num_output
+                if first:
+                    self.first_weight, first = i, False
+            elif L.type == FC:
+                self.params[(i, 0)] = dict(w=np.zeros((L.num_output, d * n * n), np.float32),
+                                           b=np.zeros(L.num_output, np.float32))
+                d, n = L.num_output, 1
+                if first:
+                    self.first_weight, first = i, False
+            elif L.type == MAXPOOL:
+                n = (n - L.kernel_size) // L.stride + 1
+            self.shapes.append((d, n))
+        for p in self.params.values():
+            p["hw"] = np.zeros(p["w"].size, np.float32)
+            p["hb"] = np.zeros(p["b"].size, np.float32)
+        self.masks = {}
+
+    def forward(self, x, labels):
+        O = self.O
+        self.acts = [x]
+        self.saved = {}
+        cur = x
+        for i, L in enumerate(self.layers):
+            if L.type == CONV:
+                g = max(L.group, 1)
+                dg = cur.shape[1] // g
+                outs = []
+                for gi in range(g):
+                    p = self.params[(i, gi)]
+                    xin = np.ascontiguousarray(cur[:, gi * dg:(gi + 1) * dg])
+                    out, low = O.conv_forward(xin, p["w"], p["b"], L.kernel_size, L.stride, L.pad)
+                    self.saved[(i, gi)] = (xin.shape, low)
+                    outs.append(out)
+                cur = np.concatenate(outs, axis=1) if g > 1 else outs[0]
+            elif L.type == FC:
+                p = self.params[(i, 0)]
+                self.saved[(i, 0)] = cur.reshape(cur.shape[0], -1).copy()
+                cur = O.fc_forward(self.saved[(i, 0)], p["w"], p["b"]).reshape(cur.shape[0], L.num_output, 1, 1)
+            elif L.type == RELU:
+                cur = O.relu_forward(cur)
+                self.acts[-1] = cur  # in place: the layer below now holds the rectified values
+            elif L.type == MAXPOOL:
+                self.saved[i] = cur.shape
+                cur, idx = O.maxpool_forward(cur, L.kernel_size, L.stride)
+                self.saved[(i, "idx")] = idx
+            elif L.type == LRN:
+                self.saved[i] = cur
+                cur, den = O.lrn_forward(cur, L.lrn_local_size, L.lrn_alpha, L.lrn_beta)
+                self.saved[(i, "den")] = den
+            elif L.type == DROPOUT:
+                cur = O.dropout_forward(cur, self.masks[i], L.dropout_ratio, threshold=True)
+                self.acts[-1] = cur
+            elif L.type == SOFTMAXLOSS:
+                cur, self.loss = O.softmax_loss_forward(cur, labels)
+                self.labels = labels
+            if L.type not in (RELU, DROPOUT):
+                self.acts.append(cur)
+        return cur
+
+    def backward(self):
+        O, s = self.O, self.solver
+        grad = None
+        self.grads = {}
+        ai = len(self.acts) - 1  # index of the activation produced by the layer being visited
+        for i in range(len(self.layers) - 1, -1, -1):
+            L = self.layers[i]
+            if L.type == SOFTMAXLOSS:
+                grad = O.softmax_loss_backward(self.acts[ai], self.labels)
+                ai -= 1
+            elif L.type == RELU:
+                grad = O.relu_backward(grad, self.acts[ai])
+            elif L.type == DROPOUT:
+                grad = O.dropout_forward(grad, self.masks[i], L.dropout_ratio, threshold=True)
+            elif L.type == MAXPOOL:
+                shp = self.saved[i]
+                grad = O.maxpool_backward(grad, self.saved[(i, "idx")], shp[2], shp[3])
+                ai -= 1
+            elif L.type == LRN:
+                grad = O.lrn_backward(grad, self.saved[i], self.saved[(i, "den")], L.lrn_local_size,
+                                      L.lrn_alpha, L.lrn_beta)
+                ai -= 1
+            elif L.type == FC:
+                p = self.params[(i, 0)]
+                need = i != self.first_weight
+                xin = self.saved[(i, 0)]
+                dx, dw, db = O.fc_backward(xin, p["w"], grad.reshape(grad.shape[0], -1), need_in_grad=need)
+                self.grads[(i, 0)] = (dw.copy(), db.copy())
+                self._update(p, L, dw, db)
+                grad = dx.reshape(self.acts[ai - 1].shape) if need else None
+                ai -= 1
+            elif L.type == CONV:
+                g = max(L.group, 1)
+                need = i != self.first_weight
+                og_d = grad.shape[1] // g
+                dxs = []
+                for gi in range(g):
+                    p = self.params[(i, gi)]
+                    shp, low = self.saved[(i, gi)]
+                    og = np.ascontiguousarray(grad[:, gi * og_d:(gi + 1) * og_d])
+                    dx, dw, db = O.conv_backward(shp, p["w"], og, low, L.kernel_size, L.stride, L.pad,
+                                                 need_in_grad=need)
+                    self.grads[(i, gi)] = (dw.copy(), db.copy())
+                    self._update(p, L, dw, db)
+                    dxs.append(dx)
+                grad = (np.concatenate(dxs, axis=1) if g > 1 else dxs[0]) if need else None
+                ai -= 1
+        return grad
+
+    def _update(self, p, L, dw, db):
+        s = self.solver
+        w = p["w"].reshape(-1)
+        self.O.sgd_update(w, dw.reshape(-1), p["hw"], s["base_lr"] * L.lr_mult[0], s["momentum"],
+                          s["weight_decay"] * L.decay_mult[0])
+        p["w"] = w.reshape(p["w"].shape)
+        self.O.sgd_update(p["b"], db, p["hb"], s["base_lr"] * L.lr_mult[1], s["momentum"],
+                          s["weight_decay"] * L.decay_mult[1])

@@ -29,6 +29,12 @@ def test_library_exports_every_declared_symbol():
     for n in bnames:
         assert hasattr(lib, n), "missing export: " + n
     assert sorted(bridges.BRIDGE_PROTOTYPES) == bnames
+    from caffecontroll_amd import nets
+    nnames = _declared_symbols("cct_bridge.h", "cct_net_")
+    assert len(nnames) >= 11
+    for n in nnames:
+        assert hasattr(lib, n), "missing export: " + n
+    assert sorted(nets.NET_PROTOTYPES) == nnames
 
 
 def test_struct_layouts_match_reference_headers():
