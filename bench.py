@@ -252,14 +252,19 @@ def main():
             ent["tflops"] = round(gemm_flop / ms / 1e9, 2)
             ent["frac_fp32_mfma_peak"] = round(gemm_flop / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)
         elif name in ("Lower Cube", "Inverse Lwr"):
-            ent["gbs"] = round(lower_bytes / ms / 1e6, 1)
-            ent["frac_hbm_peak"] = round(lower_bytes / ms / 1e6 / PEAK_HBM_GBS, 4)
+            nbytes = lower_bytes
+            if name == "Inverse Lwr" and not args.unfused:
+                # the same launch also reads the output gradient once for the bias gradient
+                nbytes += 4.0 * b * o * m * m
+                ent["includes"] = "bias-gradient reduction in the same launch"
+            ent["gbs"] = round(nbytes / ms / 1e6, 1)
+            ent["frac_hbm_peak"] = round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)
         per_stage[name] = ent
     # dominant kernel = the GEMM instance with the longest average launch
     gemm_names = [g for g in ("GEMM", "GEMM Data", "GEMM Wghts") if g in stages]
     dom = max(gemm_names, key=lambda g: stages[g])
     kernel_of = {"GEMM": "gemm_kernel<256x128x16, A k-contig, B k-contig> (forward, conv epilogue)",
-                 "GEMM Data": "gemm_kernel<256x128x16, A m-contig, B n-contig> (data gradient)",
+                 "GEMM Data": "gemm_kernel<128x256x16, A m-contig, B n-contig> (data gradient)",
                  "GEMM Wghts": "gemm_kernel<256x128x16, A k-contig, B n-contig> split-K (weight gradient)"}
     achieved = gemm_flop / stages[dom] / 1e9
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,

@@ -36,6 +36,7 @@ static int init_locked(int device_id) {
     g_ctx.compute_units = prop.multiProcessorCount;
     g_ctx.workspace = nullptr;
     g_ctx.workspace_bytes = 0;
+    g_ctx.counters = nullptr;
   }
   return 0;
 }
@@ -67,6 +68,17 @@ int get_workspace(size_t bytes, void **out) {
     g_ctx.workspace_bytes = want;
   }
   *out = g_ctx.workspace;
+  return 0;
+}
+
+int get_counters(unsigned int **out) {
+  std::lock_guard<std::mutex> lk(g_mu);
+  if (!g_ctx.counters) {
+    CCT_HIP_CHECK(hipMalloc((void **)&g_ctx.counters, kMaxCounters * sizeof(unsigned int)));
+    CCT_HIP_CHECK(hipMemset(g_ctx.counters, 0, kMaxCounters * sizeof(unsigned int)));
+    CCT_HIP_CHECK(hipDeviceSynchronize());
+  }
+  *out = g_ctx.counters;
   return 0;
 }
 

@@ -18,6 +18,8 @@ struct Context {
   // grow-only device workspace for split-K partial sums
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
+  // zero-initialised arrival counters for reductions finished by the last workgroup (self-resetting)
+  unsigned int *counters = nullptr;
   // dropout generator state: seed and number of rand_uint_initialize calls so far
   uint64_t rng_seed = 0;
   uint64_t rng_calls = 0;
@@ -27,6 +29,8 @@ Context &ctx();
 int ensure_init();
 int set_error(int code, const char *fmt, ...);
 int get_workspace(size_t bytes, void **out);
+constexpr int kMaxCounters = 16384;
+int get_counters(unsigned int **out);
 
 #define CCT_HIP_CHECK(expr)                                                                    \
   do {                                                                                         \

@@ -88,6 +88,17 @@ __global__ __launch_bounds__(TPB) void bias_forward_kernel(float *__restrict__ o
   for (uint32_t i = blockIdx.y * TPB + threadIdx.x; i < fmap; i += gridDim.y * TPB) o[i] += bv;
 }
 
+// small feature maps (FC layers have fmap = 1): one lane per element
+__global__ __launch_bounds__(TPB) void bias_forward_flat_kernel(float *__restrict__ out,
+                                                                const float *__restrict__ bias, uint32_t total,
+                                                                FastDiv div_fmap, FastDiv div_depth) {
+  const uint32_t e = blockIdx.x * TPB + threadIdx.x;
+  if (e >= total) return;
+  const uint32_t sl = fdiv(e, div_fmap);
+  const uint32_t q = fdiv(sl, div_depth);
+  out[e] += bias[sl - q * div_depth.div];
+}
+
 // ---- FC bias gradient: bias[d] = sum_b out[b][d] ------------------------------------------------
 __global__ __launch_bounds__(TPB) void bias_backward_fc_kernel(float *__restrict__ bias,
                                                                const float *__restrict__ og, int D, int B) {
@@ -435,6 +446,13 @@ int cct_hip_forward_bias(const float *bias, float *out, int fmap_size, int depth
   if (batch_size == 0) return 0;
   const size_t slices = (size_t)depth * batch_size;
   CCT_REQUIRE(slices < (1ull << 31), "forward_bias: too many slices");
+  if (fmap_size < 128 && slices * (size_t)fmap_size < (1ull << 31)) {
+    const uint32_t total = (uint32_t)(slices * fmap_size);
+    hipLaunchKernelGGL(bias_forward_flat_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, out, bias,
+                       total, make_fastdiv((uint32_t)fmap_size), make_fastdiv((uint32_t)depth));
+    CCT_LAUNCH_CHECK();
+    return 0;
+  }
   uint32_t gy = (uint32_t)((fmap_size + TPB - 1) / TPB);
   if (gy > 64) gy = 64;
   hipLaunchKernelGGL(bias_forward_kernel, dim3((uint32_t)slices, gy), dim3(TPB), 0, ctx().stream, out, bias,

@@ -29,10 +29,15 @@ struct LiftParams {
                       // serial reductions start at once and overlap the lift blocks
   size_t plane;       // iB*m*m
   FastDiv div_c, div_r, div_d;
-  // bias part
+  // bias part: nbias = depth * bsplit workgroups; workgroup (o, s) reduces images
+  // [s*bchunk, (s+1)*bchunk) of channel o into partial[o*bsplit + s]; the last one to arrive for a
+  // channel adds the partials in ascending s and writes bias_grad[o] (fixed order: deterministic)
   const float *out_grad;
   float *bias_grad;
+  float *partial;
+  unsigned int *counters;
   int fmap, depth, batch;
+  int bsplit, bchunk;
 };
 
 constexpr int LIFT_THREADS = 256;
@@ -43,21 +48,24 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-__device__ void bias_backward_block(const LiftParams &P, int o) {
+__device__ void bias_backward_block(const LiftParams &P, int blk) {
   __shared__ float wave_part[LIFT_THREADS / 64];
+  __shared__ unsigned int arrived;
   const int tid = threadIdx.x;
+  const int o = blk / P.bsplit, sp = blk - o * P.bsplit;
+  const int b0 = sp * P.bchunk, b1 = min(P.batch, b0 + P.bchunk);
   // four images at a time with independent partial sums keeps several loads in flight per lane
   float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f, a3 = 0.0f;
   const size_t img = (size_t)P.depth * P.fmap;
-  int bi = 0;
-  for (; bi + 4 <= P.batch; bi += 4) {
+  int bi = b0;
+  for (; bi + 4 <= b1; bi += 4) {
     const float *g = P.out_grad + ((size_t)bi * P.depth + o) * P.fmap;
     for (int i = tid; i < P.fmap; i += LIFT_THREADS) {
       const float v0 = g[i], v1 = g[img + i], v2 = g[2 * img + i], v3 = g[3 * img + i];
       a0 += v0; a1 += v1; a2 += v2; a3 += v3;
     }
   }
-  for (; bi < P.batch; ++bi) {
+  for (; bi < b1; ++bi) {
     const float *g = P.out_grad + ((size_t)bi * P.depth + o) * P.fmap;
     for (int i = tid; i < P.fmap; i += LIFT_THREADS) a0 += g[i];
   }
@@ -68,8 +76,49 @@ __device__ void bias_backward_block(const LiftParams &P, int o) {
     float t = 0.0f;
 #pragma unroll
     for (int w = 0; w < LIFT_THREADS / 64; ++w) t += wave_part[w];
-    P.bias_grad[o] = t;
+    if (P.bsplit == 1) {
+      P.bias_grad[o] = t;
+    } else {
+      __hip_atomic_store(&P.partial[blk], t, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __threadfence();
+      arrived = atomicAdd(&P.counters[o], 1u);
+      if (arrived == (unsigned int)P.bsplit - 1) {
+        __threadfence();
+        float sum = 0.0f;
+        for (int q = 0; q < P.bsplit; ++q)
+          sum += __hip_atomic_load(&P.partial[o * P.bsplit + q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        P.bias_grad[o] = sum;
+        P.counters[o] = 0;  // ready for the next launch
+      }
+    }
   }
+}
+
+// host side: choose the batch split of the bias reduction and fetch its scratch
+static int setup_bias(LiftParams &P, float *bias_grad, const float *out_grad, int fmap, int depth, int batch,
+                      bool fused_with_lift) {
+  P.out_grad = out_grad; P.bias_grad = bias_grad; P.fmap = fmap; P.depth = depth; P.batch = batch;
+  P.partial = nullptr; P.counters = nullptr; P.bsplit = 1; P.bchunk = batch; P.nbias = 0;
+  if (!bias_grad) return 0;
+  const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
+  // alone: two workgroups per CU; next to the lift blocks: about one per CU, so that the reduction
+  // streams alongside the gather without crowding it out
+  int split = fused_with_lift ? cus / depth : (2 * cus + depth - 1) / depth;
+  if (split > batch / 4) split = batch / 4;
+  if (split < 1 || depth > kMaxCounters) split = 1;
+  const int chunk = (batch + split - 1) / split;
+  split = (batch + chunk - 1) / chunk;
+  P.bsplit = split; P.bchunk = chunk;
+  P.nbias = (uint32_t)depth * split;
+  if (split > 1) {
+    void *ws = nullptr;
+    int rc = get_workspace((size_t)depth * split * sizeof(float), &ws);
+    if (rc) return rc;
+    P.partial = (float *)ws;
+    rc = get_counters(&P.counters);
+    if (rc) return rc;
+  }
+  return 0;
 }
 
 // KT/ST: compile-time kernel size / stride (0 = read from P at run time)
@@ -146,8 +195,8 @@ static int launch_lift(float *dst, const float *src, const cct_inverse_lower_cub
   P.nblocks = (uint32_t)((npix + LIFT_THREADS - 1) / LIFT_THREADS);
   P.plane = a->iB * m * m;
   P.div_c = make_fastdiv(P.iC); P.div_r = make_fastdiv(P.iR); P.div_d = make_fastdiv(P.iD);
-  P.out_grad = out_grad; P.bias_grad = bias_grad; P.fmap = fmap; P.depth = depth; P.batch = batch;
-  P.nbias = bias_grad ? (uint32_t)depth : 0;
+  int rc = setup_bias(P, bias_grad, out_grad, fmap, depth, batch, true);
+  if (rc) return rc;
   const uint32_t grid = P.nblocks + P.nbias;
   if (grid == 0) return 0;
   hipStream_t st = ctx().stream;
@@ -193,10 +242,9 @@ extern "C" int cct_hip_backward_bias(float *bias_grad, const float *out_grad, in
   // the same kernel with zero lift blocks
   LiftParams P = {};
   P.nblocks = 0;
-  P.nbias = (uint32_t)depth;
-  P.out_grad = out_grad; P.bias_grad = bias_grad; P.fmap = fmap_size; P.depth = depth;
-  P.batch = batch_size;
-  hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(depth), dim3(LIFT_THREADS), 0, ctx().stream,
+  int rc = setup_bias(P, bias_grad, out_grad, fmap_size, depth, batch_size, false);
+  if (rc) return rc;
+  hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(P.nbias), dim3(LIFT_THREADS), 0, ctx().stream,
                      (float *)nullptr, (const float *)nullptr, P);
   CCT_LAUNCH_CHECK();
   return 0;
