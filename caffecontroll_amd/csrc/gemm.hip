@@ -276,6 +276,51 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs &g, float *smem, v1
 #undef CCT_FRAGS
 }
 
+// Epilogue of a tile that lies wholly inside C and reads nothing back: per lane one row pointer
+// advancing by a row stride and TN fixed column offsets, no bounds tests.  row0/col0 are the
+// lane's first row and column.
+template <class T, int MODE>
+__device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&acc)[T::TM][T::TN], int row0,
+                                              int col0, uint32_t kslice) {
+  if (MODE == EPI_CONV_FORWARD) {
+    size_t coff[T::TN];
+#pragma unroll
+    for (int b = 0; b < T::TN; ++b) {
+      const uint32_t col = col0 + b * 32;
+      const uint32_t img = fdiv(col, g.div_fmap);
+      coff[b] = (size_t)img * g.M * g.fmap + (col - img * g.fmap);
+    }
+#pragma unroll
+    for (int a = 0; a < T::TM; ++a)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int row = row0 + a * 32 + 8 * j + i;
+          float *c = g.C + (size_t)row * g.fmap;
+          const float add = g.bias ? g.bias[row] : 0.0f;
+#pragma unroll
+          for (int b = 0; b < T::TN; ++b) c[coff[b]] = acc[a][b][4 * j + i] + add;
+        }
+  } else {
+    const size_t rstride = (MODE == EPI_SPLITK_PARTIAL) ? (size_t)g.N : (size_t)g.ldc;
+    float *crow = ((MODE == EPI_SPLITK_PARTIAL) ? g.ws + (size_t)kslice * g.M * g.N : g.C) +
+                  (size_t)row0 * rstride + col0;
+    const float alpha = g.alpha;
+#pragma unroll
+    for (int a = 0; a < T::TM; ++a)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float *c = crow + (size_t)(a * 32 + 8 * j + i) * rstride;
+#pragma unroll
+          for (int b = 0; b < T::TN; ++b)
+            c[b * 32] = (MODE == EPI_SPLITK_PARTIAL) ? acc[a][b][4 * j + i] : alpha * acc[a][b][4 * j + i];
+        }
+  }
+}
+
 template <class T, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
   using LA = OperandLayout<T, A_KC, T::BM>;
@@ -320,6 +365,15 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
 
   // epilogue: accumulator register v of lane (r,h) is C[8*(v/4) + 4*h + v%4][r] of its 32x32 tile
   const int r = lane & 31, h = lane >> 5;
+  if (interior && !(g.epi == EPI_ALPHA_BETA && g.beta != 0.0f)) {
+    if (g.epi == EPI_ALPHA_BETA)
+      fast_epilogue<T, EPI_ALPHA_BETA>(g, acc, m0 + wm0 + 4 * h, n0 + wn0 + r, kslice);
+    else if (g.epi == EPI_SPLITK_PARTIAL)
+      fast_epilogue<T, EPI_SPLITK_PARTIAL>(g, acc, m0 + wm0 + 4 * h, n0 + wn0 + r, kslice);
+    else
+      fast_epilogue<T, EPI_CONV_FORWARD>(g, acc, m0 + wm0 + 4 * h, n0 + wn0 + r, kslice);
+    return;
+  }
 #pragma unroll
   for (int b = 0; b < T::TN; ++b) {
     const int col = n0 + wn0 + b * 32 + r;
