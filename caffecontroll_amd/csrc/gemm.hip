@@ -166,38 +166,58 @@ __device__ __forceinline__ void mfma_group(v16f (&acc)[TM][TN], const f4 (&fa)[T
   mfma_step<3>(acc, fa, fb);
 }
 
-// Unguarded loader state for interior tiles: one 16-byte pointer per f4 a lane fetches,
-// advanced by one K step per tile.
+// Loader for whole K steps: no bounds tests.  Rows (and columns) that fall outside the matrix are
+// clamped to the last valid one -- they only feed accumulators that the epilogue never stores --
+// so every tile, edge tiles included, streams its operands with straight-line loads.  `vec`
+// selects one aligned 16-byte load per f4; otherwise four dword loads (unaligned leading
+// dimension or base, e.g. k*k*d = 363).
 template <class T, bool KC, int ROWS>
 struct FastLoader {
   static constexpr int NV = OperandLayout<T, KC, ROWS>::NV;
-  const f4 *p[NV];
-  size_t step;  // f4 units per K step
-  __device__ __forceinline__ void init(const float *g, int ld, int row0, int k0, int tid) {
+  const float *p[NV];
+  int lim[NV];  // row-contiguous scalar mode: element j of the f4 sits at offset min(j, lim)
+  size_t step;  // floats per K step
+  __device__ __forceinline__ void init(const float *g, int ld, int row0, int k0, int rows_total, int tid) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int f = tid + i * T::THREADS;
       if (KC) {
-        const int row = f / (T::BK / 4), kq = f % (T::BK / 4);
-        p[i] = reinterpret_cast<const f4 *>(g + (size_t)(row0 + row) * ld + k0 + kq * 4);
+        const int row = min(row0 + f / (T::BK / 4), rows_total - 1), kq = f % (T::BK / 4);
+        p[i] = g + (size_t)row * ld + k0 + kq * 4;
+        lim[i] = 3;
       } else {
         const int kk = f / (ROWS / 4), rq = f % (ROWS / 4);
-        p[i] = reinterpret_cast<const f4 *>(g + (size_t)(k0 + kk) * ld + row0 + rq * 4);
+        // an f4 starting past the end moves back to the last one that fits (16-byte mode needs
+        // rows_total % 4 == 0, which the host guarantees before choosing it)
+        int start = row0 + rq * 4;
+        lim[i] = min(3, rows_total - 1 - start);
+        if (lim[i] < 0) {
+          start = max(rows_total - 4, 0);
+          lim[i] = min(3, rows_total - 1 - start);
+        }
+        p[i] = g + (size_t)(k0 + kk) * ld + start;
       }
     }
-    step = KC ? (size_t)(T::BK / 4) : (size_t)T::BK * ld / 4;
+    step = KC ? (size_t)T::BK : (size_t)T::BK * ld;
   }
-  __device__ __forceinline__ void load(f4 *__restrict__ r) {
+  __device__ __forceinline__ void load(f4 *__restrict__ r, int vec) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      r[i] = *p[i];
+      if (vec) {
+        r[i] = *reinterpret_cast<const f4 *>(p[i]);
+      } else if (KC) {
+        r[i] = f4{p[i][0], p[i][1], p[i][2], p[i][3]};
+      } else {
+        const int l = lim[i];
+        r[i] = f4{p[i][0], p[i][min(1, l)], p[i][min(2, l)], p[i][min(3, l)]};
+      }
       p[i] += step;
     }
   }
 };
 
-// Main K loop of one macro tile.  GUARD = false: the tile lies inside the matrices, K steps are
-// whole and both operands allow aligned 16-byte loads, so the loaders carry no bounds tests.
+// Main K loop of one macro tile.  Whole K steps go through FastLoader; only a partial last step
+// (K not a multiple of 16) uses the guarded, zero-filling loader.
 //
 // Software pipeline (BK = 16 = two k-groups of 8, two LDS stages, ONE barrier per K step):
 //   step t, first half : MFMAs of k-group 0 of stage t (fragments fetched during step t-1);
@@ -207,7 +227,7 @@ struct FastLoader {
 //   step t, second half: fragments of k-group 0 of stage t+1 are requested, MFMAs of k-group 1
 //                        of stage t run, then the fragments of k-group 1 of stage t+1 are requested
 // so LDS and HBM latencies are covered by 32 MFMAs (2048 matrix-pipe cycles) each.
-template <class T, bool A_KC, bool B_KC, bool GUARD>
+template <class T, bool A_KC, bool B_KC>
 __device__ __forceinline__ void gemm_mainloop(const GemmArgs &g, float *smem, v16f (&acc)[T::TM][T::TN], int m0,
                                               int n0, int kbeg, int kend, int nk, int tid, int lane, int wm0,
                                               int wn0) {
@@ -218,20 +238,19 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs &g, float *smem, v1
   f4 ra[LA::NV], rb[LB::NV];
   FastLoader<T, A_KC, T::BM> la;
   FastLoader<T, B_KC, T::BN> lb;
-  if (!GUARD) {
-    la.init(g.A, g.lda, m0, kbeg, tid);
-    lb.init(g.B, g.ldb, n0, kbeg, tid);
-  }
+  la.init(g.A, g.lda, m0, kbeg, g.M, tid);
+  lb.init(g.B, g.ldb, n0, kbeg, g.N, tid);
+  const int nk_full = (kend - kbeg) / T::BK;
 // global -> registers for K step t
 #define CCT_FETCH(t)                                                                         \
   do {                                                                                       \
-    if (GUARD) {                                                                             \
+    if ((t) >= nk_full) {                                                                    \
       const int k0_ = kbeg + (t) * T::BK;                                                    \
-      load_tile<T, A_KC, T::BM>(ra, g.A, g.lda, m0, k0_, g.M, kend, g.a_vec, tid);           \
-      load_tile<T, B_KC, T::BN>(rb, g.B, g.ldb, n0, k0_, g.N, kend, g.b_vec, tid);           \
+      load_tile<T, A_KC, T::BM>(ra, g.A, g.lda, m0, k0_, g.M, kend, 0, tid);                 \
+      load_tile<T, B_KC, T::BN>(rb, g.B, g.ldb, n0, k0_, g.N, kend, 0, tid);                 \
     } else {                                                                                 \
-      la.load(ra);                                                                           \
-      lb.load(rb);                                                                           \
+      la.load(ra, g.a_vec);                                                                  \
+      lb.load(rb, g.b_vec);                                                                  \
     }                                                                                        \
   } while (0)
 // registers -> LDS stage
@@ -356,12 +375,8 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  const bool interior = g.a_vec && g.b_vec && (m0 + T::BM <= g.M) && (n0 + T::BN <= g.N) &&
-                        ((kend - kbeg) % T::BK == 0);
-  if (interior)
-    gemm_mainloop<T, A_KC, B_KC, false>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
-  else
-    gemm_mainloop<T, A_KC, B_KC, true>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
+  gemm_mainloop<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
+  const bool interior = (m0 + T::BM <= g.M) && (n0 + T::BN <= g.N);
 
   // epilogue: accumulator register v of lane (r,h) is C[8*(v/4) + 4*h + v%4][r] of its 32x32 tile
   const int r = lane & 31, h = lane >> 5;
@@ -459,8 +474,10 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
   g.alpha = alpha; g.beta = beta; g.epi = epi; g.fmap = fmap > 0 ? fmap : 1;
   g.div_fmap = make_fastdiv((uint32_t)g.fmap); g.bias = bias; g.ws = nullptr;
-  g.a_vec = ((uintptr_t)A % 16 == 0) && (lda % 4 == 0);
-  g.b_vec = ((uintptr_t)B % 16 == 0) && (ldb % 4 == 0);
+  // 16-byte loads need an aligned base and leading dimension; a row-contiguous operand also
+  // needs its row count to be a multiple of 4 so that the clamped last f4 stays aligned
+  g.a_vec = ((uintptr_t)A % 16 == 0) && (lda % 4 == 0) && (a_kc || M % 4 == 0);
+  g.b_vec = ((uintptr_t)B % 16 == 0) && (ldb % 4 == 0) && (b_kc || N % 4 == 0);
   {
     const char *e = getenv("CCT_HIP_GEMM_NT");
     g.nt_store = e ? atoi(e) : 0;
