@@ -261,17 +261,20 @@ def test_conv_forward_backward_vs_oracle(oracle, shape):
     assert rel_err(host(db2), rdb) <= TOL
 
 
-def test_full_size_conv2_against_torch_fp64_sample():
-    """BASELINE config 2 at full size (b=256): forward output and all three gradients agree with
-    float64 torch convolutions on the whole tensor (tolerance 1e-4 of the tensor's max)."""
+@pytest.mark.parametrize("shape", [(256, 96, 27, 5, 1, 2, 256), (256, 3, 227, 11, 4, 0, 96)],
+                         ids=["alexnet_conv2", "alexnet_conv1"])
+def test_full_size_conv_against_torch_fp64(shape):
+    """BASELINE configs 2 and 3 at full size (b=256): forward output and all three gradients agree
+    with float64 torch convolutions on the whole tensor (tolerance 1e-4 of the tensor's max)."""
     import torch
     import torch.nn.functional as F
-    b, d, n, k, s, p, o = 256, 96, 27, 5, 1, 2, 256
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
     g = torch.Generator(device="cuda").manual_seed(1236)
     x = torch.randn((b, d, n, n), device="cuda", generator=g)
     w = torch.randn((o, d, k, k), device="cuda", generator=g) * 0.01
     bias = torch.full((o,), 0.1, device="cuda")
-    og = torch.randn((b, o, n, n), device="cuda", generator=g)
+    og = torch.randn((b, o, m, m), device="cuda", generator=g)
     out, lowered = conv_forward_gpu(host(x), host(w), host(bias), k, s, p, fused=True)
     dx, dw, db = conv_backward_gpu(tuple(x.shape), host(w), host(og), lowered, k, s, p)
     torch.cuda.synchronize()
