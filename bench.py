@@ -27,6 +27,15 @@ CONFIGS = {
 }
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the three GEMM instances at the alexnet_conv2 shape, from rocprofv3 --pmc
+# FETCH_SIZE and WRITE_SIZE runs of this file (one counter per run), each scaled by what the same
+# counter reads for a 1 GiB device copy (factors 2.000 and 1.000); the counter summary is kept
+# under profiles/.  fetched + written, in bytes.
+GEMM_TRAFFIC_BYTES = {
+    "GEMM": (1868.7 + 192.4) * 1e6,
+    "GEMM Data": (1450.5 + 1990.2) * 1e6,
+    "GEMM Wghts": (2143.1 + 63.9) * 1e6,
+}
 
 
 def synth(cfg, seed, torch):
@@ -268,7 +277,8 @@ def main():
                  "GEMM Wghts": "gemm_kernel<256x128x16, A k-contig, B n-contig> split-K (weight gradient)"}
     achieved = gemm_flop / stages[dom] / 1e9
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                "traffic": GEMM_TRAFFIC_BYTES[dom] if (cfg == "alexnet_conv2" and not args.unfused) else None,
                 "kernel": kernel_of[dom], "stage": dom, "flop_per_launch": gemm_flop,
                 "avg_launch_ms": round(stages[dom], 4)}
 
