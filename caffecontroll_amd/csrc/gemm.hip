@@ -484,36 +484,48 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   }
   if (K <= 0) g.K = 0;  // degenerate: C = beta*C through the normal epilogue with zero accumulators
 
-  // tile choice: the big tiles (256x128 or 128x256, whichever pads M x N less) when the problem is
-  // large enough to fill the device with them, else 128x128, else 64x64
+  // Tile shape and split-K factor come from a small occupancy model.  A compute unit holds `occ`
+  // workgroups of a shape; the busiest unit gets n = ceil(blocks / units) of them and works them off
+  // in groups of occ.  A group of j co-resident workgroups runs at min(j * 0.55, 1) of the unit's
+  // MFMA rate (one workgroup alone cannot hide its own barriers), every workgroup pays a fixed
+  // prologue/epilogue worth `k0` K-steps, and the smaller shapes lose a little to their lower
+  // flop-per-LDS-byte ratio (`eff`).  The constants are fitted to measured times of the
+  // AlexNet/CaffeNet convolution and inner-product shapes.
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
-  auto ntiles = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-  auto padded = [&](int bm, int bn) { return (double)ntiles(bm, bn) * bm * bn; };
-  int cfg;  // 0 = L (256x128), 1 = M (128x128), 2 = S (64x64), 3 = LT (128x256)
-  if (M > 128 && N > 128 && padded(256, 128) <= 1.15 * padded(128, 128) && padded(256, 128) <= padded(128, 256))
-    cfg = 0;
-  else if (M > 64 && N > 128 && padded(128, 256) <= 1.15 * padded(128, 128))
-    cfg = 3;
-  else if (M > 64 && N > 64)
-    cfg = 1;
-  else
-    cfg = 2;
-  const int bm = cfg == 0 ? 256 : cfg == 2 ? 64 : 128, bn = cfg == 3 ? 256 : cfg == 2 ? 64 : 128, bk = 16;
-  const long tiles = ntiles(bm, bn);
-
-  // split-K only for the plain epilogue when the tile grid cannot fill the device
-  int splits = 1;
-  const long slots = 2L * cus;
-  if (epi == EPI_ALPHA_BETA && tiles < cus && K >= 1024) {
-    splits = (int)(slots / tiles);
-    const int max_splits = K / 256;
-    if (splits > max_splits) splits = max_splits;
-    if (splits < 1) splits = 1;
-  }
-  int kchunk = g.K > 0 ? g.K : bk;
-  if (splits > 1) {
-    kchunk = (((K + splits - 1) / splits) + bk - 1) / bk * bk;
-    splits = (K + kchunk - 1) / kchunk;
+  const int bk = 16;
+  struct Shape { int bm, bn, occ, k0; double eff; };
+  static const Shape shapes[4] = {{256, 128, 2, 32, 1.0}, {128, 128, 3, 8, 0.96}, {64, 64, 6, 8, 0.80},
+                                  {128, 256, 2, 32, 1.0}};  // L, M, S, LT
+  const double cu_rate = 0.8 * 157.3e12 / 256.0, hbm_rate = 4.0e12;
+  int cfg = 1, splits = 1, kchunk = g.K > 0 ? g.K : bk;
+  double best = 1e30;
+  static const int forced = [] { const char *e = getenv("CCT_HIP_GEMM_TILE"); return e ? atoi(e) : -1; }();
+  for (int c = 0; c < 4; ++c) {
+    if (forced >= 0 && forced <= 3 && c != forced) continue;  // tuning override, read once
+    const Shape &sh = shapes[c];
+    const long tiles = (long)((M + sh.bm - 1) / sh.bm) * ((N + sh.bn - 1) / sh.bn);
+    const long slots = (long)sh.occ * cus;
+    for (int pass = 0; pass < 2; ++pass) {
+      int sp = 1, kc = g.K > 0 ? g.K : bk;
+      if (pass == 1) {
+        // split-K: plain epilogue only, when the tile grid alone cannot fill the device
+        if (epi != EPI_ALPHA_BETA || tiles >= slots || K < 512) break;
+        sp = (int)(slots / tiles);
+        if (sp > K / 256) sp = K / 256;
+        if (sp < 2) break;
+        kc = (((K + sp - 1) / sp) + bk - 1) / bk * bk;
+        sp = (K + kc - 1) / kc;
+        if (sp < 2) break;
+      }
+      const long blocks = tiles * sp;
+      const long n = (blocks + cus - 1) / cus;
+      const double w = 2.0 * sh.bm * sh.bn * (double)(kc + sh.k0) / (cu_rate * sh.eff);
+      const long rem = n % sh.occ;
+      double t = (double)(n / sh.occ) * sh.occ * w;
+      if (rem) t += rem * w / (rem * 0.55 < 1.0 ? rem * 0.55 : 1.0);
+      if (sp > 1) t += 3e-6 + 8.0 * sp * (double)M * N / hbm_rate;  // partial sums out and back in
+      if (t < best) { best = t; cfg = c; splits = sp; kchunk = kc; }
+    }
   }
   g.kchunk = kchunk;
   if (splits > 1) {
@@ -524,9 +536,9 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
     g.epi = EPI_SPLITK_PARTIAL;
   }
   int rc = cfg == 0   ? launch_cfg<TileL>(g, a_kc, b_kc, splits, st)
-           : cfg == 3 ? launch_cfg<TileLT>(g, a_kc, b_kc, splits, st)
            : cfg == 1 ? launch_cfg<TileM>(g, a_kc, b_kc, splits, st)
-                      : launch_cfg<TileS>(g, a_kc, b_kc, splits, st);
+           : cfg == 2 ? launch_cfg<TileS>(g, a_kc, b_kc, splits, st)
+                      : launch_cfg<TileLT>(g, a_kc, b_kc, splits, st);
   if (rc) return rc;
   if (splits > 1) {
     CCT_REQUIRE((size_t)M * N < (1ull << 31), "sgemm: split-K result too large");
