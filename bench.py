@@ -31,10 +31,13 @@ PEAK_HBM_GBS = 8000.0
 # FETCH_SIZE and WRITE_SIZE runs of this file (one counter per run), each scaled by what the same
 # counter reads for a 1 GiB device copy (factors 2.000 and 1.000); the counter summary is kept
 # under profiles/.  fetched + written, in bytes.
+# Keyed by (path level, stage).
 GEMM_TRAFFIC_BYTES = {
-    "GEMM": (1868.7 + 192.4) * 1e6,
-    "GEMM Data": (1450.5 + 1990.2) * 1e6,
-    "GEMM Wghts": (2143.1 + 63.9) * 1e6,
+    (1, "GEMM"): (1868.7 + 192.4) * 1e6,
+    (1, "GEMM Data"): (1450.5 + 1990.2) * 1e6,
+    (1, "GEMM Wghts"): (2143.1 + 63.9) * 1e6,
+    (2, "GEMM"): (1868.7 + 192.4) * 1e6,
+    (2, "GEMM Wghts"): (2143.1 + 63.9) * 1e6,
 }
 
 
@@ -180,6 +183,9 @@ def main():
                          "iteration of LeNet (b=64) / CaffeNet (b=256, grouped conv2/4/5)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--unfused", action="store_true", help="staged forward (GEMM, remap, bias) and separate bias gradient")
+    ap.add_argument("--path", type=int, default=-1, choices=[-1, 0, 1, 2, 3],
+                    help="conv path level: 0 separate passes, 1 fused epilogues, 2 direct data gradient, 3 all "
+                         "direct kernels (no lowered matrix); -1 = the bridge's default")
     ap.add_argument("--no-data-grad", action="store_true", help="first-layer mode: skip data-gradient GEMM and lift")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 5 device-to-device copies of 1 GiB (a plain copy kernel of known size, used "
@@ -229,7 +235,9 @@ def main():
     drv.memcpy(layer.model_ptr(), w.ctypes.data, w.nbytes, 0)
     drv.memcpy(layer.bias_ptr(), bias.ctypes.data, bias.nbytes, 0)
     need_dgrad = not args.no_data_grad
-    layer.set_options(fused=not args.unfused, profile=True, needs_backward_grad=need_dgrad)
+    layer.set_options(fused=0 if args.unfused else (None if args.path < 0 else args.path), profile=True,
+                      needs_backward_grad=need_dgrad)
+    path = layer.path()
 
     def step():
         layer.forward()
@@ -262,7 +270,7 @@ def main():
             ent["frac_fp32_mfma_peak"] = round(gemm_flop / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)
         elif name in ("Lower Cube", "Inverse Lwr"):
             nbytes = lower_bytes
-            if name == "Inverse Lwr" and not args.unfused:
+            if name == "Inverse Lwr" and path == 1:
                 # the same launch also reads the output gradient once for the bias gradient
                 nbytes += 4.0 * b * o * m * m
                 ent["includes"] = "bias-gradient reduction in the same launch"
@@ -275,10 +283,15 @@ def main():
     kernel_of = {"GEMM": "gemm_kernel<256x128x16, A k-contig, B k-contig> (forward, conv epilogue)",
                  "GEMM Data": "gemm_kernel<128x256x16, A m-contig, B n-contig> (data gradient)",
                  "GEMM Wghts": "gemm_kernel<256x128x16, A k-contig, B n-contig> split-K (weight gradient)"}
+    if path >= 2 and need_dgrad:
+        kernel_of["GEMM Data"] = "conv_direct_kernel (data gradient: remap + GEMM + lifting in one launch)"
+    if path == 3:
+        kernel_of["GEMM"] = "conv_direct_kernel (forward: lowering + GEMM + remap + bias in one launch)"
+        kernel_of["GEMM Wghts"] = "conv_direct_wgrad_kernel (weight gradient from input and output gradient)"
     achieved = gemm_flop / stages[dom] / 1e9
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
                 "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                "traffic": GEMM_TRAFFIC_BYTES[dom] if (cfg == "alexnet_conv2" and not args.unfused) else None,
+                "traffic": GEMM_TRAFFIC_BYTES.get((path, dom)) if cfg == "alexnet_conv2" else None,
                 "kernel": kernel_of[dom], "stage": dom, "flop_per_launch": gemm_flop,
                 "avg_launch_ms": round(stages[dom], 4)}
 
@@ -289,7 +302,7 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: conv fwd+bwd b=%d d=%d n=%d k=%d s=%d p=%d o=%d%s%s" % (
             cfg, b, d, n, k, s, p, o, "" if need_dgrad else " (no data gradient)",
-            " (staged forward)" if args.unfused else "")},
+            " (path level %d)" % path)},
         "roofline": roofline, "stages": per_stage,
     }
     if not args.no_cpu_baseline:

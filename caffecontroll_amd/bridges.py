@@ -28,6 +28,7 @@ BRIDGE_PROTOTYPES = {
                                 _P, _P, _P, _P], _I),
     "cct_conv_bridge_destroy": ([_P], _I),
     "cct_conv_bridge_set_options": ([_P, _I, _I, _I], _I),
+    "cct_conv_bridge_path": ([_P], _I),
     "cct_conv_bridge_model": ([_P], _P),
     "cct_conv_bridge_bias": ([_P], _P),
     "cct_conv_bridge_model_grad": ([_P], _P),
@@ -82,9 +83,22 @@ class ConvolutionLayer:
               "conv_bridge_create")
         self.h = h
 
-    def set_options(self, fused=True, profile=False, needs_backward_grad=True):
-        check(self.lib.cct_conv_bridge_set_options(self.h, int(fused), int(profile), int(needs_backward_grad)),
+    def set_options(self, fused=None, profile=False, needs_backward_grad=True):
+        """fused: path level 0..3 (0 separate passes, 1 fused epilogues, 2 direct data gradient,
+        3 all-direct, no lowered matrix); None keeps the bridge's default (2 where the geometry is
+        covered by the direct kernels, else 1).  True/False mean "default" / 0."""
+        if fused is None or fused is True:
+            level = -1
+        elif fused is False:
+            level = 0
+        else:
+            level = int(fused)
+        check(self.lib.cct_conv_bridge_set_options(self.h, level, int(profile), int(needs_backward_grad)),
               "conv_bridge_set_options")
+
+    def path(self):
+        """Path level in effect (0..3)."""
+        return self.lib.cct_conv_bridge_path(self.h)
 
     # device addresses of the cubes the reference exposes on the bridge
     def model_ptr(self):

@@ -66,12 +66,14 @@ int cct_conv_bridge_destroy(cct_conv_bridge *h) {
 
 int cct_conv_bridge_set_options(cct_conv_bridge *h, int fused, int profile, int needs_backward_grad) {
   if (!h) return CCT_HIP_EINVAL;
-  h->pbridge->sub_bridge()->set_fused(fused != 0);
+  if (fused >= 0) h->pbridge->sub_bridge()->set_path(fused);
   h->pbridge->sub_bridge()->set_stage_profiling(profile != 0);
   h->pbridge->needs_to_calc_backward_grad = needs_backward_grad != 0;
   h->pbridge->sub_bridge()->needs_to_calc_backward_grad = needs_backward_grad != 0;
   return 0;
 }
+
+int cct_conv_bridge_path(cct_conv_bridge *h) { return h ? h->pbridge->sub_bridge()->path() : -1; }
 
 float *cct_conv_bridge_model(cct_conv_bridge *h) { return h->pbridge->p_model_cube->get_p_data(); }
 float *cct_conv_bridge_bias(cct_conv_bridge *h) {

@@ -11,7 +11,12 @@
 //   * by default the forward GEMM writes [b][o][m*m] and adds the bias in its epilogue instead
 //     of running remap_output and the bias map as separate passes (set_fused(false) restores
 //     the staged sequence);
-//   * the bias gradient is reduced in the same launch as the lifting kernel.
+//   * the bias gradient is reduced in the same launch as the lifting kernel;
+//   * for stride-1 layers with k = 3 or 5 the data gradient (path level 2, the default where the
+//     geometry allows it) or all three products (level 3) come from direct-convolution kernels
+//     that never materialise the lowered matrices; results then agree with the lowering path to
+//     fp32 rounding instead of bit for bit.  The lowered buffers are allocated on first use, so
+//     level 3 runs without them.
 #pragma once
 #include <cstdio>
 #include <cstdlib>
@@ -22,6 +27,14 @@
 #include "Kernel.h"
 
 namespace cct {
+
+// How much of the lowering pipeline is replaced (set_path).
+enum ConvPath {
+  PATH_STAGED = 0,       // the reference's sequence of separate passes
+  PATH_FUSED = 1,        // GEMM epilogue does remap + bias; bias gradient rides with the lifting
+  PATH_DIRECT_DATA = 2,  // as 1, data gradient by the direct kernel (no data-gradient GEMM, no lifting)
+  PATH_DIRECT_ALL = 3    // forward, weight gradient and data gradient by direct kernels, no lowering
+};
 
 // Stage labels of the reference's detailed profiling output (_impl.hxx:325-366, 601-623).
 enum ConvStage {
@@ -84,22 +97,28 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       DeviceMemoryPointer bg = p_bias_gradient_cube->get_device_pointer(p_driver);
       p_driver->sconstant_initialize(&bg, DataType(0.));
     }
-    // cubes used inside the bridge only; sized for the whole batch
-    p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
-    p_backward_inputgrad = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
-    p_staging_cube = new LogicalCubeType(oR, oC, oD, oB, p_driver);  // [o][b][m*m] view of output / out-grad
+    // cubes used inside the bridge only, sized for the whole batch, allocated on first use
+    p_forward_lowered_data = nullptr;
+    p_backward_inputgrad = nullptr;
+    p_staging_cube = nullptr;
+    p_forward_slabs = nullptr;
+    p_backward_slabs = nullptr;
 
-    LogicalCubeType lowered_forward_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
-    LogicalCubeType lowered_forward_output(p_staging_cube->get_p_data(), num_output_features, oR * oC * iB, 1, 1);
+    LogicalCubeType lowered_forward_model(nullptr, num_output_features, K * K * iD, 1, 1);
+    LogicalCubeType lowered_forward_output(nullptr, num_output_features, oR * oC * iB, 1, 1);
+    LogicalCubeType lowered_data(nullptr, K * K * iD, oR * oC * iB, 1, 1);
     LogicalCubeType dummy_data_cube(nullptr, iR, iC, iD, iB);
     p_forward_lower_connector =
-        new Connector<DataType, DriverClass>(&dummy_data_cube, p_forward_lowered_data, K, padding, stride, p_driver);
+        new Connector<DataType, DriverClass>(&dummy_data_cube, &lowered_data, K, padding, stride, p_driver);
     p_forward_gemm_kernel = new Kernel<DataType, KernelConfig_GEMM_NOTRANS_TRANS_NO_DIM_FLIP, DriverClass>(
-        &lowered_forward_model, p_forward_lowered_data, &lowered_forward_output, p_driver);
+        &lowered_forward_model, &lowered_data, &lowered_forward_output, p_driver);
     p_backward_gemm_updateweight_kernel = new Kernel<DataType, KernelConfig_GEMM_NOTRANS_NOTRANS_DIM_FLIP, DriverClass>(
-        &lowered_forward_output, p_forward_lowered_data, &lowered_forward_model, p_driver);
+        &lowered_forward_output, &lowered_data, &lowered_forward_model, p_driver);
     p_backward_gemm_updategrad_kernel = new Kernel<DataType, KernelConfig_GEMM_TRANS_NOTRANS, DriverClass>(
-        &lowered_forward_model, &lowered_forward_output, p_backward_inputgrad, p_driver);
+        &lowered_forward_model, &lowered_forward_output, &lowered_data, p_driver);
+    direct_ok_ = p_driver->conv_direct_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
+                                                 (int)num_output_features);
+    path_ = direct_ok_ ? PATH_DIRECT_DATA : PATH_FUSED;
     for (int i = 0; i < STAGE_COUNT; ++i) { timers_[i] = nullptr; stage_ms_[i] = 0.f; }
   }
 
@@ -113,6 +132,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     delete p_forward_lowered_data;
     delete p_backward_inputgrad;
     delete p_staging_cube;
+    delete p_forward_slabs;
+    delete p_backward_slabs;
     delete p_forward_lower_connector;
     delete p_forward_gemm_kernel;
     delete p_backward_gemm_updateweight_kernel;
@@ -123,9 +144,18 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   LogicalCubeType *get_bias_cube() override { return p_bias_cube; }
   LogicalCubeType *get_model_grad_cube() override { return p_model_gradient_cube; }
   LogicalCubeType *get_bias_grad_cube() override { return p_bias_gradient_cube; }
-  LogicalCubeType *get_lowered_cube() { return p_forward_lowered_data; }
+  LogicalCubeType *get_lowered_cube() { return lowered(); }
 
-  void set_fused(bool on) { fused_ = on; }
+  // Path level (ConvPath); levels 2 and 3 fall back to 1 where the direct kernels do not cover
+  // the layer's geometry.
+  void set_path(int level) {
+    if (level < PATH_STAGED) level = PATH_STAGED;
+    if (level > PATH_DIRECT_ALL) level = PATH_DIRECT_ALL;
+    if (level >= PATH_DIRECT_DATA && !direct_ok_) level = PATH_FUSED;
+    path_ = level;
+  }
+  int path() const { return path_; }
+  void set_fused(bool on) { set_path(on ? (direct_ok_ ? PATH_DIRECT_DATA : PATH_FUSED) : PATH_STAGED); }
   // per-stage hipEvent timing (the reference's -D_DETAILED_PROFILING stage prints)
   void set_stage_profiling(bool on) { profile_ = on; }
   float stage_ms(int stage) {
@@ -142,22 +172,34 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     LogicalCubeType *output_d_cube = p_output_layer->p_data_cube;
     LogicalCubeType lowered_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
 
+    if (path_ == PATH_DIRECT_ALL) {
+      // slabs are rebuilt every pass: the model changes between iterations
+      begin(STAGE_GEMM);
+      p_driver->conv_direct_slabs(forward_slabs()->get_p_data(), p_model_cube->get_p_data(),
+                                  (int)num_output_features, (int)iD, (int)K, 0);
+      p_driver->conv_direct_forward(output_d_cube->get_p_data(), input_d_cube->get_p_data(),
+                                    forward_slabs()->get_p_data(), bias_term ? p_bias_cube->get_p_data() : nullptr,
+                                    (int)iB, (int)iD, (int)iR, (int)K, (int)padding, (int)num_output_features);
+      end(STAGE_GEMM);
+      report_forward_history.end();
+      return;
+    }
     begin(STAGE_LOWER);
-    p_forward_lower_connector->lower_cube(input_d_cube, p_forward_lowered_data);
+    p_forward_lower_connector->lower_cube(input_d_cube, lowered());
     end(STAGE_LOWER);
-    if (fused_) {
+    if (path_ >= PATH_FUSED) {
       begin(STAGE_GEMM);
       p_driver->sgemm_conv_forward((int)num_output_features, (int)iB, (int)(oR * oC), (int)(K * K * iD),
-                                   p_model_cube->get_p_data(), p_forward_lowered_data->get_p_data(),
+                                   p_model_cube->get_p_data(), lowered()->get_p_data(),
                                    bias_term ? p_bias_cube->get_p_data() : nullptr, output_d_cube->get_p_data());
       end(STAGE_GEMM);
     } else {
-      LogicalCubeType lowered_output(p_staging_cube->get_p_data(), num_output_features, oR * oC * iB, 1, 1);
+      LogicalCubeType lowered_output(staging()->get_p_data(), num_output_features, oR * oC * iB, 1, 1);
       begin(STAGE_GEMM);
-      p_forward_gemm_kernel->compute(&lowered_model, p_forward_lowered_data, &lowered_output);
+      p_forward_gemm_kernel->compute(&lowered_model, lowered(), &lowered_output);
       end(STAGE_GEMM);
       begin(STAGE_REMAP);
-      p_forward_lower_connector->remap_output(*output_d_cube, *p_staging_cube, num_output_features, iB);
+      p_forward_lower_connector->remap_output(*output_d_cube, *staging(), num_output_features, iB);
       end(STAGE_REMAP);
       if (bias_term) {
         begin(STAGE_BIAS);
@@ -179,22 +221,27 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     LogicalCubeType *input_g_cube = p_input_layer->p_gradient_cube;
     LogicalCubeType lowered_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
     LogicalCubeType lowered_model_grad(p_model_gradient_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
-    LogicalCubeType lowered_outputgrad(p_staging_cube->get_p_data(), num_output_features, oR * oC * iB, 1, 1);
     DeviceMemoryPointer og = output_g_cube->get_device_pointer(p_driver);
+    const bool direct_data = path_ >= PATH_DIRECT_DATA && needs_to_calc_backward_grad;
+    const bool direct_weights = path_ == PATH_DIRECT_ALL;
 
-    const bool fuse_bias_into_lift = bias_term && needs_to_calc_backward_grad && fused_;
+    const bool fuse_bias_into_lift = bias_term && needs_to_calc_backward_grad && path_ == PATH_FUSED;
     if (bias_term && !fuse_bias_into_lift) {
       begin(STAGE_BW_BIAS);
       DeviceMemoryPointer bias = p_bias_gradient_cube->get_device_pointer(p_driver);
       p_driver->backward_bias(&bias, &og, (int)(oR * oC), (int)oD, (int)iB);
       end(STAGE_BW_BIAS);
     }
-    begin(STAGE_BW_REMAP);
-    p_forward_lower_connector->remap_output(*p_staging_cube, *output_g_cube, oB, num_output_features);
-    end(STAGE_BW_REMAP);
-    if (needs_to_calc_backward_grad) {
+    if (!direct_weights) {
+      begin(STAGE_BW_REMAP);
+      p_forward_lower_connector->remap_output(*staging(), *output_g_cube, oB, num_output_features);
+      end(STAGE_BW_REMAP);
+    }
+    LogicalCubeType lowered_outputgrad(direct_weights ? nullptr : staging()->get_p_data(), num_output_features,
+                                       oR * oC * iB, 1, 1);
+    if (needs_to_calc_backward_grad && !direct_data) {
       begin(STAGE_GEMM_DATA);
-      p_backward_gemm_updategrad_kernel->compute(&lowered_model, &lowered_outputgrad, p_backward_inputgrad);
+      p_backward_gemm_updategrad_kernel->compute(&lowered_model, &lowered_outputgrad, backward_inputgrad());
       end(STAGE_GEMM_DATA);
     }
     // The weight-gradient GEMM is issued between the data-gradient GEMM and the lifting (the
@@ -202,20 +249,35 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     // lifting kernel is HBM-bound and runs faster once the 1.8 GB written by the data-gradient
     // GEMM has drained from the caches.
     begin(STAGE_GEMM_WEIGHTS);
-    p_backward_gemm_updateweight_kernel->alpha = 1.0;
-    p_backward_gemm_updateweight_kernel->beta = 0.0;
-    p_backward_gemm_updateweight_kernel->compute(&lowered_outputgrad, p_forward_lowered_data, &lowered_model_grad);
+    if (direct_weights) {
+      p_driver->conv_direct_backward_weights(p_model_gradient_cube->get_p_data(), output_g_cube->get_p_data(),
+                                             p_input_layer->p_data_cube->get_p_data(), (int)iB, (int)iD, (int)iR,
+                                             (int)K, (int)padding, (int)num_output_features);
+    } else {
+      p_backward_gemm_updateweight_kernel->alpha = 1.0;
+      p_backward_gemm_updateweight_kernel->beta = 0.0;
+      p_backward_gemm_updateweight_kernel->compute(&lowered_outputgrad, lowered(), &lowered_model_grad);
+    }
     end(STAGE_GEMM_WEIGHTS);
-    if (needs_to_calc_backward_grad) {
+    if (direct_data) {
+      // remap + data-gradient GEMM + lifting in one kernel, reading the output gradient in place
+      begin(STAGE_GEMM_DATA);
+      p_driver->conv_direct_slabs(backward_slabs()->get_p_data(), p_model_cube->get_p_data(),
+                                  (int)num_output_features, (int)iD, (int)K, 1);
+      p_driver->conv_direct_backward_data(input_g_cube->get_p_data(), output_g_cube->get_p_data(),
+                                          backward_slabs()->get_p_data(), (int)iB, (int)iD, (int)iR, (int)K,
+                                          (int)padding, (int)num_output_features);
+      end(STAGE_GEMM_DATA);
+    } else if (needs_to_calc_backward_grad) {
       begin(STAGE_INVERSE_LOWER);
       if (fuse_bias_into_lift) {
         DeviceMemoryPointer input = input_g_cube->get_device_pointer(p_driver);
-        DeviceMemoryPointer lowered_grad = p_backward_inputgrad->get_device_pointer(p_driver);
+        DeviceMemoryPointer lowered_grad = backward_inputgrad()->get_device_pointer(p_driver);
         DeviceMemoryPointer bias = p_bias_gradient_cube->get_device_pointer(p_driver);
         p_driver->inverse_lower_cube_bias_backward(&input, &lowered_grad, p_forward_lower_connector->inverse_args(),
                                                    &bias, &og, (int)(oR * oC), (int)oD, (int)iB);
       } else {
-        p_forward_lower_connector->inverse_lower_cube(p_backward_inputgrad, input_g_cube);
+        p_forward_lower_connector->inverse_lower_cube(backward_inputgrad(), input_g_cube);
       }
       end(STAGE_INVERSE_LOWER);
     }
@@ -228,6 +290,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   LogicalCubeType *p_forward_lowered_data;
   LogicalCubeType *p_backward_inputgrad;
   LogicalCubeType *p_staging_cube;
+  LogicalCubeType *p_forward_slabs;   // model as [d][o][k*k] for the direct forward kernel
+  LogicalCubeType *p_backward_slabs;  // model as [o][d][k*k], filters reversed, for the direct data gradient
   Connector<DataType, DriverClass> *p_forward_lower_connector;
   Kernel<DataType, KernelConfig_GEMM_NOTRANS_TRANS_NO_DIM_FLIP, DriverClass> *p_forward_gemm_kernel;
   Kernel<DataType, KernelConfig_GEMM_NOTRANS_NOTRANS_DIM_FLIP, DriverClass> *p_backward_gemm_updateweight_kernel;
@@ -253,7 +317,28 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   }
 
  private:
-  bool fused_ = true, profile_ = false;
+  int path_ = PATH_FUSED;
+  bool direct_ok_ = false, profile_ = false;
+  LogicalCubeType *lowered() {
+    if (!p_forward_lowered_data) p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
+    return p_forward_lowered_data;
+  }
+  LogicalCubeType *backward_inputgrad() {
+    if (!p_backward_inputgrad) p_backward_inputgrad = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
+    return p_backward_inputgrad;
+  }
+  LogicalCubeType *staging() {  // [o][b][m*m] view of output / output gradient
+    if (!p_staging_cube) p_staging_cube = new LogicalCubeType(oR, oC, oD, oB, p_driver);
+    return p_staging_cube;
+  }
+  LogicalCubeType *forward_slabs() {
+    if (!p_forward_slabs) p_forward_slabs = new LogicalCubeType(K, K, iD, num_output_features, p_driver);
+    return p_forward_slabs;
+  }
+  LogicalCubeType *backward_slabs() {
+    if (!p_backward_slabs) p_backward_slabs = new LogicalCubeType(K, K, iD, num_output_features, p_driver);
+    return p_backward_slabs;
+  }
   void *timers_[STAGE_COUNT];
   bool stage_ran_[STAGE_COUNT] = {};
   float stage_ms_[STAGE_COUNT];

@@ -172,6 +172,31 @@ class HIPDriver {
                           const float *bias, float *out) {
     ok(cct_hip_sgemm_conv_forward(o, batch, fmap, K, model, lowered, bias, out), "sgemm_conv_forward");
   }
+  // ---- stride-1 convolution without the lowered matrix (no counterpart in DeviceDriver.h) ----
+  bool conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs) {
+    return cct_hip_conv_direct_supported(batch, depth, n, k, stride, padding, num_outputs) != 0;
+  }
+  void conv_direct_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
+                         int for_data_gradient) {
+    ok(cct_hip_conv_direct_slabs(slabs, model, num_outputs, depth, k, for_data_gradient), "conv_direct_slabs");
+  }
+  void conv_direct_forward(float *output, const float *input, const float *slabs, const float *bias, int batch,
+                           int depth, int n, int k, int padding, int num_outputs) {
+    ok(cct_hip_conv_direct_forward(output, input, slabs, bias, batch, depth, n, k, padding, num_outputs),
+       "conv_direct_forward");
+  }
+  void conv_direct_backward_data(float *input_grad, const float *output_grad, const float *slabs, int batch,
+                                 int depth, int n, int k, int padding, int num_outputs) {
+    ok(cct_hip_conv_direct_backward_data(input_grad, output_grad, slabs, batch, depth, n, k, padding,
+                                         num_outputs),
+       "conv_direct_backward_data");
+  }
+  void conv_direct_backward_weights(float *model_grad, const float *output_grad, const float *input, int batch,
+                                    int depth, int n, int k, int padding, int num_outputs) {
+    ok(cct_hip_conv_direct_backward_weights(model_grad, output_grad, input, batch, depth, n, k, padding,
+                                            num_outputs),
+       "conv_direct_backward_weights");
+  }
   void sgemv(const CBLAS_TRANSPOSE TA, const int M, const int N, const float alpha, const float *pA,
              const float *px, const float beta, float *py) {
     ok(cct_hip_sgemv(TA, M, N, alpha, pA, px, beta, py), "sgemv");

@@ -113,6 +113,25 @@ class HIPDriver:
         check(self.lib.cct_hip_sgemm_conv_forward(o, batch, fmap, K, _p(model), _p(lowered), _p(bias),
                                                   _p(out)), "sgemm_conv_forward")
 
+    def conv_direct_supported(self, b, d, n, k, s, p, o):
+        return bool(self.lib.cct_hip_conv_direct_supported(b, d, n, k, s, p, o))
+
+    def conv_direct_slabs(self, slabs, model, o, d, k, for_data_gradient):
+        check(self.lib.cct_hip_conv_direct_slabs(_p(slabs), _p(model), o, d, k, int(for_data_gradient)),
+              "conv_direct_slabs")
+
+    def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o):
+        check(self.lib.cct_hip_conv_direct_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o),
+              "conv_direct_forward")
+
+    def conv_direct_backward_data(self, din, dout, slabs, b, d, n, k, p, o):
+        check(self.lib.cct_hip_conv_direct_backward_data(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o),
+              "conv_direct_backward_data")
+
+    def conv_direct_backward_weights(self, dw, dout, inp, b, d, n, k, p, o):
+        check(self.lib.cct_hip_conv_direct_backward_weights(_p(dw), _p(dout), _p(inp), b, d, n, k, p, o),
+              "conv_direct_backward_weights")
+
     def sgemv(self, TA, M, N, alpha, A, x, beta, y):
         check(self.lib.cct_hip_sgemv(TA, M, N, alpha, _p(A), _p(x), beta, _p(y)), "sgemv")
 

@@ -51,15 +51,21 @@ int cct_conv_bridge_create(cct_conv_bridge **out, int b, int d, int n, const cct
                            const cct_solver_param *solver, float *in_data, float *in_grad, float *out_data,
                            float *out_grad);
 int cct_conv_bridge_destroy(cct_conv_bridge *h);
-/* fused: single-GEMM forward epilogue + bias gradient inside the lift launch (default 1);
+/* fused: how much of the lowering pipeline is replaced.  0 = the reference's separate passes;
+ * 1 = forward GEMM epilogue does remap + bias, bias gradient inside the lift launch; 2 = as 1 with
+ * the data gradient from the direct-convolution kernel; 3 = forward and both gradients from direct
+ * kernels, no lowered matrix.  2 and 3 fall back to 1 where cct_hip_conv_direct_supported() says
+ * no.  A negative value keeps the bridge's default (2 where supported, else 1).
  * profile: per-stage hipEvent timing; needs_backward_grad: compute the input gradient
  * (the first weight layer of a net does not, src/DeepNet.h:1108-1110). */
 int cct_conv_bridge_set_options(cct_conv_bridge *h, int fused, int profile, int needs_backward_grad);
+/* The level in effect (0..3, see above). */
+int cct_conv_bridge_path(cct_conv_bridge *h);
 float *cct_conv_bridge_model(cct_conv_bridge *h);      /* [o][d][k][k] */
 float *cct_conv_bridge_bias(cct_conv_bridge *h);       /* [o] or NULL */
 float *cct_conv_bridge_model_grad(cct_conv_bridge *h);
 float *cct_conv_bridge_bias_grad(cct_conv_bridge *h);
-float *cct_conv_bridge_lowered(cct_conv_bridge *h);    /* [b*m*m][k*k*d], valid after forward */
+float *cct_conv_bridge_lowered(cct_conv_bridge *h);    /* [b*m*m][k*k*d], valid after forward (levels 0-2) */
 float *cct_conv_bridge_history(cct_conv_bridge *h);    /* momentum buffer of the weights */
 int cct_conv_bridge_forward(cct_conv_bridge *h);
 /* with_update != 0: ParallelizedBridge::backward (gradients, then SGD on weights and bias);

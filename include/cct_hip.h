@@ -155,6 +155,33 @@ int cct_hip_sgemm_new(int TA, int TB, int M, int N, int K, float alpha, const fl
  * epilogue: out[b][o][fmap] = model[o x K] * lowered[b*fmap x K]^T + bias[o] (bias may be NULL). */
 int cct_hip_sgemm_conv_forward(int o, int batch, int fmap, int K, const float *model,
                                const float *lowered, const float *bias, float *out);
+/* ---- stride-1 convolution without the lowered matrix ------------------------------------ */
+/* Fused replacements for chains of ConvolutionBridge's lowering pipeline when stride == 1 and
+ * k is 3 or 5 (padded image at most 32 wide).  Results agree with the lowering path to fp32
+ * rounding (the sums run in another order), not bit for bit.
+ * cct_hip_conv_direct_supported: 1 if both directions cover the geometry, else 0. */
+int cct_hip_conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding,
+                                  int num_outputs);
+/* Re-lays the model [o][d][k][k] into per-channel slabs: for_data_gradient == 0 gives
+ * [d][o][k*k] (forward), != 0 gives [o][d][k*k] with every filter reversed. */
+int cct_hip_conv_direct_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
+                              int for_data_gradient);
+/* lower_cube + forward GEMM + remap_output + bias of ConvolutionBridge::forward
+ * (src/bridges/ConvolutionBridge_impl.hxx:316-364) in one kernel:
+ * output[b][o][m][m] from input[b][d][n][n], forward slabs, bias[o] (may be NULL). */
+int cct_hip_conv_direct_forward(float *output, const float *input, const float *slabs,
+                                const float *bias, int batch, int depth, int n, int k, int padding,
+                                int num_outputs);
+/* Gradient remap + data-gradient GEMM + inverse_lower_cube of ConvolutionBridge::backward
+ * (src/bridges/ConvolutionBridge_impl.hxx:601-616) in one kernel: input_grad[b][d][n][n] from
+ * output_grad[b][o][m][m] (read in place, not permuted) and data-gradient slabs. */
+int cct_hip_conv_direct_backward_data(float *input_grad, const float *output_grad, const float *slabs,
+                                      int batch, int depth, int n, int k, int padding, int num_outputs);
+/* Weight-gradient GEMM of ConvolutionBridge::backward (src/bridges/ConvolutionBridge_impl.hxx:
+ * 619-621) without the lowered matrix or the gradient remap: model_grad[o][d][k][k] (overwritten,
+ * beta = 0) from output_grad[b][o][m][m] and input[b][d][n][n]. */
+int cct_hip_conv_direct_backward_weights(float *model_grad, const float *output_grad, const float *input,
+                                         int batch, int depth, int n, int k, int padding, int num_outputs);
 /* DeviceDriver::sgemv (src/sched/DeviceDriver.h:214-215): row-major M x N, lda = N. */
 int cct_hip_sgemv(int TA, int M, int N, float alpha, const float *A, const float *x, float beta,
                   float *y);

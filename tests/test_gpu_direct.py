@@ -1,0 +1,219 @@
+"""GPU parity of the direct-convolution kernels (stride 1, k = 3 or 5: forward, data gradient and
+weight gradient without the lowered matrix) against the CPU oracle's lowering pipeline, and of the
+ConvolutionBridge path levels against each other.  These kernels sum in another order than the
+lowered GEMMs, so the bar is the fp32 one: max|gpu - ref| / max|ref| <= 1e-4."""
+import numpy as np
+import pytest
+
+from gpu_util import dev, driver, empty, host, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+# b d n k p o  (stride is 1 throughout)
+SHAPES = [
+    (64, 1, 28, 5, 0, 20),    # LeNet conv1 (BASELINE config 1)
+    (8, 20, 12, 5, 0, 50),    # LeNet conv2: odd number of 32-row blocks, slabs not 16-byte aligned
+    (3, 96, 27, 5, 2, 256),   # AlexNet conv2 geometry
+    (2, 48, 27, 5, 2, 128),   # one group of CaffeNet conv2
+    (3, 256, 13, 3, 1, 384),  # AlexNet conv3 geometry
+    (2, 192, 13, 3, 1, 192),  # one group of conv4
+    (2, 4, 8, 3, 1, 5),       # tiny: tiles straddle several images
+    (3, 3, 12, 5, 2, 7),      # odd channel count in both directions
+    (3, 5, 9, 5, 4, 6),       # full padding (p = k-1)
+    (2, 6, 10, 3, 0, 40),     # no padding
+    (1, 7, 5, 5, 2, 3),       # image as small as the filter
+    (5, 9, 30, 3, 1, 33),     # padded width 32: the widest the kernels take
+    (4, 5, 7, 3, 1, 4),       # 7x7 images: a 128-pixel tile spans four of them
+]
+
+
+def _ids(s):
+    return "b%d_d%d_n%d_k%d_p%d_o%d" % s
+
+
+def _tensors(shape, seed):
+    b, d, n, k, p, o = shape
+    m = n + 2 * p - k + 1
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+    w = (rng.standard_normal((o, d, k, k)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(o).astype(np.float32)
+    og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+    return x, w, bias, og, m
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=_ids)
+def test_direct_kernels_match_oracle(oracle, shape):
+    b, d, n, k, p, o = shape
+    x, w, bias, og, m = _tensors(shape, 4321 + sum(shape))
+    drv = driver()
+    assert drv.conv_direct_supported(b, d, n, k, 1, p, o)
+    ref_out, lowered = oracle.conv_forward(x, w, bias, k, 1, p)
+    ref_dx, ref_dw, ref_db = oracle.conv_backward(x.shape, w, og, lowered, k, 1, p)
+
+    d_x, d_w, d_og = dev(x), dev(w), dev(og)
+    slabs_f, slabs_b = empty((d * o * k * k,)), empty((d * o * k * k,))
+    drv.conv_direct_slabs(slabs_f, d_w, o, d, k, 0)
+    drv.conv_direct_slabs(slabs_b, d_w, o, d, k, 1)
+    # slab layouts: [d][o][k*k] and [o][d][k*k] with reversed filters
+    np.testing.assert_array_equal(host(slabs_f).reshape(d, o, k * k), w.reshape(o, d, k * k).transpose(1, 0, 2))
+    np.testing.assert_array_equal(host(slabs_b).reshape(o, d, k * k), w.reshape(o, d, k * k)[:, :, ::-1])
+
+    out = empty((b, o, m, m))
+    drv.conv_direct_forward(out, d_x, slabs_f, dev(bias), b, d, n, k, p, o)
+    assert rel_err(host(out), ref_out) <= TOL
+    out_nb = empty((b, o, m, m))
+    drv.conv_direct_forward(out_nb, d_x, slabs_f, None, b, d, n, k, p, o)
+    assert rel_err(host(out_nb), ref_out - bias.reshape(1, o, 1, 1)) <= TOL
+
+    dx = empty((b, d, n, n))
+    drv.conv_direct_backward_data(dx, d_og, slabs_b, b, d, n, k, p, o)
+    assert rel_err(host(dx), ref_dx) <= TOL
+    np.testing.assert_array_equal(host(d_og), og)  # the output gradient is read in place, not permuted
+
+    dw = empty((o, d, k, k))
+    drv.conv_direct_backward_weights(dw, d_og, d_x, b, d, n, k, p, o)
+    assert rel_err(host(dw), ref_dw) <= TOL
+    # split-K partial sums are added in a fixed order: a second run gives the same bits
+    dw2 = empty((o, d, k, k))
+    drv.conv_direct_backward_weights(dw2, d_og, d_x, b, d, n, k, p, o)
+    np.testing.assert_array_equal(host(dw2), host(dw))
+
+
+def test_direct_exact_on_small_integers(oracle):
+    """Small-integer tensors make every sum exact in fp32, so the direct kernels must reproduce the
+    lowering pipeline bit for bit whatever the summation order."""
+    b, d, n, k, p, o = 3, 6, 11, 5, 2, 9
+    m = n + 2 * p - k + 1
+    rng = np.random.default_rng(99)
+    x = rng.integers(-3, 4, (b, d, n, n)).astype(np.float32)
+    w = rng.integers(-2, 3, (o, d, k, k)).astype(np.float32)
+    bias = rng.integers(-4, 5, o).astype(np.float32)
+    og = rng.integers(-3, 4, (b, o, m, m)).astype(np.float32)
+    ref_out, lowered = oracle.conv_forward(x, w, bias, k, 1, p)
+    ref_dx, ref_dw, _ = oracle.conv_backward(x.shape, w, og, lowered, k, 1, p)
+    drv = driver()
+    d_x, d_w, d_og = dev(x), dev(w), dev(og)
+    sf, sb = empty((w.size,)), empty((w.size,))
+    drv.conv_direct_slabs(sf, d_w, o, d, k, 0)
+    drv.conv_direct_slabs(sb, d_w, o, d, k, 1)
+    out, dx, dw = empty((b, o, m, m)), empty((b, d, n, n)), empty((o, d, k, k))
+    drv.conv_direct_forward(out, d_x, sf, dev(bias), b, d, n, k, p, o)
+    drv.conv_direct_backward_data(dx, d_og, sb, b, d, n, k, p, o)
+    drv.conv_direct_backward_weights(dw, d_og, d_x, b, d, n, k, p, o)
+    np.testing.assert_array_equal(host(out), ref_out)
+    np.testing.assert_array_equal(host(dx), ref_dx)
+    np.testing.assert_array_equal(host(dw).reshape(-1), np.asarray(ref_dw).reshape(-1))
+
+
+def test_direct_support_matrix_and_errors():
+    from caffecontroll_amd import CctHipError
+    drv = driver()
+    assert drv.conv_direct_supported(256, 96, 27, 5, 1, 2, 256)
+    assert drv.conv_direct_supported(256, 256, 13, 3, 1, 1, 384)
+    assert not drv.conv_direct_supported(256, 3, 227, 11, 4, 0, 96)   # k = 11, stride 4
+    assert not drv.conv_direct_supported(4, 3, 20, 5, 4, 2, 10)       # stride 4
+    assert not drv.conv_direct_supported(4, 3, 40, 5, 1, 2, 10)       # padded image wider than 32
+    assert not drv.conv_direct_supported(4, 3, 20, 5, 1, 5, 10)       # padding above k-1
+    assert not drv.conv_direct_supported(1, 2, 3, 3, 1, 0, 2)         # 1x1 output: a tile would span 128 images
+    with pytest.raises(CctHipError):
+        drv.conv_direct_forward(empty((1,)), empty((1,)), empty((1,)), None, 4, 3, 40, 5, 2, 10)
+    with pytest.raises(CctHipError):
+        drv.conv_direct_backward_weights(empty((1,)), empty((1,)), empty((1,)), 4, 3, 20, 7, 3, 10)
+    w = empty((10 * 3 * 25,), fill=1.0)
+    with pytest.raises(CctHipError):
+        drv.conv_direct_slabs(w, w, 10, 3, 5, 0)
+
+
+@pytest.mark.parametrize("shape", [(8, 96, 27, 5, 2, 256), (16, 20, 12, 5, 0, 50), (4, 256, 13, 3, 1, 384)],
+                         ids=_ids)
+def test_bridge_path_levels_agree(oracle, shape):
+    """ConvolutionBridge at path levels 0..3 (separate passes, fused epilogues, direct data
+    gradient, all direct): every level within 1e-4 of the oracle's CPU ConvolutionBridge."""
+    from caffecontroll_amd.bridges import ConvolutionLayer
+    b, d, n, k, p, o = shape
+    x, w, bias, og, m = _tensors(shape, 777 + sum(shape))
+    ref_out, lowered = oracle.conv_forward(x, w, bias, k, 1, p)
+    ref_dx, ref_dw, ref_db = oracle.conv_backward(x.shape, w, og, lowered, k, 1, p)
+    drv = driver()
+    for level in (0, 1, 2, 3):
+        in_data, in_grad = dev(x), empty((b, d, n, n))
+        out_data, out_grad = empty((b, o, m, m)), dev(og)
+        layer = ConvolutionLayer(b, d, n, k, 1, p, o, in_data, in_grad, out_data, out_grad)
+        assert layer.path() == 2  # default where the direct kernels cover the geometry
+        layer.set_options(fused=level)
+        assert layer.path() == level
+        drv.memcpy(layer.model_ptr(), w.ctypes.data, w.nbytes, 0)
+        drv.memcpy(layer.bias_ptr(), bias.ctypes.data, bias.nbytes, 0)
+        layer.forward()
+        layer.backward(with_update=False)
+        assert rel_err(host(out_data), ref_out) <= TOL, level
+        assert rel_err(host(in_grad), ref_dx) <= TOL, level
+        dw = np.empty((o, d, k, k), np.float32)
+        db = np.empty((o,), np.float32)
+        drv.memcpy(dw.ctypes.data, layer.model_grad_ptr(), dw.nbytes, 1)
+        drv.memcpy(db.ctypes.data, layer.bias_grad_ptr(), db.nbytes, 1)
+        assert rel_err(dw, np.asarray(ref_dw).reshape(dw.shape)) <= TOL, level
+        assert rel_err(db, ref_db) <= TOL, level
+        np.testing.assert_array_equal(host(out_grad), og)
+        layer.close()
+
+
+def test_bridge_falls_back_where_direct_does_not_apply():
+    from caffecontroll_amd.bridges import ConvolutionLayer
+    b, d, n, k, s, p, o = 2, 3, 20, 5, 4, 2, 10
+    m = (n + 2 * p - k) // s + 1
+    layer = ConvolutionLayer(b, d, n, k, s, p, o, empty((b, d, n, n), fill=0.0), empty((b, d, n, n)),
+                             empty((b, o, m, m)), empty((b, o, m, m), fill=0.0))
+    assert layer.path() == 1
+    layer.set_options(fused=3)
+    assert layer.path() == 1
+    layer.close()
+
+
+CFG2 = (256, 96, 27, 5, 2, 256)
+
+
+def test_full_size_direct_vs_float64():
+    """BASELINE config 2 at full size: the three direct kernels against torch's float64
+    convolution and its gradients (independent of this library and of the oracle)."""
+    import torch
+    import torch.nn.functional as F
+    b, d, n, k, p, o = CFG2
+    m = n + 2 * p - k + 1
+    drv = driver()
+    g = torch.Generator(device="cuda").manual_seed(1235)
+    x = torch.randn((b, d, n, n), device="cuda", generator=g)
+    w = torch.randn((o, d, k, k), device="cuda", generator=g) * 0.01
+    bias = torch.full((o,), 0.1, device="cuda")
+    og = torch.randn((b, o, m, m), device="cuda", generator=g)
+    sf, sb = empty((w.numel(),)), empty((w.numel(),))
+    drv.conv_direct_slabs(sf, w, o, d, k, 0)
+    drv.conv_direct_slabs(sb, w, o, d, k, 1)
+    out, dx, dw = empty((b, o, m, m)), empty((b, d, n, n)), empty((o, d, k, k))
+    drv.conv_direct_forward(out, x, sf, bias, b, d, n, k, p, o)
+    drv.conv_direct_backward_data(dx, og, sb, b, d, n, k, p, o)
+    drv.conv_direct_backward_weights(dw, og, x, b, d, n, k, p, o)
+    torch.cuda.synchronize()
+
+    def err(got, ref):
+        return ((got.double() - ref).abs().max() / ref.abs().max()).item()
+
+    # float64 references in chunks of 32 images to bound memory
+    worst_out = worst_dx = 0.0
+    dw_ref = torch.zeros((o, d, k, k), dtype=torch.float64, device="cuda")
+    wd = w.double()
+    scale_out = scale_dx = 0.0
+    for i in range(0, b, 32):
+        xs, gs = x[i:i + 32].double(), og[i:i + 32].double()
+        ro = F.conv2d(xs, wd, bias.double(), padding=p)
+        rdx = torch.nn.grad.conv2d_input(xs.shape, wd, gs, padding=p)
+        dw_ref += torch.nn.grad.conv2d_weight(xs, wd.shape, gs, padding=p)
+        worst_out = max(worst_out, (out[i:i + 32].double() - ro).abs().max().item())
+        worst_dx = max(worst_dx, (dx[i:i + 32].double() - rdx).abs().max().item())
+        scale_out = max(scale_out, ro.abs().max().item())
+        scale_dx = max(scale_dx, rdx.abs().max().item())
+    assert worst_out / scale_out <= TOL
+    assert worst_dx / scale_dx <= TOL
+    assert err(dw, dw_ref) <= TOL
