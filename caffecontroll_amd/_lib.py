@@ -73,6 +73,7 @@ PROTOTYPES = {
     "cct_hip_sgemm_new": [_I, _I, _I, _I, _I, _F, _P, _P, _F, _P],
     "cct_hip_sgemm_conv_forward": [_I, _I, _I, _I, _P, _P, _P, _P],
     "cct_hip_conv_direct_supported": [_I, _I, _I, _I, _I, _I, _I],
+    "cct_hip_conv_direct_slab_floats": [_I, _I, _I, _I],
     "cct_hip_conv_direct_slabs": [_P, _P, _I, _I, _I, _I],
     "cct_hip_conv_direct_forward": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I],
     "cct_hip_conv_direct_backward_data": [_P, _P, _P, _I, _I, _I, _I, _I, _I],
@@ -103,7 +104,7 @@ PROTOTYPES = {
     "cct_hip_timer_stop": [_P],
     "cct_hip_timer_elapsed_ms": [_P, C.POINTER(_F)],
 }
-_RESTYPE = {"cct_hip_last_error": C.c_char_p}
+_RESTYPE = {"cct_hip_last_error": C.c_char_p, "cct_hip_conv_direct_slab_floats": C.c_size_t}
 
 _lib = None
 

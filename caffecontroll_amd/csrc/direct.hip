@@ -37,7 +37,7 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float f4 __attribute__((ext_vector_type(4)));
 
 struct DirectArgs {
-  const float *wt;    // [kc][mtot][KS*KS]
+  const float *wt;    // slab buffer [kc padded to 4][mtot padded to whole tiles][KS*KS], zero padding
   const float *src;   // [batch][kc][hs][hs]
   float *dst;         // [batch][mtot][ho][ho]
   const float *bias;  // [mtot] or null
@@ -45,13 +45,26 @@ struct DirectArgs {
   int hp;             // ho + KS - 1 = hs + 2*pad: rows (and columns) of a zero-padded source image
   int pr;             // patch rows per channel
   int nsteps;         // ceil(kc / channels per step)
-  int wvec;           // weight slabs may be read with 16-byte loads
+  int slab_stride;    // floats between channels of the slab buffer (padded map count * KS*KS)
   uint32_t ptot;      // batch * ho * ho
   uint32_t tiles_m, ntiles;
   FastDiv div_ho, div_ho2, div_hp, div_pr;
 };
 
 constexpr int kDirectPatchLoads = 8;  // source elements per lane per step, at most
+
+// global -> LDS without passing through registers.  `lds_wave_base` is the wave-uniform LDS address
+// that lane 0's data goes to; lane l's 16 (or 4) bytes land 16*l (4*l) bytes further on.
+typedef __attribute__((address_space(3))) void lds_void;
+typedef const __attribute__((address_space(1))) void glb_void;
+__device__ __forceinline__ void lds_dma16(const float *g, float *lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(uintptr_t)lds_wave_base, 16, 0, 0);
+}
+__device__ __forceinline__ void lds_dma4(const float *g, float *lds_wave_base) {
+  __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(uintptr_t)lds_wave_base, 4, 0, 0);
+}
+// all of this wave's global->LDS loads have landed (vmcnt(0); expcnt/lgkmcnt left alone)
+__device__ __forceinline__ void lds_dma_wait() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
 // Fragments of contraction index idx = cp*KS*KS + j (idx is a constant after unrolling): weights of
 // tap j of channel pair cp for TMB row blocks, source elements under tap j for TNB pixel blocks.
@@ -92,8 +105,26 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
   const int v_lo = img0 * g.hp + y0;
 
   // ---- per-lane loader state -------------------------------------------------------------
-  // patch element e = (channel c, patch row, patch column): LDS offset e, source offset or -1
-  int psrc[NPL];
+  // Operands go from global memory straight into LDS (global_load_lds): a wave's load writes its
+  // 64 lanes' data to consecutive LDS addresses, so LDS element e is fetched by lane e % 64 of the
+  // wave-instruction that covers e.  Every address is a wave-uniform base that advances per step
+  // plus a per-lane offset fixed for the whole tile.
+  //   weights: the slab buffer is padded with zero rows and zero channels up to whole tiles and
+  //            whole steps, so the loads need no bounds tests;
+  //   source : patch element e = (channel c, patch row, patch column); elements outside the image
+  //            are never loaded -- their LDS words are cleared once below and stay zero.  A
+  //            channel past the last one (final step only) is not loaded either: whatever the
+  //            patch holds there is finite and meets zero weights.
+  uint32_t aoff[NA4];
+#pragma unroll
+  for (int i = 0; i < NA4; ++i) {
+    const int e4 = tid + i * 256;
+    const int c = e4 / SLAB4, f = (e4 - c * SLAB4) * 4;
+    aoff[i] = (uint32_t)(c * g.slab_stride + f);
+  }
+  uint32_t psrc[NPL];
+  uint32_t mask_all = 0, mask_last = 0;  // bit i: element i is loaded (any step / final step)
+  const int last_channels = g.kc - (g.nsteps - 1) * NC;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
     const uint32_t e = tid + i * 256;
@@ -104,62 +135,33 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     const int srow = (int)(v - img * g.hp) - g.pad, scol = (int)pc - g.pad;
     const bool ok = c < (uint32_t)NC && img < (uint32_t)g.batch && (unsigned)srow < (unsigned)g.hs &&
                     (unsigned)scol < (unsigned)g.hs;
-    psrc[i] = ok ? (int)(((img * g.kc + c) * g.hs + srow) * g.hs + scol) : -1;
+    psrc[i] = ok ? ((img * g.kc + c) * g.hs + srow) * g.hs + scol : 0u;
+    mask_all |= (ok ? 1u : 0u) << i;
+    mask_last |= ((ok && (int)c < last_channels) ? 1u : 0u) << i;
   }
-  const int chan_elems = g.hs * g.hs;
-  const int rows_valid = min(BM, g.mtot - m0);
-  const int slab_valid = rows_valid * KK;  // floats of a slab that belong to real output maps
+  const size_t a_step = (size_t)NC * g.slab_stride, b_step = (size_t)NC * g.hs * g.hs;
+  const float *a_tile = g.wt + (size_t)m0 * KK;
+  const int wave_elem0 = wave * 64;  // first element of this wave within a 256-element pass
 
-  f4 ra[NA4];
-  float rp[NPL];
-
-// global -> registers for step t
-#define CCT_DIRECT_FETCH(t)                                                                    \
+// global -> LDS stage s for step t (asynchronous; completion = vmcnt)
+#define CCT_DIRECT_ISSUE(t, s)                                                                 \
   do {                                                                                         \
-    const int c0_ = (t) * NC;                                                                  \
+    float *st_ = smem + (s) * stage;                                                           \
+    const float *ga_ = a_tile + (size_t)(t) * a_step;                                          \
     _Pragma("unroll") for (int i = 0; i < NA4; ++i) {                                          \
-      const int e4 = tid + i * 256;                                                            \
-      const int c = e4 / SLAB4, f = (e4 - c * SLAB4) * 4;                                      \
-      f4 v = f4{0.f, 0.f, 0.f, 0.f};                                                           \
-      if (e4 < ASZ / 4 && c0_ + c < g.kc) {                                                    \
-        const float *p = g.wt + ((size_t)(c0_ + c) * g.mtot + m0) * KK + f;                    \
-        if (g.wvec) {                                                                          \
-          if (f < slab_valid) v = *reinterpret_cast<const f4 *>(p);                            \
-        } else {                                                                               \
-          if (f + 0 < slab_valid) v.x = p[0];                                                  \
-          if (f + 1 < slab_valid) v.y = p[1];                                                  \
-          if (f + 2 < slab_valid) v.z = p[2];                                                  \
-          if (f + 3 < slab_valid) v.w = p[3];                                                  \
-        }                                                                                      \
-      }                                                                                        \
-      ra[i] = v;                                                                               \
+      if ((i + 1) * 256 <= ASZ / 4 || tid + i * 256 < ASZ / 4)                                 \
+        lds_dma16(ga_ + aoff[i], st_ + (i * 256 + wave_elem0) * 4);                            \
     }                                                                                          \
+    const float *gb_ = g.src + (size_t)(t) * b_step;                                           \
+    const uint32_t bm_ = ((t) == g.nsteps - 1) ? mask_last : mask_all;                         \
     _Pragma("unroll") for (int i = 0; i < NPL; ++i) {                                          \
-      float v = 0.f;                                                                           \
-      /* only the last step can run past the last channel */                                   \
-      if (psrc[i] >= 0 &&                                                                      \
-          (c0_ + NC <= g.kc || c0_ + (int)fdiv((uint32_t)(tid + i * 256) / PW, g.div_pr) < g.kc)) \
-        v = g.src[(size_t)psrc[i] + (size_t)c0_ * chan_elems];                                 \
-      rp[i] = v;                                                                               \
-    }                                                                                          \
-  } while (0)
-
-// registers -> LDS stage s
-#define CCT_DIRECT_STASH(s)                                                                    \
-  do {                                                                                         \
-    float *sa_ = smem + (s) * stage;                                                           \
-    _Pragma("unroll") for (int i = 0; i < NA4; ++i) {                                          \
-      const int e4 = tid + i * 256;                                                            \
-      if (e4 < ASZ / 4) *reinterpret_cast<f4 *>(sa_ + e4 * 4) = ra[i];                         \
-    }                                                                                          \
-    _Pragma("unroll") for (int i = 0; i < NPL; ++i) {                                          \
-      if (psrc[i] >= 0) sa_[ASZ + tid + i * 256] = rp[i];                                      \
+      if ((bm_ >> i) & 1u) lds_dma4(gb_ + psrc[i], st_ + ASZ + i * 256 + wave_elem0);          \
     }                                                                                          \
   } while (0)
 
   // clear the patches of both stages once: borders and rows outside the images stay zero
-  for (int s = 0; s < 2; ++s)
-    for (int e = tid; e < psz; e += 256) smem[s * stage + ASZ + e] = 0.f;
+  for (int s2 = 0; s2 < 2; ++s2)
+    for (int e = tid; e < psz; e += 256) smem[s2 * stage + ASZ + e] = 0.f;
   __syncthreads();
 
   // ---- per-lane fragment bases --------------------------------------------------------------
@@ -184,36 +186,57 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.0f;
 
-  CCT_DIRECT_FETCH(0);
-  CCT_DIRECT_STASH(0);
-  if (g.nsteps > 1) CCT_DIRECT_FETCH(1);
+  CCT_DIRECT_ISSUE(0, 0);
+  lds_dma_wait();
   __syncthreads();
 
   for (int t = 0; t < g.nsteps; ++t) {
     const float *sm = smem + (t & 1) * stage;
-    const bool more = t + 1 < g.nsteps;
-    float fa[2][TMB], fb[2][TNB];
-    direct_frags<KS, TMB, TNB, PW>(fa[0], fb[0], sm, abase, bbase, pair_stride, 0);
+    // every wave finished reading the other stage before the barrier that ended step t-1
+    if (t + 1 < g.nsteps) CCT_DIRECT_ISSUE(t + 1, (t & 1) ^ 1);
+    // Contraction indices are taken two at a time (neighbouring taps sit in neighbouring LDS words,
+    // which lets the compiler fetch both with one ds_read2); the fragments of pair q+1 are
+    // requested before the MFMAs of pair q.
+    constexpr int NI = CP * KK, NQ = (NI + 1) / 2;
+    float fa[2][2][TMB], fb[2][2][TNB];
+    direct_frags<KS, TMB, TNB, PW>(fa[0][0], fb[0][0], sm, abase, bbase, pair_stride, 0);
+    if (NI > 1) direct_frags<KS, TMB, TNB, PW>(fa[0][1], fb[0][1], sm, abase, bbase, pair_stride, 1);
 #pragma unroll
-    for (int idx = 0; idx < CP * KK; ++idx) {
-      // fragments of the next contraction index are requested before this one's MFMAs
-      if (idx + 1 < CP * KK)
-        direct_frags<KS, TMB, TNB, PW>(fa[(idx + 1) & 1], fb[(idx + 1) & 1], sm, abase, bbase, pair_stride,
-                                       idx + 1);
+    for (int q = 0; q < NQ; ++q) {
+      const int nb = (q + 1) & 1, cb = q & 1;
+      if (2 * q + 2 < NI)
+        direct_frags<KS, TMB, TNB, PW>(fa[nb][0], fb[nb][0], sm, abase, bbase, pair_stride, 2 * q + 2);
+      if (2 * q + 3 < NI)
+        direct_frags<KS, TMB, TNB, PW>(fa[nb][1], fb[nb][1], sm, abase, bbase, pair_stride, 2 * q + 3);
 #pragma unroll
-      for (int a = 0; a < TMB; ++a)
+      for (int e = 0; e < 2; ++e) {
+        if (2 * q + e < NI) {
 #pragma unroll
-        for (int b = 0; b < TNB; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[idx & 1][a], fb[idx & 1][b], acc[a][b], 0, 0, 0);
-      if (idx == 1 && more) {
-        CCT_DIRECT_STASH((t & 1) ^ 1);
-        if (t + 2 < g.nsteps) CCT_DIRECT_FETCH(t + 2);
+          for (int a2 = 0; a2 < TMB; ++a2)
+#pragma unroll
+            for (int b2 = 0; b2 < TNB; ++b2)
+              acc[a2][b2] =
+                  __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][e][a2], fb[cb][e][b2], acc[a2][b2], 0, 0, 0);
+        }
+      }
+      // Issue order inside this pair: one LDS read (of the next pair's fragments) after every few
+      // MFMAs, so the reads are in flight a whole pair ahead of their use and the matrix pipe never
+      // waits on LDS latency; the fence keeps the next pair's instructions from drifting up.
+      {
+        constexpr int NR = TMB + TNB, NM = 2 * TMB * TNB, PER = NM / (NR + 1) > 0 ? NM / (NR + 1) : 1;
+#pragma unroll
+        for (int k2 = 0; k2 < NR; ++k2) {
+          __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, NM - NR * PER > 0 ? NM - NR * PER : 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+    lds_dma_wait();
     __syncthreads();
   }
-#undef CCT_DIRECT_FETCH
-#undef CCT_DIRECT_STASH
+#undef CCT_DIRECT_ISSUE
 
   // ---- epilogue: accumulator register v of lane (r,h) is row 8*(v/4) + 4*h + v%4, column r ----
 #pragma unroll
@@ -232,16 +255,37 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
   }
 }
 
+// Output-map tile (in 32-row blocks) for `mtot` maps: least padding, larger tile on ties.
+static int direct_tmb(int mtot) {
+  int tmb = 4;
+  long best = -1;
+  for (int cand = 4; cand >= 2; --cand) {
+    const long padded = (long)((mtot + 32 * cand - 1) / (32 * cand)) * 32 * cand;
+    if (best < 0 || padded < best) { best = padded; tmb = cand; }
+  }
+  return tmb;
+}
+// Slab buffer dimensions: maps padded to whole tiles, channels to a multiple of 4 (a whole step).
+static int direct_padded_maps(int mtot) {
+  const int bm = 32 * direct_tmb(mtot);
+  return (mtot + bm - 1) / bm * bm;
+}
+static int direct_padded_channels(int kc) { return (kc + 3) / 4 * 4; }
+
 // wt[c][m][j] = w[m][c][j] (forward slabs) or w[c][m][KK-1-j] (data-gradient slabs: every filter
-// reversed).  `n_c`, `n_m` are the slab dimensions.
+// reversed), zero for padding maps and channels.  `n_c`, `n_m` are the real slab dimensions,
+// `p_m` the padded map count; one thread per element of the padded buffer.
 __global__ __launch_bounds__(256) void direct_slab_kernel(float *__restrict__ wt, const float *__restrict__ w,
-                                                          int n_c, int n_m, int kk, int reversed,
-                                                          FastDiv div_kk, FastDiv div_m) {
+                                                          int n_c, int n_m, int p_m, uint32_t total, int kk,
+                                                          int reversed, FastDiv div_kk, FastDiv div_m) {
   const uint32_t e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= (uint32_t)n_c * n_m * kk) return;
+  if (e >= total) return;
   const uint32_t cm = fdiv(e, div_kk), j = e - cm * kk;
-  const uint32_t c = fdiv(cm, div_m), m = cm - c * n_m;
-  wt[e] = reversed ? w[(size_t)cm * kk + (kk - 1 - j)] : w[((size_t)m * n_c + c) * kk + j];
+  const uint32_t c = fdiv(cm, div_m), m = cm - c * p_m;
+  float v = 0.f;
+  if (c < (uint32_t)n_c && m < (uint32_t)n_m)
+    v = reversed ? w[((size_t)c * n_m + m) * kk + (kk - 1 - j)] : w[((size_t)m * n_c + c) * kk + j];
+  wt[e] = v;
 }
 
 struct DirectPlan {
@@ -259,13 +303,7 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   if (hp > pw) return false;
   if ((double)batch * kc * hs * hs >= 2147483648.0 || (double)batch * ho * ho >= 2147483648.0) return false;
   const int cp = ks == 3 ? 2 : 1;
-  // output-map tile: least padding, larger tile on ties
-  int tmb = 4;
-  long best = -1;
-  for (int cand = 4; cand >= 2; --cand) {
-    const long padded = (long)((mtot + 32 * cand - 1) / (32 * cand)) * 32 * cand;
-    if (best < 0 || padded < best) { best = padded; tmb = cand; }
-  }
+  const int tmb = direct_tmb(mtot);
   const long tiles_m = (mtot + 32 * tmb - 1) / (32 * tmb);
   const long ptot = (long)batch * ho * ho;
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
@@ -313,7 +351,8 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
   g.hp = g.ho + ks - 1;
   g.pr = pl.pr;
   g.nsteps = (kc + 2 * pl.cp - 1) / (2 * pl.cp);
-  g.wvec = ((uintptr_t)wt % 16 == 0) && (((long)mtot * ks * ks) % 4 == 0);
+  CCT_REQUIRE((uintptr_t)wt % 16 == 0, "conv_direct: slab buffer must be 16-byte aligned");
+  g.slab_stride = direct_padded_maps(mtot) * ks * ks;
   g.ptot = (uint32_t)((long)batch * g.ho * g.ho);
   g.tiles_m = (uint32_t)((mtot + 32 * pl.tmb - 1) / (32 * pl.tmb));
   const uint32_t bn = 128 * pl.tnb;
@@ -628,18 +667,25 @@ extern "C" int cct_hip_conv_direct_supported(int batch, int depth, int n, int k,
              : 0;
 }
 
+extern "C" size_t cct_hip_conv_direct_slab_floats(int num_outputs, int depth, int k, int for_data_gradient) {
+  if (num_outputs <= 0 || depth <= 0 || k <= 0) return 0;
+  const int n_c = for_data_gradient ? num_outputs : depth, n_m = for_data_gradient ? depth : num_outputs;
+  return (size_t)direct_padded_channels(n_c) * direct_padded_maps(n_m) * k * k;
+}
+
 extern "C" int cct_hip_conv_direct_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
                                          int for_data_gradient) {
   CCT_ENSURE_INIT();
   CCT_REQUIRE(num_outputs > 0 && depth > 0 && k > 0, "conv_direct_slabs: bad dimensions");
   CCT_REQUIRE(slabs != model, "conv_direct_slabs: in-place use");
-  const long total = (long)num_outputs * depth * k * k;
-  CCT_REQUIRE(total < (1L << 31), "conv_direct_slabs: model too large");
+  const size_t total = cct_hip_conv_direct_slab_floats(num_outputs, depth, k, for_data_gradient);
+  CCT_REQUIRE(total < (1ull << 31), "conv_direct_slabs: model too large");
   // forward slabs: [depth][outputs][k*k]; data-gradient slabs: [outputs][depth][k*k] reversed
   const int n_c = for_data_gradient ? num_outputs : depth, n_m = for_data_gradient ? depth : num_outputs;
+  const int p_m = direct_padded_maps(n_m);
   hipLaunchKernelGGL(direct_slab_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, ctx().stream,
-                     slabs, model, n_c, n_m, k * k, for_data_gradient ? 1 : 0, make_fastdiv((uint32_t)(k * k)),
-                     make_fastdiv((uint32_t)n_m));
+                     slabs, model, n_c, n_m, p_m, (uint32_t)total, k * k, for_data_gradient ? 1 : 0,
+                     make_fastdiv((uint32_t)(k * k)), make_fastdiv((uint32_t)p_m));
   CCT_LAUNCH_CHECK();
   return 0;
 }

@@ -290,7 +290,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   LogicalCubeType *p_forward_lowered_data;
   LogicalCubeType *p_backward_inputgrad;
   LogicalCubeType *p_staging_cube;
-  LogicalCubeType *p_forward_slabs;   // model as [d][o][k*k] for the direct forward kernel
+  LogicalCubeType *p_forward_slabs;   // model as zero-padded [d][o][k*k] for the direct forward kernel
   LogicalCubeType *p_backward_slabs;  // model as [o][d][k*k], filters reversed, for the direct data gradient
   Connector<DataType, DriverClass> *p_forward_lower_connector;
   Kernel<DataType, KernelConfig_GEMM_NOTRANS_TRANS_NO_DIM_FLIP, DriverClass> *p_forward_gemm_kernel;
@@ -332,11 +332,15 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     return p_staging_cube;
   }
   LogicalCubeType *forward_slabs() {
-    if (!p_forward_slabs) p_forward_slabs = new LogicalCubeType(K, K, iD, num_output_features, p_driver);
+    if (!p_forward_slabs)
+      p_forward_slabs = new LogicalCubeType(
+          p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 0), 1, 1, 1, p_driver);
     return p_forward_slabs;
   }
   LogicalCubeType *backward_slabs() {
-    if (!p_backward_slabs) p_backward_slabs = new LogicalCubeType(K, K, iD, num_output_features, p_driver);
+    if (!p_backward_slabs)
+      p_backward_slabs = new LogicalCubeType(
+          p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 1), 1, 1, 1, p_driver);
     return p_backward_slabs;
   }
   void *timers_[STAGE_COUNT];

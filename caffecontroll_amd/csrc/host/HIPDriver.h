@@ -176,6 +176,9 @@ class HIPDriver {
   bool conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs) {
     return cct_hip_conv_direct_supported(batch, depth, n, k, stride, padding, num_outputs) != 0;
   }
+  size_t conv_direct_slab_floats(int num_outputs, int depth, int k, int for_data_gradient) {
+    return cct_hip_conv_direct_slab_floats(num_outputs, depth, k, for_data_gradient);
+  }
   void conv_direct_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
                          int for_data_gradient) {
     ok(cct_hip_conv_direct_slabs(slabs, model, num_outputs, depth, k, for_data_gradient), "conv_direct_slabs");

@@ -116,6 +116,9 @@ class HIPDriver:
     def conv_direct_supported(self, b, d, n, k, s, p, o):
         return bool(self.lib.cct_hip_conv_direct_supported(b, d, n, k, s, p, o))
 
+    def conv_direct_slab_floats(self, o, d, k, for_data_gradient):
+        return int(self.lib.cct_hip_conv_direct_slab_floats(o, d, k, int(for_data_gradient)))
+
     def conv_direct_slabs(self, slabs, model, o, d, k, for_data_gradient):
         check(self.lib.cct_hip_conv_direct_slabs(_p(slabs), _p(model), o, d, k, int(for_data_gradient)),
               "conv_direct_slabs")

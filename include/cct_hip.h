@@ -163,7 +163,11 @@ int cct_hip_sgemm_conv_forward(int o, int batch, int fmap, int K, const float *m
 int cct_hip_conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding,
                                   int num_outputs);
 /* Re-lays the model [o][d][k][k] into per-channel slabs: for_data_gradient == 0 gives
- * [d][o][k*k] (forward), != 0 gives [o][d][k*k] with every filter reversed. */
+ * [d][o][k*k] (forward), != 0 gives [o][d][k*k] with every filter reversed.  Both slab dimensions
+ * are padded with zeros (channels to a multiple of 4, maps to whole kernel tiles) so that the
+ * convolution kernels read them without bounds tests: `slabs` must hold
+ * cct_hip_conv_direct_slab_floats() floats and be 16-byte aligned. */
+size_t cct_hip_conv_direct_slab_floats(int num_outputs, int depth, int k, int for_data_gradient);
 int cct_hip_conv_direct_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
                               int for_data_gradient);
 /* lower_cube + forward GEMM + remap_output + bias of ConvolutionBridge::forward

@@ -32,6 +32,17 @@ def _ids(s):
     return "b%d_d%d_n%d_k%d_p%d_o%d" % s
 
 
+def _slabs(d_w, o, d, k):
+    """Forward and data-gradient slab buffers of the device model d_w."""
+    drv = driver()
+    out = []
+    for for_dgrad in (0, 1):
+        buf = empty((drv.conv_direct_slab_floats(o, d, k, for_dgrad),))
+        drv.conv_direct_slabs(buf, d_w, o, d, k, for_dgrad)
+        out.append(buf)
+    return out
+
+
 def _tensors(shape, seed):
     b, d, n, k, p, o = shape
     m = n + 2 * p - k + 1
@@ -53,12 +64,15 @@ def test_direct_kernels_match_oracle(oracle, shape):
     ref_dx, ref_dw, ref_db = oracle.conv_backward(x.shape, w, og, lowered, k, 1, p)
 
     d_x, d_w, d_og = dev(x), dev(w), dev(og)
-    slabs_f, slabs_b = empty((d * o * k * k,)), empty((d * o * k * k,))
-    drv.conv_direct_slabs(slabs_f, d_w, o, d, k, 0)
-    drv.conv_direct_slabs(slabs_b, d_w, o, d, k, 1)
-    # slab layouts: [d][o][k*k] and [o][d][k*k] with reversed filters
-    np.testing.assert_array_equal(host(slabs_f).reshape(d, o, k * k), w.reshape(o, d, k * k).transpose(1, 0, 2))
-    np.testing.assert_array_equal(host(slabs_b).reshape(o, d, k * k), w.reshape(o, d, k * k)[:, :, ::-1])
+    slabs_f, slabs_b = _slabs(d_w, o, d, k)
+    # slab layouts: [d][o][k*k] and [o][d][k*k] with reversed filters, zero-padded in both dimensions
+    for buf, n_c, n_m, ref in ((slabs_f, d, o, w.reshape(o, d, k * k).transpose(1, 0, 2)),
+                               (slabs_b, o, d, w.reshape(o, d, k * k)[:, :, ::-1])):
+        pc = -(-n_c // 4) * 4
+        got = host(buf).reshape(pc, -1, k * k)
+        assert got.shape[1] >= n_m and got.shape[1] % 32 == 0
+        np.testing.assert_array_equal(got[:n_c, :n_m], ref)
+        assert not got[n_c:].any() and not got[:, n_m:].any()
 
     out = empty((b, o, m, m))
     drv.conv_direct_forward(out, d_x, slabs_f, dev(bias), b, d, n, k, p, o)
@@ -95,9 +109,7 @@ def test_direct_exact_on_small_integers(oracle):
     ref_dx, ref_dw, _ = oracle.conv_backward(x.shape, w, og, lowered, k, 1, p)
     drv = driver()
     d_x, d_w, d_og = dev(x), dev(w), dev(og)
-    sf, sb = empty((w.size,)), empty((w.size,))
-    drv.conv_direct_slabs(sf, d_w, o, d, k, 0)
-    drv.conv_direct_slabs(sb, d_w, o, d, k, 1)
+    sf, sb = _slabs(d_w, o, d, k)
     out, dx, dw = empty((b, o, m, m)), empty((b, d, n, n)), empty((o, d, k, k))
     drv.conv_direct_forward(out, d_x, sf, dev(bias), b, d, n, k, p, o)
     drv.conv_direct_backward_data(dx, d_og, sb, b, d, n, k, p, o)
@@ -118,10 +130,10 @@ def test_direct_support_matrix_and_errors():
     assert not drv.conv_direct_supported(4, 3, 20, 5, 1, 5, 10)       # padding above k-1
     assert not drv.conv_direct_supported(1, 2, 3, 3, 1, 0, 2)         # 1x1 output: a tile would span 128 images
     with pytest.raises(CctHipError):
-        drv.conv_direct_forward(empty((1,)), empty((1,)), empty((1,)), None, 4, 3, 40, 5, 2, 10)
+        drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 40, 5, 2, 10)
     with pytest.raises(CctHipError):
         drv.conv_direct_backward_weights(empty((1,)), empty((1,)), empty((1,)), 4, 3, 20, 7, 3, 10)
-    w = empty((10 * 3 * 25,), fill=1.0)
+    w = empty((drv.conv_direct_slab_floats(10, 3, 5, 0),), fill=1.0)
     with pytest.raises(CctHipError):
         drv.conv_direct_slabs(w, w, 10, 3, 5, 0)
 
@@ -188,9 +200,7 @@ def test_full_size_direct_vs_float64():
     w = torch.randn((o, d, k, k), device="cuda", generator=g) * 0.01
     bias = torch.full((o,), 0.1, device="cuda")
     og = torch.randn((b, o, m, m), device="cuda", generator=g)
-    sf, sb = empty((w.numel(),)), empty((w.numel(),))
-    drv.conv_direct_slabs(sf, w, o, d, k, 0)
-    drv.conv_direct_slabs(sb, w, o, d, k, 1)
+    sf, sb = _slabs(w, o, d, k)
     out, dx, dw = empty((b, o, m, m)), empty((b, d, n, n)), empty((o, d, k, k))
     drv.conv_direct_forward(out, x, sf, bias, b, d, n, k, p, o)
     drv.conv_direct_backward_data(dx, og, sb, b, d, n, k, p, o)
