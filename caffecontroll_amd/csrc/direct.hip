@@ -53,15 +53,23 @@ struct DirectArgs {
 
 constexpr int kDirectPatchLoads = 8;  // source elements per lane per step, at most
 
-// global -> LDS without passing through registers.  `lds_wave_base` is the wave-uniform LDS address
-// that lane 0's data goes to; lane l's 16 (or 4) bytes land 16*l (4*l) bytes further on.
+// global -> LDS without passing through registers, as buffer loads: the address is
+// descriptor base + scalar offset + per-lane 32-bit byte offset, and a lane whose offset is
+// kOutOfRange (>= the descriptor's size) fetches nothing and writes zero.  `lds_wave_base` is the
+// wave-uniform LDS address that lane 0's data goes to; lane l's 16 (or 4) bytes land 16*l (4*l)
+// bytes further on.  The scalar offset does not take part in the range test, so every descriptor
+// is given the size 2^31 and the real bounds are kept by the callers' own index logic.
 typedef __attribute__((address_space(3))) void lds_void;
-typedef const __attribute__((address_space(1))) void glb_void;
-__device__ __forceinline__ void lds_dma16(const float *g, float *lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(uintptr_t)lds_wave_base, 16, 0, 0);
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr uint32_t kOutOfRange = 0x80000000u;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)kOutOfRange, 0x00020000);
 }
-__device__ __forceinline__ void lds_dma4(const float *g, float *lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((glb_void *)g, (lds_void *)(uintptr_t)lds_wave_base, 4, 0, 0);
+__device__ __forceinline__ void lds_dma16(rsrc_t r, uint32_t lane_bytes, uint32_t wave_bytes, float *lds_wave_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void *)(uintptr_t)lds_wave_base, 16, lane_bytes, wave_bytes, 0, 0);
+}
+__device__ __forceinline__ void lds_dma4(rsrc_t r, uint32_t lane_bytes, uint32_t wave_bytes, float *lds_wave_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void *)(uintptr_t)lds_wave_base, 4, lane_bytes, wave_bytes, 0, 0);
 }
 // all of this wave's global->LDS loads have landed (vmcnt(0); expcnt/lgkmcnt left alone)
 __device__ __forceinline__ void lds_dma_wait() { __builtin_amdgcn_s_waitcnt(0x0F70); }
@@ -83,15 +91,17 @@ template <int KS, int TMB, int TNB, int CP, int PW>
 __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g) {
   constexpr int KK = KS * KS, BM = 32 * TMB, BN = 128 * TNB, NC = 2 * CP;
   constexpr int ASZ = NC * BM * KK;           // floats of weight slabs per stage
+  constexpr int ASZP = (ASZ + 255) / 256 * 256;  // LDS room for them: whole 64-lane 16-byte loads
   constexpr int SLAB4 = BM * KK / 4;          // 16-byte vectors per slab
-  constexpr int NA4 = (ASZ / 4 + 255) / 256;  // 16-byte vectors per lane per stage
+  constexpr int NA4 = (ASZP / 4 + 255) / 256;  // 16-byte vectors per lane per stage
   constexpr int NPL = kDirectPatchLoads;
   extern __shared__ __attribute__((aligned(16))) float smem[];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // known to be wave-uniform
   const int r = lane & 31, h = lane >> 5;
-  const int psz = NC * g.pr * PW;  // floats of patches per stage
-  const int stage = ASZ + psz;     // multiple of 4: PW is
+  const int psz = (NC * g.pr * PW + 63) & ~63;  // floats of patches per stage: whole 64-lane loads
+  const int stage = ASZP + psz;
 
   const uint32_t id = xcd_remap(blockIdx.x, g.ntiles);
   const uint32_t tn = id / g.tiles_m, tm = id - tn * g.tiles_m;
@@ -112,18 +122,16 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
   //   weights: the slab buffer is padded with zero rows and zero channels up to whole tiles and
   //            whole steps, so the loads need no bounds tests;
   //   source : patch element e = (channel c, patch row, patch column); elements outside the image
-  //            are never loaded -- their LDS words are cleared once below and stay zero.  A
-  //            channel past the last one (final step only) is not loaded either: whatever the
-  //            patch holds there is finite and meets zero weights.
+  //            get the out-of-range offset and arrive as zeros, so do channels past the last one
+  //            in the final step.
   uint32_t aoff[NA4];
 #pragma unroll
   for (int i = 0; i < NA4; ++i) {
     const int e4 = tid + i * 256;
     const int c = e4 / SLAB4, f = (e4 - c * SLAB4) * 4;
-    aoff[i] = (uint32_t)(c * g.slab_stride + f);
+    aoff[i] = (uint32_t)(c * g.slab_stride + f) * 4u;  // bytes
   }
-  uint32_t psrc[NPL];
-  uint32_t mask_all = 0, mask_last = 0;  // bit i: element i is loaded (any step / final step)
+  uint32_t psrc[NPL], psrc_last[NPL];  // byte offsets for any step / for the final step
   const int last_channels = g.kc - (g.nsteps - 1) * NC;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
@@ -135,34 +143,29 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     const int srow = (int)(v - img * g.hp) - g.pad, scol = (int)pc - g.pad;
     const bool ok = c < (uint32_t)NC && img < (uint32_t)g.batch && (unsigned)srow < (unsigned)g.hs &&
                     (unsigned)scol < (unsigned)g.hs;
-    psrc[i] = ok ? ((img * g.kc + c) * g.hs + srow) * g.hs + scol : 0u;
-    mask_all |= (ok ? 1u : 0u) << i;
-    mask_last |= ((ok && (int)c < last_channels) ? 1u : 0u) << i;
+    psrc[i] = ok ? (((img * g.kc + c) * g.hs + srow) * g.hs + scol) * 4u : kOutOfRange;
+    psrc_last[i] = (ok && (int)c < last_channels) ? psrc[i] : kOutOfRange;
   }
-  const size_t a_step = (size_t)NC * g.slab_stride, b_step = (size_t)NC * g.hs * g.hs;
-  const float *a_tile = g.wt + (size_t)m0 * KK;
+  const uint32_t a_step = (uint32_t)NC * g.slab_stride * 4u, b_step = (uint32_t)NC * g.hs * g.hs * 4u;  // bytes
+  const rsrc_t a_rsrc = make_rsrc(g.wt + (size_t)m0 * KK), b_rsrc = make_rsrc(g.src);
   const int wave_elem0 = wave * 64;  // first element of this wave within a 256-element pass
 
 // global -> LDS stage s for step t (asynchronous; completion = vmcnt)
 #define CCT_DIRECT_ISSUE(t, s)                                                                 \
   do {                                                                                         \
     float *st_ = smem + (s) * stage;                                                           \
-    const float *ga_ = a_tile + (size_t)(t) * a_step;                                          \
+    const uint32_t ga_ = (uint32_t)(t) * a_step, gb_ = (uint32_t)(t) * b_step;                 \
     _Pragma("unroll") for (int i = 0; i < NA4; ++i) {                                          \
-      if ((i + 1) * 256 <= ASZ / 4 || tid + i * 256 < ASZ / 4)                                 \
-        lds_dma16(ga_ + aoff[i], st_ + (i * 256 + wave_elem0) * 4);                            \
+      if (i * 256 + wave_elem0 < ASZP / 4)                                                     \
+        lds_dma16(a_rsrc, (i * 256 + tid < ASZ / 4) ? aoff[i] : kOutOfRange, ga_,              \
+                  st_ + (i * 256 + wave_elem0) * 4);                                           \
     }                                                                                          \
-    const float *gb_ = g.src + (size_t)(t) * b_step;                                           \
-    const uint32_t bm_ = ((t) == g.nsteps - 1) ? mask_last : mask_all;                         \
+    const bool last_ = (t) == g.nsteps - 1;                                                    \
     _Pragma("unroll") for (int i = 0; i < NPL; ++i) {                                          \
-      if ((bm_ >> i) & 1u) lds_dma4(gb_ + psrc[i], st_ + ASZ + i * 256 + wave_elem0);          \
+      if (i * 256 + wave_elem0 < psz)                                                          \
+        lds_dma4(b_rsrc, last_ ? psrc_last[i] : psrc[i], gb_, st_ + ASZP + i * 256 + wave_elem0); \
     }                                                                                          \
   } while (0)
-
-  // clear the patches of both stages once: borders and rows outside the images stay zero
-  for (int s2 = 0; s2 < 2; ++s2)
-    for (int e = tid; e < psz; e += 256) smem[s2 * stage + ASZ + e] = 0.f;
-  __syncthreads();
 
   // ---- per-lane fragment bases --------------------------------------------------------------
   const int abase = h * (BM * KK) + r * KK;
@@ -174,7 +177,7 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     const uint32_t img = fdiv(p, g.div_ho2);
     const uint32_t pix = p - img * ho2;
     const uint32_t y = fdiv(pix, g.div_ho), x = pix - y * g.ho;
-    bbase[b] = ASZ + h * (g.pr * PW) + (int)(img * g.hp + y - v_lo) * PW + (int)x;
+    bbase[b] = ASZP + h * (g.pr * PW) + (int)(img * g.hp + y - v_lo) * PW + (int)x;
   }
   const int pair_stride = 2 * g.pr * PW;  // patch floats per channel pair
 
@@ -301,7 +304,8 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   if (ho <= 0) return false;
   const int pw = hp <= 16 ? 16 : 32;
   if (hp > pw) return false;
-  if ((double)batch * kc * hs * hs >= 2147483648.0 || (double)batch * ho * ho >= 2147483648.0) return false;
+  // buffer loads address a tensor through 32-bit byte offsets
+  if ((double)batch * kc * hs * hs >= 1073741824.0 || (double)batch * ho * ho >= 2147483648.0) return false;
   const int cp = ks == 3 ? 2 : 1;
   const int tmb = direct_tmb(mtot);
   const long tiles_m = (mtot + 32 * tmb - 1) / (32 * tmb);
@@ -312,7 +316,8 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
     const int rows = (ho - 1 + bn - 1) / ho + 1, imgs = (ho * ho - 1 + bn - 1) / (ho * ho) + 1;
     const int pr = rows - 1 + (imgs - 1) * (ks - 1) + ks;
     const long patch = 2L * cp * pr * pw;
-    const size_t lds = 2 * (size_t)(2 * cp * 32 * tmb * ks * ks + patch) * sizeof(float);
+    const size_t lds =
+        2 * (size_t)((2 * cp * 32 * tmb * ks * ks + 255) / 256 * 256 + (patch + 63) / 64 * 64) * sizeof(float);
     const long tiles = tiles_m * ((ptot + bn - 1) / bn);
     const bool fits = patch <= 256L * kDirectPatchLoads && lds <= 64 * 1024;
     // the wide tile only when it still gives every compute unit several workgroups
@@ -371,175 +376,228 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
 // Weight gradient without the lowered matrix:
 //   dW[oo][c][kr][kc] = sum_{img,r,x} dout[img][oo][r][x] * src[img][c][r-pad+kr][x-pad+kc]
 // as a GEMM with M = output maps, N = (c,kr,kc) columns and the contraction over output pixels.
-// A workgroup owns BM x BN of dW and a range of contraction steps; one step is two output rows
-// (r0, r0+1) of one image: MFMA lanes 0-31 take pixel (r0, x), lanes 32-63 pixel (r0+1, x).  Per
-// step the workgroup stages dout[img][m0..m0+BM)[rows r0,r0+1] (row stride odd: conflict-free
-// fragment reads) and, for the channels its columns touch, the KS+1 zero-padded source rows
-// under those two output rows; each lane's fragment addresses are base + x, so the loop over x
-// only bumps two offsets.  Single LDS stage with the next step's global loads parked in
-// registers during the MFMAs.  Partial sums of the step ranges go to a workspace and are added in
-// a fixed order by direct_reduce_kernel (run-to-run identical results).
+//
+// A workgroup of W wavefronts (W = 4..8) owns BM = 32*W maps x BN = 32*TB columns of dW and a range
+// of contraction steps; wavefront w holds rows 32w..32w+31 for all TB column blocks.  One step is
+// output row y of an image pair: MFMA lanes 0-31 take pixel (img0, y, x), lanes 32-63 pixel
+// (img0+1, y, x), x = 0..ho-1.  Per step the workgroup stages, straight from global memory into
+// LDS (global_load_lds, two LDS stages, one barrier per step):
+//   * the dout slab [BM][ast]: words 0..ho-1 of a row = row y of img0, ho..2ho-1 = row y of img0+1
+//     (ast odd, so the 32 rows a wavefront reads hit 32 banks).  The slab is filled as one flat run
+//     of 64-word chunks with per-lane source offsets that are fixed for the whole tile;
+//   * for the NCH channels its columns touch, the KS source rows under output row y of both
+//     images, zero-padded ([NCH][2*KS][PWS]); every word is rewritten every step, out-of-image
+//     words as zeros (out-of-range buffer loads).  PWS = KS and the channel stride = KS*KS (mod 32) make a
+//     wavefront's 32 consecutive (c,kr,kc) columns read 32 different banks.
+// Each lane's fragment addresses are base + x, so the loop over x only bumps offsets; fragments of
+// the next two x are requested while the MFMAs of the current two run.  Partial sums of the step
+// ranges go to a workspace and are added in a fixed order by direct_reduce_kernel (run-to-run
+// identical results).
 struct WgradArgs {
-  const float *dout;  // [batch][o][ho][ho]
-  const float *src;   // [batch][d][hs][hs]
-  float *out;         // [splits][o][ncols]
+  const float *dout;   // [batch][o][ho][ho]
+  const float *src;    // [batch][d][hs][hs]
+  float *out;          // [splits][o][ncols]
   int batch, o, d, hs, ho, pad;
-  int ncols;          // d * KS * KS
-  int chunks;         // row pairs per image: ceil(ho / 2)
-  int ast;            // floats between rows of the staged dout slab (odd)
-  int steps_total, steps_per_split;
+  int ncols;           // d * KS * KS
+  int ast;             // floats between rows of the staged dout slab (odd)
+  int bm;              // maps per workgroup = 32 * wavefronts
+  int a_floats;        // slab floats per stage, multiple of 64
+  int stage;           // floats per LDS stage
+  int steps_total, steps_per_split;  // a step = (image pair, output row)
   uint32_t tiles_m, tiles_n, ntiles, nblocks;
-  FastDiv div_chunks;
+  FastDiv div_ho, div_ast;
 };
 
 template <int KS, int PW>
 struct WgradStrides {
-  static constexpr int PWS = PW + ((KS - PW) % 32 + 32) % 32;                 // >= PW, == KS (mod 32)
-  static constexpr int RAW = (KS + 1) * PWS;
-  static constexpr int PCH = RAW + ((KS * KS - RAW) % 32 + 32) % 32;          // >= RAW, == KS*KS (mod 32)
+  static constexpr int PWS = PW + ((KS - PW) % 32 + 32) % 32;            // >= PW, == KS (mod 32)
+  static constexpr int RAW = 2 * KS * PWS;                               // two images' rows
+  static constexpr int PCH = RAW + ((KS * KS - RAW) % 32 + 32) % 32;     // >= RAW, == KS*KS (mod 32)
 };
 
-template <int KS, int TMB, int TNB, int PW>
-__global__ __launch_bounds__(256, 2) void conv_direct_wgrad_kernel(const WgradArgs g) {
-  constexpr int KK = KS * KS, BM = 32 * TMB, BN = 128 * TNB;
-  constexpr int PRW = KS + 1;                   // patch rows per channel
-  // LDS strides of the patch.  A wave's 32 columns are consecutive (c,kr,kc) triples that read
-  // patch offset c*PCH + kr*PWS + kc + x: with PWS = KS and PCH = KS*KS (mod 32) that offset is the
-  // column number plus a constant, i.e. 32 different banks.
-  constexpr int PWS = WgradStrides<KS, PW>::PWS, PCH = WgradStrides<KS, PW>::PCH;
-  constexpr int NCH = (BN - 1) / KK + 2;        // channels a column tile can touch
-  constexpr int NAL = BM / 4;                   // dout loads per lane per step (4 maps per pass)
-  constexpr int RPP = 256 / PW;                 // patch rows per pass
-  constexpr int CPP = RPP / PRW;                // whole channels per pass
-  constexpr int NBL = (NCH + CPP - 1) / CPP;    // source loads per lane per step
-  static_assert(CPP >= 1, "a pass must hold one channel's patch rows");
-  extern __shared__ __attribute__((aligned(16))) float smem[];
-  float *sa = smem;
-  float *sb = smem + ((BM * g.ast + 3) & ~3);
+constexpr int kWgradSlabLoads = 33;  // 64-word chunks of the dout slab per wavefront: ast/2 <= 32.5
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+template <int KS, int TB, int PW>
+__global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs g) {
+  constexpr int KK = KS * KS, BN = 32 * TB;
+  constexpr int PWS = WgradStrides<KS, PW>::PWS, PCH = WgradStrides<KS, PW>::PCH;
+  constexpr int NCH = (BN - 1) / KK + 2;                 // channels a column tile can touch
+  constexpr int BSZ = (NCH * PCH + 63) / 64 * 64;        // patch floats per stage
+  constexpr int NBL = (BSZ + 255) / 256;                 // source loads per lane per step (4 wavefronts)
+  constexpr int NAL = kWgradSlabLoads;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // known to be wave-uniform
+  const int nthreads = blockDim.x, nwaves = nthreads >> 6;
   const int r = lane & 31, h = lane >> 5;
   const uint32_t flat = xcd_remap(blockIdx.x, g.nblocks);
   const uint32_t z = flat / g.ntiles, id = flat - z * g.ntiles;
   const uint32_t tm = id / g.tiles_n, tn = id - tm * g.tiles_n;  // column tiles of one row tile run together
-  const int m0 = tm * BM, n0 = tn * BN, ch0 = n0 / KK;
+  const int m0 = tm * g.bm, n0 = tn * BN, ch0 = n0 / KK;
   const int s_beg = z * g.steps_per_split, s_end = min(g.steps_total, s_beg + g.steps_per_split);
   const int ho2 = g.ho * g.ho, hs2 = g.hs * g.hs;
 
-  // Loaders.  Every load address is a wave-uniform base (image, pass) plus a per-lane offset that
-  // does not change between steps.
-  //   dout: lane -> staged column ai (two output rows side by side), map arow + 4*pass
-  //   src : lane -> patch column pcol, patch row prow of channel chsub + CPP*pass
-  const int ai = tid & 63, arow = tid >> 6;
-  const bool a_ok = ai < 2 * g.ho;
-  const int a_lane = arow * ho2 + ai;
-  const int pcol = tid % PW, q = tid / PW;
-  const int chsub = q / PRW, prow = q - chsub * PRW;
-  const int scol = pcol - g.pad;
-  const bool b_lane_ok = chsub < CPP && (unsigned)scol < (unsigned)g.hs;
-  const int b_lane = chsub * hs2 + prow * g.hs + scol;
-  const int sb_lane = chsub * PCH + prow * PWS + pcol;
-
-  float ra[NAL], rb[NBL];
-#define CCT_WGRAD_FETCH(s)                                                                        \
-  do {                                                                                            \
-    const uint32_t img_ = fdiv((uint32_t)(s), g.div_chunks);                                      \
-    const int r0_ = 2 * ((s) - (int)img_ * g.chunks);                                             \
-    const bool pok_ = a_ok && r0_ * g.ho + ai < ho2;                                              \
-    const float *pa_ = g.dout + ((size_t)img_ * g.o + m0) * ho2 + r0_ * g.ho;                     \
-    _Pragma("unroll") for (int k = 0; k < NAL; ++k) {                                             \
-      ra[k] = (pok_ && m0 + arow + 4 * k < g.o) ? (pa_ + (size_t)k * 4 * ho2)[a_lane] : 0.f;      \
-    }                                                                                             \
-    const bool rok_ = b_lane_ok && (unsigned)(r0_ + prow - g.pad) < (unsigned)g.hs;               \
-    const float *pb_ = g.src + ((size_t)img_ * g.d + ch0) * hs2 + (r0_ - g.pad) * g.hs;           \
-    _Pragma("unroll") for (int k = 0; k < NBL; ++k) {                                             \
-      const int ch = k * CPP + chsub;                                                             \
-      rb[k] = (rok_ && ch < NCH && ch0 + ch < g.d) ? (pb_ + (size_t)k * CPP * hs2)[b_lane] : 0.f; \
-    }                                                                                             \
-  } while (0)
-#define CCT_WGRAD_STASH()                                                                         \
-  do {                                                                                            \
-    if (a_ok) {                                                                                   \
-      _Pragma("unroll") for (int k = 0; k < NAL; ++k) sa[(arow + 4 * k) * g.ast + ai] = ra[k];    \
-    }                                                                                             \
-    if (chsub < CPP) {                                                                            \
-      _Pragma("unroll") for (int k = 0; k < NBL; ++k) {                                           \
-        if (k * CPP + chsub < NCH) sb[k * (CPP * PCH) + sb_lane] = rb[k];                         \
-      }                                                                                           \
-    }                                                                                             \
-  } while (0)
-
-  // fragment bases: dout slab row (map) r of block a, half h -> second staged row; patch position of
-  // this lane's column (c, kr, kc), half h -> one patch row further down
-  int abase[TMB], bbase[TNB];
+  // ---- dout slab: chunk k of this wavefront covers slab words (k*nwaves + wave)*64 + lane ----
+  const int a_chunks = g.a_floats >> 6;
+  uint32_t aoff[NAL];   // source offset from the step base (img0, map m0, row y)
+  uint32_t a_second = 0;  // bit k: the word belongs to the second image of the pair
 #pragma unroll
-  for (int a = 0; a < TMB; ++a) abase[a] = (a * 32 + r) * g.ast + h * g.ho;
-#pragma unroll
-  for (int b = 0; b < TNB; ++b) {
-    const int col = min(n0 + wave * (32 * TNB) + b * 32 + r, g.ncols - 1);
-    const int c = col / KK, j = col - c * KK, kr = j / KS, kc = j - kr * KS;
-    bbase[b] = (c - ch0) * PCH + (h + kr) * PWS + kc;
-  }
-
-  v16f acc[TMB][TNB];
-#pragma unroll
-  for (int a = 0; a < TMB; ++a)
-#pragma unroll
-    for (int b = 0; b < TNB; ++b)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.0f;
-
-  if (s_beg < s_end) CCT_WGRAD_FETCH(s_beg);
-  for (int s = s_beg; s < s_end; ++s) {
-    CCT_WGRAD_STASH();
-    __syncthreads();
-    if (s + 1 < s_end) CCT_WGRAD_FETCH(s + 1);
-    float fa[2][TMB], fb[2][TNB];
-#pragma unroll
-    for (int a = 0; a < TMB; ++a) fa[0][a] = sa[abase[a]];
-#pragma unroll
-    for (int b = 0; b < TNB; ++b) fb[0][b] = sb[bbase[b]];
-    // x runs over the output row; two iterations per trip so the fragment buffers alternate statically
-    for (int x = 0; x < g.ho; x += 2) {
-      const int x1 = min(x + 1, g.ho - 1), x2 = min(x + 2, g.ho - 1);
-#pragma unroll
-      for (int a = 0; a < TMB; ++a) fa[1][a] = sa[abase[a] + x1];
-#pragma unroll
-      for (int b = 0; b < TNB; ++b) fb[1][b] = sb[bbase[b] + x1];
-#pragma unroll
-      for (int a = 0; a < TMB; ++a)
-#pragma unroll
-        for (int b = 0; b < TNB; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[0][a], fb[0][b], acc[a][b], 0, 0, 0);
-#pragma unroll
-      for (int a = 0; a < TMB; ++a) fa[0][a] = sa[abase[a] + x2];
-#pragma unroll
-      for (int b = 0; b < TNB; ++b) fb[0][b] = sb[bbase[b] + x2];
-      if (x + 1 < g.ho) {
-#pragma unroll
-        for (int a = 0; a < TMB; ++a)
-#pragma unroll
-          for (int b = 0; b < TNB; ++b)
-            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[1][a], fb[1][b], acc[a][b], 0, 0, 0);
-      }
+  for (int k = 0; k < NAL; ++k) {
+    const uint32_t e = (uint32_t)((k * nwaves + wave) * 64 + lane);
+    const uint32_t m = fdiv(e, g.div_ast), i = e - m * g.ast;
+    const uint32_t map = min((uint32_t)m0 + m, (uint32_t)g.o - 1) - m0;  // rows past the last map: any valid one
+    uint32_t off = map * ho2;
+    if (i < (uint32_t)g.ho) {
+      off += i;
+    } else if (i < 2u * g.ho) {
+      off += (uint32_t)g.o * ho2 + (i - g.ho);
+      a_second |= 1u << k;
     }
+    aoff[k] = off * 4u;  // bytes; pad words and words past the slab read word 0 of a valid row
+  }
+
+  // ---- source patches: element e = pass*nthreads + tid of the dense [NCH][PCH] array ----
+  uint32_t boff[NBL];  // source offset from the step base (img0, channel ch0, row y - pad)
+  uint32_t bmeta[NBL]; // bits 0-3: patch row within the image (0..KS-1); bit 4: second image; bit 5: statically valid
+#pragma unroll
+  for (int k = 0; k < NBL; ++k) {
+    const uint32_t e = (uint32_t)(k * nthreads + tid);
+    const uint32_t ch = e / PCH, rem = e - ch * PCH;
+    const uint32_t prow = rem / PWS, pcol = rem - prow * PWS;
+    const uint32_t second = prow >= (uint32_t)KS ? 1u : 0u, kr = prow - second * KS;
+    const int scol = (int)pcol - g.pad;
+    const bool ok = e < (uint32_t)(NCH * PCH) && prow < 2u * KS && ch0 + (int)ch < g.d &&
+                    (unsigned)scol < (unsigned)g.hs;
+    boff[k] = ok ? ((second * (uint32_t)g.d + ch) * hs2 + kr * g.hs + (uint32_t)scol) * 4u : 0u;  // bytes
+    bmeta[k] = kr | (second << 4) | ((ok ? 1u : 0u) << 5);
+  }
+
+  const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
+
+// global -> LDS stage st for step s
+#define CCT_WGRAD_ISSUE(s, st)                                                                    \
+  do {                                                                                            \
+    const uint32_t pair_ = fdiv((uint32_t)(s), g.div_ho);                                         \
+    const int y_ = (s) - (int)pair_ * g.ho;                                                       \
+    const int img0_ = 2 * (int)pair_;                                                             \
+    const bool two_ = img0_ + 1 < g.batch;                                                        \
+    float *sa_ = smem + (st) * g.stage;                                                           \
+    const uint32_t ga_ = (uint32_t)((((size_t)img0_ * g.o + m0) * ho2 + y_ * g.ho) * 4);          \
+    /* odd batch, last image alone: the second image's half reads zeros */                        \
+    const uint32_t second_ = two_ ? 0u : a_second;                                                \
+    _Pragma("unroll") for (int k = 0; k < NAL; ++k) {                                             \
+      if (k * nwaves + wave < a_chunks)                                                           \
+        lds_dma4(a_rsrc, ((second_ >> k) & 1u) ? kOutOfRange : aoff[k], ga_,                      \
+                 sa_ + (k * nwaves + wave) * 64);                                                 \
+    }                                                                                             \
+    float *sb_ = sa_ + g.a_floats;                                                                \
+    const uint32_t gb_ = (uint32_t)(((size_t)img0_ * g.d + ch0) * hs2 * 4);                       \
+    /* first patch row may lie above the image: that (negative) term goes into the lane offset, */ \
+    /* whose sum is non-negative for every lane that passes the row test                        */ \
+    const uint32_t row0_ = (uint32_t)((y_ - g.pad) * g.hs * 4);                                   \
+    _Pragma("unroll") for (int k = 0; k < NBL; ++k) {                                             \
+      const uint32_t mt_ = bmeta[k];                                                              \
+      const int srow_ = y_ - g.pad + (int)(mt_ & 15u);                                            \
+      const bool ok_ = (mt_ & 32u) && (unsigned)srow_ < (unsigned)g.hs && (two_ || !(mt_ & 16u)); \
+      if (k * nthreads + wave * 64 < BSZ)                                                         \
+        lds_dma4(b_rsrc, ok_ ? boff[k] + row0_ : kOutOfRange, gb_, sb_ + k * nthreads + wave * 64); \
+    }                                                                                             \
+  } while (0)
+
+  // ---- fragment bases ----------------------------------------------------------------------
+  const int abase = (wave * 32 + r) * g.ast + h * g.ho;
+  int bbase[TB];
+#pragma unroll
+  for (int b = 0; b < TB; ++b) {
+    const int col = min(n0 + b * 32 + r, g.ncols - 1);
+    const int c = col / KK, j = col - c * KK, kr = j / KS, kc = j - kr * KS;
+    bbase[b] = g.a_floats + (c - ch0) * PCH + (h * KS + kr) * PWS + kc;
+  }
+
+  v16f acc[TB];
+#pragma unroll
+  for (int b = 0; b < TB; ++b)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+
+  if (s_beg < s_end) {
+    CCT_WGRAD_ISSUE(s_beg, 0);
+    lds_dma_wait();
+  }
+  __syncthreads();
+
+  const int quads = g.ho >> 2, rest = g.ho & 3;
+  for (int s = s_beg; s < s_end; ++s) {
+    const int cur = (s - s_beg) & 1;
+    if (s + 1 < s_end) CCT_WGRAD_ISSUE(s + 1, cur ^ 1);
+    const float *sa = smem + cur * g.stage + abase;
+    const float *sb[TB];
+#pragma unroll
+    for (int b = 0; b < TB; ++b) sb[b] = smem + cur * g.stage + bbase[b];
+    // fragment buffers: [buffer][x parity]; loads past ho stay inside the stage and are not used
+    float fa[2][2], fb[2][2][TB];
+#define CCT_WGRAD_FRAGS(buf, x)                                                                   \
+  do {                                                                                            \
+    fa[buf][0] = sa[(x)];                                                                         \
+    fa[buf][1] = sa[(x) + 1];                                                                     \
+    _Pragma("unroll") for (int b = 0; b < TB; ++b) {                                              \
+      fb[buf][0][b] = sb[b][(x)];                                                                 \
+      fb[buf][1][b] = sb[b][(x) + 1];                                                             \
+    }                                                                                             \
+  } while (0)
+#define CCT_WGRAD_MFMA(buf, e)                                                                    \
+  do {                                                                                            \
+    _Pragma("unroll") for (int b = 0; b < TB; ++b)                                                \
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[buf][e], fb[buf][e][b], acc[b], 0, 0, 0); \
+  } while (0)
+// issue order of one x pair: an LDS read after every MFMA until the next pair's reads are out
+#define CCT_WGRAD_ORDER()                                                                         \
+  do {                                                                                            \
+    _Pragma("unroll") for (int k2 = 0; k2 < TB + 1; ++k2) {                                       \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                          \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                          \
+    }                                                                                             \
+    __builtin_amdgcn_sched_group_barrier(0x008, TB - 1, 0);                                       \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+  } while (0)
+    CCT_WGRAD_FRAGS(0, 0);
+    for (int qd = 0; qd < quads; ++qd) {
+      const int x = 4 * qd;
+      CCT_WGRAD_FRAGS(1, x + 2);
+      CCT_WGRAD_MFMA(0, 0);
+      CCT_WGRAD_MFMA(0, 1);
+      CCT_WGRAD_ORDER();
+      CCT_WGRAD_FRAGS(0, x + 4);
+      CCT_WGRAD_MFMA(1, 0);
+      CCT_WGRAD_MFMA(1, 1);
+      CCT_WGRAD_ORDER();
+    }
+    // remaining 0..3 columns; buffer 0 holds x = 4*quads and the one after it
+    if (rest >= 1) CCT_WGRAD_MFMA(0, 0);
+    if (rest >= 2) CCT_WGRAD_MFMA(0, 1);
+    if (rest == 3) {
+      CCT_WGRAD_FRAGS(1, 4 * quads + 2);
+      CCT_WGRAD_MFMA(1, 0);
+    }
+#undef CCT_WGRAD_FRAGS
+#undef CCT_WGRAD_MFMA
+#undef CCT_WGRAD_ORDER
+    lds_dma_wait();
     __syncthreads();
   }
-#undef CCT_WGRAD_FETCH
-#undef CCT_WGRAD_STASH
+#undef CCT_WGRAD_ISSUE
 
   float *out = g.out + (size_t)z * g.o * g.ncols;
 #pragma unroll
-  for (int b = 0; b < TNB; ++b) {
-    const int col = n0 + wave * (32 * TNB) + b * 32 + r;
+  for (int b = 0; b < TB; ++b) {
+    const int col = n0 + b * 32 + r;
     if (col >= g.ncols) continue;
 #pragma unroll
-    for (int a = 0; a < TMB; ++a)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int row = m0 + a * 32 + 8 * (v / 4) + 4 * h + (v % 4);
-        if (row < g.o) out[(size_t)row * g.ncols + col] = acc[a][b][v];
-      }
+    for (int v = 0; v < 16; ++v) {
+      const int row = m0 + wave * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+      if (row < g.o) out[(size_t)row * g.ncols + col] = acc[b][v];
+    }
   }
 }
 
@@ -553,78 +611,99 @@ __global__ __launch_bounds__(256) void direct_reduce_kernel(float *__restrict__ 
   dst[e] = s;
 }
 
-template <int KS, int PW>
-static int wgrad_launch(WgradArgs &g, int tmb, int tnb, size_t lds, hipStream_t st) {
-  dim3 grid(g.nblocks), block(256);
-#define CCT_WGRAD_CASE(TMB, TNB)                                                                       \
-  if (tmb == TMB && tnb == TNB) {                                                                      \
-    hipLaunchKernelGGL((conv_direct_wgrad_kernel<KS, TMB, TNB, PW>), grid, block, lds, st, g);         \
-    CCT_LAUNCH_CHECK();                                                                                \
-    return 0;                                                                                          \
-  }
-  CCT_WGRAD_CASE(2, 1) CCT_WGRAD_CASE(3, 1) CCT_WGRAD_CASE(4, 1)
-  CCT_WGRAD_CASE(2, 2) CCT_WGRAD_CASE(3, 2) CCT_WGRAD_CASE(4, 2)
-#undef CCT_WGRAD_CASE
-  return set_error(CCT_HIP_EINVAL, "conv_direct wgrad: no kernel instance for tile %dx%d", tmb, tnb);
-}
+struct WgradPlan {
+  int waves, tb, pw, ast, a_floats, stage;
+  size_t lds;
+};
 
-static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, int *tmb, int *tnb, int *pw,
-                       size_t *lds) {
+static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPlan *pl) {
   if (ks != 3 && ks != 5) return false;
   const int ho = n + 2 * pad - ks + 1, hp = ho + ks - 1;
   if (pad < 0 || pad > ks - 1 || ho <= 0 || hp > 32 || batch <= 0 || d <= 0 || o <= 0) return false;
-  if ((double)batch * o * ho * ho >= 2147483648.0 || (double)batch * d * n * n >= 2147483648.0 ||
+  // buffer loads address a tensor through 32-bit byte offsets
+  if ((double)batch * o * ho * ho >= 1073741824.0 || (double)batch * d * n * n >= 1073741824.0 ||
       (double)o * d * ks * ks >= 2147483648.0)
     return false;
-  *pw = hp <= 16 ? 16 : 32;
-  int best_tmb = 4;
+  pl->pw = hp <= 16 ? 16 : 32;
+  // wavefronts per workgroup (32 maps each): least padding of the map count, more wavefronts on ties
+  int best_w = 8;
   long best = -1;
-  for (int cand = 4; cand >= 2; --cand) {
-    const long padded = (long)((o + 32 * cand - 1) / (32 * cand)) * 32 * cand;
-    if (best < 0 || padded < best) { best = padded; best_tmb = cand; }
+  for (int w = 8; w >= 4; --w) {
+    const long padded = (long)((o + 32 * w - 1) / (32 * w)) * 32 * w;
+    if (best < 0 || padded < best) { best = padded; best_w = w; }
   }
-  *tmb = best_tmb;
-  // wide column tiles unless they pad the columns noticeably more than narrow ones
+  pl->waves = best_w;
+  // column blocks per tile: least padding of the column count, wider tile on ties
   const long ncols = (long)d * ks * ks;
-  const long pad2 = (ncols + 255) / 256 * 256, pad1 = (ncols + 127) / 128 * 128;
-  *tnb = (pad2 * 100 <= pad1 * 108) ? 2 : 1;
-  {
-    static const int forced = [] { const char *e = getenv("CCT_HIP_DIRECT_TNB"); return e ? atoi(e) : 0; }();
-    if (forced == 1 || forced == 2) *tnb = forced;
+  int best_tb = 6;
+  best = -1;
+  for (int tb = 6; tb >= 1; --tb) {
+    const long padded = (ncols + 32 * tb - 1) / (32 * tb) * 32 * tb;
+    if (best < 0 || padded < best) { best = padded; best_tb = tb; }
   }
-  const int ast = (2 * ho) | 1;
-  const int nch = (128 * *tnb - 1) / (ks * ks) + 2;
-  const int pws = *pw + (((ks - *pw) % 32) + 32) % 32, raw = (ks + 1) * pws;
+  {
+    static const int forced = [] { const char *e = getenv("CCT_HIP_DIRECT_TB"); return e ? atoi(e) : 0; }();
+    if (forced >= 1 && forced <= 6) best_tb = forced;  // tuning override, read once
+  }
+  pl->tb = best_tb;
+  pl->ast = (2 * ho) | 1;
+  pl->a_floats = (32 * pl->waves * pl->ast + 63) / 64 * 64;
+  if ((pl->a_floats / 64 + pl->waves - 1) / pl->waves > kWgradSlabLoads) return false;
+  const int pws = pl->pw + (((ks - pl->pw) % 32) + 32) % 32, raw = 2 * ks * pws;
   const int pch = raw + (((ks * ks - raw) % 32) + 32) % 32;  // WgradStrides<ks, pw>
-  *lds = (size_t)(((32 * *tmb * ast + 3) & ~3) + nch * pch) * sizeof(float);
-  return *lds <= 64 * 1024;
+  const int nch = (32 * pl->tb - 1) / (ks * ks) + 2;
+  const int bsz = (nch * pch + 63) / 64 * 64;
+  pl->stage = pl->a_floats + bsz;
+  pl->lds = (size_t)(2 * pl->stage + 16) * sizeof(float);  // slack: fragment loads may run a few words past
+  return pl->lds <= 160 * 1024;
+}
+
+template <int KS, int PW>
+static int wgrad_launch(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
+  dim3 grid(g.nblocks), block(64 * pl.waves);
+#define CCT_WGRAD_CASE(TB)                                                                              \
+  if (pl.tb == TB) {                                                                                    \
+    auto kern = conv_direct_wgrad_kernel<KS, TB, PW>;                                                   \
+    if (pl.lds > 64 * 1024)                                                                             \
+      CCT_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                        (int)pl.lds));                                                  \
+    hipLaunchKernelGGL(kern, grid, block, pl.lds, st, g);                                               \
+    CCT_LAUNCH_CHECK();                                                                                 \
+    return 0;                                                                                           \
+  }
+  CCT_WGRAD_CASE(1) CCT_WGRAD_CASE(2) CCT_WGRAD_CASE(3) CCT_WGRAD_CASE(4) CCT_WGRAD_CASE(5) CCT_WGRAD_CASE(6)
+#undef CCT_WGRAD_CASE
+  return set_error(CCT_HIP_EINVAL, "conv_direct wgrad: no kernel instance for %d column blocks", pl.tb);
 }
 
 static int conv_direct_wgrad(float *dw, const float *dout, const float *src, int batch, int d, int n, int ks,
                              int pad, int o) {
-  int tmb, tnb, pw;
-  size_t lds;
-  CCT_REQUIRE(wgrad_plan(batch, d, n, ks, pad, o, &tmb, &tnb, &pw, &lds),
+  WgradPlan pl;
+  CCT_REQUIRE(wgrad_plan(batch, d, n, ks, pad, o, &pl),
               "conv_direct wgrad: geometry not covered (k=%d pad=%d size=%d)", ks, pad, n);
   WgradArgs g;
   g.dout = dout; g.src = src;
   g.batch = batch; g.o = o; g.d = d; g.hs = n; g.pad = pad;
   g.ho = n + 2 * pad - ks + 1;
   g.ncols = d * ks * ks;
-  g.chunks = (g.ho + 1) / 2;
-  g.ast = (2 * g.ho) | 1;
-  g.steps_total = batch * g.chunks;
-  g.tiles_m = (uint32_t)((o + 32 * tmb - 1) / (32 * tmb));
-  g.tiles_n = (uint32_t)((g.ncols + 128 * tnb - 1) / (128 * tnb));
+  g.ast = pl.ast; g.bm = 32 * pl.waves; g.a_floats = pl.a_floats; g.stage = pl.stage;
+  g.steps_total = ((batch + 1) / 2) * g.ho;
+  g.tiles_m = (uint32_t)((o + g.bm - 1) / g.bm);
+  g.tiles_n = (uint32_t)((g.ncols + 32 * pl.tb - 1) / (32 * pl.tb));
   g.ntiles = g.tiles_m * g.tiles_n;
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
-  int splits = (int)(2L * cus / g.ntiles);
+  // workgroups resident per compute unit: LDS and wavefront slots (two per SIMD is plenty here)
+  int per_cu = (int)((160 * 1024) / pl.lds);
+  if (per_cu > 8 / pl.waves) per_cu = 8 / pl.waves;
+  if (per_cu < 1) per_cu = 1;
+  int splits = (int)((long)per_cu * cus / g.ntiles);
   if (splits < 1) splits = 1;
   if (splits > g.steps_total) splits = g.steps_total;
   g.steps_per_split = (g.steps_total + splits - 1) / splits;
   splits = (g.steps_total + g.steps_per_split - 1) / g.steps_per_split;
   g.nblocks = g.ntiles * (uint32_t)splits;
-  g.div_chunks = make_fastdiv((uint32_t)g.chunks);
+  g.div_ho = make_fastdiv((uint32_t)g.ho);
+  g.div_ast = make_fastdiv((uint32_t)g.ast);
   const size_t n_out = (size_t)o * g.ncols;
   if (splits > 1) {
     void *ws = nullptr;
@@ -636,8 +715,8 @@ static int conv_direct_wgrad(float *dw, const float *dout, const float *src, int
   }
   hipStream_t st = ctx().stream;
   int rc;
-  if (ks == 5) rc = pw == 16 ? wgrad_launch<5, 16>(g, tmb, tnb, lds, st) : wgrad_launch<5, 32>(g, tmb, tnb, lds, st);
-  else rc = pw == 16 ? wgrad_launch<3, 16>(g, tmb, tnb, lds, st) : wgrad_launch<3, 32>(g, tmb, tnb, lds, st);
+  if (ks == 5) rc = pl.pw == 16 ? wgrad_launch<5, 16>(g, pl, st) : wgrad_launch<5, 32>(g, pl, st);
+  else rc = pl.pw == 16 ? wgrad_launch<3, 16>(g, pl, st) : wgrad_launch<3, 32>(g, pl, st);
   if (rc) return rc;
   if (splits > 1) {
     hipLaunchKernelGGL(direct_reduce_kernel, dim3((uint32_t)((n_out + 255) / 256)), dim3(256), 0, st, dw, g.out,
@@ -658,11 +737,10 @@ extern "C" int cct_hip_conv_direct_supported(int batch, int depth, int n, int k,
   const int m = n + 2 * padding - k + 1;
   // forward: channels = depth, maps = outputs, source n, pad p; data gradient: channels = outputs,
   // maps = depth, source m, pad k-1-p
-  int tmb, tnb, pw;
-  size_t lds;
+  WgradPlan wp;
   return direct_plan(batch, depth, num_outputs, n, k, padding, &pl) &&
                  direct_plan(batch, num_outputs, depth, m, k, k - 1 - padding, &pl) &&
-                 wgrad_plan(batch, depth, n, k, padding, num_outputs, &tmb, &tnb, &pw, &lds)
+                 wgrad_plan(batch, depth, n, k, padding, num_outputs, &wp)
              ? 1
              : 0;
 }
