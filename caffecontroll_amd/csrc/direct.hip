@@ -410,7 +410,7 @@ struct WgradArgs {
 
 template <int KS, int PW>
 struct WgradStrides {
-  static constexpr int PWS = PW + ((KS - PW) % 32 + 32) % 32;            // >= PW, == KS (mod 32)
+  static constexpr int PWS = PW + KS;                                    // >= padded width; == KS (mod 32) for PW = 32
   static constexpr int RAW = 2 * KS * PWS;                               // two images' rows
   static constexpr int PCH = RAW + ((KS * KS - RAW) % 32 + 32) % 32;     // >= RAW, == KS*KS (mod 32)
 };
@@ -601,6 +601,191 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
   }
 }
 
+
+// The same computation with the output size, the wavefront count and hence every trip count known
+// at compile time (the AlexNet/CaffeNet shapes): the whole step is one straight line of code, so
+// the loads of the next step are spread between the MFMAs of this one instead of forming a phase
+// of their own.  Differences from the generic kernel: each wavefront stages its own 32 rows of the
+// dout slab (private, padded to whole 64-word loads), and the prefetch is unconditional -- the
+// last step of a range re-fetches itself into the idle stage.
+template <int KS, int TB, int PW, int HO, int W>
+__global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const WgradArgs g) {
+  constexpr int KK = KS * KS, BN = 32 * TB;
+  constexpr int PWS = WgradStrides<KS, PW>::PWS, PCH = WgradStrides<KS, PW>::PCH;
+  constexpr int NCH = (BN - 1) / KK + 2;
+  constexpr int BSZ = (NCH * PCH + 64 * W - 1) / (64 * W) * (64 * W);  // patch floats: whole passes
+  constexpr int NBW = BSZ / (64 * W);                                   // patch loads per lane per step
+  constexpr int AST = (2 * HO) | 1;
+  constexpr int RW = (32 * AST + 63) / 64 * 64;  // slab floats per wavefront
+  constexpr int NAW = RW / 64;                    // slab loads per lane per step
+  constexpr int AFL = W * RW, STAGE = AFL + BSZ;
+  constexpr int NQ = (HO + 1) / 2;                // x pairs per step
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, h = lane >> 5;
+  const uint32_t flat = xcd_remap(blockIdx.x, g.nblocks);
+  const uint32_t z = flat / g.ntiles, id = flat - z * g.ntiles;
+  const uint32_t tm = id / g.tiles_n, tn = id - tm * g.tiles_n;
+  const int m0 = tm * (32 * W), n0 = tn * BN, ch0 = n0 / KK;
+  const int s_beg = z * g.steps_per_split, s_end = min(g.steps_total, s_beg + g.steps_per_split);
+  constexpr int ho2 = HO * HO;
+  const int hs2 = g.hs * g.hs;
+
+  uint32_t aoff[NAW];
+  uint32_t a_second = 0;
+#pragma unroll
+  for (int k = 0; k < NAW; ++k) {
+    const uint32_t e = (uint32_t)(k * 64 + lane);
+    const uint32_t m = e / AST, i = e - m * AST;
+    const uint32_t map = min((uint32_t)(m0 + wave * 32) + min(m, 31u), (uint32_t)g.o - 1) - m0;
+    uint32_t off = map * ho2;
+    if (i < (uint32_t)HO) {
+      off += i;
+    } else if (i < 2u * HO) {
+      off += (uint32_t)g.o * ho2 + (i - HO);
+      a_second |= 1u << k;
+    }
+    aoff[k] = off * 4u;
+  }
+  uint32_t boff[NBW], bmeta[NBW];
+#pragma unroll
+  for (int k = 0; k < NBW; ++k) {
+    const uint32_t e = (uint32_t)(k * 64 * W + tid);
+    const uint32_t ch = e / PCH, rem = e - ch * PCH;
+    const uint32_t prow = rem / PWS, pcol = rem - prow * PWS;
+    const uint32_t second = prow >= (uint32_t)KS ? 1u : 0u, kr = prow - second * KS;
+    const int scol = (int)pcol - g.pad;
+    const bool ok = e < (uint32_t)(NCH * PCH) && prow < 2u * KS && ch0 + (int)ch < g.d &&
+                    (unsigned)scol < (unsigned)g.hs;
+    boff[k] = ok ? ((second * (uint32_t)g.d + ch) * hs2 + kr * g.hs + (uint32_t)scol) * 4u : 0u;
+    bmeta[k] = kr | (second << 4) | ((ok ? 1u : 0u) << 5);
+  }
+  const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
+
+  const int abase = wave * RW + r * AST + h * HO;
+  int bbase[TB];
+#pragma unroll
+  for (int b = 0; b < TB; ++b) {
+    const int col = min(n0 + b * 32 + r, g.ncols - 1);
+    const int c = col / KK, j = col - c * KK, kr = j / KS, kc = j - kr * KS;
+    bbase[b] = AFL + (c - ch0) * PCH + (h * KS + kr) * PWS + kc;
+  }
+
+  v16f acc[TB];
+#pragma unroll
+  for (int b = 0; b < TB; ++b)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+
+// per-step scalars of step s
+#define CCT_WSPEC_STEP(s)                                                                         \
+  const uint32_t pair_ = fdiv((uint32_t)(s), g.div_ho);                                           \
+  const int y_ = (s) - (int)pair_ * HO;                                                           \
+  const int img0_ = 2 * (int)pair_;                                                               \
+  const bool two_ = img0_ + 1 < g.batch;                                                          \
+  const uint32_t ga_ = (uint32_t)((((size_t)img0_ * g.o + m0) * ho2 + y_ * HO) * 4);              \
+  const uint32_t second_ = two_ ? 0u : a_second;                                                  \
+  const uint32_t gb_ = (uint32_t)(((size_t)img0_ * g.d + ch0) * hs2 * 4);                         \
+  const uint32_t row0_ = (uint32_t)((y_ - g.pad) * g.hs * 4)
+#define CCT_WSPEC_A(k, st)                                                                        \
+  lds_dma4(a_rsrc, ((second_ >> (k)) & 1u) ? kOutOfRange : aoff[k], ga_,                          \
+           smem + (st) * STAGE + wave * RW + (k) * 64)
+#define CCT_WSPEC_B(k, st)                                                                        \
+  do {                                                                                            \
+    const uint32_t mt_ = bmeta[k];                                                                \
+    const int srow_ = y_ - g.pad + (int)(mt_ & 15u);                                              \
+    const bool ok_ = (mt_ & 32u) && (unsigned)srow_ < (unsigned)g.hs && (two_ || !(mt_ & 16u));   \
+    lds_dma4(b_rsrc, ok_ ? boff[k] + row0_ : kOutOfRange, gb_,                                    \
+             smem + (st) * STAGE + AFL + (k) * 64 * W + wave * 64);                               \
+  } while (0)
+
+  if (s_beg < s_end) {
+    CCT_WSPEC_STEP(s_beg);
+#pragma unroll
+    for (int k = 0; k < NAW; ++k) CCT_WSPEC_A(k, 0);
+#pragma unroll
+    for (int k = 0; k < NBW; ++k) CCT_WSPEC_B(k, 0);
+    lds_dma_wait();
+  }
+  __syncthreads();
+
+  for (int s = s_beg; s < s_end; ++s) {
+    const int cur = (s - s_beg) & 1, nxt = cur ^ 1;
+    CCT_WSPEC_STEP(min(s + 1, s_end - 1));
+    const float *sa = smem + cur * STAGE + abase;
+    const float *sb = smem + cur * STAGE;
+    float fa[2][2], fb[2][2][TB];
+#define CCT_WSPEC_FRAGS(buf, x)                                                                   \
+  do {                                                                                            \
+    fa[buf][0] = sa[(x)];                                                                         \
+    fa[buf][1] = sa[(x) + 1];                                                                     \
+    _Pragma("unroll") for (int b = 0; b < TB; ++b) {                                              \
+      fb[buf][0][b] = sb[bbase[b] + (x)];                                                         \
+      fb[buf][1][b] = sb[bbase[b] + (x) + 1];                                                     \
+    }                                                                                             \
+  } while (0)
+    CCT_WSPEC_FRAGS(0, 0);
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+      const int cb = q & 1, nb = cb ^ 1;
+      if (q + 1 < NQ) CCT_WSPEC_FRAGS(nb, 2 * q + 2);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        if (2 * q + e < HO) {
+#pragma unroll
+          for (int b = 0; b < TB; ++b)
+            acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][e], fb[cb][e][b], acc[b], 0, 0, 0);
+        }
+      }
+      // this pair's share of the next step's loads
+      constexpr int A0 = 0;
+      (void)A0;
+      const int a_lo = q * NAW / NQ, a_hi = (q + 1) * NAW / NQ;
+      const int b_lo = q * NBW / NQ, b_hi = (q + 1) * NBW / NQ;
+#pragma unroll
+      for (int k = 0; k < NAW; ++k)
+        if (k >= a_lo && k < a_hi) CCT_WSPEC_A(k, nxt);
+#pragma unroll
+      for (int k = 0; k < NBW; ++k)
+        if (k >= b_lo && k < b_hi) CCT_WSPEC_B(k, nxt);
+      // issue order: LDS reads of the next pair first, one per MFMA, then the global loads
+      {
+        constexpr int NM = 2 * TB;
+        const int nr = (q + 1 < NQ) ? TB + 1 : 0;
+        const int nv = (a_hi - a_lo) + (b_hi - b_lo);
+        const int nm = (2 * q + 1 < HO) ? NM : TB;
+#pragma unroll
+        for (int k2 = 0; k2 < NM; ++k2) {
+          if (k2 < nm) __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          if (k2 < nr) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          else if (k2 - nr < nv) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#undef CCT_WSPEC_FRAGS
+    lds_dma_wait();
+    __syncthreads();
+  }
+#undef CCT_WSPEC_STEP
+#undef CCT_WSPEC_A
+#undef CCT_WSPEC_B
+
+  float *out = g.out + (size_t)z * g.o * g.ncols;
+#pragma unroll
+  for (int b = 0; b < TB; ++b) {
+    const int col = n0 + b * 32 + r;
+    if (col >= g.ncols) continue;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = m0 + wave * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+      if (row < g.o) out[(size_t)row * g.ncols + col] = acc[b][v];
+    }
+  }
+}
+
 // dst[e] = sum_z ws[z][e], z ascending
 __global__ __launch_bounds__(256) void direct_reduce_kernel(float *__restrict__ dst, const float *__restrict__ ws,
                                                             uint32_t n, int splits) {
@@ -613,6 +798,7 @@ __global__ __launch_bounds__(256) void direct_reduce_kernel(float *__restrict__ 
 
 struct WgradPlan {
   int waves, tb, pw, ast, a_floats, stage;
+  bool spec;  // a compile-time specialised instance exists for this shape
   size_t lds;
 };
 
@@ -626,9 +812,11 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
     return false;
   pl->pw = hp <= 16 ? 16 : 32;
   // wavefronts per workgroup (32 maps each): least padding of the map count, more wavefronts on ties
+  // (8 and 4 first: they load the four SIMDs of a compute unit evenly)
   int best_w = 8;
   long best = -1;
-  for (int w = 8; w >= 4; --w) {
+  static const int wave_choices[5] = {8, 4, 6, 7, 5};
+  for (int w : wave_choices) {
     const long padded = (long)((o + 32 * w - 1) / (32 * w)) * 32 * w;
     if (best < 0 || padded < best) { best = padded; best_w = w; }
   }
@@ -649,13 +837,36 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
   pl->ast = (2 * ho) | 1;
   pl->a_floats = (32 * pl->waves * pl->ast + 63) / 64 * 64;
   if ((pl->a_floats / 64 + pl->waves - 1) / pl->waves > kWgradSlabLoads) return false;
-  const int pws = pl->pw + (((ks - pl->pw) % 32) + 32) % 32, raw = 2 * ks * pws;
+  const int pws = pl->pw + ks, raw = 2 * ks * pws;
   const int pch = raw + (((ks * ks - raw) % 32) + 32) % 32;  // WgradStrides<ks, pw>
   const int nch = (32 * pl->tb - 1) / (ks * ks) + 2;
   const int bsz = (nch * pch + 63) / 64 * 64;
   pl->stage = pl->a_floats + bsz;
+  pl->spec = (ks == 5 && ho == 27 && pl->pw == 32 && pl->tb == 5 && (pl->waves == 4 || pl->waves == 8)) ||
+             (ks == 3 && ho == 13 && pl->pw == 16 && pl->tb == 6 &&
+              (pl->waves == 4 || pl->waves == 6 || pl->waves == 8));
+  {
+    static const int off = [] { const char *e = getenv("CCT_HIP_DIRECT_NOSPEC"); return e ? atoi(e) : 0; }();
+    if (off) pl->spec = false;  // tuning override, read once
+  }
+  if (pl->spec) {
+    // layout of conv_direct_wgrad_spec_kernel: private slab per wavefront, patches in whole passes
+    const int rw = (32 * pl->ast + 63) / 64 * 64;
+    pl->a_floats = pl->waves * rw;
+    pl->stage = pl->a_floats + (nch * pch + 64 * pl->waves - 1) / (64 * pl->waves) * (64 * pl->waves);
+  }
   pl->lds = (size_t)(2 * pl->stage + 16) * sizeof(float);  // slack: fragment loads may run a few words past
   return pl->lds <= 160 * 1024;
+}
+
+template <int KS, int TB, int PW, int HO, int W>
+static int wgrad_launch_spec(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
+  auto kern = conv_direct_wgrad_spec_kernel<KS, TB, PW, HO, W>;
+  if (pl.lds > 64 * 1024)
+    CCT_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds));
+  hipLaunchKernelGGL(kern, dim3(g.nblocks), dim3(64 * W), pl.lds, st, g);
+  CCT_LAUNCH_CHECK();
+  return 0;
 }
 
 template <int KS, int PW>
@@ -715,7 +926,13 @@ static int conv_direct_wgrad(float *dw, const float *dout, const float *src, int
   }
   hipStream_t st = ctx().stream;
   int rc;
-  if (ks == 5) rc = pl.pw == 16 ? wgrad_launch<5, 16>(g, pl, st) : wgrad_launch<5, 32>(g, pl, st);
+  if (pl.spec && ks == 5)
+    rc = pl.waves == 8 ? wgrad_launch_spec<5, 5, 32, 27, 8>(g, pl, st) : wgrad_launch_spec<5, 5, 32, 27, 4>(g, pl, st);
+  else if (pl.spec)
+    rc = pl.waves == 8   ? wgrad_launch_spec<3, 6, 16, 13, 8>(g, pl, st)
+         : pl.waves == 6 ? wgrad_launch_spec<3, 6, 16, 13, 6>(g, pl, st)
+                         : wgrad_launch_spec<3, 6, 16, 13, 4>(g, pl, st);
+  else if (ks == 5) rc = pl.pw == 16 ? wgrad_launch<5, 16>(g, pl, st) : wgrad_launch<5, 32>(g, pl, st);
   else rc = pl.pw == 16 ? wgrad_launch<3, 16>(g, pl, st) : wgrad_launch<3, 32>(g, pl, st);
   if (rc) return rc;
   if (splits > 1) {
