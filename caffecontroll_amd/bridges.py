@@ -85,7 +85,7 @@ class ConvolutionLayer:
 
     def set_options(self, fused=None, profile=False, needs_backward_grad=True):
         """fused: path level 0..3 (0 separate passes, 1 fused epilogues, 2 direct data gradient,
-        3 all-direct, no lowered matrix); None keeps the bridge's default (2 where the geometry is
+        3 all-direct, no lowered matrix); None keeps the bridge's default (3 where the geometry is
         covered by the direct kernels, else 1).  True/False mean "default" / 0."""
         if fused is None or fused is True:
             level = -1

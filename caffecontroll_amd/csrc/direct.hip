@@ -855,7 +855,10 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
     pl->a_floats = pl->waves * rw;
     pl->stage = pl->a_floats + (nch * pch + 64 * pl->waves - 1) / (64 * pl->waves) * (64 * pl->waves);
   }
-  pl->lds = (size_t)(2 * pl->stage + 16) * sizeof(float);  // slack: fragment loads may run a few words past
+  // fragment loads may run a few words past the last patch row: the padding of the patch region
+  // absorbs that, else a little slack is added
+  const int tail_pad = pl->stage - pl->a_floats - nch * pch;
+  pl->lds = (size_t)(2 * pl->stage + (tail_pad >= 8 ? 0 : 16)) * sizeof(float);
   return pl->lds <= 160 * 1024;
 }
 

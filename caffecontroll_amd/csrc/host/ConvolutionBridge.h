@@ -12,8 +12,8 @@
 //     of running remap_output and the bias map as separate passes (set_fused(false) restores
 //     the staged sequence);
 //   * the bias gradient is reduced in the same launch as the lifting kernel;
-//   * for stride-1 layers with k = 3 or 5 the data gradient (path level 2, the default where the
-//     geometry allows it) or all three products (level 3) come from direct-convolution kernels
+//   * for stride-1 layers with k = 3 or 5 the data gradient (path level 2) or all three products
+//     (level 3, the default where the geometry allows it) come from direct-convolution kernels
 //     that never materialise the lowered matrices; results then agree with the lowering path to
 //     fp32 rounding instead of bit for bit.  The lowered buffers are allocated on first use, so
 //     level 3 runs without them.
@@ -118,7 +118,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
         &lowered_forward_model, &lowered_forward_output, &lowered_data, p_driver);
     direct_ok_ = p_driver->conv_direct_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
                                                  (int)num_output_features);
-    path_ = direct_ok_ ? PATH_DIRECT_DATA : PATH_FUSED;
+    path_ = direct_ok_ ? PATH_DIRECT_ALL : PATH_FUSED;
     for (int i = 0; i < STAGE_COUNT; ++i) { timers_[i] = nullptr; stage_ms_[i] = 0.f; }
   }
 
@@ -155,7 +155,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     path_ = level;
   }
   int path() const { return path_; }
-  void set_fused(bool on) { set_path(on ? (direct_ok_ ? PATH_DIRECT_DATA : PATH_FUSED) : PATH_STAGED); }
+  void set_fused(bool on) { set_path(on ? (direct_ok_ ? PATH_DIRECT_ALL : PATH_FUSED) : PATH_STAGED); }
   // per-stage hipEvent timing (the reference's -D_DETAILED_PROFILING stage prints)
   void set_stage_profiling(bool on) { profile_ = on; }
   float stage_ms(int stage) {

@@ -153,7 +153,7 @@ def test_bridge_path_levels_agree(oracle, shape):
         in_data, in_grad = dev(x), empty((b, d, n, n))
         out_data, out_grad = empty((b, o, m, m)), dev(og)
         layer = ConvolutionLayer(b, d, n, k, 1, p, o, in_data, in_grad, out_data, out_grad)
-        assert layer.path() == 2  # default where the direct kernels cover the geometry
+        assert layer.path() == 3  # default where the direct kernels cover the geometry
         layer.set_options(fused=level)
         assert layer.path() == level
         drv.memcpy(layer.model_ptr(), w.ctypes.data, w.nbytes, 0)
