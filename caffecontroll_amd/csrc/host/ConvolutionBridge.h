@@ -118,7 +118,11 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
         &lowered_forward_model, &lowered_forward_output, &lowered_data, p_driver);
     direct_ok_ = p_driver->conv_direct_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
                                                  (int)num_output_features);
-    path_ = direct_ok_ ? PATH_DIRECT_ALL : PATH_FUSED;
+    // Small layers (LeNet-sized) stay on the fused lowering path by default: the direct kernels'
+    // fixed costs (slab re-layout, partial-sum reduction) outweigh what they save below a few GFLOP.
+    const double gemm_flop = 2.0 * num_output_features * (double)(oR * oC * iB) * (double)(K * K * iD);
+    default_path_ = (direct_ok_ && gemm_flop >= 2e9) ? PATH_DIRECT_ALL : PATH_FUSED;
+    path_ = default_path_;
     for (int i = 0; i < STAGE_COUNT; ++i) { timers_[i] = nullptr; stage_ms_[i] = 0.f; }
   }
 
@@ -155,7 +159,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     path_ = level;
   }
   int path() const { return path_; }
-  void set_fused(bool on) { set_path(on ? (direct_ok_ ? PATH_DIRECT_ALL : PATH_FUSED) : PATH_STAGED); }
+  void set_fused(bool on) { set_path(on ? default_path_ : PATH_STAGED); }
   // per-stage hipEvent timing (the reference's -D_DETAILED_PROFILING stage prints)
   void set_stage_profiling(bool on) { profile_ = on; }
   float stage_ms(int stage) {
@@ -317,7 +321,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   }
 
  private:
-  int path_ = PATH_FUSED;
+  int path_ = PATH_FUSED, default_path_ = PATH_FUSED;
   bool direct_ok_ = false, profile_ = false;
   LogicalCubeType *lowered() {
     if (!p_forward_lowered_data) p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);

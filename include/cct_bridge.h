@@ -55,7 +55,8 @@ int cct_conv_bridge_destroy(cct_conv_bridge *h);
  * 1 = forward GEMM epilogue does remap + bias, bias gradient inside the lift launch; 2 = as 1 with
  * the data gradient from the direct-convolution kernel; 3 = forward and both gradients from direct
  * kernels, no lowered matrix.  2 and 3 fall back to 1 where cct_hip_conv_direct_supported() says
- * no.  A negative value keeps the bridge's default (3 where supported, else 1).
+ * no.  A negative value keeps the bridge's default (3 where supported and the layer's
+ * GEMMs are at least 2 GFLOP each, else 1).
  * profile: per-stage hipEvent timing; needs_backward_grad: compute the input gradient
  * (the first weight layer of a net does not, src/DeepNet.h:1108-1110). */
 int cct_conv_bridge_set_options(cct_conv_bridge *h, int fused, int profile, int needs_backward_grad);
