@@ -823,9 +823,10 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
   pl->waves = best_w;
   // column blocks per tile: least padding of the column count, wider tile on ties
   const long ncols = (long)d * ks * ks;
+  // (narrow tiles re-read the dout slab for few MFMAs each: below 4 blocks only for small layers)
   int best_tb = 6;
   best = -1;
-  for (int tb = 6; tb >= 1; --tb) {
+  for (int tb = 6; tb >= (ncols > 128 ? 4 : 1); --tb) {
     const long padded = (ncols + 32 * tb - 1) / (32 * tb) * 32 * tb;
     if (best < 0 || padded < best) { best = padded; best_tb = tb; }
   }
