@@ -33,11 +33,15 @@ PEAK_HBM_GBS = 8000.0
 # under profiles/.  fetched + written, in bytes.
 # Keyed by (path level, stage).
 GEMM_TRAFFIC_BYTES = {
-    (1, "GEMM"): (1868.7 + 192.4) * 1e6,
-    (1, "GEMM Data"): (1450.5 + 1990.2) * 1e6,
-    (1, "GEMM Wghts"): (2143.1 + 63.9) * 1e6,
-    (2, "GEMM"): (1868.7 + 192.4) * 1e6,
-    (2, "GEMM Wghts"): (2143.1 + 63.9) * 1e6,
+    (1, "GEMM"): (1868.6 + 192.4) * 1e6,
+    (1, "GEMM Data"): (1137.0 + 1791.6) * 1e6,
+    (1, "GEMM Wghts"): (2143.4 + 63.9) * 1e6,
+    (2, "GEMM"): (1868.6 + 192.4) * 1e6,
+    (2, "GEMM Data"): (280.4 + 73.5) * 1e6,
+    (2, "GEMM Wghts"): (2143.4 + 63.9) * 1e6,
+    (3, "GEMM"): (136.1 + 249.1) * 1e6,
+    (3, "GEMM Data"): (280.4 + 73.5) * 1e6,
+    (3, "GEMM Wghts"): (359.6 + 41.8) * 1e6,
 }
 
 
@@ -281,7 +285,7 @@ def main():
     gemm_names = [g for g in ("GEMM", "GEMM Data", "GEMM Wghts") if g in stages]
     dom = max(gemm_names, key=lambda g: stages[g])
     kernel_of = {"GEMM": "gemm_kernel<256x128x16, A k-contig, B k-contig> (forward, conv epilogue)",
-                 "GEMM Data": "gemm_kernel<128x256x16, A m-contig, B n-contig> (data gradient)",
+                 "GEMM Data": "gemm_kernel<128x128x16, A m-contig, B n-contig> (data gradient)",
                  "GEMM Wghts": "gemm_kernel<256x128x16, A k-contig, B n-contig> split-K (weight gradient)"}
     if path >= 2 and need_dgrad:
         kernel_of["GEMM Data"] = "conv_direct_kernel (data gradient: remap + GEMM + lifting in one launch)"
