@@ -186,15 +186,21 @@ def test_bridge_falls_back_where_direct_does_not_apply():
     layer.close()
 
 
-CFG2 = (256, 96, 27, 5, 2, 256)
+# full-size layers of the CaffeNet iteration (batch 256): conv2 whole and one group of it, conv3,
+# one group of conv4; between them they run every compile-time specialised weight-gradient instance
+# (8, 4 and 6 wavefronts)
+FULL_SIZE = [(256, 96, 27, 5, 2, 256), (256, 48, 27, 5, 2, 128), (256, 256, 13, 3, 1, 384),
+             (256, 192, 13, 3, 1, 192), (255, 192, 13, 3, 1, 128)]
 
 
-def test_full_size_direct_vs_float64():
-    """BASELINE config 2 at full size: the three direct kernels against torch's float64
-    convolution and its gradients (independent of this library and of the oracle)."""
+@pytest.mark.parametrize("cfg", FULL_SIZE, ids=_ids)
+def test_full_size_direct_vs_float64(cfg):
+    """Full-size layers (BASELINE config 2 first; the last one with an odd batch): the three direct
+    kernels against torch's float64 convolution and its gradients (independent of this library
+    and of the oracle)."""
     import torch
     import torch.nn.functional as F
-    b, d, n, k, p, o = CFG2
+    b, d, n, k, p, o = cfg
     m = n + 2 * p - k + 1
     drv = driver()
     g = torch.Generator(device="cuda").manual_seed(1235)
