@@ -742,8 +742,11 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
       // this pair's share of the next step's loads
       constexpr int A0 = 0;
       (void)A0;
-      const int a_lo = q * NAW / NQ, a_hi = (q + 1) * NAW / NQ;
-      const int b_lo = q * NBW / NQ, b_hi = (q + 1) * NBW / NQ;
+      // (all of them within the first NQI pairs, so that the last ones have landed by the barrier)
+      constexpr int NQI = (NQ * 5 + 7) / 8;
+      const int qi = q < NQI ? q : NQI, qj = q + 1 < NQI ? q + 1 : NQI;
+      const int a_lo = qi * NAW / NQI, a_hi = qj * NAW / NQI;
+      const int b_lo = qi * NBW / NQI, b_hi = qj * NBW / NQI;
 #pragma unroll
       for (int k = 0; k < NAW; ++k)
         if (k >= a_lo && k < a_hi) CCT_WSPEC_A(k, nxt);
