@@ -157,6 +157,7 @@ __global__ __launch_bounds__(TPB) void maxpool_fwd_kernel(float *__restrict__ ou
 // backward as a gather: one lane per input element sums the output gradients whose argmax is this
 // element, scanning candidate windows in (ph, pw) ascending order = the order of the
 // reference's scatter loop, so sums with several contributors are bit-identical
+template <bool TWO_BY_TWO>
 __global__ __launch_bounds__(TPB) void maxpool_bwd_kernel(float *__restrict__ ig, const float *__restrict__ og,
                                                           const int *__restrict__ idx, cct_pool_args a,
                                                           uint32_t total, FastDiv div_ic, FastDiv div_ir) {
@@ -172,48 +173,60 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_kernel(float *__restrict__ ig
   const int me = h * a.iC + w;
   const size_t obase = (size_t)plane * a.oR * a.oC;
   float acc = 0.0f;
-  for (int ph = ph_lo; ph <= ph_hi; ++ph)
-    for (int pw = pw_lo; pw <= pw_hi; ++pw) {
-      const size_t o = obase + ph * a.oC + pw;
-      if (idx[o] == me) acc += og[o];
-    }
+  if (TWO_BY_TWO) {
+    // kernel <= 2*stride: an element lies in at most two windows per direction.  All candidates are
+    // fetched at once (clamped positions, so the loads need no branches) and added in (ph, pw) order.
+    int cidx[2][2];
+    float cog[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const size_t o = obase + min(ph_lo + i, a.oR - 1) * a.oC + min(pw_lo + j, a.oC - 1);
+        cidx[i][j] = idx[o];
+        cog[i][j] = og[o];
+      }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        if (ph_lo + i <= ph_hi && pw_lo + j <= pw_hi && cidx[i][j] == me) acc += cog[i][j];
+  } else {
+    for (int ph = ph_lo; ph <= ph_hi; ++ph)
+      for (int pw = pw_lo; pw <= pw_hi; ++pw) {
+        const size_t o = obase + ph * a.oC + pw;
+        if (idx[o] == me) acc += og[o];
+      }
+  }
   ig[e] = acc;
 }
 
 // ---- LRN (across channels) -----------------------------------------------------------------------
-// forward: one lane per (image, pixel) walks the depth with the running window of
-// _f_lrn_forward (copy previous, subtract leaving square, add entering square), then applies
-// scale = 1 + alpha/size * sum and out = in / scale^beta.  denoms keeps scale.
+// forward: one lane per element sums the squares of its window [ch-w, ch+w] (clipped to the depth)
+// in ascending channel order, then scale = 1 + alpha/size * sum and out = in / scale^beta; denoms
+// keeps scale.  _f_lrn_forward carries a running window sum along the depth (src/kernels/lrn.hxx:
+// 46-100); summing each window afresh differs from it by rounding only (a few ulp of the sum).
 __global__ __launch_bounds__(TPB) void lrn_fwd_kernel(float *__restrict__ out, float *__restrict__ denoms,
                                                       const float *__restrict__ in, int rc, int D,
                                                       uint32_t total, int w, float aos, float beta,
-                                                      FastDiv div_rc) {
+                                                      FastDiv div_rc, FastDiv div_d) {
   const uint32_t e = blockIdx.x * TPB + threadIdx.x;
   if (e >= total) return;
-  const uint32_t ib = fdiv(e, div_rc);
-  const uint32_t q = e - ib * rc;
-  const size_t base = (size_t)ib * D * rc + q;
-  float sum = 0.0f;
-  for (int i = 0; i <= w; ++i)
-    if (i < D) {
-      const float x = in[base + (size_t)i * rc];
-      sum += x * x;
-    }
-  for (int d = 0; d < D; ++d) {
-    if (d > 0) {
-      if (d - w - 1 >= 0) {
-        const float x = in[base + (size_t)(d - w - 1) * rc];
-        sum -= x * x;
-      }
-      if (d + w < D) {
-        const float x = in[base + (size_t)(d + w) * rc];
-        sum += x * x;
-      }
-    }
-    const float scale = aos * sum + 1.0f;
-    denoms[base + (size_t)d * rc] = scale;
-    out[base + (size_t)d * rc] = in[base + (size_t)d * rc] / powf(scale, beta);
+  // e = (ib*D + ch)*rc + q
+  const uint32_t t1 = fdiv(e, div_rc);
+  const uint32_t ib = fdiv(t1, div_d);
+  const int ch = t1 - ib * D;
+  const int lo = max(0, ch - w), hi = min(D - 1, ch + w);
+  const float *p = in + (size_t)e + (ptrdiff_t)(lo - ch) * rc;
+  float sum = 0.0f, xv = 0.0f;
+  for (int c = lo; c <= hi; ++c, p += rc) {
+    const float x = *p;
+    sum += x * x;
+    if (c == ch) xv = x;
   }
+  const float scale = aos * sum + 1.0f;
+  denoms[e] = scale;
+  out[e] = xv / powf(scale, beta);
 }
 
 // backward as a gather over the window: in_grad[ch] = sum over od in [ch-w, ch+w] (ascending, the
@@ -245,6 +258,62 @@ __global__ __launch_bounds__(TPB) void lrn_bwd_kernel(float *__restrict__ ig, co
     acc += gv * og[o];
   }
   ig[e] = acc;
+}
+
+// The same gather with one lane per (image, pixel, run of CH channels): the per-channel terms of
+// the window (scale^beta, the factor g2, x and out_grad) are computed once per lane and reused by
+// the up to 2*WN+1 output channels that touch them, instead of once per (channel, window slot).
+// Every product and sum is the one lrn_bwd_kernel forms, in the same order: identical results.
+template <int WN, int CH>
+__global__ __launch_bounds__(TPB) void lrn_bwd_run_kernel(float *__restrict__ ig, const float *__restrict__ og,
+                                                          const float *__restrict__ x,
+                                                          const float *__restrict__ den, int rc, int D,
+                                                          uint32_t total, int nruns, float aos, float beta,
+                                                          FastDiv div_rc, FastDiv div_runs) {
+  const uint32_t e = blockIdx.x * TPB + threadIdx.x;
+  if (e >= total) return;
+  // e = (ib*nruns + run)*rc + q
+  const uint32_t t1 = fdiv(e, div_rc);
+  const uint32_t q = e - t1 * rc;
+  const uint32_t ib = fdiv(t1, div_runs);
+  const int c0 = (int)(t1 - ib * nruns) * CH;
+  const size_t base = (size_t)ib * D * rc + q;
+  constexpr int NW = CH + 2 * WN;
+  float denom[NW], g2[NW], xw[NW], ow[NW];
+#pragma unroll
+  for (int i = 0; i < NW; ++i) {
+    const int od = c0 - WN + i;
+    denom[i] = 1.0f; g2[i] = 0.0f; xw[i] = 0.0f; ow[i] = 0.0f;
+    if (od >= 0 && od < D) {
+      const size_t o = base + (size_t)od * rc;
+      const float dne = den[o];
+      const float dn = powf(dne, beta);
+      const float denom_n1 = (float)(1.0 / (double)(dn * dne));
+      const float wd = x[o];
+      denom[i] = dn;
+      g2[i] = beta * denom_n1 * aos * 2 * wd;
+      xw[i] = wd;
+      ow[i] = og[o];
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int ch = c0 + c;
+    if (ch >= D) break;
+    const float xv = xw[c + WN];
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j <= 2 * WN; ++j) {
+      const int od = ch - WN + j;
+      if (od < 0 || od >= D) continue;
+      const int i = c + j;
+      float gv;
+      if (j == WN) gv = (float)(1.0 / (double)denom[i] - (double)(g2[i] * xv));
+      else gv = -g2[i] * xv;
+      acc += gv * ow[i];
+    }
+    ig[base + (size_t)ch * rc] = acc;
+  }
 }
 
 // ---- dropout -------------------------------------------------------------------------------------
@@ -521,8 +590,12 @@ int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_po
   if (rc) return rc;
   const size_t total = (size_t)a->D * a->B * a->iR * a->iC;
   if (total == 0) return 0;
-  hipLaunchKernelGGL(maxpool_bwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad,
-                     out_grad, a->max_index, *a, (uint32_t)total, make_fastdiv(a->iC), make_fastdiv(a->iR));
+  if (a->kernel_size <= 2 * a->stride)
+    hipLaunchKernelGGL(maxpool_bwd_kernel<true>, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad,
+                       out_grad, a->max_index, *a, (uint32_t)total, make_fastdiv(a->iC), make_fastdiv(a->iR));
+  else
+    hipLaunchKernelGGL(maxpool_bwd_kernel<false>, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad,
+                       out_grad, a->max_index, *a, (uint32_t)total, make_fastdiv(a->iC), make_fastdiv(a->iR));
   CCT_LAUNCH_CHECK();
   return 0;
 }
@@ -532,12 +605,12 @@ int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args 
   CCT_ENSURE_INIT();
   CCT_REQUIRE(out && in && a && a2 && a->denoms, "lrn_forward: null argument");
   CCT_REQUIRE(a->iR > 0 && a->iC > 0 && a->iD > 0 && a->iB >= 0 && a->norm_window >= 0, "lrn_forward: bad sizes");
-  const size_t total = (size_t)a->iB * a->iR * a->iC;
-  CCT_REQUIRE(total * a->iD < (1ull << 31), "lrn_forward: tensor too large");
+  const size_t total = (size_t)a->iB * a->iD * a->iR * a->iC;
+  CCT_REQUIRE(total < (1ull << 31), "lrn_forward: tensor too large");
   if (total == 0) return 0;
   hipLaunchKernelGGL(lrn_fwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, out,
                      (float *)a->denoms, in, a->iR * a->iC, a->iD, (uint32_t)total, a->norm_window,
-                     a2->alpha_over_size, a2->beta, make_fastdiv(a->iR * a->iC));
+                     a2->alpha_over_size, a2->beta, make_fastdiv(a->iR * a->iC), make_fastdiv(a->iD));
   CCT_LAUNCH_CHECK();
   return 0;
 }
@@ -549,6 +622,17 @@ int cct_hip_lrn_backward(float *in_grad, const float *out_grad, const cct_lrn_ba
   const size_t total = (size_t)a->oB * a->oD * a->oR * a->oC;
   CCT_REQUIRE(total < (1ull << 31), "lrn_backward: tensor too large");
   if (total == 0) return 0;
+  if (a->norm_window == 2) {
+    constexpr int CH = 8;
+    const int nruns = (a->oD + CH - 1) / CH;
+    const size_t lanes = (size_t)a->oB * nruns * a->oR * a->oC;
+    hipLaunchKernelGGL((lrn_bwd_run_kernel<2, CH>), dim3(blocks_for(lanes)), dim3(TPB), 0, ctx().stream, in_grad,
+                       out_grad, (const float *)a->input_data, (const float *)a->denoms, a->oR * a->oC, a->oD,
+                       (uint32_t)lanes, nruns, a->alpha_over_size, a->beta, make_fastdiv(a->oR * a->oC),
+                       make_fastdiv(nruns));
+    CCT_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL(lrn_bwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad, out_grad,
                      (const float *)a->input_data, (const float *)a->denoms, a->oR * a->oC, a->oD,
                      (uint32_t)total, a->norm_window, a->alpha_over_size, a->beta,
