@@ -27,6 +27,8 @@ namespace cct {
 typedef float v16f __attribute__((ext_vector_type(16)));
 // native 4-float vector: stays in registers where HIP's f4 struct (a union) can end up in scratch
 typedef float f4 __attribute__((ext_vector_type(4)));
+// the same vector where only dword alignment may be assumed (global memory operands)
+typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
 
 enum EpilogueMode { EPI_ALPHA_BETA = 0, EPI_SPLITK_PARTIAL = 1, EPI_CONV_FORWARD = 2 };
 
@@ -57,7 +59,7 @@ __device__ __forceinline__ f4 ldg4(const float *__restrict__ base, int major, in
   if (major < major_lim) {
     const float *p = base + (size_t)major * ld + minor;
     if (vec && minor + 3 < minor_lim) {
-      v = *reinterpret_cast<const f4 *>(p);
+      v = *reinterpret_cast<const f4u *>(p);
     } else {
       if (minor + 0 < minor_lim) v.x = p[0];
       if (minor + 1 < minor_lim) v.y = p[1];
@@ -168,9 +170,11 @@ __device__ __forceinline__ void mfma_group(v16f (&acc)[TM][TN], const f4 (&fa)[T
 
 // Loader for whole K steps: no bounds tests.  Rows (and columns) that fall outside the matrix are
 // clamped to the last valid one -- they only feed accumulators that the epilogue never stores --
-// so every tile, edge tiles included, streams its operands with straight-line loads.  `vec`
-// selects one aligned 16-byte load per f4; otherwise four dword loads (unaligned leading
-// dimension or base, e.g. k*k*d = 363).
+// so every tile, edge tiles included, streams its operands with straight-line loads.  An f4 that
+// lies wholly inside its row is fetched with one 16-byte load whatever its alignment (global
+// loads only need dword alignment, so leading dimensions like k*k*d = 363 cost nothing extra);
+// `vec` = 0 forces four dword loads.  The last f4 of a row-contiguous operand whose row count is
+// not a multiple of 4 is assembled from clamped dword loads.
 template <class T, bool KC, int ROWS>
 struct FastLoader {
   static constexpr int NV = OperandLayout<T, KC, ROWS>::NV;
@@ -187,8 +191,7 @@ struct FastLoader {
         lim[i] = 3;
       } else {
         const int kk = f / (ROWS / 4), rq = f % (ROWS / 4);
-        // an f4 starting past the end moves back to the last one that fits (16-byte mode needs
-        // rows_total % 4 == 0, which the host guarantees before choosing it)
+        // an f4 starting past the end moves back to the last one that fits
         int start = row0 + rq * 4;
         lim[i] = min(3, rows_total - 1 - start);
         if (lim[i] < 0) {
@@ -203,8 +206,8 @@ struct FastLoader {
   __device__ __forceinline__ void load(f4 *__restrict__ r, int vec) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      if (vec) {
-        r[i] = *reinterpret_cast<const f4 *>(p[i]);
+      if (vec && (KC || lim[i] == 3)) {
+        r[i] = *reinterpret_cast<const f4u *>(p[i]);
       } else if (KC) {
         r[i] = f4{p[i][0], p[i][1], p[i][2], p[i][3]};
       } else {
@@ -295,10 +298,11 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs &g, float *smem, v1
 #undef CCT_FRAGS
 }
 
-// Epilogue of a tile that lies wholly inside C and reads nothing back: per lane one row pointer
-// advancing by a row stride and TN fixed column offsets, no bounds tests.  row0/col0 are the
-// lane's first row and column.
-template <class T, int MODE>
+// Epilogue of a tile whose columns lie wholly inside C and that reads nothing back: per lane one
+// row pointer advancing by a row stride and TN fixed column offsets.  ROWGUARD = false: the rows
+// lie inside C too, no bounds tests at all; true: rows past M are skipped (M not a multiple of the
+// tile height, e.g. 96 output maps).  row0/col0 are the lane's first row and column.
+template <class T, int MODE, bool ROWGUARD>
 __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&acc)[T::TM][T::TN], int row0,
                                               int col0, uint32_t kslice) {
   if (MODE == EPI_CONV_FORWARD) {
@@ -316,6 +320,7 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int row = row0 + a * 32 + 8 * j + i;
+          if (ROWGUARD && row >= g.M) continue;
           float *c = g.C + (size_t)row * g.fmap;
           const float add = g.bias ? g.bias[row] : 0.0f;
 #pragma unroll
@@ -332,6 +337,7 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
+          if (ROWGUARD && row0 + a * 32 + 8 * j + i >= g.M) continue;
           float *c = crow + (size_t)(a * 32 + 8 * j + i) * rstride;
 #pragma unroll
           for (int b = 0; b < T::TN; ++b)
@@ -376,17 +382,21 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
   gemm_mainloop<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
-  const bool interior = (m0 + T::BM <= g.M) && (n0 + T::BN <= g.N);
+  const bool rows_inside = m0 + T::BM <= g.M, cols_inside = n0 + T::BN <= g.N;
 
   // epilogue: accumulator register v of lane (r,h) is C[8*(v/4) + 4*h + v%4][r] of its 32x32 tile
   const int r = lane & 31, h = lane >> 5;
-  if (interior && !(g.epi == EPI_ALPHA_BETA && g.beta != 0.0f)) {
-    if (g.epi == EPI_ALPHA_BETA)
-      fast_epilogue<T, EPI_ALPHA_BETA>(g, acc, m0 + wm0 + 4 * h, n0 + wn0 + r, kslice);
-    else if (g.epi == EPI_SPLITK_PARTIAL)
-      fast_epilogue<T, EPI_SPLITK_PARTIAL>(g, acc, m0 + wm0 + 4 * h, n0 + wn0 + r, kslice);
-    else
-      fast_epilogue<T, EPI_CONV_FORWARD>(g, acc, m0 + wm0 + 4 * h, n0 + wn0 + r, kslice);
+  if (cols_inside && !(g.epi == EPI_ALPHA_BETA && g.beta != 0.0f)) {
+    const int er = m0 + wm0 + 4 * h, ec = n0 + wn0 + r;
+    if (rows_inside) {
+      if (g.epi == EPI_ALPHA_BETA) fast_epilogue<T, EPI_ALPHA_BETA, false>(g, acc, er, ec, kslice);
+      else if (g.epi == EPI_SPLITK_PARTIAL) fast_epilogue<T, EPI_SPLITK_PARTIAL, false>(g, acc, er, ec, kslice);
+      else fast_epilogue<T, EPI_CONV_FORWARD, false>(g, acc, er, ec, kslice);
+    } else {
+      if (g.epi == EPI_ALPHA_BETA) fast_epilogue<T, EPI_ALPHA_BETA, true>(g, acc, er, ec, kslice);
+      else if (g.epi == EPI_SPLITK_PARTIAL) fast_epilogue<T, EPI_SPLITK_PARTIAL, true>(g, acc, er, ec, kslice);
+      else fast_epilogue<T, EPI_CONV_FORWARD, true>(g, acc, er, ec, kslice);
+    }
     return;
   }
 #pragma unroll
@@ -474,10 +484,9 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
   g.alpha = alpha; g.beta = beta; g.epi = epi; g.fmap = fmap > 0 ? fmap : 1;
   g.div_fmap = make_fastdiv((uint32_t)g.fmap); g.bias = bias; g.ws = nullptr;
-  // 16-byte loads need an aligned base and leading dimension; a row-contiguous operand also
-  // needs its row count to be a multiple of 4 so that the clamped last f4 stays aligned
-  g.a_vec = ((uintptr_t)A % 16 == 0) && (lda % 4 == 0) && (a_kc || M % 4 == 0);
-  g.b_vec = ((uintptr_t)B % 16 == 0) && (ldb % 4 == 0) && (b_kc || N % 4 == 0);
+  // 16-byte global loads need dword alignment only
+  g.a_vec = ((uintptr_t)A % 4 == 0);
+  g.b_vec = ((uintptr_t)B % 4 == 0);
   {
     const char *e = getenv("CCT_HIP_GEMM_NT");
     g.nt_store = e ? atoi(e) : 0;
