@@ -397,6 +397,7 @@ struct WgradArgs {
   const float *dout;   // [batch][o][ho][ho]
   const float *src;    // [batch][d][hs][hs]
   float *out;          // [splits][o][ncols]
+  float *out_bias;     // [splits][o] bias-gradient partial sums, or null
   int batch, o, d, hs, ho, pad;
   int ncols;           // d * KS * KS
   int ast;             // floats between rows of the staged dout slab (odd)
@@ -520,6 +521,8 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
   for (int b = 0; b < TB; ++b)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+  // bias gradient: lane (r, h) adds up dout[map r][image h of every pair][every row][every x]
+  float bsum = 0.0f;
 
   if (s_beg < s_end) {
     CCT_WGRAD_ISSUE(s_beg, 0);
@@ -548,6 +551,7 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
   } while (0)
 #define CCT_WGRAD_MFMA(buf, e)                                                                    \
   do {                                                                                            \
+    bsum += fa[buf][e]; /* the dout fragment is also this lane's bias-gradient addend */         \
     _Pragma("unroll") for (int b = 0; b < TB; ++b)                                                \
         acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[buf][e], fb[buf][e][b], acc[b], 0, 0, 0); \
   } while (0)
@@ -588,6 +592,12 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
   }
 #undef CCT_WGRAD_ISSUE
 
+  if (g.out_bias && tn == 0) {
+    // the two images of the pairs sit in the two lane halves; only the first column tile reports
+    const float both = bsum + __shfl_xor(bsum, 32);
+    const int row = m0 + wave * 32 + r;
+    if (h == 0 && row < g.o) g.out_bias[(size_t)z * g.o + row] = both;
+  }
   float *out = g.out + (size_t)z * g.o * g.ncols;
 #pragma unroll
   for (int b = 0; b < TB; ++b) {
@@ -678,6 +688,8 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   for (int b = 0; b < TB; ++b)
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+  // bias gradient: lane (r, h) adds up dout[map r][image h of every pair][every row][every x]
+  float bsum = 0.0f;
 
 // per-step scalars of step s
 #define CCT_WSPEC_STEP(s)                                                                         \
@@ -734,6 +746,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
         if (2 * q + e < HO) {
+          bsum += fa[cb][e];  // the dout fragment is also this lane's bias-gradient addend
 #pragma unroll
           for (int b = 0; b < TB; ++b)
             acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][e], fb[cb][e][b], acc[b], 0, 0, 0);
@@ -776,6 +789,12 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
 #undef CCT_WSPEC_A
 #undef CCT_WSPEC_B
 
+  if (g.out_bias && tn == 0) {
+    // the two images of the pairs sit in the two lane halves; only the first column tile reports
+    const float both = bsum + __shfl_xor(bsum, 32);
+    const int row = m0 + wave * 32 + r;
+    if (h == 0 && row < g.o) g.out_bias[(size_t)z * g.o + row] = both;
+  }
   float *out = g.out + (size_t)z * g.o * g.ncols;
 #pragma unroll
   for (int b = 0; b < TB; ++b) {
@@ -789,11 +808,16 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   }
 }
 
-// dst[e] = sum_z ws[z][e], z ascending
+// dst[e] = sum_z ws[z][e] for e < n, and dst2[e - n] = sum_z ws2[z][e - n] for n <= e < n + n2;
+// z ascending
 __global__ __launch_bounds__(256) void direct_reduce_kernel(float *__restrict__ dst, const float *__restrict__ ws,
-                                                            uint32_t n, int splits) {
-  const uint32_t e = blockIdx.x * 256 + threadIdx.x;
-  if (e >= n) return;
+                                                            uint32_t n, float *__restrict__ dst2,
+                                                            const float *__restrict__ ws2, uint32_t n2, int splits) {
+  uint32_t e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= n + n2) return;
+  if (e >= n) {
+    e -= n; dst = dst2; ws = ws2; n = n2;
+  }
   float s = 0.f;
   for (int z = 0; z < splits; ++z) s += ws[(size_t)z * n + e];
   dst[e] = s;
@@ -894,8 +918,8 @@ static int wgrad_launch(const WgradArgs &g, const WgradPlan &pl, hipStream_t st)
   return set_error(CCT_HIP_EINVAL, "conv_direct wgrad: no kernel instance for %d column blocks", pl.tb);
 }
 
-static int conv_direct_wgrad(float *dw, const float *dout, const float *src, int batch, int d, int n, int ks,
-                             int pad, int o) {
+static int conv_direct_wgrad(float *dw, float *db, const float *dout, const float *src, int batch, int d, int n,
+                             int ks, int pad, int o) {
   WgradPlan pl;
   CCT_REQUIRE(wgrad_plan(batch, d, n, ks, pad, o, &pl),
               "conv_direct wgrad: geometry not covered (k=%d pad=%d size=%d)", ks, pad, n);
@@ -925,11 +949,13 @@ static int conv_direct_wgrad(float *dw, const float *dout, const float *src, int
   const size_t n_out = (size_t)o * g.ncols;
   if (splits > 1) {
     void *ws = nullptr;
-    int rc = get_workspace((size_t)splits * n_out * sizeof(float), &ws);
+    int rc = get_workspace((size_t)splits * (n_out + (db ? o : 0)) * sizeof(float), &ws);
     if (rc) return rc;
     g.out = (float *)ws;
+    g.out_bias = db ? g.out + (size_t)splits * n_out : nullptr;
   } else {
     g.out = dw;
+    g.out_bias = db;
   }
   hipStream_t st = ctx().stream;
   int rc;
@@ -943,8 +969,9 @@ static int conv_direct_wgrad(float *dw, const float *dout, const float *src, int
   else rc = pl.pw == 16 ? wgrad_launch<3, 16>(g, pl, st) : wgrad_launch<3, 32>(g, pl, st);
   if (rc) return rc;
   if (splits > 1) {
-    hipLaunchKernelGGL(direct_reduce_kernel, dim3((uint32_t)((n_out + 255) / 256)), dim3(256), 0, st, dw, g.out,
-                       (uint32_t)n_out, splits);
+    const uint32_t n2 = db ? (uint32_t)o : 0u;
+    hipLaunchKernelGGL(direct_reduce_kernel, dim3((uint32_t)((n_out + n2 + 255) / 256)), dim3(256), 0, st, dw,
+                       g.out, (uint32_t)n_out, db, g.out_bias, n2, splits);
     CCT_LAUNCH_CHECK();
   }
   return 0;
@@ -1010,10 +1037,10 @@ extern "C" int cct_hip_conv_direct_backward_data(float *input_grad, const float 
                      k - 1 - padding);
 }
 
-extern "C" int cct_hip_conv_direct_backward_weights(float *model_grad, const float *output_grad,
+extern "C" int cct_hip_conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                                     const float *input, int batch, int depth, int n, int k,
                                                     int padding, int num_outputs) {
   CCT_ENSURE_INIT();
   CCT_REQUIRE(batch > 0, "conv_direct_backward_weights: empty batch");
-  return conv_direct_wgrad(model_grad, output_grad, input, batch, depth, n, k, padding, num_outputs);
+  return conv_direct_wgrad(model_grad, bias_grad, output_grad, input, batch, depth, n, k, padding, num_outputs);
 }

@@ -230,7 +230,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     const bool direct_weights = path_ == PATH_DIRECT_ALL;
 
     const bool fuse_bias_into_lift = bias_term && needs_to_calc_backward_grad && path_ == PATH_FUSED;
-    if (bias_term && !fuse_bias_into_lift) {
+    // on the all-direct path the weight-gradient kernel reduces the bias gradient as well
+    if (bias_term && !fuse_bias_into_lift && !direct_weights) {
       begin(STAGE_BW_BIAS);
       DeviceMemoryPointer bias = p_bias_gradient_cube->get_device_pointer(p_driver);
       p_driver->backward_bias(&bias, &og, (int)(oR * oC), (int)oD, (int)iB);
@@ -254,9 +255,11 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     // GEMM has drained from the caches.
     begin(STAGE_GEMM_WEIGHTS);
     if (direct_weights) {
-      p_driver->conv_direct_backward_weights(p_model_gradient_cube->get_p_data(), output_g_cube->get_p_data(),
-                                             p_input_layer->p_data_cube->get_p_data(), (int)iB, (int)iD, (int)iR,
-                                             (int)K, (int)padding, (int)num_output_features);
+      p_driver->conv_direct_backward_weights(p_model_gradient_cube->get_p_data(),
+                                             bias_term ? p_bias_gradient_cube->get_p_data() : nullptr,
+                                             output_g_cube->get_p_data(), p_input_layer->p_data_cube->get_p_data(),
+                                             (int)iB, (int)iD, (int)iR, (int)K, (int)padding,
+                                             (int)num_output_features);
     } else {
       p_backward_gemm_updateweight_kernel->alpha = 1.0;
       p_backward_gemm_updateweight_kernel->beta = 0.0;

@@ -194,9 +194,10 @@ class HIPDriver {
                                          num_outputs),
        "conv_direct_backward_data");
   }
-  void conv_direct_backward_weights(float *model_grad, const float *output_grad, const float *input, int batch,
-                                    int depth, int n, int k, int padding, int num_outputs) {
-    ok(cct_hip_conv_direct_backward_weights(model_grad, output_grad, input, batch, depth, n, k, padding,
+  void conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
+                                    const float *input, int batch, int depth, int n, int k, int padding,
+                                    int num_outputs) {
+    ok(cct_hip_conv_direct_backward_weights(model_grad, bias_grad, output_grad, input, batch, depth, n, k, padding,
                                             num_outputs),
        "conv_direct_backward_weights");
   }

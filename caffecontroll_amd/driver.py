@@ -131,8 +131,8 @@ class HIPDriver:
         check(self.lib.cct_hip_conv_direct_backward_data(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o),
               "conv_direct_backward_data")
 
-    def conv_direct_backward_weights(self, dw, dout, inp, b, d, n, k, p, o):
-        check(self.lib.cct_hip_conv_direct_backward_weights(_p(dw), _p(dout), _p(inp), b, d, n, k, p, o),
+    def conv_direct_backward_weights(self, dw, dout, inp, b, d, n, k, p, o, db=None):
+        check(self.lib.cct_hip_conv_direct_backward_weights(_p(dw), _p(db), _p(dout), _p(inp), b, d, n, k, p, o),
               "conv_direct_backward_weights")
 
     def sgemv(self, TA, M, N, alpha, A, x, beta, y):

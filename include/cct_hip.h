@@ -183,9 +183,12 @@ int cct_hip_conv_direct_backward_data(float *input_grad, const float *output_gra
                                       int batch, int depth, int n, int k, int padding, int num_outputs);
 /* Weight-gradient GEMM of ConvolutionBridge::backward (src/bridges/ConvolutionBridge_impl.hxx:
  * 619-621) without the lowered matrix or the gradient remap: model_grad[o][d][k][k] (overwritten,
- * beta = 0) from output_grad[b][o][m][m] and input[b][d][n][n]. */
-int cct_hip_conv_direct_backward_weights(float *model_grad, const float *output_grad, const float *input,
-                                         int batch, int depth, int n, int k, int padding, int num_outputs);
+ * beta = 0) from output_grad[b][o][m][m] and input[b][d][n][n].  If bias_grad is not NULL the same
+ * launch also produces the bias gradient bias_grad[o] = sum of output_grad over batch and pixels
+ * (:575-599), in a fixed summation order. */
+int cct_hip_conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
+                                         const float *input, int batch, int depth, int n, int k, int padding,
+                                         int num_outputs);
 /* DeviceDriver::sgemv (src/sched/DeviceDriver.h:214-215): row-major M x N, lda = N. */
 int cct_hip_sgemv(int TA, int M, int N, float alpha, const float *A, const float *x, float beta,
                   float *y);

@@ -86,13 +86,20 @@ def test_direct_kernels_match_oracle(oracle, shape):
     assert rel_err(host(dx), ref_dx) <= TOL
     np.testing.assert_array_equal(host(d_og), og)  # the output gradient is read in place, not permuted
 
-    dw = empty((o, d, k, k))
-    drv.conv_direct_backward_weights(dw, d_og, d_x, b, d, n, k, p, o)
+    dw, db = empty((o, d, k, k)), empty((o,))
+    drv.conv_direct_backward_weights(dw, d_og, d_x, b, d, n, k, p, o, db=db)
     assert rel_err(host(dw), ref_dw) <= TOL
-    # split-K partial sums are added in a fixed order: a second run gives the same bits
+    # the same launch reduces the bias gradient; both the oracle's order and float64 must agree
+    assert rel_err(host(db), ref_db) <= TOL
+    assert rel_err(host(db), og.astype(np.float64).sum(axis=(0, 2, 3))) <= TOL
+    # split-K partial sums are added in a fixed order: a second run gives the same bits, with or
+    # without the bias gradient
     dw2 = empty((o, d, k, k))
     drv.conv_direct_backward_weights(dw2, d_og, d_x, b, d, n, k, p, o)
     np.testing.assert_array_equal(host(dw2), host(dw))
+    db2 = empty((o,))
+    drv.conv_direct_backward_weights(dw2, d_og, d_x, b, d, n, k, p, o, db=db2)
+    np.testing.assert_array_equal(host(db2), host(db))
 
 
 def test_direct_exact_on_small_integers(oracle):
@@ -212,8 +219,11 @@ def test_full_size_direct_vs_float64(cfg):
     out, dx, dw = empty((b, o, m, m)), empty((b, d, n, n)), empty((o, d, k, k))
     drv.conv_direct_forward(out, x, sf, bias, b, d, n, k, p, o)
     drv.conv_direct_backward_data(dx, og, sb, b, d, n, k, p, o)
-    drv.conv_direct_backward_weights(dw, og, x, b, d, n, k, p, o)
+    db = empty((o,))
+    drv.conv_direct_backward_weights(dw, og, x, b, d, n, k, p, o, db=db)
     torch.cuda.synchronize()
+    db_ref = og.double().sum(dim=(0, 2, 3))
+    assert ((db.double() - db_ref).abs().max() / db_ref.abs().max()).item() <= TOL
 
     def err(got, ref):
         return ((got.double() - ref).abs().max() / ref.abs().max()).item()
