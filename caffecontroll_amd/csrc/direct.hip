@@ -46,6 +46,7 @@ struct DirectArgs {
   int pr;             // patch rows per channel
   int nsteps;         // ceil(kc / channels per step)
   int slab_stride;    // floats between channels of the slab buffer (padded map count * KS*KS)
+  uint32_t src_img_stride, dst_img_stride;  // floats between images (>= kc*hs*hs, mtot*ho*ho: channel-slice views)
   uint32_t ptot;      // batch * ho * ho
   uint32_t tiles_m, ntiles;
   FastDiv div_ho, div_ho2, div_hp, div_pr;
@@ -143,7 +144,7 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     const int srow = (int)(v - img * g.hp) - g.pad, scol = (int)pc - g.pad;
     const bool ok = c < (uint32_t)NC && img < (uint32_t)g.batch && (unsigned)srow < (unsigned)g.hs &&
                     (unsigned)scol < (unsigned)g.hs;
-    psrc[i] = ok ? (((img * g.kc + c) * g.hs + srow) * g.hs + scol) * 4u : kOutOfRange;
+    psrc[i] = ok ? (img * g.src_img_stride + (c * g.hs + srow) * g.hs + scol) * 4u : kOutOfRange;
     psrc_last[i] = (ok && (int)c < last_channels) ? psrc[i] : kOutOfRange;
   }
   const uint32_t a_step = (uint32_t)NC * g.slab_stride * 4u, b_step = (uint32_t)NC * g.hs * g.hs * 4u;  // bytes
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     const uint32_t p = p0 + wave * (32 * TNB) + b * 32 + r;
     if (p >= g.ptot) continue;
     const uint32_t img = fdiv(p, g.div_ho2);
-    float *out = g.dst + (size_t)img * g.mtot * ho2 + (p - img * ho2);
+    float *out = g.dst + (size_t)img * g.dst_img_stride + (p - img * ho2);
 #pragma unroll
     for (int a = 0; a < TMB; ++a)
 #pragma unroll
@@ -345,7 +346,7 @@ static int direct_launch_ks(const DirectArgs &g, const DirectPlan &pl, hipStream
 }
 
 static int conv_direct(const float *wt, const float *src, float *dst, const float *bias, int batch, int kc,
-                       int mtot, int hs, int ks, int pad) {
+                       int mtot, int hs, int ks, int pad, size_t src_img_stride, size_t dst_img_stride) {
   DirectPlan pl;
   CCT_REQUIRE(direct_plan(batch, kc, mtot, hs, ks, pad, &pl),
               "conv_direct: geometry not covered (k=%d pad=%d size=%d)", ks, pad, hs);
@@ -353,6 +354,16 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
   g.wt = wt; g.src = src; g.dst = dst; g.bias = bias;
   g.batch = batch; g.kc = kc; g.mtot = mtot; g.hs = hs; g.pad = pad;
   g.ho = hs + 2 * pad - ks + 1;
+  {
+    const size_t dense_src = (size_t)kc * hs * hs, dense_dst = (size_t)mtot * g.ho * g.ho;
+    if (!src_img_stride) src_img_stride = dense_src;
+    if (!dst_img_stride) dst_img_stride = dense_dst;
+    CCT_REQUIRE(src_img_stride >= dense_src && dst_img_stride >= dense_dst, "conv_direct: image stride smaller than an image");
+    CCT_REQUIRE((double)batch * src_img_stride < 1073741824.0 && (double)batch * dst_img_stride < 2147483648.0,
+                "conv_direct: strided tensor too large for 32-bit byte offsets");
+    g.src_img_stride = (uint32_t)src_img_stride;
+    g.dst_img_stride = (uint32_t)dst_img_stride;
+  }
   g.hp = g.ho + ks - 1;
   g.pr = pl.pr;
   g.nsteps = (kc + 2 * pl.cp - 1) / (2 * pl.cp);
@@ -405,6 +416,7 @@ struct WgradArgs {
   int a_floats;        // slab floats per stage, multiple of 64
   int stage;           // floats per LDS stage
   int steps_total, steps_per_split;  // a step = (image pair, output row)
+  uint32_t dout_img_stride, src_img_stride;  // floats between images (channel-slice views)
   uint32_t tiles_m, tiles_n, ntiles, nblocks;
   FastDiv div_ho, div_ast;
 };
@@ -452,7 +464,7 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
     if (i < (uint32_t)g.ho) {
       off += i;
     } else if (i < 2u * g.ho) {
-      off += (uint32_t)g.o * ho2 + (i - g.ho);
+      off += g.dout_img_stride + (i - g.ho);
       a_second |= 1u << k;
     }
     aoff[k] = off * 4u;  // bytes; pad words and words past the slab read word 0 of a valid row
@@ -470,7 +482,7 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
     const int scol = (int)pcol - g.pad;
     const bool ok = e < (uint32_t)(NCH * PCH) && prow < 2u * KS && ch0 + (int)ch < g.d &&
                     (unsigned)scol < (unsigned)g.hs;
-    boff[k] = ok ? ((second * (uint32_t)g.d + ch) * hs2 + kr * g.hs + (uint32_t)scol) * 4u : 0u;  // bytes
+    boff[k] = ok ? (second * g.src_img_stride + ch * hs2 + kr * g.hs + (uint32_t)scol) * 4u : 0u;  // bytes
     bmeta[k] = kr | (second << 4) | ((ok ? 1u : 0u) << 5);
   }
 
@@ -484,7 +496,7 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
     const int img0_ = 2 * (int)pair_;                                                             \
     const bool two_ = img0_ + 1 < g.batch;                                                        \
     float *sa_ = smem + (st) * g.stage;                                                           \
-    const uint32_t ga_ = (uint32_t)((((size_t)img0_ * g.o + m0) * ho2 + y_ * g.ho) * 4);          \
+    const uint32_t ga_ = (uint32_t)(((size_t)img0_ * g.dout_img_stride + m0 * ho2 + y_ * g.ho) * 4); \
     /* odd batch, last image alone: the second image's half reads zeros */                        \
     const uint32_t second_ = two_ ? 0u : a_second;                                                \
     _Pragma("unroll") for (int k = 0; k < NAL; ++k) {                                             \
@@ -493,7 +505,7 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
                  sa_ + (k * nwaves + wave) * 64);                                                 \
     }                                                                                             \
     float *sb_ = sa_ + g.a_floats;                                                                \
-    const uint32_t gb_ = (uint32_t)(((size_t)img0_ * g.d + ch0) * hs2 * 4);                       \
+    const uint32_t gb_ = (uint32_t)(((size_t)img0_ * g.src_img_stride + ch0 * hs2) * 4);          \
     /* first patch row may lie above the image: that (negative) term goes into the lane offset, */ \
     /* whose sum is non-negative for every lane that passes the row test                        */ \
     const uint32_t row0_ = (uint32_t)((y_ - g.pad) * g.hs * 4);                                   \
@@ -654,7 +666,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
     if (i < (uint32_t)HO) {
       off += i;
     } else if (i < 2u * HO) {
-      off += (uint32_t)g.o * ho2 + (i - HO);
+      off += g.dout_img_stride + (i - HO);
       a_second |= 1u << k;
     }
     aoff[k] = off * 4u;
@@ -669,7 +681,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
     const int scol = (int)pcol - g.pad;
     const bool ok = e < (uint32_t)(NCH * PCH) && prow < 2u * KS && ch0 + (int)ch < g.d &&
                     (unsigned)scol < (unsigned)g.hs;
-    boff[k] = ok ? ((second * (uint32_t)g.d + ch) * hs2 + kr * g.hs + (uint32_t)scol) * 4u : 0u;
+    boff[k] = ok ? (second * g.src_img_stride + ch * hs2 + kr * g.hs + (uint32_t)scol) * 4u : 0u;
     bmeta[k] = kr | (second << 4) | ((ok ? 1u : 0u) << 5);
   }
   const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
@@ -697,9 +709,9 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   const int y_ = (s) - (int)pair_ * HO;                                                           \
   const int img0_ = 2 * (int)pair_;                                                               \
   const bool two_ = img0_ + 1 < g.batch;                                                          \
-  const uint32_t ga_ = (uint32_t)((((size_t)img0_ * g.o + m0) * ho2 + y_ * HO) * 4);              \
+  const uint32_t ga_ = (uint32_t)(((size_t)img0_ * g.dout_img_stride + m0 * ho2 + y_ * HO) * 4);  \
   const uint32_t second_ = two_ ? 0u : a_second;                                                  \
-  const uint32_t gb_ = (uint32_t)(((size_t)img0_ * g.d + ch0) * hs2 * 4);                         \
+  const uint32_t gb_ = (uint32_t)(((size_t)img0_ * g.src_img_stride + ch0 * hs2) * 4);            \
   const uint32_t row0_ = (uint32_t)((y_ - g.pad) * g.hs * 4)
 #define CCT_WSPEC_A(k, st)                                                                        \
   lds_dma4(a_rsrc, ((second_ >> (k)) & 1u) ? kOutOfRange : aoff[k], ga_,                          \
@@ -919,7 +931,7 @@ static int wgrad_launch(const WgradArgs &g, const WgradPlan &pl, hipStream_t st)
 }
 
 static int conv_direct_wgrad(float *dw, float *db, const float *dout, const float *src, int batch, int d, int n,
-                             int ks, int pad, int o) {
+                             int ks, int pad, int o, size_t src_img_stride, size_t dout_img_stride) {
   WgradPlan pl;
   CCT_REQUIRE(wgrad_plan(batch, d, n, ks, pad, o, &pl),
               "conv_direct wgrad: geometry not covered (k=%d pad=%d size=%d)", ks, pad, n);
@@ -928,6 +940,17 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   g.batch = batch; g.o = o; g.d = d; g.hs = n; g.pad = pad;
   g.ho = n + 2 * pad - ks + 1;
   g.ncols = d * ks * ks;
+  {
+    const size_t dense_src = (size_t)d * n * n, dense_dout = (size_t)o * g.ho * g.ho;
+    if (!src_img_stride) src_img_stride = dense_src;
+    if (!dout_img_stride) dout_img_stride = dense_dout;
+    CCT_REQUIRE(src_img_stride >= dense_src && dout_img_stride >= dense_dout,
+                "conv_direct wgrad: image stride smaller than an image");
+    CCT_REQUIRE((double)batch * src_img_stride < 1073741824.0 && (double)batch * dout_img_stride < 1073741824.0,
+                "conv_direct wgrad: strided tensor too large for 32-bit byte offsets");
+    g.src_img_stride = (uint32_t)src_img_stride;
+    g.dout_img_stride = (uint32_t)dout_img_stride;
+  }
   g.ast = pl.ast; g.bm = 32 * pl.waves; g.a_floats = pl.a_floats; g.stage = pl.stage;
   g.steps_total = ((batch + 1) / 2) * g.ho;
   g.tiles_m = (uint32_t)((o + g.bm - 1) / g.bm);
@@ -1021,26 +1044,30 @@ extern "C" int cct_hip_conv_direct_slabs(float *slabs, const float *model, int n
 
 extern "C" int cct_hip_conv_direct_forward(float *output, const float *input, const float *slabs,
                                            const float *bias, int batch, int depth, int n, int k, int padding,
-                                           int num_outputs) {
+                                           int num_outputs, size_t input_image_stride, size_t output_image_stride) {
   CCT_ENSURE_INIT();
   if (batch <= 0) return 0;
-  return conv_direct(slabs, input, output, bias, batch, depth, num_outputs, n, k, padding);
+  return conv_direct(slabs, input, output, bias, batch, depth, num_outputs, n, k, padding, input_image_stride,
+                     output_image_stride);
 }
 
 extern "C" int cct_hip_conv_direct_backward_data(float *input_grad, const float *output_grad,
                                                  const float *slabs, int batch, int depth, int n, int k,
-                                                 int padding, int num_outputs) {
+                                                 int padding, int num_outputs, size_t input_image_stride,
+                                                 size_t output_image_stride) {
   CCT_ENSURE_INIT();
   if (batch <= 0) return 0;
   const int m = n + 2 * padding - k + 1;
   return conv_direct(slabs, output_grad, input_grad, nullptr, batch, num_outputs, depth, m, k,
-                     k - 1 - padding);
+                     k - 1 - padding, output_image_stride, input_image_stride);
 }
 
 extern "C" int cct_hip_conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                                     const float *input, int batch, int depth, int n, int k,
-                                                    int padding, int num_outputs) {
+                                                    int padding, int num_outputs, size_t input_image_stride,
+                                                    size_t output_image_stride) {
   CCT_ENSURE_INIT();
   CCT_REQUIRE(batch > 0, "conv_direct_backward_weights: empty batch");
-  return conv_direct_wgrad(model_grad, bias_grad, output_grad, input, batch, depth, n, k, padding, num_outputs);
+  return conv_direct_wgrad(model_grad, bias_grad, output_grad, input, batch, depth, n, k, padding, num_outputs,
+                           input_image_stride, output_image_stride);
 }

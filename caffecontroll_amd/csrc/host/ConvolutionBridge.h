@@ -36,6 +36,9 @@ enum ConvPath {
   PATH_DIRECT_ALL = 3    // forward, weight gradient and data gradient by direct kernels, no lowering
 };
 
+// GEMM size (FLOP) from which a layer takes the all-direct path by default.
+constexpr double kConvDirectMinFlop = 2e9;
+
 // Stage labels of the reference's detailed profiling output (_impl.hxx:325-366, 601-623).
 enum ConvStage {
   STAGE_LOWER = 0, STAGE_GEMM, STAGE_REMAP, STAGE_BIAS,            // forward
@@ -121,7 +124,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     // Small layers (LeNet-sized) stay on the fused lowering path by default: the direct kernels'
     // fixed costs (slab re-layout, partial-sum reduction) outweigh what they save below a few GFLOP.
     const double gemm_flop = 2.0 * num_output_features * (double)(oR * oC * iB) * (double)(K * K * iD);
-    default_path_ = (direct_ok_ && gemm_flop >= 2e9) ? PATH_DIRECT_ALL : PATH_FUSED;
+    default_path_ = (direct_ok_ && gemm_flop >= kConvDirectMinFlop) ? PATH_DIRECT_ALL : PATH_FUSED;
     path_ = default_path_;
     for (int i = 0; i < STAGE_COUNT; ++i) { timers_[i] = nullptr; stage_ms_[i] = 0.f; }
   }
@@ -156,9 +159,25 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     if (level < PATH_STAGED) level = PATH_STAGED;
     if (level > PATH_DIRECT_ALL) level = PATH_DIRECT_ALL;
     if (level >= PATH_DIRECT_DATA && !direct_ok_) level = PATH_FUSED;
+    if (views_) level = PATH_DIRECT_ALL;  // the lowering path cannot address channel-slice views
     path_ = level;
   }
   int path() const { return path_; }
+  // True if this geometry runs on the all-direct path by default.
+  bool direct_by_default() const { return default_path_ == PATH_DIRECT_ALL; }
+  // The layers' cubes are channel slices of wider tensors: `in_stride` / `out_stride` floats lie
+  // between consecutive images (0 = dense).  Only the all-direct path can work on such views; the
+  // bridge then stays on it.
+  void set_image_strides(size_t in_stride, size_t out_stride) {
+    if (!direct_ok_) {
+      std::fprintf(stderr, "ConvolutionBridge: channel-slice views need the direct kernels\n");
+      std::abort();
+    }
+    in_image_stride_ = in_stride;
+    out_image_stride_ = out_stride;
+    path_ = PATH_DIRECT_ALL;
+    views_ = true;
+  }
   void set_fused(bool on) { set_path(on ? default_path_ : PATH_STAGED); }
   // per-stage hipEvent timing (the reference's -D_DETAILED_PROFILING stage prints)
   void set_stage_profiling(bool on) { profile_ = on; }
@@ -183,7 +202,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                   (int)num_output_features, (int)iD, (int)K, 0);
       p_driver->conv_direct_forward(output_d_cube->get_p_data(), input_d_cube->get_p_data(),
                                     forward_slabs()->get_p_data(), bias_term ? p_bias_cube->get_p_data() : nullptr,
-                                    (int)iB, (int)iD, (int)iR, (int)K, (int)padding, (int)num_output_features);
+                                    (int)iB, (int)iD, (int)iR, (int)K, (int)padding, (int)num_output_features,
+                                    in_image_stride_, out_image_stride_);
       end(STAGE_GEMM);
       report_forward_history.end();
       return;
@@ -259,7 +279,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                              bias_term ? p_bias_gradient_cube->get_p_data() : nullptr,
                                              output_g_cube->get_p_data(), p_input_layer->p_data_cube->get_p_data(),
                                              (int)iB, (int)iD, (int)iR, (int)K, (int)padding,
-                                             (int)num_output_features);
+                                             (int)num_output_features, in_image_stride_, out_image_stride_);
     } else {
       p_backward_gemm_updateweight_kernel->alpha = 1.0;
       p_backward_gemm_updateweight_kernel->beta = 0.0;
@@ -273,7 +293,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                   (int)num_output_features, (int)iD, (int)K, 1);
       p_driver->conv_direct_backward_data(input_g_cube->get_p_data(), output_g_cube->get_p_data(),
                                           backward_slabs()->get_p_data(), (int)iB, (int)iD, (int)iR, (int)K,
-                                          (int)padding, (int)num_output_features);
+                                          (int)padding, (int)num_output_features, in_image_stride_,
+                                          out_image_stride_);
       end(STAGE_GEMM_DATA);
     } else if (needs_to_calc_backward_grad) {
       begin(STAGE_INVERSE_LOWER);
@@ -325,6 +346,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
 
  private:
   int path_ = PATH_FUSED, default_path_ = PATH_FUSED;
+  size_t in_image_stride_ = 0, out_image_stride_ = 0;
+  bool views_ = false;
   bool direct_ok_ = false, profile_ = false;
   LogicalCubeType *lowered() {
     if (!p_forward_lowered_data) p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);

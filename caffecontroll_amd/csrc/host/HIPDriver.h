@@ -184,21 +184,24 @@ class HIPDriver {
     ok(cct_hip_conv_direct_slabs(slabs, model, num_outputs, depth, k, for_data_gradient), "conv_direct_slabs");
   }
   void conv_direct_forward(float *output, const float *input, const float *slabs, const float *bias, int batch,
-                           int depth, int n, int k, int padding, int num_outputs) {
-    ok(cct_hip_conv_direct_forward(output, input, slabs, bias, batch, depth, n, k, padding, num_outputs),
+                           int depth, int n, int k, int padding, int num_outputs, size_t in_stride = 0,
+                           size_t out_stride = 0) {
+    ok(cct_hip_conv_direct_forward(output, input, slabs, bias, batch, depth, n, k, padding, num_outputs, in_stride,
+                                   out_stride),
        "conv_direct_forward");
   }
   void conv_direct_backward_data(float *input_grad, const float *output_grad, const float *slabs, int batch,
-                                 int depth, int n, int k, int padding, int num_outputs) {
-    ok(cct_hip_conv_direct_backward_data(input_grad, output_grad, slabs, batch, depth, n, k, padding,
-                                         num_outputs),
+                                 int depth, int n, int k, int padding, int num_outputs, size_t in_stride = 0,
+                                 size_t out_stride = 0) {
+    ok(cct_hip_conv_direct_backward_data(input_grad, output_grad, slabs, batch, depth, n, k, padding, num_outputs,
+                                         in_stride, out_stride),
        "conv_direct_backward_data");
   }
   void conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                     const float *input, int batch, int depth, int n, int k, int padding,
-                                    int num_outputs) {
+                                    int num_outputs, size_t in_stride = 0, size_t out_stride = 0) {
     ok(cct_hip_conv_direct_backward_weights(model_grad, bias_grad, output_grad, input, batch, depth, n, k, padding,
-                                            num_outputs),
+                                            num_outputs, in_stride, out_stride),
        "conv_direct_backward_weights");
   }
   void sgemv(const CBLAS_TRANSPOSE TA, const int M, const int N, const float alpha, const float *pA,

@@ -72,13 +72,22 @@ class Network {
             lp->convolution_param_.bias_term_ = s.bias_term != 0;
             nd.params.push_back(lp);
             LayerT *gin = cur, *gout = nd.out;
-            if (g > 1) {
+            // A group works in place on its channel slices of the whole tensors when the direct
+            // kernels take the layer (they accept an image stride); otherwise the slices are
+            // gathered into contiguous per-group layers and scattered back.
+            const bool in_place = g > 1 && group_in_place(R, D / g, s, s.num_output / g, m);
+            if (g > 1 && in_place) {
+              const size_t din = D / g, dout = s.num_output / g;
+              gin = view_layer(cur, gi * din * R * R, R, R, din);
+              gout = view_layer(nd.out, gi * dout * m * m, m, m, dout);
+            } else if (g > 1) {
               gin = new_layer(R, R, D / g);
               gout = new_layer(m, m, s.num_output / g);
               nd.group_in.push_back(gin);
               nd.group_out.push_back(gout);
             }
             auto *b = new ParallelizedBridge<float, ConvolutionBridge, HIPDriver>(gin, gout, lp, &solver_, &driver_);
+            if (in_place) b->sub_bridge()->set_image_strides(D * R * R, (size_t)s.num_output * m * m);
             b->needs_to_calc_backward_grad = !first_weight_layer;
             nd.bridges.push_back(b);
           }
@@ -215,6 +224,18 @@ class Network {
     LayerT *l = new LayerT(new CubeT(R, C, D, batch_, &driver_), new CubeT(R, C, D, batch_, &driver_));
     layers_.push_back(l);
     return l;
+  }
+  // non-owning layer over a channel slice (first element at `offset` floats) of `whole`
+  LayerT *view_layer(LayerT *whole, size_t offset, size_t R, size_t C, size_t D) {
+    LayerT *l = new LayerT(new CubeT(whole->p_data_cube->get_p_data() + offset, R, C, D, batch_),
+                           new CubeT(whole->p_gradient_cube->get_p_data() + offset, R, C, D, batch_));
+    layers_.push_back(l);
+    return l;
+  }
+  // the condition under which ConvolutionBridge picks the all-direct path on its own
+  bool group_in_place(size_t R, size_t d, const cct_layer_spec &s, size_t o, size_t m) {
+    if (!driver_.conv_direct_supported(batch_, (int)d, (int)R, s.kernel_size, s.stride, s.pad, (int)o)) return false;
+    return 2.0 * o * (double)(m * m * batch_) * (double)(s.kernel_size * s.kernel_size * d) >= kConvDirectMinFlop;
   }
   static cnn::LayerParameter *new_param(const cct_layer_spec &s) {
     cnn::LayerParameter *lp = new cnn::LayerParameter;

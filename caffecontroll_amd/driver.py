@@ -123,16 +123,17 @@ class HIPDriver:
         check(self.lib.cct_hip_conv_direct_slabs(_p(slabs), _p(model), o, d, k, int(for_data_gradient)),
               "conv_direct_slabs")
 
-    def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o):
-        check(self.lib.cct_hip_conv_direct_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o),
-              "conv_direct_forward")
+    def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o, in_stride=0, out_stride=0):
+        check(self.lib.cct_hip_conv_direct_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o,
+                                                   in_stride, out_stride), "conv_direct_forward")
 
-    def conv_direct_backward_data(self, din, dout, slabs, b, d, n, k, p, o):
-        check(self.lib.cct_hip_conv_direct_backward_data(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o),
-              "conv_direct_backward_data")
+    def conv_direct_backward_data(self, din, dout, slabs, b, d, n, k, p, o, in_stride=0, out_stride=0):
+        check(self.lib.cct_hip_conv_direct_backward_data(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o,
+                                                         in_stride, out_stride), "conv_direct_backward_data")
 
-    def conv_direct_backward_weights(self, dw, dout, inp, b, d, n, k, p, o, db=None):
-        check(self.lib.cct_hip_conv_direct_backward_weights(_p(dw), _p(db), _p(dout), _p(inp), b, d, n, k, p, o),
+    def conv_direct_backward_weights(self, dw, dout, inp, b, d, n, k, p, o, db=None, in_stride=0, out_stride=0):
+        check(self.lib.cct_hip_conv_direct_backward_weights(_p(dw), _p(db), _p(dout), _p(inp), b, d, n, k, p, o,
+                                                            in_stride, out_stride),
               "conv_direct_backward_weights")
 
     def sgemv(self, TA, M, N, alpha, A, x, beta, y):

@@ -170,17 +170,24 @@ int cct_hip_conv_direct_supported(int batch, int depth, int n, int k, int stride
 size_t cct_hip_conv_direct_slab_floats(int num_outputs, int depth, int k, int for_data_gradient);
 int cct_hip_conv_direct_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
                               int for_data_gradient);
-/* lower_cube + forward GEMM + remap_output + bias of ConvolutionBridge::forward
+/* The three kernels below take the distance in floats between consecutive images of the input
+ * tensor and of the output tensor (input_image_stride, output_image_stride; 0 = dense, i.e.
+ * d*n*n and o*m*m).  A larger stride addresses a channel slice of a wider tensor in place, which
+ * is how a grouped convolution runs without gathering its slices
+ * (DeepNet's Split/Concat grouping, src/DeepNet.h:1700-1757).
+ *
+ * lower_cube + forward GEMM + remap_output + bias of ConvolutionBridge::forward
  * (src/bridges/ConvolutionBridge_impl.hxx:316-364) in one kernel:
  * output[b][o][m][m] from input[b][d][n][n], forward slabs, bias[o] (may be NULL). */
 int cct_hip_conv_direct_forward(float *output, const float *input, const float *slabs,
                                 const float *bias, int batch, int depth, int n, int k, int padding,
-                                int num_outputs);
+                                int num_outputs, size_t input_image_stride, size_t output_image_stride);
 /* Gradient remap + data-gradient GEMM + inverse_lower_cube of ConvolutionBridge::backward
  * (src/bridges/ConvolutionBridge_impl.hxx:601-616) in one kernel: input_grad[b][d][n][n] from
  * output_grad[b][o][m][m] (read in place, not permuted) and data-gradient slabs. */
 int cct_hip_conv_direct_backward_data(float *input_grad, const float *output_grad, const float *slabs,
-                                      int batch, int depth, int n, int k, int padding, int num_outputs);
+                                      int batch, int depth, int n, int k, int padding, int num_outputs,
+                                      size_t input_image_stride, size_t output_image_stride);
 /* Weight-gradient GEMM of ConvolutionBridge::backward (src/bridges/ConvolutionBridge_impl.hxx:
  * 619-621) without the lowered matrix or the gradient remap: model_grad[o][d][k][k] (overwritten,
  * beta = 0) from output_grad[b][o][m][m] and input[b][d][n][n].  If bias_grad is not NULL the same
@@ -188,7 +195,7 @@ int cct_hip_conv_direct_backward_data(float *input_grad, const float *output_gra
  * (:575-599), in a fixed summation order. */
 int cct_hip_conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                          const float *input, int batch, int depth, int n, int k, int padding,
-                                         int num_outputs);
+                                         int num_outputs, size_t input_image_stride, size_t output_image_stride);
 /* DeviceDriver::sgemv (src/sched/DeviceDriver.h:214-215): row-major M x N, lda = N. */
 int cct_hip_sgemv(int TA, int M, int N, float alpha, const float *A, const float *x, float beta,
                   float *y);

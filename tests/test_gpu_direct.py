@@ -102,6 +102,51 @@ def test_direct_kernels_match_oracle(oracle, shape):
     np.testing.assert_array_equal(host(db2), host(db))
 
 
+@pytest.mark.parametrize("shape", [(4, 6, 13, 3, 1, 10), (3, 8, 27, 5, 2, 36)], ids=_ids)
+def test_direct_kernels_on_channel_slices(oracle, shape):
+    """Grouped convolution in place: each group reads its channel slice of the whole input and
+    writes its slice of the whole output (image strides of the whole tensors); results equal the
+    kernels run on gathered, contiguous slices bit for bit, and nothing outside a slice is touched."""
+    b, d, n, k, p, o = shape
+    groups = 2
+    m = n + 2 * p - k + 1
+    rng = np.random.default_rng(55 + sum(shape))
+    x = rng.standard_normal((b, groups * d, n, n)).astype(np.float32)
+    og = rng.standard_normal((b, groups * o, m, m)).astype(np.float32)
+    ws = [(rng.standard_normal((o, d, k, k)) * 0.1).astype(np.float32) for _ in range(groups)]
+    bias = rng.standard_normal(groups * o).astype(np.float32)
+    drv = driver()
+    d_x, d_og, d_bias = dev(x), dev(og), dev(bias)
+    out_whole, dx_whole = empty((b, groups * o, m, m)), empty((b, groups * d, n, n))
+    in_stride, out_stride = groups * d * n * n, groups * o * m * m
+    for gi in range(groups):
+        d_w = dev(ws[gi])
+        sf, sb = _slabs(d_w, o, d, k)
+        xs, ogs = d_x[:, gi * d:(gi + 1) * d], d_og[:, gi * o:(gi + 1) * o]   # views into the whole tensors
+        outs, dxs = out_whole[:, gi * o:(gi + 1) * o], dx_whole[:, gi * d:(gi + 1) * d]
+        bs = d_bias[gi * o:(gi + 1) * o]
+        drv.conv_direct_forward(outs, xs, sf, bs, b, d, n, k, p, o, in_stride, out_stride)
+        drv.conv_direct_backward_data(dxs, ogs, sb, b, d, n, k, p, o, in_stride, out_stride)
+        dw, db = empty((o, d, k, k)), empty((o,))
+        drv.conv_direct_backward_weights(dw, ogs, xs, b, d, n, k, p, o, db=db, in_stride=in_stride,
+                                         out_stride=out_stride)
+        # the same on contiguous copies of the slices
+        xc, ogc = xs.contiguous(), ogs.contiguous()
+        outc, dxc, dwc, dbc = empty((b, o, m, m)), empty((b, d, n, n)), empty((o, d, k, k)), empty((o,))
+        drv.conv_direct_forward(outc, xc, sf, bs, b, d, n, k, p, o)
+        drv.conv_direct_backward_data(dxc, ogc, sb, b, d, n, k, p, o)
+        drv.conv_direct_backward_weights(dwc, ogc, xc, b, d, n, k, p, o, db=dbc)
+        np.testing.assert_array_equal(host(outs), host(outc))
+        np.testing.assert_array_equal(host(dxs), host(dxc))
+        np.testing.assert_array_equal(host(dw), host(dwc))
+        np.testing.assert_array_equal(host(db), host(dbc))
+        ref_out, _ = oracle.conv_forward(host(xc), ws[gi], bias[gi * o:(gi + 1) * o], k, 1, p)
+        assert rel_err(host(outc), ref_out) <= TOL
+    assert not np.isnan(host(out_whole)).any() and not np.isnan(host(dx_whole)).any()
+    np.testing.assert_array_equal(host(d_x), x)
+    np.testing.assert_array_equal(host(d_og), og)
+
+
 def test_direct_exact_on_small_integers(oracle):
     """Small-integer tensors make every sum exact in fp32, so the direct kernels must reproduce the
     lowering pipeline bit for bit whatever the summation order."""
