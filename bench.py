@@ -102,11 +102,22 @@ def cpu_baseline(cfg, seed):
     times = sorted(run() for _ in range(reps))
     med = times[len(times) // 2]
     O.unbind_openblas()
-    return {
+    result = {
         "value": b / med, "unit": "images/sec", "cores": P, "kind": "port",
         "sample": "full %s workload (b=%d), 1 warm-up + %d timed passes, median; %d batch partitions x 1 BLAS "
                   "thread; sgemm=%s" % (cfg, b, reps, P, "OpenBLAS (scipy bundle)" if blas else "plain loops"),
     }
+    # the other way to spend the same cores: one partition, all of them inside the BLAS calls
+    if O.bind_openblas(cores):
+        def whole():
+            t0 = time.perf_counter()
+            part((0, b))
+            return time.perf_counter() - t0
+        whole()
+        t2 = sorted(whole() for _ in range(reps))[reps // 2]
+        O.unbind_openblas()
+        result["one_partition_all_blas_threads"] = {"value": b / t2, "unit": "images/sec", "cores": cores}
+    return result
 
 
 def net_iteration(args, torch, np):
