@@ -2,6 +2,7 @@
 #include <string>
 
 #include "../../include/cct_bridge.h"
+#include "cct_common.h"
 #include "host/ConvolutionBridge.h"
 #include "host/Network.h"
 #include "host/ParallelizedBridge.h"
@@ -152,6 +153,8 @@ void *cct_net_tensor(cct_net *h, int layer, int group, int which, size_t *n) {
     case 3: c = b->get_bias_grad_cube(); break;
     case 4: c = nd.out->p_data_cube; break;
     case 5: c = nd.in->p_gradient_cube; break;
+    case 7: c = b->get_model_history_cube(); break;
+    case 8: c = b->get_bias_history_cube(); break;
     case 6:
       if (nd.spec.type == CCT_LAYER_DROPOUT) {
         auto *m = static_cast<DropoutBridge<float, HIPDriver> *>(b)->get_mask_cube();
@@ -204,5 +207,39 @@ int cct_net_loss(cct_net *h, float *loss_sum) {
   *loss_sum = h->net->loss();
   return 0;
 }
+
+namespace {
+int io_result(cct_net *h, bool ok) {
+  return ok ? 0 : cct::set_error(CCT_HIP_EINVAL, "%s", h->net->io_error().c_str());
+}
+}  // namespace
+
+int cct_net_write_model(cct_net *h, const char *file) {
+  if (!h || !file) return CCT_HIP_EINVAL;
+  return io_result(h, h->net->write_blobs(file, Network::BLOB_MODEL));
+}
+
+int cct_net_read_model(cct_net *h, const char *file) {
+  if (!h || !file) return CCT_HIP_EINVAL;
+  return io_result(h, h->net->read_blobs(file, Network::BLOB_MODEL));
+}
+
+int cct_net_write_snapshot(cct_net *h, const char *base_filename, int iter) {
+  if (!h || !base_filename || iter < 0) return CCT_HIP_EINVAL;
+  return io_result(h, h->net->write_snapshot(base_filename, iter));
+}
+
+int cct_net_read_snapshot(cct_net *h, const char *stem, int *iter) {
+  if (!h || !stem) return CCT_HIP_EINVAL;
+  return io_result(h, h->net->read_snapshot(stem, iter));
+}
+
+int cct_net_set_iter(cct_net *h, int iter) {
+  if (!h || iter < 0) return CCT_HIP_EINVAL;
+  h->net->set_current_iter(iter);
+  return 0;
+}
+
+size_t cct_net_parameter_size(cct_net *h) { return h ? h->net->parameter_size() : 0; }
 
 }  // extern "C"

@@ -60,6 +60,11 @@ class AbstractBridge {
   virtual LogicalCubeType *get_bias_cube() { return nullptr; }
   virtual LogicalCubeType *get_model_grad_cube() { return nullptr; }
   virtual LogicalCubeType *get_bias_grad_cube() { return nullptr; }
+  // momentum buffers of the two updaters and their iteration counter (what the reference's
+  // snapshots carry besides the model: src/DeepNet.h:268-330, 386-422)
+  virtual LogicalCubeType *get_model_history_cube() { return nullptr; }
+  virtual LogicalCubeType *get_bias_history_cube() { return nullptr; }
+  virtual void set_current_iter(int) {}
 };
 
 }  // namespace cct

@@ -11,9 +11,16 @@
 //     GPU: ParallelizedBridge.h:183-198);
 //   * `group` > 1 is realised as `group` independent convolutions on channel slices whose outputs
 //     are concatenated along depth (the reference's two-tower Split/Concat arrangement,
-//     src/DeepNet.h:1700-1757); slices are moved with a strided device copy.
+//     src/DeepNet.h:1700-1757); a group runs in place on its channel slices when the direct
+//     kernels take the layer, otherwise the slices are moved with a strided device copy.
+//
+// Model files and snapshots use the reference's format (src/DeepNet.h:268-422): raw fp32, for
+// every bridge in order its model cube and then its bias cube; a snapshot is three files
+// <base>.snapshot_iter<N>.{MODEL,HISTORY,ITER}.bin (weights, momentum buffers, one int).
 #pragma once
+#include <cstdio>
 #include <memory>
+#include <string>
 #include <vector>
 
 #include "../../../include/cct_bridge.h"
@@ -70,6 +77,8 @@ class Network {
             lp->convolution_param_.stride_ = s.stride;
             lp->convolution_param_.pad_ = s.pad;
             lp->convolution_param_.bias_term_ = s.bias_term != 0;
+            set_filler(lp->convolution_param_.weight_filler_, s.weight_filler);
+            set_filler(lp->convolution_param_.bias_filler_, s.bias_filler);
             nd.params.push_back(lp);
             LayerT *gin = cur, *gout = nd.out;
             // A group works in place on its channel slices of the whole tensors when the direct
@@ -99,6 +108,8 @@ class Network {
           cnn::LayerParameter *lp = new_param(s);
           lp->inner_product_param_.num_output_ = s.num_output;
           lp->inner_product_param_.bias_term_ = s.bias_term != 0;
+          set_filler(lp->inner_product_param_.weight_filler_, s.weight_filler);
+          set_filler(lp->inner_product_param_.bias_filler_, s.bias_filler);
           nd.params.push_back(lp);
           auto *b = new ParallelizedBridge<float, FullyConnectedBridge, HIPDriver>(cur, nd.out, lp, &solver_, &driver_);
           b->needs_to_calc_backward_grad = !first_weight_layer;
@@ -207,6 +218,79 @@ class Network {
 
   float loss() { return softmax_ ? softmax_->get_loss() : 0.f; }
 
+  // ---- model files and snapshots (src/DeepNet.h:268-422) ----
+  enum Blob { BLOB_MODEL, BLOB_HISTORY };
+  const std::string &io_error() const { return io_error_; }
+
+  // DeepNet::write_model_to_file / write_momentum_to_file
+  bool write_blobs(const std::string &file, Blob what) {
+    FILE *f = std::fopen(file.c_str(), "wb");
+    if (!f) return io_fail("Error opening " + file);
+    bool ok = true;
+    std::vector<float> host;
+    for_each_blob(what, [&](CubeT *c) {
+      host.resize(c->n_elements);
+      if (cct_hip_memcpy(host.data(), c->get_p_data(), host.size() * sizeof(float), 1)) fail(cct_hip_last_error());
+      ok = ok && std::fwrite(host.data(), sizeof(float), host.size(), f) == host.size();
+    });
+    ok = (std::fclose(f) == 0) && ok;
+    return ok ? true : io_fail("short write to " + file);
+  }
+
+  // DeepNet::read_model_from_file / read_momentum_from_file; the file must hold every blob
+  bool read_blobs(const std::string &file, Blob what) {
+    FILE *f = std::fopen(file.c_str(), "rb");
+    if (!f) return io_fail("Error opening " + file);
+    bool ok = true;
+    std::vector<float> host;
+    for_each_blob(what, [&](CubeT *c) {
+      if (!ok) return;
+      host.resize(c->n_elements);
+      ok = std::fread(host.data(), sizeof(float), host.size(), f) == host.size();
+      if (ok && cct_hip_memcpy(c->get_p_data(), host.data(), host.size() * sizeof(float), 0)) fail(cct_hip_last_error());
+    });
+    std::fclose(f);
+    return ok ? true : io_fail(file + " holds fewer values than the network's blobs");
+  }
+
+  // DeepNet::get_parameter_size (src/DeepNet.h:425-441)
+  size_t parameter_size() {
+    size_t n = 0;
+    for_each_blob(BLOB_MODEL, [&](CubeT *c) { n += c->n_elements; });
+    return n;
+  }
+
+  void set_current_iter(int iter) {
+    for (Node &nd : nodes_)
+      for (BridgeT *b : nd.bridges) b->set_current_iter(iter);
+  }
+
+  // DeepNet::write_full_snapshot (src/DeepNet.h:268-295)
+  bool write_snapshot(const std::string &base_filename, int iter) {
+    const std::string stem = base_filename + ".snapshot_iter" + std::to_string(iter);
+    if (!write_blobs(stem + ".MODEL.bin", BLOB_MODEL) || !write_blobs(stem + ".HISTORY.bin", BLOB_HISTORY))
+      return false;
+    FILE *f = std::fopen((stem + ".ITER.bin").c_str(), "wb");
+    if (!f) return io_fail("Error opening " + stem + ".ITER.bin");
+    const bool ok = std::fwrite(&iter, sizeof(int), 1, f) == 1;
+    return (std::fclose(f) == 0 && ok) ? true : io_fail("short write to " + stem + ".ITER.bin");
+  }
+
+  // DeepNet::read_full_snapshot (src/DeepNet.h:297-326); `stem` ends in ".snapshot_iter<N>"
+  bool read_snapshot(const std::string &stem, int *iter_out) {
+    if (!read_blobs(stem + ".MODEL.bin", BLOB_MODEL) || !read_blobs(stem + ".HISTORY.bin", BLOB_HISTORY))
+      return false;
+    FILE *f = std::fopen((stem + ".ITER.bin").c_str(), "rb");
+    if (!f) return io_fail("Error opening " + stem + ".ITER.bin");
+    int iter = 0;
+    const bool ok = std::fread(&iter, sizeof(int), 1, f) == 1;
+    std::fclose(f);
+    if (!ok) return io_fail(stem + ".ITER.bin is empty");
+    set_current_iter(iter);
+    if (iter_out) *iter_out = iter;
+    return true;
+  }
+
  private:
   HIPDriver driver_;
   cnn::SolverParameter solver_;
@@ -216,6 +300,29 @@ class Network {
   std::vector<Node> nodes_;
   SoftmaxLossBridge<float, HIPDriver> *softmax_ = nullptr;
 
+  std::string io_error_;
+  bool io_fail(const std::string &msg) {
+    io_error_ = msg;
+    return false;
+  }
+  // Bridges in order; per bridge model then bias (src/DeepNet.h:335-352).  The groups of a grouped
+  // convolution are written as ONE layer -- all group models in order ([o][d/g][k][k]), then all
+  // group biases ([o]) -- the blob layout such a layer has in Caffe; the reference ignores `group`.
+  template <typename F>
+  void for_each_blob(Blob what, F f) {
+    for (Node &nd : nodes_) {
+      for (BridgeT *b : nd.bridges)
+        if (CubeT *c = what == BLOB_MODEL ? b->get_model_cube() : b->get_model_history_cube()) f(c);
+      for (BridgeT *b : nd.bridges)
+        if (CubeT *c = what == BLOB_MODEL ? b->get_bias_cube() : b->get_bias_history_cube()) f(c);
+    }
+  }
+  static void set_filler(cnn::FillerParameter &dst, const cct_filler &src) {
+    static const char *const names[] = {"constant", "xavier", "gaussian", "bernoulli"};
+    if (src.type < 0 || src.type > 3) fail("unknown filler type");
+    dst.type_ = names[src.type];
+    dst.value_ = src.value; dst.mean_ = src.mean; dst.std_ = src.std;
+  }
   static void fail(const char *msg) {
     std::fprintf(stderr, "Network: %s\n", msg);
     std::abort();

@@ -74,6 +74,17 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
   LogicalCubeType *get_bias_cube() override { return p_bias_cube; }
   LogicalCubeType *get_model_grad_cube() override { return p_model_grad; }
   LogicalCubeType *get_bias_grad_cube() override { return p_bias_grad; }
+  LogicalCubeType *get_model_history_cube() override {
+    return p_grad_updater ? p_grad_updater->get_p_history_updates_cube() : nullptr;
+  }
+  LogicalCubeType *get_bias_history_cube() override {
+    return p_grad_updater_bias ? p_grad_updater_bias->get_p_history_updates_cube() : nullptr;
+  }
+  // src/bridges/ParallelizedBridge.h:331-354: both updaters resume from `iter`
+  void set_current_iter(int iter) override {
+    if (p_grad_updater) p_grad_updater->set_current_iter(iter);
+    if (p_grad_updater_bias) p_grad_updater_bias->set_current_iter(iter);
+  }
 
   void forward() override {
     this->report_forward_history.reset();

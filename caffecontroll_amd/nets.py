@@ -1,6 +1,7 @@
 """Layer chains on the device (``cct_net_*`` of ``include/cct_bridge.h``) and the two networks of
 the benchmark configurations: LeNet and CaffeNet/AlexNet."""
 import ctypes as C
+import os
 
 from . import _lib
 from ._lib import check
@@ -9,17 +10,33 @@ from .bridges import SolverParam, solver_param  # noqa: F401
 CONV, FC, RELU, MAXPOOL, LRN, DROPOUT, SOFTMAXLOSS = 1, 2, 3, 4, 5, 6, 7
 
 
+FILLER_TYPES = {"constant": 0, "xavier": 1, "gaussian": 2, "bernoulli": 3}
+
+
+class Filler(C.Structure):
+    """cnn.proto FillerParameter: type, value (constant / bernoulli p), mean and std (gaussian)."""
+    _fields_ = [("type", C.c_int), ("value", C.c_float), ("mean", C.c_float), ("std", C.c_float)]
+
+
+def filler(type="constant", value=0.0, mean=0.0, std=1.0):
+    if type not in FILLER_TYPES:
+        raise ValueError("unknown filler type %r" % (type,))
+    return Filler(FILLER_TYPES[type], value, mean, std)
+
+
 class LayerSpec(C.Structure):
     _fields_ = [("type", C.c_int), ("num_output", C.c_int), ("kernel_size", C.c_int), ("stride", C.c_int),
                 ("pad", C.c_int), ("group", C.c_int), ("bias_term", C.c_int), ("lrn_local_size", C.c_int),
                 ("lrn_alpha", C.c_float), ("lrn_beta", C.c_float), ("dropout_ratio", C.c_float),
-                ("lr_mult", C.c_float * 2), ("decay_mult", C.c_float * 2)]
+                ("lr_mult", C.c_float * 2), ("decay_mult", C.c_float * 2),
+                ("weight_filler", Filler), ("bias_filler", Filler)]
 
 
 def _spec(t, **kw):
     s = LayerSpec()
     s.type, s.stride, s.group, s.bias_term = t, 1, 1, 1
     s.lr_mult[0], s.lr_mult[1], s.decay_mult[0], s.decay_mult[1] = 1.0, 2.0, 1.0, 0.0
+    s.weight_filler, s.bias_filler = filler(), filler()
     for k, v in kw.items():
         if k in ("lr_mult", "decay_mult"):
             getattr(s, k)[0], getattr(s, k)[1] = v
@@ -58,8 +75,11 @@ def softmax_loss():
 
 def lenet_layers():
     """tests/lenet_train/lenet_train_test.prototxt of the reference: conv(20,5)-pool2-conv(50,5)-pool2-
-    ip500-relu-ip10-softmax loss; lr_mult 1 (weights) / 2 (bias)."""
-    return [conv(20, 5), maxpool(2, 2), conv(50, 5), maxpool(2, 2), fc(500), relu(), fc(10), softmax_loss()]
+    ip500-relu-ip10-softmax loss; lr_mult 1 (weights) / 2 (bias), decay_mult left at its default 1 for
+    both, xavier weights and zero biases."""
+    kw = dict(decay_mult=(1.0, 1.0), weight_filler=filler("xavier"))
+    return [conv(20, 5, **kw), maxpool(2, 2), conv(50, 5, **kw), maxpool(2, 2), fc(500, **kw), relu(), fc(10, **kw),
+            softmax_loss()]
 
 
 def caffenet_layers(groups=True, num_classes=1000):
@@ -88,6 +108,12 @@ NET_PROTOTYPES = {
     "cct_net_forward": ([_P], _I),
     "cct_net_backward": ([_P], _I),
     "cct_net_loss": ([_P, C.POINTER(C.c_float)], _I),
+    "cct_net_write_model": ([_P, C.c_char_p], _I),
+    "cct_net_read_model": ([_P, C.c_char_p], _I),
+    "cct_net_write_snapshot": ([_P, C.c_char_p, _I], _I),
+    "cct_net_read_snapshot": ([_P, C.c_char_p, C.POINTER(_I)], _I),
+    "cct_net_set_iter": ([_P, _I], _I),
+    "cct_net_parameter_size": ([_P], C.c_size_t),
 }
 _bound = False
 
@@ -103,7 +129,7 @@ def _bind():
     return lib
 
 
-MODEL, BIAS, MODEL_GRAD, BIAS_GRAD, OUTPUT, INPUT_GRAD, AUX = range(7)
+MODEL, BIAS, MODEL_GRAD, BIAS_GRAD, OUTPUT, INPUT_GRAD, AUX, MODEL_HISTORY, BIAS_HISTORY = range(9)
 
 
 class Net:
@@ -149,6 +175,30 @@ class Net:
         v = C.c_float()
         check(self.lib.cct_net_loss(self.h, C.byref(v)), "net_loss")
         return v.value
+
+    # ---- model files and snapshots in the reference's format (src/DeepNet.h:268-422) ----
+    def write_model(self, path):
+        check(self.lib.cct_net_write_model(self.h, os.fsencode(path)), "net_write_model")
+
+    def read_model(self, path):
+        check(self.lib.cct_net_read_model(self.h, os.fsencode(path)), "net_read_model")
+
+    def write_snapshot(self, base_filename, iteration):
+        """Writes <base>.snapshot_iter<N>.MODEL.bin / .HISTORY.bin / .ITER.bin; returns the common stem."""
+        check(self.lib.cct_net_write_snapshot(self.h, os.fsencode(base_filename), iteration), "net_write_snapshot")
+        return "%s.snapshot_iter%d" % (base_filename, iteration)
+
+    def read_snapshot(self, stem):
+        """Restores weights, momentum and the iteration counter; returns the iteration."""
+        it = C.c_int()
+        check(self.lib.cct_net_read_snapshot(self.h, os.fsencode(stem), C.byref(it)), "net_read_snapshot")
+        return it.value
+
+    def set_iter(self, iteration):
+        check(self.lib.cct_net_set_iter(self.h, iteration), "net_set_iter")
+
+    def parameter_size(self):
+        return self.lib.cct_net_parameter_size(self.h)
 
     def close(self):
         if self.h:

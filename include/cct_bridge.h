@@ -83,6 +83,15 @@ enum cct_layer_type {
   CCT_LAYER_DROPOUT = 6, CCT_LAYER_SOFTMAXLOSS = 7
 };
 
+/* cnn::FillerParameter (src/parser/cnn.proto:21-32).  A zeroed struct is the proto default for
+ * type and value ("constant", 0); set std explicitly for a gaussian filler (proto default 1). */
+enum cct_filler_type { CCT_FILLER_CONSTANT = 0, CCT_FILLER_XAVIER = 1, CCT_FILLER_GAUSSIAN = 2, CCT_FILLER_BERNOULLI = 3 };
+typedef struct cct_filler {
+  int type;          /* enum cct_filler_type */
+  float value;       /* constant: the value; bernoulli: the probability */
+  float mean, std;   /* gaussian */
+} cct_filler;
+
 /* The fields of cnn::LayerParameter this path reads; unused ones are ignored per type. */
 typedef struct cct_layer_spec {
   int type;                 /* enum cct_layer_type */
@@ -95,6 +104,7 @@ typedef struct cct_layer_spec {
   float dropout_ratio;
   float lr_mult[2];         /* weights, bias */
   float decay_mult[2];
+  cct_filler weight_filler, bias_filler; /* conv, fc; random fillers draw from solver.random_seed */
 } cct_layer_spec;
 
 typedef struct cct_net cct_net;
@@ -107,7 +117,8 @@ float *cct_net_labels(cct_net *net);  /* device, one float per image */
 int cct_net_num_layers(cct_net *net);
 /* Device pointer + element count of a tensor of layer `layer`, channel group `group`:
  * which = 0 model, 1 bias, 2 model gradient, 3 bias gradient, 4 output data of the layer,
- * 5 gradient w.r.t. the layer's input, 6 dropout mask (uint32) / max-pool argmax (int32).
+ * 5 gradient w.r.t. the layer's input, 6 dropout mask (uint32) / max-pool argmax (int32),
+ * 7 momentum buffer of the model, 8 momentum buffer of the bias.
  * Returns NULL (and *n = 0) when the layer has no such tensor. */
 void *cct_net_tensor(cct_net *net, int layer, int group, int which, size_t *n);
 int cct_net_set_train(cct_net *net, int train);
@@ -116,6 +127,24 @@ int cct_net_freeze_dropout_masks(cct_net *net, int freeze);
 int cct_net_forward(cct_net *net);
 int cct_net_backward(cct_net *net);   /* gradients + SGD update of every layer */
 int cct_net_loss(cct_net *net, float *loss_sum); /* batch-summed loss of the last forward (syncs) */
+
+/* Model files and snapshots in the reference's format: raw fp32, per bridge its model then its
+ * bias (DeepNet::write_model_to_file / read_model_from_file, src/DeepNet.h:328-374; the
+ * `-output-model-file` / `-input-model-file` options of `caffe-ct`).  The groups of a grouped
+ * convolution are stored as one layer: [o][d/g][k][k] then [o]. */
+int cct_net_write_model(cct_net *net, const char *file);
+int cct_net_read_model(cct_net *net, const char *file);
+/* DeepNet::write_full_snapshot (src/DeepNet.h:268-295): writes
+ * <base>.snapshot_iter<iter>.MODEL.bin, .HISTORY.bin (momentum buffers) and .ITER.bin (one int). */
+int cct_net_write_snapshot(cct_net *net, const char *base_filename, int iter);
+/* DeepNet::read_full_snapshot (src/DeepNet.h:297-326): `stem` is the common prefix of the three
+ * files (ends in ".snapshot_iter<N>"); restores weights, momentum and the updaters' iteration
+ * counter, which is also returned through *iter. */
+int cct_net_read_snapshot(cct_net *net, const char *stem, int *iter);
+/* Iteration counter of every gradient updater (learning-rate schedule position). */
+int cct_net_set_iter(cct_net *net, int iter);
+/* DeepNet::get_parameter_size (src/DeepNet.h:425-441): weights + biases of all layers. */
+size_t cct_net_parameter_size(cct_net *net);
 
 #ifdef __cplusplus
 }
