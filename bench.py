@@ -163,9 +163,57 @@ def net_iteration(args, torch, np):
     drv.memcpy(net.input_ptr(), x.ctypes.data, x.nbytes, 0)
     drv.memcpy(net.labels_ptr(), labels.ctypes.data, labels.nbytes, 0)
 
+    pipeline = None
+    if args.input_pipeline:
+        # Raw 256x256 byte images in host memory stand in for the LMDB records; every step the
+        # loader copies one batch into pinned staging, uploads it on its copy stream while the
+        # previous iteration computes, and the transform kernel (mean, random crop, mirror, scale)
+        # writes the network's input.
+        from caffecontroll_amd import corpus
+        H = 256 if args.workload == "caffenet" else S
+        crop = S if H != S else 0
+        mean = rng.uniform(100, 125, (D, H, H)).astype(np.float32) if args.workload == "caffenet" else None
+        scale = 1.0 if args.workload == "caffenet" else 0.00390625
+        cp = corpus.Corpus.create(B, D, H, H, crop_size=crop, scale=scale, mirror=crop > 0, phase=0, mean=mean, seed=1)
+        pool = [(rng.integers(0, 256, (B, D, H, H), dtype=np.uint8), rng.integers(0, classes, B).astype(np.float32))
+                for _ in range(2)]
+        fed = [0]
+
+        def feed():
+            px, lb, _ = cp.stage()
+            src = pool[fed[0] % len(pool)]
+            for i in range(B):          # one copy per record, as the per-image workers do
+                px[i] = src[0][i]
+            lb[...] = src[1]
+            cp.submit()
+            fed[0] += 1
+
+        feed()
+        # the transform kernel alone: bytes read (raw + mean) and written (float batch) per launch
+        raw_dev = torch.from_numpy(pool[0][0]).cuda()
+        par_dev = torch.zeros((B, 3), dtype=torch.int32, device="cuda")
+        mean_dev = torch.from_numpy(mean).cuda() if mean is not None else None
+        out_dev = torch.empty((B, D, S, S), device="cuda")
+        tm = drv.timer()
+        for rep in range(3):
+            if rep == 1:
+                tm.start()
+            for _ in range(10 if rep else 2):
+                corpus.transform_batch(out_dev, raw_dev, mean_dev, par_dev, B, D, H, H, crop, scale)
+        tm.stop()
+        t_ms = tm.elapsed_ms() / 20
+        t_bytes = B * D * S * S * (1 + 4 + (4 if mean is not None else 0))
+        pipeline = {"raw_bytes_per_batch": int(B * D * H * H), "float_bytes_per_batch": int(B * D * S * S * 4),
+                    "transform_kernel_ms": round(t_ms, 4), "transform_kernel_GBps": round(t_bytes / t_ms / 1e6, 1)}
+        del raw_dev, out_dev
+
     def step():
+        if pipeline is not None:
+            cp.consume(net.input_ptr(), net.labels_ptr())
         net.forward()
         net.backward()
+        if pipeline is not None:
+            feed()
 
     for _ in range(args.warmup):
         step()
@@ -185,6 +233,7 @@ def net_iteration(args, torch, np):
         "config": {"workload": "%s: fwd+bwd+SGD, batch %d, %dx%dx%d inputs, %d classes%s" % (
             args.workload, B, D, S, S, classes, ", conv2/4/5 in 2 groups" if args.workload == "caffenet" else "")},
         "final_loss_per_image": round(float(loss), 5),
+        **({"input_pipeline": pipeline} if pipeline is not None else {}),
     }
 
 
@@ -197,6 +246,9 @@ def main():
                     help="a single conv layer (default: AlexNet conv2, the headline config) or a whole training "
                          "iteration of LeNet (b=64) / CaffeNet (b=256, grouped conv2/4/5)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--input-pipeline", action="store_true",
+                    help="lenet/caffenet: feed every iteration through the input pipeline (raw bytes in host memory "
+                         "-> pinned staging -> asynchronous upload -> transform kernel)")
     ap.add_argument("--unfused", action="store_true", help="staged forward (GEMM, remap, bias) and separate bias gradient")
     ap.add_argument("--path", type=int, default=-1, choices=[-1, 0, 1, 2, 3],
                     help="conv path level: 0 separate passes, 1 fused epilogues, 2 direct data gradient, 3 all "

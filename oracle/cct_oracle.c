@@ -520,3 +520,29 @@ void cct_oracle_fc_backward(float *in_grad, float *model_grad, float *bias_grad,
     cct_oracle_sgemm_new(CCT_NO_TRANS, CCT_NO_TRANS, B, I, O, 1.0f, out_grad, model, 0.0f, in_grad);
   cct_oracle_sgemm_new(CCT_TRANS, CCT_NO_TRANS, O, I, B, 1.0f, out_grad, in, 0.0f, model_grad);
 }
+
+/* ------------------------------------------------------------------------------------
+ * One image through the input transform.  Restates Corpus::process_image
+ * (src/parser/corpus.h:262-333) for byte data: with a crop, the window starting at
+ * (h_off, w_off) is copied, columns reversed when `mirror` is set; element =
+ * (float(byte) - mean[same source index]) * scale.  Without a crop the whole image is converted.
+ * The caller supplies h_off / w_off / mirror (the reference draws them with rand()).
+ * ---------------------------------------------------------------------------------- */
+void cct_oracle_process_image(float *out, const unsigned char *data, const float *mean, int channels,
+                              int height, int width, int crop_size, int h_off, int w_off, int mirror,
+                              float scale) {
+  if (crop_size > 0) {
+    for (int c = 0; c < channels; ++c)
+      for (int h = 0; h < crop_size; ++h)
+        for (int w = 0; w < crop_size; ++w) {
+          const int data_index = (c * height + h + h_off) * width + w + w_off;
+          const int top_index = mirror ? (c * crop_size + h) * crop_size + (crop_size - 1 - w)
+                                       : (c * crop_size + h) * crop_size + w;
+          const float e = (float)data[data_index];
+          out[top_index] = (e - (mean ? mean[data_index] : 0.0f)) * scale;
+        }
+  } else {
+    const long n = (long)channels * height * width;
+    for (long i = 0; i < n; ++i) out[i] = ((float)data[i] - (mean ? mean[i] : 0.0f)) * scale;
+  }
+}

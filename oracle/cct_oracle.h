@@ -25,6 +25,8 @@
  *   relu, maxpool, dropout, softmax   reference fixtures (relu_*, pooling_*, dropout_*, softmax_*)
  *   lrn_forward/backward  reference fixtures lrn_* at 1e-3 (the fixtures were produced by a
  *                         build using an approximate pow; this oracle uses exact powf)
+ *   process_image         numpy slicing formulation (window slice, [..., ::-1] for the mirror) on
+ *                         random shapes; the reference holds no fixture for it
  *   fillers (mt19937 streams)         not restated; configs inject their own tensors
  */
 #ifndef CCT_ORACLE_H
@@ -136,6 +138,11 @@ void cct_oracle_fc_forward(float *out, const float *in, const float *model, cons
 void cct_oracle_fc_backward(float *in_grad, float *model_grad, float *bias_grad, const float *in,
                             const float *model, const float *out_grad, int B, int I, int O,
                             int need_in_grad);
+
+/* --- input transform (Corpus::process_image, src/parser/corpus.h:262-333) ---------- */
+void cct_oracle_process_image(float *out, const unsigned char *data, const float *mean, int channels,
+                              int height, int width, int crop_size, int h_off, int w_off, int mirror,
+                              float scale);
 
 #ifdef __cplusplus
 }

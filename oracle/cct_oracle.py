@@ -95,6 +95,8 @@ def lib():
     L.cct_oracle_fc_forward.argtypes = [_f32p, _f32p, _f32p, C.c_void_p, i, i, i]
     L.cct_oracle_fc_backward.argtypes = [C.c_void_p, _f32p, C.c_void_p, _f32p, _f32p, _f32p,
                                          i, i, i, i]
+    L.cct_oracle_process_image.argtypes = [_f32p, np.ctypeslib.ndpointer(dtype=np.uint8, flags="C_CONTIGUOUS"),
+                                           C.c_void_p, i, i, i, i, i, i, i, f]
     _lib = L
     return L
 
@@ -353,3 +355,17 @@ def fc_backward(x, model, out_grad, need_in_grad=True, bias_term=True):
     lib().cct_oracle_fc_backward(_vp(in_grad), model_grad, _vp(bias_grad), x, model, out_grad,
                                  B, I, O, int(need_in_grad))
     return in_grad, model_grad, bias_grad
+
+
+def transform_batch(raw, mean, crop_size, params, scale):
+    """Corpus::process_image over a batch: raw uint8 [b][c][h][w], mean [c][h][w] or None,
+    params int [b][3] = (h_off, w_off, mirror)."""
+    raw = np.ascontiguousarray(raw, dtype=np.uint8)
+    b, c, h, w = raw.shape
+    rows, cols = (crop_size, crop_size) if crop_size else (h, w)
+    out = np.empty((b, c, rows, cols), np.float32)
+    mean = None if mean is None else _f32(mean)
+    for i_ in range(b):
+        ho, wo, mi = (int(v) for v in params[i_]) if crop_size else (0, 0, 0)
+        lib().cct_oracle_process_image(out[i_], raw[i_], _vp(mean), c, h, w, crop_size, ho, wo, mi, scale)
+    return out

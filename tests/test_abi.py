@@ -35,6 +35,14 @@ def test_library_exports_every_declared_symbol():
     for n in nnames:
         assert hasattr(lib, n), "missing export: " + n
     assert sorted(nets.NET_PROTOTYPES) == nnames
+    # input pipeline
+    from caffecontroll_amd import corpus
+    cnames = sorted(set(_declared_symbols("cct_corpus.h", "cct_corpus_") + _declared_symbols("cct_corpus.h", "cct_lmdb_") +
+                        _declared_symbols("cct_corpus.h", "cct_hip_") + ["cct_datum_parse", "cct_mean_read"]))
+    assert len(cnames) >= 16
+    for n in cnames:
+        assert hasattr(lib, n), "missing export: " + n
+    assert sorted(corpus.CORPUS_PROTOTYPES) == cnames
 
 
 def test_struct_layouts_match_reference_headers():
