@@ -2,10 +2,11 @@
 (DeepNet::train_network / load_and_train_network, src/DeepNet.h:2030-2215, 2386-2445), driven by
 the fields of a solver prototxt (`prototxt.solver_from_prototxt`).
 
-Mini-batches come from any iterable of (images, labels) host arrays -- float32 [b][d][n][n] and one
-float label per image, what Corpus::LoadLmdbData leaves in its two cubes
-(src/parser/corpus.h:111-161); the iterable is restarted when it runs out (the reference wraps
-around the training set and counts an epoch).  Reading LMDB files is not part of this module.
+Mini-batches come from a `corpus.Corpus` opened on an LMDB (raw bytes uploaded asynchronously and
+transformed on the device, one batch ahead of the computation) or from any iterable of
+(images, labels) host arrays -- float32 [b][d][n][n] and one float label per image, what
+Corpus::LoadLmdbData leaves in its two cubes (src/parser/corpus.h:111-161); the iterable is
+restarted when it runs out (the reference wraps around the training set and counts an epoch).
 """
 import ctypes as C
 import time
@@ -49,6 +50,28 @@ def batch_accuracy(net, labels):
     _d2h(lib, prob, ptr)
     prob = prob.reshape(net.batch, -1)
     return int(np.count_nonzero(prob.argmax(axis=1) == np.asarray(labels).reshape(-1).astype(np.int64)))
+
+
+class _CorpusSource:
+    """Feeds the network from a `corpus.Corpus` on an LMDB: one batch is always uploading while
+    the previous one trains."""
+
+    def __init__(self, net, cp):
+        if (cp.info.batch, cp.info.channels, cp.info.out_rows, cp.info.out_cols) != (net.batch, net.depth, net.size, net.size):
+            raise ValueError("the corpus produces %dx%dx%dx%d batches, the network takes %dx%dx%dx%d" % (
+                cp.info.batch, cp.info.channels, cp.info.out_rows, cp.info.out_cols, net.batch, net.depth, net.size, net.size))
+        self.net, self.cp = net, cp
+        self.epoch_of_next = cp.load_next()
+
+    def next_into_network(self):
+        """Transform the batch in flight into the input cube, start loading the one after it;
+        returns (epoch, labels on the host)."""
+        epoch = self.epoch_of_next
+        self.cp.consume(self.net.input_ptr(), self.net.labels_ptr())
+        self.epoch_of_next = self.cp.load_next()
+        labels = np.empty(self.net.batch, np.float32)
+        _d2h(_lib.load(), labels, self.net.labels_ptr())
+        return epoch, labels
 
 
 def _cycle(batches):
@@ -115,14 +138,19 @@ def train(net, solver, control, batches, test_batches=None, output_model_file=No
     test_interval, max_iter = control.get("test_interval", 0), control["max_iter"]
     reports, loss, acc = [], 0.0, 0.0
     window = 0
-    source = _cycle(batches)
+    from .corpus import Corpus
+    from_corpus = isinstance(batches, Corpus)
+    source = _CorpusSource(net, batches) if from_corpus else _cycle(batches)
     net.set_train(True)
     if start_iter:
         net.set_iter(start_iter)
     t0 = time.time()
     for it in range(start_iter, max_iter):
-        epoch, images, labels = next(source)
-        upload_batch(net, images, labels)
+        if from_corpus:
+            epoch, labels = source.next_into_network()
+        else:
+            epoch, images, labels = next(source)
+            upload_batch(net, images, labels)
         net.forward()
         loss += net.loss() / net.batch
         acc += batch_accuracy(net, labels) / float(net.batch)

@@ -145,3 +145,44 @@ def test_lmdb_fed_loader_wraps_around(oracle, tmp_path):
     with pytest.raises(CctHipError, match="record 1"):
         cp.load_next()
     cp.close()
+
+
+def test_training_loop_fed_from_lmdb(tmp_path):
+    """solver prototxt + network prototxt + LMDB -> training: the loop of `caffe-ct train`."""
+    from caffecontroll_amd import corpus, prototxt as P, solver as S
+    driver()
+    rng = np.random.default_rng(21)
+    n, c, h = 40, 1, 14
+    labels = rng.integers(0, 4, n)
+    px = rng.integers(0, 40, (n, c, h, h), dtype=np.uint8)
+    for i, y in enumerate(labels):   # the class decides the bright quadrant
+        px[i, :, (y // 2) * 7:(y // 2) * 7 + 7, (y % 2) * 7:(y % 2) * 7 + 7] += 200
+    W.write_lmdb(str(tmp_path / "train_lmdb"), [(b"%08d" % i, W.datum(c, h, h, px[i].tobytes(), int(labels[i])))
+                                                for i in range(n)])
+    (tmp_path / "net.prototxt").write_text("""
+      name: "quadrants"
+      layer { name: "data" type: "Data" top: "data" top: "label" include { phase: TRAIN }
+              transform_param { scale: 0.00390625 crop_size: 12 mirror: false }
+              data_param { source: "train_lmdb" batch_size: 8 backend: LMDB } }
+      layer { name: "conv1" type: "Convolution" bottom: "data" top: "conv1"
+              convolution_param { num_output: 4 kernel_size: 3 weight_filler { type: "xavier" } } }
+      layer { name: "relu1" type: "ReLU" bottom: "conv1" top: "conv1" }
+      layer { name: "pool1" type: "Pooling" bottom: "conv1" top: "pool1" pooling_param { kernel_size: 2 stride: 2 } }
+      layer { name: "ip1" type: "InnerProduct" bottom: "pool1" top: "ip1"
+              inner_product_param { num_output: 4 weight_filler { type: "xavier" } } }
+      layer { name: "loss" type: "SoftmaxWithLoss" bottom: "ip1" bottom: "label" top: "loss" }
+    """)
+    (tmp_path / "solver.prototxt").write_text(
+        'net: "net.prototxt"\nbase_lr: 0.1 momentum: 0.9 lr_policy: "fixed" max_iter: 30 display: 10 random_seed: 3\n')
+    sp, ctl, nd = P.load_solver(str(tmp_path / "solver.prototxt"), root=str(tmp_path))
+    cp = corpus.Corpus.open(str(tmp_path / nd.source), nd.batch_size, crop_size=nd.crop_size, scale=nd.scale,
+                            mirror=nd.mirror, phase=0, seed=1)
+    net = nd.build(depth=cp.info.channels, solver=sp)
+    lines = []
+    reports = S.train(net, sp, ctl, cp, log=lines.append)
+    assert [r[0] for r in reports] == [9, 19, 29]
+    assert reports[-1][1] < 0.5 * reports[0][1] and reports[-1][2] > 0.9
+    # 40 records, batches of 8: iteration 29 reads records 232..239 -> epoch 5
+    assert any(l.startswith("Training Status Report (Epoch 5 / Mini-batch iter 29)") for l in lines)
+    net.close()
+    cp.close()
