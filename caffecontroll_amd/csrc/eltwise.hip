@@ -201,6 +201,128 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_kernel(float *__restrict__ ig
   ig[e] = acc;
 }
 
+// Plane-tiled variants: a workgroup owns `pp` consecutive (image, channel) planes, brings what the
+// gathers read into LDS with contiguous 16-byte loads (forward: the input planes; backward: the
+// output gradient and argmax planes; several loads in flight per lane) and writes contiguous
+// results, so HBM sees every byte once and the strided / repeated accesses hit LDS.  Same scan
+// orders as the kernels above, hence the same bits.
+constexpr int kPoolLdsWords = 8192;  // 32 KB
+typedef float pool_f4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef int pool_i4u __attribute__((ext_vector_type(4), aligned(4)));
+
+// dst[0..n) (LDS) = src[0..n) (global, 4-byte aligned): 16-byte loads, UNR of them in flight per lane
+template <typename V4, typename T, int UNR>
+__device__ __forceinline__ void pool_stage(T *dst, const T *__restrict__ src, uint32_t n) {
+  const uint32_t n4 = n >> 2;
+  for (uint32_t base = 0; base < n4; base += TPB * UNR) {
+    V4 v[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const uint32_t q = base + u * TPB + threadIdx.x;
+      if (q < n4) v[u] = *reinterpret_cast<const V4 *>(src + 4 * q);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const uint32_t q = base + u * TPB + threadIdx.x;
+      if (q < n4) {
+        dst[4 * q] = v[u][0]; dst[4 * q + 1] = v[u][1]; dst[4 * q + 2] = v[u][2]; dst[4 * q + 3] = v[u][3];
+      }
+    }
+  }
+  if (threadIdx.x < (n & 3u)) dst[4 * n4 + threadIdx.x] = src[4 * n4 + threadIdx.x];
+}
+
+__global__ __launch_bounds__(TPB) void maxpool_fwd_plane_kernel(float *__restrict__ out, int *__restrict__ idx,
+                                                                const float *__restrict__ in, cct_pool_args a,
+                                                                uint32_t planes, int pp, FastDiv div_oc,
+                                                                FastDiv div_oplane) {
+  __shared__ float tile[kPoolLdsWords];
+  const uint32_t p0 = blockIdx.x * (uint32_t)pp;
+  const uint32_t np = min((uint32_t)pp, planes - p0);
+  const uint32_t iplane = (uint32_t)(a.iR * a.iC), oplane = (uint32_t)(a.oR * a.oC);
+  pool_stage<pool_f4u, float, 8>(tile, in + (size_t)p0 * iplane, np * iplane);
+  __syncthreads();
+  for (uint32_t i = threadIdx.x; i < np * oplane; i += TPB) {
+    const uint32_t pl = fdiv(i, div_oplane), e = i - pl * oplane;
+    const int ph = (int)fdiv(e, div_oc), pw = (int)e - ph * a.oC;
+    const float *t = tile + pl * iplane;
+    const int h0 = ph * a.stride, w0 = pw * a.stride;
+    const int h1 = min(h0 + a.kernel_size, a.iR), w1 = min(w0 + a.kernel_size, a.iC);
+    float best = -FLT_MAX;
+    int besti = 0;
+    for (int h = h0; h < h1; ++h)
+      for (int w = w0; w < w1; ++w) {
+        const float v = t[h * a.iC + w];
+        if (v > best) {
+          best = v;
+          besti = h * a.iC + w;
+        }
+      }
+    out[(size_t)p0 * oplane + i] = best;
+    idx[(size_t)p0 * oplane + i] = besti;
+  }
+}
+
+template <bool TWO_BY_TWO>
+__global__ __launch_bounds__(TPB) void maxpool_bwd_plane_kernel(float *__restrict__ ig, const float *__restrict__ og,
+                                                                const int *__restrict__ idx, cct_pool_args a,
+                                                                uint32_t planes, int pp, FastDiv div_ic,
+                                                                FastDiv div_iplane, FastDiv div_s) {
+  __shared__ float tog[kPoolLdsWords / 2];
+  __shared__ int tidx[kPoolLdsWords / 2];
+  const uint32_t p0 = blockIdx.x * (uint32_t)pp;
+  const uint32_t np = min((uint32_t)pp, planes - p0);
+  const uint32_t iplane = (uint32_t)(a.iR * a.iC), oplane = (uint32_t)(a.oR * a.oC);
+  pool_stage<pool_f4u, float, 4>(tog, og + (size_t)p0 * oplane, np * oplane);
+  pool_stage<pool_i4u, int, 4>(tidx, idx + (size_t)p0 * oplane, np * oplane);
+  __syncthreads();
+  const int k = a.kernel_size;
+  for (uint32_t i = threadIdx.x; i < np * iplane; i += TPB) {
+    const uint32_t pl = fdiv(i, div_iplane), me = i - pl * iplane;
+    const int h = (int)fdiv(me, div_ic), w = (int)me - h * a.iC;
+    const int ph_lo = h < k ? 0 : (int)fdiv((uint32_t)(h - k), div_s) + 1, ph_hi = min((int)fdiv((uint32_t)h, div_s), a.oR - 1);
+    const int pw_lo = w < k ? 0 : (int)fdiv((uint32_t)(w - k), div_s) + 1, pw_hi = min((int)fdiv((uint32_t)w, div_s), a.oC - 1);
+    const float *g = tog + pl * oplane;
+    const int *x = tidx + pl * oplane;
+    float acc = 0.0f;
+    if (TWO_BY_TWO) {
+      // kernel <= 2*stride: at most two windows per direction; clamped positions keep the reads branch-free
+      const int r0 = ph_lo * a.oC, r1 = min(ph_lo + 1, a.oR - 1) * a.oC;
+      const int c0 = pw_lo, c1 = min(pw_lo + 1, a.oC - 1);
+      const int x00 = x[r0 + c0], x01 = x[r0 + c1], x10 = x[r1 + c0], x11 = x[r1 + c1];
+      const float g00 = g[r0 + c0], g01 = g[r0 + c1], g10 = g[r1 + c0], g11 = g[r1 + c1];
+      const bool row1 = ph_lo + 1 <= ph_hi, col1 = pw_lo + 1 <= pw_hi, any = ph_lo <= ph_hi && pw_lo <= pw_hi;
+      if (any && x00 == (int)me) acc += g00;
+      if (any && col1 && x01 == (int)me) acc += g01;
+      if (any && row1 && x10 == (int)me) acc += g10;
+      if (any && row1 && col1 && x11 == (int)me) acc += g11;
+    } else {
+      for (int ph = ph_lo; ph <= ph_hi; ++ph)
+        for (int pw = pw_lo; pw <= pw_hi; ++pw)
+          if (x[ph * a.oC + pw] == (int)me) acc += g[ph * a.oC + pw];
+    }
+    ig[(size_t)p0 * iplane + i] = acc;
+  }
+}
+
+// CCT_HIP_POOL_PLANE=1 takes the plane-tiled kernels at any size (used by the tests on small shapes)
+static bool force_pool_plane() {
+  const char *e = getenv("CCT_HIP_POOL_PLANE");
+  return e && e[0] == '1';
+}
+
+// planes per workgroup: enough elements to keep 256 lanes busy for a few rounds, within the LDS tile
+static int pool_planes_per_block(size_t plane_words, size_t work_words, size_t planes) {
+  // small tensors are launch-bound; the one-lane-per-element kernels finish them sooner
+  if (planes * (plane_words > work_words ? plane_words : work_words) < (1u << 20) && !force_pool_plane()) return 0;
+  if (plane_words == 0 || plane_words > (size_t)kPoolLdsWords) return 0;
+  size_t pp = kPoolLdsWords / plane_words;
+  const size_t want = (2048 + work_words - 1) / work_words;  // ~8 elements per lane
+  if (pp > want) pp = want;
+  if (pp > planes) pp = planes;
+  return (int)(pp < 1 ? 1 : pp);
+}
+
 // ---- LRN (across channels) -----------------------------------------------------------------------
 // forward: one lane per element sums the squares of its window [ch-w, ch+w] (clipped to the depth)
 // in ascending channel order, then scale = 1 + alpha/size * sum and out = in / scale^beta; denoms
@@ -577,6 +699,14 @@ int cct_hip_maxpool_forward(float *out, const float *in, const cct_pool_args *a)
   if (rc) return rc;
   const size_t total = (size_t)a->D * a->B * a->oR * a->oC;
   if (total == 0) return 0;
+  const size_t planes = (size_t)a->D * a->B, iplane = (size_t)a->iR * a->iC, oplane = (size_t)a->oR * a->oC;
+  if (const int pp = pool_planes_per_block(iplane, oplane, planes)) {
+    hipLaunchKernelGGL(maxpool_fwd_plane_kernel, dim3((uint32_t)((planes + pp - 1) / pp)), dim3(TPB), 0, ctx().stream,
+                       out, a->max_index, in, *a, (uint32_t)planes, pp, make_fastdiv(a->oC),
+                       make_fastdiv((uint32_t)oplane));
+    CCT_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL(maxpool_fwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, out,
                      a->max_index, in, *a, (uint32_t)total, make_fastdiv(a->oC), make_fastdiv(a->oR));
   CCT_LAUNCH_CHECK();
@@ -590,6 +720,20 @@ int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_po
   if (rc) return rc;
   const size_t total = (size_t)a->D * a->B * a->iR * a->iC;
   if (total == 0) return 0;
+  const size_t planes = (size_t)a->D * a->B, iplane = (size_t)a->iR * a->iC, oplane = (size_t)a->oR * a->oC;
+  if (const int pp = pool_planes_per_block(2 * oplane, iplane, planes)) {
+    const dim3 grid((uint32_t)((planes + pp - 1) / pp));
+    if (a->kernel_size <= 2 * a->stride)
+      hipLaunchKernelGGL(maxpool_bwd_plane_kernel<true>, grid, dim3(TPB), 0, ctx().stream, in_grad, out_grad,
+                         a->max_index, *a, (uint32_t)planes, pp, make_fastdiv(a->iC), make_fastdiv((uint32_t)iplane),
+                         make_fastdiv(a->stride));
+    else
+      hipLaunchKernelGGL(maxpool_bwd_plane_kernel<false>, grid, dim3(TPB), 0, ctx().stream, in_grad, out_grad,
+                         a->max_index, *a, (uint32_t)planes, pp, make_fastdiv(a->iC), make_fastdiv((uint32_t)iplane),
+                         make_fastdiv(a->stride));
+    CCT_LAUNCH_CHECK();
+    return 0;
+  }
   if (a->kernel_size <= 2 * a->stride)
     hipLaunchKernelGGL(maxpool_bwd_kernel<true>, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad,
                        out_grad, a->max_index, *a, (uint32_t)total, make_fastdiv(a->iC), make_fastdiv(a->iR));

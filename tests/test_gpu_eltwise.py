@@ -32,8 +32,17 @@ def test_relu_fixture_and_oracle(oracle):
     assert torch.cuda.is_available()
 
 
-@pytest.mark.parametrize("cfg", [(5, 3, 10, 4, 2), (2, 4, 13, 3, 2), (3, 2, 24, 2, 2), (2, 3, 55, 3, 2), (1, 2, 7, 3, 1)])
-def test_maxpool_bit_exact(oracle, cfg):
+@pytest.mark.parametrize("cfg", [(5, 3, 10, 4, 2), (2, 4, 13, 3, 2), (3, 2, 24, 2, 2), (2, 3, 55, 3, 2), (1, 2, 7, 3, 1),
+                                 # several planes per workgroup with a partial last group; planes too large
+                                 # for the LDS-tiled kernels (forward only, both, window wider than 2 strides)
+                                 (7, 11, 13, 3, 2), (1, 2, 100, 3, 2), (1, 1, 150, 2, 2), (1, 1, 140, 5, 2)])
+@pytest.mark.parametrize("plane_tiled", [False, True])
+def test_maxpool_bit_exact(oracle, cfg, plane_tiled, monkeypatch):
+    # small tensors take the one-lane-per-element kernels unless the plane-tiled ones are forced
+    if plane_tiled:
+        monkeypatch.setenv("CCT_HIP_POOL_PLANE", "1")
+    else:
+        monkeypatch.delenv("CCT_HIP_POOL_PLANE", raising=False)
     B, D, n, k, s = cfg
     rng = np.random.default_rng(sum(cfg))
     if cfg == (5, 3, 10, 4, 2):
