@@ -80,14 +80,20 @@ struct Tile {
   static constexpr int PR = 8;  // pad of row-contiguous LDS rows
   static_assert(BK % 8 == 0, "BK must hold whole k-groups");
   static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile is made of 32x32 MFMA tiles");
-  static_assert((BM * BK / 4) % THREADS == 0 && (BN * BK / 4) % THREADS == 0, "loader coverage");
+  static_assert((BM * BK / 4) % 64 == 0 && (BN * BK / 4) % 64 == 0, "whole wavefronts load an operand tile");
 };
 
 template <class T, bool KC, int ROWS>
 struct OperandLayout {
   // floats per LDS stage
   static constexpr int SIZE = KC ? ROWS * (T::BK + T::PK) : T::BK * (ROWS + T::PR);
-  static constexpr int NV = ROWS * T::BK / 4 / T::THREADS;  // f4 per lane per stage
+  static constexpr int TOTAL = ROWS * T::BK / 4;                        // f4 per stage
+  static constexpr int NV = (TOTAL + T::THREADS - 1) / T::THREADS;      // f4 per lane per stage
+  // Slot i of a lane exists when its f4 index is inside the tile; only the last slot can be partial
+  // (a 96-row tile loaded by 256 lanes: 1.5 f4 per lane), and then whole wavefronts are in or out.
+  static __device__ __forceinline__ bool active(int i, int tid) {
+    return (i + 1) * T::THREADS <= TOTAL || tid + i * T::THREADS < TOTAL;
+  }
 };
 
 // global -> registers for one operand tile (rows x BK) starting at (row0, k0)
@@ -95,9 +101,11 @@ template <class T, bool KC, int ROWS>
 __device__ __forceinline__ void load_tile(f4 *__restrict__ r,
                                           const float *__restrict__ g, int ld, int row0, int k0,
                                           int row_lim, int k_lim, int vec, int tid) {
-  constexpr int NV = OperandLayout<T, KC, ROWS>::NV;
+  using L = OperandLayout<T, KC, ROWS>;
+  constexpr int NV = L::NV;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
+    if (!L::active(i, tid)) continue;
     const int f = tid + i * T::THREADS;
     if (KC) {
       const int row = f / (T::BK / 4), kq = f % (T::BK / 4);
@@ -112,9 +120,11 @@ __device__ __forceinline__ void load_tile(f4 *__restrict__ r,
 template <class T, bool KC, int ROWS>
 __device__ __forceinline__ void store_tile(float *__restrict__ lds, const f4 *__restrict__ r,
                                            int tid) {
-  constexpr int NV = OperandLayout<T, KC, ROWS>::NV;
+  using L = OperandLayout<T, KC, ROWS>;
+  constexpr int NV = L::NV;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
+    if (!L::active(i, tid)) continue;
     const int f = tid + i * T::THREADS;
     if (KC) {
       const int row = f / (T::BK / 4), kq = f % (T::BK / 4);
@@ -177,14 +187,18 @@ __device__ __forceinline__ void mfma_group(v16f (&acc)[TM][TN], const f4 (&fa)[T
 // not a multiple of 4 is assembled from clamped dword loads.
 template <class T, bool KC, int ROWS>
 struct FastLoader {
-  static constexpr int NV = OperandLayout<T, KC, ROWS>::NV;
+  using L = OperandLayout<T, KC, ROWS>;
+  static constexpr int NV = L::NV;
   const float *p[NV];
   int lim[NV];  // row-contiguous scalar mode: element j of the f4 sits at offset min(j, lim)
   size_t step;  // floats per K step
+  bool last_active;  // whether this lane owns the (possibly partial) last slot
   __device__ __forceinline__ void init(const float *g, int ld, int row0, int k0, int rows_total, int tid) {
+    last_active = L::active(NV - 1, tid);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int f = tid + i * T::THREADS;
+      // lanes without the last slot point it at their first f4: valid memory, never loaded
+      const int f = L::active(i, tid) ? tid + i * T::THREADS : tid;
       if (KC) {
         const int row = min(row0 + f / (T::BK / 4), rows_total - 1), kq = f % (T::BK / 4);
         p[i] = g + (size_t)row * ld + k0 + kq * 4;
@@ -206,6 +220,7 @@ struct FastLoader {
   __device__ __forceinline__ void load(f4 *__restrict__ r, int vec) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
+      if (i == NV - 1 && !last_active) continue;
       if (vec && (KC || lim[i] == 3)) {
         r[i] = *reinterpret_cast<const f4u *>(p[i]);
       } else if (KC) {
@@ -454,6 +469,9 @@ typedef Tile<256, 128, 16, 2, 2> TileL;
 typedef Tile<128, 256, 16, 2, 2> TileLT;  // same wave work as TileL with the long side along N
 typedef Tile<128, 128, 16, 2, 2> TileM;
 typedef Tile<64, 64, 16, 2, 2> TileS;
+// 96 rows (AlexNet conv1's 96 output maps would waste a quarter of a 128-row tile): the four
+// wavefronts sit side by side, each owning 96 x 32
+typedef Tile<96, 128, 16, 1, 4> TileR;
 
 template <class T>
 static int launch_cfg(GemmArgs &g, bool a_kc, bool b_kc, int splits, hipStream_t st) {
@@ -503,14 +521,14 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
   const int bk = 16;
   struct Shape { int bm, bn, occ, k0; double eff; };
-  static const Shape shapes[4] = {{256, 128, 2, 32, 1.0}, {128, 128, 3, 8, 0.96}, {64, 64, 6, 8, 0.80},
-                                  {128, 256, 2, 32, 1.0}};  // L, M, S, LT
+  static const Shape shapes[5] = {{256, 128, 2, 32, 1.0}, {128, 128, 3, 8, 0.96}, {64, 64, 6, 8, 0.80},
+                                  {128, 256, 2, 32, 1.0}, {96, 128, 3, 8, 0.90}};  // L, M, S, LT, R
   const double cu_rate = 0.8 * 157.3e12 / 256.0, hbm_rate = 4.0e12;
   int cfg = 1, splits = 1, kchunk = g.K > 0 ? g.K : bk;
   double best = 1e30;
   static const int forced = [] { const char *e = getenv("CCT_HIP_GEMM_TILE"); return e ? atoi(e) : -1; }();
-  for (int c = 0; c < 4; ++c) {
-    if (forced >= 0 && forced <= 3 && c != forced) continue;  // tuning override, read once
+  for (int c = 0; c < 5; ++c) {
+    if (forced >= 0 && forced <= 4 && c != forced) continue;  // tuning override, read once
     const Shape &sh = shapes[c];
     const long tiles = (long)((M + sh.bm - 1) / sh.bm) * ((N + sh.bn - 1) / sh.bn);
     const long slots = (long)sh.occ * cus;
@@ -547,7 +565,8 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   int rc = cfg == 0   ? launch_cfg<TileL>(g, a_kc, b_kc, splits, st)
            : cfg == 1 ? launch_cfg<TileM>(g, a_kc, b_kc, splits, st)
            : cfg == 2 ? launch_cfg<TileS>(g, a_kc, b_kc, splits, st)
-                      : launch_cfg<TileLT>(g, a_kc, b_kc, splits, st);
+           : cfg == 3 ? launch_cfg<TileLT>(g, a_kc, b_kc, splits, st)
+                      : launch_cfg<TileR>(g, a_kc, b_kc, splits, st);
   if (rc) return rc;
   if (splits > 1) {
     CCT_REQUIRE((size_t)M * N < (1ull << 31), "sgemm: split-K result too large");
