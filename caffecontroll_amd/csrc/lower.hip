@@ -4,8 +4,8 @@
 //
 // One workgroup owns (image bi, band of RB output rows, slab of DS input channels).  It stages
 // the zero-padded input window of that band in LDS with coalesced row reads, then streams out
-// the lowered rows: consecutive lanes write consecutive addresses of one lowered row, each
-// lowered element is written exactly once, padding zeros come from the LDS tile so the store
+// the lowered rows with 16-byte stores: consecutive lanes write consecutive addresses of one lowered
+// row, each lowered element is written exactly once, padding zeros come from the LDS tile so the store
 // loop has no bounds tests.  The per-row-position LDS offsets (the (dd,kr,kc) decomposition)
 // are tabulated once per workgroup.
 //
@@ -31,7 +31,8 @@ struct LowerParams {
 constexpr int LOWER_MAX_THREADS = 512;  // block size is chosen per launch (multiple of 64)
 
 // dynamic LDS: [DS*TH*TW floats tile][seglen uint16 offsets]
-template <bool VEC4>
+typedef float lower_f4u __attribute__((ext_vector_type(4), aligned(4)));
+
 __global__ __launch_bounds__(LOWER_MAX_THREADS) void lower_kernel(float *__restrict__ dst,
                                                               const float *__restrict__ src,
                                                               const LowerParams P) {
@@ -108,41 +109,37 @@ __global__ __launch_bounds__(LOWER_MAX_THREADS) void lower_kernel(float *__restr
   }
   __syncthreads();
 
-  // (3) stream the lowered rows
+  // (3) stream the lowered rows.  A lane owns a unit -- 4 consecutive positions of a lowered row
+  // (one 16-byte store; dword alignment is all such a store needs, so row lengths like 363 cost
+  // nothing) or one of the seg % 4 positions left over -- and a group of output columns, and walks
+  // over the band.  Short rows (few units) are spread over several column groups so that the
+  // whole workgroup stores.
   float *out_band = dst + ((size_t)bi * P.m + r0) * P.m * P.rowlen + (size_t)dd0 * P.k * P.k;
-  if (VEC4) {
-    // seg % 4 == 0 and every segment start is 16-byte aligned: a lane owns 4 consecutive row
-    // positions and walks over the output positions of the band
-    const int nq = seg >> 2;
-    for (int q = tid; q < nq; q += T) {
-      const int o0 = offs[4 * q], o1 = offs[4 * q + 1], o2 = offs[4 * q + 2], o3 = offs[4 * q + 3];
-      float *outq = out_band + 4 * q;
+  const int nq = seg >> 2, units = nq + (seg & 3);
+  const int groups = units < T ? min(T / units, P.m) : 1;
+  const int cpg = (P.m + groups - 1) / groups;
+  for (int wi = tid; wi < units * groups; wi += T) {
+    const int cg = groups > 1 ? wi / units : 0, u = wi - cg * units;
+    const int c_lo = cg * cpg, c_hi = min(P.m, c_lo + cpg);
+    if (u < nq) {
+      const int o0 = offs[4 * u], o1 = offs[4 * u + 1], o2 = offs[4 * u + 2], o3 = offs[4 * u + 3];
+      float *outq = out_band + 4 * u;
       for (int rl = 0; rl < rb; ++rl) {
         const float *trow = tile + rl * P.s * P.TW;
         float *orow = outq + (size_t)rl * P.m * P.rowlen;
 #pragma unroll 4
-        for (int c = 0; c < P.m; ++c) {
+        for (int c = c_lo; c < c_hi; ++c) {
           const float *t = trow + c * P.s;
-          float4 v = make_float4(t[o0], t[o1], t[o2], t[o3]);
-          *reinterpret_cast<float4 *>(orow + (size_t)c * P.rowlen) = v;
+          const lower_f4u v = {t[o0], t[o1], t[o2], t[o3]};
+          *reinterpret_cast<lower_f4u *>(orow + (size_t)c * P.rowlen) = v;
         }
       }
-    }
-  } else {
-    // general shapes: flat index over (c, j) of one band row; lanes write consecutive floats
-    const uint32_t per_row = (uint32_t)P.m * seg;
-    const bool contiguous = (ds == P.d);
-    for (int rl = 0; rl < rb; ++rl) {
-      const float *trow = tile + rl * P.s * P.TW;
-      float *orow = out_band + (size_t)rl * P.m * P.rowlen;
-      for (uint32_t e = tid; e < per_row; e += T) {
-        const uint32_t c = (seg == P.seglen) ? fdiv(e, P.div_seg) : e / (uint32_t)seg;
-        const uint32_t j = e - c * seg;
-        const float v = trow[c * P.s + offs[j]];
-        if (contiguous)
-          orow[e] = v;
-        else
-          orow[(size_t)c * P.rowlen + j] = v;
+    } else {
+      const int j = 4 * nq + (u - nq), o = offs[j];
+      for (int rl = 0; rl < rb; ++rl) {
+        const float *trow = tile + rl * P.s * P.TW;
+        float *orow = out_band + j + (size_t)rl * P.m * P.rowlen;
+        for (int c = c_lo; c < c_hi; ++c) orow[(size_t)c * P.rowlen] = trow[c * P.s + o];
       }
     }
   }
@@ -207,31 +204,30 @@ extern "C" int cct_hip_lower_cube(float *dst, const float *src, const cct_pmap_h
   P.div_chunk = make_fastdiv(P.chunk_full);
 
   const size_t lds_bytes = lds_need(P.RB, P.DS);
-  // float4 stores need every (position, slab) segment to start 16-byte aligned and to hold a
-  // whole number of float4: k*k*DS % 4 == 0 covers both when dst itself is aligned.
-  const bool vec4 = ((uintptr_t)dst % 16 == 0) && (P.rowlen % 4 == 0) && ((P.DS * P.k * P.k) % 4 == 0) &&
-                    (P.d % P.DS == 0);
-  // block size: the multiple of 64 that wastes the fewest lanes in the store loop
-  const long units = vec4 ? P.seglen / 4 : (long)P.m * P.seglen;
+  // block size: a multiple of 64 close to a whole number of (unit, column group) work items; rows
+  // with many units take the size that wastes the fewest lanes of the last pass
+  const long units = P.seglen / 4 + P.seglen % 4;
   int threads = 256;
-  double best = 1e30;
-  for (int t = 128; t <= LOWER_MAX_THREADS; t += 64) {
-    const double waste = (double)((units + t - 1) / t * t) / (double)units;
-    if (waste < best - 1e-9 || (waste < best + 1e-9 && t <= 320)) {
-      best = waste;
-      threads = t;
+  if (units < LOWER_MAX_THREADS) {
+    // several column groups per workgroup: as many lanes as the groups use, rounded up to wavefronts
+    const long groups = LOWER_MAX_THREADS / units < P.m ? LOWER_MAX_THREADS / units : P.m;
+    threads = (int)((units * groups + 63) / 64 * 64);
+    if (threads > LOWER_MAX_THREADS) threads = LOWER_MAX_THREADS;
+    if (threads < 128) threads = 128;
+  } else {
+    double best = 1e30;
+    for (int t = 128; t <= LOWER_MAX_THREADS; t += 64) {
+      const double waste = (double)((units + t - 1) / t * t) / (double)units;
+      if (waste < best - 1e-9 || (waste < best + 1e-9 && t <= 320)) {
+        best = waste;
+        threads = t;
+      }
     }
   }
   hipStream_t st = ctx().stream;
-  if (vec4) {
-    CCT_HIP_CHECK(hipFuncSetAttribute((const void *)lower_kernel<true>,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    hipLaunchKernelGGL(lower_kernel<true>, dim3(P.nblocks), dim3(threads), lds_bytes, st, dst, src, P);
-  } else {
-    CCT_HIP_CHECK(hipFuncSetAttribute((const void *)lower_kernel<false>,
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes));
-    hipLaunchKernelGGL(lower_kernel<false>, dim3(P.nblocks), dim3(threads), lds_bytes, st, dst, src, P);
-  }
+  CCT_HIP_CHECK(hipFuncSetAttribute((const void *)lower_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)lds_bytes));
+  hipLaunchKernelGGL(lower_kernel, dim3(P.nblocks), dim3(threads), lds_bytes, st, dst, src, P);
   CCT_LAUNCH_CHECK();
   return 0;
 }
