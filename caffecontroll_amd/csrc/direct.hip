@@ -831,7 +831,17 @@ __global__ __launch_bounds__(256) void direct_reduce_kernel(float *__restrict__ 
     e -= n; dst = dst2; ws = ws2; n = n2;
   }
   float s = 0.f;
-  for (int z = 0; z < splits; ++z) s += ws[(size_t)z * n + e];
+  const float *p = ws + e;
+  int z = 0;
+  // eight partial sums in flight per lane; added in range order
+  for (; z + 8 <= splits; z += 8, p += (size_t)8 * n) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = p[(size_t)j * n];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += v[j];
+  }
+  for (; z < splits; ++z, p += n) s += *p;
   dst[e] = s;
 }
 

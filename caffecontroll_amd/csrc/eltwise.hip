@@ -100,13 +100,30 @@ __global__ __launch_bounds__(TPB) void bias_forward_flat_kernel(float *__restric
 }
 
 // ---- FC bias gradient: bias[d] = sum_b out[b][d] ------------------------------------------------
+// A workgroup owns 64 columns; its four wavefronts sum a quarter of the rows each, eight loads in
+// flight per lane, and the four partial sums are added in a fixed order.
 __global__ __launch_bounds__(TPB) void bias_backward_fc_kernel(float *__restrict__ bias,
                                                                const float *__restrict__ og, int D, int B) {
-  const int d = blockIdx.x * TPB + threadIdx.x;
-  if (d >= D) return;
+  __shared__ float part[4][64];
+  const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const int d = blockIdx.x * 64 + lane;
+  const int per = (B + 3) / 4, b0 = q * per, b1 = min(B, b0 + per);
   float s = 0.0f;
-  for (int b = 0; b < B; ++b) s += og[(size_t)b * D + d];
-  bias[d] = s;
+  if (d < D) {
+    const float *p = og + (size_t)b0 * D + d;
+    int b = b0;
+    for (; b + 8 <= b1; b += 8, p += (size_t)8 * D) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = p[(size_t)j * D];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s += v[j];
+    }
+    for (; b < b1; ++b, p += D) s += *p;
+  }
+  part[q][lane] = s;
+  __syncthreads();
+  if (q == 0 && d < D) bias[d] = ((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane];
 }
 
 // ---- ReLU ----------------------------------------------------------------------------------
@@ -655,7 +672,8 @@ int cct_hip_forward_bias(const float *bias, float *out, int fmap_size, int depth
 int cct_hip_backward_bias_fc(float *bias_grad, const float *out_grad, int D, int B) {
   CCT_ENSURE_INIT();
   CCT_REQUIRE(bias_grad && out_grad && D > 0 && B >= 0, "backward_bias_fc: bad argument");
-  hipLaunchKernelGGL(bias_backward_fc_kernel, dim3(blocks_for(D)), dim3(TPB), 0, ctx().stream, bias_grad,
+  static_assert(TPB == 256, "bias_backward_fc_kernel: four wavefronts per workgroup");
+  hipLaunchKernelGGL(bias_backward_fc_kernel, dim3((uint32_t)((D + 63) / 64)), dim3(TPB), 0, ctx().stream, bias_grad,
                      out_grad, D, B);
   CCT_LAUNCH_CHECK();
   return 0;

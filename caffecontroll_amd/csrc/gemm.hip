@@ -460,7 +460,17 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *__restrict__ 
   const uint32_t col = e - row * N;
   float s = 0.0f;
   const size_t mn = (size_t)M * N;
-  for (int z = 0; z < splits; ++z) s += ws[(size_t)z * mn + e];
+  const float *p = ws + e;
+  int z = 0;
+  // eight partial sums in flight per lane; added in slice order
+  for (; z + 8 <= splits; z += 8, p += 8 * mn) {
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = p[(size_t)j * mn];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += v[j];
+  }
+  for (; z < splits; ++z, p += mn) s += *p;
   float *c = C + (size_t)row * ldc + col;
   *c = (beta == 0.0f) ? alpha * s : alpha * s + beta * (*c);
 }
