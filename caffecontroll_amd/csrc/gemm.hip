@@ -546,9 +546,12 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
       int sp = 1, kc = g.K > 0 ? g.K : bk;
       if (pass == 1) {
         // split-K: plain epilogue only, when the tile grid alone cannot fill the device
-        if (epi != EPI_ALPHA_BETA || tiles >= slots || K < 512) break;
+        // (K slices of at least 256, or 128 when the result is small enough for a cheap reduction:
+        // those problems are bound by the latency of their few K steps, not by throughput)
+        const int min_chunk = (size_t)M * N <= 65536 ? 128 : 256;
+        if (epi != EPI_ALPHA_BETA || tiles >= slots || K < 2 * min_chunk) break;
         sp = (int)(slots / tiles);
-        if (sp > K / 256) sp = K / 256;
+        if (sp > K / min_chunk) sp = K / min_chunk;
         if (sp < 2) break;
         kc = (((K + sp - 1) / sp) + bk - 1) / bk * bk;
         sp = (K + kc - 1) / kc;
