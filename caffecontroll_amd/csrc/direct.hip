@@ -41,6 +41,7 @@ struct DirectArgs {
   const float *src;   // [batch][kc][hs][hs]
   float *dst;         // [batch][mtot][ho][ho]
   const float *bias;  // [mtot] or null
+  int relu;           // epilogue clamps at zero (ReLU of the layer that follows, folded in)
   int batch, kc, mtot, hs, ho, pad;
   int hp;             // ho + KS - 1 = hs + 2*pad: rows (and columns) of a zero-padded source image
   int pr;             // patch rows per channel
@@ -254,7 +255,10 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = m0 + a * 32 + 8 * (v / 4) + 4 * h + (v % 4);
-        if (row < g.mtot) out[(size_t)row * ho2] = acc[a][b][v] + (g.bias ? g.bias[row] : 0.f);
+        if (row < g.mtot) {
+          const float y = acc[a][b][v] + (g.bias ? g.bias[row] : 0.f);
+          out[(size_t)row * ho2] = (g.relu && !(y > 0.f)) ? 0.f : y;
+        }
       }
   }
 }
@@ -345,13 +349,13 @@ static int direct_launch_ks(const DirectArgs &g, const DirectPlan &pl, hipStream
   return set_error(CCT_HIP_EINVAL, "conv_direct: no kernel instance for tile %dx%d", pl.tmb, pl.tnb);
 }
 
-static int conv_direct(const float *wt, const float *src, float *dst, const float *bias, int batch, int kc,
+static int conv_direct(const float *wt, const float *src, float *dst, const float *bias, int relu, int batch, int kc,
                        int mtot, int hs, int ks, int pad, size_t src_img_stride, size_t dst_img_stride) {
   DirectPlan pl;
   CCT_REQUIRE(direct_plan(batch, kc, mtot, hs, ks, pad, &pl),
               "conv_direct: geometry not covered (k=%d pad=%d size=%d)", ks, pad, hs);
   DirectArgs g;
-  g.wt = wt; g.src = src; g.dst = dst; g.bias = bias;
+  g.wt = wt; g.src = src; g.dst = dst; g.bias = bias; g.relu = relu;
   g.batch = batch; g.kc = kc; g.mtot = mtot; g.hs = hs; g.pad = pad;
   g.ho = hs + 2 * pad - ks + 1;
   {
@@ -1054,11 +1058,12 @@ extern "C" int cct_hip_conv_direct_slabs(float *slabs, const float *model, int n
 
 extern "C" int cct_hip_conv_direct_forward(float *output, const float *input, const float *slabs,
                                            const float *bias, int batch, int depth, int n, int k, int padding,
-                                           int num_outputs, size_t input_image_stride, size_t output_image_stride) {
+                                           int num_outputs, size_t input_image_stride, size_t output_image_stride,
+                                           int relu) {
   CCT_ENSURE_INIT();
   if (batch <= 0) return 0;
-  return conv_direct(slabs, input, output, bias, batch, depth, num_outputs, n, k, padding, input_image_stride,
-                     output_image_stride);
+  return conv_direct(slabs, input, output, bias, relu != 0, batch, depth, num_outputs, n, k, padding,
+                     input_image_stride, output_image_stride);
 }
 
 extern "C" int cct_hip_conv_direct_backward_data(float *input_grad, const float *output_grad,
@@ -1068,7 +1073,7 @@ extern "C" int cct_hip_conv_direct_backward_data(float *input_grad, const float 
   CCT_ENSURE_INIT();
   if (batch <= 0) return 0;
   const int m = n + 2 * padding - k + 1;
-  return conv_direct(slabs, output_grad, input_grad, nullptr, batch, num_outputs, depth, m, k,
+  return conv_direct(slabs, output_grad, input_grad, nullptr, 0, batch, num_outputs, depth, m, k,
                      k - 1 - padding, output_image_stride, input_image_stride);
 }
 

@@ -45,6 +45,7 @@ struct GemmArgs {
   int fmap;         // EPI_CONV_FORWARD: columns per image
   FastDiv div_fmap;
   const float *bias;
+  int relu;         // EPI_CONV_FORWARD: clamp at zero after the bias
   int tiles_m, tiles_n;
   uint32_t ntiles;
   int a_vec, b_vec;  // operand allows aligned 16-byte global loads
@@ -339,7 +340,10 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
           float *c = g.C + (size_t)row * g.fmap;
           const float add = g.bias ? g.bias[row] : 0.0f;
 #pragma unroll
-          for (int b = 0; b < T::TN; ++b) c[coff[b]] = acc[a][b][4 * j + i] + add;
+          for (int b = 0; b < T::TN; ++b) {
+            const float y = acc[a][b][4 * j + i] + add;
+            c[coff[b]] = (g.relu && !(y > 0.0f)) ? 0.0f : y;
+          }
         }
   } else {
     const size_t rstride = (MODE == EPI_SPLITK_PARTIAL) ? (size_t)g.N : (size_t)g.ldc;
@@ -440,7 +444,8 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
         } else if (g.epi == EPI_SPLITK_PARTIAL) {
           g.ws[((size_t)kslice * g.M + row) * g.N + col_off] = x;
         } else {
-          const float y = g.bias ? x + g.bias[row] : x;
+          float y = g.bias ? x + g.bias[row] : x;
+          if (g.relu && !(y > 0.0f)) y = 0.0f;
           if (g.nt_store) __builtin_nontemporal_store(y, g.C + (size_t)row * g.fmap + col_off);
           else g.C[(size_t)row * g.fmap + col_off] = y;
         }
@@ -505,13 +510,13 @@ static int launch_cfg(GemmArgs &g, bool a_kc, bool b_kc, int splits, hipStream_t
 // (cblas Trans).
 static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha, const float *A, int lda,
                          const float *B, int ldb, float beta, float *C, int ldc, int epi, int fmap,
-                         const float *bias) {
+                         const float *bias, int relu = 0) {
   if (M <= 0 || N <= 0) return 0;
   hipStream_t st = ctx().stream;
   GemmArgs g;
   g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
   g.alpha = alpha; g.beta = beta; g.epi = epi; g.fmap = fmap > 0 ? fmap : 1;
-  g.div_fmap = make_fastdiv((uint32_t)g.fmap); g.bias = bias; g.ws = nullptr;
+  g.div_fmap = make_fastdiv((uint32_t)g.fmap); g.bias = bias; g.relu = relu; g.ws = nullptr;
   // 16-byte global loads need dword alignment only
   g.a_vec = ((uintptr_t)A % 4 == 0);
   g.b_vec = ((uintptr_t)B % 4 == 0);
@@ -627,11 +632,11 @@ extern "C" int cct_hip_sgemm_new(int TA, int TB, int M, int N, int K, float alph
 }
 
 extern "C" int cct_hip_sgemm_conv_forward(int o, int batch, int fmap, int K, const float *model,
-                                          const float *lowered, const float *bias, float *out) {
+                                          const float *lowered, const float *bias, float *out, int relu) {
   CCT_ENSURE_INIT();
   CCT_REQUIRE(o > 0 && batch > 0 && fmap > 0 && K > 0, "sgemm_conv_forward: non-positive dimension");
   CCT_REQUIRE(model && lowered && out, "sgemm_conv_forward: null matrix");
   CCT_REQUIRE((size_t)batch * fmap < (1ull << 31), "sgemm_conv_forward: too many output positions");
   return gemm_rowmajor(true, true, o, batch * fmap, K, 1.0f, model, K, lowered, K, 0.0f, out, batch * fmap,
-                       EPI_CONV_FORWARD, fmap, bias);
+                       EPI_CONV_FORWARD, fmap, bias, relu != 0);
 }

@@ -179,6 +179,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     views_ = true;
   }
   void set_fused(bool on) { set_path(on ? default_path_ : PATH_STAGED); }
+  // Apply the ReLU of a following in-place ReLUBridge (y = max(x, 0)) while the output is stored,
+  // instead of in a pass of its own; the ReLU bridge then skips its forward.
+  void set_fuse_relu(bool on) { fuse_relu_ = on; }
+  bool fuse_relu() const { return fuse_relu_; }
   // per-stage hipEvent timing (the reference's -D_DETAILED_PROFILING stage prints)
   void set_stage_profiling(bool on) { profile_ = on; }
   float stage_ms(int stage) {
@@ -203,7 +207,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       p_driver->conv_direct_forward(output_d_cube->get_p_data(), input_d_cube->get_p_data(),
                                     forward_slabs()->get_p_data(), bias_term ? p_bias_cube->get_p_data() : nullptr,
                                     (int)iB, (int)iD, (int)iR, (int)K, (int)padding, (int)num_output_features,
-                                    in_image_stride_, out_image_stride_);
+                                    in_image_stride_, out_image_stride_, fuse_relu_);
       end(STAGE_GEMM);
       report_forward_history.end();
       return;
@@ -215,7 +219,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       begin(STAGE_GEMM);
       p_driver->sgemm_conv_forward((int)num_output_features, (int)iB, (int)(oR * oC), (int)(K * K * iD),
                                    p_model_cube->get_p_data(), lowered()->get_p_data(),
-                                   bias_term ? p_bias_cube->get_p_data() : nullptr, output_d_cube->get_p_data());
+                                   bias_term ? p_bias_cube->get_p_data() : nullptr, output_d_cube->get_p_data(),
+                                   fuse_relu_);
       end(STAGE_GEMM);
     } else {
       LogicalCubeType lowered_output(staging()->get_p_data(), num_output_features, oR * oC * iB, 1, 1);
@@ -231,6 +236,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
         DeviceMemoryPointer bias = p_bias_cube->get_device_pointer(p_driver);
         p_driver->forward_bias(&bias, &output, (int)(oR * oC), (int)oD, (int)iB);
         end(STAGE_BIAS);
+      }
+      if (fuse_relu_) {  // the staged sequence has no epilogue to fold it into
+        DeviceMemoryPointer output = output_d_cube->get_device_pointer(p_driver);
+        p_driver->relu_forward(&output, &output);
       }
     }
     report_forward_history.end();
@@ -348,6 +357,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   int path_ = PATH_FUSED, default_path_ = PATH_FUSED;
   size_t in_image_stride_ = 0, out_image_stride_ = 0;
   bool views_ = false;
+  bool fuse_relu_ = false;
   bool direct_ok_ = false, profile_ = false;
   LogicalCubeType *lowered() {
     if (!p_forward_lowered_data) p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);

@@ -169,8 +169,8 @@ class HIPDriver {
     ok(cct_hip_sgemm_new(TA, TB, M, N, K, alpha, pA, pB, beta, pC), "sgemm_new");
   }
   void sgemm_conv_forward(int o, int batch, int fmap, int K, const float *model, const float *lowered,
-                          const float *bias, float *out) {
-    ok(cct_hip_sgemm_conv_forward(o, batch, fmap, K, model, lowered, bias, out), "sgemm_conv_forward");
+                          const float *bias, float *out, bool relu = false) {
+    ok(cct_hip_sgemm_conv_forward(o, batch, fmap, K, model, lowered, bias, out, relu ? 1 : 0), "sgemm_conv_forward");
   }
   // ---- stride-1 convolution without the lowered matrix (no counterpart in DeviceDriver.h) ----
   bool conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs) {
@@ -185,9 +185,9 @@ class HIPDriver {
   }
   void conv_direct_forward(float *output, const float *input, const float *slabs, const float *bias, int batch,
                            int depth, int n, int k, int padding, int num_outputs, size_t in_stride = 0,
-                           size_t out_stride = 0) {
+                           size_t out_stride = 0, bool relu = false) {
     ok(cct_hip_conv_direct_forward(output, input, slabs, bias, batch, depth, n, k, padding, num_outputs, in_stride,
-                                   out_stride),
+                                   out_stride, relu ? 1 : 0),
        "conv_direct_forward");
   }
   void conv_direct_backward_data(float *input_grad, const float *output_grad, const float *slabs, int batch,

@@ -8,7 +8,8 @@
 //   * output sizes: conv (R+2p-K)/s+1 (:112-115), pooling floor((R-K)/s)+1 unpadded (:1374-1376);
 //   * the first weight layer does not compute a data gradient (:1108-1110);
 //   * ReLU and dropout run in place on their input layer (the reference shares the layers on the
-//     GPU: ParallelizedBridge.h:183-198);
+//     GPU: ParallelizedBridge.h:183-198); an in-place ReLU directly after a convolution is applied
+//     by the convolution's output store (same values, one pass over the tensor less);
 //   * `group` > 1 is realised as `group` independent convolutions on channel slices whose outputs
 //     are concatenated along depth (the reference's two-tower Split/Concat arrangement,
 //     src/DeepNet.h:1700-1757); a group runs in place on its channel slices when the direct
@@ -120,7 +121,14 @@ class Network {
         case CCT_LAYER_RELU: {
           nd.out = cur;  // in place
           nd.params.push_back(new_param(s));
-          nd.bridges.push_back(new ReLUBridge<float, HIPDriver>(cur, cur, nd.params[0], &solver_, &driver_));
+          auto *rb = new ReLUBridge<float, HIPDriver>(cur, cur, nd.params[0], &solver_, &driver_);
+          // directly after a convolution the clamp rides on the convolution's output store
+          if (!nodes_.empty() && nodes_.back().spec.type == CCT_LAYER_CONV && nodes_.back().out == cur) {
+            for (BridgeT *cb : nodes_.back().bridges)
+              static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(cb)->sub_bridge()->set_fuse_relu(true);
+            rb->forward_done_by_producer = true;
+          }
+          nd.bridges.push_back(rb);
           break;
         }
         case CCT_LAYER_DROPOUT: {

@@ -38,7 +38,10 @@ class ReLUBridge : public AbstractBridge<DataType, DriverClass> {
       std::abort();
     }
   }
+  // set when the producing bridge clamps at zero while it stores (in-place ReLU after a convolution)
+  bool forward_done_by_producer = false;
   void forward() override {
+    if (forward_done_by_producer) return;
     DeviceMemoryPointer input = p_input_layer->p_data_cube->get_device_pointer(p_driver);
     DeviceMemoryPointer output = p_output_layer->p_data_cube->get_device_pointer(p_driver);
     p_driver->relu_forward(&output, &input);

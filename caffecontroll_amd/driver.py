@@ -109,9 +109,9 @@ class HIPDriver:
     def sgemm_new(self, TA, TB, M, N, K, alpha, A, B, beta, Cm):
         check(self.lib.cct_hip_sgemm_new(TA, TB, M, N, K, alpha, _p(A), _p(B), beta, _p(Cm)), "sgemm_new")
 
-    def sgemm_conv_forward(self, o, batch, fmap, K, model, lowered, bias, out):
+    def sgemm_conv_forward(self, o, batch, fmap, K, model, lowered, bias, out, relu=False):
         check(self.lib.cct_hip_sgemm_conv_forward(o, batch, fmap, K, _p(model), _p(lowered), _p(bias),
-                                                  _p(out)), "sgemm_conv_forward")
+                                                  _p(out), int(relu)), "sgemm_conv_forward")
 
     def conv_direct_supported(self, b, d, n, k, s, p, o):
         return bool(self.lib.cct_hip_conv_direct_supported(b, d, n, k, s, p, o))
@@ -123,9 +123,9 @@ class HIPDriver:
         check(self.lib.cct_hip_conv_direct_slabs(_p(slabs), _p(model), o, d, k, int(for_data_gradient)),
               "conv_direct_slabs")
 
-    def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o, in_stride=0, out_stride=0):
+    def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o, in_stride=0, out_stride=0, relu=False):
         check(self.lib.cct_hip_conv_direct_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o,
-                                                   in_stride, out_stride), "conv_direct_forward")
+                                                   in_stride, out_stride, int(relu)), "conv_direct_forward")
 
     def conv_direct_backward_data(self, din, dout, slabs, b, d, n, k, p, o, in_stride=0, out_stride=0):
         check(self.lib.cct_hip_conv_direct_backward_data(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o,

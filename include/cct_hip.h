@@ -152,9 +152,11 @@ int cct_hip_sgemm_new(int TA, int TB, int M, int N, int K, float alpha, const fl
                       const float *B, float beta, float *C);
 /* Forward-convolution GEMM with the output permutation and bias of
  * ConvolutionBridge::forward (src/bridges/ConvolutionBridge_impl.hxx:328-364) folded into the
- * epilogue: out[b][o][fmap] = model[o x K] * lowered[b*fmap x K]^T + bias[o] (bias may be NULL). */
+ * epilogue: out[b][o][fmap] = model[o x K] * lowered[b*fmap x K]^T + bias[o] (bias may be NULL).
+ * relu != 0 also applies the ReLU of a following in-place ReLUBridge (max(x, 0),
+ * src/kernels/relu.hxx:10-25) before the store. */
 int cct_hip_sgemm_conv_forward(int o, int batch, int fmap, int K, const float *model,
-                               const float *lowered, const float *bias, float *out);
+                               const float *lowered, const float *bias, float *out, int relu);
 /* ---- stride-1 convolution without the lowered matrix ------------------------------------ */
 /* Fused replacements for chains of ConvolutionBridge's lowering pipeline when stride == 1 and
  * k is 3 or 5 (padded image at most 32 wide).  Results agree with the lowering path to fp32
@@ -178,10 +180,12 @@ int cct_hip_conv_direct_slabs(float *slabs, const float *model, int num_outputs,
  *
  * lower_cube + forward GEMM + remap_output + bias of ConvolutionBridge::forward
  * (src/bridges/ConvolutionBridge_impl.hxx:316-364) in one kernel:
- * output[b][o][m][m] from input[b][d][n][n], forward slabs, bias[o] (may be NULL). */
+ * output[b][o][m][m] from input[b][d][n][n], forward slabs, bias[o] (may be NULL); relu != 0
+ * folds a following in-place ReLU into the store. */
 int cct_hip_conv_direct_forward(float *output, const float *input, const float *slabs,
                                 const float *bias, int batch, int depth, int n, int k, int padding,
-                                int num_outputs, size_t input_image_stride, size_t output_image_stride);
+                                int num_outputs, size_t input_image_stride, size_t output_image_stride,
+                                int relu);
 /* Gradient remap + data-gradient GEMM + inverse_lower_cube of ConvolutionBridge::backward
  * (src/bridges/ConvolutionBridge_impl.hxx:601-616) in one kernel: input_grad[b][d][n][n] from
  * output_grad[b][o][m][m] (read in place, not permuted) and data-gradient slabs. */

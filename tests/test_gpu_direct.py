@@ -80,6 +80,11 @@ def test_direct_kernels_match_oracle(oracle, shape):
     out_nb = empty((b, o, m, m))
     drv.conv_direct_forward(out_nb, d_x, slabs_f, None, b, d, n, k, p, o)
     assert rel_err(host(out_nb), ref_out - bias.reshape(1, o, 1, 1)) <= TOL
+    # a following ReLU folded into the store: exactly max(x, 0) of the unfused result
+    out_relu = empty((b, o, m, m))
+    drv.conv_direct_forward(out_relu, d_x, slabs_f, dev(bias), b, d, n, k, p, o, relu=True)
+    np.testing.assert_array_equal(host(out_relu), oracle.relu_forward(host(out)))
+    assert (host(out) < 0).any()
 
     dx = empty((b, d, n, n))
     drv.conv_direct_backward_data(dx, d_og, slabs_b, b, d, n, k, p, o)

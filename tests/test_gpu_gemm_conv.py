@@ -141,6 +141,10 @@ def conv_forward_gpu(x, w, bias, k, s, p, fused):
     out = empty((b, o, m, m))
     if fused:
         drv.sgemm_conv_forward(o, b, m * m, kkd, dw, lowered, dbias, out)
+        # with the ReLU of a following layer folded into the epilogue: max(x, 0) of the same result
+        out_relu = empty((b, o, m, m))
+        drv.sgemm_conv_forward(o, b, m * m, kkd, dw, lowered, dbias, out_relu, relu=True)
+        np.testing.assert_array_equal(host(out_relu), np.maximum(host(out), np.float32(0)))
     else:
         tmp = empty((o, bmm))
         drv.sgemm(RM, N_, T_, o, bmm, kkd, 1.0, dw, kkd, lowered, kkd, 0.0, tmp, bmm)
