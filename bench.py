@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the convolution training hot path on one MI355X.
 
-Workload (BASELINE.json configs[1]): AlexNet conv2 shape, ungrouped -- batch 256, input 96x27x27
+Workload (benchmark configuration 2): AlexNet conv2 shape, ungrouped -- batch 256, input 96x27x27
 N(0,1), 256 filters 5x5, stride 1, pad 2, weights N(0,0.01), bias 0.1, output gradient N(0,1).
 One step = ConvolutionBridge forward + backward (lower, forward GEMM with remap+bias epilogue,
 out-grad remap, data-gradient GEMM, lift + bias gradient, weight-gradient GEMM) on tensors that
@@ -46,7 +46,7 @@ GEMM_TRAFFIC_BYTES = {
 
 
 def synth(cfg, seed, torch):
-    """Seeded synthetic tensors of BASELINE.json's configs, generated on the host and uploaded."""
+    """Seeded synthetic tensors of the benchmark configurations, generated on the host and uploaded."""
     import numpy as np
     b, d, n, k, s, p, o = CONFIGS[cfg]
     m = (n + 2 * p - k) // s + 1
@@ -121,7 +121,7 @@ def cpu_baseline(cfg, seed):
 
 
 def net_iteration(args, torch, np):
-    """BASELINE.json configs[3] / configs[4]: one step = forward + backward + SGD update of every layer,
+    """benchmark configurations 4 and 5: one step = forward + backward + SGD update of every layer,
     synthetic images and labels already on the device."""
     from caffecontroll_amd import HIPDriver, nets
     drv = HIPDriver(0)

@@ -12,7 +12,7 @@ TOL = 1e-4
 
 # b d n k p o  (stride is 1 throughout)
 SHAPES = [
-    (64, 1, 28, 5, 0, 20),    # LeNet conv1 (BASELINE config 1)
+    (64, 1, 28, 5, 0, 20),    # LeNet conv1 (benchmark configuration 1)
     (8, 20, 12, 5, 0, 50),    # LeNet conv2: odd number of 32-row blocks, slabs not 16-byte aligned
     (3, 96, 27, 5, 2, 256),   # AlexNet conv2 geometry
     (2, 48, 27, 5, 2, 128),   # one group of CaffeNet conv2
@@ -252,7 +252,7 @@ FULL_SIZE = [(256, 96, 27, 5, 2, 256), (256, 48, 27, 5, 2, 128), (256, 256, 13, 
 
 @pytest.mark.parametrize("cfg", FULL_SIZE, ids=_ids)
 def test_full_size_direct_vs_float64(cfg):
-    """Full-size layers (BASELINE config 2 first; the last one with an odd batch): the three direct
+    """Full-size layers (benchmark configuration 2 first; the last one with an odd batch): the three direct
     kernels against torch's float64 convolution and its gradients (independent of this library
     and of the oracle)."""
     import torch

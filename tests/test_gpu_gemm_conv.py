@@ -1,7 +1,7 @@
 """GPU parity: sgemm / sgemm_new / sgemv and the whole convolution forward+backward (driver-level
 call sequence of ConvolutionBridge) against the CPU oracle and the reference's golden files.
 
-fp32 tolerance (BASELINE north_star): max|gpu - ref| / max|ref| <= 1e-4 per tensor, arbitrated
+fp32 tolerance (the bar this path is held to): max|gpu - ref| / max|ref| <= 1e-4 per tensor, arbitrated
 against a float64-accumulating reference."""
 import numpy as np
 import pytest
@@ -227,9 +227,9 @@ def test_conv_reference_fixtures(oracle, case, fused):
 
 
 CONV_SHAPES = [  # b d n k s p o
-    (64, 1, 28, 5, 1, 0, 20),   # BASELINE config 1 (LeNet conv1), full size
-    (8, 96, 27, 5, 1, 2, 256),  # BASELINE config 2 geometry, batch 8
-    (4, 3, 227, 11, 4, 0, 96),  # BASELINE config 3 geometry, batch 4
+    (64, 1, 28, 5, 1, 0, 20),   # benchmark configuration 1 (LeNet conv1), full size
+    (8, 96, 27, 5, 1, 2, 256),  # benchmark configuration 2 geometry, batch 8
+    (4, 3, 227, 11, 4, 0, 96),  # benchmark configuration 3 geometry, batch 4
     (16, 20, 12, 5, 1, 0, 50),  # LeNet conv2
     (4, 256, 13, 3, 1, 1, 384), # AlexNet conv3 geometry
 ]
@@ -268,7 +268,7 @@ def test_conv_forward_backward_vs_oracle(oracle, shape):
 @pytest.mark.parametrize("shape", [(256, 96, 27, 5, 1, 2, 256), (256, 3, 227, 11, 4, 0, 96)],
                          ids=["alexnet_conv2", "alexnet_conv1"])
 def test_full_size_conv_against_torch_fp64(shape):
-    """BASELINE configs 2 and 3 at full size (b=256): forward output and all three gradients agree
+    """benchmark configurations 2 and 3 at full size (b=256): forward output and all three gradients agree
     with float64 torch convolutions on the whole tensor (tolerance 1e-4 of the tensor's max)."""
     import torch
     import torch.nn.functional as F

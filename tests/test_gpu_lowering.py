@@ -9,7 +9,7 @@ pytestmark = pytest.mark.gpu
 
 # b d n k s p
 SHAPES = [
-    (64, 1, 28, 5, 1, 0),     # LeNet conv1 (BASELINE config 1)
+    (64, 1, 28, 5, 1, 0),     # LeNet conv1 (benchmark configuration 1)
     (4, 3, 20, 5, 4, 2),      # reference small fixture shape
     (4, 3, 127, 11, 4, 2),    # reference large fixture shape
     (3, 96, 27, 5, 1, 2),     # AlexNet conv2 geometry, small batch (vector-store path, 2-row bands)
@@ -117,7 +117,7 @@ def test_empty_batch_is_a_no_op():
 
 
 # ---------------------------------------------------------------------------------------------
-# Full AlexNet-conv2 size (BASELINE config 2): properties that do not need the slow CPU oracle.
+# Full AlexNet-conv2 size (benchmark configuration 2): properties that do not need the slow CPU oracle.
 CFG2 = (256, 96, 27, 5, 1, 2)
 
 
@@ -126,7 +126,7 @@ CFG3 = (256, 3, 227, 11, 4, 0)
 
 @pytest.mark.parametrize("cfg", [CFG2, CFG3], ids=["alexnet_conv2", "alexnet_conv1"])
 def test_full_size_lower_matches_unfold_and_adjoint(cfg):
-    """At the full BASELINE sizes (config 2: b=256,d=96,n=27,k=5,p=2; config 3: b=256,d=3,n=227,
+    """At the full benchmark sizes (config 2: b=256,d=96,n=27,k=5,p=2; config 3: b=256,d=3,n=227,
     k=11,s=4): (i) the lowered matrix equals torch's unfold (an independent im2col) bit for bit;
     (ii) lift(lower(x)) == x * multiplicity; (iii) <lower(x),y> == <x,lift(y)> in float64 within
     rounding."""

@@ -1,4 +1,4 @@
-"""GPU parity for whole training iterations (BASELINE configs 4 and 5): LeNet at its full batch and
+"""GPU parity for whole training iterations (benchmark configurations 4 and 5): LeNet at its full batch and
 CaffeNet/AlexNet at a small batch, layer chain on the device against the CPU oracle chain."""
 import numpy as np
 import pytest
@@ -65,7 +65,7 @@ def _compare_params(net, ref, tol):
 
 
 def test_lenet_training_iterations(oracle):
-    """BASELINE config 4: batch 64, 1x28x28 uniform[0,1) images, 10 classes, lr 0.01, momentum 0.9."""
+    """benchmark configuration 4: batch 64, 1x28x28 uniform[0,1) images, 10 classes, lr 0.01, momentum 0.9."""
     from caffecontroll_amd import nets
     rng = np.random.default_rng(1234 + 4)
     B = 64
@@ -101,7 +101,7 @@ def test_lenet_training_iterations(oracle):
 
 @pytest.mark.parametrize("groups", [True, False])
 def test_caffenet_training_iteration_small_batch(oracle, groups):
-    """BASELINE config 5 geometry (3x227x227, 1000 classes, grouped conv2/4/5, LRN, dropout) at
+    """benchmark configuration 5 geometry (3x227x227, 1000 classes, grouped conv2/4/5, LRN, dropout) at
     batch 2; dropout masks are injected so both sides drop the same units."""
     from caffecontroll_amd import nets
     rng = np.random.default_rng(1234 + 5)
