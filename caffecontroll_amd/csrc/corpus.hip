@@ -14,29 +14,50 @@
 
 namespace cct {
 
-// One lane per output pixel; blockIdx.y = image * channels + channel, so the crop parameters are
-// wavefront-uniform.  Reads run along the source row, writes along the destination row (reversed
-// for a mirrored image), both contiguous per wavefront.
+// One lane per run of four output pixels of a row; blockIdx.y = image * channels + channel, so the
+// crop parameters are wavefront-uniform.  Reads run along the source row (four bytes and one
+// 16-byte mean load per lane), the four results leave in one 16-byte store (reversed for a
+// mirrored image); all of them need dword alignment at most.
+typedef float corpus_f4u __attribute__((ext_vector_type(4), aligned(4)));
+
 __global__ void __launch_bounds__(256)
 transform_kernel(float *__restrict__ dst, const unsigned char *__restrict__ raw, const float *__restrict__ mean,
                  const int *__restrict__ params, int channels, int height, int width, int out_rows, int out_cols,
-                 int crop, float scale, FastDiv div_cols) {
+                 int crop, float scale, int quads_per_row, FastDiv div_quads) {
   const uint32_t p = blockIdx.x * 256u + threadIdx.x;
-  if (p >= (uint32_t)(out_rows * out_cols)) return;
+  if (p >= (uint32_t)(out_rows * quads_per_row)) return;
   const uint32_t plane = blockIdx.y;  // image * channels + c
   const uint32_t img = plane / (uint32_t)channels, c = plane - img * (uint32_t)channels;
-  const uint32_t h = fdiv(p, div_cols), w = p - h * (uint32_t)out_cols;
+  const uint32_t h = fdiv(p, div_quads), w0 = (p - h * (uint32_t)quads_per_row) * 4u;
   int h_off = 0, w_off = 0, mirror = 0;
   if (crop > 0) {
     h_off = params[3 * img];
     w_off = params[3 * img + 1];
     mirror = params[3 * img + 2];
   }
-  const size_t in_plane = (size_t)(c * (uint32_t)height + h + (uint32_t)h_off) * (uint32_t)width + w + (uint32_t)w_off;
-  const float x = (float)raw[(size_t)img * channels * height * width + in_plane];
-  const float m = mean ? mean[in_plane] : 0.f;
-  const uint32_t wd = mirror ? (uint32_t)out_cols - 1u - w : w;
-  dst[((size_t)plane * out_rows + h) * out_cols + wd] = (x - m) * scale;
+  const size_t in_plane = (size_t)(c * (uint32_t)height + h + (uint32_t)h_off) * (uint32_t)width + w0 + (uint32_t)w_off;
+  const unsigned char *src = raw + (size_t)img * channels * height * width + in_plane;
+  float *drow = dst + ((size_t)plane * out_rows + h) * out_cols;
+  const int n = min(4, out_cols - (int)w0);  // pixels of this run inside the row
+  float v[4];
+  if (n == 4) {
+    const corpus_f4u m = mean ? *reinterpret_cast<const corpus_f4u *>(mean + in_plane) : corpus_f4u{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) v[j] = ((float)src[j] - m[j]) * scale;
+    if (mirror) {
+      const corpus_f4u o = {v[3], v[2], v[1], v[0]};
+      *reinterpret_cast<corpus_f4u *>(drow + (out_cols - 4 - (int)w0)) = o;
+    } else {
+      const corpus_f4u o = {v[0], v[1], v[2], v[3]};
+      *reinterpret_cast<corpus_f4u *>(drow + w0) = o;
+    }
+  } else {
+    for (int j = 0; j < n; ++j) {
+      const float x = ((float)src[j] - (mean ? mean[in_plane + j] : 0.f)) * scale;
+      const int w = (int)w0 + j;
+      drow[mirror ? out_cols - 1 - w : w] = x;
+    }
+  }
 }
 
 static int transform_batch(float *dst, const unsigned char *raw, const float *mean, const int *params,
@@ -49,15 +70,17 @@ static int transform_batch(float *dst, const unsigned char *raw, const float *me
   const int rows = a.crop_size ? a.crop_size : a.height, cols = a.crop_size ? a.crop_size : a.width;
   CCT_REQUIRE(a.channels <= 65535 && (size_t)rows * cols < (1u << 30) && (size_t)a.height * a.width < (1u << 30),
               "transform_batch: image too large");
+  CCT_REQUIRE((uintptr_t)dst % 4 == 0 && (!mean || (uintptr_t)mean % 4 == 0), "transform_batch: misaligned float pointer");
+  const int quads = (cols + 3) / 4;
   // grid.y is limited to 65535: launch in slices of planes (whole images per slice)
   const size_t imgs_per_launch = std::max<size_t>(1, 65535u / (size_t)a.channels);
   for (size_t i0 = 0; i0 < (size_t)a.batch; i0 += imgs_per_launch) {
     const size_t ni = std::min(imgs_per_launch, (size_t)a.batch - i0);
-    dim3 grid((unsigned)((rows * cols + 255) / 256), (unsigned)(ni * a.channels));
+    dim3 grid((unsigned)((rows * quads + 255) / 256), (unsigned)(ni * a.channels));
     transform_kernel<<<grid, 256, 0, stream>>>(dst + i0 * a.channels * rows * cols,
                                                raw + i0 * a.channels * a.height * a.width, mean,
                                                params ? params + 3 * i0 : nullptr, a.channels, a.height, a.width,
-                                               rows, cols, a.crop_size, a.scale, make_fastdiv((uint32_t)cols));
+                                               rows, cols, a.crop_size, a.scale, quads, make_fastdiv((uint32_t)quads));
     CCT_LAUNCH_CHECK();
   }
   return 0;
