@@ -98,6 +98,8 @@ class Corpus {
   int init(int batch, int channels, int height, int width, int crop, float scale, int mirror_, int phase_,
            const float *mean_host, unsigned seed) {
     CCT_REQUIRE(batch > 0 && channels > 0 && height > 0 && width > 0, "corpus: bad geometry");
+    CCT_REQUIRE(phase_ == 0 || phase_ == 1, "corpus: phase must be 0 (TRAIN) or 1 (TEST)");
+    CCT_REQUIRE((double)batch * channels * height * width < 2147483648.0, "corpus: a batch of raw images must stay below 2 GiB");
     CCT_REQUIRE(crop >= 0 && crop <= height && crop <= width, "corpus: crop_size %d does not fit %dx%d images", crop,
                 height, width);
     geo.batch = batch; geo.channels = channels; geo.height = height; geo.width = width;
@@ -149,6 +151,15 @@ class Corpus {
   int submit() {
     CCT_REQUIRE(staged_, "corpus: nothing staged");
     const int s = head_;
+    if (geo.crop_size > 0) {
+      // a caller may have overwritten the drawn parameters: the kernel trusts them, so check here
+      const int *p = (const int *)((const char *)host_[s] + params_off_);
+      for (int b = 0; b < geo.batch; ++b)
+        CCT_REQUIRE(p[3 * b] >= 0 && p[3 * b] <= geo.height - geo.crop_size && p[3 * b + 1] >= 0 &&
+                        p[3 * b + 1] <= geo.width - geo.crop_size && (p[3 * b + 2] == 0 || p[3 * b + 2] == 1),
+                    "corpus: crop parameters of image %d (%d, %d, %d) are out of range", b, p[3 * b], p[3 * b + 1],
+                    p[3 * b + 2]);
+    }
     // the device buffer of this slot may still be read by the transform of two batches ago
     if (consume_recorded_[s]) CCT_HIP_CHECK(hipStreamWaitEvent(copy_stream_, consumed_[s], 0));
     CCT_HIP_CHECK(hipMemcpyAsync(dev_[s], host_[s], slot_bytes_, hipMemcpyHostToDevice, copy_stream_));
