@@ -96,6 +96,7 @@ def test_memory_fed_loader_double_buffering(oracle):
     cp.submit()
     params = cp.consume(images, labels, want_params=True)
     assert tuple(params[0]) == (0, 0, 1)
+    assert np.array_equal(host(images), oracle.transform_batch(batches[0][0], None, crop, params, 1.0))
     px, lb, pr = cp.stage()
     pr[1] = (h - crop + 1, 0, 0)   # one row too far down: refused on the host, nothing is launched
     with pytest.raises(CctHipError, match="out of range"):
@@ -103,7 +104,6 @@ def test_memory_fed_loader_double_buffering(oracle):
     pr[1] = (h - crop, w - crop, 0)
     cp.submit()
     cp.consume(images, labels)
-    assert np.array_equal(host(images), oracle.transform_batch(batches[0][0], None, crop, params, 1.0))
     cp.close()
 
 
