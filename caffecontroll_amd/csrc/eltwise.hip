@@ -54,6 +54,10 @@ __global__ __launch_bounds__(TPB) void fill_u8_kernel(unsigned char *__restrict_
 }
 
 // ---- slice remap: dst slice (j / sB) + (j % sB) * sD  <-  src slice j --------------------------
+// A workgroup moves one slice (or, for long slices, one of gridDim.y parts of it) with 16-byte loads
+// and stores at dword alignment, four of them in flight per lane.
+typedef float remap_f4u __attribute__((ext_vector_type(4), aligned(4)));
+
 __global__ __launch_bounds__(TPB) void remap_kernel(float *__restrict__ dst, const float *__restrict__ src,
                                                     uint32_t rc, uint32_t sD, FastDiv div_b) {
   const uint32_t j = blockIdx.x;  // source slice
@@ -61,7 +65,17 @@ __global__ __launch_bounds__(TPB) void remap_kernel(float *__restrict__ dst, con
   const uint32_t realb = j - reald * div_b.div;
   const float *s = src + (size_t)j * rc;
   float *d = dst + ((size_t)reald + (size_t)realb * sD) * rc;
-  for (uint32_t i = blockIdx.y * TPB + threadIdx.x; i < rc; i += gridDim.y * TPB) d[i] = s[i];
+  const uint32_t nq = rc >> 2, stride = gridDim.y * TPB;
+  for (uint32_t q0 = blockIdx.y * TPB + threadIdx.x; q0 < nq; q0 += 4 * stride) {
+    remap_f4u v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (q0 + u * stride < nq) v[u] = *reinterpret_cast<const remap_f4u *>(s + 4 * (size_t)(q0 + u * stride));
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (q0 + u * stride < nq) *reinterpret_cast<remap_f4u *>(d + 4 * (size_t)(q0 + u * stride)) = v[u];
+  }
+  if (blockIdx.y == 0 && threadIdx.x < (rc & 3u)) d[4 * nq + threadIdx.x] = s[4 * nq + threadIdx.x];
 }
 
 // ---- depth-slice copy: part [B][dc][rc] <-> channels [d_off, d_off+dc) of whole [B][D][rc] ----------
@@ -622,7 +636,9 @@ int cct_hip_remap(float *dst, const float *src, const cct_pmap_helper *a) {
   const char *d0 = (const char *)dst, *s0 = (const char *)src;
   const size_t bytes = rc * slices * 4;
   CCT_REQUIRE(d0 + bytes <= s0 || s0 + bytes <= d0, "remap: dst and src overlap");
-  uint32_t gy = (uint32_t)((rc + TPB - 1) / TPB);
+  // parts per slice: each lane moves up to 64 bytes; few slices with long rows are cut further
+  uint32_t gy = (uint32_t)((rc / 4 + 4 * TPB - 1) / (4 * TPB));
+  if (gy < 1) gy = 1;
   if (gy > 64) gy = 64;
   hipLaunchKernelGGL(remap_kernel, dim3((uint32_t)slices, gy), dim3(TPB), 0, ctx().stream, dst, src,
                      (uint32_t)rc, (uint32_t)a->sD, make_fastdiv((uint32_t)a->sB));
