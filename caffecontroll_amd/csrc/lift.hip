@@ -184,6 +184,74 @@ __global__ __launch_bounds__(LIFT_THREADS) void lift_kernel(float *__restrict__ 
   dst[pix] = acc;
 }
 
+// Strided layers (stride ST > 1): a lane owns ST consecutive destination pixels of a row.  Pixel
+// x = ST*l + ph draws on the planes kc == (x + p) mod ST, so for a fixed phase ph the lanes of a
+// wavefront read consecutive addresses of ONE (kr, kc) plane -- with one pixel per lane they would
+// alternate between ST planes.  Each pixel still adds its terms in (kr, kc) ascending order; the
+// ST results leave in one store.
+typedef float lift_f4u __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int KT, int ST>
+__global__ __launch_bounds__(LIFT_THREADS) void lift_strided_kernel(float *__restrict__ dst,
+                                                                    const float *__restrict__ src,
+                                                                    const LiftParams P, uint32_t nruns,
+                                                                    FastDiv div_runs) {
+  if (blockIdx.x < P.nbias) {
+    bias_backward_block(P, (int)blockIdx.x);
+    return;
+  }
+  const uint32_t run = (blockIdx.x - P.nbias) * LIFT_THREADS + threadIdx.x;
+  if (run >= nruns) return;
+  // run = ((ib*iD + id)*iR + y)*runs_per_row + l
+  const uint32_t t1 = fdiv(run, div_runs);
+  const int l = run - t1 * div_runs.div;
+  const uint32_t t2 = fdiv(t1, P.div_r);
+  const int y = t1 - t2 * P.iR;
+  const uint32_t ib = fdiv(t2, P.div_d);
+  const int id = t2 - ib * P.iD;
+  const int m = P.m;
+  const float *base = src + (size_t)id * KT * KT * P.plane + (size_t)ib * m * m;
+  const int yp = y + P.p;
+  // every candidate (jr, jc) is loaded from a clamped address without a branch, so all loads of a
+  // lane are in flight together; candidates outside the kernel or the output contribute an exact +0
+  constexpr int NJ = (KT + ST - 1) / ST;
+  float acc[ST];
+#pragma unroll
+  for (int ph = 0; ph < ST; ++ph) {
+    const int xp = l * ST + ph + P.p;
+    float v[NJ][NJ];
+#pragma unroll
+    for (int jr = 0; jr < NJ; ++jr) {
+      const int kr = yp % ST + jr * ST, cr = (yp - kr) / ST;  // yp - kr is a multiple of ST
+      const bool rok = kr < KT && yp >= kr && cr < m;
+#pragma unroll
+      for (int jc = 0; jc < NJ; ++jc) {
+        const int kc = xp % ST + jc * ST, cc = (xp - kc) / ST;
+        const bool ok = rok && kc < KT && xp >= kc && cc < m;
+        const size_t off = ok ? (size_t)(kr * KT + kc) * P.plane + (size_t)(cr * m + cc) : 0;
+        const float t = base[off];
+        v[jr][jc] = ok ? t : 0.0f;
+      }
+    }
+    float a = 0.0f;
+#pragma unroll
+    for (int jr = 0; jr < NJ; ++jr)
+#pragma unroll
+      for (int jc = 0; jc < NJ; ++jc) a += v[jr][jc];
+    acc[ph] = a;
+  }
+  float *out = dst + (size_t)t1 * P.iC + (size_t)l * ST;
+  const int n = min(ST, P.iC - l * ST);
+  if (ST == 4 && n == 4) {
+    const lift_f4u v = {acc[0], acc[1], acc[2], acc[3]};
+    *reinterpret_cast<lift_f4u *>(out) = v;
+  } else {
+#pragma unroll
+    for (int ph = 0; ph < ST; ++ph)
+      if (ph < n) out[ph] = acc[ph];
+  }
+}
+
 static int launch_lift(float *dst, const float *src, const cct_inverse_lower_cube_args *a,
                        float *bias_grad, const float *out_grad, int fmap, int depth, int batch) {
   CCT_REQUIRE(dst && src && a, "inverse_lower_cube: null argument");
@@ -211,9 +279,13 @@ static int launch_lift(float *dst, const float *src, const cct_inverse_lower_cub
     hipLaunchKernelGGL((lift_kernel<5, 1>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
   else if (P.k == 3 && P.s == 1)
     hipLaunchKernelGGL((lift_kernel<3, 1>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
-  else if (P.k == 11 && P.s == 4)
-    hipLaunchKernelGGL((lift_kernel<11, 4>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
-  else
+  else if (P.k == 11 && P.s == 4) {
+    const uint32_t per_row = (uint32_t)((P.iC + 3) / 4);
+    const size_t nruns = (size_t)P.iB * P.iD * P.iR * per_row;
+    const uint32_t blocks = (uint32_t)((nruns + LIFT_THREADS - 1) / LIFT_THREADS);
+    hipLaunchKernelGGL((lift_strided_kernel<11, 4>), dim3(blocks + P.nbias), dim3(LIFT_THREADS), 0, st, dst, src, P,
+                       (uint32_t)nruns, make_fastdiv(per_row));
+  } else
     hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
   CCT_LAUNCH_CHECK();
   return 0;
