@@ -28,6 +28,24 @@ SHAPES = [
 ]
 
 
+def _random_shapes(count, seed):
+    """Seeded random geometries inside the kernels' range: k in {3, 5}, any padding 0..k-1, padded
+    width up to 32, channel and map counts around the 4-channel steps and 32-row blocks."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        k = int(rng.choice([3, 5]))
+        p = int(rng.integers(0, k))
+        n = int(rng.integers(max(k - 2 * p, 2), 32 - 2 * p + 1))
+        if n + 2 * p - k + 1 < 7:   # the kernels want outputs of at least 7x7
+            continue
+        b = int(rng.integers(1, 7))
+        d = int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 13, 16, 31]))
+        o = int(rng.choice([1, 3, 16, 31, 32, 33, 47, 64, 65, 96, 100, 129]))
+        out.append((b, d, n, k, p, o))
+    return out
+
+
 def _ids(s):
     return "b%d_d%d_n%d_k%d_p%d_o%d" % s
 
@@ -54,9 +72,11 @@ def _tensors(shape, seed):
     return x, w, bias, og, m
 
 
-@pytest.mark.parametrize("shape", SHAPES, ids=_ids)
+@pytest.mark.parametrize("shape", SHAPES + _random_shapes(24, 2024), ids=_ids)
 def test_direct_kernels_match_oracle(oracle, shape):
     b, d, n, k, p, o = shape
+    if shape not in SHAPES and not driver().conv_direct_supported(b, d, n, k, 1, p, o):
+        pytest.skip("random geometry outside the direct kernels' range")
     x, w, bias, og, m = _tensors(shape, 4321 + sum(shape))
     drv = driver()
     assert drv.conv_direct_supported(b, d, n, k, 1, p, o)

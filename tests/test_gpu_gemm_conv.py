@@ -28,6 +28,9 @@ GEMM_CASES = [
     # (M, N, K, pad) -- pad != 0 exercises leading dimensions that break 16-byte alignment
     (7, 11, 13, 0), (64, 64, 16, 0), (65, 63, 17, 3), (128, 128, 64, 0), (256, 384, 100, 0),
     (300, 200, 75, 1), (20, 576, 25, 0), (500, 64, 800, 0), (10, 500, 64, 0), (256, 130, 8, 4),
+    # row counts for which the 96-row tile pads least (AlexNet conv1 has 96 output maps), with ragged
+    # columns, a K tail and unaligned leading dimensions
+    (96, 4000, 363, 0), (90, 1100, 50, 1), (192, 3000, 40, 0), (96, 130, 1100, 3),
 ]
 
 
