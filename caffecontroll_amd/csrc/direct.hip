@@ -641,9 +641,15 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   constexpr int NCH = (BN - 1) / KK + 2;
   constexpr int BSZ = (NCH * PCH + 64 * W - 1) / (64 * W) * (64 * W);  // patch floats: whole passes
   constexpr int NBW = BSZ / (64 * W);                                   // patch loads per lane per step
-  constexpr int AST = (2 * HO) | 1;
-  constexpr int RW = (32 * AST + 63) / 64 * 64;  // slab floats per wavefront
-  constexpr int NAW = RW / 64;                    // slab loads per lane per step
+  // dout slab of a wavefront: per map and image the HO row values as NQD runs of four floats (the
+  // last run starts at HO - 4 and overlaps its neighbour when HO is not a multiple of 4), QPM runs
+  // per map including one empty run that makes the map stride an odd number of runs (16-byte reads
+  // of eight neighbouring lanes then fall into eight different bank groups).  One 16-byte global->LDS
+  // load per lane moves a run: a quarter of the load instructions a float-wise copy would take, and
+  // those instructions are what the MFMA pipe otherwise waits on.
+  constexpr int NQD = (HO + 3) / 4, QPM = 2 * NQD + 1;
+  constexpr int NAW = (32 * QPM + 63) / 64;      // slab loads (16 bytes per lane) per lane per step
+  constexpr int RW = NAW * 256;                  // slab floats per wavefront
   constexpr int AFL = W * RW, STAGE = AFL + BSZ;
   constexpr int NQ = (HO + 1) / 2;                // x pairs per step
   extern __shared__ __attribute__((aligned(16))) float smem[];
@@ -663,17 +669,17 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   uint32_t a_second = 0;
 #pragma unroll
   for (int k = 0; k < NAW; ++k) {
-    const uint32_t e = (uint32_t)(k * 64 + lane);
-    const uint32_t m = e / AST, i = e - m * AST;
+    const uint32_t e = (uint32_t)(k * 64 + lane);  // run index inside the wavefront's slab
+    const uint32_t m = e / QPM, q = e - m * QPM;
     const uint32_t map = min((uint32_t)(m0 + wave * 32) + min(m, 31u), (uint32_t)g.o - 1) - m0;
-    uint32_t off = map * ho2;
-    if (i < (uint32_t)HO) {
-      off += i;
-    } else if (i < 2u * HO) {
-      off += g.dout_img_stride + (i - HO);
-      a_second |= 1u << k;
+    const uint32_t second = q >= (uint32_t)NQD ? 1u : 0u, j = q - second * NQD;
+    const uint32_t start = j + 1 < (uint32_t)NQD ? 4u * j : (uint32_t)(HO - 4);
+    if (m < 32u && q < 2u * NQD) {
+      aoff[k] = (map * ho2 + second * g.dout_img_stride + start) * 4u;
+      a_second |= second << k;
+    } else {
+      aoff[k] = kOutOfRange;  // the empty run of a map, and the runs past the 32nd map: zeros
     }
-    aoff[k] = off * 4u;
   }
   uint32_t boff[NBW], bmeta[NBW];
 #pragma unroll
@@ -690,7 +696,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   }
   const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
 
-  const int abase = wave * RW + r * AST + h * HO;
+  const int abase = wave * RW + (r * QPM + h * NQD) * 4;
   int bbase[TB];
 #pragma unroll
   for (int b = 0; b < TB; ++b) {
@@ -718,8 +724,8 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   const uint32_t gb_ = (uint32_t)(((size_t)img0_ * g.src_img_stride + ch0 * hs2) * 4);            \
   const uint32_t row0_ = (uint32_t)((y_ - g.pad) * g.hs * 4)
 #define CCT_WSPEC_A(k, st)                                                                        \
-  lds_dma4(a_rsrc, ((second_ >> (k)) & 1u) ? kOutOfRange : aoff[k], ga_,                          \
-           smem + (st) * STAGE + wave * RW + (k) * 64)
+  lds_dma16(a_rsrc, ((second_ >> (k)) & 1u) ? kOutOfRange : aoff[k], ga_,                         \
+            smem + (st) * STAGE + wave * RW + (k) * 256)
 #define CCT_WSPEC_B(k, st)                                                                        \
   do {                                                                                            \
     const uint32_t mt_ = bmeta[k];                                                                \
@@ -744,11 +750,17 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
     CCT_WSPEC_STEP(min(s + 1, s_end - 1));
     const float *sa = smem + cur * STAGE + abase;
     const float *sb = smem + cur * STAGE;
+    // this lane's dout row: all runs at once (NQD 16-byte reads), pixel x is component
+    // x % 4 of run x / 4, or of the overlapping last run
+    f4 aq[NQD];
+#pragma unroll
+    for (int j = 0; j < NQD; ++j) aq[j] = *reinterpret_cast<const f4 *>(sa + 4 * j);
     float fa[2][2], fb[2][2][TB];
+#define CCT_WSPEC_AVAL(x) ((x) < 4 * (NQD - 1) ? aq[(x) / 4][(x) % 4] : aq[NQD - 1][((x) - (HO - 4)) & 3])
 #define CCT_WSPEC_FRAGS(buf, x)                                                                   \
   do {                                                                                            \
-    fa[buf][0] = sa[(x)];                                                                         \
-    fa[buf][1] = sa[(x) + 1];                                                                     \
+    fa[buf][0] = CCT_WSPEC_AVAL(x);                                                               \
+    fa[buf][1] = (x) + 1 < HO ? CCT_WSPEC_AVAL((x) + 1) : 0.0f;                                   \
     _Pragma("unroll") for (int b = 0; b < TB; ++b) {                                              \
       fb[buf][0][b] = sb[bbase[b] + (x)];                                                         \
       fb[buf][1][b] = sb[bbase[b] + (x) + 1];                                                     \
@@ -785,7 +797,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
       // issue order: LDS reads of the next pair first, one per MFMA, then the global loads
       {
         constexpr int NM = 2 * TB;
-        const int nr = (q + 1 < NQ) ? TB + 1 : 0;
+        const int nr = (q + 1 < NQ) ? TB : 0;
         const int nv = (a_hi - a_lo) + (b_hi - b_lo);
         const int nm = (2 * q + 1 < HO) ? NM : TB;
 #pragma unroll
@@ -798,6 +810,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
       }
     }
 #undef CCT_WSPEC_FRAGS
+#undef CCT_WSPEC_AVAL
     lds_dma_wait();
     __syncthreads();
   }
@@ -905,7 +918,7 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
   }
   if (pl->spec) {
     // layout of conv_direct_wgrad_spec_kernel: private slab per wavefront, patches in whole passes
-    const int rw = (32 * pl->ast + 63) / 64 * 64;
+    const int nqd = (ho + 3) / 4, rw = (32 * (2 * nqd + 1) + 63) / 64 * 256;
     pl->a_floats = pl->waves * rw;
     pl->stage = pl->a_floats + (nch * pch + 64 * pl->waves - 1) / (64 * pl->waves) * (64 * pl->waves);
   }
