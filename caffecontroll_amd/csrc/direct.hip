@@ -312,26 +312,63 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   // buffer loads address a tensor through 32-bit byte offsets
   if ((double)batch * kc * hs * hs >= 1073741824.0 || (double)batch * ho * ho >= 2147483648.0) return false;
   const int cp = ks == 3 ? 2 : 1;
-  const int tmb = direct_tmb(mtot);
-  const long tiles_m = (mtot + 32 * tmb - 1) / (32 * tmb);
   const long ptot = (long)batch * ho * ho;
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
-  for (int tnb = 2; tnb >= 1; --tnb) {
-    const int bn = 128 * tnb;
-    const int rows = (ho - 1 + bn - 1) / ho + 1, imgs = (ho * ho - 1 + bn - 1) / (ho * ho) + 1;
-    const int pr = rows - 1 + (imgs - 1) * (ks - 1) + ks;
-    const long patch = 2L * cp * pr * pw;
-    const size_t lds =
-        2 * (size_t)((2 * cp * 32 * tmb * ks * ks + 255) / 256 * 256 + (patch + 63) / 64 * 64) * sizeof(float);
-    const long tiles = tiles_m * ((ptot + bn - 1) / bn);
-    const bool fits = patch <= 256L * kDirectPatchLoads && lds <= 64 * 1024;
-    // the wide tile only when it still gives every compute unit several workgroups
-    if (fits && (tnb == 1 || tiles >= 4L * cus)) {
-      pl->ks = ks; pl->tmb = tmb; pl->tnb = tnb; pl->cp = cp; pl->pw = pw; pl->pr = pr; pl->lds = lds;
-      return true;
+  const int padded = direct_padded_maps(mtot);
+  // tuning override "<map blocks><pixel blocks>", e.g. 22
+  const char *forced_env = getenv("CCT_HIP_DIRECT_TILE");
+  const int forced = forced_env ? atoi(forced_env) : 0;
+  // Candidate tiles: map tiles that divide the padded map count (the slab layout does not depend
+  // on the choice), 128 or 256 pixels.  Estimated time, in units of one 32x128 block on a whole
+  // compute unit: workgroups are handed out as residency slots free up, so the launch runs as
+  // whole rounds of `slots` workgroups per unit plus a last partial round spread over the units; a
+  // unit with one or two resident workgroups does not keep its MFMA pipes full.  The residency
+  // figures follow the register use of the instances (wavefronts per SIMD: 8, 7, 5, 4 for 1..4 map
+  // blocks x 128 pixels; 6, 4, 3, 2 for 256 pixels); a wrong figure costs speed, not correctness.
+  static const int reg_slots[5][3] = {{0, 0, 0}, {0, 8, 6}, {0, 7, 4}, {0, 5, 3}, {0, 4, 2}};
+  static const double fill[4] = {1.0, 0.7, 0.93, 0.97};  // MFMA rate with 1, 2, 3 workgroups on a unit
+  struct Candidate { DirectPlan plan; double cost; } cand[8];
+  int ncand = 0;
+  double best = -1;
+  for (int tmb = 4; tmb >= 1; --tmb) {
+    if (padded % (32 * tmb)) continue;
+    const long tiles_m = padded / (32 * tmb);
+    for (int tnb = 2; tnb >= 1; --tnb) {
+      if (forced && forced != 10 * tmb + tnb) continue;
+      const int bn = 128 * tnb;
+      const int rows = (ho - 1 + bn - 1) / ho + 1, imgs = (ho * ho - 1 + bn - 1) / (ho * ho) + 1;
+      const int pr = rows - 1 + (imgs - 1) * (ks - 1) + ks;
+      const long patch = 2L * cp * pr * pw;
+      const size_t lds =
+          2 * (size_t)((2 * cp * 32 * tmb * ks * ks + 255) / 256 * 256 + (patch + 63) / 64 * 64) * sizeof(float);
+      if (patch > 256L * kDirectPatchLoads || lds > 64 * 1024) continue;
+      const long tiles = tiles_m * ((ptot + bn - 1) / bn);
+      long slots = (long)(160 * 1024 / lds);
+      if (slots > reg_slots[tmb][tnb]) slots = reg_slots[tmb][tnb];
+      const long full = tiles / (cus * slots), rest = tiles - full * cus * slots;
+      const long last = (rest + cus - 1) / cus;
+      const double work = tmb * tnb;
+      const double cost = full * slots * work / (slots < 4 ? fill[slots] : 1.0) +
+                          last * work / (last < 4 ? fill[last] : 1.0);
+      Candidate &c = cand[ncand++];
+      c.plan.ks = ks; c.plan.tmb = tmb; c.plan.tnb = tnb; c.plan.cp = cp; c.plan.pw = pw; c.plan.pr = pr;
+      c.plan.lds = lds;
+      c.cost = cost;
+      if (best < 0 || cost < best) best = cost;
     }
   }
-  return false;
+  if (ncand == 0) return false;
+  // the estimate is good to a few percent: among the candidates that close to the best, the wider
+  // pixel tile (measured a little faster at equal balance), then the lower estimate
+  const Candidate *pick = nullptr;
+  for (int i = 0; i < ncand; ++i) {
+    if (cand[i].cost > best * 1.025) continue;
+    if (!pick || cand[i].plan.tnb > pick->plan.tnb ||
+        (cand[i].plan.tnb == pick->plan.tnb && cand[i].cost < pick->cost))
+      pick = &cand[i];
+  }
+  *pl = pick->plan;
+  return true;
 }
 
 template <int KS, int CP, int PW>
@@ -343,8 +380,8 @@ static int direct_launch_ks(const DirectArgs &g, const DirectPlan &pl, hipStream
     CCT_LAUNCH_CHECK();                                                                                \
     return 0;                                                                                          \
   }
-  CCT_DIRECT_CASE(2, 1) CCT_DIRECT_CASE(3, 1) CCT_DIRECT_CASE(4, 1)
-  CCT_DIRECT_CASE(2, 2) CCT_DIRECT_CASE(3, 2) CCT_DIRECT_CASE(4, 2)
+  CCT_DIRECT_CASE(1, 1) CCT_DIRECT_CASE(2, 1) CCT_DIRECT_CASE(3, 1) CCT_DIRECT_CASE(4, 1)
+  CCT_DIRECT_CASE(1, 2) CCT_DIRECT_CASE(2, 2) CCT_DIRECT_CASE(3, 2) CCT_DIRECT_CASE(4, 2)
 #undef CCT_DIRECT_CASE
   return set_error(CCT_HIP_EINVAL, "conv_direct: no kernel instance for tile %dx%d", pl.tmb, pl.tnb);
 }
