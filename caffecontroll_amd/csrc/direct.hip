@@ -678,16 +678,15 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   constexpr int NCH = (BN - 1) / KK + 2;
   constexpr int BSZ = (NCH * PCH + 64 * W - 1) / (64 * W) * (64 * W);  // patch floats: whole passes
   constexpr int NBW = BSZ / (64 * W);                                   // patch loads per lane per step
-  // dout slab of a wavefront: per map and image the HO row values as NQD runs of four floats (the
-  // last run starts at HO - 4 and overlaps its neighbour when HO is not a multiple of 4), QPM runs
-  // per map including one empty run that makes the map stride an odd number of runs (16-byte reads
-  // of eight neighbouring lanes then fall into eight different bank groups).  One 16-byte global->LDS
-  // load per lane moves a run: a quarter of the load instructions a float-wise copy would take, and
-  // those instructions are what the MFMA pipe otherwise waits on.
-  constexpr int NQD = (HO + 3) / 4, QPM = 2 * NQD + 1;
-  constexpr int NAW = (32 * QPM + 63) / 64;      // slab loads (16 bytes per lane) per lane per step
-  constexpr int RW = NAW * 256;                  // slab floats per wavefront
-  constexpr int AFL = W * RW, STAGE = AFL + BSZ;
+  // dout never passes through LDS: lane (r, h) of a wavefront is the only reader of row y of map r
+  // of image h, so it fetches that row itself, as NQD 16-byte buffer loads (runs of four floats;
+  // the last run starts at HO - 4 and overlaps its neighbour when HO is not a multiple of 4) one
+  // step ahead, into registers.  LDS then holds the source patches only, which lets several
+  // workgroups share a compute unit: their barriers fall at different times and the MFMA pipes
+  // stay fed across them.
+  constexpr int NQD = (HO + 3) / 4;
+  constexpr int NAW = NQD;                       // dout loads (16 bytes per lane) per lane per step
+  constexpr int STAGE = BSZ;
   constexpr int NQ = (HO + 1) / 2;                // x pairs per step
   extern __shared__ __attribute__((aligned(16))) float smem[];
 
@@ -702,22 +701,9 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   constexpr int ho2 = HO * HO;
   const int hs2 = g.hs * g.hs;
 
-  uint32_t aoff[NAW];
-  uint32_t a_second = 0;
-#pragma unroll
-  for (int k = 0; k < NAW; ++k) {
-    const uint32_t e = (uint32_t)(k * 64 + lane);  // run index inside the wavefront's slab
-    const uint32_t m = e / QPM, q = e - m * QPM;
-    const uint32_t map = min((uint32_t)(m0 + wave * 32) + min(m, 31u), (uint32_t)g.o - 1) - m0;
-    const uint32_t second = q >= (uint32_t)NQD ? 1u : 0u, j = q - second * NQD;
-    const uint32_t start = j + 1 < (uint32_t)NQD ? 4u * j : (uint32_t)(HO - 4);
-    if (m < 32u && q < 2u * NQD) {
-      aoff[k] = (map * ho2 + second * g.dout_img_stride + start) * 4u;
-      a_second |= second << k;
-    } else {
-      aoff[k] = kOutOfRange;  // the empty run of a map, and the runs past the 32nd map: zeros
-    }
-  }
+  // byte offset of this lane's dout row within (image pair, first map of the tile, row y)
+  const uint32_t avoff =
+      ((min((uint32_t)(m0 + wave * 32 + r), (uint32_t)g.o - 1) - m0) * ho2 + h * g.dout_img_stride) * 4u;
   uint32_t boff[NBW], bmeta[NBW];
 #pragma unroll
   for (int k = 0; k < NBW; ++k) {
@@ -733,13 +719,12 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   }
   const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
 
-  const int abase = wave * RW + (r * QPM + h * NQD) * 4;
   int bbase[TB];
 #pragma unroll
   for (int b = 0; b < TB; ++b) {
     const int col = min(n0 + b * 32 + r, g.ncols - 1);
     const int c = col / KK, j = col - c * KK, kr = j / KS, kc = j - kr * KS;
-    bbase[b] = AFL + (c - ch0) * PCH + (h * KS + kr) * PWS + kc;
+    bbase[b] = (c - ch0) * PCH + (h * KS + kr) * PWS + kc;
   }
 
   v16f acc[TB];
@@ -757,25 +742,28 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   const int img0_ = 2 * (int)pair_;                                                               \
   const bool two_ = img0_ + 1 < g.batch;                                                          \
   const uint32_t ga_ = (uint32_t)(((size_t)img0_ * g.dout_img_stride + m0 * ho2 + y_ * HO) * 4);  \
-  const uint32_t second_ = two_ ? 0u : a_second;                                                  \
+  const uint32_t av_ = (h && !two_) ? kOutOfRange : avoff;                                        \
   const uint32_t gb_ = (uint32_t)(((size_t)img0_ * g.src_img_stride + ch0 * hs2) * 4);            \
   const uint32_t row0_ = (uint32_t)((y_ - g.pad) * g.hs * 4)
-#define CCT_WSPEC_A(k, st)                                                                        \
-  lds_dma16(a_rsrc, ((second_ >> (k)) & 1u) ? kOutOfRange : aoff[k], ga_,                         \
-            smem + (st) * STAGE + wave * RW + (k) * 256)
+#define CCT_WSPEC_A(k)                                                                            \
+  an[k] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(                           \
+      a_rsrc, av_ + ((k) + 1 < NQD ? 16u * (k) : 4u * (HO - 4)), ga_, 0))
 #define CCT_WSPEC_B(k, st)                                                                        \
   do {                                                                                            \
     const uint32_t mt_ = bmeta[k];                                                                \
     const int srow_ = y_ - g.pad + (int)(mt_ & 15u);                                              \
     const bool ok_ = (mt_ & 32u) && (unsigned)srow_ < (unsigned)g.hs && (two_ || !(mt_ & 16u));   \
     lds_dma4(b_rsrc, ok_ ? boff[k] + row0_ : kOutOfRange, gb_,                                    \
-             smem + (st) * STAGE + AFL + (k) * 64 * W + wave * 64);                               \
+             smem + (st) * STAGE + (k) * 64 * W + wave * 64);                                     \
   } while (0)
 
+  f4 an[NQD];  // this lane's dout row of the coming step
+#pragma unroll
+  for (int k = 0; k < NQD; ++k) an[k] = f4{0.f, 0.f, 0.f, 0.f};
   if (s_beg < s_end) {
     CCT_WSPEC_STEP(s_beg);
 #pragma unroll
-    for (int k = 0; k < NAW; ++k) CCT_WSPEC_A(k, 0);
+    for (int k = 0; k < NAW; ++k) CCT_WSPEC_A(k);
 #pragma unroll
     for (int k = 0; k < NBW; ++k) CCT_WSPEC_B(k, 0);
     lds_dma_wait();
@@ -785,13 +773,12 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   for (int s = s_beg; s < s_end; ++s) {
     const int cur = (s - s_beg) & 1, nxt = cur ^ 1;
     CCT_WSPEC_STEP(min(s + 1, s_end - 1));
-    const float *sa = smem + cur * STAGE + abase;
     const float *sb = smem + cur * STAGE;
-    // this lane's dout row: all runs at once (NQD 16-byte reads), pixel x is component
-    // x % 4 of run x / 4, or of the overlapping last run
+    // this lane's dout row, fetched during the previous step: pixel x is component x % 4 of run
+    // x / 4, or of the overlapping last run
     f4 aq[NQD];
 #pragma unroll
-    for (int j = 0; j < NQD; ++j) aq[j] = *reinterpret_cast<const f4 *>(sa + 4 * j);
+    for (int j = 0; j < NQD; ++j) aq[j] = an[j];
     float fa[2][2], fb[2][2][TB];
 #define CCT_WSPEC_AVAL(x) ((x) < 4 * (NQD - 1) ? aq[(x) / 4][(x) % 4] : aq[NQD - 1][((x) - (HO - 4)) & 3])
 #define CCT_WSPEC_FRAGS(buf, x)                                                                   \
@@ -827,7 +814,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
       const int b_lo = qi * NBW / NQI, b_hi = qj * NBW / NQI;
 #pragma unroll
       for (int k = 0; k < NAW; ++k)
-        if (k >= a_lo && k < a_hi) CCT_WSPEC_A(k, nxt);
+        if (k >= a_lo && k < a_hi) CCT_WSPEC_A(k);
 #pragma unroll
       for (int k = 0; k < NBW; ++k)
         if (k >= b_lo && k < b_hi) CCT_WSPEC_B(k, nxt);
@@ -924,6 +911,10 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
     if (best < 0 || padded < best) { best = padded; best_w = w; }
   }
   pl->waves = best_w;
+  if (const char *e = getenv("CCT_HIP_DIRECT_WAVES")) {  // tuning override
+    const int forced = atoi(e);
+    if (forced >= 4 && forced <= 8) pl->waves = forced;
+  }
   // column blocks per tile: least padding of the column count, wider tile on ties
   const long ncols = (long)d * ks * ks;
   // (narrow tiles re-read the dout slab for few MFMAs each: below 4 blocks only for small layers)
@@ -934,8 +925,9 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
     if (best < 0 || padded < best) { best = padded; best_tb = tb; }
   }
   {
-    static const int forced = [] { const char *e = getenv("CCT_HIP_DIRECT_TB"); return e ? atoi(e) : 0; }();
-    if (forced >= 1 && forced <= 6) best_tb = forced;  // tuning override, read once
+    const char *e = getenv("CCT_HIP_DIRECT_TB");  // tuning override
+    const int forced = e ? atoi(e) : 0;
+    if (forced >= 1 && forced <= 6) best_tb = forced;
   }
   pl->tb = best_tb;
   pl->ast = (2 * ho) | 1;
@@ -954,10 +946,9 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
     if (off) pl->spec = false;  // tuning override, read once
   }
   if (pl->spec) {
-    // layout of conv_direct_wgrad_spec_kernel: private slab per wavefront, patches in whole passes
-    const int nqd = (ho + 3) / 4, rw = (32 * (2 * nqd + 1) + 63) / 64 * 256;
-    pl->a_floats = pl->waves * rw;
-    pl->stage = pl->a_floats + (nch * pch + 64 * pl->waves - 1) / (64 * pl->waves) * (64 * pl->waves);
+    // layout of conv_direct_wgrad_spec_kernel: dout stays out of LDS, patches in whole passes
+    pl->a_floats = 0;
+    pl->stage = (nch * pch + 64 * pl->waves - 1) / (64 * pl->waves) * (64 * pl->waves);
   }
   // fragment loads may run a few words past the last patch row: the padding of the patch region
   // absorbs that, else a little slack is added
