@@ -39,8 +39,8 @@ GEMM_TRAFFIC_BYTES = {
     (2, "GEMM"): (1868.6 + 192.4) * 1e6,
     (2, "GEMM Data"): (280.4 + 73.5) * 1e6,
     (2, "GEMM Wghts"): (2143.4 + 63.9) * 1e6,
-    (3, "GEMM"): (136.1 + 249.1) * 1e6,
-    (3, "GEMM Data"): (280.4 + 73.5) * 1e6,
+    (3, "GEMM"): (230.1 + 223.7) * 1e6,
+    (3, "GEMM Data"): (322.3 + 75.7) * 1e6,
     (3, "GEMM Wghts"): (359.6 + 41.8) * 1e6,
 }
 
