@@ -267,7 +267,8 @@ __global__ __launch_bounds__(TPB) void maxpool_fwd_plane_kernel(float *__restric
                                                                 const float *__restrict__ in, cct_pool_args a,
                                                                 uint32_t planes, int pp, FastDiv div_oc,
                                                                 FastDiv div_oplane) {
-  __shared__ float tile[kPoolLdsWords];
+  extern __shared__ float pool_lds[];  // pp * iplane words, sized by the launch
+  float *tile = pool_lds;
   const uint32_t p0 = blockIdx.x * (uint32_t)pp;
   const uint32_t np = min((uint32_t)pp, planes - p0);
   const uint32_t iplane = (uint32_t)(a.iR * a.iC), oplane = (uint32_t)(a.oR * a.oC);
@@ -336,6 +337,81 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_plane_kernel(float *__restric
   }
 }
 
+// The same for 2 <= stride, kernel <= 2*stride and rows of at most 256 elements, four consecutive
+// elements of a row per lane: `lpr` lanes per row (the power of two >= ceil(iC / 4)), 64 / lpr rows
+// per wavefront and pass.  The windows that can hold any of the four elements lie in two window
+// rows and at most four window columns; the lane reads those eight (argmax, gradient) pairs once
+// and tests each against its four positions -- an argmax equals a position only if the window
+// contains it, so no range logic is needed beyond masking the clamped duplicates at the borders.
+// Additions stay in (ph, pw) order.  One 16-byte store per lane instead of four 4-byte ones, and
+// a quarter of the LDS reads and index arithmetic of the element-wise kernel.
+__global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict__ ig, const float *__restrict__ og,
+                                                               const int *__restrict__ idx, cct_pool_args a,
+                                                               uint32_t planes, int pp, int lpr_shift, FastDiv div_ir,
+                                                               FastDiv div_s) {
+  // LDS sized by the launch (2 * pp * oplane words): small planes leave room for more workgroups
+  // per compute unit, whose load and store phases then overlap
+  extern __shared__ float pool_lds[];
+  const uint32_t p0 = blockIdx.x * (uint32_t)pp;
+  const uint32_t np = min((uint32_t)pp, planes - p0);
+  const uint32_t iplane = (uint32_t)(a.iR * a.iC), oplane = (uint32_t)(a.oR * a.oC);
+  float *tog = pool_lds;
+  int *tidx = reinterpret_cast<int *>(pool_lds + (size_t)pp * oplane);
+  pool_stage<pool_f4u, float, 4>(tog, og + (size_t)p0 * oplane, np * oplane);
+  pool_stage<pool_i4u, int, 4>(tidx, idx + (size_t)p0 * oplane, np * oplane);
+  __syncthreads();
+  const int k = a.kernel_size;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int w0 = 4 * (lane & ((1 << lpr_shift) - 1)), rows_per_wave = 64 >> lpr_shift;
+  if (w0 >= a.iC) return;
+  const int nw = min(4, a.iC - w0);  // elements of this lane's quad inside the row
+  // window columns pc0 .. pc0+3 (clamped; cv[j] false for the duplicates the clamp makes)
+  const int pc0 = w0 < k ? 0 : (int)fdiv((uint32_t)(w0 - k), div_s) + 1;
+  int pc[4];
+  bool cv[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    pc[j] = min(pc0 + j, a.oC - 1);
+    cv[j] = pc0 + j <= a.oC - 1;
+  }
+  float *dst = ig + (size_t)p0 * iplane + w0;
+  const uint32_t nrows = np * (uint32_t)a.iR;
+  for (uint32_t row = wave * rows_per_wave + (lane >> lpr_shift); row < nrows; row += (TPB / 64) * rows_per_wave) {
+    const uint32_t pl = fdiv(row, div_ir);
+    const int h = (int)(row - pl * a.iR), me0 = h * a.iC + w0;
+    const int ph_lo = h < k ? 0 : (int)fdiv((uint32_t)(h - k), div_s) + 1;
+    const bool row1 = ph_lo + 1 <= a.oR - 1;
+    const float *g = tog + pl * oplane;
+    const int *x = tidx + pl * oplane;
+    const int r0 = ph_lo * a.oC, r1 = min(ph_lo + 1, a.oR - 1) * a.oC;
+    int xi[2][4];
+    float gv[2][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      xi[0][j] = x[r0 + pc[j]]; gv[0][j] = g[r0 + pc[j]];
+      xi[1][j] = x[r1 + pc[j]]; gv[1][j] = g[r1 + pc[j]];
+    }
+    pool_f4u acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool ok = cv[j] && (i == 0 || row1);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (ok && xi[i][j] == me0 + e) acc[e] += gv[i][j];
+      }
+    float *o = dst + (size_t)row * a.iC;
+    if (nw == 4) {
+      *reinterpret_cast<pool_f4u *>(o) = acc;
+    } else {
+      o[0] = acc[0];
+      if (nw > 1) o[1] = acc[1];
+      if (nw > 2) o[2] = acc[2];
+    }
+  }
+}
+
 // CCT_HIP_POOL_PLANE=1 takes the plane-tiled kernels at any size (used by the tests on small shapes)
 static bool force_pool_plane() {
   const char *e = getenv("CCT_HIP_POOL_PLANE");
@@ -347,7 +423,9 @@ static int pool_planes_per_block(size_t plane_words, size_t work_words, size_t p
   // small tensors are launch-bound; the one-lane-per-element kernels finish them sooner
   if (planes * (plane_words > work_words ? plane_words : work_words) < (1u << 20) && !force_pool_plane()) return 0;
   if (plane_words == 0 || plane_words > (size_t)kPoolLdsWords) return 0;
-  size_t pp = kPoolLdsWords / plane_words;
+  // at most 20 KB of LDS per workgroup where a plane allows it: eight workgroups share a compute
+  // unit and their load and store phases overlap
+  size_t pp = plane_words > 5120 ? 1 : 5120 / plane_words;
   const size_t want = (2048 + work_words - 1) / work_words;  // ~8 elements per lane
   if (pp > want) pp = want;
   if (pp > planes) pp = planes;
@@ -735,7 +813,8 @@ int cct_hip_maxpool_forward(float *out, const float *in, const cct_pool_args *a)
   if (total == 0) return 0;
   const size_t planes = (size_t)a->D * a->B, iplane = (size_t)a->iR * a->iC, oplane = (size_t)a->oR * a->oC;
   if (const int pp = pool_planes_per_block(iplane, oplane, planes)) {
-    hipLaunchKernelGGL(maxpool_fwd_plane_kernel, dim3((uint32_t)((planes + pp - 1) / pp)), dim3(TPB), 0, ctx().stream,
+    hipLaunchKernelGGL(maxpool_fwd_plane_kernel, dim3((uint32_t)((planes + pp - 1) / pp)), dim3(TPB),
+                       (size_t)pp * iplane * sizeof(float), ctx().stream,
                        out, a->max_index, in, *a, (uint32_t)planes, pp, make_fastdiv(a->oC),
                        make_fastdiv((uint32_t)oplane));
     CCT_LAUNCH_CHECK();
@@ -757,7 +836,12 @@ int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_po
   const size_t planes = (size_t)a->D * a->B, iplane = (size_t)a->iR * a->iC, oplane = (size_t)a->oR * a->oC;
   if (const int pp = pool_planes_per_block(2 * oplane, iplane, planes)) {
     const dim3 grid((uint32_t)((planes + pp - 1) / pp));
-    if (a->kernel_size <= 2 * a->stride)
+    if (a->stride >= 2 && a->kernel_size <= 2 * a->stride && a->iC <= 256) {
+      int lpr_shift = 0;
+      while ((4 << lpr_shift) < a->iC) ++lpr_shift;
+      hipLaunchKernelGGL(maxpool_bwd_quad_kernel, grid, dim3(TPB), (size_t)2 * pp * oplane * sizeof(float), ctx().stream, in_grad, out_grad, a->max_index,
+                         *a, (uint32_t)planes, pp, lpr_shift, make_fastdiv(a->iR), make_fastdiv(a->stride));
+    } else if (a->kernel_size <= 2 * a->stride)
       hipLaunchKernelGGL(maxpool_bwd_plane_kernel<true>, grid, dim3(TPB), 0, ctx().stream, in_grad, out_grad,
                          a->max_index, *a, (uint32_t)planes, pp, make_fastdiv(a->iC), make_fastdiv((uint32_t)iplane),
                          make_fastdiv(a->stride));

@@ -35,7 +35,9 @@ def test_relu_fixture_and_oracle(oracle):
 @pytest.mark.parametrize("cfg", [(5, 3, 10, 4, 2), (2, 4, 13, 3, 2), (3, 2, 24, 2, 2), (2, 3, 55, 3, 2), (1, 2, 7, 3, 1),
                                  # several planes per workgroup with a partial last group; planes too large
                                  # for the LDS-tiled kernels (forward only, both, window wider than 2 strides)
-                                 (7, 11, 13, 3, 2), (1, 2, 100, 3, 2), (1, 1, 150, 2, 2), (1, 1, 140, 5, 2)])
+                                 (7, 11, 13, 3, 2), (1, 2, 100, 3, 2), (1, 1, 150, 2, 2), (1, 1, 140, 5, 2),
+                                 # rows of 27, 64 and 65 elements: the lanes-over-rows backward kernel and its limit
+                                 (3, 5, 27, 3, 2), (2, 3, 64, 3, 2), (2, 3, 65, 2, 2)])
 @pytest.mark.parametrize("plane_tiled", [False, True])
 def test_maxpool_bit_exact(oracle, cfg, plane_tiled, monkeypatch):
     # small tensors take the one-lane-per-element kernels unless the plane-tiled ones are forced
