@@ -348,7 +348,9 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_plane_kernel(float *__restric
 __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict__ ig, const float *__restrict__ og,
                                                                const int *__restrict__ idx, cct_pool_args a,
                                                                uint32_t planes, int pp, int lpr_shift, FastDiv div_ir,
-                                                               FastDiv div_s) {
+                                                               FastDiv div_s, const float *__restrict__ relu_data) {
+  // relu_data (optional): the pooled tensor itself when it is the output of an in-place ReLU; the
+  // gradient is then stored already masked with (relu_data > 0), which is that ReLU's backward.
   // LDS sized by the launch (2 * pp * oplane words): small planes leave room for more workgroups
   // per compute unit, whose load and store phases then overlap
   extern __shared__ float pool_lds[];
@@ -402,6 +404,16 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict
           if (ok && xi[i][j] == me0 + e) acc[e] += gv[i][j];
       }
     float *o = dst + (size_t)row * a.iC;
+    if (relu_data) {
+      const float *y = relu_data + (o - ig);
+      if (nw == 4) {
+        const pool_f4u yv = *reinterpret_cast<const pool_f4u *>(y);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] = yv[e] > 0.0f ? acc[e] : 0.0f;
+      } else {
+        for (int e = 0; e < nw; ++e) acc[e] = y[e] > 0.0f ? acc[e] : 0.0f;
+      }
+    }
     if (nw == 4) {
       *reinterpret_cast<pool_f4u *>(o) = acc;
     } else {
@@ -826,8 +838,8 @@ int cct_hip_maxpool_forward(float *out, const float *in, const cct_pool_args *a)
   return 0;
 }
 
-int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_pool_args *a) {
-  CCT_ENSURE_INIT();
+static int maxpool_backward_impl(float *in_grad, const float *out_grad, const cct_pool_args *a,
+                                 const float *relu_data) {
   CCT_REQUIRE(in_grad && out_grad, "maxpool_backward: null argument");
   int rc = check_pool(a, "maxpool_backward");
   if (rc) return rc;
@@ -839,8 +851,10 @@ int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_po
     if (a->stride >= 2 && a->kernel_size <= 2 * a->stride && a->iC <= 256) {
       int lpr_shift = 0;
       while ((4 << lpr_shift) < a->iC) ++lpr_shift;
-      hipLaunchKernelGGL(maxpool_bwd_quad_kernel, grid, dim3(TPB), (size_t)2 * pp * oplane * sizeof(float), ctx().stream, in_grad, out_grad, a->max_index,
-                         *a, (uint32_t)planes, pp, lpr_shift, make_fastdiv(a->iR), make_fastdiv(a->stride));
+      hipLaunchKernelGGL(maxpool_bwd_quad_kernel, grid, dim3(TPB), (size_t)2 * pp * oplane * sizeof(float),
+                         ctx().stream, in_grad, out_grad, a->max_index, *a, (uint32_t)planes, pp, lpr_shift,
+                         make_fastdiv(a->iR), make_fastdiv(a->stride), relu_data);
+      relu_data = nullptr;  // done inside the kernel
     } else if (a->kernel_size <= 2 * a->stride)
       hipLaunchKernelGGL(maxpool_bwd_plane_kernel<true>, grid, dim3(TPB), 0, ctx().stream, in_grad, out_grad,
                          a->max_index, *a, (uint32_t)planes, pp, make_fastdiv(a->iC), make_fastdiv((uint32_t)iplane),
@@ -850,7 +864,8 @@ int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_po
                          a->max_index, *a, (uint32_t)planes, pp, make_fastdiv(a->iC), make_fastdiv((uint32_t)iplane),
                          make_fastdiv(a->stride));
     CCT_LAUNCH_CHECK();
-    return 0;
+    // the other kernels do not mask: a separate pass does
+    return relu_data ? cct_hip_relu_backward(in_grad, in_grad, relu_data, total) : 0;
   }
   if (a->kernel_size <= 2 * a->stride)
     hipLaunchKernelGGL(maxpool_bwd_kernel<true>, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad,
@@ -859,7 +874,19 @@ int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_po
     hipLaunchKernelGGL(maxpool_bwd_kernel<false>, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad,
                        out_grad, a->max_index, *a, (uint32_t)total, make_fastdiv(a->iC), make_fastdiv(a->iR));
   CCT_LAUNCH_CHECK();
-  return 0;
+  return relu_data ? cct_hip_relu_backward(in_grad, in_grad, relu_data, total) : 0;
+}
+
+int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_pool_args *a) {
+  CCT_ENSURE_INIT();
+  return maxpool_backward_impl(in_grad, out_grad, a, nullptr);
+}
+
+int cct_hip_maxpool_backward_relu(float *in_grad, const float *out_grad, const cct_pool_args *a,
+                                  const float *relu_data) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(relu_data, "maxpool_backward_relu: null activation tensor");
+  return maxpool_backward_impl(in_grad, out_grad, a, relu_data);
 }
 
 int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args *a,

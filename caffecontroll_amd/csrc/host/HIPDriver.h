@@ -110,6 +110,12 @@ class HIPDriver {
     // (output_grad, input_grad) -- CPUDriver::maxpool_backward reads dst and writes src
     ok(cct_hip_maxpool_backward((float *)src->ptr, (const float *)dst->ptr, &args), "maxpool_backward");
   }
+  // the same followed by the backward of an in-place ReLU on the pooled tensor `relu_data`
+  void maxpool_backward_relu(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const _pool_backward_arg_helper args,
+                             const float *relu_data) {
+    ok(cct_hip_maxpool_backward_relu((float *)src->ptr, (const float *)dst->ptr, &args, relu_data),
+       "maxpool_backward_relu");
+  }
 
   // ---- the parallel_map pairs of the reference, by name ----
   void relu_forward(DeviceMemoryPointer *dst, DeviceMemoryPointer *src) {

@@ -146,7 +146,14 @@ class Network {
           lp->pooling_param_.kernel_size_ = s.kernel_size;
           lp->pooling_param_.stride_ = s.stride;
           nd.params.push_back(lp);
-          nd.bridges.push_back(new MaxPoolingBridge<float, HIPDriver>(cur, nd.out, lp, &solver_, &driver_));
+          auto *pb = new MaxPoolingBridge<float, HIPDriver>(cur, nd.out, lp, &solver_, &driver_);
+          // directly after an in-place ReLU the pooling backward stores the gradient already masked
+          // and the ReLU bridge skips its own backward pass over the tensor
+          if (!nodes_.empty() && nodes_.back().spec.type == CCT_LAYER_RELU && nodes_.back().out == cur) {
+            pb->input_is_relu_output = true;
+            static_cast<ReLUBridge<float, HIPDriver> *>(nodes_.back().bridges[0])->backward_done_by_consumer = true;
+          }
+          nd.bridges.push_back(pb);
           break;
         }
         case CCT_LAYER_LRN: {

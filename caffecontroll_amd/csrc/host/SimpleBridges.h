@@ -48,7 +48,10 @@ class ReLUBridge : public AbstractBridge<DataType, DriverClass> {
   }
   // With shared layers the data cube holds y = max(x,0) by now; (y > 0) == (x > 0), so the same
   // mask results, as in the reference (ReLUBridge_impl.hxx:80-88 passes the input data pointer).
+  // set when the consuming bridge (max pooling after an in-place ReLU) masks the gradient it stores
+  bool backward_done_by_consumer = false;
   void backward() override {
+    if (backward_done_by_consumer) return;
     DeviceMemoryPointer in_grad = p_input_layer->p_gradient_cube->get_device_pointer(p_driver);
     DeviceMemoryPointer out_grad = p_output_layer->p_gradient_cube->get_device_pointer(p_driver);
     p_driver->relu_backward(&in_grad, &out_grad, p_input_layer->p_data_cube->get_p_data());
@@ -84,8 +87,14 @@ class MaxPoolingBridge : public AbstractBridge<DataType, DriverClass> {
   void backward() override {
     DeviceMemoryPointer input = p_input_layer->p_gradient_cube->get_device_pointer(p_driver);
     DeviceMemoryPointer output = p_output_layer->p_gradient_cube->get_device_pointer(p_driver);
-    p_driver->maxpool_backward(&output, &input, args());
+    if (input_is_relu_output)
+      p_driver->maxpool_backward_relu(&output, &input, args(), p_input_layer->p_data_cube->get_p_data());
+    else
+      p_driver->maxpool_backward(&output, &input, args());
   }
+  // the input layer is the output of an in-place ReLU whose backward this bridge performs while it
+  // stores the gradient (the ReLU bridge then skips its own)
+  bool input_is_relu_output = false;
 
  private:
   LogicalCube<int> *max_index;

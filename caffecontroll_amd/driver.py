@@ -190,7 +190,13 @@ class HIPDriver:
     def maxpool_forward(self, out, inp, args):
         check(self.lib.cct_hip_maxpool_forward(_p(out), _p(inp), C.byref(args)), "maxpool_forward")
 
-    def maxpool_backward(self, in_grad, out_grad, args):
+    def maxpool_backward(self, in_grad, out_grad, args, relu_data=None):
+        """relu_data: the pooled tensor when it is the output of an in-place ReLU; the gradient then
+        comes out already masked with (relu_data > 0)."""
+        if relu_data is not None:
+            check(self.lib.cct_hip_maxpool_backward_relu(_p(in_grad), _p(out_grad), C.byref(args), _p(relu_data)),
+                  "maxpool_backward_relu")
+            return
         check(self.lib.cct_hip_maxpool_backward(_p(in_grad), _p(out_grad), C.byref(args)), "maxpool_backward")
 
     def lrn_forward(self, out, inp, R, Cc, D, B, local_size, alpha, beta, denoms):

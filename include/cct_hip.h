@@ -238,6 +238,12 @@ int cct_hip_relu_backward(float *in_grad, const float *out_grad, const float *in
  * (no -FLT_MAX pre-fill needed); backward overwrites in_grad (no zero fill needed). */
 int cct_hip_maxpool_forward(float *out, const float *in, const cct_pool_args *args);
 int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_pool_args *args);
+/* MaxPoolingBridge::backward followed by the backward of an in-place ReLU on the pooled tensor
+ * (src/bridges/MaxPoolingBridge_impl.hxx:114-151 then src/bridges/ReLUBridge_impl.hxx:62-100, the
+ * order DeepNet::run_backward_pass visits them): in_grad = pooling gradient where relu_data > 0,
+ * else 0; relu_data is the pooled tensor (the ReLU's output), same shape as in_grad. */
+int cct_hip_maxpool_backward_relu(float *in_grad, const float *out_grad, const cct_pool_args *args,
+                                  const float *relu_data);
 /* DeviceDriver::lrn_forward/lrn_backward, src/sched/DeviceDriver.h:140-147. */
 int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args *args,
                         const cct_lrn_forward_normalize_args *args2);

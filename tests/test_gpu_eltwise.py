@@ -67,6 +67,12 @@ def test_maxpool_bit_exact(oracle, cfg, plane_tiled, monkeypatch):
     g = empty(x.shape)
     drv.maxpool_backward(g, dev(og), args)
     np.testing.assert_array_equal(host(g), oracle.maxpool_backward(og, ridx, n, n))
+    # with the backward of an in-place ReLU on the pooled tensor folded in: the same gradient where
+    # the tensor is positive, zero elsewhere (x holds zeros, so the mask bites)
+    g2 = empty(x.shape)
+    drv.maxpool_backward(g2, dev(og), args, relu_data=dev(x))
+    np.testing.assert_array_equal(host(g2), oracle.relu_backward(host(g), x))
+    assert cfg == (5, 3, 10, 4, 2) or (x <= 0).any()
     if cfg == (5, 3, 10, 4, 2):
         np.testing.assert_allclose(host(y).reshape(-1), load_fixture("output", "pooling_forward.txt"), atol=1e-3)
         np.testing.assert_allclose(host(g).reshape(-1), load_fixture("output", "pooling_backward.txt"), atol=1e-3)
