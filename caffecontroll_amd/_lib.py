@@ -68,6 +68,7 @@ PROTOTYPES = {
     "cct_hip_inverse_lower_cube": [_P, _P, C.POINTER(InverseLowerCubeArgs)],
     "cct_hip_inverse_lower_cube_bias_backward": [_P, _P, C.POINTER(InverseLowerCubeArgs), _P, _P, _I, _I, _I],
     "cct_hip_remap": [_P, _P, C.POINTER(PMapHelper)],
+    "cct_hip_remap_bias_backward": [_P, _P, C.POINTER(PMapHelper), _P],
     "cct_hip_copy_depth_slice": [_P, _P, _I, _I, _I, _I, _Z, _I],
     "cct_hip_sgemm": [_I, _I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I],
     "cct_hip_sgemm_new": [_I, _I, _I, _I, _I, _F, _P, _P, _F, _P],

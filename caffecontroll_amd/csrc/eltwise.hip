@@ -78,6 +78,56 @@ __global__ __launch_bounds__(TPB) void remap_kernel(float *__restrict__ dst, con
   if (blockIdx.y == 0 && threadIdx.x < (rc & 3u)) d[4 * nq + threadIdx.x] = s[4 * nq + threadIdx.x];
 }
 
+// The same copy for the backward pass of a convolution that also wants its bias gradient: source
+// slice j = (image j / sB, map j % sB); while a workgroup moves its part of a slice it adds up
+// what it moves (lanes in a fixed pattern, then a workgroup reduction) and leaves the sum in
+// partial[j * gridDim.y + part].  bias_partial_sum_kernel adds those per map in a fixed order.
+__global__ __launch_bounds__(TPB) void remap_bias_kernel(float *__restrict__ dst, const float *__restrict__ src,
+                                                         uint32_t rc, uint32_t sD, FastDiv div_b,
+                                                         float *__restrict__ partial) {
+  __shared__ float red[8];
+  const uint32_t j = blockIdx.x;  // source slice
+  const uint32_t reald = fdiv(j, div_b);
+  const uint32_t realb = j - reald * div_b.div;
+  const float *s = src + (size_t)j * rc;
+  float *d = dst + ((size_t)reald + (size_t)realb * sD) * rc;
+  const uint32_t nq = rc >> 2, stride = gridDim.y * TPB;
+  float sum = 0.0f;
+  for (uint32_t q0 = blockIdx.y * TPB + threadIdx.x; q0 < nq; q0 += 4 * stride) {
+    remap_f4u v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (q0 + u * stride < nq) v[u] = *reinterpret_cast<const remap_f4u *>(s + 4 * (size_t)(q0 + u * stride));
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (q0 + u * stride < nq) {
+        *reinterpret_cast<remap_f4u *>(d + 4 * (size_t)(q0 + u * stride)) = v[u];
+        sum += (v[u][0] + v[u][1]) + (v[u][2] + v[u][3]);
+      }
+  }
+  if (blockIdx.y == 0 && threadIdx.x < (rc & 3u)) {
+    const float t = s[4 * nq + threadIdx.x];
+    d[4 * nq + threadIdx.x] = t;
+    sum += t;
+  }
+  sum = block_reduce<false>(sum, red);
+  if (threadIdx.x == 0) partial[(size_t)j * gridDim.y + blockIdx.y] = sum;
+}
+
+// bias[o] = sum over images b and parts of partial[(b * O + o) * parts + part]; one workgroup per map
+__global__ __launch_bounds__(TPB) void bias_partial_sum_kernel(float *__restrict__ bias, const float *__restrict__ partial,
+                                                               uint32_t O, uint32_t B, uint32_t parts) {
+  __shared__ float red[8];
+  const uint32_t o = blockIdx.x;
+  float sum = 0.0f;
+  for (uint32_t i = threadIdx.x; i < B * parts; i += TPB) {
+    const uint32_t b = i / parts, part = i - b * parts;
+    sum += partial[((size_t)b * O + o) * parts + part];
+  }
+  sum = block_reduce<false>(sum, red);
+  if (threadIdx.x == 0) bias[o] = sum;
+}
+
 // ---- depth-slice copy: part [B][dc][rc] <-> channels [d_off, d_off+dc) of whole [B][D][rc] ----------
 __global__ __launch_bounds__(TPB) void depth_slice_kernel(float *__restrict__ part, float *__restrict__ whole,
                                                           uint32_t per_image, uint32_t whole_stride,
@@ -732,6 +782,31 @@ int cct_hip_remap(float *dst, const float *src, const cct_pmap_helper *a) {
   if (gy > 64) gy = 64;
   hipLaunchKernelGGL(remap_kernel, dim3((uint32_t)slices, gy), dim3(TPB), 0, ctx().stream, dst, src,
                      (uint32_t)rc, (uint32_t)a->sD, make_fastdiv((uint32_t)a->sB));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_remap_bias_backward(float *dst, const float *src, const cct_pmap_helper *a, float *bias_grad) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(dst && src && a && bias_grad, "remap_bias_backward: null argument");
+  const size_t rc = a->sR * a->sC, slices = a->sD * a->sB;
+  if (a->sB == 0) return 0;
+  if (rc == 0 || a->sD == 0) return cct_hip_sconstant_initialize(bias_grad, a->sB, 0.0f);
+  CCT_REQUIRE(slices < (1ull << 31) && rc < (1ull << 31), "remap_bias_backward: too many slices");
+  const char *d0 = (const char *)dst, *s0 = (const char *)src;
+  const size_t bytes = rc * slices * 4;
+  CCT_REQUIRE(d0 + bytes <= s0 || s0 + bytes <= d0, "remap_bias_backward: dst and src overlap");
+  uint32_t gy = (uint32_t)((rc / 4 + 4 * TPB - 1) / (4 * TPB));
+  if (gy < 1) gy = 1;
+  if (gy > 64) gy = 64;
+  void *ws = nullptr;
+  int rc_ws = get_workspace(slices * gy * sizeof(float), &ws);
+  if (rc_ws) return rc_ws;
+  hipLaunchKernelGGL(remap_bias_kernel, dim3((uint32_t)slices, gy), dim3(TPB), 0, ctx().stream, dst, src,
+                     (uint32_t)rc, (uint32_t)a->sD, make_fastdiv((uint32_t)a->sB), (float *)ws);
+  CCT_LAUNCH_CHECK();
+  hipLaunchKernelGGL(bias_partial_sum_kernel, dim3((uint32_t)a->sB), dim3(TPB), 0, ctx().stream, bias_grad,
+                     (const float *)ws, (uint32_t)a->sB, (uint32_t)a->sD, gy);
   CCT_LAUNCH_CHECK();
   return 0;
 }

@@ -46,8 +46,10 @@ class Connector {
 
   // [depth][batch] slices of `src` -> [batch][depth] slices of `dst` (out of place; the reference
   // copies the cube and permutes back into it, Connector_impl_Lowering_type1.hxx:92-128)
+  // With `bias_grad` (backward pass, `batch` = number of maps) the same pass also leaves the maps'
+  // bias gradient there.
   void remap_output(LogicalCube<DataType> &dst, const LogicalCube<DataType> &src, const size_t depth,
-                    const size_t batch) {
+                    const size_t batch, const LogicalCube<DataType> *bias_grad = nullptr) {
     DeviceMemoryPointer d = dst.get_device_pointer(p_driver);
     DeviceMemoryPointer s = src.get_device_pointer(p_driver);
     PMapHelper args = {};
@@ -57,7 +59,12 @@ class Connector {
     args.sBR = std::min((size_t)16, args.sR); args.sBC = std::min((size_t)16, args.sC);
     args.stride = stride;
     args.padding = padding;
-    p_driver->pmap2d_read_coalesce_remap(&d, &s, args);
+    if (bias_grad) {
+      DeviceMemoryPointer b = bias_grad->get_device_pointer(p_driver);
+      p_driver->pmap2d_read_coalesce_remap_bias_backward(&d, &s, args, &b);
+    } else {
+      p_driver->pmap2d_read_coalesce_remap(&d, &s, args);
+    }
   }
 
   _inverse_lower_cube_arg_helper inverse_args() const {

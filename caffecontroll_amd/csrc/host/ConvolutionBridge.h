@@ -260,7 +260,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
 
     const bool fuse_bias_into_lift = bias_term && needs_to_calc_backward_grad && path_ == PATH_FUSED;
     // on the all-direct path the weight-gradient kernel reduces the bias gradient as well
-    if (bias_term && !fuse_bias_into_lift && !direct_weights) {
+    // a layer without an input gradient has no lifting kernel to carry the bias gradient: the
+    // remap pass sums it while it copies (staged path: the separate passes of the reference)
+    const bool fuse_bias_into_remap = bias_term && !fuse_bias_into_lift && !direct_weights && path_ >= PATH_FUSED;
+    if (bias_term && !fuse_bias_into_lift && !direct_weights && !fuse_bias_into_remap) {
       begin(STAGE_BW_BIAS);
       DeviceMemoryPointer bias = p_bias_gradient_cube->get_device_pointer(p_driver);
       p_driver->backward_bias(&bias, &og, (int)(oR * oC), (int)oD, (int)iB);
@@ -268,7 +271,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     }
     if (!direct_weights) {
       begin(STAGE_BW_REMAP);
-      p_forward_lower_connector->remap_output(*staging(), *output_g_cube, oB, num_output_features);
+      p_forward_lower_connector->remap_output(*staging(), *output_g_cube, oB, num_output_features,
+                                              fuse_bias_into_remap ? p_bias_gradient_cube : nullptr);
       end(STAGE_BW_REMAP);
     }
     LogicalCubeType lowered_outputgrad(direct_weights ? nullptr : staging()->get_p_data(), num_output_features,

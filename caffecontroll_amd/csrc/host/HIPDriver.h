@@ -62,6 +62,12 @@ class HIPDriver {
   void pmap2d_read_coalesce_remap(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const PMapHelper args) {
     ok(cct_hip_remap((float *)dst->ptr, (const float *)src->ptr, &args), "remap");
   }
+  // the backward remap of a convolution together with its bias gradient (one pass over the tensor)
+  void pmap2d_read_coalesce_remap_bias_backward(DeviceMemoryPointer *dst, DeviceMemoryPointer *src,
+                                                const PMapHelper args, DeviceMemoryPointer *bias) {
+    ok(cct_hip_remap_bias_backward((float *)dst->ptr, (const float *)src->ptr, &args, (float *)bias->ptr),
+       "remap_bias_backward");
+  }
   void inverse_lower_cube(DeviceMemoryPointer *dst, DeviceMemoryPointer *src,
                           const _inverse_lower_cube_arg_helper args) {
     ok(cct_hip_inverse_lower_cube((float *)dst->ptr, (const float *)src->ptr, &args), "inverse_lower_cube");

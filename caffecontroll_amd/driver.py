@@ -101,6 +101,11 @@ class HIPDriver:
     def remap(self, dst, src, args):
         check(self.lib.cct_hip_remap(_p(dst), _p(src), C.byref(args)), "remap")
 
+    def remap_bias_backward(self, dst, src, args, bias_grad):
+        """remap plus the bias gradient of the maps (source slice j belongs to map j % sB)."""
+        check(self.lib.cct_hip_remap_bias_backward(_p(dst), _p(src), C.byref(args), _p(bias_grad)),
+              "remap_bias_backward")
+
     # -- BLAS-shaped ------------------------------------------------------------------------
     def sgemm(self, order, TA, TB, M, N, K, alpha, A, lda, B, ldb, beta, Cm, ldc):
         check(self.lib.cct_hip_sgemm(order, TA, TB, M, N, K, alpha, _p(A), lda, _p(B), ldb, beta,

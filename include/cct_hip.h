@@ -134,6 +134,12 @@ int cct_hip_inverse_lower_cube_bias_backward(float *dst, const float *src,
  * src/kernels/lowering.hxx:241-258): slice j of src (sR*sC floats, j < sD*sB) goes to slice
  * (j / sB) + (j % sB) * sD of dst.  dst and src must not overlap. */
 int cct_hip_remap(float *dst, const float *src, const cct_pmap_helper *args);
+/* The backward remap of a convolution's output gradient ([image][map] slices -> [map][image]
+ * slices, src/bridges/ConvolutionBridge_impl.hxx:601-605) together with the bias gradient
+ * (ConvolutionBridge_impl.hxx:575-599) in one pass over the tensor: source slice j belongs to map
+ * j % sB, and bias_grad[o] (sB entries) = sum of every element of map o's slices.  Used when the
+ * layer needs no input gradient (first layer), so no lifting kernel is there to carry the sum. */
+int cct_hip_remap_bias_backward(float *dst, const float *src, const cct_pmap_helper *args, float *bias_grad);
 
 /* Depth-slice copy between a contiguous cube part [B][d_count][rc] and channels
  * [d_off, d_off + d_count) of whole [B][d_total][rc]; gather != 0: whole -> part, else part -> whole.

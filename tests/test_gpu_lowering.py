@@ -83,6 +83,27 @@ def test_remap_bit_exact(oracle, dims):
     np.testing.assert_array_equal(host(dst), oracle.remap(x, R, Cc, depth, batch))
 
 
+@pytest.mark.parametrize("dims", [(5, 5, 4, 10), (55, 55, 3, 6), (1, 1, 7, 5), (70, 70, 2, 3), (3, 2, 1, 1)])
+def test_remap_with_bias_gradient(oracle, dims):
+    """The backward remap of a convolution ([image][map] -> [map][image] slices) that also sums each
+    map's slices: the copy is bit-exact, the sums agree with the oracle's bias gradient and with
+    float64 within the fp32 tolerance, and a second run gives the same bits."""
+    from caffecontroll_amd.driver import remap_pmap
+    R, Cc, images, maps = dims
+    rng = np.random.default_rng(17 + sum(dims))
+    x = rng.standard_normal((images, maps, R, Cc)).astype(np.float32)
+    dst, bias = empty(x.shape), empty((maps,))
+    driver().remap_bias_backward(dst, dev(x), remap_pmap(R, Cc, images, maps), bias)
+    np.testing.assert_array_equal(host(dst).reshape(-1), oracle.remap(x.reshape(images * maps, R, Cc), R, Cc, images, maps).reshape(-1))
+    ref = oracle.bias_backward(x, R * Cc, maps, images)
+    scale = max(np.abs(ref).max(), 1.0)
+    assert np.abs(host(bias) - ref).max() / scale <= 1e-4
+    assert np.abs(host(bias) - x.astype(np.float64).sum(axis=(0, 2, 3))).max() / scale <= 1e-4
+    bias2 = empty((maps,))
+    driver().remap_bias_backward(empty(x.shape), dev(x), remap_pmap(R, Cc, images, maps), bias2)
+    np.testing.assert_array_equal(host(bias2), host(bias))
+
+
 def test_remap_rejects_overlap():
     from caffecontroll_amd import CctHipError
     from caffecontroll_amd.driver import remap_pmap
