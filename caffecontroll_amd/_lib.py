@@ -35,6 +35,12 @@ class PoolArgs(C.Structure):
                [("max_index", C.c_void_p)]
 
 
+class SgdJob(C.Structure):
+    """cct_sgd_job: one tensor of a batched SGD update."""
+    _fields_ = [("n", C.c_size_t), ("model", C.c_void_p), ("gradient", C.c_void_p), ("history", C.c_void_p),
+                ("stepsize", C.c_float), ("momentum", C.c_float), ("lam", C.c_float), ("l1", C.c_int)]
+
+
 class LrnForwardArgs(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("iR", "iC", "iD", "iB", "norm_window", "local_size")] + \
                [("denoms", C.c_void_p)]
@@ -84,6 +90,7 @@ PROTOTYPES = {
     "cct_hip_math_saxpby": [_Z, _F, _P, _F, _P],
     "cct_hip_L1_update": [_I, _P, _F, _P],
     "cct_hip_sgd_update": [_Z, _P, _P, _P, _F, _F, _F, _I],
+    "cct_hip_sgd_update_batch": [C.POINTER(SgdJob), _I],
     "cct_hip_sconstant_initialize": [_P, _Z, _F],
     "cct_hip_init_rng": [_I],
     "cct_hip_rand_uint_initialize": [_P, _I],

@@ -687,21 +687,43 @@ __global__ __launch_bounds__(TPB) void l1_update_kernel(int n, float *__restrict
 }
 // one pass: the three BLAS-1 calls of SGDGradientUpdater::update applied per element in the same
 // order, each product/sum rounded to fp32 as the separate calls would
+__device__ __forceinline__ void sgd_element(float *__restrict__ w, float *__restrict__ g, float *__restrict__ h,
+                                            size_t i, float step, float mom, float lambda, int l1) {
+  const float wi = w[i];
+  float gi = g[i];
+  if (lambda != 0.0f) {
+    gi = l1 ? gi + lambda * (wi > 0 ? 1.0f : -1.0f) : __fadd_rn(__fmul_rn(lambda, wi), gi);
+    g[i] = gi;
+  }
+  const float hi = __fadd_rn(__fmul_rn(step, gi), __fmul_rn(mom, h[i]));
+  h[i] = hi;
+  w[i] = __fadd_rn(__fmul_rn(-1.0f, hi), wi);
+}
 __global__ __launch_bounds__(TPB) void sgd_kernel(size_t n, float *__restrict__ w, float *__restrict__ g,
                                                   float *__restrict__ h, float step, float mom, float lambda,
                                                   int l1) {
   const size_t stride = (size_t)gridDim.x * TPB;
-  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) {
-    const float wi = w[i];
-    float gi = g[i];
-    if (lambda != 0.0f) {
-      gi = l1 ? gi + lambda * (wi > 0 ? 1.0f : -1.0f) : __fadd_rn(__fmul_rn(lambda, wi), gi);
-      g[i] = gi;
-    }
-    const float hi = __fadd_rn(__fmul_rn(step, gi), __fmul_rn(mom, h[i]));
-    h[i] = hi;
-    w[i] = __fadd_rn(__fmul_rn(-1.0f, hi), wi);
-  }
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride)
+    sgd_element(w, g, h, i, step, mom, lambda, l1);
+}
+
+// Several small tensors in one launch (the biases and small filters of a network: a launch each
+// costs more than their update).  The job table travels as a kernel argument; a workgroup handles
+// kSgdChunk elements of one job, found from the first-block table.
+constexpr int kSgdBatch = 16, kSgdChunk = TPB * 8;
+struct SgdBatch {
+  cct_sgd_job job[kSgdBatch];
+  uint32_t first_block[kSgdBatch + 1];
+  int count;
+};
+__global__ __launch_bounds__(TPB) void sgd_batch_kernel(const SgdBatch b) {
+  int j = 0;
+  while (j + 1 < b.count && blockIdx.x >= b.first_block[j + 1]) ++j;
+  const cct_sgd_job &job = b.job[j];
+  const size_t i0 = (size_t)(blockIdx.x - b.first_block[j]) * kSgdChunk;
+  const size_t i1 = i0 + kSgdChunk < job.n ? i0 + kSgdChunk : job.n;
+  for (size_t i = i0 + threadIdx.x; i < i1; i += TPB)
+    sgd_element(job.model, job.gradient, job.history, i, job.stepsize, job.momentum, job.lambda, job.l1);
 }
 
 // ---- gemv (row-major M x N, lda = N) -------------------------------------------------------------------
@@ -1106,6 +1128,31 @@ int cct_hip_sgd_update(size_t n, float *model, float *gradient, float *history, 
   hipLaunchKernelGGL(sgd_kernel, dim3(grid_stride_blocks(n)), dim3(TPB), 0, ctx().stream, n, model, gradient,
                      history, stepsize, momentum, lambda, l1);
   CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+int cct_hip_sgd_update_batch(const cct_sgd_job *jobs, int count) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(count >= 0 && (jobs || count == 0), "sgd_update_batch: null job table");
+  for (int at = 0; at < count;) {
+    SgdBatch b;
+    b.count = 0;
+    uint32_t blocks = 0;
+    for (; at < count && b.count < kSgdBatch; ++at) {
+      const cct_sgd_job &j = jobs[at];
+      if (j.n == 0) continue;
+      CCT_REQUIRE(j.model && j.gradient && j.history, "sgd_update_batch: null argument in job %d", at);
+      CCT_REQUIRE(j.n < ((size_t)1 << 40), "sgd_update_batch: job %d too large", at);
+      b.job[b.count] = j;
+      b.first_block[b.count] = blocks;
+      blocks += (uint32_t)((j.n + kSgdChunk - 1) / kSgdChunk);
+      ++b.count;
+    }
+    if (b.count == 0) continue;
+    b.first_block[b.count] = blocks;
+    hipLaunchKernelGGL(sgd_batch_kernel, dim3(blocks), dim3(TPB), 0, ctx().stream, b);
+    CCT_LAUNCH_CHECK();
+  }
   return 0;
 }
 

@@ -13,6 +13,7 @@
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
+#include <mutex>
 #include <random>
 #include <vector>
 
@@ -169,7 +170,36 @@ class HIPDriver {
   }
   void sgd_update(size_t n, float *model, float *gradient, float *history, float stepsize, float momentum,
                   float lambda, bool l1) {
+    if (defer_sgd_) {
+      cct_sgd_job job = {n, model, gradient, history, stepsize, momentum, lambda, l1 ? 1 : 0};
+      std::lock_guard<std::mutex> lk(sgd_mu_);
+      sgd_jobs_.push_back(job);
+      return;
+    }
     ok(cct_hip_sgd_update(n, model, gradient, history, stepsize, momentum, lambda, l1 ? 1 : 0), "sgd_update");
+  }
+  // Between begin_deferred_sgd() and flush_deferred_sgd() the updates are collected instead of
+  // launched (a whole network's backward pass: no layer reads another layer's weights in it);
+  // the flush applies the large tensors one launch each and all small ones together.
+  void begin_deferred_sgd() {
+    static const bool off = [] { const char *e = std::getenv("CCT_HIP_SGD_BATCH"); return e && std::atoi(e) == 0; }();
+    defer_sgd_ = !off;  // (tuning override, read once: CCT_HIP_SGD_BATCH=0 keeps one launch per tensor)
+  }
+  void flush_deferred_sgd() {
+    defer_sgd_ = false;
+    std::vector<cct_sgd_job> jobs, small;
+    {
+      std::lock_guard<std::mutex> lk(sgd_mu_);
+      jobs.swap(sgd_jobs_);
+    }
+    for (const cct_sgd_job &j : jobs) {
+      if (j.n >= kLargeSgdTensor)
+        ok(cct_hip_sgd_update(j.n, j.model, j.gradient, j.history, j.stepsize, j.momentum, j.lambda, j.l1),
+           "sgd_update");
+      else
+        small.push_back(j);
+    }
+    if (!small.empty()) ok(cct_hip_sgd_update_batch(small.data(), (int)small.size()), "sgd_update_batch");
   }
   void set_num_threads(const int) {}
   void sgemm(const enum CBLAS_ORDER order, CBLAS_TRANSPOSE TA, CBLAS_TRANSPOSE TB, int M, int N, int K,
@@ -279,6 +309,12 @@ class HIPDriver {
       std::abort();
     }
   }
+
+ private:
+  static constexpr size_t kLargeSgdTensor = (size_t)1 << 20;  // elements; above this a launch of its own pays
+  bool defer_sgd_ = false;
+  std::mutex sgd_mu_;
+  std::vector<cct_sgd_job> sgd_jobs_;
 };
 
 }  // namespace cct

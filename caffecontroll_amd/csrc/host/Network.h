@@ -219,6 +219,9 @@ class Network {
   // DeepNet::run_backward_pass: every bridge in reverse order; ParallelizedBridge::backward applies
   // the SGD update of its layer
   void backward() {
+    // the layers' SGD updates are collected and applied after the last backward: the many small
+    // tensors then share one launch
+    driver_.begin_deferred_sgd();
     for (int i = (int)nodes_.size() - 1; i >= 0; --i) {
       Node &nd = nodes_[i];
       const size_t g = nd.group_in.size();
@@ -229,6 +232,7 @@ class Network {
         for (size_t gi = 0; gi < g; ++gi)
           slice_copy(nd.group_in[gi]->p_gradient_cube, nd.in->p_gradient_cube, gi, /*gather=*/false);
     }
+    driver_.flush_deferred_sgd();
   }
 
   float loss() { return softmax_ ? softmax_->get_loss() : 0.f; }

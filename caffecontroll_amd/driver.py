@@ -157,6 +157,16 @@ class HIPDriver:
         check(self.lib.cct_hip_sgd_update(n, _p(model), _p(gradient), _p(history), stepsize, momentum,
                                           lam, int(l1)), "sgd_update")
 
+    def sgd_update_batch(self, jobs):
+        """jobs: sequence of (n, model, gradient, history, stepsize, momentum, lam, l1); one launch
+        per 16 tensors, the arithmetic of `sgd_update` on every element."""
+        from ._lib import SgdJob
+        table = (SgdJob * len(jobs))()
+        for t, (n, model, gradient, history, stepsize, momentum, lam, l1) in zip(table, jobs):
+            t.n, t.model, t.gradient, t.history = n, _p(model), _p(gradient), _p(history)
+            t.stepsize, t.momentum, t.lam, t.l1 = stepsize, momentum, lam, int(l1)
+        check(self.lib.cct_hip_sgd_update_batch(table, len(jobs)), "sgd_update_batch")
+
     def sconstant_initialize(self, arr, n, value):
         check(self.lib.cct_hip_sconstant_initialize(_p(arr), n, value), "sconstant_initialize")
 

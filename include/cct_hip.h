@@ -218,6 +218,18 @@ int cct_hip_L1_update(int n, float *gradient, float lambda, const float *model);
  * g += lambda*w (or lambda*sign(w) when l1), h = stepsize*g + momentum*h, w -= h. */
 int cct_hip_sgd_update(size_t n, float *model, float *gradient, float *history, float stepsize,
                        float momentum, float lambda, int l1);
+/* The same update for several tensors in one launch: the updates DeepNet::run_backward_pass
+ * (src/DeepNet.h:2012-2028) triggers layer by layer, collected and applied after the last layer's
+ * backward (no layer reads another layer's weights in between, so the result is the same).  Meant
+ * for the many small tensors (biases, small filters) whose separate launches cost more than their
+ * arithmetic; every element sees exactly the arithmetic of cct_hip_sgd_update. */
+typedef struct {
+  size_t n;
+  float *model, *gradient, *history;
+  float stepsize, momentum, lambda;
+  int l1;
+} cct_sgd_job;
+int cct_hip_sgd_update_batch(const cct_sgd_job *jobs, int count);
 /* DeviceDriver::sconstant_initialize (src/sched/DeviceDriver.h:258-260). */
 int cct_hip_sconstant_initialize(float *arr, size_t n, float value);
 /* DeviceDriver::rand_uint_initialize (src/sched/DeviceDriver.h:250-252) after init_rng(seed):

@@ -191,6 +191,34 @@ def test_sgd_and_blas1(oracle):
     np.testing.assert_array_equal(host(dg), g + np.float32(0.25) * np.where(w > 0, 1, -1).astype(np.float32))
 
 
+def test_sgd_batch_matches_single_updates(oracle):
+    """Several tensors in one launch (more than one table of 16, sizes around the 2048-element
+    chunks, an empty one, every regulariser): the bits of the oracle's update for each."""
+    drv = driver()
+    rng = np.random.default_rng(77)
+    sizes = [1, 10, 256, 2047, 2048, 2049, 0, 4097, 500, 20, 50, 96, 384, 4096, 1000, 34848, 25000, 307200, 7, 800]
+    jobs, refs, devs = [], [], []
+    for t, n in enumerate(sizes):
+        w, g, h = (rng.standard_normal(n).astype(np.float32) for _ in range(3))
+        step, mom = np.float32(0.01 * (1 + t % 3)), np.float32(0.9 if t % 2 else 0.0)
+        lam, l1 = [(0.0, False), (0.0005, False), (0.001, True)][t % 3]
+        rw, rg, rh = w.copy(), g.copy(), h.copy()
+        if n:
+            oracle.sgd_update(rw, rg, rh, float(step), float(mom), lam, l1)
+        dw, dg, dh = (dev(a) if n else empty((1,)) for a in (w, g, h))
+        jobs.append((n, dw, dg, dh, float(step), float(mom), lam, l1))
+        refs.append((rw, rg, rh))
+        devs.append((dw, dg, dh))
+    drv.sgd_update_batch(jobs)
+    for n, (rw, rg, rh), (dw, dg, dh) in zip(sizes, refs, devs):
+        if n == 0:
+            continue
+        np.testing.assert_array_equal(host(dw), rw)
+        np.testing.assert_array_equal(host(dg), rg)
+        np.testing.assert_array_equal(host(dh), rh)
+    drv.sgd_update_batch([])  # nothing to do
+
+
 def test_fill_and_memory():
     """tests/test_device_driver_cpu.cpp:22-206 counterparts: constant init, memset, memcpy."""
     import ctypes as C
