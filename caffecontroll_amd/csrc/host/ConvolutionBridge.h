@@ -124,7 +124,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     // Small layers (LeNet-sized) stay on the fused lowering path by default: the direct kernels'
     // fixed costs (slab re-layout, partial-sum reduction) outweigh what they save below a few GFLOP.
     const double gemm_flop = 2.0 * num_output_features * (double)(oR * oC * iB) * (double)(K * K * iD);
-    default_path_ = (direct_ok_ && gemm_flop >= kConvDirectMinFlop) ? PATH_DIRECT_ALL : PATH_FUSED;
+    // (a very short contraction -- LeNet conv1 has k*k*d = 25 -- makes the lowered GEMM all prologue and
+    // epilogue; there the direct kernels win at any size)
+    const bool short_contraction = K * K * iD <= 64;
+    default_path_ = (direct_ok_ && (gemm_flop >= kConvDirectMinFlop || short_contraction)) ? PATH_DIRECT_ALL : PATH_FUSED;
     path_ = default_path_;
     for (int i = 0; i < STAGE_COUNT; ++i) { timers_[i] = nullptr; stage_ms_[i] = 0.f; }
   }
