@@ -553,6 +553,47 @@ __global__ __launch_bounds__(TPB) void lrn_bwd_kernel(float *__restrict__ ig, co
   ig[e] = acc;
 }
 
+// Forward with one lane per (image, pixel, run of CH channels): the CH + 2*WN inputs under the run
+// are loaded once (all loads in flight together) and every channel's window is summed afresh from
+// them in ascending channel order -- the sums lrn_fwd_kernel forms (terms outside the depth enter
+// as +0, which leaves a sum of squares unchanged), a third of its loads and an eighth of its index
+// arithmetic.
+template <int WN, int CH>
+__global__ __launch_bounds__(TPB) void lrn_fwd_run_kernel(float *__restrict__ out, float *__restrict__ denoms,
+                                                          const float *__restrict__ in, int rc, int D,
+                                                          uint32_t total, int nruns, float aos, float beta,
+                                                          FastDiv div_rc, FastDiv div_runs) {
+  const uint32_t e = blockIdx.x * TPB + threadIdx.x;
+  if (e >= total) return;
+  // e = (ib*nruns + run)*rc + q
+  const uint32_t t1 = fdiv(e, div_rc);
+  const uint32_t q = e - t1 * rc;
+  const uint32_t ib = fdiv(t1, div_runs);
+  const int c0 = (int)(t1 - ib * nruns) * CH;
+  const size_t base = (size_t)ib * D * rc + q;
+  constexpr int NW = CH + 2 * WN;
+  float xw[NW];
+#pragma unroll
+  for (int i = 0; i < NW; ++i) {
+    const int c = c0 - WN + i;
+    const int cc = min(max(c, 0), D - 1);           // clamped: the load needs no branch
+    const float v = in[base + (size_t)cc * rc];
+    xw[i] = (c >= 0 && c < D) ? v : 0.0f;
+  }
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int ch = c0 + c;
+    if (ch >= D) break;
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j <= 2 * WN; ++j) sum += xw[c + j] * xw[c + j];
+    const float scale = aos * sum + 1.0f;
+    const size_t o = base + (size_t)ch * rc;
+    denoms[o] = scale;
+    out[o] = xw[c + WN] / powf(scale, beta);
+  }
+}
+
 // The same gather with one lane per (image, pixel, run of CH channels): the per-channel terms of
 // the window (scale^beta, the factor g2, x and out_grad) are computed once per lane and reused by
 // the up to 2*WN+1 output channels that touch them, instead of once per (channel, window slot).
@@ -994,6 +1035,16 @@ int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args 
   const size_t total = (size_t)a->iB * a->iD * a->iR * a->iC;
   CCT_REQUIRE(total < (1ull << 31), "lrn_forward: tensor too large");
   if (total == 0) return 0;
+  if (a->norm_window == 2) {
+    constexpr int CH = 8;
+    const int nruns = (a->iD + CH - 1) / CH, rc = a->iR * a->iC;
+    const size_t lanes = (size_t)a->iB * nruns * rc;
+    hipLaunchKernelGGL((lrn_fwd_run_kernel<2, CH>), dim3(blocks_for(lanes)), dim3(TPB), 0, ctx().stream, out,
+                       (float *)a->denoms, in, rc, a->iD, (uint32_t)lanes, nruns, a2->alpha_over_size, a2->beta,
+                       make_fastdiv(rc), make_fastdiv(nruns));
+    CCT_LAUNCH_CHECK();
+    return 0;
+  }
   hipLaunchKernelGGL(lrn_fwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, out,
                      (float *)a->denoms, in, a->iR * a->iC, a->iD, (uint32_t)total, a->norm_window,
                      a2->alpha_over_size, a2->beta, make_fastdiv(a->iR * a->iC), make_fastdiv(a->iD));
