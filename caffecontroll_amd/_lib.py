@@ -84,6 +84,7 @@ PROTOTYPES = {
     "cct_hip_conv_direct_slabs": [_P, _P, _I, _I, _I, _I],
     "cct_hip_conv_direct_forward": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z, _I],
     "cct_hip_conv_direct_backward_data": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z],
+    "cct_hip_conv_direct_backward_data_relu": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z, _P],
     "cct_hip_conv_direct_backward_weights": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z],
     "cct_hip_sgemv": [_I, _I, _I, _F, _P, _P, _F, _P],
     "cct_hip_math_saxpy": [_Z, _F, _P, _P],

@@ -42,6 +42,7 @@ struct DirectArgs {
   float *dst;         // [batch][mtot][ho][ho]
   const float *bias;  // [mtot] or null
   int relu;           // epilogue clamps at zero (ReLU of the layer that follows, folded in)
+  const float *mask;  // same shape as dst, or null: store 0 where mask <= 0 (data gradient through the ReLU before the layer)
   int batch, kc, mtot, hs, ho, pad;
   int hp;             // ho + KS - 1 = hs + 2*pad: rows (and columns) of a zero-padded source image
   int pr;             // patch rows per channel
@@ -249,14 +250,16 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     const uint32_t p = p0 + wave * (32 * TNB) + b * 32 + r;
     if (p >= g.ptot) continue;
     const uint32_t img = fdiv(p, g.div_ho2);
-    float *out = g.dst + (size_t)img * g.dst_img_stride + (p - img * ho2);
+    const size_t pix = (size_t)img * g.dst_img_stride + (p - img * ho2);
+    float *out = g.dst + pix;
 #pragma unroll
     for (int a = 0; a < TMB; ++a)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = m0 + a * 32 + 8 * (v / 4) + 4 * h + (v % 4);
         if (row < g.mtot) {
-          const float y = acc[a][b][v] + (g.bias ? g.bias[row] : 0.f);
+          float y = acc[a][b][v] + (g.bias ? g.bias[row] : 0.f);
+          if (g.mask && !(g.mask[pix + (size_t)row * ho2] > 0.f)) y = 0.f;
           out[(size_t)row * ho2] = (g.relu && !(y > 0.f)) ? 0.f : y;
         }
       }
@@ -387,12 +390,13 @@ static int direct_launch_ks(const DirectArgs &g, const DirectPlan &pl, hipStream
 }
 
 static int conv_direct(const float *wt, const float *src, float *dst, const float *bias, int relu, int batch, int kc,
-                       int mtot, int hs, int ks, int pad, size_t src_img_stride, size_t dst_img_stride) {
+                       int mtot, int hs, int ks, int pad, size_t src_img_stride, size_t dst_img_stride,
+                       const float *mask = nullptr) {
   DirectPlan pl;
   CCT_REQUIRE(direct_plan(batch, kc, mtot, hs, ks, pad, &pl),
               "conv_direct: geometry not covered (k=%d pad=%d size=%d)", ks, pad, hs);
   DirectArgs g;
-  g.wt = wt; g.src = src; g.dst = dst; g.bias = bias; g.relu = relu;
+  g.wt = wt; g.src = src; g.dst = dst; g.bias = bias; g.relu = relu; g.mask = mask;
   g.batch = batch; g.kc = kc; g.mtot = mtot; g.hs = hs; g.pad = pad;
   g.ho = hs + 2 * pad - ks + 1;
   {
@@ -1116,6 +1120,18 @@ extern "C" int cct_hip_conv_direct_backward_data(float *input_grad, const float 
   const int m = n + 2 * padding - k + 1;
   return conv_direct(slabs, output_grad, input_grad, nullptr, 0, batch, num_outputs, depth, m, k,
                      k - 1 - padding, output_image_stride, input_image_stride);
+}
+
+extern "C" int cct_hip_conv_direct_backward_data_relu(float *input_grad, const float *output_grad,
+                                                      const float *slabs, int batch, int depth, int n, int k,
+                                                      int padding, int num_outputs, size_t input_image_stride,
+                                                      size_t output_image_stride, const float *relu_data) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(relu_data, "conv_direct_backward_data_relu: null activation tensor");
+  if (batch <= 0) return 0;
+  const int m = n + 2 * padding - k + 1;
+  return conv_direct(slabs, output_grad, input_grad, nullptr, 0, batch, num_outputs, depth, m, k,
+                     k - 1 - padding, output_image_stride, input_image_stride, relu_data);
 }
 
 extern "C" int cct_hip_conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,

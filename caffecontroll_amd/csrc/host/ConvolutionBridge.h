@@ -185,6 +185,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   // Apply the ReLU of a following in-place ReLUBridge (y = max(x, 0)) while the output is stored,
   // instead of in a pass of its own; the ReLU bridge then skips its forward.
   void set_fuse_relu(bool on) { fuse_relu_ = on; }
+  // The input layer is the output of an in-place ReLU whose backward this bridge performs on the
+  // input gradient it produces (masked in the direct kernel's store, or by a pass after the lifting);
+  // the ReLU bridge then skips its own.  Only meaningful with needs_to_calc_backward_grad.
+  bool input_is_relu_output = false;
   bool fuse_relu() const { return fuse_relu_; }
   // per-stage hipEvent timing (the reference's -D_DETAILED_PROFILING stage prints)
   void set_stage_profiling(bool on) { profile_ = on; }
@@ -310,7 +314,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       p_driver->conv_direct_backward_data(input_g_cube->get_p_data(), output_g_cube->get_p_data(),
                                           backward_slabs()->get_p_data(), (int)iB, (int)iD, (int)iR, (int)K,
                                           (int)padding, (int)num_output_features, in_image_stride_,
-                                          out_image_stride_);
+                                          out_image_stride_,
+                                          input_is_relu_output ? p_input_layer->p_data_cube->get_p_data() : nullptr);
       end(STAGE_GEMM_DATA);
     } else if (needs_to_calc_backward_grad) {
       begin(STAGE_INVERSE_LOWER);
@@ -324,6 +329,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
         p_forward_lower_connector->inverse_lower_cube(backward_inputgrad(), input_g_cube);
       }
       end(STAGE_INVERSE_LOWER);
+      if (input_is_relu_output) {  // the lowering path has no store to fold the mask into
+        DeviceMemoryPointer in_grad = input_g_cube->get_device_pointer(p_driver);
+        p_driver->relu_backward(&in_grad, &in_grad, p_input_layer->p_data_cube->get_p_data());
+      }
     }
     report_backward_updateweight_history.end();
   }

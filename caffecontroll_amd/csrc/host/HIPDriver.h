@@ -232,12 +232,19 @@ class HIPDriver {
                                    out_stride, relu ? 1 : 0),
        "conv_direct_forward");
   }
+  // relu_data (optional): the layer's input tensor when it is the output of an in-place ReLU -- the
+  // gradient is then stored already masked with (relu_data > 0)
   void conv_direct_backward_data(float *input_grad, const float *output_grad, const float *slabs, int batch,
                                  int depth, int n, int k, int padding, int num_outputs, size_t in_stride = 0,
-                                 size_t out_stride = 0) {
-    ok(cct_hip_conv_direct_backward_data(input_grad, output_grad, slabs, batch, depth, n, k, padding, num_outputs,
-                                         in_stride, out_stride),
-       "conv_direct_backward_data");
+                                 size_t out_stride = 0, const float *relu_data = nullptr) {
+    if (relu_data)
+      ok(cct_hip_conv_direct_backward_data_relu(input_grad, output_grad, slabs, batch, depth, n, k, padding,
+                                                num_outputs, in_stride, out_stride, relu_data),
+         "conv_direct_backward_data_relu");
+    else
+      ok(cct_hip_conv_direct_backward_data(input_grad, output_grad, slabs, batch, depth, n, k, padding,
+                                           num_outputs, in_stride, out_stride),
+         "conv_direct_backward_data");
   }
   void conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                     const float *input, int batch, int depth, int n, int k, int padding,

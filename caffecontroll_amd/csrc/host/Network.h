@@ -101,6 +101,14 @@ class Network {
             b->needs_to_calc_backward_grad = !first_weight_layer;
             nd.bridges.push_back(b);
           }
+          // directly after an in-place ReLU the layer masks the input gradient it produces (in the
+          // direct kernel's store) and the ReLU bridge skips its own backward pass over the tensor
+          if (!first_weight_layer && !nodes_.empty() && nodes_.back().spec.type == CCT_LAYER_RELU &&
+              nodes_.back().out == cur) {
+            for (BridgeT *cb : nd.bridges)
+              static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(cb)->sub_bridge()->input_is_relu_output = true;
+            static_cast<ReLUBridge<float, HIPDriver> *>(nodes_.back().bridges[0])->backward_done_by_consumer = true;
+          }
           first_weight_layer = false;
           break;
         }

@@ -132,7 +132,15 @@ class HIPDriver:
         check(self.lib.cct_hip_conv_direct_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o,
                                                    in_stride, out_stride, int(relu)), "conv_direct_forward")
 
-    def conv_direct_backward_data(self, din, dout, slabs, b, d, n, k, p, o, in_stride=0, out_stride=0):
+    def conv_direct_backward_data(self, din, dout, slabs, b, d, n, k, p, o, in_stride=0, out_stride=0,
+                                  relu_data=None):
+        """relu_data: the layer's input tensor when it is the output of an in-place ReLU; the gradient
+        then comes out already masked with (relu_data > 0)."""
+        if relu_data is not None:
+            check(self.lib.cct_hip_conv_direct_backward_data_relu(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o,
+                                                                  in_stride, out_stride, _p(relu_data)),
+                  "conv_direct_backward_data_relu")
+            return
         check(self.lib.cct_hip_conv_direct_backward_data(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o,
                                                          in_stride, out_stride), "conv_direct_backward_data")
 

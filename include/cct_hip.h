@@ -198,6 +198,14 @@ int cct_hip_conv_direct_forward(float *output, const float *input, const float *
 int cct_hip_conv_direct_backward_data(float *input_grad, const float *output_grad, const float *slabs,
                                       int batch, int depth, int n, int k, int padding, int num_outputs,
                                       size_t input_image_stride, size_t output_image_stride);
+/* The same followed by the backward of an in-place ReLU whose output is this layer's input
+ * (src/bridges/ReLUBridge_impl.hxx:62-100, the next bridge DeepNet::run_backward_pass visits):
+ * input_grad is stored as 0 wherever relu_data (the layer's input tensor, same shape and image
+ * stride as input_grad) is not positive. */
+int cct_hip_conv_direct_backward_data_relu(float *input_grad, const float *output_grad, const float *slabs,
+                                           int batch, int depth, int n, int k, int padding, int num_outputs,
+                                           size_t input_image_stride, size_t output_image_stride,
+                                           const float *relu_data);
 /* Weight-gradient GEMM of ConvolutionBridge::backward (src/bridges/ConvolutionBridge_impl.hxx:
  * 619-621) without the lowered matrix or the gradient remap: model_grad[o][d][k][k] (overwritten,
  * beta = 0) from output_grad[b][o][m][m] and input[b][d][n][n].  If bias_grad is not NULL the same

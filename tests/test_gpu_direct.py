@@ -110,6 +110,11 @@ def test_direct_kernels_match_oracle(oracle, shape):
     drv.conv_direct_backward_data(dx, d_og, slabs_b, b, d, n, k, p, o)
     assert rel_err(host(dx), ref_dx) <= TOL
     np.testing.assert_array_equal(host(d_og), og)  # the output gradient is read in place, not permuted
+    # the backward of an in-place ReLU before the layer folded into the store: the same gradient
+    # where the layer's input is positive, zero elsewhere
+    dx_relu = empty((b, d, n, n))
+    drv.conv_direct_backward_data(dx_relu, d_og, slabs_b, b, d, n, k, p, o, relu_data=d_x)
+    np.testing.assert_array_equal(host(dx_relu), oracle.relu_backward(host(dx), x))
 
     dw, db = empty((o, d, k, k)), empty((o,))
     drv.conv_direct_backward_weights(dw, d_og, d_x, b, d, n, k, p, o, db=db)
