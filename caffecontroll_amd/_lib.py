@@ -63,6 +63,7 @@ _P, _I, _F, _Z, _U = C.c_void_p, C.c_int, C.c_float, C.c_size_t, C.c_uint
 PROTOTYPES = {
     "cct_hip_init": [_I],
     "cct_hip_set_stream": [_P],
+    "cct_hip_set_tuning": [C.c_char_p, _I],
     "cct_hip_device_sync": [],
     "cct_hip_last_error": [],
     "cct_hip_compute_units": [],

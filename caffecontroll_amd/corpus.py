@@ -29,6 +29,7 @@ CORPUS_PROTOTYPES = {
     "cct_corpus_create": ([_PP, _I, _I, _I, _I, _I, C.c_float, _I, _I, _P, C.c_uint], _I),
     "cct_corpus_close": ([_P], _I),
     "cct_corpus_get_info": ([_P, C.POINTER(CorpusInfo)], _I),
+    "cct_corpus_set_num_classes": ([_P, _I], _I),
     "cct_corpus_load_next": ([_P, C.POINTER(_I)], _I),
     "cct_corpus_stage": ([_P, _PP, _PP, _PP], _I),
     "cct_corpus_submit": ([_P], _I),
@@ -161,6 +162,11 @@ class Corpus:
         check(lib.cct_corpus_create(C.byref(h), batch, channels, height, width, crop_size, scale, int(mirror), phase,
                                     m.ctypes.data_as(_P) if m is not None else None, seed), "corpus_create")
         return cls(h)
+
+    def set_num_classes(self, num_classes):
+        """Class count of the loss layer: batches with a label outside [0, num_classes) are refused on
+        the host by `load_next` / `submit` (0 switches the check off)."""
+        check(self.lib.cct_corpus_set_num_classes(self.h, int(num_classes)), "corpus_set_num_classes")
 
     def load_next(self):
         """Next LMDB mini-batch -> staging -> asynchronous upload; returns the epoch count."""

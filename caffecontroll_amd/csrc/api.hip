@@ -8,10 +8,42 @@
 namespace cct {
 
 static Context g_ctx;
+static Tuning g_tuning;
+static std::once_flag g_tuning_once;
+static bool g_counters_dirty = false;
 static std::mutex g_mu;
 static thread_local char g_err[512] = "";
 
 Context &ctx() { return g_ctx; }
+Tuning &tuning() { return g_tuning; }
+
+static void read_tuning_from_env() {
+  auto geti = [](const char *name, int dflt) {
+    const char *e = getenv(name);
+    return e && *e ? atoi(e) : dflt;
+  };
+  g_tuning.direct_tile = geti("CCT_HIP_DIRECT_TILE", 0);
+  g_tuning.direct_waves = geti("CCT_HIP_DIRECT_WAVES", 0);
+  g_tuning.direct_tb = geti("CCT_HIP_DIRECT_TB", 0);
+  g_tuning.direct_nospec = geti("CCT_HIP_DIRECT_NOSPEC", 0);
+  g_tuning.pool_plane = geti("CCT_HIP_POOL_PLANE", 0);
+  g_tuning.gemm_nt = geti("CCT_HIP_GEMM_NT", 0);
+  g_tuning.gemm_tile = geti("CCT_HIP_GEMM_TILE", -1);
+}
+
+void mark_counters_dirty() {
+  std::lock_guard<std::mutex> lk(g_mu);
+  g_counters_dirty = true;
+}
+
+int grant_dynamic_lds(const void *kernel, size_t bytes, LdsGrant &st) {
+  if (bytes <= 64 * 1024) return 0;
+  if (st.device == g_ctx.device && st.bytes >= bytes) return 0;
+  CCT_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
+  st.device = g_ctx.device;
+  st.bytes = bytes;
+  return 0;
+}
 
 int set_error(int code, const char *fmt, ...) {
   va_list ap;
@@ -22,6 +54,7 @@ int set_error(int code, const char *fmt, ...) {
 }
 
 static int init_locked(int device_id) {
+  std::call_once(g_tuning_once, read_tuning_from_env);
   int count = 0;
   CCT_HIP_CHECK(hipGetDeviceCount(&count));
   CCT_REQUIRE(device_id >= 0 && device_id < count, "device %d not present (%d devices)", device_id,
@@ -71,12 +104,21 @@ int get_workspace(size_t bytes, void **out) {
   return 0;
 }
 
+// The arrival counters must read zero when a launch starts; the workgroup that finishes a reduction
+// puts its counter back to zero.  They are cleared here when they are created, after
+// cct_hip_init() and after a launch that used them was refused (mark_counters_dirty).  All users
+// run on the library's one stream, so a clear ordered on that stream is ordered before them.
 int get_counters(unsigned int **out) {
   std::lock_guard<std::mutex> lk(g_mu);
   if (!g_ctx.counters) {
     CCT_HIP_CHECK(hipMalloc((void **)&g_ctx.counters, kMaxCounters * sizeof(unsigned int)));
+    g_counters_dirty = true;
+  }
+  if (g_counters_dirty) {
+    CCT_HIP_CHECK(hipStreamSynchronize(g_ctx.stream));
     CCT_HIP_CHECK(hipMemset(g_ctx.counters, 0, kMaxCounters * sizeof(unsigned int)));
     CCT_HIP_CHECK(hipDeviceSynchronize());
+    g_counters_dirty = false;
   }
   *out = g_ctx.counters;
   return 0;
@@ -94,7 +136,26 @@ extern "C" {
 
 int cct_hip_init(int device_id) {
   std::lock_guard<std::mutex> lk(g_mu);
-  return init_locked(device_id);
+  const int rc = init_locked(device_id);
+  // an explicit (re-)initialisation also puts the reduction counters back to a known state
+  if (!rc && g_ctx.counters) g_counters_dirty = true;
+  return rc;
+}
+
+int cct_hip_set_tuning(const char *name, int value) {
+  CCT_REQUIRE(name != nullptr, "set_tuning: null name");
+  std::call_once(g_tuning_once, read_tuning_from_env);
+  Tuning &t = tuning();
+  struct { const char *name; int *field; } const table[] = {
+      {"direct_tile", &t.direct_tile}, {"direct_waves", &t.direct_waves}, {"direct_tb", &t.direct_tb},
+      {"direct_nospec", &t.direct_nospec}, {"pool_plane", &t.pool_plane}, {"gemm_nt", &t.gemm_nt},
+      {"gemm_tile", &t.gemm_tile}};
+  for (const auto &e : table)
+    if (!strcmp(e.name, name)) {
+      *e.field = value;
+      return 0;
+    }
+  return set_error(CCT_HIP_EINVAL, "set_tuning: unknown knob \"%s\"", name);
 }
 
 int cct_hip_set_stream(void *hip_stream) {

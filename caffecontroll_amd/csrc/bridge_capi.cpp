@@ -1,4 +1,6 @@
 // C entry points over the C++ host layer (see include/cct_bridge.h).
+#include <cmath>
+#include <exception>
 #include <string>
 
 #include "../../include/cct_bridge.h"
@@ -119,12 +121,26 @@ struct cct_net {
   Network *net;
 };
 
+int cct_net_validate(int batch, int depth, int size, const cct_layer_spec *layers, int n_layers,
+                     const cct_solver_param *solver) {
+  const std::string why = Network::validate(batch, depth, size, layers, n_layers, solver);
+  return why.empty() ? 0 : cct::set_error(CCT_HIP_EINVAL, "net: %s", why.c_str());
+}
+
 int cct_net_create(cct_net **out, int batch, int depth, int size, const cct_layer_spec *layers, int n_layers,
                    const cct_solver_param *solver) {
-  if (!out || !layers || batch <= 0 || depth <= 0 || size <= 0 || n_layers <= 0) return CCT_HIP_EINVAL;
-  cct_net *h = new cct_net;
-  h->net = new Network(batch, depth, size, layers, n_layers, solver);
-  *out = h;
+  if (!out) return cct::set_error(CCT_HIP_EINVAL, "net_create: null result pointer");
+  *out = nullptr;
+  int rc = cct_net_validate(batch, depth, size, layers, n_layers, solver);
+  if (rc) return rc;
+  try {
+    Network *net = new Network(batch, depth, size, layers, n_layers, solver);
+    cct_net *h = new cct_net;
+    h->net = net;
+    *out = h;
+  } catch (const std::exception &e) {
+    return cct::set_error(CCT_HIP_EINVAL, "net_create: %s", e.what());
+  }
   return 0;
 }
 
@@ -240,6 +256,18 @@ int cct_net_set_iter(cct_net *h, int iter) {
   return 0;
 }
 
+int cct_net_get_iter(cct_net *h) { return h ? h->net->current_iter() : -1; }
+
+int cct_net_num_classes(cct_net *h) { return h ? h->net->num_classes() : 0; }
+
 size_t cct_net_parameter_size(cct_net *h) { return h ? h->net->parameter_size() : 0; }
+
+float cct_solver_learning_rate(const cct_solver_param *solver, int iter) {
+  float rate = NAN;
+  if (!solver || !solver->lr_policy) return rate;
+  Util::try_get_learning_rate(solver->lr_policy, solver->base_lr, solver->gamma, (float)iter, (float)solver->stepsize,
+                              solver->power, (float)solver->max_iter, &rate);
+  return rate;
+}
 
 }  // extern "C"

@@ -25,12 +25,37 @@ struct Context {
   uint64_t rng_calls = 0;
 };
 
+// Tuning overrides, for experiments and for tests that pin a kernel instance.  Read ONCE from the
+// environment when the library initialises (CCT_HIP_DIRECT_TILE, _DIRECT_WAVES, _DIRECT_TB,
+// _DIRECT_NOSPEC, _POOL_PLANE, _GEMM_NT, _GEMM_TILE), changed afterwards only through
+// cct_hip_set_tuning(); the launch paths read this struct, never the environment.
+struct Tuning {
+  int direct_tile = 0;    // "<map blocks><pixel blocks>" of conv_direct_kernel, 0 = model's choice
+  int direct_waves = 0;   // wavefronts of the weight-gradient workgroup (4..8), 0 = model's choice
+  int direct_tb = 0;      // column blocks of the weight-gradient tile (1..6), 0 = model's choice
+  int direct_nospec = 0;  // 1: never take the shape-specialised weight-gradient instances
+  int pool_plane = 0;     // 1: plane-tiled pooling kernels at any size
+  int gemm_nt = 0;        // 1: non-temporal stores in the GEMM epilogue
+  int gemm_tile = -1;     // index of the GEMM tile shape, -1 = model's choice
+};
+Tuning &tuning();
+
 Context &ctx();
 int ensure_init();
 int set_error(int code, const char *fmt, ...);
 int get_workspace(size_t bytes, void **out);
 constexpr int kMaxCounters = 16384;
 int get_counters(unsigned int **out);
+// A launch that used the arrival counters failed or was refused: they are cleared before their next use.
+void mark_counters_dirty();
+
+// Kernels that need more than 64 KB of dynamic LDS must be granted it once per device; `st` (one
+// static object per kernel instance) remembers the grant so that later launches skip the call.
+struct LdsGrant {
+  int device = -1;
+  size_t bytes = 0;
+};
+int grant_dynamic_lds(const void *kernel, size_t bytes, LdsGrant &st);
 
 #define CCT_HIP_CHECK(expr)                                                                    \
   do {                                                                                         \

@@ -148,9 +148,19 @@ class Corpus {
     return 0;
   }
 
+  // Labels index the class scores in the loss layer: with a class count set, a batch holding a
+  // label outside [0, num_classes) (or a NaN) is refused on the host, before anything is uploaded.
+  void set_num_classes(int n) { num_classes_ = n; }
+
   int submit() {
     CCT_REQUIRE(staged_, "corpus: nothing staged");
     const int s = head_;
+    if (num_classes_ > 0) {
+      const float *l = (const float *)((const char *)host_[s] + labels_off_);
+      for (int b = 0; b < geo.batch; ++b)
+        CCT_REQUIRE(l[b] >= 0.0f && l[b] < (float)num_classes_,
+                    "corpus: label %g of image %d is outside [0, %d)", (double)l[b], b, num_classes_);
+    }
     if (geo.crop_size > 0) {
       // a caller may have overwritten the drawn parameters: the kernel trusts them, so check here
       const int *p = (const int *)((const char *)host_[s] + params_off_);
@@ -246,7 +256,7 @@ class Corpus {
   bool upload_recorded_[2] = {false, false}, consume_recorded_[2] = {false, false};
   float *mean_dev_ = nullptr;
   size_t pixel_bytes_ = 0, labels_off_ = 0, params_off_ = 0, slot_bytes_ = 0;
-  int head_ = 0, tail_ = 0, in_flight_ = 0, epoch_ = 0;
+  int head_ = 0, tail_ = 0, in_flight_ = 0, epoch_ = 0, num_classes_ = 0;
   bool staged_ = false;
 
   // process_image's choices (src/parser/corpus.h:266-276): random offsets in [0, size - crop) and a
@@ -392,6 +402,12 @@ int cct_corpus_get_info(cct_corpus *c, cct_corpus_info *info) {
   info->batch = g.batch; info->channels = g.channels; info->height = g.height; info->width = g.width;
   info->out_rows = g.crop_size ? g.crop_size : g.height;
   info->out_cols = g.crop_size ? g.crop_size : g.width;
+  return 0;
+}
+
+int cct_corpus_set_num_classes(cct_corpus *c, int num_classes) {
+  CCT_REQUIRE(c && num_classes >= 0, "corpus_set_num_classes: bad argument");
+  c->impl.set_num_classes(num_classes);
   return 0;
 }
 

@@ -319,8 +319,7 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
   const int padded = direct_padded_maps(mtot);
   // tuning override "<map blocks><pixel blocks>", e.g. 22
-  const char *forced_env = getenv("CCT_HIP_DIRECT_TILE");
-  const int forced = forced_env ? atoi(forced_env) : 0;
+  const int forced = tuning().direct_tile;
   // Candidate tiles: map tiles that divide the padded map count (the slab layout does not depend
   // on the choice), 128 or 256 pixels.  Estimated time, in units of one 32x128 block on a whole
   // compute unit: workgroups are handed out as residency slots free up, so the launch runs as
@@ -915,8 +914,7 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
     if (best < 0 || padded < best) { best = padded; best_w = w; }
   }
   pl->waves = best_w;
-  if (const char *e = getenv("CCT_HIP_DIRECT_WAVES")) {  // tuning override
-    const int forced = atoi(e);
+  if (const int forced = tuning().direct_waves) {  // tuning override
     if (forced >= 4 && forced <= 8) pl->waves = forced;
   }
   // column blocks per tile: least padding of the column count, wider tile on ties
@@ -929,8 +927,7 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
     if (best < 0 || padded < best) { best = padded; best_tb = tb; }
   }
   {
-    const char *e = getenv("CCT_HIP_DIRECT_TB");  // tuning override
-    const int forced = e ? atoi(e) : 0;
+    const int forced = tuning().direct_tb;  // tuning override
     if (forced >= 1 && forced <= 6) best_tb = forced;
   }
   pl->tb = best_tb;
@@ -945,10 +942,7 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
   pl->spec = (ks == 5 && ho == 27 && pl->pw == 32 && pl->tb == 5 && (pl->waves == 4 || pl->waves == 8)) ||
              (ks == 3 && ho == 13 && pl->pw == 16 && pl->tb == 6 &&
               (pl->waves == 4 || pl->waves == 6 || pl->waves == 8));
-  {
-    static const int off = [] { const char *e = getenv("CCT_HIP_DIRECT_NOSPEC"); return e ? atoi(e) : 0; }();
-    if (off) pl->spec = false;  // tuning override, read once
-  }
+  if (tuning().direct_nospec) pl->spec = false;  // tuning override
   if (pl->spec) {
     // layout of conv_direct_wgrad_spec_kernel: dout stays out of LDS, patches in whole passes
     pl->a_floats = 0;
@@ -964,8 +958,8 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
 template <int KS, int TB, int PW, int HO, int W>
 static int wgrad_launch_spec(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
   auto kern = conv_direct_wgrad_spec_kernel<KS, TB, PW, HO, W>;
-  if (pl.lds > 64 * 1024)
-    CCT_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)pl.lds));
+  static LdsGrant grant;
+  if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;
   hipLaunchKernelGGL(kern, dim3(g.nblocks), dim3(64 * W), pl.lds, st, g);
   CCT_LAUNCH_CHECK();
   return 0;
@@ -977,9 +971,8 @@ static int wgrad_launch(const WgradArgs &g, const WgradPlan &pl, hipStream_t st)
 #define CCT_WGRAD_CASE(TB)                                                                              \
   if (pl.tb == TB) {                                                                                    \
     auto kern = conv_direct_wgrad_kernel<KS, TB, PW>;                                                   \
-    if (pl.lds > 64 * 1024)                                                                             \
-      CCT_HIP_CHECK(hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                        (int)pl.lds));                                                  \
+    static LdsGrant grant;                                                                              \
+    if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;                       \
     hipLaunchKernelGGL(kern, grid, block, pl.lds, st, g);                                               \
     CCT_LAUNCH_CHECK();                                                                                 \
     return 0;                                                                                           \

@@ -474,11 +474,8 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict
   }
 }
 
-// CCT_HIP_POOL_PLANE=1 takes the plane-tiled kernels at any size (used by the tests on small shapes)
-static bool force_pool_plane() {
-  const char *e = getenv("CCT_HIP_POOL_PLANE");
-  return e && e[0] == '1';
-}
+// tuning knob pool_plane = 1 takes the plane-tiled kernels at any size (used by the tests on small shapes)
+static bool force_pool_plane() { return tuning().pool_plane == 1; }
 
 // planes per workgroup: enough elements to keep 256 lanes busy for a few rounds, within the LDS tile
 static int pool_planes_per_block(size_t plane_words, size_t work_words, size_t planes) {
@@ -689,8 +686,10 @@ __global__ __launch_bounds__(TPB) void softmax_fwd_kernel(float *__restrict__ pr
   for (int i = tid; i < len; i += TPB) y[i] = expf(x[i] - mx) / s;
   __syncthreads();
   if (tid == 0) {
-    const float pl = y[(int)labels[ib]];
-    loss_per_image[ib] = -logf(fmaxf(pl, FLT_MIN));
+    // a label outside [0, len) (NaN included) is never used as an index: the image's loss is NaN
+    const float lf = labels[ib];
+    const bool valid = lf >= 0.0f && lf < (float)len;
+    loss_per_image[ib] = valid ? -logf(fmaxf(y[(int)lf], FLT_MIN)) : __int_as_float(0x7fc00000);
   }
 }
 // batch sum in ascending image order (the order the reference accumulates its scalar loss)
@@ -710,7 +709,8 @@ __global__ __launch_bounds__(TPB) void softmax_bwd_kernel(float *__restrict__ ig
   const uint32_t ib = fdiv(e, div_len);
   const int i = e - ib * len;
   float v = prob[e];
-  if (i == (int)labels[ib]) v -= 1.0f;
+  const float lf = labels[ib];
+  if (lf >= 0.0f && lf < (float)len && i == (int)lf) v -= 1.0f;
   ig[e] = (float)((double)v * factor);
 }
 

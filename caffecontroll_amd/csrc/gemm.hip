@@ -520,10 +520,7 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   // 16-byte global loads need dword alignment only
   g.a_vec = ((uintptr_t)A % 4 == 0);
   g.b_vec = ((uintptr_t)B % 4 == 0);
-  {
-    const char *e = getenv("CCT_HIP_GEMM_NT");
-    g.nt_store = e ? atoi(e) : 0;
-  }
+  g.nt_store = tuning().gemm_nt;
   if (K <= 0) g.K = 0;  // degenerate: C = beta*C through the normal epilogue with zero accumulators
 
   // Tile shape and split-K factor come from a small occupancy model.  A compute unit holds `occ`
@@ -541,9 +538,9 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   const double cu_rate = 0.8 * 157.3e12 / 256.0, hbm_rate = 4.0e12;
   int cfg = 1, splits = 1, kchunk = g.K > 0 ? g.K : bk;
   double best = 1e30;
-  static const int forced = [] { const char *e = getenv("CCT_HIP_GEMM_TILE"); return e ? atoi(e) : -1; }();
+  const int forced = tuning().gemm_tile;
   for (int c = 0; c < 5; ++c) {
-    if (forced >= 0 && forced <= 4 && c != forced) continue;  // tuning override, read once
+    if (forced >= 0 && forced <= 4 && c != forced) continue;  // tuning override
     const Shape &sh = shapes[c];
     const long tiles = (long)((M + sh.bm - 1) / sh.bm) * ((N + sh.bn - 1) / sh.bn);
     const long slots = (long)sh.occ * cus;

@@ -65,6 +65,7 @@ class AbstractBridge {
   virtual LogicalCubeType *get_model_history_cube() { return nullptr; }
   virtual LogicalCubeType *get_bias_history_cube() { return nullptr; }
   virtual void set_current_iter(int) {}
+  virtual int get_current_iter() { return -1; }  // -1: no updater
 };
 
 }  // namespace cct

@@ -94,6 +94,8 @@ class LmdbReader {
     base_ = nullptr;
     fd_ = -1;
     entries_ = 0;
+    root_ = ~0ull;  // next() after close() reports the end instead of walking unmapped pages
+    started_ = false;
     stack_.clear();
   }
 

@@ -19,8 +19,10 @@
 // every bridge in order its model cube and then its bias cube; a snapshot is three files
 // <base>.snapshot_iter<N>.{MODEL,HISTORY,ITER}.bin (weights, momentum buffers, one int).
 #pragma once
+#include <cmath>
 #include <cstdio>
 #include <memory>
+#include <stdexcept>
 #include <string>
 #include <vector>
 
@@ -47,8 +49,85 @@ class Network {
     std::vector<cnn::LayerParameter *> params;
   };
 
+  // Walks the chain with the reference's size rules (conv (R+2p-K)/s+1, src/DeepNet.h:112-115;
+  // pooling (R-K)/s+1, :1374-1376) and returns "" if every layer can be built, else a message that
+  // names the layer.  Host arithmetic only; the constructor runs it first, so a bad description
+  // ends in an exception instead of an unsigned wrap-around, a division by zero or a huge allocation.
+  static std::string validate(int batch, int depth, int size, const cct_layer_spec *specs, int n_specs,
+                              const cct_solver_param *sp) {
+    auto at = [](int i, const std::string &what) { return "layer " + std::to_string(i) + ": " + what; };
+    if (batch <= 0 || depth <= 0 || size <= 0) return "batch, depth and size must be positive";
+    if (!specs || n_specs <= 0) return "no layers";
+    if (sp) {
+      float r;
+      if (sp->lr_policy && !Util::try_get_learning_rate(sp->lr_policy, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, &r))
+        return std::string("unknown or unsupported lr_policy \"") + sp->lr_policy + "\"";
+      if (sp->lr_policy && std::string(sp->lr_policy) == "step" && sp->stepsize <= 0)
+        return "lr_policy \"step\" needs stepsize >= 1";
+      if (sp->lr_policy && std::string(sp->lr_policy) == "poly" && sp->max_iter <= 0)
+        return "lr_policy \"poly\" needs max_iter >= 1";
+      if (sp->regularization_type && std::string(sp->regularization_type) != "L2" &&
+          std::string(sp->regularization_type) != "L1")
+        return std::string("regularization_type must be L2 or L1, not \"") + sp->regularization_type + "\"";
+    }
+    long R = size, D = depth;
+    for (int i = 0; i < n_specs; ++i) {
+      const cct_layer_spec &s = specs[i];
+      switch (s.type) {
+        case CCT_LAYER_CONV: {
+          if (s.num_output <= 0) return at(i, "convolution needs num_output >= 1");
+          if (s.kernel_size < 1 || s.stride < 1 || s.pad < 0)
+            return at(i, "convolution needs kernel_size >= 1, stride >= 1 and pad >= 0");
+          if (s.kernel_size > R + 2L * s.pad)
+            return at(i, "kernel_size " + std::to_string(s.kernel_size) + " exceeds the padded input (" +
+                             std::to_string(R + 2L * s.pad) + ")");
+          const int g = s.group > 1 ? s.group : 1;
+          if (D % g || s.num_output % g) return at(i, "group must divide input depth and num_output");
+          if (s.weight_filler.type < 0 || s.weight_filler.type > 3 || s.bias_filler.type < 0 || s.bias_filler.type > 3)
+            return at(i, "unknown filler type");
+          R = (R + 2L * s.pad - s.kernel_size) / s.stride + 1;
+          D = s.num_output;
+          break;
+        }
+        case CCT_LAYER_FC:
+          if (s.num_output <= 0) return at(i, "inner product needs num_output >= 1");
+          if (s.weight_filler.type < 0 || s.weight_filler.type > 3 || s.bias_filler.type < 0 || s.bias_filler.type > 3)
+            return at(i, "unknown filler type");
+          R = 1;
+          D = s.num_output;
+          break;
+        case CCT_LAYER_MAXPOOL:
+          if (s.kernel_size < 1 || s.stride < 1) return at(i, "pooling needs kernel_size >= 1 and stride >= 1");
+          if (s.kernel_size > R)
+            return at(i, "pooling kernel_size " + std::to_string(s.kernel_size) + " exceeds the input (" +
+                             std::to_string(R) + ")");
+          R = (R - s.kernel_size) / s.stride + 1;
+          break;
+        case CCT_LAYER_LRN:
+          if (s.lrn_local_size < 1 || s.lrn_local_size % 2 == 0) return at(i, "LRN local_size must be odd and >= 1");
+          if (!std::isfinite(s.lrn_alpha) || !std::isfinite(s.lrn_beta)) return at(i, "LRN alpha and beta must be finite");
+          break;
+        case CCT_LAYER_DROPOUT:
+          if (!(s.dropout_ratio >= 0.f && s.dropout_ratio < 1.f)) return at(i, "dropout_ratio must be in [0, 1)");
+          break;
+        case CCT_LAYER_RELU:
+        case CCT_LAYER_SOFTMAXLOSS:
+          break;
+        default:
+          return at(i, "unknown layer type " + std::to_string(s.type));
+      }
+      if ((double)batch * (double)D * (double)R * (double)R >= 2147483648.0)
+        return at(i, "output tensor has 2^31 elements or more");
+    }
+    return "";
+  }
+
   Network(int batch, int depth, int size, const cct_layer_spec *specs, int n_specs, const cct_solver_param *sp)
       : batch_(batch) {
+    {
+      const std::string why = validate(batch, depth, size, specs, n_specs, sp);
+      if (!why.empty()) throw std::invalid_argument(why);
+    }
     if (sp) {
       solver_.base_lr_ = sp->base_lr; solver_.momentum_ = sp->momentum; solver_.gamma_ = sp->gamma;
       solver_.power_ = sp->power; solver_.weight_decay_ = sp->weight_decay; solver_.stepsize_ = sp->stepsize;
@@ -291,6 +370,15 @@ class Network {
     for (Node &nd : nodes_)
       for (BridgeT *b : nd.bridges) b->set_current_iter(iter);
   }
+  // updates applied so far by the first layer that has a model (all updaters advance together)
+  int current_iter() {
+    for (Node &nd : nodes_)
+      for (BridgeT *b : nd.bridges)
+        if (b->get_current_iter() >= 0) return b->get_current_iter();
+    return 0;
+  }
+  // scores per image entering the loss layer (0 without one): labels must lie in [0, this)
+  int num_classes() const { return softmax_ ? (int)(softmax_->iR * softmax_->iC * softmax_->iD) : 0; }
 
   // DeepNet::write_full_snapshot (src/DeepNet.h:268-295)
   bool write_snapshot(const std::string &base_filename, int iter) {
@@ -350,10 +438,8 @@ class Network {
     dst.type_ = names[src.type];
     dst.value_ = src.value; dst.mean_ = src.mean; dst.std_ = src.std;
   }
-  static void fail(const char *msg) {
-    std::fprintf(stderr, "Network: %s\n", msg);
-    std::abort();
-  }
+  // caught at the C boundary (cct_net_create and friends return an error code and message)
+  [[noreturn]] static void fail(const char *msg) { throw std::runtime_error(std::string("Network: ") + msg); }
   LayerT *new_layer(size_t R, size_t C, size_t D) {
     LayerT *l = new LayerT(new CubeT(R, C, D, batch_, &driver_), new CubeT(R, C, D, batch_, &driver_));
     layers_.push_back(l);

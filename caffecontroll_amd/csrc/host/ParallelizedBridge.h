@@ -86,6 +86,10 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
     if (p_grad_updater_bias) p_grad_updater_bias->set_current_iter(iter);
   }
 
+  int get_current_iter() override {
+    return p_grad_updater ? p_grad_updater->current_iter : p_grad_updater_bias ? p_grad_updater_bias->current_iter : -1;
+  }
+
   void forward() override {
     this->report_forward_history.reset();
     p_sub_bridge->forward();

@@ -101,6 +101,15 @@ __device__ void bias_backward_block(const LiftParams &P, int blk) {
   }
 }
 
+// Checks the launch just enqueued.  If it was refused while it was meant to use the arrival
+// counters, they are flagged so that they are cleared before their next use.
+static int check_counter_launch(const LiftParams &P) {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return 0;
+  if (P.counters) mark_counters_dirty();
+  return set_error((int)e, "lift / bias-gradient launch failed: %s", hipGetErrorString(e));
+}
+
 // host side: choose the batch split of the bias reduction and fetch its scratch
 static int setup_bias(LiftParams &P, float *bias_grad, const float *out_grad, int fmap, int depth, int batch,
                       bool fused_with_lift) {
@@ -287,8 +296,7 @@ static int launch_lift(float *dst, const float *src, const cct_inverse_lower_cub
                        (uint32_t)nruns, make_fastdiv(per_row));
   } else
     hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
-  CCT_LAUNCH_CHECK();
-  return 0;
+  return check_counter_launch(P);
 }
 
 }  // namespace cct
@@ -325,6 +333,5 @@ extern "C" int cct_hip_backward_bias(float *bias_grad, const float *out_grad, in
   if (rc) return rc;
   hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(P.nbias), dim3(LIFT_THREADS), 0, ctx().stream,
                      (float *)nullptr, (const float *)nullptr, P);
-  CCT_LAUNCH_CHECK();
-  return 0;
+  return check_counter_launch(P);
 }

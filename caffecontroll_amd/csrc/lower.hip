@@ -225,8 +225,8 @@ extern "C" int cct_hip_lower_cube(float *dst, const float *src, const cct_pmap_h
     }
   }
   hipStream_t st = ctx().stream;
-  CCT_HIP_CHECK(hipFuncSetAttribute((const void *)lower_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)lds_bytes));
+  static LdsGrant grant;
+  if (int rc = grant_dynamic_lds((const void *)lower_kernel, lds_bytes, grant)) return rc;
   hipLaunchKernelGGL(lower_kernel, dim3(P.nblocks), dim3(threads), lds_bytes, st, dst, src, P);
   CCT_LAUNCH_CHECK();
   return 0;

@@ -65,6 +65,10 @@ class HIPDriver:
     def set_stream(self, stream_handle):
         check(self.lib.cct_hip_set_stream(stream_handle), "set_stream")
 
+    def set_tuning(self, name, value):
+        """Tuning knob (see cct_hip_set_tuning in include/cct_hip.h), e.g. ("direct_tile", 22)."""
+        check(self.lib.cct_hip_set_tuning(name.encode(), int(value)), "set_tuning")
+
     def device_sync(self):
         check(self.lib.cct_hip_device_sync(), "device_sync")
 

@@ -113,6 +113,10 @@ NET_PROTOTYPES = {
     "cct_net_write_snapshot": ([_P, C.c_char_p, _I], _I),
     "cct_net_read_snapshot": ([_P, C.c_char_p, C.POINTER(_I)], _I),
     "cct_net_set_iter": ([_P, _I], _I),
+    "cct_net_get_iter": ([_P], _I),
+    "cct_net_num_classes": ([_P], _I),
+    "cct_net_validate": ([_I, _I, _I, C.POINTER(LayerSpec), _I, C.POINTER(SolverParam)], _I),
+    "cct_solver_learning_rate": ([C.POINTER(SolverParam), _I], C.c_float),
     "cct_net_parameter_size": ([_P], C.c_size_t),
 }
 _bound = False
@@ -130,6 +134,22 @@ def _bind():
 
 
 MODEL, BIAS, MODEL_GRAD, BIAS_GRAD, OUTPUT, INPUT_GRAD, AUX, MODEL_HISTORY, BIAS_HISTORY = range(9)
+
+
+def solver_learning_rate(solver, iteration):
+    """Util::get_learning_rate (src/util.h:76-93) for the solver's policy at `iteration`, from the
+    C++ host layer (no device needed); NaN for a policy the reference rejects."""
+    return _bind().cct_solver_learning_rate(C.byref(solver), int(iteration))
+
+
+def validate(batch, depth, size, layers, solver=None):
+    """Checks a layer chain the way `Net` does, without touching a device; raises CctHipError with
+    the offending layer in the message."""
+    lib = _bind()
+    layers = list(layers)
+    arr = (LayerSpec * len(layers))(*layers)
+    sp = solver or solver_param()
+    check(lib.cct_net_validate(batch, depth, size, arr, len(layers), C.byref(sp)), "net_validate")
 
 
 class Net:
@@ -196,6 +216,14 @@ class Net:
 
     def set_iter(self, iteration):
         check(self.lib.cct_net_set_iter(self.h, iteration), "net_set_iter")
+
+    def get_iter(self):
+        """Number of updates the gradient updaters have applied (their schedule position)."""
+        return self.lib.cct_net_get_iter(self.h)
+
+    def num_classes(self):
+        """Scores per image entering the loss layer (0 if the chain has none)."""
+        return self.lib.cct_net_num_classes(self.h)
 
     def parameter_size(self):
         return self.lib.cct_net_parameter_size(self.h)

@@ -27,7 +27,7 @@ are outside this front end and are rejected with the layer's name in the message
 import os
 import re
 
-from . import nets
+from . import _lib, nets
 from .bridges import solver_param
 
 __all__ = ["Message", "parse", "parse_file", "solver_from_prototxt", "network_from_prototxt", "NetworkDef",
@@ -231,11 +231,26 @@ class NetworkDef:
             out.append((depth, size))
         return out
 
-    def build(self, depth, size=None, solver=None, batch=None):
-        """`nets.Net` on the device; `size` defaults to the data layer's crop size."""
+    def validate(self, depth, size=None, solver=None, batch=None):
+        """Checks the chain against an input of `depth` x `size` x `size` on the host (no device):
+        every kernel must fit its (padded) input, groups must divide the depths, and so on.  Raises
+        PrototxtError naming the layer as the prototxt does."""
         size = size or self.crop_size
         if not size:
             raise PrototxtError("input size is neither given nor set by crop_size")
+        try:
+            nets.validate(batch or self.batch_size, depth, size, self.layers, solver)
+        except _lib.CctHipError as e:
+            msg = str(e)
+            hit = re.search(r"layer (\d+): (.*)$", msg)
+            if hit:
+                raise PrototxtError("layer %r: %s" % (self.names[int(hit.group(1))], hit.group(2))) from None
+            raise PrototxtError(msg) from None
+
+    def build(self, depth, size=None, solver=None, batch=None):
+        """`nets.Net` on the device; `size` defaults to the data layer's crop size."""
+        self.validate(depth, size, solver, batch)
+        size = size or self.crop_size
         return nets.Net(batch or self.batch_size, depth, size, self.layers, solver)
 
 
@@ -332,11 +347,17 @@ def network_from_prototxt(text_or_message, phase="TRAIN", groups="honor"):
                                 % name)
         in_place = tops[0] == bottoms[0]
         lr, decay = _multipliers(l)
+
+        def need(cond, what):
+            if not cond:
+                raise PrototxtError("layer %r: %s" % (name, what))
         if typ == "CONVOLUTION":
             c = l.msg("convolution_param")
             if not c.has("num_output") or not c.has("kernel_size"):
                 raise PrototxtError("layer %r: num_output and kernel_size are required" % name)
             g = int(c.get("group", 1))
+            need(int(c.get("num_output")) >= 1 and int(c.get("kernel_size")) >= 1, "num_output and kernel_size must be >= 1")
+            need(int(c.get("stride", 1)) >= 1 and int(c.get("pad", 0)) >= 0 and g >= 1, "stride and group must be >= 1, pad >= 0")
             spec = nets.conv(int(c.get("num_output")), int(c.get("kernel_size")), stride=int(c.get("stride", 1)),
                              pad=int(c.get("pad", 0)), group=g if groups == "honor" else 1,
                              bias_term=int(bool(c.get("bias_term", True))), lr_mult=lr, decay_mult=decay)
@@ -346,6 +367,7 @@ def network_from_prototxt(text_or_message, phase="TRAIN", groups="honor"):
             c = l.msg("inner_product_param")
             if not c.has("num_output"):
                 raise PrototxtError("layer %r: num_output is required" % name)
+            need(int(c.get("num_output")) >= 1, "num_output must be >= 1")
             spec = nets.fc(int(c.get("num_output")), bias_term=int(bool(c.get("bias_term", True))),
                            lr_mult=lr, decay_mult=decay)
             spec.weight_filler = _filler(c.msg("weight_filler"), "weight_filler", name)
@@ -358,6 +380,7 @@ def network_from_prototxt(text_or_message, phase="TRAIN", groups="honor"):
                 raise PrototxtError("layer %r: padded pooling is not supported (src/DeepNet.h:1374-1376)" % name)
             if not c.has("kernel_size"):
                 raise PrototxtError("layer %r: kernel_size is required" % name)
+            need(int(c.get("kernel_size")) >= 1 and int(c.get("stride", 1)) >= 1, "kernel_size and stride must be >= 1")
             spec = nets.maxpool(int(c.get("kernel_size")), int(c.get("stride", 1)))
         elif typ == "RELU":
             spec = nets.relu()
@@ -365,9 +388,12 @@ def network_from_prototxt(text_or_message, phase="TRAIN", groups="honor"):
             c = l.msg("lrn_param")
             if str(c.get("norm_region", "ACROSS_CHANNELS")) not in ("ACROSS_CHANNELS", "0"):
                 raise PrototxtError("layer %r: only ACROSS_CHANNELS normalisation is on this path" % name)
+            need(int(c.get("local_size", 5)) >= 1 and int(c.get("local_size", 5)) % 2 == 1, "local_size must be odd and >= 1")
             spec = nets.lrn(int(c.get("local_size", 5)), float(c.get("alpha", 1.0)), float(c.get("beta", 0.75)))
         elif typ == "DROPOUT":
-            spec = nets.dropout(float(l.msg("dropout_param").get("dropout_ratio", 0.5)))
+            ratio = float(l.msg("dropout_param").get("dropout_ratio", 0.5))
+            need(0.0 <= ratio < 1.0, "dropout_ratio must be in [0, 1)")
+            spec = nets.dropout(ratio)
         else:
             raise PrototxtError("layer %r: type %r is not supported by this front end" % (name, l.get("type")))
         if in_place and typ not in ("RELU", "DROPOUT"):

@@ -16,7 +16,19 @@ import numpy as np
 from . import _lib, nets
 from ._lib import check
 
-__all__ = ["train", "test", "upload_batch", "batch_accuracy"]
+__all__ = ["train", "test", "upload_batch", "batch_accuracy", "check_labels", "learning_rate"]
+
+
+def check_labels(labels, num_classes):
+    """The loss layer indexes the class scores with the label (src/kernels/softmax.hxx:49-52), so a
+    label outside [0, num_classes) -- or a NaN -- is refused here, on the host, before it can reach
+    the device.  Returns the labels as a flat float32 array."""
+    labels = np.ascontiguousarray(labels, dtype=np.float32).reshape(-1)
+    ok = (labels >= 0) & (labels < num_classes)   # False for NaN
+    if not ok.all():
+        i = int(np.flatnonzero(~ok)[0])
+        raise ValueError("label %r of image %d is outside [0, %d)" % (float(labels[i]), i, num_classes))
+    return labels
 
 
 def _h2d(lib, dev_ptr, arr):
@@ -32,6 +44,8 @@ def upload_batch(net, images, labels):
     lib = _lib.load()
     images = np.ascontiguousarray(images, dtype=np.float32)
     labels = np.ascontiguousarray(labels, dtype=np.float32).reshape(-1)
+    if net.num_classes():
+        labels = check_labels(labels, net.num_classes())
     if images.shape != (net.batch, net.depth, net.size, net.size):
         raise ValueError("images have shape %r, the network takes %r"
                          % (images.shape, (net.batch, net.depth, net.size, net.size)))
@@ -61,6 +75,7 @@ class _CorpusSource:
             raise ValueError("the corpus produces %dx%dx%dx%d batches, the network takes %dx%dx%dx%d" % (
                 cp.info.batch, cp.info.channels, cp.info.out_rows, cp.info.out_cols, net.batch, net.depth, net.size, net.size))
         self.net, self.cp = net, cp
+        cp.set_num_classes(net.num_classes())
         self.epoch_of_next = cp.load_next()
 
     def next_into_network(self):
@@ -88,23 +103,9 @@ def _cycle(batches):
 
 
 def learning_rate(solver, iteration):
-    """Util::get_learning_rate (src/util.h:66-93) for the status line; the updaters on the device
-    evaluate the same schedule themselves."""
-    policy = solver.lr_policy.decode()
-    lr, g, it = solver.base_lr, solver.gamma, float(iteration)
-    if policy == "fixed":
-        return lr
-    if policy == "step":
-        return lr * g ** (int(iteration) // solver.stepsize)
-    if policy == "exp":
-        return lr * g ** it
-    if policy == "inv":
-        return lr * (1.0 + g * it) ** (-solver.power)
-    if policy == "poly":
-        return lr * (1.0 - it / solver.max_iter) ** solver.power
-    if policy == "sigmoid":
-        return lr * (1.0 / (1.0 + np.exp(-g * (it - solver.stepsize))))
-    raise ValueError("unknown lr_policy %r" % policy)
+    """Util::get_learning_rate (src/util.h:76-93) at `iteration`, for the status line: evaluated by
+    the same C++ function the updaters on the device use (`cct_solver_learning_rate`)."""
+    return nets.solver_learning_rate(solver, iteration)
 
 
 def test(net, batches, log=print):

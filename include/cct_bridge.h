@@ -109,6 +109,14 @@ typedef struct cct_layer_spec {
 
 typedef struct cct_net cct_net;
 
+/* Checks a description the way cct_net_create does, on the host only (no device is touched):
+ * positive sizes, stride >= 1, 1 <= kernel_size <= (padded) input, num_output >= 1, group divides
+ * both depths, odd LRN window, dropout_ratio in [0, 1), known filler / layer / lr_policy names,
+ * tensors below 2^31 elements.  The reference asserts or divides by zero on such input
+ * (src/DeepNet.h:112-115, 1374-1376); here the call returns CCT_HIP_EINVAL and
+ * cct_hip_last_error() names the layer. */
+int cct_net_validate(int batch, int depth, int size, const cct_layer_spec *layers, int n_layers,
+                     const cct_solver_param *solver);
 int cct_net_create(cct_net **out, int batch, int depth, int size, const cct_layer_spec *layers, int n_layers,
                    const cct_solver_param *solver);
 int cct_net_destroy(cct_net *net);
@@ -143,6 +151,16 @@ int cct_net_write_snapshot(cct_net *net, const char *base_filename, int iter);
 int cct_net_read_snapshot(cct_net *net, const char *stem, int *iter);
 /* Iteration counter of every gradient updater (learning-rate schedule position). */
 int cct_net_set_iter(cct_net *net, int iter);
+/* Updates applied so far (GradientUpdater::current_iter, src/algorithms/GradientUpdater.h:24,156). */
+int cct_net_get_iter(cct_net *net);
+/* Scores per image entering the SoftmaxWithLoss layer (0 without one): every label must lie in
+ * [0, this) -- the loss indexes the scores with it (src/kernels/softmax.hxx:49-52). */
+int cct_net_num_classes(cct_net *net);
+/* Util::get_learning_rate (src/util.h:76-93) for the solver's policy at iteration `iter`: the value
+ * SGDGradientUpdater::get_stepsize multiplies with the layer's lr_mult
+ * (src/algorithms/GradientUpdater.h:42-45).  Host arithmetic only.  NaN for a policy the reference
+ * rejects ("multistep", unknown names). */
+float cct_solver_learning_rate(const cct_solver_param *solver, int iter);
 /* DeepNet::get_parameter_size (src/DeepNet.h:425-441): weights + biases of all layers. */
 size_t cct_net_parameter_size(cct_net *net);
 

@@ -61,6 +61,11 @@ int cct_corpus_create(cct_corpus **out, int batch, int channels, int height, int
                       float scale, int mirror, int phase, const float *mean, unsigned int seed);
 int cct_corpus_close(cct_corpus *c);
 int cct_corpus_get_info(cct_corpus *c, cct_corpus_info *info);
+/* Number of classes of the network's loss layer (0 = unknown, the default).  Once set, a batch that
+ * holds a label outside [0, num_classes) is refused by cct_corpus_load_next / cct_corpus_submit on
+ * the host and nothing of it is uploaded.  The reference indexes the class scores with the label
+ * unchecked (src/kernels/softmax.hxx:49-52); on a device that would be an out-of-bounds read. */
+int cct_corpus_set_num_classes(cct_corpus *c, int num_classes);
 
 /* Host stage, LMDB-fed: reads the next `batch` records (LoadLmdbData; wraps to the first record at
  * the end of the database and counts an epoch, as DeepNet::train_network does, src/DeepNet.h:2083-2095),

@@ -95,8 +95,17 @@ typedef struct cct_lrn_backward_args {
 /* DeviceDriver::set_device_id + init_thread (src/sched/DeviceDriver.h:269-272): selects the
  * device for the calling thread and creates the library state on first use. */
 int cct_hip_init(int device_id);
-/* Use an existing hipStream_t (passed as void*) for all later work; NULL = null stream. */
+/* Use an existing hipStream_t (passed as void*) for all later work; NULL = null stream.  The
+ * library works on ONE stream at a time: its split-K workspace and reduction counters are shared
+ * by all calls, so work must not be spread over several streams by switching between them while
+ * earlier calls are still running (synchronise before switching). */
 int cct_hip_set_stream(void *hip_stream);
+/* Tuning knobs, for experiments and for tests that pin a kernel instance.  Names: "direct_tile"
+ * (<map blocks><pixel blocks> of the direct convolution tile, 0 = automatic), "direct_waves",
+ * "direct_tb", "direct_nospec", "pool_plane", "gemm_nt", "gemm_tile" (-1 = automatic).  The
+ * environment variables CCT_HIP_<NAME IN CAPITALS> give the initial values; they are read once,
+ * when the library initialises, never on a launch path.  No counterpart in the reference. */
+int cct_hip_set_tuning(const char *name, int value);
 /* DeviceDriver::device_sync, src/sched/DeviceDriver.h:267. */
 int cct_hip_device_sync(void);
 const char *cct_hip_last_error(void);
@@ -279,7 +288,9 @@ int cct_hip_lrn_backward(float *in_grad, const float *out_grad, const cct_lrn_ba
 int cct_hip_dropout_forward_train(float *out, const float *in, const unsigned int *mask,
                                   float scale, unsigned int threshold, size_t n);
 /* parallel_map<_f_src_to_dst_softmax_forward,_f_softmax_forward>, src/kernels/softmax.hxx:19-60.
- * labels: device floats, one per image. loss_sum: device float, overwritten with the batch sum. */
+ * labels: device floats, one per image. loss_sum: device float, overwritten with the batch sum.
+ * A label outside [0, len_per_image) is never used as an index: that image's loss (and so the
+ * sum) becomes NaN, and the backward pass subtracts no 1 for it. */
 int cct_hip_softmax_loss_forward(float *prob, const float *in, const float *labels,
                                  float *loss_sum, int len_per_image, int batch);
 /* parallel_map<_f_src_to_dst_softmax_backward,_f_softmax_backward>, src/kernels/softmax.hxx:62-81:

@@ -307,7 +307,12 @@ void cct_oracle_sgd_update(size_t n, float *model, float *grad, float *history, 
   cct_oracle_saxpy(n, -1.0f, history, model);
 }
 
-/* Util::get_learning_rate, src/util.h:66-93 (multistep is unsupported there as well). */
+/* Util::get_learning_rate, src/util.h:76-93 (multistep is unsupported there as well).
+ * The reference is C++ with <math.h>: pow/exp on float arguments pick the float overloads
+ * (step, exp: powf; sigmoid: expf), mixed float/double arguments promote to double (inv, poly),
+ * and the product with base_lr is rounded to float on return.  Pinned in
+ * tests/test_learning_rate.py by float64 closed forms, schedule identities and the learning
+ * rates Caffe's LeNet tutorial log prints for the inv policy. */
 float cct_oracle_learning_rate(const char *policy, float base_lr, float gamma, float iter,
                                float stepsize, float power, float max_iter) {
   if (!strcmp(policy, "fixed")) return base_lr;
@@ -319,7 +324,7 @@ float cct_oracle_learning_rate(const char *policy, float base_lr, float gamma, f
   if (!strcmp(policy, "inv")) return (float)(base_lr * pow(1.0 + gamma * iter, -power));
   if (!strcmp(policy, "poly")) return (float)(base_lr * pow(1.0 - (iter / max_iter), power));
   if (!strcmp(policy, "sigmoid"))
-    return (float)(base_lr * (1.0 / (1.0 + exp(-gamma * (iter - stepsize)))));
+    return (float)(base_lr * (1.0 / (1.0 + expf(-gamma * (iter - stepsize)))));
   return NAN;
 }
 

@@ -18,6 +18,19 @@ def driver():
     return _state["drv"]
 
 
+class tuning:
+    """`with tuning("direct_tile", 22): ...` pins a library tuning knob and puts `default` back after."""
+
+    def __init__(self, name, value, default=0):
+        self.name, self.value, self.default = name, value, default
+
+    def __enter__(self):
+        driver().set_tuning(self.name, self.value)
+
+    def __exit__(self, *exc):
+        driver().set_tuning(self.name, self.default)
+
+
 def dev(a, dtype=None):
     import torch
     t = torch.from_numpy(np.ascontiguousarray(a if dtype is None else a.astype(dtype)))

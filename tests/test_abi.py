@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), "missing export: " + n
     assert sorted(bridges.BRIDGE_PROTOTYPES) == bnames
     from caffecontroll_amd import nets
-    nnames = _declared_symbols("cct_bridge.h", "cct_net_")
+    nnames = sorted(_declared_symbols("cct_bridge.h", "cct_net_") + _declared_symbols("cct_bridge.h", "cct_solver_"))
     assert len(nnames) >= 11
     for n in nnames:
         assert hasattr(lib, n), "missing export: " + n

@@ -134,3 +134,63 @@ def test_stage_profile_and_first_layer_mode():
     driver().memcpy(bg.ctypes.data, layer.bias_grad_ptr(), bg.nbytes, 1)
     assert (bg == b * n * n).all()
     layer.close()
+
+
+POLICIES = [
+    # (policy, base_lr, gamma, stepsize, power, max_iter)
+    ("fixed", 0.05, 0.3, 3, 2.0, 50),
+    ("step", 0.02, 0.5, 3, 3.0, 50),
+    ("exp", 0.05, 0.9, 3, 3.0, 50),
+    ("inv", 0.05, 0.05, 3, 0.75, 50),
+    ("poly", 0.05, 0.05, 3, 2.0, 12),
+    ("sigmoid", 0.05, -0.7, 4, 2.0, 50),
+]
+
+
+@pytest.mark.parametrize("policy", POLICIES, ids=lambda c: c[0])
+@pytest.mark.parametrize("l1", [False, True], ids=["L2", "L1"])
+def test_stepped_sgd_follows_the_schedule_bit_for_bit(oracle, policy, l1):
+    """SGDGradientUpdater::update with get_stepsize = lr_mult * Util::get_learning_rate(policy, ...,
+    iter) (src/algorithms/GradientUpdater.h:42-45, 154-193; src/util.h:76-93) over nine iterations,
+    across two `step` boundaries.  Input and output gradient are small integers, so the weight and
+    bias gradients are exact and the same in every iteration (they do not depend on the weights):
+    the weights on the device must then equal the oracle's updater, driven by the oracle's
+    schedule, bit for bit after every iteration."""
+    from caffecontroll_amd.bridges import ConvolutionLayer, solver_param
+    name, base, gamma, stepsize, power, max_iter = policy
+    b, d, n, k, s, p, o = 2, 3, 8, 3, 1, 1, 4
+    m = (n + 2 * p - k) // s + 1
+    rng = np.random.default_rng(31)
+    x = rng.integers(-3, 4, size=(b, d, n, n)).astype(np.float32)
+    og = rng.integers(-2, 3, size=(b, o, m, m)).astype(np.float32)
+    w = (rng.standard_normal((o, d, k, k)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(o).astype(np.float32)
+    driver()
+    in_data, in_grad = dev(x), empty((b, d, n, n))
+    out_data, out_grad = empty((b, o, m, m)), dev(og)
+    mom, wd, lr_mult, decay_mult = 0.9, 0.0005, (1.0, 2.0), (1.0, 0.5)
+    sp = solver_param(base_lr=base, momentum=mom, weight_decay=wd, lr_policy=name, gamma=gamma, stepsize=stepsize,
+                      power=power, max_iter=max_iter, regularization_type="L1" if l1 else "L2")
+    layer = ConvolutionLayer(b, d, n, k, s, p, o, in_data, in_grad, out_data, out_grad, solver=sp,
+                             lr_mult=lr_mult, decay_mult=decay_mult)
+    _copy_to(layer.model_ptr(), w)
+    _copy_to(layer.bias_ptr(), bias)
+    _, lowered = oracle.conv_forward(x, w, bias, k, s, p)
+    _, dw, db = oracle.conv_backward(x.shape, w, og, lowered, k, s, p)
+    rw, rb = w.reshape(-1).copy(), bias.copy()
+    hw, hb = np.zeros(w.size, np.float32), np.zeros(o, np.float32)
+    f32 = np.float32
+    rates = []
+    for it in range(1, 10):
+        layer.forward()
+        layer.backward(with_update=True)
+        rate = f32(oracle.learning_rate(name, base, gamma, it, stepsize, power, max_iter))
+        rates.append(float(rate))
+        oracle.sgd_update(rw, dw.reshape(-1).copy(), hw, f32(lr_mult[0]) * rate, mom, f32(wd) * f32(decay_mult[0]), l1)
+        oracle.sgd_update(rb, db.copy(), hb, f32(lr_mult[1]) * rate, mom, f32(wd) * f32(decay_mult[1]), l1)
+        np.testing.assert_array_equal(_read(layer.model_ptr(), (w.size,)), rw, err_msg="weights, iteration %d" % it)
+        np.testing.assert_array_equal(_read(layer.bias_ptr(), (o,)), rb, err_msg="bias, iteration %d" % it)
+        np.testing.assert_array_equal(_read(layer.history_ptr(), (w.size,)), hw, err_msg="momentum, iteration %d" % it)
+    if name != "fixed":
+        assert len(set(rates)) > 2, rates   # the schedule moved during the run, so it was exercised
+    layer.close()

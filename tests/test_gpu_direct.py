@@ -5,7 +5,7 @@ lowered GEMMs, so the bar is the fp32 one: max|gpu - ref| / max|ref| <= 1e-4."""
 import numpy as np
 import pytest
 
-from gpu_util import dev, driver, empty, host, rel_err
+from gpu_util import dev, driver, empty, host, rel_err, tuning
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4
@@ -134,9 +134,9 @@ def test_direct_kernels_match_oracle(oracle, shape):
 
 @pytest.mark.parametrize("tile", [11, 12, 21, 22, 31, 32, 41, 42])
 @pytest.mark.parametrize("shape", [(3, 96, 27, 5, 2, 256), (3, 256, 13, 3, 1, 384), (2, 20, 12, 5, 0, 50)], ids=_ids)
-def test_direct_every_tile_instance(oracle, shape, tile, monkeypatch):
+def test_direct_every_tile_instance(oracle, shape, tile):
     """The library picks the tile (32*t1 maps x 128*t2 pixels) from an occupancy estimate; every
-    instance must give the same convolution.  CCT_HIP_DIRECT_TILE=<t1><t2> pins the choice; a map
+    instance must give the same convolution.  The tuning knob direct_tile=<t1><t2> pins the choice; a map
     tile that does not divide the padded map count is refused, never run."""
     b, d, n, k, p, o = shape
     x, w, bias, og, m = _tensors(shape, 99 + sum(shape))
@@ -145,20 +145,20 @@ def test_direct_every_tile_instance(oracle, shape, tile, monkeypatch):
     ref_dx, _, _ = oracle.conv_backward(x.shape, w, og, lowered, k, 1, p)
     d_x, d_w, d_og = dev(x), dev(w), dev(og)
     slabs_f, slabs_b = _slabs(d_w, o, d, k)
-    monkeypatch.setenv("CCT_HIP_DIRECT_TILE", str(tile))
     ran = 0
-    for maps, call, ref in (
-            (o, lambda t: drv.conv_direct_forward(t, d_x, slabs_f, dev(bias), b, d, n, k, p, o), ref_out),
-            (d, lambda t: drv.conv_direct_backward_data(t, d_og, slabs_b, b, d, n, k, p, o), ref_dx)):
-        padded = min(-(-maps // (32 * t)) * 32 * t for t in (2, 3, 4))
-        got = empty(ref.shape)
-        if padded % (32 * (tile // 10)):
-            with pytest.raises(Exception, match="not covered"):
-                call(got)
-            continue
-        call(got)
-        assert rel_err(host(got), ref) <= TOL
-        ran += 1
+    with tuning("direct_tile", tile):
+        for maps, call, ref in (
+                (o, lambda t: drv.conv_direct_forward(t, d_x, slabs_f, dev(bias), b, d, n, k, p, o), ref_out),
+                (d, lambda t: drv.conv_direct_backward_data(t, d_og, slabs_b, b, d, n, k, p, o), ref_dx)):
+            padded = min(-(-maps // (32 * t)) * 32 * t for t in (2, 3, 4))
+            got = empty(ref.shape)
+            if padded % (32 * (tile // 10)):
+                with pytest.raises(Exception, match="not covered"):
+                    call(got)
+                continue
+            call(got)
+            assert rel_err(host(got), ref) <= TOL
+            ran += 1
     if tile // 10 == 1:
         assert ran == 2  # single-block map tiles fit every map count
 

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from conftest import load_fixture
-from gpu_util import dev, driver, empty, host, rel_err
+from gpu_util import dev, driver, empty, host, rel_err, tuning
 
 pytestmark = pytest.mark.gpu
 
@@ -39,12 +39,13 @@ def test_relu_fixture_and_oracle(oracle):
                                  # rows of 27, 64 and 65 elements: the lanes-over-rows backward kernel and its limit
                                  (3, 5, 27, 3, 2), (2, 3, 64, 3, 2), (2, 3, 65, 2, 2)])
 @pytest.mark.parametrize("plane_tiled", [False, True])
-def test_maxpool_bit_exact(oracle, cfg, plane_tiled, monkeypatch):
+def test_maxpool_bit_exact(oracle, cfg, plane_tiled):
     # small tensors take the one-lane-per-element kernels unless the plane-tiled ones are forced
-    if plane_tiled:
-        monkeypatch.setenv("CCT_HIP_POOL_PLANE", "1")
-    else:
-        monkeypatch.delenv("CCT_HIP_POOL_PLANE", raising=False)
+    with tuning("pool_plane", int(plane_tiled)):
+        _maxpool_bit_exact(oracle, cfg)
+
+
+def _maxpool_bit_exact(oracle, cfg):
     B, D, n, k, s = cfg
     rng = np.random.default_rng(sum(cfg))
     if cfg == (5, 3, 10, 4, 2):
