@@ -98,6 +98,7 @@ PROTOTYPES = {
     "cct_hip_rand_uint_initialize": [_P, _I],
     "cct_hip_forward_bias": [_P, _P, _I, _I, _I],
     "cct_hip_backward_bias": [_P, _P, _I, _I, _I],
+    "cct_hip_backward_bias_noalloc": [_P, _P, _I, _I, _I],
     "cct_hip_backward_bias_fc": [_P, _P, _I, _I],
     "cct_hip_relu_forward": [_P, _P, _Z],
     "cct_hip_relu_backward": [_P, _P, _P, _Z],

@@ -15,6 +15,8 @@
 // Bias gradient (fused variant): workgroups past the lift range each own one output channel and
 // reduce out_grad[b][o][fmap] over b and fmap with per-lane partial sums, a wavefront
 // (cross-lane) reduction and a final pass over the workgroup's wave sums.
+#include <mutex>
+
 #include "cct_common.h"
 
 namespace cct {
@@ -110,12 +112,12 @@ static int check_counter_launch(const LiftParams &P) {
   return set_error((int)e, "lift / bias-gradient launch failed: %s", hipGetErrorString(e));
 }
 
-// host side: choose the batch split of the bias reduction and fetch its scratch
-static int setup_bias(LiftParams &P, float *bias_grad, const float *out_grad, int fmap, int depth, int batch,
+// host side: choose the batch split of the bias reduction (no scratch yet)
+static void plan_bias(LiftParams &P, float *bias_grad, const float *out_grad, int fmap, int depth, int batch,
                       bool fused_with_lift) {
   P.out_grad = out_grad; P.bias_grad = bias_grad; P.fmap = fmap; P.depth = depth; P.batch = batch;
   P.partial = nullptr; P.counters = nullptr; P.bsplit = 1; P.bchunk = batch; P.nbias = 0;
-  if (!bias_grad) return 0;
+  if (!bias_grad) return;
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
   // alone: two workgroups per CU; next to the lift blocks: about one per CU, so that the reduction
   // streams alongside the gather without crowding it out
@@ -126,9 +128,15 @@ static int setup_bias(LiftParams &P, float *bias_grad, const float *out_grad, in
   split = (batch + chunk - 1) / chunk;
   P.bsplit = split; P.bchunk = chunk;
   P.nbias = (uint32_t)depth * split;
-  if (split > 1) {
+}
+
+// the same, with the scratch of a split reduction taken from the library's grow-only workspace
+static int setup_bias(LiftParams &P, float *bias_grad, const float *out_grad, int fmap, int depth, int batch,
+                      bool fused_with_lift) {
+  plan_bias(P, bias_grad, out_grad, fmap, depth, batch, fused_with_lift);
+  if (P.bsplit > 1) {
     void *ws = nullptr;
-    int rc = get_workspace((size_t)depth * split * sizeof(float), &ws);
+    int rc = get_workspace((size_t)depth * P.bsplit * sizeof(float), &ws);
     if (rc) return rc;
     P.partial = (float *)ws;
     rc = get_counters(&P.counters);
@@ -303,6 +311,40 @@ static int launch_lift(float *dst, const float *src, const cct_inverse_lower_cub
 
 using namespace cct;
 
+// ---- scratch of the entry point that allocates nothing ------------------------------------------
+// Arrival counters (one per channel) followed by the partial sums of a split reduction.  Every GPU
+// the library runs on holds its own copy of this array until the process ends.
+constexpr int kNoAllocMaxDepth = 4096;       // channels
+constexpr int kNoAllocMaxPartials = 16384;   // depth * batch split
+constexpr size_t kNoAllocCounterBytes = (size_t)kNoAllocMaxDepth * sizeof(unsigned int);
+constexpr size_t kNoAllocScratchBytes = kNoAllocCounterBytes + (size_t)kNoAllocMaxPartials * sizeof(float);
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+
+// The array's name is only a host-side stand-in: its device address differs per GPU and comes from
+// hipGetSymbolAddress, asked once per device with that device current.
+constexpr int kMaxDevices = 64;
+static void *g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mu;
+
+static int scratch_address(void **out) {
+  const int dev = ctx().device;
+  CCT_REQUIRE(dev >= 0 && dev < kMaxDevices, "backward_bias_noalloc: device %d out of range", dev);
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    CCT_HIP_CHECK(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    CCT_REQUIRE(ptr != nullptr, "backward_bias_noalloc: no device address for the scratch array");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
+__global__ void zero_words_kernel(unsigned int *__restrict__ p, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
 extern "C" int cct_hip_inverse_lower_cube(float *dst, const float *src,
                                           const cct_inverse_lower_cube_args *args) {
   CCT_ENSURE_INIT();
@@ -334,4 +376,39 @@ extern "C" int cct_hip_backward_bias(float *bias_grad, const float *out_grad, in
   hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(P.nbias), dim3(LIFT_THREADS), 0, ctx().stream,
                      (float *)nullptr, (const float *)nullptr, P);
   return check_counter_launch(P);
+}
+
+extern "C" int cct_hip_backward_bias_noalloc(float *bias_grad, const float *out_grad, int fmap_size,
+                                             int depth, int batch_size) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(bias_grad && out_grad, "backward_bias_noalloc: null argument");
+  CCT_REQUIRE(fmap_size > 0 && depth > 0 && batch_size > 0,
+              "backward_bias_noalloc: fmap/depth/batch must be positive");
+  CCT_REQUIRE(depth <= kNoAllocMaxDepth,
+              "backward_bias_noalloc: depth %d exceeds the built-in scratch (at most %d channels); "
+              "use cct_hip_backward_bias",
+              depth, kNoAllocMaxDepth);
+  LiftParams P = {};
+  P.nblocks = 0;
+  plan_bias(P, bias_grad, out_grad, fmap_size, depth, batch_size, false);
+  CCT_REQUIRE((long)depth * P.bsplit <= kNoAllocMaxPartials,
+              "backward_bias_noalloc: %d x %d partial sums exceed the built-in scratch (at most %d); "
+              "use cct_hip_backward_bias",
+              depth, P.bsplit, kNoAllocMaxPartials);
+  hipStream_t st = ctx().stream;
+  if (P.bsplit > 1) {
+    void *base = nullptr;
+    int rc = scratch_address(&base);
+    if (rc) return rc;
+    P.counters = (unsigned int *)base;
+    P.partial = (float *)((unsigned char *)base + kNoAllocCounterBytes);
+    // the array keeps the last call's contents: the counters this launch uses must start at zero
+    // (a fill kernel, not a memset node, so that a caller may capture the call into a graph)
+    hipLaunchKernelGGL(zero_words_kernel, dim3((depth + 255) / 256), dim3(256), 0, st, P.counters, depth);
+    CCT_LAUNCH_CHECK();
+  }
+  hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(P.nbias), dim3(LIFT_THREADS), 0, st, (float *)nullptr,
+                     (const float *)nullptr, P);
+  CCT_LAUNCH_CHECK();
+  return 0;
 }

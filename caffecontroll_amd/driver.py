@@ -196,6 +196,10 @@ class HIPDriver:
         check(self.lib.cct_hip_backward_bias(_p(bias_grad), _p(out_grad), fmap, depth, batch),
               "backward_bias")
 
+    def backward_bias_noalloc(self, bias_grad, out_grad, fmap, depth, batch):
+        check(self.lib.cct_hip_backward_bias_noalloc(_p(bias_grad), _p(out_grad), fmap, depth, batch),
+              "backward_bias_noalloc")
+
     def backward_bias_fc(self, bias_grad, out_grad, D, B):
         check(self.lib.cct_hip_backward_bias_fc(_p(bias_grad), _p(out_grad), D, B), "backward_bias_fc")
 

@@ -260,6 +260,16 @@ int cct_hip_forward_bias(const float *bias, float *out, int fmap_size, int depth
 /* DeviceDriver::backward_bias (src/sched/DeviceDriver.h:129-133): bias_grad[d] = sum_b sum_fmap. */
 int cct_hip_backward_bias(float *bias_grad, const float *out_grad, int fmap_size, int depth,
                           int batch_size);
+/* cct_hip_backward_bias for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arithmetic and summation order as cct_hip_backward_bias, but the partial sums and arrival
+ * counters of the split reduction live in an array built into the library (80 KB per GPU, held
+ * until the process ends) instead of the library's grow-only workspace: the call allocates and
+ * frees nothing.  Limits: depth <= 4096 and depth x (batch split) <= 16384, else CCT_HIP_EINVAL.
+ * Every call on a GPU shares that GPU's array: calls that overlap on one GPU (two streams, two
+ * host threads) race. */
+int cct_hip_backward_bias_noalloc(float *bias_grad, const float *out_grad, int fmap_size, int depth,
+                                  int batch_size);
 /* DeviceDriver::backward_bias_fc (src/sched/DeviceDriver.h:135-138): bias[d] = sum_b out[b][d]. */
 int cct_hip_backward_bias_fc(float *bias_grad, const float *out_grad, int D, int B);
 

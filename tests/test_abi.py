@@ -70,3 +70,26 @@ def test_host_helpers_fill_structs_like_the_connector():
     assert (l.data_output_width, l.kernel_size, l.stride, l.iR, l.iD, l.iB) == (55, 11, 4, 227, 3, 256)
     r = remap_pmap(27, 27, 256, 8)
     assert (r.sD, r.sB, r.sBR) == (256, 8, 16)
+
+
+def test_noalloc_scratch_array_is_exported_by_the_device_code():
+    """hipGetSymbolAddress resolves the built-in scratch array by the name the host side registers;
+    the gfx950 code object must export that name (a symbol left local cannot be resolved and the
+    HIP runtime ends the process).  Checked on the object file the library was linked from."""
+    import shutil
+    import subprocess
+    import tempfile
+    import pytest
+    obj = os.path.join(ROOT, "caffecontroll_amd", "csrc", "lift.o")
+    bundler = "/opt/rocm/llvm/bin/clang-offload-bundler"
+    if not (os.path.exists(obj) and os.path.exists(bundler) and shutil.which("objcopy") and shutil.which("readelf")):
+        pytest.skip("object file or binutils not present")
+    with tempfile.TemporaryDirectory() as tmp:
+        fat, co = os.path.join(tmp, "fat.bin"), os.path.join(tmp, "dev.co")
+        subprocess.check_call(["objcopy", "-O", "binary", "--only-section=.hip_fatbin", obj, fat])
+        subprocess.check_call([bundler, "--unbundle", "--type=o", "--input=" + fat,
+                               "--targets=hipv4-amdgcn-amd-amdhsa--gfx950", "--output=" + co])
+        table = subprocess.check_output(["readelf", "--dyn-syms", "-W", co], text=True)
+    rows = [l.split() for l in table.splitlines() if l.strip().endswith("scratch")]
+    assert rows, "the scratch array is missing from the exported symbols"
+    assert all(r[4] == "GLOBAL" and r[3] == "OBJECT" and int(r[2]) == 81920 for r in rows), rows
