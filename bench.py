@@ -27,22 +27,33 @@ CONFIGS = {
 }
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the three GEMM instances at the alexnet_conv2 shape, from rocprofv3 --pmc
-# FETCH_SIZE and WRITE_SIZE runs of this file (one counter per run), each scaled by what the same
-# counter reads for a 1 GiB device copy (factors 2.000 and 1.000); the counter summary is kept
-# under profiles/.  fetched + written, in bytes.
-# Keyed by (path level, stage).
-GEMM_TRAFFIC_BYTES = {
-    (1, "GEMM"): (1868.6 + 192.4) * 1e6,
-    (1, "GEMM Data"): (1137.0 + 1791.6) * 1e6,
-    (1, "GEMM Wghts"): (2143.4 + 63.9) * 1e6,
-    (2, "GEMM"): (1868.6 + 192.4) * 1e6,
-    (2, "GEMM Data"): (280.4 + 73.5) * 1e6,
-    (2, "GEMM Wghts"): (2143.4 + 63.9) * 1e6,
-    (3, "GEMM"): (230.1 + 223.7) * 1e6,
-    (3, "GEMM Data"): (322.3 + 75.7) * 1e6,
-    (3, "GEMM Wghts"): (359.6 + 41.8) * 1e6,
+# HBM bytes per launch (fetched + written) at the alexnet_conv2 shape, from rocprofv3 --pmc FETCH_SIZE
+# and WRITE_SIZE runs of this file (one counter per run), each scaled by what the same counter
+# reads for a 1 GiB device copy (factors 2.000 and 1.000).  Not measured by this run: the record
+# names the summary under profiles/ the figure comes from.  Keyed by (stage, the kernel instance
+# the library reports it launched), so that a change of tile choice leaves `traffic` null instead
+# of attaching an old figure to another kernel.
+TRAFFIC_SOURCE = {"direct": "profiles/conv2_fwd_bwd_hbm_traffic_and_mfma.md",
+                  "lowering": "profiles/conv2_lowering_path_hbm_traffic_and_mfma.md"}
+TRAFFIC_BYTES = {
+    ("GEMM", "conv_direct_kernel<5,1,2,1,32>"): ((230.1 + 223.7) * 1e6, "direct"),
+    ("GEMM Data", "conv_direct_kernel<5,1,2,1,32>"): ((322.3 + 75.7) * 1e6, "direct"),
+    ("GEMM Wghts", "conv_direct_wgrad_spec_kernel<5,5,32,27,8>"): ((359.6 + 41.8) * 1e6, "direct"),
+    ("GEMM", "gemm_kernel<Tile<256,128,16,2,2>,true,true> splits=1"): ((1867.6 + 192.7) * 1e6, "lowering"),
+    ("GEMM Data", "gemm_kernel<Tile<128,128,16,2,2>,false,false> splits=1"): ((1209.0 + 1791.6) * 1e6, "lowering"),
+    ("GEMM Wghts", "gemm_kernel<Tile<256,128,16,2,2>,true,false> splits=26"): ((2203.8 + 63.9) * 1e6, "lowering"),
+    ("Lower Cube", "lower_kernel threads=320"): ((80.4 + 1791.6) * 1e6, "lowering"),
+    ("Inverse Lwr", "lift_kernel<5,1> bias_blocks=256"): ((2190.6 + 71.7) * 1e6, "lowering"),
 }
+
+
+def traffic_of(cfg, stage, kernel):
+    """(bytes, source file) from the committed counter summaries, or (None, None) when the kernel
+    instance that ran is not the one that was profiled."""
+    if cfg != "alexnet_conv2":
+        return None, None
+    ent = TRAFFIC_BYTES.get((stage, kernel))
+    return (ent[0], TRAFFIC_SOURCE[ent[1]]) if ent else (None, None)
 
 
 def synth(cfg, seed, torch):
@@ -253,6 +264,8 @@ def main():
     ap.add_argument("--path", type=int, default=-1, choices=[-1, 0, 1, 2, 3],
                     help="conv path level: 0 separate passes, 1 fused epilogues, 2 direct data gradient, 3 all "
                          "direct kernels (no lowered matrix); -1 = the bridge's default")
+    ap.add_argument("--no-lowering-path", action="store_true",
+                    help="skip the extra passes at path level 1 that report the lowering / lifting stages")
     ap.add_argument("--no-data-grad", action="store_true", help="first-layer mode: skip data-gradient GEMM and lift")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run 5 device-to-device copies of 1 GiB (a plain copy kernel of known size, used "
@@ -298,69 +311,81 @@ def main():
     in_grad = torch.empty_like(in_data)
     out_data = torch.empty((b, o, m, m), device="cuda")
     out_grad = torch.from_numpy(og).cuda()
-    layer = ConvolutionLayer(b, d, n, k, s, p, o, in_data, in_grad, out_data, out_grad)
-    drv.memcpy(layer.model_ptr(), w.ctypes.data, w.nbytes, 0)
-    drv.memcpy(layer.bias_ptr(), bias.ctypes.data, bias.nbytes, 0)
     need_dgrad = not args.no_data_grad
-    layer.set_options(fused=0 if args.unfused else (None if args.path < 0 else args.path), profile=True,
-                      needs_backward_grad=need_dgrad)
-    path = layer.path()
-
-    def step():
-        layer.forward()
-        layer.backward(with_update=False)
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    stage_sum = {}
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-        # reading the stage events waits for the step's last kernel (one host sync per step,
-        # as a training loop that reads its loss does)
-        for name, ms in layer.stage_ms().items():
-            stage_sum[name] = stage_sum.get(name, 0.0) + ms
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-    stages = {name: v / args.steps for name, v in stage_sum.items() if v > 0}
-
     # algorithmic work per launch
     lower_bytes = 4.0 * (b * d * n * n + b * m * m * k * k * d)
     gemm_flop = 2.0 * o * (b * m * m) * (k * k * d)
-    per_stage = {}
-    for name, ms in stages.items():
-        ent = {"ms": round(ms, 4)}
-        if name in ("GEMM", "GEMM Data", "GEMM Wghts"):
-            ent["tflops"] = round(gemm_flop / ms / 1e9, 2)
-            ent["frac_fp32_mfma_peak"] = round(gemm_flop / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)
-        elif name in ("Lower Cube", "Inverse Lwr"):
-            nbytes = lower_bytes
-            if name == "Inverse Lwr" and path == 1:
-                # the same launch also reads the output gradient once for the bias gradient
-                nbytes += 4.0 * b * o * m * m
-                ent["includes"] = "bias-gradient reduction in the same launch"
-            ent["gbs"] = round(nbytes / ms / 1e6, 1)
-            ent["frac_hbm_peak"] = round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)
-        per_stage[name] = ent
-    # dominant kernel = the GEMM instance with the longest average launch
-    gemm_names = [g for g in ("GEMM", "GEMM Data", "GEMM Wghts") if g in stages]
-    dom = max(gemm_names, key=lambda g: stages[g])
-    kernel_of = {"GEMM": "gemm_kernel<256x128x16, A k-contig, B k-contig> (forward, conv epilogue)",
-                 "GEMM Data": "gemm_kernel<128x128x16, A m-contig, B n-contig> (data gradient)",
-                 "GEMM Wghts": "gemm_kernel<256x128x16, A k-contig, B n-contig> split-K (weight gradient)"}
-    if path >= 2 and need_dgrad:
-        kernel_of["GEMM Data"] = "conv_direct_kernel (data gradient: remap + GEMM + lifting in one launch)"
-    if path == 3:
-        kernel_of["GEMM"] = "conv_direct_kernel (forward: lowering + GEMM + remap + bias in one launch)"
-        kernel_of["GEMM Wghts"] = "conv_direct_wgrad_kernel (weight gradient from input and output gradient)"
-    achieved = gemm_flop / stages[dom] / 1e9
-    roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-                "traffic": GEMM_TRAFFIC_BYTES.get((path, dom)) if cfg == "alexnet_conv2" else None,
-                "kernel": kernel_of[dom], "stage": dom, "flop_per_launch": gemm_flop,
-                "avg_launch_ms": round(stages[dom], 4)}
+
+    def run_path(level, steps, warmup):
+        """`steps` timed passes of forward + backward at one path level (None = the bridge's default);
+        returns (level in effect, wall seconds, per-stage records with the kernel instance that ran)."""
+        layer = ConvolutionLayer(b, d, n, k, s, p, o, in_data, in_grad, out_data, out_grad)
+        drv.memcpy(layer.model_ptr(), w.ctypes.data, w.nbytes, 0)
+        drv.memcpy(layer.bias_ptr(), bias.ctypes.data, bias.nbytes, 0)
+        layer.set_options(fused=level, profile=True, needs_backward_grad=need_dgrad)
+        path = layer.path()
+        for _ in range(warmup):
+            layer.forward()
+            layer.backward(with_update=False)
+        torch.cuda.synchronize()
+        stage_sum = {}
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            layer.forward()
+            layer.backward(with_update=False)
+            # reading the stage events waits for the step's last kernel (one host sync per step,
+            # as a training loop that reads its loss does)
+            for name, ms in layer.stage_ms().items():
+                stage_sum[name] = stage_sum.get(name, 0.0) + ms
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        kernels = layer.stage_kernels()
+        layer.close()
+        per_stage = {}
+        for name, total in stage_sum.items():
+            if total <= 0:
+                continue
+            ms = total / steps
+            ent = {"ms": round(ms, 4), "kernel": kernels.get(name, "")}
+            if name in ("GEMM", "GEMM Data", "GEMM Wghts"):
+                ent["tflops"] = round(gemm_flop / ms / 1e9, 2)
+                ent["frac_fp32_mfma_peak"] = round(gemm_flop / ms / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4)
+            elif name in ("Lower Cube", "Inverse Lwr"):
+                nbytes = lower_bytes
+                if name == "Inverse Lwr" and path == 1:
+                    # the same launch also reads the output gradient once for the bias gradient
+                    nbytes += 4.0 * b * o * m * m
+                    ent["includes"] = "bias-gradient reduction in the same launch"
+                ent["algorithmic_bytes"] = nbytes
+                ent["gbs"] = round(nbytes / ms / 1e6, 1)
+                ent["frac_hbm_peak"] = round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)
+            per_stage[name] = ent
+        return path, elapsed, per_stage
+
+    path, elapsed, per_stage = run_path(0 if args.unfused else (None if args.path < 0 else args.path),
+                                        args.steps, args.warmup)
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    def mfma_roofline(stages):
+        # dominant kernel = the product kernel with the longest average launch
+        dom = max((g for g in ("GEMM", "GEMM Data", "GEMM Wghts") if g in stages), key=lambda g: stages[g]["ms"])
+        ent = stages[dom]
+        traffic, source = traffic_of(cfg, dom, ent["kernel"])
+        return {"bound": "mfma", "achieved": ent["tflops"], "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                "frac": ent["frac_fp32_mfma_peak"], "traffic": traffic, "traffic_source": source,
+                "kernel": ent["kernel"], "stage": dom, "flop_per_launch": gemm_flop, "avg_launch_ms": ent["ms"]}
+
+    def hbm_roofline(stages):
+        # the HBM-bound kernels of the lowering path: the one further from the peak
+        names = [g for g in ("Lower Cube", "Inverse Lwr") if g in stages]
+        if not names:
+            return None
+        worst = min(names, key=lambda g: stages[g]["frac_hbm_peak"])
+        ent = stages[worst]
+        traffic, source = traffic_of(cfg, worst, ent["kernel"])
+        return {"bound": "hbm", "achieved": ent["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                "frac": ent["frac_hbm_peak"], "traffic": traffic, "traffic_source": source, "kernel": ent["kernel"],
+                "stage": worst, "bytes_per_launch": ent["algorithmic_bytes"], "avg_launch_ms": ent["ms"]}
 
     result = {
         "metric": "images/sec conv fwd+bwd (1 GPU)", "value": round(b * args.steps / elapsed, 1),
@@ -370,10 +395,20 @@ def main():
         "config": {"workload": "%s: conv fwd+bwd b=%d d=%d n=%d k=%d s=%d p=%d o=%d%s%s" % (
             cfg, b, d, n, k, s, p, o, "" if need_dgrad else " (no data gradient)",
             " (path level %d)" % path)},
-        "roofline": roofline, "stages": per_stage,
+        "roofline": mfma_roofline(per_stage), "stages": per_stage,
     }
+    if hbm_roofline(per_stage):
+        result["roofline_hbm"] = hbm_roofline(per_stage)
+    elif not args.no_lowering_path:
+        # The same layer once more through the reference's stage sequence (lower, GEMM, remap, GEMM,
+        # lift, GEMM; path level 1), outside `value`: per-stage times of the lowering path and the
+        # HBM-bound lowering / lifting kernels against the 8 TB/s roofline.
+        _, low_elapsed, low_stages = run_path(1, max(3, min(args.steps, 10)), 2)
+        result["stages_lowering_path"] = low_stages
+        result["lowering_path_ms_per_step"] = round(low_elapsed * 1e3 / max(3, min(args.steps, 10)), 4)
+        result["roofline_hbm"] = hbm_roofline(low_stages)
+        result["roofline_mfma_lowering_path"] = mfma_roofline(low_stages)
     if not args.no_cpu_baseline:
-        layer.close()
         del in_data, in_grad, out_data, out_grad
         result["cpu_baseline"] = cpu_baseline(cfg, seed)
     print(json.dumps(result))

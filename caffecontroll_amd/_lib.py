@@ -66,6 +66,7 @@ PROTOTYPES = {
     "cct_hip_set_tuning": [C.c_char_p, _I],
     "cct_hip_device_sync": [],
     "cct_hip_last_error": [],
+    "cct_hip_last_kernel": [],
     "cct_hip_compute_units": [],
     "cct_hip_malloc": [C.POINTER(_P), _Z],
     "cct_hip_free": [_P],
@@ -94,6 +95,12 @@ PROTOTYPES = {
     "cct_hip_sgd_update": [_Z, _P, _P, _P, _F, _F, _F, _I],
     "cct_hip_sgd_update_batch": [C.POINTER(SgdJob), _I],
     "cct_hip_sconstant_initialize": [_P, _Z, _F],
+    "cct_hip_fill_xavier": [_P, _Z, _Z, _I],
+    "cct_hip_fill_bernoulli": [_P, _Z, _F, _I],
+    "cct_hip_fill_gaussian": [_P, _Z, _F, _F, _I],
+    "cct_filler_draw_xavier": [_P, _Z, _Z, _I],
+    "cct_filler_draw_bernoulli": [_P, _Z, _F, _I],
+    "cct_filler_draw_gaussian": [_P, _Z, _F, _F, _I],
     "cct_hip_init_rng": [_I],
     "cct_hip_rand_uint_initialize": [_P, _I],
     "cct_hip_forward_bias": [_P, _P, _I, _I, _I],
@@ -116,7 +123,7 @@ PROTOTYPES = {
     "cct_hip_timer_stop": [_P],
     "cct_hip_timer_elapsed_ms": [_P, C.POINTER(_F)],
 }
-_RESTYPE = {"cct_hip_last_error": C.c_char_p, "cct_hip_conv_direct_slab_floats": C.c_size_t}
+_RESTYPE = {"cct_hip_last_error": C.c_char_p, "cct_hip_last_kernel": C.c_char_p, "cct_hip_conv_direct_slab_floats": C.c_size_t}
 
 _lib = None
 

@@ -38,6 +38,7 @@ BRIDGE_PROTOTYPES = {
     "cct_conv_bridge_forward": ([_P], _I),
     "cct_conv_bridge_backward": ([_P, _I], _I),
     "cct_conv_bridge_stage_ms": ([_P, C.POINTER(C.c_float)], _I),
+    "cct_conv_bridge_stage_kernel": ([_P, _I], C.c_char_p),
 }
 _bound = False
 
@@ -129,6 +130,11 @@ class ConvolutionLayer:
         arr = (C.c_float * len(STAGE_NAMES))()
         check(self.lib.cct_conv_bridge_stage_ms(self.h, arr), "conv_bridge_stage_ms")
         return dict(zip(STAGE_NAMES, list(arr)))
+
+    def stage_kernels(self):
+        """Stage name -> kernel instance the library launched for it ("" if the stage did not run)."""
+        return {name: (self.lib.cct_conv_bridge_stage_kernel(self.h, i) or b"").decode()
+                for i, name in enumerate(STAGE_NAMES)}
 
     def close(self):
         if self.h:

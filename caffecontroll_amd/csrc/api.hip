@@ -1,7 +1,10 @@
 // Process state, memory management and timing entry points of the driver library.
 #include <cstdarg>
 #include <cstring>
+#include <cmath>
 #include <mutex>
+#include <random>
+#include <vector>
 
 #include "cct_common.h"
 
@@ -29,6 +32,15 @@ static void read_tuning_from_env() {
   g_tuning.pool_plane = geti("CCT_HIP_POOL_PLANE", 0);
   g_tuning.gemm_nt = geti("CCT_HIP_GEMM_NT", 0);
   g_tuning.gemm_tile = geti("CCT_HIP_GEMM_TILE", -1);
+}
+
+static char g_last_kernel[192] = "";
+
+void note_kernel(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_kernel, sizeof(g_last_kernel), fmt, ap);
+  va_end(ap);
 }
 
 void mark_counters_dirty() {
@@ -172,6 +184,8 @@ int cct_hip_device_sync(void) {
 
 const char *cct_hip_last_error(void) { return g_err; }
 
+const char *cct_hip_last_kernel(void) { return g_last_kernel; }
+
 int cct_hip_compute_units(void) { return ctx().compute_units; }
 
 int cct_hip_malloc(void **dev_ptr, size_t size_in_byte) {
@@ -198,6 +212,71 @@ int cct_hip_memcpy(void *dst, const void *src, size_t size_in_byte, int kind) {
   CCT_HIP_CHECK(hipMemcpyAsync(dst, src, size_in_byte, k, ctx().stream));
   if (kind != 2) CCT_HIP_CHECK(hipStreamSynchronize(ctx().stream));
   return 0;
+}
+
+// ---- random fillers: drawn on the host exactly as CPUDriver does, then copied to the device ------
+// std::mt19937 seeded with random_seed (std::random_device when -1) and the standard library's
+// distribution objects, one draw per element in index order (src/sched/DeviceDriver_CPU.cpp:661-699).
+
+static unsigned filler_seed(int random_seed) {
+  if (random_seed != -1) return (unsigned)random_seed;
+  std::random_device rd;
+  return rd();
+}
+
+int cct_filler_draw_xavier(float *host, size_t n, size_t n_batch, int random_seed) {
+  CCT_REQUIRE(host || n == 0, "filler_draw_xavier: null array");
+  CCT_REQUIRE(n_batch > 0 && n / n_batch > 0, "filler_draw_xavier: fan-in must be positive");
+  const size_t fan_in = n / n_batch;
+  const float scale = std::sqrt(3.0 / fan_in);
+  std::mt19937 gen(filler_seed(random_seed));
+  std::uniform_real_distribution<float> uni(-scale, scale);
+  for (size_t i = 0; i < n; ++i) host[i] = uni(gen);
+  return 0;
+}
+
+int cct_filler_draw_bernoulli(float *host, size_t n, float p, int random_seed) {
+  CCT_REQUIRE(host || n == 0, "filler_draw_bernoulli: null array");
+  CCT_REQUIRE(p >= 0.0f && p <= 1.0f, "filler_draw_bernoulli: p must be in [0, 1]");
+  std::mt19937 gen(filler_seed(random_seed));
+  std::bernoulli_distribution bern(p);
+  for (size_t i = 0; i < n; ++i) host[i] = bern(gen);
+  return 0;
+}
+
+int cct_filler_draw_gaussian(float *host, size_t n, float mean, float std_dev, int random_seed) {
+  CCT_REQUIRE(host || n == 0, "filler_draw_gaussian: null array");
+  CCT_REQUIRE(std_dev > 0.0f, "filler_draw_gaussian: std must be positive");
+  std::mt19937 gen(filler_seed(random_seed));
+  std::normal_distribution<float> gaussian(mean, std_dev);
+  for (size_t i = 0; i < n; ++i) host[i] = gaussian(gen);
+  return 0;
+}
+
+static int upload_filler(float *arr, const std::vector<float> &host) {
+  CCT_REQUIRE(arr || host.empty(), "fill: null device array");
+  return cct_hip_memcpy(arr, host.data(), host.size() * sizeof(float), 0);
+}
+
+int cct_hip_fill_xavier(float *arr, size_t n, size_t n_batch, int random_seed) {
+  CCT_ENSURE_INIT();
+  std::vector<float> host(n);
+  int rc = cct_filler_draw_xavier(host.data(), n, n_batch, random_seed);
+  return rc ? rc : upload_filler(arr, host);
+}
+
+int cct_hip_fill_bernoulli(float *arr, size_t n, float p, int random_seed) {
+  CCT_ENSURE_INIT();
+  std::vector<float> host(n);
+  int rc = cct_filler_draw_bernoulli(host.data(), n, p, random_seed);
+  return rc ? rc : upload_filler(arr, host);
+}
+
+int cct_hip_fill_gaussian(float *arr, size_t n, float mean, float std_dev, int random_seed) {
+  CCT_ENSURE_INIT();
+  std::vector<float> host(n);
+  int rc = cct_filler_draw_gaussian(host.data(), n, mean, std_dev, random_seed);
+  return rc ? rc : upload_filler(arr, host);
 }
 
 int cct_hip_timer_create(void **timer) {

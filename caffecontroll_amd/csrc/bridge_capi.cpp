@@ -117,6 +117,11 @@ int cct_conv_bridge_stage_ms(cct_conv_bridge *h, float ms[CCT_CONV_STAGE_COUNT])
   return 0;
 }
 
+const char *cct_conv_bridge_stage_kernel(cct_conv_bridge *h, int stage) {
+  if (!h || stage < 0 || stage >= STAGE_COUNT) return "";
+  return h->pbridge->sub_bridge()->stage_kernel(stage).c_str();
+}
+
 struct cct_net {
   Network *net;
 };

@@ -57,6 +57,11 @@ struct LdsGrant {
 };
 int grant_dynamic_lds(const void *kernel, size_t bytes, LdsGrant &st);
 
+// Records the instance the launch path chose for the product kernel it just enqueued (template
+// arguments in the order a kernel trace prints them, plus launch-time choices such as the split
+// count); cct_hip_last_kernel() returns the most recent record.
+void note_kernel(const char *fmt, ...);
+
 #define CCT_HIP_CHECK(expr)                                                                    \
   do {                                                                                         \
     hipError_t _e = (expr);                                                                    \

@@ -380,6 +380,7 @@ static int direct_launch_ks(const DirectArgs &g, const DirectPlan &pl, hipStream
   if (pl.tmb == TMB && pl.tnb == TNB) {                                                                \
     hipLaunchKernelGGL((conv_direct_kernel<KS, TMB, TNB, CP, PW>), grid, block, pl.lds, st, g);        \
     CCT_LAUNCH_CHECK();                                                                                \
+    note_kernel("conv_direct_kernel<%d,%d,%d,%d,%d>", KS, TMB, TNB, CP, PW);                           \
     return 0;                                                                                          \
   }
   CCT_DIRECT_CASE(1, 1) CCT_DIRECT_CASE(2, 1) CCT_DIRECT_CASE(3, 1) CCT_DIRECT_CASE(4, 1)
@@ -962,6 +963,7 @@ static int wgrad_launch_spec(const WgradArgs &g, const WgradPlan &pl, hipStream_
   if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;
   hipLaunchKernelGGL(kern, dim3(g.nblocks), dim3(64 * W), pl.lds, st, g);
   CCT_LAUNCH_CHECK();
+  note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d>", KS, TB, PW, HO, W);
   return 0;
 }
 
@@ -975,6 +977,7 @@ static int wgrad_launch(const WgradArgs &g, const WgradPlan &pl, hipStream_t st)
     if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;                       \
     hipLaunchKernelGGL(kern, grid, block, pl.lds, st, g);                                               \
     CCT_LAUNCH_CHECK();                                                                                 \
+    note_kernel("conv_direct_wgrad_kernel<%d,%d,%d> waves=%d", KS, TB, PW, pl.waves);                   \
     return 0;                                                                                           \
   }
   CCT_WGRAD_CASE(1) CCT_WGRAD_CASE(2) CCT_WGRAD_CASE(3) CCT_WGRAD_CASE(4) CCT_WGRAD_CASE(5) CCT_WGRAD_CASE(6)

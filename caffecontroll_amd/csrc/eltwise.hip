@@ -846,6 +846,7 @@ int cct_hip_remap(float *dst, const float *src, const cct_pmap_helper *a) {
   hipLaunchKernelGGL(remap_kernel, dim3((uint32_t)slices, gy), dim3(TPB), 0, ctx().stream, dst, src,
                      (uint32_t)rc, (uint32_t)a->sD, make_fastdiv((uint32_t)a->sB));
   CCT_LAUNCH_CHECK();
+  note_kernel("remap_kernel");
   return 0;
 }
 
@@ -871,6 +872,7 @@ int cct_hip_remap_bias_backward(float *dst, const float *src, const cct_pmap_hel
   hipLaunchKernelGGL(bias_partial_sum_kernel, dim3((uint32_t)a->sB), dim3(TPB), 0, ctx().stream, bias_grad,
                      (const float *)ws, (uint32_t)a->sB, (uint32_t)a->sD, gy);
   CCT_LAUNCH_CHECK();
+  note_kernel("remap_bias_kernel");
   return 0;
 }
 

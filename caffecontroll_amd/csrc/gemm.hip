@@ -503,6 +503,8 @@ static int launch_cfg(GemmArgs &g, bool a_kc, bool b_kc, int splits, hipStream_t
   else if (!a_kc && b_kc) hipLaunchKernelGGL((gemm_kernel<T, false, true>), grid, block, 0, st, g);
   else hipLaunchKernelGGL((gemm_kernel<T, false, false>), grid, block, 0, st, g);
   CCT_LAUNCH_CHECK();
+  note_kernel("gemm_kernel<Tile<%d,%d,%d,%d,%d>,%s,%s> splits=%d", T::BM, T::BN, T::BK, T::WGM, T::WGN,
+              a_kc ? "true" : "false", b_kc ? "true" : "false", splits);
   return 0;
 }
 

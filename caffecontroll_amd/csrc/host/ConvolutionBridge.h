@@ -197,11 +197,14 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     if (timers_[stage] && stage_ran_[stage]) cct_hip_timer_elapsed_ms(timers_[stage], &ms);
     return ms;
   }
+  // the kernel instance the driver chose for the stage's product kernel the last time it ran with
+  // stage profiling on ("" if it has not)
+  const std::string &stage_kernel(int stage) const { return stage_kernel_[stage]; }
 
   // (1) input --lowering--> lowered  (2) model x lowered^T --> output  (3) remap + bias
   void forward() override {
     report_forward_history.reset();
-    for (int i = STAGE_LOWER; i <= STAGE_BIAS; ++i) stage_ran_[i] = false;
+    for (int i = STAGE_LOWER; i <= STAGE_BIAS; ++i) { stage_ran_[i] = false; if (profile_) stage_kernel_[i].clear(); }
     LogicalCubeType *input_d_cube = p_input_layer->p_data_cube;
     LogicalCubeType *output_d_cube = p_output_layer->p_data_cube;
     LogicalCubeType lowered_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
@@ -256,7 +259,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   // weight-gradient GEMM against the lowered data kept from forward()
   void backward() override {
     report_backward_updateweight_history.reset();
-    for (int i = STAGE_BW_BIAS; i < STAGE_COUNT; ++i) stage_ran_[i] = false;
+    for (int i = STAGE_BW_BIAS; i < STAGE_COUNT; ++i) { stage_ran_[i] = false; if (profile_) stage_kernel_[i].clear(); }
     LogicalCubeType *output_g_cube = p_output_layer->p_gradient_cube;
     LogicalCubeType *input_g_cube = p_input_layer->p_gradient_cube;
     LogicalCubeType lowered_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
@@ -411,7 +414,9 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     if (!profile_) return;
     cct_hip_timer_stop(timers_[s]);
     stage_ran_[s] = true;
+    stage_kernel_[s] = cct_hip_last_kernel();
   }
+  std::string stage_kernel_[STAGE_COUNT];
 };
 
 }  // namespace cct

@@ -201,6 +201,10 @@ class HIPDriver {
     }
     if (!small.empty()) ok(cct_hip_sgd_update_batch(small.data(), (int)small.size()), "sgd_update_batch");
   }
+  // DeviceDriver.h:262-264: X -= Y
+  void smath_apply_grad(DeviceMemoryPointer *X, DeviceMemoryPointer *Y) { math_saxpy(-1.0f, Y, X); }
+  // CPUDriver forwards this to openblas_set_num_threads (DeviceDriver_CPU.cpp:535-545); a device
+  // GEMM has no host thread count, so the call is accepted and ignored
   void set_num_threads(const int) {}
   void sgemm(const enum CBLAS_ORDER order, CBLAS_TRANSPOSE TA, CBLAS_TRANSPOSE TB, int M, int N, int K,
              float alpha, float *pA, int LDA, float *pB, int LDB, float beta, float *pC, int LDC) {
@@ -263,34 +267,20 @@ class HIPDriver {
   void rand_uint_initialize(unsigned int *buf, const int n) {
     ok(cct_hip_rand_uint_initialize(buf, n), "rand_uint_initialize");
   }
-  // Random fillers draw on the host from std::mt19937 with the same distributions and call
-  // order as CPUDriver (src/sched/DeviceDriver_CPU.cpp:661-699), then copy to the device.
+  // Random fillers: host draws from std::mt19937 with the same distributions and call order as
+  // CPUDriver (src/sched/DeviceDriver_CPU.cpp:661-699), copied to the device by the library.
   void sinitialize_xavier(DeviceMemoryPointer *arr, const size_t n_batch, const int random_seed = -1) {
-    const size_t n = arr->size_in_byte / sizeof(float);
-    const size_t fan_in = n / n_batch;
-    const float scale = std::sqrt(3.0 / fan_in);
-    std::mt19937 gen(seed_or_random(random_seed));
-    std::uniform_real_distribution<float> uni(-scale, scale);
-    std::vector<float> tmp(n);
-    for (size_t i = 0; i < n; ++i) tmp[i] = uni(gen);
-    ok(cct_hip_memcpy(arr->ptr, tmp.data(), arr->size_in_byte, 0), "sinitialize_xavier");
+    ok(cct_hip_fill_xavier((float *)arr->ptr, arr->size_in_byte / sizeof(float), n_batch, random_seed),
+       "sinitialize_xavier");
   }
   void sbernoulli_initialize(DeviceMemoryPointer *arr, const float p, const int random_seed = -1) {
-    const size_t n = arr->size_in_byte / sizeof(float);
-    std::mt19937 gen(seed_or_random(random_seed));
-    std::bernoulli_distribution bern(p);
-    std::vector<float> tmp(n);
-    for (size_t i = 0; i < n; ++i) tmp[i] = bern(gen);
-    ok(cct_hip_memcpy(arr->ptr, tmp.data(), arr->size_in_byte, 0), "sbernoulli_initialize");
+    ok(cct_hip_fill_bernoulli((float *)arr->ptr, arr->size_in_byte / sizeof(float), p, random_seed),
+       "sbernoulli_initialize");
   }
   void sgaussian_initialize(DeviceMemoryPointer *arr, const float mean, const float std_dev,
                             const int random_seed = -1) {
-    const size_t n = arr->size_in_byte / sizeof(float);
-    std::mt19937 gen(seed_or_random(random_seed));
-    std::normal_distribution<float> gaussian(mean, std_dev);
-    std::vector<float> tmp(n);
-    for (size_t i = 0; i < n; ++i) tmp[i] = gaussian(gen);
-    ok(cct_hip_memcpy(arr->ptr, tmp.data(), arr->size_in_byte, 0), "sgaussian_initialize");
+    ok(cct_hip_fill_gaussian((float *)arr->ptr, arr->size_in_byte / sizeof(float), mean, std_dev, random_seed),
+       "sgaussian_initialize");
   }
   void sconstant_initialize(DeviceMemoryPointer *arr, const float value) {
     ok(cct_hip_sconstant_initialize((float *)arr->ptr, arr->size_in_byte / sizeof(float), value),
@@ -305,11 +295,6 @@ class HIPDriver {
 
  private:
   int device_id_ = 0;
-  static unsigned seed_or_random(int random_seed) {
-    if (random_seed != -1) return (unsigned)random_seed;
-    std::random_device rd;
-    return rd();
-  }
   static void ok(int rc, const char *what) {
     if (rc != 0) {
       std::fprintf(stderr, "HIPDriver::%s failed (%d): %s\n", what, rc, cct_hip_last_error());

@@ -292,18 +292,23 @@ static int launch_lift(float *dst, const float *src, const cct_inverse_lower_cub
   const uint32_t grid = P.nblocks + P.nbias;
   if (grid == 0) return 0;
   hipStream_t st = ctx().stream;
-  if (P.k == 5 && P.s == 1)
+  if (P.k == 5 && P.s == 1) {
     hipLaunchKernelGGL((lift_kernel<5, 1>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
-  else if (P.k == 3 && P.s == 1)
+    note_kernel("lift_kernel<5,1> bias_blocks=%u", P.nbias);
+  } else if (P.k == 3 && P.s == 1) {
     hipLaunchKernelGGL((lift_kernel<3, 1>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
-  else if (P.k == 11 && P.s == 4) {
+    note_kernel("lift_kernel<3,1> bias_blocks=%u", P.nbias);
+  } else if (P.k == 11 && P.s == 4) {
     const uint32_t per_row = (uint32_t)((P.iC + 3) / 4);
     const size_t nruns = (size_t)P.iB * P.iD * P.iR * per_row;
     const uint32_t blocks = (uint32_t)((nruns + LIFT_THREADS - 1) / LIFT_THREADS);
     hipLaunchKernelGGL((lift_strided_kernel<11, 4>), dim3(blocks + P.nbias), dim3(LIFT_THREADS), 0, st, dst, src, P,
                        (uint32_t)nruns, make_fastdiv(per_row));
-  } else
+    note_kernel("lift_strided_kernel<11,4> bias_blocks=%u", P.nbias);
+  } else {
     hipLaunchKernelGGL((lift_kernel<0, 0>), dim3(grid), dim3(LIFT_THREADS), 0, st, dst, src, P);
+    note_kernel("lift_kernel<0,0> bias_blocks=%u", P.nbias);
+  }
   return check_counter_launch(P);
 }
 

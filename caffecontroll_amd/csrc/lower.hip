@@ -229,5 +229,6 @@ extern "C" int cct_hip_lower_cube(float *dst, const float *src, const cct_pmap_h
   if (int rc = grant_dynamic_lds((const void *)lower_kernel, lds_bytes, grant)) return rc;
   hipLaunchKernelGGL(lower_kernel, dim3(P.nblocks), dim3(threads), lds_bytes, st, dst, src, P);
   CCT_LAUNCH_CHECK();
+  note_kernel("lower_kernel threads=%d", threads);
   return 0;
 }

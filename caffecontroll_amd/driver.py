@@ -182,6 +182,15 @@ class HIPDriver:
     def sconstant_initialize(self, arr, n, value):
         check(self.lib.cct_hip_sconstant_initialize(_p(arr), n, value), "sconstant_initialize")
 
+    def fill_xavier(self, arr, n, n_batch, seed):
+        check(self.lib.cct_hip_fill_xavier(_p(arr), n, n_batch, seed), "fill_xavier")
+
+    def fill_bernoulli(self, arr, n, p, seed):
+        check(self.lib.cct_hip_fill_bernoulli(_p(arr), n, p, seed), "fill_bernoulli")
+
+    def fill_gaussian(self, arr, n, mean, std, seed):
+        check(self.lib.cct_hip_fill_gaussian(_p(arr), n, mean, std, seed), "fill_gaussian")
+
     def init_rng(self, seed):
         check(self.lib.cct_hip_init_rng(seed), "init_rng")
 

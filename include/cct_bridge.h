@@ -73,6 +73,10 @@ int cct_conv_bridge_forward(cct_conv_bridge *h);
  * with_update == 0: ConvolutionBridge::backward only. */
 int cct_conv_bridge_backward(cct_conv_bridge *h, int with_update);
 int cct_conv_bridge_stage_ms(cct_conv_bridge *h, float ms[CCT_CONV_STAGE_COUNT]);
+/* The kernel instance that ran as the stage's product kernel (cct_hip_last_kernel() taken when the
+ * stage ended; needs profile != 0), "" for a stage that has not run.  Valid until the next
+ * forward/backward of the bridge. */
+const char *cct_conv_bridge_stage_kernel(cct_conv_bridge *h, int stage);
 
 /* ---- a chain of layers (LeNet / CaffeNet style) --------------------------------------------
  * Stands for DeepNet::construct_network + run_forward_pass / run_backward_pass

@@ -109,6 +109,11 @@ int cct_hip_set_tuning(const char *name, int value);
 /* DeviceDriver::device_sync, src/sched/DeviceDriver.h:267. */
 int cct_hip_device_sync(void);
 const char *cct_hip_last_error(void);
+/* The kernel instance the library chose for the most recent lowering, lifting, GEMM or direct
+ * convolution call: kernel name with its template arguments as a kernel trace prints them, then
+ * launch-time choices (e.g. "gemm_kernel<Tile<256,128,16,2,2>,true,false> splits=26").  For
+ * harnesses that label measurements with what actually ran.  No counterpart in the reference. */
+const char *cct_hip_last_kernel(void);
 /* Number of compute units of the selected device (0 before init). */
 int cct_hip_compute_units(void);
 
@@ -249,6 +254,20 @@ typedef struct {
 int cct_hip_sgd_update_batch(const cct_sgd_job *jobs, int count);
 /* DeviceDriver::sconstant_initialize (src/sched/DeviceDriver.h:258-260). */
 int cct_hip_sconstant_initialize(float *arr, size_t n, float value);
+/* DeviceDriver::sinitialize_xavier / sbernoulli_initialize / sgaussian_initialize
+ * (src/sched/DeviceDriver.h:242-256; CPUDriver src/sched/DeviceDriver_CPU.cpp:661-699): n floats
+ * at the device pointer arr.  Drawn on the host the way CPUDriver draws them -- std::mt19937 seeded
+ * with random_seed (std::random_device if -1), then one draw per element in index order from
+ * uniform_real_distribution<float>(-s, s) with s = sqrt(3 / (n / n_batch)),
+ * bernoulli_distribution(p), normal_distribution<float>(mean, std_dev) -- and copied to the device
+ * (synchronous).  The cct_filler_draw_* forms write the same values to a HOST array and touch no
+ * device. */
+int cct_hip_fill_xavier(float *arr, size_t n, size_t n_batch, int random_seed);
+int cct_hip_fill_bernoulli(float *arr, size_t n, float p, int random_seed);
+int cct_hip_fill_gaussian(float *arr, size_t n, float mean, float std_dev, int random_seed);
+int cct_filler_draw_xavier(float *host, size_t n, size_t n_batch, int random_seed);
+int cct_filler_draw_bernoulli(float *host, size_t n, float p, int random_seed);
+int cct_filler_draw_gaussian(float *host, size_t n, float mean, float std_dev, int random_seed);
 /* DeviceDriver::rand_uint_initialize (src/sched/DeviceDriver.h:250-252) after init_rng(seed):
  * counter-based generator, word i of call c depends only on (seed, c, i). */
 int cct_hip_init_rng(int random_seed);

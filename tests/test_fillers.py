@@ -1,0 +1,100 @@
+"""The random fillers (DeviceDriver::sinitialize_xavier / sbernoulli_initialize /
+sgaussian_initialize; CPUDriver draws them from std::mt19937 and the standard library's
+distribution objects, src/sched/DeviceDriver_CPU.cpp:661-699).
+
+What fixes the values: the C++ standard fixes mt19937 (the 10000th output of a default-seeded
+engine is 4123659995); the distributions are those of GNU libstdc++, which the reference is built
+with: generate_canonical takes one 32-bit draw per float and two per double, uniform_real is
+a + (b - a) * canonical, bernoulli is canonical<double> < p, normal is Marsaglia's polar method
+that returns y * mult first and keeps x * mult for the next call.  The test restates those
+algorithms with numpy on the raw engine stream and demands bit equality, so a changed call order,
+a double where the reference has a float, or a different engine would show."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from caffecontroll_amd import _lib
+
+
+def raw_stream(seed, n):
+    bg = np.random.MT19937()
+    bg._legacy_seeding(seed)          # init_genrand(seed): the seeding of std::mt19937(seed)
+    return bg.random_raw(n).astype(np.uint64)
+
+
+def canonical_float(u32):
+    """std::generate_canonical<float, 24> on a 32-bit engine: one draw, float(u) / 2^32, clamped below 1."""
+    r = u32.astype(np.float32) / np.float32(4294967296.0)
+    return np.where(r >= 1, np.nextafter(np.float32(1), np.float32(0)), r).astype(np.float32)
+
+
+def draw(name, n, *args):
+    lib = _lib.load()
+    out = np.empty(n, np.float32)
+    _lib.check(getattr(lib, "cct_filler_draw_" + name)(out.ctypes.data_as(C.c_void_p), n, *args), name)
+    return out
+
+
+def test_engine_is_the_standard_mt19937():
+    assert int(raw_stream(5489, 10000)[-1]) == 4123659995
+
+
+@pytest.mark.parametrize("seed, n, n_batch", [(1, 500, 20), (77, 2400, 96)])
+def test_xavier(seed, n, n_batch):
+    got = draw("xavier", n, n_batch, seed)
+    scale = np.float32(np.sqrt(3.0 / (n // n_batch)))
+    a, b = -scale, scale
+    want = canonical_float(raw_stream(seed, n)) * np.float32(b - a) + a
+    np.testing.assert_array_equal(got, want.astype(np.float32))
+    assert np.abs(got).max() <= scale and got.std() == pytest.approx(scale / np.sqrt(3), rel=0.1)
+
+
+@pytest.mark.parametrize("p", [0.5, 0.1])
+def test_bernoulli(p):
+    n, seed = 400, 9
+    got = draw("bernoulli", n, p, seed)
+    u = raw_stream(seed, 2 * n)
+    # generate_canonical<double, 53>: two draws, the first is the low word
+    lo, hi = u[0::2].astype(np.float64), u[1::2].astype(np.float64)
+    canon = (lo + hi * 4294967296.0) / 18446744073709551616.0
+    want = (canon < np.float64(np.float32(p))).astype(np.float32)
+    np.testing.assert_array_equal(got, want)
+    assert set(np.unique(got)) <= {0.0, 1.0} and abs(got.mean() - p) < 0.08
+
+
+@pytest.mark.parametrize("mean, std", [(0.0, 0.01), (1.5, 2.0)])
+def test_gaussian(mean, std):
+    n, seed = 301, 4   # odd n: the last value is the first of a pair whose second is never used
+    got = draw("gaussian", n, mean, std, seed)
+    libm = C.CDLL("libm.so.6")
+    libm.logf.restype, libm.logf.argtypes = C.c_float, [C.c_float]
+    libm.sqrtf.restype, libm.sqrtf.argtypes = C.c_float, [C.c_float]
+    f32 = np.float32
+    u = canonical_float(raw_stream(seed, 4 * n))
+    want, pos, saved = [], 0, None
+    while len(want) < n:
+        if saved is not None:
+            ret, saved = saved, None
+        else:
+            while True:
+                x = f32(np.float64(f32(2.0) * u[pos]) - 1.0)
+                y = f32(np.float64(f32(2.0) * u[pos + 1]) - 1.0)
+                pos += 2
+                r2 = f32(f32(x * x) + f32(y * y))
+                if not (r2 > 1.0 or r2 == 0.0):
+                    break
+            mult = f32(libm.sqrtf(f32(f32(f32(-2.0) * f32(libm.logf(r2))) / r2)))
+            saved, ret = f32(x * mult), f32(y * mult)
+        want.append(f32(f32(ret * f32(std)) + f32(mean)))
+    np.testing.assert_array_equal(got, np.array(want, np.float32))
+    assert got.mean() == pytest.approx(mean, abs=4 * std / np.sqrt(n)) and got.std() == pytest.approx(std, rel=0.15)
+
+
+def test_rejected_arguments():
+    lib = _lib.load()
+    buf = np.empty(4, np.float32)
+    p = buf.ctypes.data_as(C.c_void_p)
+    assert lib.cct_filler_draw_xavier(p, 4, 0, 1) != 0
+    assert lib.cct_filler_draw_bernoulli(p, 4, 1.5, 1) != 0
+    assert lib.cct_filler_draw_gaussian(p, 4, 0.0, 0.0, 1) != 0

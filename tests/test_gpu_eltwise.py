@@ -243,3 +243,18 @@ def test_fill_and_memory():
     np.testing.assert_array_equal(out, src)
     drv.free(p)
     assert C.sizeof(C.c_void_p) == 8
+
+
+def test_fillers_on_the_device_equal_the_host_draws():
+    """cct_hip_fill_* = the host draw (pinned in tests/test_fillers.py) copied to the device."""
+    import ctypes as C
+    from caffecontroll_amd import _lib
+    drv = driver()
+    lib = _lib.load()
+    n = 1200
+    want = np.empty(n, np.float32)
+    for name, args in (("xavier", (48, 3)), ("bernoulli", (0.3, 5)), ("gaussian", (0.5, 0.01, 7))):
+        t = empty((n,))
+        getattr(drv, "fill_" + name)(t, n, *args)
+        _lib.check(getattr(lib, "cct_filler_draw_" + name)(want.ctypes.data_as(C.c_void_p), n, *args), name)
+        np.testing.assert_array_equal(host(t), want)
