@@ -112,6 +112,7 @@ PROTOTYPES = {
     "cct_hip_maxpool_forward": [_P, _P, C.POINTER(PoolArgs)],
     "cct_hip_maxpool_backward": [_P, _P, C.POINTER(PoolArgs)],
     "cct_hip_maxpool_backward_relu": [_P, _P, C.POINTER(PoolArgs), _P],
+    "cct_hip_maxpool_backward_relu_pooled": [_P, _P, C.POINTER(PoolArgs), _P],
     "cct_hip_lrn_forward": [_P, _P, C.POINTER(LrnForwardArgs), C.POINTER(LrnForwardNormalizeArgs)],
     "cct_hip_lrn_backward": [_P, _P, C.POINTER(LrnBackwardArgs)],
     "cct_hip_dropout_forward_train": [_P, _P, _P, _F, _U, _Z],

@@ -313,6 +313,44 @@ __device__ __forceinline__ void pool_stage(T *dst, const T *__restrict__ src, ui
   if (threadIdx.x < (n & 3u)) dst[4 * n4 + threadIdx.x] = src[4 * n4 + threadIdx.x];
 }
 
+// dst[i] (LDS) = y[i] > 0 ? g[i] : 0 for i in [0, n): the output gradient of a pooling layer with
+// the windows whose maximum is not positive switched off (both global arrays 4-byte aligned)
+template <int UNR>
+__device__ __forceinline__ void pool_stage_masked(float *dst, const float *__restrict__ g,
+                                                  const float *__restrict__ y, uint32_t n) {
+  const uint32_t n4 = n >> 2;
+  for (uint32_t base = 0; base < n4; base += TPB * UNR) {
+    pool_f4u gv[UNR], yv[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const uint32_t q = base + u * TPB + threadIdx.x;
+      if (q < n4) {
+        gv[u] = *reinterpret_cast<const pool_f4u *>(g + 4 * q);
+        yv[u] = *reinterpret_cast<const pool_f4u *>(y + 4 * q);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const uint32_t q = base + u * TPB + threadIdx.x;
+      if (q < n4) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dst[4 * q + e] = yv[u][e] > 0.0f ? gv[u][e] : 0.0f;
+      }
+    }
+  }
+  if (threadIdx.x < (n & 3u)) {
+    const uint32_t i = 4 * n4 + threadIdx.x;
+    dst[i] = y[i] > 0.0f ? g[i] : 0.0f;
+  }
+}
+
+// out[i] = y[i] > 0 ? g[i] : 0 in global memory (the same switch for the kernels that do not stage)
+__global__ __launch_bounds__(TPB) void mask_positive_kernel(float *__restrict__ out, const float *__restrict__ g,
+                                                            const float *__restrict__ y, size_t n) {
+  const size_t stride = (size_t)gridDim.x * TPB;
+  for (size_t i = (size_t)blockIdx.x * TPB + threadIdx.x; i < n; i += stride) out[i] = y[i] > 0.0f ? g[i] : 0.0f;
+}
+
 __global__ __launch_bounds__(TPB) void maxpool_fwd_plane_kernel(float *__restrict__ out, int *__restrict__ idx,
                                                                 const float *__restrict__ in, cct_pool_args a,
                                                                 uint32_t planes, int pp, FastDiv div_oc,
@@ -398,9 +436,13 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_plane_kernel(float *__restric
 __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict__ ig, const float *__restrict__ og,
                                                                const int *__restrict__ idx, cct_pool_args a,
                                                                uint32_t planes, int pp, int lpr_shift, FastDiv div_ir,
-                                                               FastDiv div_s, const float *__restrict__ relu_data) {
+                                                               FastDiv div_s, const float *__restrict__ relu_data,
+                                                               const float *__restrict__ pooled) {
   // relu_data (optional): the pooled tensor itself when it is the output of an in-place ReLU; the
   // gradient is then stored already masked with (relu_data > 0), which is that ReLU's backward.
+  // pooled (optional, instead of relu_data): the pooling OUTPUT.  A gradient lands only on a
+  // window's arg-max, whose activation is the window's maximum, so masking every window's gradient
+  // with (pooled > 0) while it is staged gives the same sums and reads a tensor a quarter the size.
   // LDS sized by the launch (2 * pp * oplane words): small planes leave room for more workgroups
   // per compute unit, whose load and store phases then overlap
   extern __shared__ float pool_lds[];
@@ -409,7 +451,8 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict
   const uint32_t iplane = (uint32_t)(a.iR * a.iC), oplane = (uint32_t)(a.oR * a.oC);
   float *tog = pool_lds;
   int *tidx = reinterpret_cast<int *>(pool_lds + (size_t)pp * oplane);
-  pool_stage<pool_f4u, float, 4>(tog, og + (size_t)p0 * oplane, np * oplane);
+  if (pooled) pool_stage_masked<4>(tog, og + (size_t)p0 * oplane, pooled + (size_t)p0 * oplane, np * oplane);
+  else pool_stage<pool_f4u, float, 4>(tog, og + (size_t)p0 * oplane, np * oplane);
   pool_stage<pool_i4u, int, 4>(tidx, idx + (size_t)p0 * oplane, np * oplane);
   __syncthreads();
   const int k = a.kernel_size;
@@ -492,6 +535,33 @@ static int pool_planes_per_block(size_t plane_words, size_t work_words, size_t p
 }
 
 // ---- LRN (across channels) -----------------------------------------------------------------------
+// scale^beta for the normalisation term scale = 1 + alpha/size * sum of squares.  The library
+// routine powf costs more instructions than the rest of either kernel; two cheaper forms are used
+// where they apply (chosen on the host, `mode` is uniform over a launch):
+//   LRN_POW_34     beta == 0.75 (AlexNet / CaffeNet): sqrt(s) * sqrt(sqrt(s)), two correctly rounded
+//                  square roots and one product;
+//   LRN_POW_EXP2   any beta with alpha >= 0 (scale >= 1): exp2(beta * log2(s)) on the hardware
+//                  transcendental units (1 ulp each; the exponent is small, so the error of the
+//                  result stays within a few ulp);
+//   LRN_POW_LIBM   everything else: powf.
+// Reciprocals use v_rcp_f32 (1 ulp).  All of it is well inside the 1e-5 bar against the oracle's
+// exact powf and double-precision reciprocals.
+enum { LRN_POW_LIBM = 0, LRN_POW_34 = 1, LRN_POW_EXP2 = 2 };
+__device__ __forceinline__ float lrn_pow(float s, float beta, int mode) {
+  if (mode == LRN_POW_34) {
+    const float r = __builtin_sqrtf(s);
+    return r * __builtin_sqrtf(r);
+  }
+  if (mode == LRN_POW_EXP2) return __builtin_amdgcn_exp2f(beta * __builtin_amdgcn_logf(s));
+  return powf(s, beta);
+}
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+static int lrn_pow_mode(float alpha_over_size, float beta) {
+  if (!(alpha_over_size >= 0.0f)) return LRN_POW_LIBM;  // scale could reach zero or below: keep powf's special cases
+  if (beta == 0.75f) return LRN_POW_34;
+  return LRN_POW_EXP2;
+}
+
 // forward: one lane per element sums the squares of its window [ch-w, ch+w] (clipped to the depth)
 // in ascending channel order, then scale = 1 + alpha/size * sum and out = in / scale^beta; denoms
 // keeps scale.  _f_lrn_forward carries a running window sum along the depth (src/kernels/lrn.hxx:
@@ -499,7 +569,7 @@ static int pool_planes_per_block(size_t plane_words, size_t work_words, size_t p
 __global__ __launch_bounds__(TPB) void lrn_fwd_kernel(float *__restrict__ out, float *__restrict__ denoms,
                                                       const float *__restrict__ in, int rc, int D,
                                                       uint32_t total, int w, float aos, float beta,
-                                                      FastDiv div_rc, FastDiv div_d) {
+                                                      int mode, FastDiv div_rc, FastDiv div_d) {
   const uint32_t e = blockIdx.x * TPB + threadIdx.x;
   if (e >= total) return;
   // e = (ib*D + ch)*rc + q
@@ -516,7 +586,7 @@ __global__ __launch_bounds__(TPB) void lrn_fwd_kernel(float *__restrict__ out, f
   }
   const float scale = aos * sum + 1.0f;
   denoms[e] = scale;
-  out[e] = xv / powf(scale, beta);
+  out[e] = mode == LRN_POW_LIBM ? xv / powf(scale, beta) : xv * fast_rcp(lrn_pow(scale, beta, mode));
 }
 
 // backward as a gather over the window: in_grad[ch] = sum over od in [ch-w, ch+w] (ascending, the
@@ -524,7 +594,7 @@ __global__ __launch_bounds__(TPB) void lrn_fwd_kernel(float *__restrict__ out, f
 __global__ __launch_bounds__(TPB) void lrn_bwd_kernel(float *__restrict__ ig, const float *__restrict__ og,
                                                       const float *__restrict__ x, const float *__restrict__ den,
                                                       int rc, int D, uint32_t total, int w, float aos,
-                                                      float beta, FastDiv div_rc, FastDiv div_d) {
+                                                      float beta, int mode, FastDiv div_rc, FastDiv div_d) {
   const uint32_t e = blockIdx.x * TPB + threadIdx.x;
   if (e >= total) return;
   // e = (ib*D + ch)*rc + q
@@ -538,12 +608,19 @@ __global__ __launch_bounds__(TPB) void lrn_bwd_kernel(float *__restrict__ ig, co
   for (int od = max(0, ch - w); od <= min(D - 1, ch + w); ++od) {
     const size_t o = base + (size_t)od * rc;
     const float dne = den[o];
-    const float denom = powf(dne, beta);
-    const float denom_n1 = (float)(1.0 / (double)(denom * dne));
+    const float denom = lrn_pow(dne, beta, mode);
+    float denom_n1, inv_denom;
+    if (mode == LRN_POW_LIBM) {
+      denom_n1 = (float)(1.0 / (double)(denom * dne));
+      inv_denom = 0.0f;  // the centre term below takes the double-precision route
+    } else {
+      denom_n1 = fast_rcp(denom * dne);
+      inv_denom = denom_n1 * dne;
+    }
     const float wd = x[o];
     const float g2 = beta * denom_n1 * aos * 2 * wd;
     float gv;
-    if (od == ch) gv = (float)(1.0 / (double)denom - (double)(g2 * xv));
+    if (od == ch) gv = mode == LRN_POW_LIBM ? (float)(1.0 / (double)denom - (double)(g2 * xv)) : inv_denom - g2 * xv;
     else gv = -g2 * xv;
     acc += gv * og[o];
   }
@@ -555,7 +632,7 @@ __global__ __launch_bounds__(TPB) void lrn_bwd_kernel(float *__restrict__ ig, co
 // them in ascending channel order -- the sums lrn_fwd_kernel forms (terms outside the depth enter
 // as +0, which leaves a sum of squares unchanged), a third of its loads and an eighth of its index
 // arithmetic.
-template <int WN, int CH>
+template <int WN, int CH, int MODE>
 __global__ __launch_bounds__(TPB) void lrn_fwd_run_kernel(float *__restrict__ out, float *__restrict__ denoms,
                                                           const float *__restrict__ in, int rc, int D,
                                                           uint32_t total, int nruns, float aos, float beta,
@@ -587,7 +664,7 @@ __global__ __launch_bounds__(TPB) void lrn_fwd_run_kernel(float *__restrict__ ou
     const float scale = aos * sum + 1.0f;
     const size_t o = base + (size_t)ch * rc;
     denoms[o] = scale;
-    out[o] = xw[c + WN] / powf(scale, beta);
+    out[o] = MODE == LRN_POW_LIBM ? xw[c + WN] / powf(scale, beta) : xw[c + WN] * fast_rcp(lrn_pow(scale, beta, MODE));
   }
 }
 
@@ -595,13 +672,16 @@ __global__ __launch_bounds__(TPB) void lrn_fwd_run_kernel(float *__restrict__ ou
 // the window (scale^beta, the factor g2, x and out_grad) are computed once per lane and reused by
 // the up to 2*WN+1 output channels that touch them, instead of once per (channel, window slot).
 // Every product and sum is the one lrn_bwd_kernel forms, in the same order: identical results.
-template <int WN, int CH>
+template <int WN, int CH, int MODE>
 __global__ __launch_bounds__(TPB) void lrn_bwd_run_kernel(float *__restrict__ ig, const float *__restrict__ og,
                                                           const float *__restrict__ x,
                                                           const float *__restrict__ den, int rc, int D,
                                                           uint32_t total, int nruns, float aos, float beta,
                                                           FastDiv div_rc, FastDiv div_runs) {
-  const uint32_t e = blockIdx.x * TPB + threadIdx.x;
+  // neighbouring runs share their halo channels (three tensors' worth here): each XCD walks a
+  // contiguous range of lanes so that the second reader of a halo finds it in its own L2 (measured:
+  // 56 -> 51 us on the CaffeNet shapes; the forward kernel, with one input tensor, loses by it)
+  const uint32_t e = xcd_remap(blockIdx.x, gridDim.x) * TPB + threadIdx.x;
   if (e >= total) return;
   // e = (ib*nruns + run)*rc + q
   const uint32_t t1 = fdiv(e, div_rc);
@@ -610,6 +690,8 @@ __global__ __launch_bounds__(TPB) void lrn_bwd_run_kernel(float *__restrict__ ig
   const int c0 = (int)(t1 - ib * nruns) * CH;
   const size_t base = (size_t)ib * D * rc + q;
   constexpr int NW = CH + 2 * WN;
+  // denom holds scale^beta (LRN_POW_LIBM: the centre term divides in double precision, as the
+  // reference's formula does) or its reciprocal (the fast modes)
   float denom[NW], g2[NW], xw[NW], ow[NW];
 #pragma unroll
   for (int i = 0; i < NW; ++i) {
@@ -618,10 +700,16 @@ __global__ __launch_bounds__(TPB) void lrn_bwd_run_kernel(float *__restrict__ ig
     if (od >= 0 && od < D) {
       const size_t o = base + (size_t)od * rc;
       const float dne = den[o];
-      const float dn = powf(dne, beta);
-      const float denom_n1 = (float)(1.0 / (double)(dn * dne));
+      const float dn = lrn_pow(dne, beta, MODE);
+      float denom_n1;
+      if (MODE == LRN_POW_LIBM) {
+        denom_n1 = (float)(1.0 / (double)(dn * dne));
+        denom[i] = dn;
+      } else {
+        denom_n1 = fast_rcp(dn * dne);
+        denom[i] = denom_n1 * dne;
+      }
       const float wd = x[o];
-      denom[i] = dn;
       g2[i] = beta * denom_n1 * aos * 2 * wd;
       xw[i] = wd;
       ow[i] = og[o];
@@ -639,7 +727,7 @@ __global__ __launch_bounds__(TPB) void lrn_bwd_run_kernel(float *__restrict__ ig
       if (od < 0 || od >= D) continue;
       const int i = c + j;
       float gv;
-      if (j == WN) gv = (float)(1.0 / (double)denom[i] - (double)(g2[i] * xv));
+      if (j == WN) gv = MODE == LRN_POW_LIBM ? (float)(1.0 / (double)denom[i] - (double)(g2[i] * xv)) : denom[i] - g2[i] * xv;
       else gv = -g2[i] * xv;
       acc += gv * ow[i];
     }
@@ -978,22 +1066,38 @@ int cct_hip_maxpool_forward(float *out, const float *in, const cct_pool_args *a)
   return 0;
 }
 
+// relu_data: mask the result with (relu_data > 0) (same shape as in_grad); pooled: mask every
+// window's gradient with (pooled > 0) (same shape as out_grad) -- at most one of the two
 static int maxpool_backward_impl(float *in_grad, const float *out_grad, const cct_pool_args *a,
-                                 const float *relu_data) {
+                                 const float *relu_data, const float *pooled = nullptr) {
   CCT_REQUIRE(in_grad && out_grad, "maxpool_backward: null argument");
   int rc = check_pool(a, "maxpool_backward");
   if (rc) return rc;
   const size_t total = (size_t)a->D * a->B * a->iR * a->iC;
   if (total == 0) return 0;
   const size_t planes = (size_t)a->D * a->B, iplane = (size_t)a->iR * a->iC, oplane = (size_t)a->oR * a->oC;
-  if (const int pp = pool_planes_per_block(2 * oplane, iplane, planes)) {
+  const int pp = pool_planes_per_block(2 * oplane, iplane, planes);
+  const bool quad = pp && a->stride >= 2 && a->kernel_size <= 2 * a->stride && a->iC <= 256;
+  if (pooled && !quad) {
+    // the other kernels do not switch windows off while they stage: a pass over the (small) output
+    // gradient does it first, into the library's workspace
+    void *ws = nullptr;
+    rc = get_workspace(planes * oplane * sizeof(float), &ws);
+    if (rc) return rc;
+    hipLaunchKernelGGL(mask_positive_kernel, dim3(grid_stride_blocks(planes * oplane)), dim3(TPB), 0, ctx().stream,
+                       (float *)ws, out_grad, pooled, planes * oplane);
+    CCT_LAUNCH_CHECK();
+    out_grad = (const float *)ws;
+    pooled = nullptr;
+  }
+  if (pp) {
     const dim3 grid((uint32_t)((planes + pp - 1) / pp));
-    if (a->stride >= 2 && a->kernel_size <= 2 * a->stride && a->iC <= 256) {
+    if (quad) {
       int lpr_shift = 0;
       while ((4 << lpr_shift) < a->iC) ++lpr_shift;
       hipLaunchKernelGGL(maxpool_bwd_quad_kernel, grid, dim3(TPB), (size_t)2 * pp * oplane * sizeof(float),
                          ctx().stream, in_grad, out_grad, a->max_index, *a, (uint32_t)planes, pp, lpr_shift,
-                         make_fastdiv(a->iR), make_fastdiv(a->stride), relu_data);
+                         make_fastdiv(a->iR), make_fastdiv(a->stride), relu_data, pooled);
       relu_data = nullptr;  // done inside the kernel
     } else if (a->kernel_size <= 2 * a->stride)
       hipLaunchKernelGGL(maxpool_bwd_plane_kernel<true>, grid, dim3(TPB), 0, ctx().stream, in_grad, out_grad,
@@ -1029,6 +1133,13 @@ int cct_hip_maxpool_backward_relu(float *in_grad, const float *out_grad, const c
   return maxpool_backward_impl(in_grad, out_grad, a, relu_data);
 }
 
+int cct_hip_maxpool_backward_relu_pooled(float *in_grad, const float *out_grad, const cct_pool_args *a,
+                                         const float *pooled) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(pooled, "maxpool_backward_relu_pooled: null pooled tensor");
+  return maxpool_backward_impl(in_grad, out_grad, a, nullptr, pooled);
+}
+
 int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args *a,
                         const cct_lrn_forward_normalize_args *a2) {
   CCT_ENSURE_INIT();
@@ -1037,19 +1148,25 @@ int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args 
   const size_t total = (size_t)a->iB * a->iD * a->iR * a->iC;
   CCT_REQUIRE(total < (1ull << 31), "lrn_forward: tensor too large");
   if (total == 0) return 0;
+  const int mode = lrn_pow_mode(a2->alpha_over_size, a2->beta);
   if (a->norm_window == 2) {
     constexpr int CH = 8;
     const int nruns = (a->iD + CH - 1) / CH, rc = a->iR * a->iC;
     const size_t lanes = (size_t)a->iB * nruns * rc;
-    hipLaunchKernelGGL((lrn_fwd_run_kernel<2, CH>), dim3(blocks_for(lanes)), dim3(TPB), 0, ctx().stream, out,
-                       (float *)a->denoms, in, rc, a->iD, (uint32_t)lanes, nruns, a2->alpha_over_size, a2->beta,
-                       make_fastdiv(rc), make_fastdiv(nruns));
+#define CCT_LRN_FWD(MODE)                                                                                      \
+  hipLaunchKernelGGL((lrn_fwd_run_kernel<2, CH, MODE>), dim3(blocks_for(lanes)), dim3(TPB), 0, ctx().stream, out, \
+                     (float *)a->denoms, in, rc, a->iD, (uint32_t)lanes, nruns, a2->alpha_over_size, a2->beta,  \
+                     make_fastdiv(rc), make_fastdiv(nruns))
+    if (mode == LRN_POW_34) CCT_LRN_FWD(LRN_POW_34);
+    else if (mode == LRN_POW_EXP2) CCT_LRN_FWD(LRN_POW_EXP2);
+    else CCT_LRN_FWD(LRN_POW_LIBM);
+#undef CCT_LRN_FWD
     CCT_LAUNCH_CHECK();
     return 0;
   }
   hipLaunchKernelGGL(lrn_fwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, out,
                      (float *)a->denoms, in, a->iR * a->iC, a->iD, (uint32_t)total, a->norm_window,
-                     a2->alpha_over_size, a2->beta, make_fastdiv(a->iR * a->iC), make_fastdiv(a->iD));
+                     a2->alpha_over_size, a2->beta, mode, make_fastdiv(a->iR * a->iC), make_fastdiv(a->iD));
   CCT_LAUNCH_CHECK();
   return 0;
 }
@@ -1061,20 +1178,26 @@ int cct_hip_lrn_backward(float *in_grad, const float *out_grad, const cct_lrn_ba
   const size_t total = (size_t)a->oB * a->oD * a->oR * a->oC;
   CCT_REQUIRE(total < (1ull << 31), "lrn_backward: tensor too large");
   if (total == 0) return 0;
+  const int mode = lrn_pow_mode(a->alpha_over_size, a->beta);
   if (a->norm_window == 2) {
     constexpr int CH = 8;
     const int nruns = (a->oD + CH - 1) / CH;
     const size_t lanes = (size_t)a->oB * nruns * a->oR * a->oC;
-    hipLaunchKernelGGL((lrn_bwd_run_kernel<2, CH>), dim3(blocks_for(lanes)), dim3(TPB), 0, ctx().stream, in_grad,
-                       out_grad, (const float *)a->input_data, (const float *)a->denoms, a->oR * a->oC, a->oD,
-                       (uint32_t)lanes, nruns, a->alpha_over_size, a->beta, make_fastdiv(a->oR * a->oC),
-                       make_fastdiv(nruns));
+#define CCT_LRN_BWD(MODE)                                                                                       \
+  hipLaunchKernelGGL((lrn_bwd_run_kernel<2, CH, MODE>), dim3(blocks_for(lanes)), dim3(TPB), 0, ctx().stream,    \
+                     in_grad, out_grad, (const float *)a->input_data, (const float *)a->denoms, a->oR * a->oC,  \
+                     a->oD, (uint32_t)lanes, nruns, a->alpha_over_size, a->beta, make_fastdiv(a->oR * a->oC),   \
+                     make_fastdiv(nruns))
+    if (mode == LRN_POW_34) CCT_LRN_BWD(LRN_POW_34);
+    else if (mode == LRN_POW_EXP2) CCT_LRN_BWD(LRN_POW_EXP2);
+    else CCT_LRN_BWD(LRN_POW_LIBM);
+#undef CCT_LRN_BWD
     CCT_LAUNCH_CHECK();
     return 0;
   }
   hipLaunchKernelGGL(lrn_bwd_kernel, dim3(blocks_for(total)), dim3(TPB), 0, ctx().stream, in_grad, out_grad,
                      (const float *)a->input_data, (const float *)a->denoms, a->oR * a->oC, a->oD,
-                     (uint32_t)total, a->norm_window, a->alpha_over_size, a->beta,
+                     (uint32_t)total, a->norm_window, a->alpha_over_size, a->beta, mode,
                      make_fastdiv(a->oR * a->oC), make_fastdiv(a->oD));
   CCT_LAUNCH_CHECK();
   return 0;

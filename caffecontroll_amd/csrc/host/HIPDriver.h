@@ -124,6 +124,13 @@ class HIPDriver {
        "maxpool_backward_relu");
   }
 
+  // the same from the pooling layer's output tensor (a quarter of the bytes): see cct_hip.h
+  void maxpool_backward_relu_pooled(DeviceMemoryPointer *dst, DeviceMemoryPointer *src,
+                                    const _pool_backward_arg_helper args, const float *pooled) {
+    ok(cct_hip_maxpool_backward_relu_pooled((float *)src->ptr, (const float *)dst->ptr, &args, pooled),
+       "maxpool_backward_relu_pooled");
+  }
+
   // ---- the parallel_map pairs of the reference, by name ----
   void relu_forward(DeviceMemoryPointer *dst, DeviceMemoryPointer *src) {
     ok(cct_hip_relu_forward((float *)dst->ptr, (const float *)src->ptr, src->size_in_byte / sizeof(float)),

@@ -266,6 +266,14 @@ class Network {
       cur = nd.out;
       nodes_.push_back(nd);
     }
+    // a pooling layer that folds a ReLU backward may take its mask from its own output, unless the
+    // layer after it rewrites that tensor in place (dropout does; a ReLU keeps the signs)
+    for (size_t i = 0; i < nodes_.size(); ++i) {
+      if (nodes_[i].spec.type != CCT_LAYER_MAXPOOL) continue;
+      const bool rewritten = i + 1 < nodes_.size() && nodes_[i + 1].out == nodes_[i].out &&
+                             nodes_[i + 1].spec.type != CCT_LAYER_RELU;
+      static_cast<MaxPoolingBridge<float, HIPDriver> *>(nodes_[i].bridges[0])->output_keeps_signs = !rewritten;
+    }
   }
 
   ~Network() {

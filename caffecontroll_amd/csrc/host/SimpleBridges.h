@@ -87,7 +87,9 @@ class MaxPoolingBridge : public AbstractBridge<DataType, DriverClass> {
   void backward() override {
     DeviceMemoryPointer input = p_input_layer->p_gradient_cube->get_device_pointer(p_driver);
     DeviceMemoryPointer output = p_output_layer->p_gradient_cube->get_device_pointer(p_driver);
-    if (input_is_relu_output)
+    if (input_is_relu_output && output_keeps_signs)
+      p_driver->maxpool_backward_relu_pooled(&output, &input, args(), p_output_layer->p_data_cube->get_p_data());
+    else if (input_is_relu_output)
       p_driver->maxpool_backward_relu(&output, &input, args(), p_input_layer->p_data_cube->get_p_data());
     else
       p_driver->maxpool_backward(&output, &input, args());
@@ -95,6 +97,10 @@ class MaxPoolingBridge : public AbstractBridge<DataType, DriverClass> {
   // the input layer is the output of an in-place ReLU whose backward this bridge performs while it
   // stores the gradient (the ReLU bridge then skips its own)
   bool input_is_relu_output = false;
+  // the output cube still holds the pooled values (or at least their signs) when backward() runs:
+  // true unless a layer that follows rewrites it in place with something other than a ReLU.  The
+  // mask of the folded ReLU backward is then taken from the (four times smaller) output tensor.
+  bool output_keeps_signs = false;
 
  private:
   LogicalCube<int> *max_index;

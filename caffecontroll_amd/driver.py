@@ -230,9 +230,14 @@ class HIPDriver:
     def maxpool_forward(self, out, inp, args):
         check(self.lib.cct_hip_maxpool_forward(_p(out), _p(inp), C.byref(args)), "maxpool_forward")
 
-    def maxpool_backward(self, in_grad, out_grad, args, relu_data=None):
+    def maxpool_backward(self, in_grad, out_grad, args, relu_data=None, pooled=None):
         """relu_data: the pooled tensor when it is the output of an in-place ReLU; the gradient then
-        comes out already masked with (relu_data > 0)."""
+        comes out already masked with (relu_data > 0).  pooled: the same result from the pooling
+        layer's output tensor instead (cct_hip_maxpool_backward_relu_pooled)."""
+        if pooled is not None:
+            check(self.lib.cct_hip_maxpool_backward_relu_pooled(_p(in_grad), _p(out_grad), C.byref(args), _p(pooled)),
+                  "maxpool_backward_relu_pooled")
+            return
         if relu_data is not None:
             check(self.lib.cct_hip_maxpool_backward_relu(_p(in_grad), _p(out_grad), C.byref(args), _p(relu_data)),
                   "maxpool_backward_relu")

@@ -308,6 +308,14 @@ int cct_hip_maxpool_backward(float *in_grad, const float *out_grad, const cct_po
  * else 0; relu_data is the pooled tensor (the ReLU's output), same shape as in_grad. */
 int cct_hip_maxpool_backward_relu(float *in_grad, const float *out_grad, const cct_pool_args *args,
                                   const float *relu_data);
+/* The same result from the pooling layer's OUTPUT tensor `pooled` (same shape as out_grad) instead
+ * of its input: a gradient lands only on a window's arg-max, whose activation IS the window's
+ * maximum, so switching off every window whose maximum is not positive gives the same sums, bit
+ * for bit, and reads a tensor a quarter the size.  `pooled` must still hold the values
+ * cct_hip_maxpool_forward wrote (a following in-place ReLU leaves their signs; in-place dropout
+ * does not: use cct_hip_maxpool_backward_relu then). */
+int cct_hip_maxpool_backward_relu_pooled(float *in_grad, const float *out_grad, const cct_pool_args *args,
+                                         const float *pooled);
 /* DeviceDriver::lrn_forward/lrn_backward, src/sched/DeviceDriver.h:140-147. */
 int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args *args,
                         const cct_lrn_forward_normalize_args *args2);

@@ -74,12 +74,20 @@ def _maxpool_bit_exact(oracle, cfg):
     drv.maxpool_backward(g2, dev(og), args, relu_data=dev(x))
     np.testing.assert_array_equal(host(g2), oracle.relu_backward(host(g), x))
     assert cfg == (5, 3, 10, 4, 2) or (x <= 0).any()
+    # the same mask taken from the pooling output (a window's arg-max holds the window's maximum)
+    g3 = empty(x.shape)
+    drv.maxpool_backward(g3, dev(og), args, pooled=y)
+    np.testing.assert_array_equal(host(g3), host(g2))
     if cfg == (5, 3, 10, 4, 2):
         np.testing.assert_allclose(host(y).reshape(-1), load_fixture("output", "pooling_forward.txt"), atol=1e-3)
         np.testing.assert_allclose(host(g).reshape(-1), load_fixture("output", "pooling_backward.txt"), atol=1e-3)
 
 
-@pytest.mark.parametrize("cfg", [(6, 3, 10, 3, 1e-4, 0.75), (2, 96, 27, 5, 1e-4, 0.75), (3, 7, 5, 5, 1e-2, 0.75)])
+@pytest.mark.parametrize("cfg", [(6, 3, 10, 3, 1e-4, 0.75), (2, 96, 27, 5, 1e-4, 0.75), (3, 7, 5, 5, 1e-2, 0.75),
+                                 # other exponents (exp2/log2 form) with windows of 5 and 3, a strong alpha,
+                                 # and a negative alpha (library powf)
+                                 (2, 16, 9, 5, 1e-2, 0.5), (2, 16, 9, 3, 2e-2, 1.25), (2, 20, 6, 5, 0.5, 0.75),
+                                 (2, 8, 6, 5, -1e-3, 0.75), (2, 8, 6, 3, -1e-3, 0.6)])
 def test_lrn(oracle, cfg):
     B, D, n, size, alpha, beta = cfg
     rng = np.random.default_rng(B + D)
