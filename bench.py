@@ -131,48 +131,87 @@ def cpu_baseline(cfg, seed):
     return result
 
 
+def net_workload(workload):
+    """Seeded synthetic tensors of benchmark configurations 4 (lenet) and 5 (caffenet): images, labels,
+    layer list, solver and one (weights, bias) pair per weight layer and channel group, generated on
+    the host.  Fillers follow the reference's prototxts: gaussian weights (std 0.01; 0.005 for
+    fc6/fc7) and bias 0.1 for CaffeNet, xavier-sized gaussian weights and zero bias for LeNet."""
+    import numpy as np
+    from caffecontroll_amd import nets
+    rng = np.random.default_rng(1234 + (4 if workload == "lenet" else 5))
+    if workload == "lenet":
+        B, D, S, classes = 64, 1, 28, 10
+        layers = nets.lenet_layers()
+        x = rng.uniform(0, 1, (B, D, S, S)).astype(np.float32)
+        solver = dict(base_lr=0.01, momentum=0.9, weight_decay=0.0005, lr_policy="inv", gamma=0.0001, power=0.75)
+    else:
+        B, D, S, classes = 256, 3, 227, 1000
+        layers = nets.caffenet_layers(groups=True)
+        x = rng.uniform(0, 255, (B, D, S, S)).astype(np.float32)
+        x -= np.array([104, 117, 123], np.float32)[None, :, None, None]
+        solver = dict(base_lr=0.01, momentum=0.9, weight_decay=0.0005, lr_policy="step", gamma=0.1, stepsize=100000)
+    labels = rng.integers(0, classes, B).astype(np.float32)
+    params = {}
+    d, n, n_fc = D, S, 0
+    for li, L in enumerate(layers):
+        if L.type == nets.CONV:
+            g = max(L.group, 1)
+            shapes = [(L.num_output // g, d // g, L.kernel_size, L.kernel_size)] * g
+            n = (n + 2 * L.pad - L.kernel_size) // L.stride + 1
+            d = L.num_output
+        elif L.type == nets.FC:
+            shapes = [(L.num_output, d * n * n)]
+            d, n = L.num_output, 1
+        elif L.type == nets.MAXPOOL:
+            n = (n - L.kernel_size) // L.stride + 1
+            continue
+        else:
+            continue
+        std = 0.01
+        if L.type == nets.FC and workload == "caffenet":
+            n_fc += 1
+            std = 0.005 if n_fc <= 2 else 0.01
+        for gi, shp in enumerate(shapes):
+            if workload == "lenet":
+                std = float(np.sqrt(1.0 / np.prod(shp[1:])))  # xavier-sized
+            w = rng.standard_normal(shp, dtype=np.float32) * np.float32(std)
+            bias = np.full(shp[0], 0.1 if workload == "caffenet" else 0.0, np.float32)
+            params[(li, gi)] = (w, bias)
+    return dict(B=B, D=D, S=S, classes=classes, layers=layers, x=x, labels=labels, solver=solver, params=params)
+
+
+# Loss per image of the FIRST forward pass of the workloads above (before any update), as the CPU
+# oracle computes it on the same tensors; tests/test_gpu_nets.py holds the device to the oracle on
+# exactly these tensors, and every bench run checks its own first loss against the figure.
+FIRST_LOSS_PER_IMAGE = {"caffenet": 6.914681, "lenet": 2.291778}
+
+
 def net_iteration(args, torch, np):
     """benchmark configurations 4 and 5: one step = forward + backward + SGD update of every layer,
     synthetic images and labels already on the device."""
     from caffecontroll_amd import HIPDriver, nets
     drv = HIPDriver(0)
     drv.set_stream(torch.cuda.current_stream().cuda_stream)
-    rng = np.random.default_rng(1234 + (4 if args.workload == "lenet" else 5))
-    if args.workload == "lenet":
-        B, D, S, classes = 64, 1, 28, 10
-        layers = nets.lenet_layers()
-        x = rng.uniform(0, 1, (B, D, S, S)).astype(np.float32)
-        solver = nets.solver_param(base_lr=0.01, momentum=0.9, weight_decay=0.0005, lr_policy="inv",
-                                   gamma=0.0001, power=0.75)
-    else:
-        B, D, S, classes = 256, 3, 227, 1000
-        layers = nets.caffenet_layers(groups=True)
-        x = rng.uniform(0, 255, (B, D, S, S)).astype(np.float32)
-        x -= np.array([104, 117, 123], np.float32)[None, :, None, None]
-        solver = nets.solver_param(base_lr=0.01, momentum=0.9, weight_decay=0.0005, lr_policy="step",
-                                   gamma=0.1, stepsize=100000)
-    labels = rng.integers(0, classes, B).astype(np.float32)
-    net = nets.Net(B, D, S, layers, solver)
-    # fillers of the reference's prototxts: gaussian weights (std 0.01; 0.005 for fc6/fc7), constant bias
-    n_fc = 0
-    for li, L in enumerate(layers):
-        for gi in range(max(L.group, 1)):
-            wp, wn = net.tensor(li, nets.MODEL, gi)
-            if not wp:
-                continue
-            std = 0.01
-            if L.type == nets.FC and args.workload == "caffenet":
-                n_fc += 1
-                std = 0.005 if n_fc <= 2 else 0.01
-            if args.workload == "lenet":
-                std = float(np.sqrt(1.0 / (wn / L.num_output)))  # xavier-sized
-            w = (rng.standard_normal(wn, dtype=np.float32) * np.float32(std))
-            drv.memcpy(wp, w.ctypes.data, w.nbytes, 0)
-            bp, bn = net.tensor(li, nets.BIAS, gi)
-            bias = np.full(bn, 0.1 if args.workload == "caffenet" else 0.0, np.float32)
-            drv.memcpy(bp, bias.ctypes.data, bias.nbytes, 0)
+    wl = net_workload(args.workload)
+    B, D, S, classes, layers, x, labels = (wl[k] for k in ("B", "D", "S", "classes", "layers", "x", "labels"))
+    rng = np.random.default_rng(99)
+    net = nets.Net(B, D, S, layers, nets.solver_param(**wl["solver"]))
+    for (li, gi), (w, bias) in wl["params"].items():
+        wp, wn = net.tensor(li, nets.MODEL, gi)
+        bp, bn = net.tensor(li, nets.BIAS, gi)
+        assert wn == w.size and bn == bias.size
+        drv.memcpy(wp, w.ctypes.data, w.nbytes, 0)
+        drv.memcpy(bp, bias.ctypes.data, bias.nbytes, 0)
     drv.memcpy(net.input_ptr(), x.ctypes.data, x.nbytes, 0)
     drv.memcpy(net.labels_ptr(), labels.ctypes.data, labels.nbytes, 0)
+    # the first forward pass (dropout off, so that nothing random enters) must reproduce the oracle's loss
+    net.set_train(False)
+    net.forward()
+    first_loss = net.loss() / B
+    net.set_train(True)
+    want = FIRST_LOSS_PER_IMAGE[args.workload]
+    if not abs(first_loss - want) <= 1e-3 * want:
+        raise SystemExit("bench.py: first-pass loss per image %.5f differs from the oracle's %.5f" % (first_loss, want))
 
     pipeline = None
     if args.input_pipeline:
@@ -243,6 +282,7 @@ def net_iteration(args, torch, np):
         "dtype": "f32", "data": "synthetic", "images_per_sec": round(B * 1e3 / ms, 1),
         "config": {"workload": "%s: fwd+bwd+SGD, batch %d, %dx%dx%d inputs, %d classes%s" % (
             args.workload, B, D, S, S, classes, ", conv2/4/5 in 2 groups" if args.workload == "caffenet" else "")},
+        "first_loss_per_image": round(float(first_loss), 5), "oracle_first_loss_per_image": want,
         "final_loss_per_image": round(float(loss), 5),
         **({"input_pipeline": pipeline} if pipeline is not None else {}),
     }

@@ -2,15 +2,24 @@
 DeepNet::run_forward_pass / run_backward_pass visit the bridges (src/DeepNet.h:171-266): ReLU and
 dropout in place, the first weight layer without a data gradient, grouped convolutions as
 independent convolutions on channel slices, one SGD update per weight layer per iteration."""
+from concurrent.futures import ThreadPoolExecutor
+
 import numpy as np
 
 CONV, FC, RELU, MAXPOOL, LRN, DROPOUT, SOFTMAXLOSS = 1, 2, 3, 4, 5, 6, 7
 
 
 class OracleNet:
-    def __init__(self, O, layers, batch, depth, size, solver):
-        """solver: dict(base_lr, momentum, weight_decay); fixed learning-rate policy."""
+    def __init__(self, O, layers, batch, depth, size, solver, partitions=1):
+        """solver: dict(base_lr, momentum, weight_decay); fixed learning-rate policy.
+        partitions > 1: convolutions run the way the reference's ParallelizedBridge runs them on a
+        CPU, the batch cut into that many contiguous partitions, one thread each, the partitions'
+        weight and bias gradients added up in partition order
+        (src/bridges/ParallelizedBridge_impl.hxx:888-955)."""
         self.O, self.layers, self.solver = O, layers, solver
+        self.partitions = max(1, min(partitions, batch))
+        self.bounds = [(i * batch // self.partitions, (i + 1) * batch // self.partitions)
+                       for i in range(self.partitions)]
         self.params = {}   # (layer, group) -> dict(w, b, hw, hb)
         self.shapes = []
         d, n = depth, size
@@ -40,6 +49,7 @@ class OracleNet:
             p["hw"] = np.zeros(p["w"].size, np.float32)
             p["hb"] = np.zeros(p["b"].size, np.float32)
         self.masks = {}
+        self.train = True   # False: dropout layers pass their input through (TEST phase)
 
     def forward(self, x, labels):
         O = self.O
@@ -54,7 +64,14 @@ class OracleNet:
                 for gi in range(g):
                     p = self.params[(i, gi)]
                     xin = np.ascontiguousarray(cur[:, gi * dg:(gi + 1) * dg])
-                    out, low = O.conv_forward(xin, p["w"], p["b"], L.kernel_size, L.stride, L.pad)
+                    if self.partitions == 1:
+                        out, low = O.conv_forward(xin, p["w"], p["b"], L.kernel_size, L.stride, L.pad)
+                    else:
+                        with ThreadPoolExecutor(self.partitions) as ex:
+                            parts = list(ex.map(lambda lh: O.conv_forward(xin[lh[0]:lh[1]], p["w"], p["b"], L.kernel_size,
+                                                                          L.stride, L.pad), self.bounds))
+                        out = np.concatenate([q[0] for q in parts], axis=0)
+                        low = [q[1] for q in parts]
                     self.saved[(i, gi)] = (xin.shape, low)
                     outs.append(out)
                 cur = np.concatenate(outs, axis=1) if g > 1 else outs[0]
@@ -74,7 +91,8 @@ class OracleNet:
                 cur, den = O.lrn_forward(cur, L.lrn_local_size, L.lrn_alpha, L.lrn_beta)
                 self.saved[(i, "den")] = den
             elif L.type == DROPOUT:
-                cur = O.dropout_forward(cur, self.masks[i], L.dropout_ratio, threshold=True)
+                if self.train:
+                    cur = O.dropout_forward(cur, self.masks[i], L.dropout_ratio, threshold=True)
                 self.acts[-1] = cur
             elif L.type == SOFTMAXLOSS:
                 cur, self.loss = O.softmax_loss_forward(cur, labels)
@@ -87,9 +105,12 @@ class OracleNet:
         O, s = self.O, self.solver
         grad = None
         self.grads = {}
+        self.in_grads = {}  # layer -> gradient with respect to the layer's input, as it leaves the layer
         ai = len(self.acts) - 1  # index of the activation produced by the layer being visited
         for i in range(len(self.layers) - 1, -1, -1):
             L = self.layers[i]
+            if i + 1 < len(self.layers) and grad is not None:
+                self.in_grads[i + 1] = grad
             if L.type == SOFTMAXLOSS:
                 grad = O.softmax_loss_backward(self.acts[ai], self.labels)
                 ai -= 1
@@ -123,8 +144,21 @@ class OracleNet:
                     p = self.params[(i, gi)]
                     shp, low = self.saved[(i, gi)]
                     og = np.ascontiguousarray(grad[:, gi * og_d:(gi + 1) * og_d])
-                    dx, dw, db = O.conv_backward(shp, p["w"], og, low, L.kernel_size, L.stride, L.pad,
-                                                 need_in_grad=need)
+                    if self.partitions == 1:
+                        dx, dw, db = O.conv_backward(shp, p["w"], og, low, L.kernel_size, L.stride, L.pad,
+                                                     need_in_grad=need)
+                    else:
+                        def part(j):
+                            lo, hi = self.bounds[j]
+                            return O.conv_backward((hi - lo,) + tuple(shp[1:]), p["w"], og[lo:hi], low[j], L.kernel_size,
+                                                   L.stride, L.pad, need_in_grad=need)
+                        with ThreadPoolExecutor(self.partitions) as ex:
+                            parts = list(ex.map(part, range(self.partitions)))
+                        dx = np.concatenate([q[0] for q in parts], axis=0) if need else None
+                        dw, db = parts[0][1].copy(), parts[0][2].copy()
+                        for q in parts[1:]:
+                            dw += q[1]
+                            db += q[2]
                     self.grads[(i, gi)] = (dw.copy(), db.copy())
                     self._update(p, L, dw, db)
                     dxs.append(dx)

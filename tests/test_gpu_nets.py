@@ -8,7 +8,6 @@ from oracle_net import OracleNet
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4
-GRAD_TOL = 5e-3
 
 
 def _up(ptr, arr):
@@ -36,6 +35,36 @@ def _init_and_sync_params(net, ref, rng, std_of=None):
         _up(bp, p["b"])
 
 
+def _check_forward_and_align_switches(net, ref, layers, tol):
+    """Every non-in-place layer's output against the oracle's (within `tol` of its largest magnitude),
+    then the oracle's activations and max-pool arg-max indices are written into the device's
+    buffers, so that both sides read the same ReLU masks and route pooled gradients to the same
+    pixels in the backward pass.  Returns (worst forward error, activations, sign disagreements,
+    pooling windows, arg-max disagreements)."""
+    from caffecontroll_amd import nets
+    ai, worst = 1, 0.0
+    elements = sign_flips = windows = argmax_flips = 0
+    for li, L in enumerate(layers):
+        if L.type in (nets.RELU, nets.DROPOUT):
+            continue
+        ptr, n = net.tensor(li, nets.OUTPUT)
+        got, want = _down(ptr, n), ref.acts[ai].reshape(-1)
+        e = rel_err(got, want)
+        worst = max(worst, e)
+        assert e <= tol, "forward layer %d (type %d): %.3g" % (li, L.type, e)
+        elements += n
+        sign_flips += int(np.count_nonzero((got > 0) != (want > 0)))
+        _up(ptr, want)
+        if L.type == nets.MAXPOOL:
+            ptr, n = net.tensor(li, nets.AUX)
+            want = ref.saved[(li, "idx")].reshape(-1).astype(np.int32)
+            windows += n
+            argmax_flips += int(np.count_nonzero(_down(ptr, n, np.int32) != want))
+            _up(ptr, want)
+        ai += 1
+    return worst, elements, sign_flips, windows, argmax_flips
+
+
 def _compare_params(net, ref, tol):
     from caffecontroll_amd import nets
     worst = 0.0
@@ -55,12 +84,8 @@ def _compare_params(net, ref, tol):
             # w before the update = w_after + h_after
             w_before = p["w" if k == 0 else "b"].reshape(-1) + p["hw" if k == 0 else "hb"]
             e = rel_err(got, want + np.float32(lam) * w_before)
-            # Looser than the per-operator bar on purpose: when two candidates of a pooling window
-            # differ by an ulp between the two sides the argmax flips, the gradient of that window
-            # is routed to the neighbouring pixel, and a weight gradient moves by ~1e-3 of its
-            # largest entry although every operator is within 1e-6 (bias gradients, which only sum
-            # the routed values, stay at 1e-6).
-            assert e <= GRAD_TOL, "layer %d group %d grad %d: %.3g" % (li, gi, k, e)
+            worst = max(worst, e)
+            assert e <= tol, "layer %d group %d grad %d: %.3g" % (li, gi, k, e)
     return worst
 
 
@@ -74,22 +99,32 @@ def test_lenet_training_iterations(oracle):
     driver()
     net = nets.Net(B, 1, 28, layers, nets.solver_param(**solver))
     ref = OracleNet(oracle, layers, B, 1, 28, solver)
-    _init_and_sync_params(net, ref, rng)
+    # the tensors `bench.py --workload lenet` times; later iterations draw new images
+    import bench
+    wl = bench.net_workload("lenet")
+    for (li, gi), p in sorted(ref.params.items()):
+        w, bias = wl["params"][(li, gi)]
+        p["w"][...] = w.reshape(p["w"].shape)
+        p["b"][...] = bias
+        _up(net.tensor(li, nets.MODEL, gi)[0], p["w"])
+        _up(net.tensor(li, nets.BIAS, gi)[0], p["b"])
     bound = oracle.bind_openblas(8)
     try:
         for it in range(3):
-            x = rng.uniform(0, 1, (B, 1, 28, 28)).astype(np.float32)
-            labels = rng.integers(0, 10, B).astype(np.float32)
+            x = wl["x"] if it == 0 else rng.uniform(0, 1, (B, 1, 28, 28)).astype(np.float32)
+            labels = wl["labels"] if it == 0 else rng.integers(0, 10, B).astype(np.float32)
             _up(net.input_ptr(), x)
             _up(net.labels_ptr(), labels)
             net.forward()
             prob = ref.forward(x, labels)
+            if it == 0:   # the loss bench.py checks its first pass against
+                assert abs(ref.loss / B - bench.FIRST_LOSS_PER_IMAGE["lenet"]) <= 1e-4 * ref.loss / B, ref.loss / B
             ptr, n = net.tensor(len(layers) - 1, nets.OUTPUT)
             assert rel_err(_down(ptr, n), prob.reshape(-1)) <= TOL
             assert abs(net.loss() - ref.loss) <= TOL * max(1.0, abs(ref.loss))
-            # pooled conv1 features and their argmax agree exactly in index, to 1e-4 in value
-            ptr, n = net.tensor(1, nets.OUTPUT)
-            assert rel_err(_down(ptr, n), ref.acts[2].reshape(-1)) <= TOL
+            # every layer to 1e-4; ReLU masks and pooling arg-max aligned before the backward pass
+            _, elements, sign_flips, windows, argmax_flips = _check_forward_and_align_switches(net, ref, layers, TOL)
+            assert sign_flips <= 1e-4 * elements and argmax_flips <= 1e-4 * windows
             net.backward()
             ref.backward()
             _compare_params(net, ref, TOL)
@@ -129,19 +164,95 @@ def test_caffenet_training_iteration_small_batch(oracle, groups):
     try:
         net.forward()
         prob = ref.forward(x, labels)
-        # layer by layer (non in-place layers), deepest error first to show
-        ai = 1
-        for li, L in enumerate(layers):
-            if L.type in (nets.RELU, nets.DROPOUT):
-                continue
-            ptr, n = net.tensor(li, nets.OUTPUT)
-            e = rel_err(_down(ptr, n), ref.acts[ai].reshape(-1))
-            assert e <= 5 * TOL, "forward layer %d (type %d): %.3g" % (li, L.type, e)
-            ai += 1
-        assert abs(net.loss() - ref.loss) <= 5 * TOL * max(1.0, abs(ref.loss))
+        _, elements, sign_flips, windows, argmax_flips = _check_forward_and_align_switches(net, ref, layers, TOL)
+        assert sign_flips <= 1e-4 * elements and argmax_flips <= 1e-4 * windows
+        assert abs(net.loss() - ref.loss) <= TOL * max(1.0, abs(ref.loss))
         net.backward()
         ref.backward()
-        _compare_params(net, ref, 5 * TOL)
+        _compare_params(net, ref, TOL)
+    finally:
+        if bound:
+            oracle.unbind_openblas()
+    net.close()
+
+
+@pytest.mark.timeout(900)
+def test_caffenet_full_batch_iteration(oracle):
+    """benchmark configuration 5 at its full size: batch 256, grouped conv2/4/5, the instances the bench
+    times (plane-tiled pooling, run-of-channels LRN, 4/6/8-wavefront weight gradients, deferred batched
+    SGD), against the oracle chain run the way the reference runs on a CPU (16 batch partitions).
+
+    Forward: every layer's output within 1e-4 of its largest magnitude, loss within 1e-4.
+    The network has two kinds of switches that a rounding difference can flip: the arg-max of a
+    pooling window and the sign test of a ReLU.  Both sides may disagree on them only where the
+    competing values agree to rounding -- on fewer than 1e-5 of the windows / activations, which is
+    asserted.  One flipped switch reroutes a whole gradient value (a single fc6 unit changes 3 % of
+    that layer's weight gradient), so before the backward pass the oracle's switches are written
+    into the device's buffers -- its arg-max indices and its activations, which the masks are read
+    from -- and the backward pass is then held to the per-operator bar of 1e-4: every weight and
+    bias gradient and every updated weight."""
+    from caffecontroll_amd import nets
+    import bench
+    wl = bench.net_workload("caffenet")          # the tensors `bench.py --workload caffenet` times
+    rng = np.random.default_rng(77)
+    B, layers, x, labels = wl["B"], wl["layers"], wl["x"], wl["labels"]
+    assert B == 256
+    solver = dict(base_lr=0.01, momentum=0.9, weight_decay=0.0005)
+    driver()
+    net = nets.Net(B, 3, 227, layers, nets.solver_param(**solver))
+    ref = OracleNet(oracle, layers, B, 3, 227, solver, partitions=16)
+    for (li, gi), p in sorted(ref.params.items()):
+        w, bias = wl["params"][(li, gi)]
+        p["w"][...] = w.reshape(p["w"].shape)
+        p["b"][...] = bias
+        _up(net.tensor(li, nets.MODEL, gi)[0], p["w"])
+        _up(net.tensor(li, nets.BIAS, gi)[0], p["b"])
+    net.freeze_dropout_masks(True)
+    for li, L in enumerate(layers):
+        if L.type == nets.DROPOUT:
+            ptr, n = net.tensor(li, nets.AUX)
+            mask = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+            _up(ptr, mask)
+            ref.masks[li] = mask
+    _up(net.input_ptr(), x)
+    _up(net.labels_ptr(), labels)
+    bound = oracle.bind_openblas(1)
+    try:
+        # TEST phase first (dropout off): the loss bench.py checks its first pass against
+        net.set_train(False)
+        ref.train = False
+        net.forward()
+        ref.forward(x, labels)
+        assert abs(net.loss() - ref.loss) <= TOL * abs(ref.loss)
+        assert abs(ref.loss / B - bench.FIRST_LOSS_PER_IMAGE["caffenet"]) <= 1e-4 * ref.loss / B, ref.loss / B
+        net.set_train(True)
+        ref.train = True
+        net.forward()
+        ref.forward(x, labels)
+        worst_fwd, elements, sign_flips, windows, argmax_flips = _check_forward_and_align_switches(net, ref, layers, TOL)
+        assert abs(net.loss() - ref.loss) <= TOL * abs(ref.loss)
+        # N(0, 0.01) weights give nearly uniform class scores: the loss per image sits at ln(1000)
+        assert abs(ref.loss / B - np.log(1000.0)) < 0.1
+        assert argmax_flips <= 1e-5 * windows, (argmax_flips, windows)
+        assert sign_flips <= 1e-5 * elements, (sign_flips, elements)
+        net.backward()
+        ref.backward()
+        worst_bwd = 0.0
+        for (li, gi), p in sorted(ref.params.items()):
+            for which, k, key, hist in ((nets.MODEL_GRAD, 0, "w", "hw"), (nets.BIAS_GRAD, 1, "b", "hb")):
+                ptr, n = net.tensor(li, which, gi)
+                lam = np.float32(solver["weight_decay"] * layers[li].decay_mult[k])
+                w_before = p[key].reshape(-1) + p[hist]          # w after the update + its momentum step
+                want = ref.grads[(li, gi)][k].reshape(-1) + lam * w_before
+                e = rel_err(_down(ptr, n), want)
+                worst_bwd = max(worst_bwd, e)
+                assert e <= TOL, "layer %d group %d gradient %d: %.3g" % (li, gi, k, e)
+            for which, key in ((nets.MODEL, "w"), (nets.BIAS, "b")):
+                ptr, n = net.tensor(li, which, gi)
+                assert rel_err(_down(ptr, n), p[key].reshape(-1)) <= TOL
+        print("full-batch CaffeNet: worst forward error %.3g, worst gradient error %.3g, arg-max differing on %d of %d "
+              "windows, ReLU sign on %d of %d activations, loss/image %.5f"
+              % (worst_fwd, worst_bwd, argmax_flips, windows, sign_flips, elements, ref.loss / B))
     finally:
         if bound:
             oracle.unbind_openblas()
