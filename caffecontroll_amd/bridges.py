@@ -26,6 +26,8 @@ _P, _I = C.c_void_p, C.c_int
 BRIDGE_PROTOTYPES = {
     "cct_conv_bridge_create": ([C.POINTER(_P), _I, _I, _I, C.POINTER(ConvParam), C.POINTER(SolverParam),
                                 _P, _P, _P, _P], _I),
+    "cct_conv_bridge_create_shared": ([C.POINTER(_P), _I, _I, _I, C.POINTER(ConvParam), C.POINTER(SolverParam),
+                                       _P, _P, _P, _P, _I, _I], _I),
     "cct_conv_bridge_destroy": ([_P], _I),
     "cct_conv_bridge_set_options": ([_P, _I, _I, _I], _I),
     "cct_conv_bridge_path": ([_P], _I),
@@ -70,7 +72,10 @@ class ConvolutionLayer:
     ``data_ptr()``; they must stay alive as long as this object)."""
 
     def __init__(self, b, d, n, k, s, p, o, in_data, in_grad, out_data, out_grad, bias_term=True,
-                 solver=None, lr_mult=(1.0, 1.0), decay_mult=(1.0, 1.0)):
+                 solver=None, lr_mult=(1.0, 1.0), decay_mult=(1.0, 1.0), share_prev=True, share_next=True):
+        """share_prev / share_next = False: the input / output layer is HOST memory (contiguous float32
+        numpy arrays); the bridge then copies to and from its own device cubes, as the reference's
+        ParallelizedBridge does for a bridge whose neighbour is not on the same device."""
         self.lib = _bind()
         self.shape = (b, d, n, k, s, p, o)
         self.m = (n + 2 * p - k) // s + 1
@@ -78,9 +83,10 @@ class ConvolutionLayer:
         self._solver = solver or solver_param()
         self._keep = (in_data, in_grad, out_data, out_grad)
         h = C.c_void_p()
-        ptr = lambda t: None if t is None else t.data_ptr()
-        check(self.lib.cct_conv_bridge_create(C.byref(h), b, d, n, C.byref(cp), C.byref(self._solver),
-                                              ptr(in_data), ptr(in_grad), ptr(out_data), ptr(out_grad)),
+        ptr = lambda t: None if t is None else (t.data_ptr() if hasattr(t, "data_ptr") else t.ctypes.data)
+        check(self.lib.cct_conv_bridge_create_shared(C.byref(h), b, d, n, C.byref(cp), C.byref(self._solver),
+                                                     ptr(in_data), ptr(in_grad), ptr(out_data), ptr(out_grad),
+                                                     int(share_prev), int(share_next)),
               "conv_bridge_create")
         self.h = h
 

@@ -37,9 +37,18 @@ extern "C" {
 int cct_conv_bridge_create(cct_conv_bridge **out, int b, int d, int n, const cct_conv_param *conv,
                            const cct_solver_param *solver, float *in_data, float *in_grad, float *out_data,
                            float *out_grad) {
+  return cct_conv_bridge_create_shared(out, b, d, n, conv, solver, in_data, in_grad, out_data, out_grad, 1, 1);
+}
+
+int cct_conv_bridge_create_shared(cct_conv_bridge **out, int b, int d, int n, const cct_conv_param *conv,
+                                  const cct_solver_param *solver, float *in_data, float *in_grad, float *out_data,
+                                  float *out_grad, int share_pointer_with_prev_bridge,
+                                  int share_pointer_with_next_bridge) {
   if (!out || !conv || b <= 0 || d <= 0 || n <= 0 || conv->kernel_size <= 0 || conv->stride <= 0 ||
-      conv->num_output <= 0 || n + 2 * conv->pad < conv->kernel_size || !in_data || !out_data)
-    return CCT_HIP_EINVAL;
+      conv->num_output <= 0 || conv->pad < 0 || n + 2 * conv->pad < conv->kernel_size || !in_data || !out_data)
+    return cct::set_error(CCT_HIP_EINVAL, "conv_bridge_create: bad geometry or null tensor");
+  if ((!share_pointer_with_prev_bridge && !in_grad) || (!share_pointer_with_next_bridge && !out_grad))
+    return cct::set_error(CCT_HIP_EINVAL, "conv_bridge_create: a host-resident layer needs both of its cubes");
   cct_conv_bridge *h = new cct_conv_bridge;
   const int k = conv->kernel_size, s = conv->stride, p = conv->pad, o = conv->num_output;
   const int m = (n + 2 * p - k) / s + 1;
@@ -53,7 +62,8 @@ int cct_conv_bridge_create(cct_conv_bridge **out, int b, int d, int n, const cct
   h->out_layer = new Layer<float>(new LogicalCube<float>(out_data, m, m, o, b),
                                   new LogicalCube<float>(out_grad, m, m, o, b));
   h->pbridge = new ParallelizedBridge<float, ConvolutionBridge, HIPDriver>(
-      h->in_layer, h->out_layer, &h->layer_param, &h->solver_param, &h->driver, 1, 1);
+      h->in_layer, h->out_layer, &h->layer_param, &h->solver_param, &h->driver, 1, 1,
+      share_pointer_with_prev_bridge != 0, share_pointer_with_next_bridge != 0, false);
   *out = h;
   return 0;
 }
@@ -164,9 +174,14 @@ void *cct_net_tensor(cct_net *h, int layer, int group, int which, size_t *n) {
   if (n) *n = 0;
   if (!h || layer < 0 || layer >= h->net->num_layers()) return nullptr;
   Network::Node &nd = h->net->node(layer);
+  LogicalCube<float> *c = nullptr;
+  if (which == 4 || which == 5) {  // tensors of the layer itself, whatever bridges it has (CONCAT has none)
+    c = which == 4 ? nd.out->p_data_cube : nd.in->p_gradient_cube;
+    if (n) *n = c->n_elements;
+    return c->get_p_data();
+  }
   if (group < 0 || group >= (int)nd.bridges.size()) return nullptr;
   Network::BridgeT *b = nd.bridges[group];
-  LogicalCube<float> *c = nullptr;
   switch (which) {
     case 0: c = b->get_model_cube(); break;
     case 1: c = b->get_bias_cube(); break;

@@ -1,8 +1,18 @@
-// A linear chain of bridges on the HIP driver, each wrapped in a one-partition ParallelizedBridge:
-// the device-resident equivalent of what DeepNet::construct_network builds from a prototxt
-// (src/DeepNet.h:968-2030) and of run_forward_pass / run_backward_pass (src/DeepNet.h:171-266),
-// for nets that are a plain sequence of layers (LeNet, CaffeNet).  Layer descriptions come as a C
-// array instead of a parsed prototxt.
+// Bridges on the HIP driver, each wrapped in a one-partition ParallelizedBridge: the device-resident
+// equivalent of what DeepNet::construct_network builds from a prototxt (src/DeepNet.h:968-2030) and
+// of run_forward_pass / run_backward_pass (src/DeepNet.h:171-266).  Layer descriptions come as a C
+// array instead of a parsed prototxt, in the prototxt's order; each layer reads the one before it
+// (LeNet, CaffeNet) or the layers its `bottoms` name (the reference's two-tower networks).
+//
+// Graph rules (src/DeepNet.h:1700-1757, 1924-2028):
+//   * a layer output read by several layers is shared, not copied: every reader sees the same data
+//     cube; the first reader writes its gradient into the producer's gradient cube, every further
+//     reader into a cube of its own, and before the producer's (or the last in-place layer's)
+//     backward step the extra cubes are added to the first in reader order -- the sum the
+//     reference's Split bridge forms;
+//   * CONCAT stacks its bottoms along the depth: forward copies each bottom into its channel slice
+//     of the output, backward copies the slices of the output gradient back;
+//   * a layer computes an input gradient only if some layer with weights lies upstream of it.
 //
 // Placement rules kept from the reference:
 //   * output sizes: conv (R+2p-K)/s+1 (:112-115), pooling floor((R-K)/s)+1 unpadded (:1374-1376);
@@ -21,6 +31,7 @@
 #pragma once
 #include <cmath>
 #include <cstdio>
+#include <map>
 #include <memory>
 #include <stdexcept>
 #include <string>
@@ -42,8 +53,10 @@ class Network {
 
   struct Node {
     cct_layer_spec spec;
-    LayerT *in = nullptr;   // not owned here (owned through layers_)
+    LayerT *in = nullptr;   // the (first) bottom as this node sees it; not owned here (owned through layers_)
     LayerT *out = nullptr;
+    std::vector<LayerT *> ins;                   // every bottom (CONCAT has several)
+    bool run_backward = true;                    // false: no layer with weights upstream and none here
     std::vector<BridgeT *> bridges;              // one per group (1 for everything but grouped conv)
     std::vector<LayerT *> group_in, group_out;   // per-group contiguous layers (grouped conv only)
     std::vector<cnn::LayerParameter *> params;
@@ -70,9 +83,17 @@ class Network {
           std::string(sp->regularization_type) != "L1")
         return std::string("regularization_type must be L2 or L1, not \"") + sp->regularization_type + "\"";
     }
-    long R = size, D = depth;
+    std::vector<long> Rs(n_specs), Ds(n_specs);
     for (int i = 0; i < n_specs; ++i) {
       const cct_layer_spec &s = specs[i];
+      if (s.n_bottoms < 0 || s.n_bottoms > CCT_MAX_BOTTOMS) return at(i, "n_bottoms out of range");
+      if (s.type != CCT_LAYER_CONCAT && s.n_bottoms > 1) return at(i, "only CONCAT reads more than one layer");
+      if (s.type == CCT_LAYER_CONCAT && s.n_bottoms < 2) return at(i, "CONCAT needs at least two bottoms");
+      for (int j = 0; j < s.n_bottoms; ++j)
+        if (s.bottoms[j] < -1 || s.bottoms[j] >= i)
+          return at(i, "bottom " + std::to_string(s.bottoms[j]) + " is not the network input (-1) or an earlier layer");
+      const int b0 = s.n_bottoms ? s.bottoms[0] : i - 1;
+      long R = b0 < 0 ? size : Rs[b0], D = b0 < 0 ? depth : Ds[b0];
       switch (s.type) {
         case CCT_LAYER_CONV: {
           if (s.num_output <= 0) return at(i, "convolution needs num_output >= 1");
@@ -110,12 +131,38 @@ class Network {
         case CCT_LAYER_DROPOUT:
           if (!(s.dropout_ratio >= 0.f && s.dropout_ratio < 1.f)) return at(i, "dropout_ratio must be in [0, 1)");
           break;
+        case CCT_LAYER_CONCAT:
+          D = 0;
+          for (int j = 0; j < s.n_bottoms; ++j) {
+            const long Rj = s.bottoms[j] < 0 ? size : Rs[s.bottoms[j]];
+            if (Rj != R) return at(i, "CONCAT bottoms differ in height / width");
+            D += s.bottoms[j] < 0 ? depth : Ds[s.bottoms[j]];
+          }
+          break;
         case CCT_LAYER_RELU:
         case CCT_LAYER_SOFTMAXLOSS:
           break;
         default:
           return at(i, "unknown layer type " + std::to_string(s.type));
       }
+      if ((s.type == CCT_LAYER_RELU || s.type == CCT_LAYER_DROPOUT) && b0 >= 0)
+        for (int q = b0 + 1; q < i; ++q) {
+          // in place on a tensor that an earlier layer already reads: that reader would see it change
+          const cct_layer_spec &t = specs[q];
+          const int nb = t.n_bottoms ? t.n_bottoms : 1;
+          for (int j = 0; j < nb; ++j) {
+            int tb = t.n_bottoms ? t.bottoms[j] : q - 1;
+            while (tb >= 0 && (specs[tb].type == CCT_LAYER_RELU || specs[tb].type == CCT_LAYER_DROPOUT))
+              tb = specs[tb].n_bottoms ? specs[tb].bottoms[0] : tb - 1;  // in-place layers write their bottom's tensor
+            int mine = b0;
+            while (mine >= 0 && (specs[mine].type == CCT_LAYER_RELU || specs[mine].type == CCT_LAYER_DROPOUT))
+              mine = specs[mine].n_bottoms ? specs[mine].bottoms[0] : mine - 1;
+            if (tb == mine && t.type != CCT_LAYER_RELU && t.type != CCT_LAYER_DROPOUT)
+              return at(i, "runs in place on a tensor that layer " + std::to_string(q) + " already reads");
+          }
+        }
+      Rs[i] = R;
+      Ds[i] = D;
       if ((double)batch * (double)D * (double)R * (double)R >= 2147483648.0)
         return at(i, "output tensor has 2^31 elements or more");
     }
@@ -136,13 +183,26 @@ class Network {
       if (sp->regularization_type) solver_.regularization_type_ = sp->regularization_type;
     }
     labels_ = new CubeT(1, 1, 1, batch, &driver_);
-    LayerT *cur = new_layer(size, size, depth);
-    bool first_weight_layer = true;
+    LayerT *const input_layer = new_layer(size, size, depth);
+    blobs_[input_layer] = TensorInfo();
     for (int i = 0; i < n_specs; ++i) {
       Node nd;
       nd.spec = specs[i];
-      nd.in = cur;
       const cct_layer_spec &s = specs[i];
+      // the tensor(s) this layer reads: the producers' layers as they are; `cur` becomes this node's
+      // own view of the first one below (the same layer for the first reader and for in-place layers)
+      std::vector<LayerT *> bottoms;
+      if (s.n_bottoms == 0) bottoms.push_back(i == 0 ? input_layer : nodes_[i - 1].out);
+      for (int j = 0; j < s.n_bottoms; ++j)
+        bottoms.push_back(s.bottoms[j] < 0 ? input_layer : nodes_[s.bottoms[j]].out);
+      const bool in_place = s.type == CCT_LAYER_RELU || s.type == CCT_LAYER_DROPOUT;
+      bool params_upstream = false;
+      for (LayerT *b : bottoms) params_upstream = params_upstream || blobs_[b].params_upstream;
+      const bool first_weight_layer = !params_upstream;
+      const int producer_node = blobs_[bottoms[0]].last_writer;  // -1: the network input
+      for (LayerT *b : bottoms) nd.ins.push_back(in_place ? b : consume(b));
+      LayerT *cur = nd.ins[0];
+      nd.in = cur;
       const size_t R = cur->dR, D = cur->dD;
       switch (s.type) {
         case CCT_LAYER_CONV: {
@@ -164,8 +224,8 @@ class Network {
             // A group works in place on its channel slices of the whole tensors when the direct
             // kernels take the layer (they accept an image stride); otherwise the slices are
             // gathered into contiguous per-group layers and scattered back.
-            const bool in_place = g > 1 && group_in_place(R, D / g, s, s.num_output / g, m);
-            if (g > 1 && in_place) {
+            const bool slices_in_place = g > 1 && group_in_place(R, D / g, s, s.num_output / g, m);
+            if (g > 1 && slices_in_place) {
               const size_t din = D / g, dout = s.num_output / g;
               gin = view_layer(cur, gi * din * R * R, R, R, din);
               gout = view_layer(nd.out, gi * dout * m * m, m, m, dout);
@@ -176,19 +236,10 @@ class Network {
               nd.group_out.push_back(gout);
             }
             auto *b = new ParallelizedBridge<float, ConvolutionBridge, HIPDriver>(gin, gout, lp, &solver_, &driver_);
-            if (in_place) b->sub_bridge()->set_image_strides(D * R * R, (size_t)s.num_output * m * m);
+            if (slices_in_place) b->sub_bridge()->set_image_strides(D * R * R, (size_t)s.num_output * m * m);
             b->needs_to_calc_backward_grad = !first_weight_layer;
             nd.bridges.push_back(b);
           }
-          // directly after an in-place ReLU the layer masks the input gradient it produces (in the
-          // direct kernel's store) and the ReLU bridge skips its own backward pass over the tensor
-          if (!first_weight_layer && !nodes_.empty() && nodes_.back().spec.type == CCT_LAYER_RELU &&
-              nodes_.back().out == cur) {
-            for (BridgeT *cb : nd.bridges)
-              static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(cb)->sub_bridge()->input_is_relu_output = true;
-            static_cast<ReLUBridge<float, HIPDriver> *>(nodes_.back().bridges[0])->backward_done_by_consumer = true;
-          }
-          first_weight_layer = false;
           break;
         }
         case CCT_LAYER_FC: {
@@ -201,7 +252,6 @@ class Network {
           nd.params.push_back(lp);
           auto *b = new ParallelizedBridge<float, FullyConnectedBridge, HIPDriver>(cur, nd.out, lp, &solver_, &driver_);
           b->needs_to_calc_backward_grad = !first_weight_layer;
-          first_weight_layer = false;
           nd.bridges.push_back(b);
           break;
         }
@@ -209,9 +259,10 @@ class Network {
           nd.out = cur;  // in place
           nd.params.push_back(new_param(s));
           auto *rb = new ReLUBridge<float, HIPDriver>(cur, cur, nd.params[0], &solver_, &driver_);
-          // directly after a convolution the clamp rides on the convolution's output store
-          if (!nodes_.empty() && nodes_.back().spec.type == CCT_LAYER_CONV && nodes_.back().out == cur) {
-            for (BridgeT *cb : nodes_.back().bridges)
+          // directly after a convolution the clamp rides on the convolution's output store (nothing
+          // reads the tensor in between: an in-place layer on a tensor that already has readers is refused)
+          if (producer_node >= 0 && nodes_[producer_node].spec.type == CCT_LAYER_CONV) {
+            for (BridgeT *cb : nodes_[producer_node].bridges)
               static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(cb)->sub_bridge()->set_fuse_relu(true);
             rb->forward_done_by_producer = true;
           }
@@ -233,14 +284,7 @@ class Network {
           lp->pooling_param_.kernel_size_ = s.kernel_size;
           lp->pooling_param_.stride_ = s.stride;
           nd.params.push_back(lp);
-          auto *pb = new MaxPoolingBridge<float, HIPDriver>(cur, nd.out, lp, &solver_, &driver_);
-          // directly after an in-place ReLU the pooling backward stores the gradient already masked
-          // and the ReLU bridge skips its own backward pass over the tensor
-          if (!nodes_.empty() && nodes_.back().spec.type == CCT_LAYER_RELU && nodes_.back().out == cur) {
-            pb->input_is_relu_output = true;
-            static_cast<ReLUBridge<float, HIPDriver> *>(nodes_.back().bridges[0])->backward_done_by_consumer = true;
-          }
-          nd.bridges.push_back(pb);
+          nd.bridges.push_back(new MaxPoolingBridge<float, HIPDriver>(cur, nd.out, lp, &solver_, &driver_));
           break;
         }
         case CCT_LAYER_LRN: {
@@ -260,19 +304,56 @@ class Network {
           nd.bridges.push_back(softmax_);
           break;
         }
+        case CCT_LAYER_CONCAT: {
+          size_t total_d = 0;
+          for (LayerT *b : nd.ins) total_d += b->dD;
+          nd.out = new_layer(R, R, total_d);
+          break;
+        }
         default:
           fail("unknown layer type");
       }
-      cur = nd.out;
+      const bool has_params = s.type == CCT_LAYER_CONV || s.type == CCT_LAYER_FC;
+      nd.run_backward = has_params || params_upstream;
+      TensorInfo &ob = blobs_[nd.out];  // created here for a new tensor, found for an in-place layer
+      ob.params_upstream = ob.params_upstream || params_upstream || has_params;
+      ob.last_writer = i;
+      ob.writers.push_back(i);
       nodes_.push_back(nd);
     }
-    // a pooling layer that folds a ReLU backward may take its mask from its own output, unless the
-    // layer after it rewrites that tensor in place (dropout does; a ReLU keeps the signs)
+    // Fusions that depend on who reads a tensor, decided now that every reader is known.
     for (size_t i = 0; i < nodes_.size(); ++i) {
-      if (nodes_[i].spec.type != CCT_LAYER_MAXPOOL) continue;
-      const bool rewritten = i + 1 < nodes_.size() && nodes_[i + 1].out == nodes_[i].out &&
-                             nodes_[i + 1].spec.type != CCT_LAYER_RELU;
-      static_cast<MaxPoolingBridge<float, HIPDriver> *>(nodes_[i].bridges[0])->output_keeps_signs = !rewritten;
+      Node &nd = nodes_[i];
+      if (nd.spec.type != CCT_LAYER_CONV && nd.spec.type != CCT_LAYER_MAXPOOL) continue;
+      const cct_layer_spec &s = nd.spec;
+      LayerT *bottom = s.n_bottoms ? (s.bottoms[0] < 0 ? layers_[0] : nodes_[s.bottoms[0]].out)
+                                   : (i == 0 ? layers_[0] : nodes_[i - 1].out);
+      const TensorInfo &bb = blobs_[bottom];
+      // the last layer that wrote the tensor before this reader came
+      int writer = -1;
+      for (int w : bb.writers)
+        if (w < (int)i) writer = w;
+      // Directly after an in-place ReLU, and as the tensor's only reader, the layer performs that
+      // ReLU's backward itself: a convolution masks the input gradient it produces (in the direct
+      // kernel's store), a pooling layer stores its gradient already masked; the ReLU bridge then
+      // skips its own backward pass over the tensor.
+      if (writer >= 0 && nodes_[writer].spec.type == CCT_LAYER_RELU && bb.readers == 1 && bb.writers.back() == writer &&
+          nd.bridges[0]->needs_to_calc_backward_grad && nd.run_backward) {
+        if (nd.spec.type == CCT_LAYER_CONV)
+          for (BridgeT *cb : nd.bridges)
+            static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(cb)->sub_bridge()->input_is_relu_output = true;
+        else
+          static_cast<MaxPoolingBridge<float, HIPDriver> *>(nd.bridges[0])->input_is_relu_output = true;
+        static_cast<ReLUBridge<float, HIPDriver> *>(nodes_[writer].bridges[0])->backward_done_by_consumer = true;
+      }
+      if (nd.spec.type == CCT_LAYER_MAXPOOL) {
+        // a pooling layer that folds a ReLU backward may take its mask from its own output, unless a
+        // later layer rewrites that tensor in place (dropout does; a ReLU keeps the signs)
+        bool rewritten = false;
+        for (int w : blobs_[nd.out].writers)
+          if (w > (int)i && nodes_[w].spec.type != CCT_LAYER_RELU) rewritten = true;
+        static_cast<MaxPoolingBridge<float, HIPDriver> *>(nd.bridges[0])->output_keeps_signs = !rewritten;
+      }
     }
   }
 
@@ -305,6 +386,7 @@ class Network {
       const size_t g = nd.group_in.size();
       for (size_t gi = 0; gi < g; ++gi)
         slice_copy(nd.group_in[gi]->p_data_cube, nd.in->p_data_cube, gi, /*gather=*/true);
+      if (nd.spec.type == CCT_LAYER_CONCAT) concat_copy(nd, /*data=*/true);
       for (BridgeT *b : nd.bridges) b->forward();
       for (size_t gi = 0; gi < g; ++gi)
         slice_copy(nd.group_out[gi]->p_data_cube, nd.out->p_data_cube, gi, /*gather=*/false);
@@ -317,8 +399,15 @@ class Network {
     // the layers' SGD updates are collected and applied after the last backward: the many small
     // tensors then share one launch
     driver_.begin_deferred_sgd();
+    for (auto &kv : blobs_) kv.second.summed = false;
     for (int i = (int)nodes_.size() - 1; i >= 0; --i) {
       Node &nd = nodes_[i];
+      if (!nd.run_backward) continue;
+      sum_reader_gradients(nd.out);
+      if (nd.spec.type == CCT_LAYER_CONCAT) {
+        concat_copy(nd, /*data=*/false);
+        continue;
+      }
       const size_t g = nd.group_in.size();
       for (size_t gi = 0; gi < g; ++gi)
         slice_copy(nd.group_out[gi]->p_gradient_cube, nd.out->p_gradient_cube, gi, /*gather=*/true);
@@ -422,6 +511,53 @@ class Network {
   std::vector<LayerT *> layers_;
   std::vector<Node> nodes_;
   SoftmaxLossBridge<float, HIPDriver> *softmax_ = nullptr;
+
+  // What the network knows about a tensor (a Layer that some node produced, or the input).
+  struct TensorInfo {
+    int readers = 0;                   // layers that read it (in-place layers do not count)
+    std::vector<CubeT *> extra_grads;  // gradient cubes of the second, third, ... reader
+    std::vector<int> writers;          // producer and in-place layers, in order
+    int last_writer = -1;
+    bool params_upstream = false;      // a layer with weights lies at or above its producer
+    bool summed = false;               // reader gradients added up in the current backward pass
+  };
+  std::map<LayerT *, TensorInfo> blobs_;
+
+  // A reader's view of tensor `L`: the layer itself for the first reader; for every further reader
+  // the same data with a gradient cube of its own (the reference's Split: shared data, one
+  // gradient per output, src/DeepNet.h:1924-2028).
+  LayerT *consume(LayerT *L) {
+    TensorInfo &b = blobs_[L];
+    if (b.readers++ == 0) return L;
+    LayerT *v = new LayerT(new CubeT(L->p_data_cube->get_p_data(), L->dR, L->dC, L->dD, batch_),
+                           new CubeT(L->dR, L->dC, L->dD, batch_, &driver_));
+    layers_.push_back(v);
+    b.extra_grads.push_back(v->p_gradient_cube);
+    return v;
+  }
+  // gradient of `L` = first reader's + second reader's + ... (ascending, fp32), once per backward pass
+  void sum_reader_gradients(LayerT *L) {
+    TensorInfo &b = blobs_[L];
+    if (b.summed) return;
+    b.summed = true;
+    DeviceMemoryPointer total = L->p_gradient_cube->get_device_pointer(&driver_);
+    for (CubeT *e : b.extra_grads) {
+      DeviceMemoryPointer part = e->get_device_pointer(&driver_);
+      driver_.math_saxpy(1.0f, &part, &total);
+    }
+  }
+  // CONCAT: bottoms -> channel slices of the output (data, forward) or back (gradient, backward)
+  void concat_copy(Node &nd, bool data) {
+    size_t d_off = 0;
+    for (LayerT *b : nd.ins) {
+      CubeT *part = data ? b->p_data_cube : b->p_gradient_cube;
+      CubeT *whole = data ? nd.out->p_data_cube : nd.out->p_gradient_cube;
+      const int rc_ = cct_hip_copy_depth_slice(part->get_p_data(), whole->get_p_data(), (int)part->B, (int)whole->D,
+                                               (int)d_off, (int)part->D, part->R * part->C, data ? 0 : 1);
+      if (rc_) fail(cct_hip_last_error());
+      d_off += part->D;
+    }
+  }
 
   std::string io_error_;
   bool io_fail(const std::string &msg) {

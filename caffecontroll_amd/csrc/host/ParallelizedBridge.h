@@ -5,8 +5,20 @@
 // exactly one sub-bridge on the device that owns model, gradient and momentum
 // (skip_model_copy_gpu, _impl.hxx:117), input/output layers shared with the neighbouring
 // bridges in device memory, gradient update issued on the device (:993-995, :1057-1059).
-// The reference's batch partitioning over CPU threads / several GPUs, the host<->device copies
-// and the host gradient sum are not part of this build.
+// The reference's batch partitioning over CPU threads / several GPUs and the host gradient sum are
+// not part of this build.
+//
+// Where the layers live (src/bridges/ParallelizedBridge.h:183-198, _impl.hxx:109-117, 217-267,
+// 595-621, 686-705): by default the bridge shares device pointers with the bridges before and after
+// it -- its input and output layers ARE device memory and nothing is copied, which is what
+// DeepNet::construct_network arranges for consecutive device bridges.  With
+// share_pointer_with_prev_bridge == false the input layer's cubes are HOST memory: the bridge owns
+// device copies, uploads the input data at the start of forward() and downloads the input gradient
+// at the end of backward().  With share_pointer_with_next_bridge == false the same holds for the
+// output layer (data downloaded after forward(), gradient uploaded before backward()).  That is
+// the mode the reference's own bridge tests run in (tests/test_parallelized_convolution.cpp).
+// share_input_output_layer (ReLU, dropout: top == bottom) tells the bridge that its output layer
+// is its input layer, so no output cubes exist.
 #pragma once
 #include "AbstractBridge.h"
 #include "GradientUpdater.h"
@@ -33,8 +45,13 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
 
   ParallelizedBridge(LayerType *const _input_layer, LayerType *const _output_layer,
                      const cnn::LayerParameter *const _layer_param, const cnn::SolverParameter *const _solver_param,
-                     DriverClass *const _p_driver, size_t _n_partition = 1, size_t _n_thread_per_partition = 1)
+                     DriverClass *const _p_driver, size_t _n_partition = 1, size_t _n_thread_per_partition = 1,
+                     bool _share_pointer_with_prev_bridge = true, bool _share_pointer_with_next_bridge = true,
+                     bool _share_input_output_layer = false)
       : Base(_input_layer, _output_layer, _layer_param, _solver_param, _p_driver), n_partition(1),
+        share_pointer_with_prev_bridge(_share_pointer_with_prev_bridge),
+        share_pointer_with_next_bridge(_share_pointer_with_next_bridge),
+        share_input_output_layer(_share_input_output_layer),
         p_model_cube(nullptr), p_model_grad(nullptr), p_bias_cube(nullptr), p_bias_grad(nullptr),
         model_base_learning_rate(_layer_param->blobs_lr(0)), bias_base_learning_rate(_layer_param->blobs_lr(1)),
         model_base_regularization(_layer_param->weight_decay(0)),
@@ -46,7 +63,23 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
                            "(n_partition=1, gpu_0_batch_proportion=1.0)\n");
       std::abort();
     }
-    p_sub_bridge = new SubBridgeType(_input_layer, _output_layer, _layer_param, _solver_param, _p_driver);
+    // device-side layers of the sub-bridge: the caller's own, or copies this bridge owns
+    LayerType *sub_in = _input_layer, *sub_out = _output_layer;
+    if (!share_pointer_with_prev_bridge) {
+      p_device_input_layer = new LayerType(
+          new LogicalCubeType(_input_layer->dR, _input_layer->dC, _input_layer->dD, _input_layer->dB, _p_driver),
+          new LogicalCubeType(_input_layer->gR, _input_layer->gC, _input_layer->gD, _input_layer->gB, _p_driver));
+      sub_in = p_device_input_layer;
+    }
+    if (share_input_output_layer) {
+      sub_out = sub_in;
+    } else if (!share_pointer_with_next_bridge) {
+      p_device_output_layer = new LayerType(
+          new LogicalCubeType(_output_layer->dR, _output_layer->dC, _output_layer->dD, _output_layer->dB, _p_driver),
+          new LogicalCubeType(_output_layer->gR, _output_layer->gC, _output_layer->gD, _output_layer->gB, _p_driver));
+      sub_out = p_device_output_layer;
+    }
+    p_sub_bridge = new SubBridgeType(sub_in, sub_out, _layer_param, _solver_param, _p_driver);
     p_model_cube = p_sub_bridge->get_model_cube();
     p_model_grad = p_sub_bridge->get_model_grad_cube();
     p_bias_cube = p_sub_bridge->get_bias_cube();
@@ -65,6 +98,25 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
     delete p_grad_updater;
     delete p_grad_updater_bias;
     delete p_sub_bridge;
+    delete p_device_input_layer;
+    delete p_device_output_layer;
+  }
+
+  // src/bridges/ParallelizedBridge.h:183-198 (the first and third are fixed at construction, as in
+  // the reference; the second is set by the builder of the next bridge, src/DeepNet.h:1116-1120)
+  bool get_share_pointer_with_prev_bridge() const { return share_pointer_with_prev_bridge; }
+  bool get_share_pointer_with_next_bridge() const { return share_pointer_with_next_bridge; }
+  bool get_share_input_output_layer() const { return share_input_output_layer; }
+  void set_share_pointer_with_next_bridge(bool share) {
+    if (share == share_pointer_with_next_bridge) return;
+    if (p_device_output_layer || share_input_output_layer || !share) {
+      // going from shared to host-resident output after construction would need new device cubes
+      // under a sub-bridge that already holds the old ones
+      std::fprintf(stderr, "ParallelizedBridge: share_pointer_with_next_bridge can only be raised, and only "
+                           "before the bridge owns device output cubes\n");
+      std::abort();
+    }
+    share_pointer_with_next_bridge = share;
   }
 
   SubBridgeType *sub_bridge() { return p_sub_bridge; }
@@ -92,21 +144,37 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
 
   void forward() override {
     this->report_forward_history.reset();
+    if (p_device_input_layer) copy_cube(p_device_input_layer->p_data_cube, this->p_input_layer->p_data_cube, true);
     p_sub_bridge->forward();
+    if (p_device_output_layer) copy_cube(this->p_output_layer->p_data_cube, p_device_output_layer->p_data_cube, false);
     this->report_forward_history.end();
   }
 
   // sub-bridge backward, then the model and bias updates on the device
   void backward() override {
     this->report_backward_updateweight_history.reset();
+    if (p_device_output_layer)
+      copy_cube(p_device_output_layer->p_gradient_cube, this->p_output_layer->p_gradient_cube, true);
     p_sub_bridge->needs_to_calc_backward_grad = needs_to_calc_backward_grad;
     p_sub_bridge->backward();
+    if (p_device_input_layer && needs_to_calc_backward_grad)
+      copy_cube(this->p_input_layer->p_gradient_cube, p_device_input_layer->p_gradient_cube, false);
     if (p_grad_updater) p_grad_updater->update(p_model_grad->get_p_data());
     if (p_grad_updater_bias) p_grad_updater_bias->update(p_bias_grad->get_p_data());
     this->report_backward_updateweight_history.end();
   }
 
  private:
+  bool share_pointer_with_prev_bridge, share_pointer_with_next_bridge, share_input_output_layer;
+  LayerType *p_device_input_layer = nullptr, *p_device_output_layer = nullptr;
+  // host <-> device copy of a whole cube (synchronous, like the reference's driver memcpy)
+  void copy_cube(LogicalCubeType *dst, LogicalCubeType *src, bool to_device) {
+    DeviceMemoryPointer d = to_device ? dst->get_device_pointer(this->p_driver)
+                                      : DeviceMemoryPointer_Local_RAM(dst->get_p_data(), dst->n_elements * sizeof(DataType));
+    DeviceMemoryPointer s_ = to_device ? DeviceMemoryPointer_Local_RAM(src->get_p_data(), src->n_elements * sizeof(DataType))
+                                       : src->get_device_pointer(this->p_driver);
+    this->p_driver->memcpy(&d, &s_);
+  }
   SubBridgeType *p_sub_bridge;
   SGDGradientUpdater<DataType, DriverClass> *p_grad_updater;
   SGDGradientUpdater<DataType, DriverClass> *p_grad_updater_bias;

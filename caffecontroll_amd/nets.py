@@ -7,7 +7,8 @@ from . import _lib
 from ._lib import check
 from .bridges import SolverParam, solver_param  # noqa: F401
 
-CONV, FC, RELU, MAXPOOL, LRN, DROPOUT, SOFTMAXLOSS = 1, 2, 3, 4, 5, 6, 7
+CONV, FC, RELU, MAXPOOL, LRN, DROPOUT, SOFTMAXLOSS, CONCAT = 1, 2, 3, 4, 5, 6, 7, 8
+MAX_BOTTOMS = 4
 
 
 FILLER_TYPES = {"constant": 0, "xavier": 1, "gaussian": 2, "bernoulli": 3}
@@ -29,7 +30,18 @@ class LayerSpec(C.Structure):
                 ("pad", C.c_int), ("group", C.c_int), ("bias_term", C.c_int), ("lrn_local_size", C.c_int),
                 ("lrn_alpha", C.c_float), ("lrn_beta", C.c_float), ("dropout_ratio", C.c_float),
                 ("lr_mult", C.c_float * 2), ("decay_mult", C.c_float * 2),
-                ("weight_filler", Filler), ("bias_filler", Filler)]
+                ("weight_filler", Filler), ("bias_filler", Filler),
+                ("n_bottoms", C.c_int), ("bottoms", C.c_int * MAX_BOTTOMS)]
+
+    def read_from(self, *layer_indices):
+        """The layers whose outputs this layer reads (index in the layer list, -1 = the network
+        input); without it a layer reads the one before it.  Returns self."""
+        if not 1 <= len(layer_indices) <= MAX_BOTTOMS:
+            raise ValueError("a layer has 1..%d bottoms" % MAX_BOTTOMS)
+        self.n_bottoms = len(layer_indices)
+        for j, b in enumerate(layer_indices):
+            self.bottoms[j] = b
+        return self
 
 
 def _spec(t, **kw):
@@ -71,6 +83,11 @@ def dropout(ratio=0.5):
 
 def softmax_loss():
     return _spec(SOFTMAXLOSS)
+
+
+def concat(*layer_indices):
+    """Depth-wise concatenation of the outputs of the given layers."""
+    return _spec(CONCAT).read_from(*layer_indices)
 
 
 def lenet_layers():

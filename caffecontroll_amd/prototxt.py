@@ -21,8 +21,11 @@ Rules kept from the reference:
   * the reference prints a warning and ignores ``group`` (src/DeepNet.h:1075-1077); here
     ``groups="honor"`` (default) runs the grouped convolution the file asks for and
     ``groups="ignore"`` reproduces the reference.
-Networks with more than one consumer per blob (Split/Concat/Eltwise DAGs) and BatchNorm/Scale layers
-are outside this front end and are rejected with the layer's name in the message.
+  * a blob read by several layers needs no Split layer in the file (the reference inserts the split
+    itself, src/DeepNet.h:1924-2028); an explicit ``Split`` layer is accepted and only renames the
+    blob; ``Concat`` stacks its bottoms along the channel axis (src/DeepNet.h:1700-1757).
+Eltwise / BatchNorm / Scale layers are outside this front end and are rejected with the layer's name
+in the message.
 """
 import os
 import re
@@ -220,7 +223,12 @@ class NetworkDef:
     def output_shapes(self, depth, size):
         """[(depth, size)] after every layer for an input of `depth` channels and `size` x `size`."""
         out = []
-        for s in self.layers:
+        in_depth, in_size = depth, size
+        for i, s in enumerate(self.layers):
+            if s.n_bottoms:
+                depth, size = (in_depth, in_size) if s.bottoms[0] < 0 else out[s.bottoms[0]]
+            if s.type == nets.CONCAT:
+                depth = sum(in_depth if s.bottoms[j] < 0 else out[s.bottoms[j]][0] for j in range(s.n_bottoms))
             if s.type == nets.CONV:
                 size = (size + 2 * s.pad - s.kernel_size) // s.stride + 1
                 depth = s.num_output
@@ -317,7 +325,8 @@ def network_from_prototxt(text_or_message, phase="TRAIN", groups="honor"):
     if nd.batch_size <= 0:
         raise PrototxtError("data layer %r: batch_size must be positive" % d.get("name"))
 
-    current = tops[0]  # blob the chain has reached
+    writer = {tops[0]: -1}     # blob name -> index (in nd.layers) of the layer that wrote it last; -1 = the data layer
+    label_blobs = set(tops[1:])
     done_loss = False
     for l in layers:
         name, typ = l.get("name"), str(l.get("type", "")).upper()
@@ -329,28 +338,43 @@ def network_from_prototxt(text_or_message, phase="TRAIN", groups="honor"):
         bottoms, tops = l.all("bottom"), l.all("top")
         if done_loss:
             raise PrototxtError("layer %r follows the loss layer" % name)
+
+        def need(cond, what):
+            if not cond:
+                raise PrototxtError("layer %r: %s" % (name, what))
+
+        def source(blob):
+            need(blob in writer, "reads %r, which no earlier layer produces" % blob)
+            return writer[blob]
         if typ in ("SOFTMAXWITHLOSS", "SOFTMAX"):
-            if current not in bottoms:
-                raise PrototxtError("loss layer %r does not read %r, the end of the layer chain" % (name, current))
-            nd.layers.append(nets.softmax_loss())
+            data_bottoms = [b for b in bottoms if b not in label_blobs]
+            need(len(data_bottoms) == 1, "a loss layer reads one score blob and the labels")
+            nd.layers.append(nets.softmax_loss().read_from(source(data_bottoms[0])))
             nd.names.append(name)
             done_loss = True
             continue
+        if typ == "SPLIT":
+            # the reference inserts splits itself; an explicit one only gives the blob more names
+            need(len(bottoms) == 1 and tops, "a Split layer has one bottom and at least one top")
+            for t in tops:
+                writer[t] = source(bottoms[0])
+            continue
+        if typ == "CONCAT":
+            need(2 <= len(bottoms) <= nets.MAX_BOTTOMS and len(tops) == 1,
+                 "Concat takes 2..%d bottoms and one top" % nets.MAX_BOTTOMS)
+            c = l.msg("concat_param")
+            need(int(c.get("axis", c.get("concat_dim", 1))) == 1, "only concatenation along the channel axis is on this path")
+            nd.layers.append(nets.concat(*[source(b) for b in bottoms]))
+            nd.names.append(name)
+            writer[tops[0]] = len(nd.layers) - 1
+            continue
         if len(bottoms) != 1 or len(tops) != 1:
-            raise PrototxtError("layer %r (%s): only single-bottom, single-top layers form a chain"
-                                % (name, l.get("type")))
-        if bottoms[0] != current:
-            raise PrototxtError("layer %r reads %r but the chain is at %r: only sequential networks are "
-                                "supported" % (name, bottoms[0], current))
+            raise PrototxtError("layer %r (%s): one bottom and one top expected" % (name, l.get("type")))
         if tops[0] != name and tops[0] != bottoms[0]:
             raise PrototxtError("layer %r: the top must be the layer's name or its bottom (src/DeepNet.h:847-850)"
                                 % name)
         in_place = tops[0] == bottoms[0]
         lr, decay = _multipliers(l)
-
-        def need(cond, what):
-            if not cond:
-                raise PrototxtError("layer %r: %s" % (name, what))
         if typ == "CONVOLUTION":
             c = l.msg("convolution_param")
             if not c.has("num_output") or not c.has("kernel_size"):
@@ -398,9 +422,11 @@ def network_from_prototxt(text_or_message, phase="TRAIN", groups="honor"):
             raise PrototxtError("layer %r: type %r is not supported by this front end" % (name, l.get("type")))
         if in_place and typ not in ("RELU", "DROPOUT"):
             raise PrototxtError("layer %r (%s) cannot run in place" % (name, l.get("type")))
-        nd.layers.append(spec)
+        if not in_place and typ in ("RELU", "DROPOUT"):
+            raise PrototxtError("layer %r (%s) must run in place (top == bottom) on this path" % (name, l.get("type")))
+        nd.layers.append(spec.read_from(source(bottoms[0])))
         nd.names.append(name)
-        current = tops[0]
+        writer[tops[0]] = len(nd.layers) - 1
     if not done_loss:
         raise PrototxtError("the network has no SoftmaxWithLoss layer")
     return nd

@@ -50,6 +50,17 @@ typedef struct cct_conv_bridge cct_conv_bridge;
 int cct_conv_bridge_create(cct_conv_bridge **out, int b, int d, int n, const cct_conv_param *conv,
                            const cct_solver_param *solver, float *in_data, float *in_grad, float *out_data,
                            float *out_grad);
+/* The same with the reference's placement flags (src/bridges/ParallelizedBridge.h:183-198):
+ * share_pointer_with_prev_bridge == 0 means in_data / in_grad are HOST arrays -- the bridge owns
+ * device copies, uploads the input data in forward() and downloads the input gradient in
+ * backward(), as the reference's bridge does when the previous bridge is not on the same device
+ * (_impl.hxx:595-621, 686-705); share_pointer_with_next_bridge == 0 does the same for the output
+ * layer.  With both flags 0 the bridge runs on plain host tensors, which is how the reference's
+ * own bridge tests drive it (tests/test_parallelized_convolution.cpp:123-270). */
+int cct_conv_bridge_create_shared(cct_conv_bridge **out, int b, int d, int n, const cct_conv_param *conv,
+                                  const cct_solver_param *solver, float *in_data, float *in_grad, float *out_data,
+                                  float *out_grad, int share_pointer_with_prev_bridge,
+                                  int share_pointer_with_next_bridge);
 int cct_conv_bridge_destroy(cct_conv_bridge *h);
 /* fused: how much of the lowering pipeline is replaced.  0 = the reference's separate passes;
  * 1 = forward GEMM epilogue does remap + bias, bias gradient inside the lift launch; 2 = as 1 with
@@ -80,12 +91,15 @@ const char *cct_conv_bridge_stage_kernel(cct_conv_bridge *h, int stage);
 
 /* ---- a chain of layers (LeNet / CaffeNet style) --------------------------------------------
  * Stands for DeepNet::construct_network + run_forward_pass / run_backward_pass
- * (src/DeepNet.h:968-2030, 171-266) for nets that are a plain sequence of layers, with every
- * layer wrapped in a one-partition ParallelizedBridge on the device. */
+ * (src/DeepNet.h:968-2030, 171-266): layers in the order the prototxt lists them (a topological
+ * order), each reading the previous one or the layers its `bottoms` name, every layer wrapped in
+ * a one-partition ParallelizedBridge on the device. */
 enum cct_layer_type {
   CCT_LAYER_CONV = 1, CCT_LAYER_FC = 2, CCT_LAYER_RELU = 3, CCT_LAYER_MAXPOOL = 4, CCT_LAYER_LRN = 5,
-  CCT_LAYER_DROPOUT = 6, CCT_LAYER_SOFTMAXLOSS = 7
+  CCT_LAYER_DROPOUT = 6, CCT_LAYER_SOFTMAXLOSS = 7,
+  CCT_LAYER_CONCAT = 8 /* depth-wise concatenation of 2..CCT_MAX_BOTTOMS bottoms (src/DeepNet.h:1700-1757) */
 };
+#define CCT_MAX_BOTTOMS 4
 
 /* cnn::FillerParameter (src/parser/cnn.proto:21-32).  A zeroed struct is the proto default for
  * type and value ("constant", 0); set std explicitly for a gaussian filler (proto default 1). */
@@ -109,6 +123,14 @@ typedef struct cct_layer_spec {
   float lr_mult[2];         /* weights, bias */
   float decay_mult[2];
   cct_filler weight_filler, bias_filler; /* conv, fc; random fillers draw from solver.random_seed */
+  /* Where the layer reads from.  n_bottoms == 0: the output of the previous layer in the array (the
+   * network input for layer 0) -- a plain chain.  Otherwise bottoms[j] is the index of the layer
+   * whose output is read, or -1 for the network input; every layer but CONCAT has one bottom.  A
+   * layer output read by several layers is the reference's Split (src/DeepNet.h:1924-2028): the
+   * readers share the data, each writes a gradient of its own, and the gradients are added up, in
+   * reader order, before the producer's backward step. */
+  int n_bottoms;
+  int bottoms[CCT_MAX_BOTTOMS];
 } cct_layer_spec;
 
 typedef struct cct_net cct_net;

@@ -6,7 +6,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 import numpy as np
 
-CONV, FC, RELU, MAXPOOL, LRN, DROPOUT, SOFTMAXLOSS = 1, 2, 3, 4, 5, 6, 7
+CONV, FC, RELU, MAXPOOL, LRN, DROPOUT, SOFTMAXLOSS, CONCAT = 1, 2, 3, 4, 5, 6, 7, 8
 
 
 class OracleNet:
@@ -174,3 +174,178 @@ class OracleNet:
         p["w"] = w.reshape(p["w"].shape)
         self.O.sgd_update(p["b"], db, p["hb"], s["base_lr"] * L.lr_mult[1], s["momentum"],
                           s["weight_decay"] * L.decay_mult[1])
+
+
+class OracleGraph:
+    """The same for layers that name their bottoms (`LayerSpec.read_from`): a tensor read by several
+    layers is shared, each reader's gradient is kept apart and the gradients are added in reader
+    order before the tensor's last writer runs its backward step (the reference's Split bridge,
+    src/DeepNet.h:1924-2028); CONCAT stacks its bottoms along the depth (src/DeepNet.h:1700-1757).
+    A layer computes an input gradient only if a layer with weights lies upstream of it."""
+
+    def __init__(self, O, layers, batch, depth, size, solver):
+        self.O, self.layers, self.solver = O, layers, solver
+        n = len(layers)
+        self.bottoms = [[L.bottoms[j] for j in range(L.n_bottoms)] if L.n_bottoms else [i - 1] for i, L in enumerate(layers)]
+        self.in_place = [L.type in (RELU, DROPOUT) for L in layers]
+        # the tensor a layer writes: its own, or its bottom's for an in-place layer (-1 = the input)
+        self.blob = []
+        for i in range(n):
+            self.blob.append(self._blob_of(self.bottoms[i][0]) if self.in_place[i] else i)
+        shape = {-1: (depth, size)}
+        self.params, self.upstream = {}, {-1: False}
+        for i, L in enumerate(layers):
+            d, s = shape[self._blob_of(self.bottoms[i][0])]
+            up = any(self.upstream[self._blob_of(b)] for b in self.bottoms[i])
+            if L.type == CONV:
+                g = max(L.group, 1)
+                for gi in range(g):
+                    self.params[(i, gi)] = dict(w=np.zeros((L.num_output // g, d // g, L.kernel_size, L.kernel_size), np.float32),
+                                                b=np.zeros(L.num_output // g, np.float32))
+                s = (s + 2 * L.pad - L.kernel_size) // L.stride + 1
+                d = L.num_output
+            elif L.type == FC:
+                self.params[(i, 0)] = dict(w=np.zeros((L.num_output, d * s * s), np.float32), b=np.zeros(L.num_output, np.float32))
+                d, s = L.num_output, 1
+            elif L.type == MAXPOOL:
+                s = (s - L.kernel_size) // L.stride + 1
+            elif L.type == CONCAT:
+                d = sum(shape[self._blob_of(b)][0] for b in self.bottoms[i])
+            shape[self.blob[i]] = (d, s)
+            self.upstream[self.blob[i]] = self.upstream.get(self.blob[i], False) or up or L.type in (CONV, FC)
+        self.needs_in_grad = [any(self._up_before(i, b) for b in self.bottoms[i]) for i in range(n)]
+        for p in self.params.values():
+            p["hw"] = np.zeros(p["w"].size, np.float32)
+            p["hb"] = np.zeros(p["b"].size, np.float32)
+        self.masks = {}
+
+    def _blob_of(self, layer_index):
+        return -1 if layer_index < 0 else self.blob[layer_index]
+
+    def _up_before(self, i, b):
+        """True if a layer with weights lies at or above the producer of bottom `b` of layer `i`."""
+        seen, todo = set(), [b]
+        while todo:
+            j = todo.pop()
+            if j < 0 or j in seen:
+                continue
+            seen.add(j)
+            if self.layers[j].type in (CONV, FC):
+                return True
+            todo.extend(self.bottoms[j])
+        return False
+
+    def forward(self, x, labels):
+        O = self.O
+        self.val = {-1: x}      # tensor -> current values (in-place layers replace them)
+        self.out = {}           # layer -> what it wrote (for comparisons)
+        self.saved = {}
+        for i, L in enumerate(self.layers):
+            ins = [self.val[self._blob_of(b)] for b in self.bottoms[i]]
+            cur = ins[0]
+            if L.type == CONV:
+                g = max(L.group, 1)
+                dg = cur.shape[1] // g
+                outs = []
+                for gi in range(g):
+                    p = self.params[(i, gi)]
+                    xin = np.ascontiguousarray(cur[:, gi * dg:(gi + 1) * dg])
+                    out, low = O.conv_forward(xin, p["w"], p["b"], L.kernel_size, L.stride, L.pad)
+                    self.saved[(i, gi)] = (xin.shape, low)
+                    outs.append(out)
+                res = np.concatenate(outs, axis=1) if g > 1 else outs[0]
+            elif L.type == FC:
+                p = self.params[(i, 0)]
+                self.saved[(i, 0)] = cur.reshape(cur.shape[0], -1).copy()
+                self.saved[(i, "shape")] = cur.shape
+                res = O.fc_forward(self.saved[(i, 0)], p["w"], p["b"]).reshape(cur.shape[0], L.num_output, 1, 1)
+            elif L.type == RELU:
+                res = O.relu_forward(cur)
+            elif L.type == MAXPOOL:
+                self.saved[i] = cur.shape
+                res, idx = O.maxpool_forward(cur, L.kernel_size, L.stride)
+                self.saved[(i, "idx")] = idx
+            elif L.type == LRN:
+                self.saved[i] = cur
+                res, den = O.lrn_forward(cur, L.lrn_local_size, L.lrn_alpha, L.lrn_beta)
+                self.saved[(i, "den")] = den
+            elif L.type == DROPOUT:
+                res = O.dropout_forward(cur, self.masks[i], L.dropout_ratio, threshold=True)
+            elif L.type == CONCAT:
+                self.saved[i] = [a.shape[1] for a in ins]
+                res = np.concatenate(ins, axis=1)
+            elif L.type == SOFTMAXLOSS:
+                res, self.loss = O.softmax_loss_forward(cur, labels)
+                self.labels = labels
+            self.val[self.blob[i]] = res
+            self.out[i] = res
+        return res
+
+    def backward(self):
+        O = self.O
+        n = len(self.layers)
+        contrib = {}            # tensor -> {reader layer: gradient}
+        total = {}              # tensor -> gradient after the readers were added up
+        self.grads, self.tensor_grads = {}, {}
+
+        def grad_of(blob):
+            if blob not in total:
+                parts = contrib.get(blob, {})
+                g = None
+                for reader in sorted(parts):      # reader order, fp32 adds
+                    g = parts[reader].copy() if g is None else g + parts[reader]
+                total[blob] = g
+            return total[blob]
+
+        for i in range(n - 1, -1, -1):
+            L = self.layers[i]
+            blob = self.blob[i]
+            bots = [self._blob_of(b) for b in self.bottoms[i]]
+            need = self.needs_in_grad[i]
+            if L.type == SOFTMAXLOSS:
+                contrib.setdefault(bots[0], {})[i] = O.softmax_loss_backward(self.out[i], self.labels)
+                continue
+            g = grad_of(blob)
+            if g is None:
+                continue        # nothing with weights upstream and none here
+            if L.type == RELU:
+                total[blob] = O.relu_backward(g, self.val[blob])
+            elif L.type == DROPOUT:
+                total[blob] = O.dropout_forward(g, self.masks[i], L.dropout_ratio, threshold=True)
+            elif L.type == MAXPOOL:
+                shp = self.saved[i]
+                if need:
+                    contrib.setdefault(bots[0], {})[i] = O.maxpool_backward(g, self.saved[(i, "idx")], shp[2], shp[3])
+            elif L.type == LRN:
+                if need:
+                    contrib.setdefault(bots[0], {})[i] = O.lrn_backward(g, self.saved[i], self.saved[(i, "den")],
+                                                                          L.lrn_local_size, L.lrn_alpha, L.lrn_beta)
+            elif L.type == CONCAT:
+                off = 0
+                for b, d in zip(bots, self.saved[i]):
+                    contrib.setdefault(b, {})[i] = np.ascontiguousarray(g[:, off:off + d])
+                    off += d
+            elif L.type == FC:
+                p = self.params[(i, 0)]
+                dx, dw, db = O.fc_backward(self.saved[(i, 0)], p["w"], g.reshape(g.shape[0], -1), need_in_grad=need)
+                self.grads[(i, 0)] = (dw.copy(), db.copy())
+                self._update(p, L, dw, db)
+                if need:
+                    contrib.setdefault(bots[0], {})[i] = dx.reshape(self.saved[(i, "shape")])
+            elif L.type == CONV:
+                gn = max(L.group, 1)
+                og_d = g.shape[1] // gn
+                dxs = []
+                for gi in range(gn):
+                    p = self.params[(i, gi)]
+                    shp, low = self.saved[(i, gi)]
+                    og = np.ascontiguousarray(g[:, gi * og_d:(gi + 1) * og_d])
+                    dx, dw, db = O.conv_backward(shp, p["w"], og, low, L.kernel_size, L.stride, L.pad, need_in_grad=need)
+                    self.grads[(i, gi)] = (dw.copy(), db.copy())
+                    self._update(p, L, dw, db)
+                    dxs.append(dx)
+                if need:
+                    contrib.setdefault(bots[0], {})[i] = np.concatenate(dxs, axis=1) if gn > 1 else dxs[0]
+        self.tensor_grads = dict(total)
+
+    _update = OracleNet._update

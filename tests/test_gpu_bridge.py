@@ -194,3 +194,39 @@ def test_stepped_sgd_follows_the_schedule_bit_for_bit(oracle, policy, l1):
     if name != "fixed":
         assert len(set(rates)) > 2, rates   # the schedule moved during the run, so it was exercised
     layer.close()
+
+
+@pytest.mark.parametrize("share", [(False, False), (False, True), (True, False)], ids=["host-host", "host-dev", "dev-host"])
+def test_pbridge_on_host_layers_like_the_reference_tests(share):
+    """share_pointer_with_prev/next_bridge = false (src/bridges/ParallelizedBridge.h:183-198): the
+    layer on that side is host memory and the bridge moves it to and from its own device cubes.  The
+    reference's golden scenario (tests/test_parallelized_convolution.cpp:123-270) run on plain host
+    arrays, as the reference test itself does, and the mixed placements against it."""
+    from caffecontroll_amd.bridges import ConvolutionLayer, solver_param
+    share_prev, share_next = share
+    c = FIX["small"]
+    b, d, n, k, s, p, o = (c[x] for x in ("b", "d", "n", "k", "s", "p", "o"))
+    m = (n + 2 * p - k) // s + 1
+    driver()
+    x = load_fixture("input", "conv_forward_in.txt").reshape(b, d, n, n)
+    og = (np.arange(b * o * m * m, dtype=np.float64) * 0.1).astype(np.float32).reshape(b, o, m, m)
+    in_data = dev(x) if share_prev else x.copy()
+    in_grad = empty((b, d, n, n)) if share_prev else np.full((b, d, n, n), np.nan, np.float32)
+    out_data = empty((b, o, m, m)) if share_next else np.full((b, o, m, m), np.nan, np.float32)
+    out_grad = dev(og) if share_next else og.copy()
+    layer = ConvolutionLayer(b, d, n, k, s, p, o, in_data, in_grad, out_data, out_grad,
+                             solver=solver_param(base_lr=0.01, momentum=0.0, lr_policy="step", stepsize=10000),
+                             share_prev=share_prev, share_next=share_next)
+    as_host = lambda t: host(t) if hasattr(t, "data_ptr") else t
+    _copy_to(layer.model_ptr(), load_fixture("input", "conv_model.txt"))
+    _copy_to(layer.bias_ptr(), load_fixture("input", "conv_bias_in.txt"))
+    layer.forward()
+    np.testing.assert_allclose(as_host(out_data).reshape(-1), load_fixture("output", "conv_forward.txt"), rtol=2e-5, atol=1e-3)
+    _copy_to(layer.model_ptr(), load_fixture("input", "conv_backward_model.txt"))
+    layer.forward()
+    layer.backward(with_update=True)
+    np.testing.assert_allclose(as_host(in_grad).reshape(-1), load_fixture("output", "conv_backward.txt"), rtol=1e-4, atol=1e-3)
+    np.testing.assert_allclose(_read(layer.model_ptr(), (o * d * k * k,)), load_fixture("output", "conv_weights.txt"),
+                               rtol=1e-4, atol=1e-3)
+    np.testing.assert_allclose(_read(layer.bias_ptr(), (o,)), load_fixture("output", "conv_bias.txt"), rtol=1e-4, atol=1e-3)
+    layer.close()

@@ -199,3 +199,84 @@ def test_training_loop_learns_and_reports(tmp_path):
     with pytest.raises(ValueError):
         S.upload_batch(net, np.zeros((8, 2, 9, 9), np.float32), np.zeros(8))
     net.close()
+
+
+TOWER_TEXT = """
+name: "towers"
+layer { name: "data" type: "Data" top: "data" top: "label" data_param { source: "none" batch_size: 6 } }
+layer { name: "conv1" type: "Convolution" bottom: "data" top: "conv1" param { lr_mult: 1 } param { lr_mult: 2 decay_mult: 0 }
+        convolution_param { num_output: 8 kernel_size: 3 pad: 1 weight_filler { type: "gaussian" std: 0.2 }
+                            bias_filler { type: "constant" value: 0.1 } } }
+layer { name: "relu1" type: "ReLU" bottom: "conv1" top: "conv1" }
+layer { name: "pool1" type: "Pooling" bottom: "conv1" top: "pool1" pooling_param { pool: MAX kernel_size: 2 stride: 2 } }
+layer { name: "norm1" type: "LRN" bottom: "pool1" top: "norm1" lrn_param { local_size: 3 alpha: 0.01 beta: 0.75 } }
+layer { name: "conv2" type: "Convolution" bottom: "norm1" top: "conv2"
+        convolution_param { num_output: 6 kernel_size: 3 pad: 1 weight_filler { type: "xavier" } } }
+layer { name: "relu2" type: "ReLU" bottom: "conv2" top: "conv2" }
+layer { name: "pool2" type: "Pooling" bottom: "conv2" top: "pool2" pooling_param { pool: MAX kernel_size: 2 stride: 2 } }
+layer { name: "conv2b" type: "Convolution" bottom: "norm1" top: "conv2b"
+        convolution_param { num_output: 10 kernel_size: 3 pad: 1 group: 2 weight_filler { type: "xavier" } } }
+layer { name: "relu2b" type: "ReLU" bottom: "conv2b" top: "conv2b" }
+layer { name: "pool2b" type: "Pooling" bottom: "conv2b" top: "pool2b" pooling_param { pool: MAX kernel_size: 2 stride: 2 } }
+layer { name: "concat" type: "Concat" bottom: "pool2" bottom: "pool2b" top: "concat" }
+layer { name: "fc6" type: "InnerProduct" bottom: "concat" top: "fc6"
+        inner_product_param { num_output: 16 weight_filler { type: "gaussian" std: 0.1 } bias_filler { type: "constant" value: 0.05 } } }
+layer { name: "relu6" type: "ReLU" bottom: "fc6" top: "fc6" }
+layer { name: "fc8" type: "InnerProduct" bottom: "fc6" top: "fc8" inner_product_param { num_output: 5 weight_filler { type: "xavier" } } }
+layer { name: "loss" type: "SoftmaxWithLoss" bottom: "fc8" bottom: "label" top: "loss" }
+"""
+TOWER_SOLVER = 'base_lr: 0.05 momentum: 0.9 weight_decay: 0.001 lr_policy: "fixed" max_iter: 4 random_seed: 11'
+
+
+@pytest.mark.parametrize("text, solver_text, depth, size", [(NET_TEXT, 'base_lr: 0.05 momentum: 0.9 weight_decay: 0.0005 lr_policy: "fixed" random_seed: 77', 2, 10),
+                                                            (TOWER_TEXT, TOWER_SOLVER, 3, 12)], ids=["chain", "two-towers"])
+def test_prototxt_network_trains_like_the_oracle(oracle, text, solver_text, depth, size):
+    """From configuration text to trained weights, against the oracle: the network the front end
+    builds (fillers, multipliers, groups, a blob read by two towers, Concat) is run for three
+    iterations on the device and by the oracle graph on the same filler-drawn weights; every
+    layer's output, every gradient and every updated weight agree within 1e-4."""
+    from caffecontroll_amd import nets, prototxt as P
+    from gpu_util import rel_err
+    from oracle_net import OracleGraph
+    sp, _ = P.solver_from_prototxt(solver_text)
+    nd = P.network_from_prototxt(text)
+    driver()
+    net = nd.build(depth=depth, size=size, solver=sp)
+    layers, B = nd.layers, nd.batch_size
+    solver = dict(base_lr=sp.base_lr, momentum=sp.momentum, weight_decay=sp.weight_decay)
+    ref = OracleGraph(oracle, layers, B, depth, size, solver)
+    for (li, gi), p in ref.params.items():          # the weights the device drew with the prototxt's fillers
+        p["w"][...] = _down(*net.tensor(li, nets.MODEL, gi)).reshape(p["w"].shape)
+        p["b"][...] = _down(*net.tensor(li, nets.BIAS, gi))
+        assert np.abs(p["w"]).max() > 0
+    classes = ref.params[max(ref.params)]["b"].size
+    rng = np.random.default_rng(21)
+    up = lambda ptr, a: driver().memcpy(ptr, np.ascontiguousarray(a).ctypes.data, a.nbytes, 0)
+    for it in range(3):
+        x = rng.standard_normal((B, depth, size, size)).astype(np.float32)
+        labels = rng.integers(0, classes, B).astype(np.float32)
+        up(net.input_ptr(), x)
+        up(net.labels_ptr(), labels)
+        net.forward()
+        ref.forward(x, labels)
+        for li, L in enumerate(layers):
+            if L.type in (nets.RELU, nets.DROPOUT):
+                continue
+            want = ref.val[ref.blob[li]] if li != len(layers) - 1 else ref.out[li]
+            assert rel_err(_down(*net.tensor(li, nets.OUTPUT)), want.reshape(-1)) <= 1e-4, (it, nd.names[li])
+            if L.type == nets.MAXPOOL:
+                ptr, n = net.tensor(li, nets.AUX)
+                want = ref.saved[(li, "idx")].reshape(-1).astype(np.int32)
+                got = np.empty(n, np.int32)
+                driver().memcpy(got.ctypes.data, ptr, got.nbytes, 1)
+                assert np.count_nonzero(got != want) <= 1
+                up(ptr, want)
+        assert abs(net.loss() - ref.loss) <= 1e-4 * max(1.0, abs(ref.loss))
+        net.backward()
+        ref.backward()
+        for (li, gi), p in sorted(ref.params.items()):
+            for which, key in ((nets.MODEL, "w"), (nets.BIAS, "b")):
+                assert rel_err(_down(*net.tensor(li, which, gi)), p[key].reshape(-1)) <= 1e-4, (it, nd.names[li], key)
+            for which, hist in ((nets.MODEL_HISTORY, "hw"), (nets.BIAS_HISTORY, "hb")):
+                assert rel_err(_down(*net.tensor(li, which, gi)), p[hist]) <= 1e-4, (it, nd.names[li], hist)
+    net.close()

@@ -105,11 +105,40 @@ def test_network_mapping():
     assert t.batch_size == 3 and t.scale == 0.5 and t.crop_size == 0 and t.names == nd.names
 
 
+def test_graph_mapping():
+    """A blob read by two layers (the reference inserts the Split itself), an explicit Split, and
+    Concat: every layer names the index of the layer that last wrote its bottom."""
+    # ip1 now reads conv1 (after its in-place ReLU) next to pool1
+    nd = P.network_from_prototxt(NET.replace('bottom: "norm1" top: "ip1"', 'bottom: "conv1" top: "ip1"'))
+    bottoms = [[s.bottoms[j] for j in range(s.n_bottoms)] for s in nd.layers]
+    assert bottoms == [[-1], [0], [1], [2], [1], [4], [5]]
+    two = """
+    layer { name: "data" type: "Data" top: "data" top: "label" data_param { batch_size: 2 } transform_param { crop_size: 12 } }
+    layer { name: "c1" type: "Convolution" bottom: "data" top: "c1" convolution_param { num_output: 4 kernel_size: 3 } }
+    layer { name: "sp" type: "Split" bottom: "c1" top: "c1_a" top: "c1_b" }
+    layer { name: "a" type: "Convolution" bottom: "c1_a" top: "a" convolution_param { num_output: 3 kernel_size: 3 } }
+    layer { name: "b" type: "Convolution" bottom: "c1_b" top: "b" convolution_param { num_output: 5 kernel_size: 3 } }
+    layer { name: "cat" type: "Concat" bottom: "a" bottom: "b" top: "cat" }
+    layer { name: "ip" type: "InnerProduct" bottom: "cat" top: "ip" inner_product_param { num_output: 2 } }
+    layer { name: "loss" type: "SoftmaxWithLoss" bottom: "ip" bottom: "label" }
+    """
+    nd = P.network_from_prototxt(two)
+    assert nd.names == ["c1", "a", "b", "cat", "ip", "loss"]
+    assert [s.type for s in nd.layers] == [nets.CONV, nets.CONV, nets.CONV, nets.CONCAT, nets.FC, nets.SOFTMAXLOSS]
+    assert [[s.bottoms[j] for j in range(s.n_bottoms)] for s in nd.layers] == [[-1], [0], [0], [1, 2], [3], [4]]
+    assert nd.output_shapes(3, 12) == [(4, 10), (3, 8), (5, 8), (8, 8), (2, 1), (2, 1)]
+    nd.validate(3)
+    with pytest.raises(P.PrototxtError, match="channel axis"):
+        P.network_from_prototxt(two.replace('top: "cat" }', 'top: "cat" concat_param { axis: 2 } }'))
+    with pytest.raises(P.PrototxtError, match="'cat'"):
+        P.network_from_prototxt(two.replace("num_output: 5 kernel_size: 3", "num_output: 5 kernel_size: 5")).validate(3)
+
+
 def test_rejected_networks():
     with pytest.raises(P.PrototxtError, match="BatchNorm"):
         P.network_from_prototxt(NET.replace('type: "LRN"', 'type: "BatchNorm"'))
-    with pytest.raises(P.PrototxtError, match="sequential"):
-        P.network_from_prototxt(NET.replace('bottom: "norm1" top: "ip1"', 'bottom: "conv1" top: "ip1"'))
+    with pytest.raises(P.PrototxtError, match="no earlier layer produces"):
+        P.network_from_prototxt(NET.replace('bottom: "norm1" top: "ip1"', 'bottom: "nowhere" top: "ip1"'))
     with pytest.raises(P.PrototxtError, match="no SoftmaxWithLoss"):
         P.network_from_prototxt(NET[:NET.index('layer { name: "loss"')])
     with pytest.raises(P.PrototxtError, match="Data layer"):
@@ -160,6 +189,14 @@ def test_reference_imagenet_files():
         assert [(tuple(s.lr_mult), tuple(s.decay_mult)) for s in convs] == [((1.0, 2.0), (1.0, 0.0))] * 5
         assert all(s.weight_filler.type == nets.FILLER_TYPES["gaussian"] for s in convs)
         assert nd.output_shapes(3, 227)[-1] == (1000, 1)
+    # the reference's two-tower network (a blob read by two towers, Concat before fc6)
+    nd = P.network_from_prototxt(P.parse_file(REF + "/benchmark/train_val/caffenet_train_val_8_split.prototxt"))
+    assert [s.type for s in nd.layers].count(nets.CONV) == 9 and nets.CONCAT in [s.type for s in nd.layers]
+    norm1 = nd.names.index("norm1")
+    readers = [nd.names[i] for i, s in enumerate(nd.layers) if norm1 in [s.bottoms[j] for j in range(s.n_bottoms)]]
+    assert readers == ["conv2", "conv2b"]
+    nd.validate(3, 227)
+    assert nd.output_shapes(3, 227)[nd.names.index("concat")] == (256, 6)
     # every solver file of the reference's tests resolves to a network this front end accepts
     import glob
     for f in glob.glob(base + "*.prototxt") + glob.glob(REF + "/tests/lenet_train/*solver*.prototxt"):
