@@ -132,6 +132,20 @@ class HIPDriver:
         check(self.lib.cct_hip_conv_direct_slabs(_p(slabs), _p(model), o, d, k, int(for_data_gradient)),
               "conv_direct_slabs")
 
+    # -- strided convolution without the lowered matrix ------------------------------------------
+    def conv_strided_supported(self, b, d, n, k, s, p, o):
+        return bool(self.lib.cct_hip_conv_strided_supported(b, d, n, k, s, p, o))
+
+    def conv_strided_slab_floats(self, o, d, k, s, p):
+        return int(self.lib.cct_hip_conv_strided_slab_floats(o, d, k, s, p))
+
+    def conv_strided_slabs(self, slabs, model, o, d, k, s, p):
+        check(self.lib.cct_hip_conv_strided_slabs(_p(slabs), _p(model), o, d, k, s, p), "conv_strided_slabs")
+
+    def conv_strided_forward(self, out, inp, slabs, bias, b, d, n, k, s, p, o, relu=False):
+        check(self.lib.cct_hip_conv_strided_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, s, p, o,
+                                                    int(relu)), "conv_strided_forward")
+
     def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o, in_stride=0, out_stride=0, relu=False):
         check(self.lib.cct_hip_conv_direct_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o,
                                                    in_stride, out_stride, int(relu)), "conv_direct_forward")

@@ -228,6 +228,29 @@ int cct_hip_conv_direct_backward_data_relu(float *input_grad, const float *outpu
 int cct_hip_conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                          const float *input, int batch, int depth, int n, int k, int padding,
                                          int num_outputs, size_t input_image_stride, size_t output_image_stride);
+/* ---- strided convolution without the lowered matrix ---------------------------------------- */
+/* The same replacement of ConvolutionBridge's lowering pipeline for strided layers: stride 4 with an
+ * 11 x 11 kernel (AlexNet / CaffeNet conv1, benchmark configuration 3; the reference's "large" golden
+ * scenario, tests/test_parallelized_convolution_large_CPU.cpp:71-80) and stride 2 with 7 x 7,
+ * 5 x 5 or 3 x 3 kernels.  cct_hip_conv_strided_supported: 1 if the geometry is covered, else 0. */
+int cct_hip_conv_strided_supported(int batch, int depth, int n, int k, int stride, int padding,
+                                   int num_outputs);
+/* Re-lays the model [o][d][k][k] for cct_hip_conv_strided_forward, zero padded: for a layer with
+ * padding as [d][k rounded up to even][o padded to whole tiles][k+1 (+1)], for a layer without as
+ * [d][pairs of tap rows][o padded to whole tiles][2k (+1)] (the two forward kernels read their
+ * weights in different orders, so `padding` must be the layer's own); `slabs` holds
+ * cct_hip_conv_strided_slab_floats() floats (0 if the kernel size / stride pair is not covered)
+ * and is 16-byte aligned. */
+size_t cct_hip_conv_strided_slab_floats(int num_outputs, int depth, int k, int stride, int padding);
+int cct_hip_conv_strided_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
+                               int stride, int padding);
+/* lower_cube + forward GEMM + remap_output + bias of ConvolutionBridge::forward
+ * (src/bridges/ConvolutionBridge_impl.hxx:316-364) in one kernel: output[b][o][m][m],
+ * m = (n + 2*padding - k) / stride + 1, from input[b][d][n][n], the slabs and bias[o] (may be NULL);
+ * relu != 0 folds a following in-place ReLU into the store. */
+int cct_hip_conv_strided_forward(float *output, const float *input, const float *slabs, const float *bias,
+                                 int batch, int depth, int n, int k, int stride, int padding,
+                                 int num_outputs, int relu);
 /* DeviceDriver::sgemv (src/sched/DeviceDriver.h:214-215): row-major M x N, lda = N. */
 int cct_hip_sgemv(int TA, int M, int N, float alpha, const float *A, const float *x, float beta,
                   float *y);

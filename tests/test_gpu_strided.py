@@ -1,0 +1,104 @@
+"""Strided convolution on the matrix cores without the lowered matrix (AlexNet / CaffeNet conv1:
+11x11, stride 4; stride-2 layers with 7x7, 5x5 and 3x3 kernels) against the oracle's lowering
+pipeline (lower_cube + GEMM + remap + bias, src/bridges/ConvolutionBridge_impl.hxx:316-364), the
+reference's "large" golden scenario, and -- at the full size of benchmark configuration 3 -- float64
+torch.  The sums run in another order than the lowered GEMM: agreement to 1e-4 of the tensor's
+largest magnitude, bit-exact on small-integer tensors."""
+import numpy as np
+import pytest
+
+from conftest import load_fixture
+from gpu_util import dev, driver, empty, host, rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+# (b, d, n, k, s, p, o)
+SHAPES = [
+    (4, 3, 127, 11, 4, 2, 8),      # the reference's large fixture
+    (3, 3, 227, 11, 4, 0, 96),     # conv1 geometry, small batch: tiles that straddle two images
+    (2, 3, 51, 11, 4, 0, 40),      # two map blocks with padding maps
+    (5, 2, 35, 11, 4, 5, 33),      # heavy padding, odd sizes
+    (2, 4, 30, 7, 2, 3, 20),       # stride 2
+    (3, 5, 17, 5, 2, 2, 64),
+    (4, 6, 13, 3, 2, 1, 70),
+    (1, 1, 11, 11, 4, 0, 1),       # a single output pixel
+    (2, 4, 31, 7, 2, 0, 20),       # no padding: the lanes fetch the source themselves
+    (3, 5, 17, 5, 2, 0, 64),
+    (4, 6, 13, 3, 2, 0, 70),
+    (2, 1, 43, 11, 4, 0, 97),      # one channel, four map blocks
+]
+_ids = lambda s: "b%d_d%d_n%d_k%d_s%d_p%d_o%d" % s
+
+
+def _forward(drv, x, w, bias, shape, relu=False):
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
+    slabs = empty((drv.conv_strided_slab_floats(o, d, k, s, p),))
+    drv.conv_strided_slabs(slabs, dev(w), o, d, k, s, p)
+    out = empty((b, o, m, m))
+    drv.conv_strided_forward(out, dev(x), slabs, None if bias is None else dev(bias), b, d, n, k, s, p, o, relu=relu)
+    return host(out)
+
+
+@pytest.mark.parametrize("shape", SHAPES, ids=_ids)
+def test_strided_forward_vs_oracle(oracle, shape):
+    b, d, n, k, s, p, o = shape
+    drv = driver()
+    assert drv.conv_strided_supported(*shape)
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+    w = (rng.standard_normal((o, d, k, k)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(o).astype(np.float32)
+    ref, _ = oracle.conv_forward(x, w, bias, k, s, p)
+    got = _forward(drv, x, w, bias, shape)
+    assert rel_err(got, ref) <= TOL
+    # without bias, with the ReLU of a following layer folded in
+    ref0, _ = oracle.conv_forward(x, w, None, k, s, p)
+    got0 = _forward(drv, x, w, None, shape, relu=True)
+    assert rel_err(got0, np.maximum(ref0, 0)) <= TOL
+    # small integers: every product and partial sum is exact, whatever the order
+    xi = rng.integers(-4, 5, size=x.shape).astype(np.float32)
+    wi = rng.integers(-3, 4, size=w.shape).astype(np.float32)
+    bi = rng.integers(-5, 6, size=o).astype(np.float32)
+    refi, _ = oracle.conv_forward(xi, wi, bi, k, s, p)
+    np.testing.assert_array_equal(_forward(drv, xi, wi, bi, shape), refi)
+
+
+def test_strided_forward_reference_large_fixture():
+    """tests/test_parallelized_convolution_large_CPU.cpp:71-80: b=4 d=3 n=127 k=11 s=4 p=2 o=8."""
+    shape = (4, 3, 127, 11, 4, 2, 8)
+    b, d, n, k, s, p, o = shape
+    x = load_fixture("input", "conv_forward_in_large.txt").reshape(b, d, n, n)
+    w = load_fixture("input", "conv_model_large.txt").reshape(o, d, k, k)
+    bias = load_fixture("input", "conv_bias_in_large.txt")
+    got = _forward(driver(), x, w, bias, shape)
+    np.testing.assert_allclose(got.reshape(-1), load_fixture("output", "conv_forward_large.txt"), rtol=2e-5, atol=1e-3)
+
+
+def test_strided_forward_full_config3_vs_float64():
+    """benchmark configuration 3 at full size (batch 256, 3x227x227, 96 filters 11x11, stride 4) against
+    torch conv2d in float64."""
+    import torch
+    shape = (256, 3, 227, 11, 4, 0, 96)
+    b, d, n, k, s, p, o = shape
+    rng = np.random.default_rng(3)
+    x = rng.uniform(0, 255, (b, d, n, n)).astype(np.float32)
+    x -= np.array([104, 117, 123], np.float32)[None, :, None, None]
+    w = (rng.standard_normal((o, d, k, k)) * 0.01).astype(np.float32)
+    bias = rng.standard_normal(o).astype(np.float32)
+    got = _forward(driver(), x, w, bias, shape)
+    ref = torch.nn.functional.conv2d(torch.from_numpy(x).cuda().double(), torch.from_numpy(w).cuda().double(),
+                                     torch.from_numpy(bias).cuda().double(), stride=s, padding=p).cpu().numpy()
+    assert rel_err(got, ref) <= TOL
+
+
+def test_unsupported_geometries_are_refused():
+    from caffecontroll_amd import CctHipError
+    drv = driver()
+    assert not drv.conv_strided_supported(2, 3, 30, 11, 3, 0, 8)     # stride 3
+    assert not drv.conv_strided_supported(2, 3, 30, 9, 4, 0, 8)      # no 9x9 instance
+    assert not drv.conv_strided_supported(2, 3, 2000, 11, 4, 2, 8)   # padded rows too long for the LDS patch
+    assert drv.conv_strided_supported(2, 3, 2000, 11, 4, 0, 8)       # without padding nothing is staged
+    with pytest.raises(CctHipError, match="not covered"):
+        drv.conv_strided_forward(empty((4,)), empty((4,)), empty((4,)), None, 2, 3, 30, 11, 3, 0, 8)
