@@ -92,6 +92,7 @@ PROTOTYPES = {
     "cct_hip_conv_strided_slab_floats": [_I, _I, _I, _I, _I],
     "cct_hip_conv_strided_slabs": [_P, _P, _I, _I, _I, _I, _I],
     "cct_hip_conv_strided_forward": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I],
+    "cct_hip_conv_strided_backward_weights": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I],
     "cct_hip_sgemv": [_I, _I, _I, _F, _P, _P, _F, _P],
     "cct_hip_math_saxpy": [_Z, _F, _P, _P],
     "cct_hip_math_saxpby": [_Z, _F, _P, _F, _P],

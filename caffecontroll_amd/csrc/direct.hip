@@ -867,6 +867,14 @@ __global__ __launch_bounds__(256) void direct_reduce_kernel(float *__restrict__ 
   dst[e] = s;
 }
 
+int reduce_partial_sums(float *dst, const float *ws, uint32_t n, float *dst2, const float *ws2, uint32_t n2,
+                        int splits, hipStream_t st) {
+  hipLaunchKernelGGL(direct_reduce_kernel, dim3((n + n2 + 255) / 256), dim3(256), 0, st, dst, ws, n, dst2, ws2, n2,
+                     splits);
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
 struct WgradPlan {
   int waves, tb, pw, ast, a_floats, stage;
   bool spec;  // a compile-time specialised instance exists for this shape
@@ -1025,9 +1033,7 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   if (rc) return rc;
   if (splits > 1) {
     const uint32_t n2 = db ? (uint32_t)o : 0u;
-    hipLaunchKernelGGL(direct_reduce_kernel, dim3((uint32_t)((n_out + n2 + 255) / 256)), dim3(256), 0, st, dw,
-                       g.out, (uint32_t)n_out, db, g.out_bias, n2, splits);
-    CCT_LAUNCH_CHECK();
+    if (int rc2 = reduce_partial_sums(dw, g.out, (uint32_t)n_out, db, g.out_bias, n2, splits, st)) return rc2;
   }
   return 0;
 }

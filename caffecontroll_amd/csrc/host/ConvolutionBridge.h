@@ -16,7 +16,10 @@
 //     (level 3, the default where the geometry allows it) come from direct-convolution kernels
 //     that never materialise the lowered matrices; results then agree with the lowering path to
 //     fp32 rounding instead of bit for bit.  The lowered buffers are allocated on first use, so
-//     level 3 runs without them.
+//     level 3 runs without them;
+//   * strided layers with k = 11 (stride 4) or k = 7, 5, 3 (stride 2) take level 3 with direct forward
+//     and weight-gradient kernels of their own; their data gradient (not needed for a first layer)
+//     still comes from the data-gradient GEMM and the lifting, which need no lowered input.
 #pragma once
 #include <cstdio>
 #include <cstdlib>
@@ -121,6 +124,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
         &lowered_forward_model, &lowered_forward_output, &lowered_data, p_driver);
     direct_ok_ = p_driver->conv_direct_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
                                                  (int)num_output_features);
+    strided_ok_ = !direct_ok_ && p_driver->conv_strided_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride,
+                                                                  (int)padding, (int)num_output_features);
     // Small layers (LeNet-sized) stay on the fused lowering path by default: the direct kernels'
     // fixed costs (slab re-layout, partial-sum reduction) outweigh what they save below a few GFLOP.
     const double gemm_flop = 2.0 * num_output_features * (double)(oR * oC * iB) * (double)(K * K * iD);
@@ -128,6 +133,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     // epilogue; there the direct kernels win at any size)
     const bool short_contraction = K * K * iD <= 64;
     default_path_ = (direct_ok_ && (gemm_flop >= kConvDirectMinFlop || short_contraction)) ? PATH_DIRECT_ALL : PATH_FUSED;
+    if (strided_ok_ && gemm_flop >= kConvDirectMinFlop) default_path_ = PATH_DIRECT_ALL;
     path_ = default_path_;
     for (int i = 0; i < STAGE_COUNT; ++i) { timers_[i] = nullptr; stage_ms_[i] = 0.f; }
   }
@@ -161,7 +167,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   void set_path(int level) {
     if (level < PATH_STAGED) level = PATH_STAGED;
     if (level > PATH_DIRECT_ALL) level = PATH_DIRECT_ALL;
-    if (level >= PATH_DIRECT_DATA && !direct_ok_) level = PATH_FUSED;
+    if (level >= PATH_DIRECT_DATA && !direct_ok_) level = (strided_ok_ && level == PATH_DIRECT_ALL) ? PATH_DIRECT_ALL : PATH_FUSED;
     if (views_) level = PATH_DIRECT_ALL;  // the lowering path cannot address channel-slice views
     path_ = level;
   }
@@ -209,6 +215,18 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     LogicalCubeType *output_d_cube = p_output_layer->p_data_cube;
     LogicalCubeType lowered_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
 
+    if (path_ == PATH_DIRECT_ALL && strided_ok_) {
+      begin(STAGE_GEMM);
+      p_driver->conv_strided_slabs(forward_slabs()->get_p_data(), p_model_cube->get_p_data(),
+                                   (int)num_output_features, (int)iD, (int)K, (int)stride, (int)padding);
+      p_driver->conv_strided_forward(output_d_cube->get_p_data(), input_d_cube->get_p_data(),
+                                     forward_slabs()->get_p_data(), bias_term ? p_bias_cube->get_p_data() : nullptr,
+                                     (int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
+                                     (int)num_output_features, fuse_relu_);
+      end(STAGE_GEMM);
+      report_forward_history.end();
+      return;
+    }
     if (path_ == PATH_DIRECT_ALL) {
       // slabs are rebuilt every pass: the model changes between iterations
       begin(STAGE_GEMM);
@@ -265,8 +283,11 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     LogicalCubeType lowered_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
     LogicalCubeType lowered_model_grad(p_model_gradient_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
     DeviceMemoryPointer og = output_g_cube->get_device_pointer(p_driver);
-    const bool direct_data = path_ >= PATH_DIRECT_DATA && needs_to_calc_backward_grad;
+    const bool direct_data = path_ >= PATH_DIRECT_DATA && needs_to_calc_backward_grad && direct_ok_;
     const bool direct_weights = path_ == PATH_DIRECT_ALL;
+    // a strided layer on the all-direct path that must hand back an input gradient: the permuted output
+    // gradient feeds the data-gradient GEMM, whose result is lifted (neither needs the lowered input)
+    const bool strided_data = direct_weights && strided_ok_ && needs_to_calc_backward_grad;
 
     const bool fuse_bias_into_lift = bias_term && needs_to_calc_backward_grad && path_ == PATH_FUSED;
     // on the all-direct path the weight-gradient kernel reduces the bias gradient as well
@@ -279,14 +300,14 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       p_driver->backward_bias(&bias, &og, (int)(oR * oC), (int)oD, (int)iB);
       end(STAGE_BW_BIAS);
     }
-    if (!direct_weights) {
+    if (!direct_weights || strided_data) {
       begin(STAGE_BW_REMAP);
       p_forward_lower_connector->remap_output(*staging(), *output_g_cube, oB, num_output_features,
                                               fuse_bias_into_remap ? p_bias_gradient_cube : nullptr);
       end(STAGE_BW_REMAP);
     }
-    LogicalCubeType lowered_outputgrad(direct_weights ? nullptr : staging()->get_p_data(), num_output_features,
-                                       oR * oC * iB, 1, 1);
+    LogicalCubeType lowered_outputgrad(direct_weights && !strided_data ? nullptr : staging()->get_p_data(),
+                                       num_output_features, oR * oC * iB, 1, 1);
     if (needs_to_calc_backward_grad && !direct_data) {
       begin(STAGE_GEMM_DATA);
       p_backward_gemm_updategrad_kernel->compute(&lowered_model, &lowered_outputgrad, backward_inputgrad());
@@ -297,7 +318,13 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     // lifting kernel is HBM-bound and runs faster once the 1.8 GB written by the data-gradient
     // GEMM has drained from the caches.
     begin(STAGE_GEMM_WEIGHTS);
-    if (direct_weights) {
+    if (direct_weights && strided_ok_) {
+      p_driver->conv_strided_backward_weights(p_model_gradient_cube->get_p_data(),
+                                              bias_term ? p_bias_gradient_cube->get_p_data() : nullptr,
+                                              output_g_cube->get_p_data(), p_input_layer->p_data_cube->get_p_data(),
+                                              (int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
+                                              (int)num_output_features);
+    } else if (direct_weights) {
       p_driver->conv_direct_backward_weights(p_model_gradient_cube->get_p_data(),
                                              bias_term ? p_bias_gradient_cube->get_p_data() : nullptr,
                                              output_g_cube->get_p_data(), p_input_layer->p_data_cube->get_p_data(),
@@ -377,7 +404,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   size_t in_image_stride_ = 0, out_image_stride_ = 0;
   bool views_ = false;
   bool fuse_relu_ = false;
-  bool direct_ok_ = false, profile_ = false;
+  bool direct_ok_ = false, strided_ok_ = false, profile_ = false;
   LogicalCubeType *lowered() {
     if (!p_forward_lowered_data) p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
     return p_forward_lowered_data;
@@ -393,7 +420,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   LogicalCubeType *forward_slabs() {
     if (!p_forward_slabs)
       p_forward_slabs = new LogicalCubeType(
-          p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 0), 1, 1, 1, p_driver);
+          strided_ok_ ? p_driver->conv_strided_slab_floats((int)num_output_features, (int)iD, (int)K, (int)stride,
+                                                           (int)padding)
+                      : p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 0),
+          1, 1, 1, p_driver);
     return p_forward_slabs;
   }
   LogicalCubeType *backward_slabs() {

@@ -264,6 +264,30 @@ class HIPDriver {
                                             num_outputs, in_stride, out_stride),
        "conv_direct_backward_weights");
   }
+  // ---- strided convolution without the lowered matrix (no counterpart in DeviceDriver.h) ----
+  bool conv_strided_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs) {
+    return cct_hip_conv_strided_supported(batch, depth, n, k, stride, padding, num_outputs) != 0;
+  }
+  size_t conv_strided_slab_floats(int num_outputs, int depth, int k, int stride, int padding) {
+    return cct_hip_conv_strided_slab_floats(num_outputs, depth, k, stride, padding);
+  }
+  void conv_strided_slabs(float *slabs, const float *model, int num_outputs, int depth, int k, int stride,
+                          int padding) {
+    ok(cct_hip_conv_strided_slabs(slabs, model, num_outputs, depth, k, stride, padding), "conv_strided_slabs");
+  }
+  void conv_strided_forward(float *output, const float *input, const float *slabs, const float *bias, int batch,
+                            int depth, int n, int k, int stride, int padding, int num_outputs, bool relu = false) {
+    ok(cct_hip_conv_strided_forward(output, input, slabs, bias, batch, depth, n, k, stride, padding, num_outputs,
+                                    relu ? 1 : 0),
+       "conv_strided_forward");
+  }
+  void conv_strided_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
+                                     const float *input, int batch, int depth, int n, int k, int stride,
+                                     int padding, int num_outputs) {
+    ok(cct_hip_conv_strided_backward_weights(model_grad, bias_grad, output_grad, input, batch, depth, n, k, stride,
+                                             padding, num_outputs),
+       "conv_strided_backward_weights");
+  }
   void sgemv(const CBLAS_TRANSPOSE TA, const int M, const int N, const float alpha, const float *pA,
              const float *px, const float beta, float *py) {
     ok(cct_hip_sgemv(TA, M, N, alpha, pA, px, beta, py), "sgemv");

@@ -30,4 +30,10 @@ __device__ __forceinline__ void lds_dma4(rsrc_t r, uint32_t lane_bytes, uint32_t
 // all of this wave's global->LDS loads have landed (vmcnt(0); expcnt/lgkmcnt left alone)
 __device__ __forceinline__ void lds_dma_wait() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+// dst[e] = sum over z of ws[z][e] for e < n, and dst2[e] = sum over z of ws2[z][e] for e < n2 (z ascending):
+// the fixed-order reduction of the partial sums the weight-gradient kernels leave in the workspace
+// (defined beside the stride-1 kernels).
+int reduce_partial_sums(float *dst, const float *ws, uint32_t n, float *dst2, const float *ws2, uint32_t n2,
+                        int splits, hipStream_t st);
+
 }  // namespace cct

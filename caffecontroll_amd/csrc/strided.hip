@@ -596,6 +596,340 @@ static int strided_launch(const StridedArgs &g, const StridedPlan &pl, hipStream
   return set_error(CCT_HIP_EINVAL, "conv_strided: no kernel instance for %d row blocks", pl.tmb);
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Weight gradient of a strided layer without the lowered matrix:
+//   dW[m][c][u][v] = sum_{img,y,x} dout[img][m][y][x] * src[img][c][S*y - pad + u][S*x - pad + v]
+// as a GEMM with M = output maps, N = (c,u,v) columns and the contraction over output pixels
+// (it replaces the output-gradient remap and the weight-gradient GEMM against the lowered matrix,
+// and with them the need to keep that matrix from the forward pass).
+//
+// A workgroup is a WM x WN grid of wavefronts and owns 32*WM maps x 32*TB*WN columns of dW and a
+// range of contraction steps; wavefront (wm, wn) holds row block wm for the TB column blocks of
+// column group wn.  One step is output row y of one image: MFMA lanes 0-31 take pixel x = 2q,
+// lanes 32-63 pixel x = 2q + 1.  Per step the workgroup stages, straight from global memory into
+// LDS (4-byte buffer loads into LDS, two stages, one barrier per step):
+//   * the dout slab [32*WM][ast]: words 0..ho-1 of a row = row y of that map, zeros behind (ast odd:
+//     the 32 rows a wavefront reads hit 32 banks);
+//   * for the channels its columns touch, the KS source rows under output row y, zero-padded:
+//     [channel][KS][pws]; pws = KS and the channel stride = KS*KS (mod 32), so a wavefront's 32
+//     consecutive (c,u,v) columns read 32 different banks, and pixel x reads its row at S*x.
+//     Every word is rewritten every step (out-of-image words arrive as zeros).
+// Partial sums of the step ranges go to a workspace and are added in a fixed order
+// (run-to-run identical results).  The bias gradient rides along: the dout fragments a wavefront
+// of column group 0 feeds to the matrix cores are also summed per lane.
+//
+// Bound: fp32 MFMA rate.  Algorithmic work 2 * o * batch*ho*ho * d*KS*KS FLOP per call.
+struct StridedWgradArgs {
+  const float *dout;   // [batch][o][ho][ho]
+  const float *src;    // [batch][d][hs][hs]
+  float *out;          // [splits][o][ncols]
+  float *out_bias;     // [splits][o] bias-gradient partial sums, or null
+  int batch, o, d, hs, ho, pad;
+  int ncols;           // d * KS * KS
+  int wm, wn;          // wavefront grid of a workgroup
+  int nch;             // channels of the source patch
+  int ast;             // floats between rows of the dout slab (odd)
+  int a_floats, b_floats;  // slab / patch floats per stage, whole passes of the workgroup
+  int nal, nbl;        // loads per lane per step: slab, patch
+  int pws, pch;        // floats between patch rows / patch channels
+  int nq2;             // groups of four pixels per output row: ceil(ho / 4)
+  int steps_total, steps_per_split;  // a step = (image, output row)
+  uint32_t tiles_m, tiles_n, ntiles, nblocks;
+  FastDiv div_ho, div_ast, div_pch, div_pws, div_wm;
+};
+
+constexpr int kSWgradSlabLoads = 12;   // per lane per step, at most
+constexpr int kSWgradPatchLoads = 20;
+
+template <int KS, int S, int TB>
+__global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWgradArgs g) {
+  constexpr int KK = KS * KS;
+  constexpr int NAL = kSWgradSlabLoads, NBL = kSWgradPatchLoads;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nthreads = blockDim.x, nwaves = nthreads >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int wni = (int)fdiv((uint32_t)wave, g.div_wm), wmi = wave - wni * g.wm;
+  const uint32_t flat = xcd_remap(blockIdx.x, g.nblocks);
+  const uint32_t z = flat / g.ntiles, id = flat - z * g.ntiles;
+  const uint32_t tm = id / g.tiles_n, tn = id - tm * g.tiles_n;
+  const int bm = 32 * g.wm;
+  const int m0 = tm * bm, n0 = tn * (32 * TB * g.wn), ch0 = n0 / KK;
+  const int s_beg = z * g.steps_per_split, s_end = min(g.steps_total, s_beg + g.steps_per_split);
+  const int ho2 = g.ho * g.ho, hs2 = g.hs * g.hs;
+  const int stage = g.a_floats + g.b_floats;
+
+  // ---- dout slab: pass k of the workgroup covers slab words k*nthreads + tid ----
+  uint32_t aoff[NAL];  // byte offset from (image, map m0, row y); kOutOfRange = a zero word
+#pragma unroll
+  for (int k = 0; k < NAL; ++k) {
+    const uint32_t e = (uint32_t)(k * nthreads + tid);
+    const uint32_t m = fdiv(e, g.div_ast), i = e - m * g.ast;
+    const bool ok = k < g.nal && m < (uint32_t)bm && m0 + (int)m < g.o && i < (uint32_t)g.ho;
+    aoff[k] = ok ? (m * ho2 + i) * 4u : kOutOfRange;
+  }
+  // ---- source patch: element e = k*nthreads + tid of the [nch][pch] array (rows of pws floats) ----
+  uint32_t boff[NBL];               // byte offset from (image, channel ch0, row S*y - pad); kOutOfRange = never valid
+  uint32_t brow[(NBL + 4) / 5];     // tap row of each element, six bits apiece
+#pragma unroll
+  for (int k = 0; k < (NBL + 4) / 5; ++k) brow[k] = 0u;
+#pragma unroll
+  for (int k = 0; k < NBL; ++k) {
+    const uint32_t e = (uint32_t)(k * nthreads + tid);
+    const uint32_t ch = fdiv(e, g.div_pch), rem = e - ch * g.pch;
+    const uint32_t prow = fdiv(rem, g.div_pws), pcol = rem - prow * g.pws;
+    const int scol = (int)pcol - g.pad;
+    const bool ok = k < g.nbl && ch < (uint32_t)g.nch && prow < (uint32_t)KS && ch0 + (int)ch < g.d &&
+                    (unsigned)scol < (unsigned)g.hs;
+    boff[k] = ok ? (ch * hs2 + prow * g.hs + (uint32_t)scol) * 4u : kOutOfRange;
+    brow[k / 5] |= (ok ? prow : 0u) << (6 * (k % 5));
+  }
+  const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
+
+// global -> LDS stage st for step s
+#define CCT_SWGRAD_ISSUE(s, st)                                                                   \
+  do {                                                                                            \
+    const uint32_t img_ = fdiv((uint32_t)(s), g.div_ho);                                          \
+    const int y_ = (s) - (int)img_ * g.ho;                                                        \
+    float *sa_ = smem + (st) * stage + wave * 64;                                                 \
+    const uint32_t ga_ = (uint32_t)(((size_t)img_ * g.o * ho2 + (size_t)m0 * ho2 + y_ * g.ho) * 4); \
+    _Pragma("unroll") for (int k = 0; k < NAL; ++k) {                                             \
+      if (k < g.nal) lds_dma4(a_rsrc, aoff[k], ga_, sa_ + k * nthreads);                          \
+    }                                                                                             \
+    float *sb_ = sa_ + g.a_floats;                                                                \
+    const uint32_t gb_ = (uint32_t)(((size_t)img_ * g.d * hs2 + (size_t)ch0 * hs2) * 4);          \
+    /* the first patch row may lie above the image: that (negative) term goes into the lane     */ \
+    /* offset, whose sum is non-negative for every lane that passes the row test                */ \
+    const int top_ = S * y_ - g.pad;                                                              \
+    const uint32_t row0_ = (uint32_t)(top_ * g.hs * 4);                                           \
+    _Pragma("unroll") for (int k = 0; k < NBL; ++k) {                                             \
+      const int srow_ = top_ + (int)((brow[k / 5] >> (6 * (k % 5))) & 63u);                       \
+      const bool ok_ = (int)boff[k] >= 0 && (unsigned)srow_ < (unsigned)g.hs;                     \
+      if (k < g.nbl) lds_dma4(b_rsrc, ok_ ? boff[k] + row0_ : kOutOfRange, gb_, sb_ + k * nthreads); \
+    }                                                                                             \
+  } while (0)
+
+  // ---- fragment bases ----------------------------------------------------------------------
+  const int abase = (wmi * 32 + r) * g.ast + h;
+  int bbase[TB];
+#pragma unroll
+  for (int b = 0; b < TB; ++b) {
+    const int col = min(n0 + (wni * TB + b) * 32 + r, g.ncols - 1);
+    const int c = col / KK, j = col - c * KK, u = j / KS, v = j - u * KS;
+    bbase[b] = g.a_floats + (c - ch0) * g.pch + u * g.pws + v + S * h;
+  }
+
+  v16f acc[TB];
+#pragma unroll
+  for (int b = 0; b < TB; ++b)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+  float bsum = 0.0f;  // lane (r, h) adds up dout[map r][every image][every row][x = h (mod 2)]
+
+  if (s_beg < s_end) {
+    CCT_SWGRAD_ISSUE(s_beg, 0);
+    lds_dma_wait();
+  }
+  __syncthreads();
+
+  for (int s = s_beg; s < s_end; ++s) {
+    const int cur = (s - s_beg) & 1;
+    if (s + 1 < s_end) CCT_SWGRAD_ISSUE(s + 1, cur ^ 1);
+    const float *sa = smem + cur * stage + abase;
+    const float *sb[TB];
+#pragma unroll
+    for (int b = 0; b < TB; ++b) sb[b] = smem + cur * stage + bbase[b];
+    // fragment buffers; reads past ho stay inside the stage and meet zero dout words
+    float fa[2], fb[2][TB];
+#define CCT_SWGRAD_FRAGS(buf, x)                                                                  \
+  do {                                                                                            \
+    fa[buf] = sa[(x)];                                                                            \
+    _Pragma("unroll") for (int b = 0; b < TB; ++b) fb[buf][b] = sb[b][S * (x)];                   \
+  } while (0)
+#define CCT_SWGRAD_MFMA(buf)                                                                      \
+  do {                                                                                            \
+    bsum += fa[buf];                                                                              \
+    _Pragma("unroll") for (int b = 0; b < TB; ++b)                                                \
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[buf], fb[buf][b], acc[b], 0, 0, 0);      \
+  } while (0)
+// issue order of one pixel pair: the LDS reads of the next pair go out between this pair's MFMAs
+#define CCT_SWGRAD_ORDER()                                                                        \
+  do {                                                                                            \
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                            \
+    __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);                                            \
+    _Pragma("unroll") for (int k2 = 1; k2 < TB; ++k2) {                                           \
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                          \
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                          \
+    }                                                                                             \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+  } while (0)
+    CCT_SWGRAD_FRAGS(0, 0);
+    for (int qd = 0; qd < g.nq2; ++qd) {
+      const int x = 4 * qd;
+      CCT_SWGRAD_FRAGS(1, x + 2);
+      CCT_SWGRAD_MFMA(0);
+      CCT_SWGRAD_ORDER();
+      CCT_SWGRAD_FRAGS(0, x + 4);
+      CCT_SWGRAD_MFMA(1);
+      CCT_SWGRAD_ORDER();
+    }
+#undef CCT_SWGRAD_FRAGS
+#undef CCT_SWGRAD_MFMA
+#undef CCT_SWGRAD_ORDER
+    lds_dma_wait();
+    __syncthreads();
+  }
+#undef CCT_SWGRAD_ISSUE
+
+  if (g.out_bias && tn == 0 && wni == 0) {
+    const float both = bsum + __shfl_xor(bsum, 32);
+    const int row = m0 + wmi * 32 + r;
+    if (h == 0 && row < g.o) g.out_bias[(size_t)z * g.o + row] = both;
+  }
+  float *out = g.out + (size_t)z * g.o * g.ncols;
+#pragma unroll
+  for (int b = 0; b < TB; ++b) {
+    const int col = n0 + (wni * TB + b) * 32 + r;
+    if (col >= g.ncols) continue;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = m0 + wmi * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+      if (row < g.o) out[(size_t)row * g.ncols + col] = acc[b][v];
+    }
+  }
+}
+
+struct StridedWgradPlan {
+  int tb, wm, wn, nch, ast, a_floats, b_floats, nal, nbl, pws, pch, nq2;
+  size_t lds;
+};
+
+static bool strided_kernel_size(int ks, int stride) {
+  return (ks == 11 && stride == 4) || (ks == 7 && stride == 2) || (ks == 5 && stride == 2) || (ks == 3 && stride == 2);
+}
+
+// Chooses the workgroup shape for a geometry; false when the strided weight-gradient kernel does not cover it.
+static bool strided_wgrad_plan(int batch, int d, int n, int ks, int stride, int pad, int o, StridedWgradPlan *pl) {
+  if (!strided_kernel_size(ks, stride)) return false;
+  if (batch <= 0 || d <= 0 || o <= 0 || pad < 0 || pad >= ks || n + 2 * pad < ks) return false;
+  const int hp = n + 2 * pad, ho = (hp - ks) / stride + 1, kk = ks * ks;
+  if ((double)batch * d * n * n >= 536870912.0 || (double)batch * o * ho * ho >= 536870912.0 ||
+      (double)o * d * kk >= 536870912.0)
+    return false;  // 32-bit byte offsets
+  const int ncols = d * kk, cb = (ncols + 31) / 32, mb = (o + 31) / 32;
+  const int nq2 = (ho + 3) / 4, ast = 4 * nq2 + 1;
+  const int tw = stride * (ho - 1) + ks;                      // source columns an output row touches
+  const int pws = tw + (((ks - tw) % 32) + 32) % 32;          // >= tw, == ks (mod 32)
+  const int raw = ks * pws, pch = raw + (((kk - raw) % 32) + 32) % 32;  // >= raw, == ks*ks (mod 32)
+  long best_cost = -1;
+  // candidates: column blocks per wavefront x column groups x row blocks; cost = MFMAs issued per step
+  for (int tb = 3; tb >= 1; --tb)
+    for (int wn = 4; wn >= 1; --wn)
+      for (int wm = 4; wm >= 1; --wm) {
+        const int w = wm * wn;
+        if (w > 12) continue;
+        if (wm > mb || (wn - 1) * tb >= cb) continue;  // wavefronts with nothing to do
+        const int nth = 64 * w;
+        const int tiles_n = (cb + tb * wn - 1) / (tb * wn), tiles_m = (mb + wm - 1) / wm;
+        int nch = (32 * tb * wn - 1) / kk + 2;
+        if (nch > d) nch = d;
+        // last word a fragment load can touch: the step's final prefetch reads pixel 4*nq2 + 1
+        const int b_need = (nch - 1) * pch + (ks - 1) * pws + (ks - 1) + stride * (4 * nq2 + 1) + 1;
+        const int b_floats = ((b_need > nch * pch ? b_need : nch * pch) + nth - 1) / nth * nth;
+        const int a_floats = (32 * wm * ast + 2 + nth - 1) / nth * nth;
+        const int nal = a_floats / nth, nbl = b_floats / nth;
+        if (nal > kSWgradSlabLoads || nbl > kSWgradPatchLoads) continue;
+        const size_t lds = (size_t)2 * (a_floats + b_floats) * sizeof(float);
+        if (lds > 160 * 1024) continue;
+        // padded work; on ties: wider per-wavefront tiles, then a wavefront count that loads the four SIMDs evenly
+        long cost = (long)tiles_n * tb * wn * tiles_m * wm * 1000;
+        cost += (3 - tb) * 40 + (w % 4 ? 20 : 0) + (12 - w);
+        if (best_cost < 0 || cost < best_cost) {
+          best_cost = cost;
+          pl->tb = tb; pl->wm = wm; pl->wn = wn; pl->nch = nch; pl->ast = ast; pl->a_floats = a_floats;
+          pl->b_floats = b_floats; pl->nal = nal; pl->nbl = nbl; pl->pws = pws; pl->pch = pch; pl->nq2 = nq2;
+          pl->lds = lds;
+        }
+      }
+  return best_cost >= 0;
+}
+
+template <int KS, int S>
+static int strided_wgrad_launch(const StridedWgradArgs &g, const StridedWgradPlan &pl, hipStream_t st) {
+  dim3 grid(g.nblocks), block(64 * pl.wm * pl.wn);
+#define CCT_SWGRAD_CASE(TB)                                                                       \
+  if (pl.tb == TB) {                                                                              \
+    auto kern = conv_strided_wgrad_kernel<KS, S, TB>;                                             \
+    static LdsGrant grant;                                                                        \
+    if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;                 \
+    hipLaunchKernelGGL(kern, grid, block, pl.lds, st, g);                                         \
+    CCT_LAUNCH_CHECK();                                                                           \
+    note_kernel("conv_strided_wgrad_kernel<%d,%d,%d> waves=%dx%d", KS, S, TB, pl.wm, pl.wn);      \
+    return 0;                                                                                     \
+  }
+  CCT_SWGRAD_CASE(1) CCT_SWGRAD_CASE(2) CCT_SWGRAD_CASE(3)
+#undef CCT_SWGRAD_CASE
+  return set_error(CCT_HIP_EINVAL, "conv_strided wgrad: no kernel instance for %d column blocks", pl.tb);
+}
+
+static int conv_strided_wgrad(float *dw, float *db, const float *dout, const float *src, int batch, int d, int n,
+                              int ks, int stride, int pad, int o) {
+  StridedWgradPlan pl;
+  CCT_REQUIRE(strided_wgrad_plan(batch, d, n, ks, stride, pad, o, &pl),
+              "conv_strided wgrad: geometry not covered (k=%d stride=%d pad=%d size=%d)", ks, stride, pad, n);
+  StridedWgradArgs g;
+  g.dout = dout; g.src = src;
+  g.batch = batch; g.o = o; g.d = d; g.hs = n; g.pad = pad;
+  g.ho = (n + 2 * pad - ks) / stride + 1;
+  g.ncols = d * ks * ks;
+  g.wm = pl.wm; g.wn = pl.wn; g.nch = pl.nch; g.ast = pl.ast; g.a_floats = pl.a_floats; g.b_floats = pl.b_floats;
+  g.nal = pl.nal; g.nbl = pl.nbl; g.pws = pl.pws; g.pch = pl.pch; g.nq2 = pl.nq2;
+  g.steps_total = batch * g.ho;
+  g.tiles_m = (uint32_t)((o + 32 * pl.wm - 1) / (32 * pl.wm));
+  g.tiles_n = (uint32_t)((g.ncols + 32 * pl.tb * pl.wn - 1) / (32 * pl.tb * pl.wn));
+  g.ntiles = g.tiles_m * g.tiles_n;
+  const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
+  // workgroups resident per compute unit: LDS, and three wavefronts per SIMD (the register budget of the kernel)
+  int per_cu = (int)((160 * 1024) / pl.lds);
+  if (per_cu > 12 / (pl.wm * pl.wn)) per_cu = 12 / (pl.wm * pl.wn);
+  if (per_cu < 1) per_cu = 1;
+  int splits = (int)((long)per_cu * cus / g.ntiles);
+  if (splits < 1) splits = 1;
+  if (splits > g.steps_total) splits = g.steps_total;
+  g.steps_per_split = (g.steps_total + splits - 1) / splits;
+  splits = (g.steps_total + g.steps_per_split - 1) / g.steps_per_split;
+  g.nblocks = g.ntiles * (uint32_t)splits;
+  g.div_ho = make_fastdiv((uint32_t)g.ho);
+  g.div_ast = make_fastdiv((uint32_t)g.ast);
+  g.div_pch = make_fastdiv((uint32_t)g.pch);
+  g.div_pws = make_fastdiv((uint32_t)g.pws);
+  g.div_wm = make_fastdiv((uint32_t)g.wm);
+  const size_t n_out = (size_t)o * g.ncols;
+  if (splits > 1) {
+    void *ws = nullptr;
+    int rc = get_workspace((size_t)splits * (n_out + (db ? o : 0)) * sizeof(float), &ws);
+    if (rc) return rc;
+    g.out = (float *)ws;
+    g.out_bias = db ? g.out + (size_t)splits * n_out : nullptr;
+  } else {
+    g.out = dw;
+    g.out_bias = db;
+  }
+  hipStream_t st = ctx().stream;
+  int rc;
+  if (ks == 11) rc = strided_wgrad_launch<11, 4>(g, pl, st);
+  else if (ks == 7) rc = strided_wgrad_launch<7, 2>(g, pl, st);
+  else if (ks == 5) rc = strided_wgrad_launch<5, 2>(g, pl, st);
+  else rc = strided_wgrad_launch<3, 2>(g, pl, st);
+  if (rc) return rc;
+  if (splits > 1)
+    return reduce_partial_sums(dw, g.out, (uint32_t)n_out, db, g.out_bias, db ? (uint32_t)o : 0u, splits, st);
+  return 0;
+}
+
 }  // namespace cct
 
 using namespace cct;
@@ -603,7 +937,11 @@ using namespace cct;
 extern "C" int cct_hip_conv_strided_supported(int batch, int depth, int n, int k, int stride, int padding,
                                               int num_outputs) {
   StridedPlan pl;
-  return strided_plan(batch, depth, n, k, stride, padding, num_outputs, &pl) ? 1 : 0;
+  StridedWgradPlan wpl;
+  return strided_plan(batch, depth, n, k, stride, padding, num_outputs, &pl) &&
+                 strided_wgrad_plan(batch, depth, n, k, stride, padding, num_outputs, &wpl)
+             ? 1
+             : 0;
 }
 
 extern "C" size_t cct_hip_conv_strided_slab_floats(int num_outputs, int depth, int k, int stride, int padding) {
@@ -666,4 +1004,13 @@ extern "C" int cct_hip_conv_strided_forward(float *output, const float *input, c
   if (k == 7 && stride == 2) return strided_launch<7, 2>(g, pl, st);
   if (k == 5 && stride == 2) return strided_launch<5, 2>(g, pl, st);
   return strided_launch<3, 2>(g, pl, st);
+}
+
+extern "C" int cct_hip_conv_strided_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
+                                                     const float *input, int batch, int depth, int n, int k,
+                                                     int stride, int padding, int num_outputs) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(model_grad && output_grad && input, "conv_strided_backward_weights: null argument");
+  return conv_strided_wgrad(model_grad, bias_grad, output_grad, input, batch, depth, n, k, stride, padding,
+                            num_outputs);
 }

@@ -146,6 +146,10 @@ class HIPDriver:
         check(self.lib.cct_hip_conv_strided_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, s, p, o,
                                                     int(relu)), "conv_strided_forward")
 
+    def conv_strided_backward_weights(self, model_grad, bias_grad, out_grad, inp, b, d, n, k, s, p, o):
+        check(self.lib.cct_hip_conv_strided_backward_weights(_p(model_grad), _p(bias_grad), _p(out_grad), _p(inp),
+                                                             b, d, n, k, s, p, o), "conv_strided_backward_weights")
+
     def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o, in_stride=0, out_stride=0, relu=False):
         check(self.lib.cct_hip_conv_direct_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o,
                                                    in_stride, out_stride, int(relu)), "conv_direct_forward")

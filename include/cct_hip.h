@@ -232,7 +232,8 @@ int cct_hip_conv_direct_backward_weights(float *model_grad, float *bias_grad, co
 /* The same replacement of ConvolutionBridge's lowering pipeline for strided layers: stride 4 with an
  * 11 x 11 kernel (AlexNet / CaffeNet conv1, benchmark configuration 3; the reference's "large" golden
  * scenario, tests/test_parallelized_convolution_large_CPU.cpp:71-80) and stride 2 with 7 x 7,
- * 5 x 5 or 3 x 3 kernels.  cct_hip_conv_strided_supported: 1 if the geometry is covered, else 0. */
+ * 5 x 5 or 3 x 3 kernels.  cct_hip_conv_strided_supported: 1 if the forward and the weight-gradient
+ * kernel both cover the geometry (the layer can then run without the lowered matrix), else 0. */
 int cct_hip_conv_strided_supported(int batch, int depth, int n, int k, int stride, int padding,
                                    int num_outputs);
 /* Re-lays the model [o][d][k][k] for cct_hip_conv_strided_forward, zero padded: for a layer with
@@ -251,6 +252,14 @@ int cct_hip_conv_strided_slabs(float *slabs, const float *model, int num_outputs
 int cct_hip_conv_strided_forward(float *output, const float *input, const float *slabs, const float *bias,
                                  int batch, int depth, int n, int k, int stride, int padding,
                                  int num_outputs, int relu);
+/* Output-gradient remap + weight-gradient GEMM (+ bias gradient) of ConvolutionBridge::backward
+ * (src/bridges/ConvolutionBridge_impl.hxx:575-604, 619-621) for a strided layer in one kernel plus a
+ * fixed-order reduction of partial sums, reading the layer's input instead of the lowered matrix of
+ * the forward pass: model_grad[o][d][k][k], bias_grad[o] (may be NULL) from output_grad[b][o][m][m]
+ * and input[b][d][n][n]. */
+int cct_hip_conv_strided_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
+                                          const float *input, int batch, int depth, int n, int k,
+                                          int stride, int padding, int num_outputs);
 /* DeviceDriver::sgemv (src/sched/DeviceDriver.h:214-215): row-major M x N, lda = N. */
 int cct_hip_sgemv(int TA, int M, int N, float alpha, const float *A, const float *x, float beta,
                   float *y);

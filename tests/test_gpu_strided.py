@@ -93,12 +93,87 @@ def test_strided_forward_full_config3_vs_float64():
     assert rel_err(got, ref) <= TOL
 
 
+@pytest.mark.parametrize("shape", SHAPES, ids=_ids)
+def test_strided_backward_weights_vs_oracle(oracle, shape):
+    """Weight and bias gradient against the oracle's remap + weight-gradient GEMM on the lowered matrix
+    (src/bridges/ConvolutionBridge_impl.hxx:575-604, 619-621)."""
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
+    drv = driver()
+    rng = np.random.default_rng(sum(shape) + 1)
+    x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+    w = (rng.standard_normal((o, d, k, k)) * 0.1).astype(np.float32)
+    og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+    _, lowered = oracle.conv_forward(x, w, None, k, s, p)
+    _, ref_dw, ref_db = oracle.conv_backward(x.shape, w, og, lowered, k, s, p, need_in_grad=False)
+    d_x, d_og = dev(x), dev(og)
+    dw, db = empty((o, d, k, k)), empty((o,))
+    drv.conv_strided_backward_weights(dw, db, d_og, d_x, b, d, n, k, s, p, o)
+    assert rel_err(host(dw), ref_dw) <= TOL
+    assert rel_err(host(db), ref_db) <= TOL
+    assert rel_err(host(db), og.astype(np.float64).sum(axis=(0, 2, 3))) <= TOL
+    np.testing.assert_array_equal(host(d_og), og)  # the output gradient is read in place, not permuted
+    # partial sums are added in a fixed order: a second run gives the same bits, with or without the bias gradient
+    dw2 = empty((o, d, k, k))
+    drv.conv_strided_backward_weights(dw2, None, d_og, d_x, b, d, n, k, s, p, o)
+    np.testing.assert_array_equal(host(dw2), host(dw))
+    # small integers: every product and partial sum is exact, whatever the order
+    xi = rng.integers(-4, 5, size=x.shape).astype(np.float32)
+    ogi = rng.integers(-3, 4, size=og.shape).astype(np.float32)
+    _, lowered_i = oracle.conv_forward(xi, w, None, k, s, p)
+    _, refi_dw, refi_db = oracle.conv_backward(x.shape, w, ogi, lowered_i, k, s, p, need_in_grad=False)
+    drv.conv_strided_backward_weights(dw, db, dev(ogi), dev(xi), b, d, n, k, s, p, o)
+    np.testing.assert_array_equal(host(dw).reshape(-1), np.asarray(refi_dw).reshape(-1))
+    np.testing.assert_array_equal(host(db), refi_db)
+
+
+def test_strided_backward_weights_reference_large_fixture():
+    """tests/test_parallelized_convolution_large_CPU.cpp:71-80, backward: weights after one SGD step with
+    learning rate 0.01 (W - 0.01 dW, b - 0.01 db), output gradient 0.1 * i."""
+    shape = (4, 3, 127, 11, 4, 2, 8)
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
+    x = load_fixture("input", "conv_forward_in_large.txt").reshape(b, d, n, n)
+    w = load_fixture("input", "conv_backward_model_large.txt").reshape(o, d, k, k)
+    bias = load_fixture("input", "conv_bias_in_large.txt")
+    og = (0.1 * np.arange(b * o * m * m, dtype=np.float64)).astype(np.float32).reshape(b, o, m, m)
+    drv = driver()
+    dw, db = empty((o, d, k, k)), empty((o,))
+    drv.conv_strided_backward_weights(dw, db, dev(og), dev(x), b, d, n, k, s, p, o)
+    want_w = load_fixture("output", "conv_weights_large.txt")
+    want_b = load_fixture("output", "conv_bias_large.txt")
+    got_w = (w - np.float32(0.01) * host(dw)).reshape(-1)
+    got_b = bias - np.float32(0.01) * host(db)
+    np.testing.assert_allclose(got_w, want_w, rtol=1e-4, atol=1e-3)
+    np.testing.assert_allclose(got_b, want_b, rtol=1e-4, atol=1e-3)
+
+
+def test_strided_backward_weights_full_config3_vs_float64():
+    """benchmark configuration 3 at full size against float64 torch (weight gradient in chunks of 32 images)."""
+    import torch
+    shape = (256, 3, 227, 11, 4, 0, 96)
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
+    g = torch.Generator(device="cuda").manual_seed(1237)
+    x = torch.rand((b, d, n, n), device="cuda", generator=g) * 255 - 115
+    og = torch.randn((b, o, m, m), device="cuda", generator=g)
+    dw, db = empty((o, d, k, k)), empty((o,))
+    driver().conv_strided_backward_weights(dw, db, og, x, b, d, n, k, s, p, o)
+    torch.cuda.synchronize()
+    ref = torch.zeros((o, d, k, k), dtype=torch.float64, device="cuda")
+    for i in range(0, b, 32):
+        ref += torch.nn.grad.conv2d_weight(x[i:i + 32].double(), (o, d, k, k), og[i:i + 32].double(), stride=s, padding=p)
+    assert ((dw.double() - ref).abs().max() / ref.abs().max()).item() <= TOL
+    db_ref = og.double().sum(dim=(0, 2, 3))
+    assert ((db.double() - db_ref).abs().max() / db_ref.abs().max()).item() <= TOL
+
+
 def test_unsupported_geometries_are_refused():
     from caffecontroll_amd import CctHipError
     drv = driver()
     assert not drv.conv_strided_supported(2, 3, 30, 11, 3, 0, 8)     # stride 3
     assert not drv.conv_strided_supported(2, 3, 30, 9, 4, 0, 8)      # no 9x9 instance
     assert not drv.conv_strided_supported(2, 3, 2000, 11, 4, 2, 8)   # padded rows too long for the LDS patch
-    assert drv.conv_strided_supported(2, 3, 2000, 11, 4, 0, 8)       # without padding nothing is staged
+    assert not drv.conv_strided_supported(2, 3, 2000, 11, 4, 0, 8)   # source rows too long for the weight gradient's patch
     with pytest.raises(CctHipError, match="not covered"):
         drv.conv_strided_forward(empty((4,)), empty((4,)), empty((4,)), None, 2, 3, 30, 11, 3, 0, 8)
