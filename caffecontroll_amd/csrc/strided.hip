@@ -802,8 +802,173 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
   }
 }
 
+// The same computation for layers without padding whose output-row length and load counts are
+// known at compile time (conv1 of AlexNet / CaffeNet).  Vector-ALU instructions do not overlap with
+// the MFMAs of the same SIMD, so this variant issues next to none inside a step: the step is one
+// straight line of code, every fragment read is base register + immediate offset, the step-dependent
+// part of every global address sits in the scalar offset of the buffer load (no padding: the rows
+// under an output row are always inside the image), the next step's loads are spread between the
+// MFMAs of this one (unconditionally: the last step of a range re-fetches itself into the idle
+// stage), and the bias gradient costs no additions at all: the first unused column of the padded
+// column range reads a row of ones, so its accumulator column IS the sum of dout.
+constexpr int kSWgradOnes = 256;  // floats of the row of ones (>= S * pixels of a padded output row)
+
+template <int KS, int S, int TB, int NQ2, int NAL, int NBL>
+__global__ __launch_bounds__(768) void conv_strided_wgrad_spec_kernel(const StridedWgradArgs g) {
+  constexpr int KK = KS * KS;
+  constexpr int NP = 2 * NQ2;          // pixel pairs per step
+  constexpr int NSLOT = NAL + NBL;     // global -> LDS loads per lane per step
+  constexpr int NQI = (NP * 5 + 7) / 8;  // pairs that carry a slice of the loads (the last ones leave time to land)
+  static_assert(S * (2 * NP + 1) < kSWgradOnes, "row of ones too short");
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int nthreads = blockDim.x;
+  const int r = lane & 31, h = lane >> 5;
+  const int wni = (int)fdiv((uint32_t)wave, g.div_wm), wmi = wave - wni * g.wm;
+  const uint32_t flat = xcd_remap(blockIdx.x, g.nblocks);
+  const uint32_t z = flat / g.ntiles, id = flat - z * g.ntiles;
+  const uint32_t tm = id / g.tiles_n, tn = id - tm * g.tiles_n;
+  const int bm = 32 * g.wm;
+  const int m0 = tm * bm, n0 = tn * (32 * TB * g.wn), ch0 = n0 / KK;
+  const int s_beg = z * g.steps_per_split, s_end = min(g.steps_total, s_beg + g.steps_per_split);
+  const int ho2 = g.ho * g.ho, hs2 = g.hs * g.hs;
+  const int stage = g.a_floats + g.b_floats;
+  float *const ones = smem + 2 * stage;
+  for (int i = tid; i < kSWgradOnes; i += nthreads) ones[i] = 1.0f;
+
+  uint32_t aoff[NAL];  // byte offset from (image, map m0, row y); kOutOfRange = a zero word
+#pragma unroll
+  for (int k = 0; k < NAL; ++k) {
+    const uint32_t e = (uint32_t)(k * nthreads + tid);
+    const uint32_t m = fdiv(e, g.div_ast), i = e - m * g.ast;
+    const bool ok = m < (uint32_t)bm && m0 + (int)m < g.o && i < (uint32_t)g.ho;
+    aoff[k] = ok ? (m * ho2 + i) * 4u : kOutOfRange;
+  }
+  uint32_t boff[NBL];  // byte offset from (image, channel ch0, row S*y); kOutOfRange = a zero word
+#pragma unroll
+  for (int k = 0; k < NBL; ++k) {
+    const uint32_t e = (uint32_t)(k * nthreads + tid);
+    const uint32_t ch = fdiv(e, g.div_pch), rem = e - ch * g.pch;
+    const uint32_t prow = fdiv(rem, g.div_pws), pcol = rem - prow * g.pws;
+    const bool ok = ch < (uint32_t)g.nch && prow < (uint32_t)KS && ch0 + (int)ch < g.d && pcol < (uint32_t)g.hs;
+    boff[k] = ok ? (ch * hs2 + prow * g.hs + pcol) * 4u : kOutOfRange;
+  }
+  const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
+
+  const int abase = (wmi * 32 + r) * g.ast + h;
+  int bbase[TB];
+  bool bias_col[TB];  // this lane's column of block b is the column of ones
+#pragma unroll
+  for (int b = 0; b < TB; ++b) {
+    const int col_raw = n0 + (wni * TB + b) * 32 + r;
+    const int col = min(col_raw, g.ncols - 1);
+    const int c = col / KK, j = col - c * KK, u = j / KS, v = j - u * KS;
+    bbase[b] = g.a_floats + (c - ch0) * g.pch + u * g.pws + v + S * h;
+    bias_col[b] = col_raw == g.ncols;
+  }
+
+  v16f acc[TB];
+#pragma unroll
+  for (int b = 0; b < TB; ++b)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
+
+// scalars of step s: the scalar offsets of its slab and patch loads
+#define CCT_SWSPEC_STEP(s)                                                                        \
+  const uint32_t img_ = fdiv((uint32_t)(s), g.div_ho);                                            \
+  const int y_ = (s) - (int)img_ * g.ho;                                                          \
+  const uint32_t ga_ = (uint32_t)(((size_t)img_ * g.o * ho2 + (size_t)m0 * ho2 + y_ * g.ho) * 4); \
+  const uint32_t gb_ = (uint32_t)(((size_t)img_ * g.d * hs2 + (size_t)ch0 * hs2 + (size_t)S * y_ * g.hs) * 4)
+#define CCT_SWSPEC_SLOT(k, st)                                                                    \
+  do {                                                                                            \
+    if ((k) < NAL)                                                                                \
+      lds_dma4(a_rsrc, aoff[(k) < NAL ? (k) : 0], ga_, smem + (st) * stage + wave * 64 + (k) * nthreads); \
+    else                                                                                          \
+      lds_dma4(b_rsrc, boff[(k) >= NAL ? (k) - NAL : 0], gb_,                                     \
+               smem + (st) * stage + g.a_floats + wave * 64 + ((k) - NAL) * nthreads);            \
+  } while (0)
+
+  if (s_beg < s_end) {
+    CCT_SWSPEC_STEP(s_beg);
+#pragma unroll
+    for (int k = 0; k < NSLOT; ++k) CCT_SWSPEC_SLOT(k, 0);
+    lds_dma_wait();
+  }
+  __syncthreads();
+
+  for (int s = s_beg; s < s_end; ++s) {
+    const int cur = (s - s_beg) & 1, nxt = cur ^ 1;
+    CCT_SWSPEC_STEP(min(s + 1, s_end - 1));
+    const float *sa = smem + cur * stage + abase;
+    const float *sb[TB];
+#pragma unroll
+    for (int b = 0; b < TB; ++b) sb[b] = bias_col[b] ? ones : smem + cur * stage + bbase[b];
+    float fa[2], fb[2][TB];
+#define CCT_SWSPEC_FRAGS(buf, x)                                                                  \
+  do {                                                                                            \
+    fa[buf] = sa[(x)];                                                                            \
+    _Pragma("unroll") for (int b = 0; b < TB; ++b) fb[buf][b] = sb[b][S * (x)];                   \
+  } while (0)
+    CCT_SWSPEC_FRAGS(0, 0);
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      const int cb = q & 1, nb = cb ^ 1;
+      if (q + 1 < NP) CCT_SWSPEC_FRAGS(nb, 2 * q + 2);
+#pragma unroll
+      for (int b = 0; b < TB; ++b)
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb], fb[cb][b], acc[b], 0, 0, 0);
+      // this pair's share of the next step's loads
+      const int qi = q < NQI ? q : NQI, qj = q + 1 < NQI ? q + 1 : NQI;
+      const int k_lo = qi * NSLOT / NQI, k_hi = qj * NSLOT / NQI;
+#pragma unroll
+      for (int k = 0; k < NSLOT; ++k)
+        if (k >= k_lo && k < k_hi) CCT_SWSPEC_SLOT(k, nxt);
+      // issue order: an LDS read of the next pair after every MFMA (two after the first), then the global loads
+      {
+        const int nr = q + 1 < NP ? TB + 1 : 0;
+        int left_r = nr, left_v = k_hi - k_lo;
+#pragma unroll
+        for (int k2 = 0; k2 < TB; ++k2) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          const int take_r = left_r > 0 ? (k2 == 0 && left_r > 1 ? 2 : 1) : 0;
+          if (take_r == 2) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+          else if (take_r == 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          left_r -= take_r;
+          if (left_v > 0) {
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            --left_v;
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#undef CCT_SWSPEC_FRAGS
+    lds_dma_wait();
+    __syncthreads();
+  }
+#undef CCT_SWSPEC_STEP
+#undef CCT_SWSPEC_SLOT
+
+  float *out = g.out + (size_t)z * g.o * g.ncols;
+#pragma unroll
+  for (int b = 0; b < TB; ++b) {
+    const int col = n0 + (wni * TB + b) * 32 + r;
+    if (col > g.ncols || (col == g.ncols && !g.out_bias)) continue;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int row = m0 + wmi * 32 + 8 * (v / 4) + 4 * h + (v % 4);
+      if (row >= g.o) continue;
+      if (col == g.ncols) g.out_bias[(size_t)z * g.o + row] = acc[b][v];  // the column of ones: sum of dout
+      else out[(size_t)row * g.ncols + col] = acc[b][v];
+    }
+  }
+}
+
 struct StridedWgradPlan {
   int tb, wm, wn, nch, ast, a_floats, b_floats, nal, nbl, pws, pch, nq2;
+  bool spec;  // a compile-time specialised instance exists for this shape
   size_t lds;
 };
 
@@ -854,7 +1019,12 @@ static bool strided_wgrad_plan(int batch, int d, int n, int ks, int stride, int 
           pl->lds = lds;
         }
       }
-  return best_cost >= 0;
+  if (best_cost < 0) return false;
+  // conv1 of AlexNet / CaffeNet: 11 x 11, stride 4, no padding, 53..56 pixels per output row, a spare column
+  pl->spec = ks == 11 && stride == 4 && pad == 0 && pl->tb == 3 && pl->nq2 == 14 && pl->nal == 8 && pl->nbl == 11 &&
+             ncols % 32 != 0 && !tuning().direct_nospec;
+  if (pl->spec) pl->lds += kSWgradOnes * sizeof(float);
+  return pl->lds <= 160 * 1024;
 }
 
 template <int KS, int S>
@@ -920,7 +1090,15 @@ static int conv_strided_wgrad(float *dw, float *db, const float *dout, const flo
   }
   hipStream_t st = ctx().stream;
   int rc;
-  if (ks == 11) rc = strided_wgrad_launch<11, 4>(g, pl, st);
+  if (pl.spec) {
+    auto kern = conv_strided_wgrad_spec_kernel<11, 4, 3, 14, 8, 11>;
+    static LdsGrant grant;
+    if (int rc2 = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc2;
+    hipLaunchKernelGGL(kern, dim3(g.nblocks), dim3(64 * pl.wm * pl.wn), pl.lds, st, g);
+    CCT_LAUNCH_CHECK();
+    note_kernel("conv_strided_wgrad_spec_kernel<11,4,3,14,8,11> waves=%dx%d", pl.wm, pl.wn);
+    rc = 0;
+  } else if (ks == 11) rc = strided_wgrad_launch<11, 4>(g, pl, st);
   else if (ks == 7) rc = strided_wgrad_launch<7, 2>(g, pl, st);
   else if (ks == 5) rc = strided_wgrad_launch<5, 2>(g, pl, st);
   else rc = strided_wgrad_launch<3, 2>(g, pl, st);
