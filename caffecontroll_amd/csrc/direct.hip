@@ -652,13 +652,16 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
 // of their own.  Differences from the generic kernel: each wavefront stages its own 32 rows of the
 // dout slab (private, padded to whole 64-word loads), and the prefetch is unconditional -- the
 // last step of a range re-fetches itself into the idle stage.
-template <int KS, int TB, int PW, int HO, int W>
-__global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const WgradArgs g) {
-  constexpr int KK = KS * KS, BN = 32 * TB;
+// With WN > 1 the workgroup is a W x WN grid of wavefronts: W row blocks times WN column groups of TB
+// blocks each (192 maps = six row blocks then run as twelve wavefronts, three on every SIMD, instead
+// of six wavefronts that leave two SIMDs half idle).
+template <int KS, int TB, int PW, int HO, int W, int WN = 1>
+__global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(const WgradArgs g) {
+  constexpr int KK = KS * KS, BN = 32 * TB * WN, NT = 64 * W * WN;
   constexpr int PWS = WgradStrides<KS, PW>::PWS, PCH = WgradStrides<KS, PW>::PCH;
   constexpr int NCH = (BN - 1) / KK + 2;
-  constexpr int BSZ = (NCH * PCH + 64 * W - 1) / (64 * W) * (64 * W);  // patch floats: whole passes
-  constexpr int NBW = BSZ / (64 * W);                                   // patch loads per lane per step
+  constexpr int BSZ = (NCH * PCH + NT - 1) / NT * NT;  // patch floats: whole passes
+  constexpr int NBW = BSZ / NT;                        // patch loads per lane per step
   // dout never passes through LDS: lane (r, h) of a wavefront is the only reader of row y of map r
   // of image h, so it fetches that row itself, as NQD 16-byte buffer loads (runs of four floats;
   // the last run starts at HO - 4 and overlaps its neighbour when HO is not a multiple of 4) one
@@ -672,7 +675,8 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   extern __shared__ __attribute__((aligned(16))) float smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wave_id = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = WN == 1 ? 0 : wave_id / W, wave = wave_id - wn * W;  // column group, row block
   const int r = lane & 31, h = lane >> 5;
   const uint32_t flat = xcd_remap(blockIdx.x, g.nblocks);
   const uint32_t z = flat / g.ntiles, id = flat - z * g.ntiles;
@@ -688,7 +692,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   uint32_t boff[NBW], bmeta[NBW];
 #pragma unroll
   for (int k = 0; k < NBW; ++k) {
-    const uint32_t e = (uint32_t)(k * 64 * W + tid);
+    const uint32_t e = (uint32_t)(k * NT + tid);
     const uint32_t ch = e / PCH, rem = e - ch * PCH;
     const uint32_t prow = rem / PWS, pcol = rem - prow * PWS;
     const uint32_t second = prow >= (uint32_t)KS ? 1u : 0u, kr = prow - second * KS;
@@ -703,7 +707,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   int bbase[TB];
 #pragma unroll
   for (int b = 0; b < TB; ++b) {
-    const int col = min(n0 + b * 32 + r, g.ncols - 1);
+    const int col = min(n0 + (wn * TB + b) * 32 + r, g.ncols - 1);
     const int c = col / KK, j = col - c * KK, kr = j / KS, kc = j - kr * KS;
     bbase[b] = (c - ch0) * PCH + (h * KS + kr) * PWS + kc;
   }
@@ -735,7 +739,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
     const int srow_ = y_ - g.pad + (int)(mt_ & 15u);                                              \
     const bool ok_ = (mt_ & 32u) && (unsigned)srow_ < (unsigned)g.hs && (two_ || !(mt_ & 16u));   \
     lds_dma4(b_rsrc, ok_ ? boff[k] + row0_ : kOutOfRange, gb_,                                    \
-             smem + (st) * STAGE + (k) * 64 * W + wave * 64);                                     \
+             smem + (st) * STAGE + (k) * NT + wave_id * 64);                                     \
   } while (0)
 
   f4 an[NQD];  // this lane's dout row of the coming step
@@ -823,7 +827,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
 #undef CCT_WSPEC_A
 #undef CCT_WSPEC_B
 
-  if (g.out_bias && tn == 0) {
+  if (g.out_bias && tn == 0 && wn == 0) {
     // the two images of the pairs sit in the two lane halves; only the first column tile reports
     const float both = bsum + __shfl_xor(bsum, 32);
     const int row = m0 + wave * 32 + r;
@@ -832,7 +836,7 @@ __global__ __launch_bounds__(64 * W) void conv_direct_wgrad_spec_kernel(const Wg
   float *out = g.out + (size_t)z * g.o * g.ncols;
 #pragma unroll
   for (int b = 0; b < TB; ++b) {
-    const int col = n0 + b * 32 + r;
+    const int col = n0 + (wn * TB + b) * 32 + r;
     if (col >= g.ncols) continue;
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
@@ -877,6 +881,7 @@ int reduce_partial_sums(float *dst, const float *ws, uint32_t n, float *dst2, co
 
 struct WgradPlan {
   int waves, tb, pw, ast, a_floats, stage;
+  int wn;  // column groups of the workgroup's wavefront grid (specialised instances only, else 1)
   bool spec;  // a compile-time specialised instance exists for this shape
   size_t lds;
 };
@@ -929,26 +934,36 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
              (ks == 3 && ho == 13 && pl->pw == 16 && pl->tb == 6 &&
               (pl->waves == 4 || pl->waves == 6 || pl->waves == 8));
   if (tuning().direct_nospec) pl->spec = false;  // tuning override
+  pl->wn = 1;
+  int nch_spec = nch;
   if (pl->spec) {
+    // six row blocks: twelve wavefronts (six row blocks x two column groups of three blocks)
+    if (pl->waves == 6) {
+      pl->wn = 2;
+      pl->tb = 3;
+      nch_spec = (32 * pl->tb * pl->wn - 1) / (ks * ks) + 2;
+    }
     // layout of conv_direct_wgrad_spec_kernel: dout stays out of LDS, patches in whole passes
+    const int nt = 64 * pl->waves * pl->wn;
     pl->a_floats = 0;
-    pl->stage = (nch * pch + 64 * pl->waves - 1) / (64 * pl->waves) * (64 * pl->waves);
+    pl->stage = (nch_spec * pch + nt - 1) / nt * nt;
   }
   // fragment loads may run a few words past the last patch row: the padding of the patch region
   // absorbs that, else a little slack is added
-  const int tail_pad = pl->stage - pl->a_floats - nch * pch;
+  const int tail_pad = pl->stage - pl->a_floats - nch_spec * pch;
   pl->lds = (size_t)(2 * pl->stage + (tail_pad >= 8 ? 0 : 16)) * sizeof(float);
   return pl->lds <= 160 * 1024;
 }
 
-template <int KS, int TB, int PW, int HO, int W>
+template <int KS, int TB, int PW, int HO, int W, int WN = 1>
 static int wgrad_launch_spec(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
-  auto kern = conv_direct_wgrad_spec_kernel<KS, TB, PW, HO, W>;
+  auto kern = conv_direct_wgrad_spec_kernel<KS, TB, PW, HO, W, WN>;
   static LdsGrant grant;
   if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;
-  hipLaunchKernelGGL(kern, dim3(g.nblocks), dim3(64 * W), pl.lds, st, g);
+  hipLaunchKernelGGL(kern, dim3(g.nblocks), dim3(64 * W * WN), pl.lds, st, g);
   CCT_LAUNCH_CHECK();
-  note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d>", KS, TB, PW, HO, W);
+  if (WN == 1) note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d>", KS, TB, PW, HO, W);
+  else note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d,%d>", KS, TB, PW, HO, W, WN);
   return 0;
 }
 
@@ -994,12 +1009,12 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   g.ast = pl.ast; g.bm = 32 * pl.waves; g.a_floats = pl.a_floats; g.stage = pl.stage;
   g.steps_total = ((batch + 1) / 2) * g.ho;
   g.tiles_m = (uint32_t)((o + g.bm - 1) / g.bm);
-  g.tiles_n = (uint32_t)((g.ncols + 32 * pl.tb - 1) / (32 * pl.tb));
+  g.tiles_n = (uint32_t)((g.ncols + 32 * pl.tb * pl.wn - 1) / (32 * pl.tb * pl.wn));
   g.ntiles = g.tiles_m * g.tiles_n;
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
   // workgroups resident per compute unit: LDS and wavefront slots (two per SIMD is plenty here)
   int per_cu = (int)((160 * 1024) / pl.lds);
-  if (per_cu > 8 / pl.waves) per_cu = 8 / pl.waves;
+  if (per_cu > 8 / (pl.waves * pl.wn)) per_cu = 8 / (pl.waves * pl.wn);
   if (per_cu < 1) per_cu = 1;
   int splits = (int)((long)per_cu * cus / g.ntiles);
   if (splits < 1) splits = 1;
@@ -1026,7 +1041,7 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
     rc = pl.waves == 8 ? wgrad_launch_spec<5, 5, 32, 27, 8>(g, pl, st) : wgrad_launch_spec<5, 5, 32, 27, 4>(g, pl, st);
   else if (pl.spec)
     rc = pl.waves == 8   ? wgrad_launch_spec<3, 6, 16, 13, 8>(g, pl, st)
-         : pl.waves == 6 ? wgrad_launch_spec<3, 6, 16, 13, 6>(g, pl, st)
+         : pl.waves == 6 ? wgrad_launch_spec<3, 3, 16, 13, 6, 2>(g, pl, st)
                          : wgrad_launch_spec<3, 6, 16, 13, 4>(g, pl, st);
   else if (ks == 5) rc = pl.pw == 16 ? wgrad_launch<5, 16>(g, pl, st) : wgrad_launch<5, 32>(g, pl, st);
   else rc = pl.pw == 16 ? wgrad_launch<3, 16>(g, pl, st) : wgrad_launch<3, 32>(g, pl, st);
