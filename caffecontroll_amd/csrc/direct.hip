@@ -50,6 +50,8 @@ struct DirectArgs {
   uint32_t ptot;      // batch * ho * ho
   uint32_t tiles_m, ntiles;
   FastDiv div_ho, div_ho2, div_hp, div_pr;
+  int cs;             // 16-row kernel: floats between the channels of a patch (pr * PW + 16)
+  FastDiv div_cs;
 };
 
 constexpr int kDirectPatchLoads = 8;  // source elements per lane per step, at most
@@ -243,6 +245,181 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
   }
 }
 
+// The same convolution on 16-row MFMA tiles (v_mfma_f32_16x16x4_f32: 16 maps x 16 pixels, four
+// contraction indices) for map counts that 32-row blocks would pad by half a block: 48 maps (one
+// group of CaffeNet conv2's data gradient) run as three 16-row blocks instead of two 32-row blocks
+// of which a quarter is zeros.  Same slab buffer, same patch layout, same two-stage pipeline; what
+// changes is the fragment geometry: a step takes FOUR channels, lanes 16q..16q+15 hold channel q of
+// the step for map (or pixel) lane % 16, and accumulator register v of lane (r, q) is row 4*q + v,
+// column r of its 16 x 16 block.  One tile covers all maps (BM = 16*TM16) x 128*TNB pixels; a
+// wavefront owns 2*TNB blocks of 16 consecutive pixels.
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+template <int KS, int TM16, int NB, int PW>
+__device__ __forceinline__ void direct16_frags(float (&fa)[TM16], float (&fb)[NB], const float *__restrict__ sm,
+                                               int abase, const int (&bbase)[NB], int j) {
+  constexpr int KK = KS * KS;
+  const int u = j / KS, v = j % KS;
+#pragma unroll
+  for (int a = 0; a < TM16; ++a) fa[a] = sm[abase + a * (16 * KK) + j];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) fb[b] = sm[bbase[b] + u * PW + v];
+}
+
+template <int KS, int TM16, int TNB, int PW>
+__global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs g) {
+  constexpr int KK = KS * KS, BM = 16 * TM16, BN = 128 * TNB, NC = 4, NB = 2 * TNB;
+  constexpr int ASZ = NC * BM * KK;
+  constexpr int ASZP = (ASZ + 255) / 256 * 256;
+  constexpr int SLAB4 = BM * KK / 4;
+  constexpr int NA4 = (ASZP / 4 + 255) / 256;
+  constexpr int NPL = kDirectPatchLoads;
+  static_assert(BM * KK % 4 == 0, "weight slabs are copied in 16-byte vectors");
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 15, q = lane >> 4;
+  // channels of a patch lie pr*PW + 16 floats apart: the four channel groups of a fragment read
+  // then fall on two bank halves instead of one
+  const int psz = (NC * g.cs + 63) & ~63;
+  const int stage = ASZP + psz;
+
+  const uint32_t tn = xcd_remap(blockIdx.x, g.ntiles);  // one map tile: the tile id is the pixel tile
+  const uint32_t p0 = tn * BN;
+  const int ho2 = g.ho * g.ho;
+  const uint32_t img0 = fdiv(p0, g.div_ho2);
+  const uint32_t y0 = fdiv(p0 - img0 * ho2, g.div_ho);
+  const int v_lo = img0 * g.hp + y0;
+
+  uint32_t aoff[NA4];
+#pragma unroll
+  for (int i = 0; i < NA4; ++i) {
+    const int e4 = tid + i * 256;
+    const int c = e4 / SLAB4, f = (e4 - c * SLAB4) * 4;
+    aoff[i] = (uint32_t)(c * g.slab_stride + f) * 4u;
+  }
+  uint32_t psrc[NPL], psrc_last[NPL];
+  const int last_channels = g.kc - (g.nsteps - 1) * NC;
+#pragma unroll
+  for (int i = 0; i < NPL; ++i) {
+    const uint32_t e = tid + i * 256;
+    const uint32_t c = fdiv(e, g.div_cs), rem = e - c * g.cs;
+    const uint32_t prow = rem / PW, pc = rem % PW;
+    const uint32_t v = v_lo + prow;
+    const uint32_t img = fdiv(v, g.div_hp);
+    const int srow = (int)(v - img * g.hp) - g.pad, scol = (int)pc - g.pad;
+    const bool ok = c < (uint32_t)NC && prow < (uint32_t)g.pr && img < (uint32_t)g.batch && (unsigned)srow < (unsigned)g.hs &&
+                    (unsigned)scol < (unsigned)g.hs;
+    psrc[i] = ok ? (img * g.src_img_stride + (c * g.hs + srow) * g.hs + scol) * 4u : kOutOfRange;
+    psrc_last[i] = (ok && (int)c < last_channels) ? psrc[i] : kOutOfRange;
+  }
+  const uint32_t a_step = (uint32_t)NC * g.slab_stride * 4u, b_step = (uint32_t)NC * g.hs * g.hs * 4u;
+  const rsrc_t a_rsrc = make_rsrc(g.wt), b_rsrc = make_rsrc(g.src);
+  const int wave_elem0 = wave * 64;
+
+#define CCT_DIRECT16_ISSUE(t, s)                                                               \
+  do {                                                                                         \
+    float *st_ = smem + (s) * stage;                                                           \
+    const uint32_t ga_ = (uint32_t)(t) * a_step, gb_ = (uint32_t)(t) * b_step;                 \
+    _Pragma("unroll") for (int i = 0; i < NA4; ++i) {                                          \
+      if (i * 256 + wave_elem0 < ASZP / 4)                                                     \
+        lds_dma16(a_rsrc, (i * 256 + tid < ASZ / 4) ? aoff[i] : kOutOfRange, ga_,              \
+                  st_ + (i * 256 + wave_elem0) * 4);                                           \
+    }                                                                                          \
+    const bool last_ = (t) == g.nsteps - 1;                                                    \
+    _Pragma("unroll") for (int i = 0; i < NPL; ++i) {                                          \
+      if (i * 256 + wave_elem0 < psz)                                                          \
+        lds_dma4(b_rsrc, last_ ? psrc_last[i] : psrc[i], gb_, st_ + ASZP + i * 256 + wave_elem0); \
+    }                                                                                          \
+  } while (0)
+
+  const int abase = q * (BM * KK) + r * KK;
+  int bbase[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    uint32_t p = p0 + wave * (32 * TNB) + b * 16 + r;
+    p = min(p, g.ptot - 1);
+    const uint32_t img = fdiv(p, g.div_ho2);
+    const uint32_t pix = p - img * ho2;
+    const uint32_t y = fdiv(pix, g.div_ho), x = pix - y * g.ho;
+    bbase[b] = ASZP + q * g.cs + (int)(img * g.hp + y - v_lo) * PW + (int)x;
+  }
+
+  v4f acc[TM16][NB];
+#pragma unroll
+  for (int a = 0; a < TM16; ++a)
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[a][b][e] = 0.0f;
+
+  CCT_DIRECT16_ISSUE(0, 0);
+  lds_dma_wait();
+  __syncthreads();
+
+  for (int t = 0; t < g.nsteps; ++t) {
+    const float *sm = smem + (t & 1) * stage;
+    if (t + 1 < g.nsteps) CCT_DIRECT16_ISSUE(t + 1, (t & 1) ^ 1);
+    // taps two at a time (neighbouring taps sit in neighbouring LDS words); the fragments of pair
+    // n+1 are requested before the MFMAs of pair n
+    constexpr int NI = KK, NQ = (NI + 1) / 2;
+    float fa[2][2][TM16], fb[2][2][NB];
+    direct16_frags<KS, TM16, NB, PW>(fa[0][0], fb[0][0], sm, abase, bbase, 0);
+    direct16_frags<KS, TM16, NB, PW>(fa[0][1], fb[0][1], sm, abase, bbase, 1);
+#pragma unroll
+    for (int n = 0; n < NQ; ++n) {
+      const int nb = (n + 1) & 1, cb = n & 1;
+      if (2 * n + 2 < NI) direct16_frags<KS, TM16, NB, PW>(fa[nb][0], fb[nb][0], sm, abase, bbase, 2 * n + 2);
+      if (2 * n + 3 < NI) direct16_frags<KS, TM16, NB, PW>(fa[nb][1], fb[nb][1], sm, abase, bbase, 2 * n + 3);
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        if (2 * n + e < NI) {
+#pragma unroll
+          for (int a2 = 0; a2 < TM16; ++a2)
+#pragma unroll
+            for (int b2 = 0; b2 < NB; ++b2)
+              acc[a2][b2] = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[cb][e][a2], fb[cb][e][b2], acc[a2][b2], 0, 0, 0);
+        }
+      }
+      {
+        constexpr int NR = TM16 + NB, NM = 2 * TM16 * NB, PER = NM / (NR + 1) > 0 ? NM / (NR + 1) : 1;
+#pragma unroll
+        for (int k2 = 0; k2 < NR; ++k2) {
+          __builtin_amdgcn_sched_group_barrier(0x008, PER, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, NM - NR * PER > 0 ? NM - NR * PER : 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    lds_dma_wait();
+    __syncthreads();
+  }
+#undef CCT_DIRECT16_ISSUE
+
+  // ---- epilogue: accumulator register v of lane (r, q) is row 4*q + v, column r ----
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const uint32_t p = p0 + wave * (32 * TNB) + b * 16 + r;
+    if (p >= g.ptot) continue;
+    const uint32_t img = fdiv(p, g.div_ho2);
+    const size_t pix = (size_t)img * g.dst_img_stride + (p - img * ho2);
+    float *out = g.dst + pix;
+#pragma unroll
+    for (int a = 0; a < TM16; ++a)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int row = a * 16 + 4 * q + v;
+        if (row < g.mtot) {
+          float y = acc[a][b][v] + (g.bias ? g.bias[row] : 0.f);
+          if (g.mask && !(g.mask[pix + (size_t)row * ho2] > 0.f)) y = 0.f;
+          out[(size_t)row * ho2] = (g.relu && !(y > 0.f)) ? 0.f : y;
+        }
+      }
+  }
+}
+
 // Output-map tile (in 32-row blocks) for `mtot` maps: least padding, larger tile on ties.
 static int direct_tmb(int mtot) {
   int tmb = 4;
@@ -278,8 +455,16 @@ __global__ __launch_bounds__(256) void direct_slab_kernel(float *__restrict__ wt
 
 struct DirectPlan {
   int ks, tmb, tnb, cp, pw, pr;
+  int tm16;  // > 0: the 16-row kernel with this many row blocks (one map tile); tmb is unused then
   size_t lds;
 };
+
+// 16-row blocks of a map count that 32-row blocks would pad by half a block, if the 16-row kernel has
+// an instance for it (1, 3 or 5 blocks in a single tile), else 0.
+static int direct_tm16(int mtot) {
+  const int blocks16 = (mtot + 15) / 16;
+  return (blocks16 & 1) && blocks16 <= 5 ? blocks16 : 0;
+}
 
 // Chooses the kernel instance for a geometry; returns false when the direct path does not cover it.
 static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, DirectPlan *pl) {
@@ -295,8 +480,22 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   const long ptot = (long)batch * ho * ho;
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
   const int padded = direct_padded_maps(mtot);
-  // tuning override "<map blocks><pixel blocks>", e.g. 22
+  // tuning override "<map blocks><pixel blocks>", e.g. 22; 161 / 162 = the 16-row kernel with 128 / 256 pixels
   const int forced = tuning().direct_tile;
+  pl->tm16 = 0;
+  if (const int tm16 = direct_tm16(mtot); tm16 && (forced == 0 || forced == 161 || forced == 162)) {
+    for (int tnb = forced == 161 ? 1 : 2; tnb >= (forced == 162 ? 2 : 1); --tnb) {
+      const int bn = 128 * tnb;
+      const int rows = (ho - 1 + bn - 1) / ho + 1, imgs = (ho * ho - 1 + bn - 1) / (ho * ho) + 1;
+      const int pr = rows - 1 + (imgs - 1) * (ks - 1) + ks;
+      const long patch = 4L * (pr * pw + 16);
+      const size_t lds =
+          2 * (size_t)((4 * 16 * tm16 * ks * ks + 255) / 256 * 256 + (patch + 63) / 64 * 64) * sizeof(float);
+      if (patch > 256L * kDirectPatchLoads || lds > 64 * 1024) continue;
+      pl->ks = ks; pl->tmb = 0; pl->tnb = tnb; pl->cp = 2; pl->pw = pw; pl->pr = pr; pl->tm16 = tm16; pl->lds = lds;
+      return true;
+    }
+  }
   // Candidate tiles: map tiles that divide the padded map count (the slab layout does not depend
   // on the choice), 128 or 256 pixels.  Estimated time, in units of one 32x128 block on a whole
   // compute unit: workgroups are handed out as residency slots free up, so the launch runs as
@@ -347,6 +546,7 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
       pick = &cand[i];
   }
   *pl = pick->plan;
+  pl->tm16 = 0;
   return true;
 }
 
@@ -364,6 +564,22 @@ static int direct_launch_ks(const DirectArgs &g, const DirectPlan &pl, hipStream
   CCT_DIRECT_CASE(1, 2) CCT_DIRECT_CASE(2, 2) CCT_DIRECT_CASE(3, 2) CCT_DIRECT_CASE(4, 2)
 #undef CCT_DIRECT_CASE
   return set_error(CCT_HIP_EINVAL, "conv_direct: no kernel instance for tile %dx%d", pl.tmb, pl.tnb);
+}
+
+template <int KS, int PW>
+static int direct_launch16(const DirectArgs &g, const DirectPlan &pl, hipStream_t st) {
+  dim3 grid(g.ntiles), block(256);
+#define CCT_DIRECT16_CASE(TM16, TNB)                                                                   \
+  if (pl.tm16 == TM16 && pl.tnb == TNB) {                                                              \
+    hipLaunchKernelGGL((conv_direct16_kernel<KS, TM16, TNB, PW>), grid, block, pl.lds, st, g);         \
+    CCT_LAUNCH_CHECK();                                                                                \
+    note_kernel("conv_direct16_kernel<%d,%d,%d,%d>", KS, TM16, TNB, PW);                               \
+    return 0;                                                                                          \
+  }
+  CCT_DIRECT16_CASE(1, 1) CCT_DIRECT16_CASE(3, 1) CCT_DIRECT16_CASE(5, 1)
+  CCT_DIRECT16_CASE(1, 2) CCT_DIRECT16_CASE(3, 2) CCT_DIRECT16_CASE(5, 2)
+#undef CCT_DIRECT16_CASE
+  return set_error(CCT_HIP_EINVAL, "conv_direct: no 16-row kernel instance for %d row blocks", pl.tm16);
 }
 
 static int conv_direct(const float *wt, const float *src, float *dst, const float *bias, int relu, int batch, int kc,
@@ -388,18 +604,24 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
   }
   g.hp = g.ho + ks - 1;
   g.pr = pl.pr;
-  g.nsteps = (kc + 2 * pl.cp - 1) / (2 * pl.cp);
+  g.nsteps = pl.tm16 ? (kc + 3) / 4 : (kc + 2 * pl.cp - 1) / (2 * pl.cp);
   CCT_REQUIRE((uintptr_t)wt % 16 == 0, "conv_direct: slab buffer must be 16-byte aligned");
   g.slab_stride = direct_padded_maps(mtot) * ks * ks;
   g.ptot = (uint32_t)((long)batch * g.ho * g.ho);
-  g.tiles_m = (uint32_t)((mtot + 32 * pl.tmb - 1) / (32 * pl.tmb));
+  g.tiles_m = pl.tm16 ? 1u : (uint32_t)((mtot + 32 * pl.tmb - 1) / (32 * pl.tmb));
   const uint32_t bn = 128 * pl.tnb;
   g.ntiles = g.tiles_m * ((g.ptot + bn - 1) / bn);
   g.div_ho = make_fastdiv((uint32_t)g.ho);
   g.div_ho2 = make_fastdiv((uint32_t)(g.ho * g.ho));
   g.div_hp = make_fastdiv((uint32_t)g.hp);
   g.div_pr = make_fastdiv((uint32_t)g.pr);
+  g.cs = g.pr * pl.pw + 16;
+  g.div_cs = make_fastdiv((uint32_t)g.cs);
   hipStream_t st = ctx().stream;
+  if (pl.tm16) {
+    if (ks == 5) return pl.pw == 16 ? direct_launch16<5, 16>(g, pl, st) : direct_launch16<5, 32>(g, pl, st);
+    return pl.pw == 16 ? direct_launch16<3, 16>(g, pl, st) : direct_launch16<3, 32>(g, pl, st);
+  }
   if (ks == 5) return pl.pw == 16 ? direct_launch_ks<5, 1, 16>(g, pl, st) : direct_launch_ks<5, 1, 32>(g, pl, st);
   return pl.pw == 16 ? direct_launch_ks<3, 2, 16>(g, pl, st) : direct_launch_ks<3, 2, 32>(g, pl, st);
 }
