@@ -93,6 +93,10 @@ PROTOTYPES = {
     "cct_hip_conv_strided_slabs": [_P, _P, _I, _I, _I, _I, _I],
     "cct_hip_conv_strided_forward": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I],
     "cct_hip_conv_strided_backward_weights": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I],
+    "cct_hip_conv_strided_backward_data_supported": [_I, _I, _I, _I, _I, _I, _I],
+    "cct_hip_conv_strided_backward_data_slab_floats": [_I, _I, _I, _I],
+    "cct_hip_conv_strided_backward_data_slabs": [_P, _P, _I, _I, _I, _I],
+    "cct_hip_conv_strided_backward_data": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I],
     "cct_hip_sgemv": [_I, _I, _I, _F, _P, _P, _F, _P],
     "cct_hip_math_saxpy": [_Z, _F, _P, _P],
     "cct_hip_math_saxpby": [_Z, _F, _P, _F, _P],
@@ -130,7 +134,8 @@ PROTOTYPES = {
     "cct_hip_timer_elapsed_ms": [_P, C.POINTER(_F)],
 }
 _RESTYPE = {"cct_hip_last_error": C.c_char_p, "cct_hip_last_kernel": C.c_char_p, "cct_hip_conv_direct_slab_floats": C.c_size_t,
-            "cct_hip_conv_strided_slab_floats": C.c_size_t}
+            "cct_hip_conv_strided_slab_floats": C.c_size_t,
+            "cct_hip_conv_strided_backward_data_slab_floats": C.c_size_t}
 
 _lib = None
 

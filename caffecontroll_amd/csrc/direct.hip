@@ -52,7 +52,13 @@ struct DirectArgs {
   FastDiv div_ho, div_ho2, div_hp, div_pr;
   int cs;             // 16-row kernel: floats between the channels of a patch (pr * PW + 16)
   FastDiv div_cs;
+  // 16-row kernel, data gradient of a strided layer: the output maps are (channel, row phase, column
+  // phase) triples of the layer's input gradient, pixel (I, J) of map (c, pi, pj) is stored at
+  // dst[img][c][S*I + pi - spad][S*J + pj - spad] of a [batch][sd][shs][shs] tensor (ss = S; 0 = plain output)
+  int ss, shs, spad, sd;
 };
+
+constexpr int kDirect16PatchLoads = 10;  // the 16-row kernel stages four channels per step
 
 constexpr int kDirectPatchLoads = 8;  // source elements per lane per step, at most
 
@@ -273,7 +279,7 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
   constexpr int ASZP = (ASZ + 255) / 256 * 256;
   constexpr int SLAB4 = BM * KK / 4;
   constexpr int NA4 = (ASZP / 4 + 255) / 256;
-  constexpr int NPL = kDirectPatchLoads;
+  constexpr int NPL = kDirect16PatchLoads;
   static_assert(BM * KK % 4 == 0, "weight slabs are copied in 16-byte vectors");
   extern __shared__ __attribute__((aligned(16))) float smem[];
 
@@ -399,6 +405,48 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
 #undef CCT_DIRECT16_ISSUE
 
   // ---- epilogue: accumulator register v of lane (r, q) is row 4*q + v, column r ----
+  if (g.ss) {
+    // maps are (channel, row phase, column phase) of a strided layer's input gradient
+    const int S = g.ss, S2 = S * S, shs2 = g.shs * g.shs;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      const uint32_t p = p0 + wave * (32 * TNB) + b * 16 + r;
+      if (p >= g.ptot) continue;
+      const uint32_t img = fdiv(p, g.div_ho2);
+      const uint32_t pix = p - img * ho2;
+      const int I = (int)fdiv(pix, g.div_ho), J = (int)pix - I * g.ho;
+      float *out = g.dst + (size_t)img * g.sd * shs2;
+#pragma unroll
+      for (int a = 0; a < TM16; ++a) {
+        const int row0 = a * 16 + 4 * q;  // this lane's four rows: row0 .. row0 + 3
+        if (S == 4) {
+          // rows 4*q .. 4*q+3 of block a are the four column phases of (channel a, row phase q): four
+          // consecutive floats of one image row
+          const int i = 4 * I + q - g.spad, j0 = 4 * J - g.spad;
+          if (a >= g.sd || (unsigned)i >= (unsigned)g.shs) continue;
+          float *o = out + ((size_t)a * g.shs + i) * g.shs + j0;
+          if (j0 >= 0 && j0 + 3 < g.shs) {
+            *reinterpret_cast<v4f *>(o) = acc[a][b];
+          } else {
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+              if ((unsigned)(j0 + v) < (unsigned)g.shs) o[v] = acc[a][b][v];
+          }
+        } else {
+#pragma unroll
+          for (int v = 0; v < 4; ++v) {
+            const int row = row0 + v;
+            if (row >= g.mtot) continue;
+            const int c = row / S2, rem = row - c * S2, pi = rem / S, pj = rem - pi * S;
+            const int i = S * I + pi - g.spad, j = S * J + pj - g.spad;
+            if ((unsigned)i < (unsigned)g.shs && (unsigned)j < (unsigned)g.shs)
+              out[((size_t)c * g.shs + i) * g.shs + j] = acc[a][b][v];
+          }
+        }
+      }
+    }
+    return;
+  }
 #pragma unroll
   for (int b = 0; b < NB; ++b) {
     const uint32_t p = p0 + wave * (32 * TNB) + b * 16 + r;
@@ -472,7 +520,8 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   if (pad < 0 || pad > ks - 1 || batch <= 0 || kc <= 0 || mtot <= 0) return false;
   const int ho = hs + 2 * pad - ks + 1, hp = ho + ks - 1;
   if (ho <= 0) return false;
-  const int pw = hp <= 16 ? 16 : 32;
+  // padded rows of up to 32 floats; up to 64 on the 16-row kernel
+  const int pw = hp <= 16 ? 16 : hp <= 32 ? 32 : 64;
   if (hp > pw) return false;
   // buffer loads address a tensor through 32-bit byte offsets
   if ((double)batch * kc * hs * hs >= 1073741824.0 || (double)batch * ho * ho >= 2147483648.0) return false;
@@ -491,11 +540,12 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
       const long patch = 4L * (pr * pw + 16);
       const size_t lds =
           2 * (size_t)((4 * 16 * tm16 * ks * ks + 255) / 256 * 256 + (patch + 63) / 64 * 64) * sizeof(float);
-      if (patch > 256L * kDirectPatchLoads || lds > 64 * 1024) continue;
+      if (patch > 256L * kDirect16PatchLoads || lds > 64 * 1024) continue;
       pl->ks = ks; pl->tmb = 0; pl->tnb = tnb; pl->cp = 2; pl->pw = pw; pl->pr = pr; pl->tm16 = tm16; pl->lds = lds;
       return true;
     }
   }
+  if (pw > 32) return false;  // the 32-row kernel has no instance for rows that wide
   // Candidate tiles: map tiles that divide the padded map count (the slab layout does not depend
   // on the choice), 128 or 256 pixels.  Estimated time, in units of one 32x128 block on a whole
   // compute unit: workgroups are handed out as residency slots free up, so the launch runs as
@@ -582,13 +632,25 @@ static int direct_launch16(const DirectArgs &g, const DirectPlan &pl, hipStream_
   return set_error(CCT_HIP_EINVAL, "conv_direct: no 16-row kernel instance for %d row blocks", pl.tm16);
 }
 
+// Phase store of a strided layer's data gradient (see DirectArgs::ss)
+struct DirectShuffle {
+  int s, hs, pad, d;
+};
+
 static int conv_direct(const float *wt, const float *src, float *dst, const float *bias, int relu, int batch, int kc,
                        int mtot, int hs, int ks, int pad, size_t src_img_stride, size_t dst_img_stride,
-                       const float *mask = nullptr) {
+                       const float *mask = nullptr, const DirectShuffle *shuffle = nullptr) {
   DirectPlan pl;
   CCT_REQUIRE(direct_plan(batch, kc, mtot, hs, ks, pad, &pl),
               "conv_direct: geometry not covered (k=%d pad=%d size=%d)", ks, pad, hs);
+  CCT_REQUIRE(!shuffle || pl.tm16, "conv_direct: the phase store needs the 16-row kernel");
   DirectArgs g;
+  g.ss = g.shs = g.spad = g.sd = 0;
+  if (shuffle) {
+    g.ss = shuffle->s; g.shs = shuffle->hs; g.spad = shuffle->pad; g.sd = shuffle->d;
+    CCT_REQUIRE((double)batch * shuffle->d * shuffle->hs * shuffle->hs < 1073741824.0,
+                "conv_direct: phase-store tensor too large");
+  }
   g.wt = wt; g.src = src; g.dst = dst; g.bias = bias; g.relu = relu; g.mask = mask;
   g.batch = batch; g.kc = kc; g.mtot = mtot; g.hs = hs; g.pad = pad;
   g.ho = hs + 2 * pad - ks + 1;
@@ -619,8 +681,11 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
   g.div_cs = make_fastdiv((uint32_t)g.cs);
   hipStream_t st = ctx().stream;
   if (pl.tm16) {
-    if (ks == 5) return pl.pw == 16 ? direct_launch16<5, 16>(g, pl, st) : direct_launch16<5, 32>(g, pl, st);
-    return pl.pw == 16 ? direct_launch16<3, 16>(g, pl, st) : direct_launch16<3, 32>(g, pl, st);
+    if (ks == 5)
+      return pl.pw == 16 ? direct_launch16<5, 16>(g, pl, st)
+                         : pl.pw == 32 ? direct_launch16<5, 32>(g, pl, st) : direct_launch16<5, 64>(g, pl, st);
+    return pl.pw == 16 ? direct_launch16<3, 16>(g, pl, st)
+                       : pl.pw == 32 ? direct_launch16<3, 32>(g, pl, st) : direct_launch16<3, 64>(g, pl, st);
   }
   if (ks == 5) return pl.pw == 16 ? direct_launch_ks<5, 1, 16>(g, pl, st) : direct_launch_ks<5, 1, 32>(g, pl, st);
   return pl.pw == 16 ? direct_launch_ks<3, 2, 16>(g, pl, st) : direct_launch_ks<3, 2, 32>(g, pl, st);
@@ -1275,6 +1340,55 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   return 0;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Data gradient of a STRIDED layer (stride S, kernel K) as a stride-1 convolution of the output
+// gradient.  Write an input coordinate (in the zero-padded image) as i = S*I + pi: the taps that
+// reach it are u = pi + S*a, a = 0 .. ceil(K/S) - 1, from output row I - a.  So each of the S*S
+// (row phase, column phase) sub-images of every input channel is a small stride-1 convolution of
+// the output gradient with its own KA x KA filter (KA = ceil(K/S), zero where pi + S*a >= K):
+//   V[(c,pi,pj)][I][J] = sum_{m,a,b} w[m][c][pi + S*a][pj + S*b] * dout[m][I - a][J - b]
+// which is conv_direct16_kernel's sum with d*S*S output maps, contraction over the layer's output
+// maps, padding KA - 1 and reversed filters; the kernel's store puts V back at
+// [c][S*I + pi - pad][S*J + pj - pad].  It replaces the gradient remap, the data-gradient GEMM, its
+// (k*k*d) x (m*m*b) result and the lifting of ConvolutionBridge::backward.
+//
+// Slab buffer for it: wt[m][vm][u*KA + v] = w[m][c][pi + S*(KA-1-u)][pj + S*(KA-1-v)] with
+// vm = (c*S + pi)*S + pj, zero for taps past the filter and for padding maps / channels.
+__global__ __launch_bounds__(256) void strided_dgrad_slab_kernel(float *__restrict__ wt, const float *__restrict__ w,
+                                                                 int n_o, int n_d, int ks, int stride, int ka,
+                                                                 int p_m, uint32_t total, FastDiv div_kk,
+                                                                 FastDiv div_m) {
+  const uint32_t e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= total) return;
+  const int kk = ka * ka, s2 = stride * stride;
+  const uint32_t mv = fdiv(e, div_kk), t = e - mv * kk;
+  const uint32_t m = fdiv(mv, div_m), vm = mv - m * p_m;
+  float val = 0.f;
+  if (m < (uint32_t)n_o && vm < (uint32_t)(n_d * s2)) {
+    const int c = vm / s2, rem = vm - c * s2, pi = rem / stride, pj = rem - pi * stride;
+    const int u = t / ka, v = t - u * ka;
+    const int uu = pi + stride * (ka - 1 - u), vv = pj + stride * (ka - 1 - v);
+    if (uu < ks && vv < ks) val = w[(((size_t)m * n_d + c) * ks + uu) * ks + vv];
+  }
+  wt[e] = val;
+}
+
+// KA of a (kernel size, stride) pair the phase decomposition covers: 3 or 5, or 0
+static int strided_dgrad_ka(int ks, int stride) {
+  if (stride < 2 || ks < stride) return 0;
+  const int taps = (ks + stride - 1) / stride;
+  return taps <= 3 ? 3 : taps <= 5 ? 5 : 0;
+}
+
+static bool strided_dgrad_plan(int batch, int d, int n, int ks, int stride, int pad, int o, DirectPlan *pl) {
+  const int ka = strided_dgrad_ka(ks, stride);
+  if (!ka || batch <= 0 || d <= 0 || o <= 0 || pad < 0 || pad >= ks || n + 2 * pad < ks) return false;
+  const int ho = (n + 2 * pad - ks) / stride + 1;
+  if (tuning().direct_tile != 0 && tuning().direct_tile != 161 && tuning().direct_tile != 162) return false;
+  if ((double)batch * d * n * n >= 1073741824.0) return false;
+  return direct_plan(batch, o, d * stride * stride, ho, ka, ka - 1, pl) && pl->tm16 > 0;
+}
+
 }  // namespace cct
 
 using namespace cct;
@@ -1358,4 +1472,53 @@ extern "C" int cct_hip_conv_direct_backward_weights(float *model_grad, float *bi
   CCT_REQUIRE(batch > 0, "conv_direct_backward_weights: empty batch");
   return conv_direct_wgrad(model_grad, bias_grad, output_grad, input, batch, depth, n, k, padding, num_outputs,
                            input_image_stride, output_image_stride);
+}
+
+extern "C" int cct_hip_conv_strided_backward_data_supported(int batch, int depth, int n, int k, int stride,
+                                                            int padding, int num_outputs) {
+  if (ensure_init() != 0) return 0;
+  DirectPlan pl;
+  return strided_dgrad_plan(batch, depth, n, k, stride, padding, num_outputs, &pl) ? 1 : 0;
+}
+
+extern "C" size_t cct_hip_conv_strided_backward_data_slab_floats(int num_outputs, int depth, int k, int stride) {
+  const int ka = strided_dgrad_ka(k, stride);
+  if (!ka || num_outputs <= 0 || depth <= 0) return 0;
+  return (size_t)direct_padded_channels(num_outputs) * direct_padded_maps(depth * stride * stride) * ka * ka;
+}
+
+extern "C" int cct_hip_conv_strided_backward_data_slabs(float *slabs, const float *model, int num_outputs, int depth,
+                                                        int k, int stride) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(slabs && model && slabs != model, "conv_strided_backward_data_slabs: null or in-place argument");
+  const int ka = strided_dgrad_ka(k, stride);
+  CCT_REQUIRE(ka && num_outputs > 0 && depth > 0, "conv_strided_backward_data_slabs: kernel size %d with stride %d is not covered", k, stride);
+  const size_t total = cct_hip_conv_strided_backward_data_slab_floats(num_outputs, depth, k, stride);
+  CCT_REQUIRE(total < (1ull << 31), "conv_strided_backward_data_slabs: model too large");
+  const int p_m = direct_padded_maps(depth * stride * stride);
+  hipLaunchKernelGGL(strided_dgrad_slab_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, ctx().stream,
+                     slabs, model, num_outputs, depth, k, stride, ka, p_m, (uint32_t)total,
+                     make_fastdiv((uint32_t)(ka * ka)), make_fastdiv((uint32_t)p_m));
+  CCT_LAUNCH_CHECK();
+  return 0;
+}
+
+extern "C" int cct_hip_conv_strided_backward_data(float *input_grad, const float *output_grad, const float *slabs,
+                                                  int batch, int depth, int n, int k, int stride, int padding,
+                                                  int num_outputs) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(input_grad && output_grad && slabs, "conv_strided_backward_data: null argument");
+  if (batch <= 0) return 0;
+  DirectPlan pl;
+  CCT_REQUIRE(strided_dgrad_plan(batch, depth, n, k, stride, padding, num_outputs, &pl),
+              "conv_strided_backward_data: geometry not covered (k=%d stride=%d pad=%d size=%d)", k, stride, padding, n);
+  const int ka = strided_dgrad_ka(k, stride);
+  const int ho = (n + 2 * padding - k) / stride + 1;
+  // rows / columns past the last one any tap reaches (the layer's floor division left them over) get no
+  // store from the kernel: their gradient is zero
+  if (stride * (ho + ka - 1) - padding < n)
+    if (int rc = cct_hip_sconstant_initialize(input_grad, (size_t)batch * depth * n * n, 0.0f)) return rc;
+  const DirectShuffle sh = {stride, n, padding, depth};
+  return conv_direct(slabs, output_grad, input_grad, nullptr, 0, batch, num_outputs, depth * stride * stride, ho, ka,
+                     ka - 1, 0, 0, nullptr, &sh);
 }

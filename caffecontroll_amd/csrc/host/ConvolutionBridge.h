@@ -19,7 +19,9 @@
 //     level 3 runs without them;
 //   * strided layers with k = 11 (stride 4) or k = 7, 5, 3 (stride 2) take level 3 with direct forward
 //     and weight-gradient kernels of their own; their data gradient (not needed for a first layer)
-//     still comes from the data-gradient GEMM and the lifting, which need no lowered input.
+//     comes from a direct kernel too where it covers the geometry (depth * stride^2 <= 80 in an odd
+//     number of 16-row blocks: AlexNet / CaffeNet conv1), else from the data-gradient GEMM and the
+//     lifting, which need no lowered input.
 #pragma once
 #include <cstdio>
 #include <cstdlib>
@@ -126,6 +128,9 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                                  (int)num_output_features);
     strided_ok_ = !direct_ok_ && p_driver->conv_strided_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride,
                                                                   (int)padding, (int)num_output_features);
+    strided_data_ok_ = strided_ok_ && p_driver->conv_strided_backward_data_supported(
+                                          (int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
+                                          (int)num_output_features);
     // Small layers (LeNet-sized) stay on the fused lowering path by default: the direct kernels'
     // fixed costs (slab re-layout, partial-sum reduction) outweigh what they save below a few GFLOP.
     const double gemm_flop = 2.0 * num_output_features * (double)(oR * oC * iB) * (double)(K * K * iD);
@@ -287,7 +292,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     const bool direct_weights = path_ == PATH_DIRECT_ALL;
     // a strided layer on the all-direct path that must hand back an input gradient: the permuted output
     // gradient feeds the data-gradient GEMM, whose result is lifted (neither needs the lowered input)
-    const bool strided_data = direct_weights && strided_ok_ && needs_to_calc_backward_grad;
+    const bool strided_direct_data = direct_weights && strided_data_ok_ && needs_to_calc_backward_grad;
+    const bool strided_data = direct_weights && strided_ok_ && needs_to_calc_backward_grad && !strided_direct_data;
 
     const bool fuse_bias_into_lift = bias_term && needs_to_calc_backward_grad && path_ == PATH_FUSED;
     // on the all-direct path the weight-gradient kernel reduces the bias gradient as well
@@ -308,7 +314,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     }
     LogicalCubeType lowered_outputgrad(direct_weights && !strided_data ? nullptr : staging()->get_p_data(),
                                        num_output_features, oR * oC * iB, 1, 1);
-    if (needs_to_calc_backward_grad && !direct_data) {
+    if (needs_to_calc_backward_grad && !direct_data && !strided_direct_data) {
       begin(STAGE_GEMM_DATA);
       p_backward_gemm_updategrad_kernel->compute(&lowered_model, &lowered_outputgrad, backward_inputgrad());
       end(STAGE_GEMM_DATA);
@@ -347,6 +353,19 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                           out_image_stride_,
                                           input_is_relu_output ? p_input_layer->p_data_cube->get_p_data() : nullptr);
       end(STAGE_GEMM_DATA);
+    } else if (strided_direct_data) {
+      // remap + data-gradient GEMM + lifting of a strided layer in one kernel (phase decomposition)
+      begin(STAGE_GEMM_DATA);
+      p_driver->conv_strided_backward_data_slabs(backward_slabs()->get_p_data(), p_model_cube->get_p_data(),
+                                                 (int)num_output_features, (int)iD, (int)K, (int)stride);
+      p_driver->conv_strided_backward_data(input_g_cube->get_p_data(), output_g_cube->get_p_data(),
+                                           backward_slabs()->get_p_data(), (int)iB, (int)iD, (int)iR, (int)K,
+                                           (int)stride, (int)padding, (int)num_output_features);
+      end(STAGE_GEMM_DATA);
+      if (input_is_relu_output) {  // this kernel's store does not carry the mask
+        DeviceMemoryPointer in_grad = input_g_cube->get_device_pointer(p_driver);
+        p_driver->relu_backward(&in_grad, &in_grad, p_input_layer->p_data_cube->get_p_data());
+      }
     } else if (needs_to_calc_backward_grad) {
       begin(STAGE_INVERSE_LOWER);
       if (fuse_bias_into_lift) {
@@ -404,7 +423,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   size_t in_image_stride_ = 0, out_image_stride_ = 0;
   bool views_ = false;
   bool fuse_relu_ = false;
-  bool direct_ok_ = false, strided_ok_ = false, profile_ = false;
+  bool direct_ok_ = false, strided_ok_ = false, strided_data_ok_ = false, profile_ = false;
   LogicalCubeType *lowered() {
     if (!p_forward_lowered_data) p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
     return p_forward_lowered_data;
@@ -429,7 +448,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   LogicalCubeType *backward_slabs() {
     if (!p_backward_slabs)
       p_backward_slabs = new LogicalCubeType(
-          p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 1), 1, 1, 1, p_driver);
+          strided_data_ok_ ? p_driver->conv_strided_backward_data_slab_floats((int)num_output_features, (int)iD,
+                                                                              (int)K, (int)stride)
+                           : p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 1),
+          1, 1, 1, p_driver);
     return p_backward_slabs;
   }
   void *timers_[STAGE_COUNT];

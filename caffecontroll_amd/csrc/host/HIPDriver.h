@@ -288,6 +288,24 @@ class HIPDriver {
                                              padding, num_outputs),
        "conv_strided_backward_weights");
   }
+  bool conv_strided_backward_data_supported(int batch, int depth, int n, int k, int stride, int padding,
+                                            int num_outputs) {
+    return cct_hip_conv_strided_backward_data_supported(batch, depth, n, k, stride, padding, num_outputs) != 0;
+  }
+  size_t conv_strided_backward_data_slab_floats(int num_outputs, int depth, int k, int stride) {
+    return cct_hip_conv_strided_backward_data_slab_floats(num_outputs, depth, k, stride);
+  }
+  void conv_strided_backward_data_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
+                                        int stride) {
+    ok(cct_hip_conv_strided_backward_data_slabs(slabs, model, num_outputs, depth, k, stride),
+       "conv_strided_backward_data_slabs");
+  }
+  void conv_strided_backward_data(float *input_grad, const float *output_grad, const float *slabs, int batch,
+                                  int depth, int n, int k, int stride, int padding, int num_outputs) {
+    ok(cct_hip_conv_strided_backward_data(input_grad, output_grad, slabs, batch, depth, n, k, stride, padding,
+                                          num_outputs),
+       "conv_strided_backward_data");
+  }
   void sgemv(const CBLAS_TRANSPOSE TA, const int M, const int N, const float alpha, const float *pA,
              const float *px, const float beta, float *py) {
     ok(cct_hip_sgemv(TA, M, N, alpha, pA, px, beta, py), "sgemv");

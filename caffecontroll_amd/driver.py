@@ -150,6 +150,20 @@ class HIPDriver:
         check(self.lib.cct_hip_conv_strided_backward_weights(_p(model_grad), _p(bias_grad), _p(out_grad), _p(inp),
                                                              b, d, n, k, s, p, o), "conv_strided_backward_weights")
 
+    def conv_strided_backward_data_supported(self, b, d, n, k, s, p, o):
+        return bool(self.lib.cct_hip_conv_strided_backward_data_supported(b, d, n, k, s, p, o))
+
+    def conv_strided_backward_data_slab_floats(self, o, d, k, s):
+        return int(self.lib.cct_hip_conv_strided_backward_data_slab_floats(o, d, k, s))
+
+    def conv_strided_backward_data_slabs(self, slabs, model, o, d, k, s):
+        check(self.lib.cct_hip_conv_strided_backward_data_slabs(_p(slabs), _p(model), o, d, k, s),
+              "conv_strided_backward_data_slabs")
+
+    def conv_strided_backward_data(self, in_grad, out_grad, slabs, b, d, n, k, s, p, o):
+        check(self.lib.cct_hip_conv_strided_backward_data(_p(in_grad), _p(out_grad), _p(slabs), b, d, n, k, s, p, o),
+              "conv_strided_backward_data")
+
     def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o, in_stride=0, out_stride=0, relu=False):
         check(self.lib.cct_hip_conv_direct_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o,
                                                    in_stride, out_stride, int(relu)), "conv_direct_forward")

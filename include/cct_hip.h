@@ -261,6 +261,21 @@ int cct_hip_conv_strided_forward(float *output, const float *input, const float 
 int cct_hip_conv_strided_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                           const float *input, int batch, int depth, int n, int k,
                                           int stride, int padding, int num_outputs);
+/* Output-gradient remap + data-gradient GEMM + inverse_lower_cube of ConvolutionBridge::backward
+ * (src/bridges/ConvolutionBridge_impl.hxx:604-616) for a strided layer in one kernel: every
+ * (row phase, column phase) sub-image of the input gradient is a stride-1 convolution of the output
+ * gradient with ceil(k/stride)^2 of the filter's taps.  Covered: depth * stride^2 of at most 80 in an odd
+ * number of 16-row blocks (3 x 16 for AlexNet / CaffeNet conv1), ceil(k/stride) <= 5, output gradient
+ * rows of at most 64 - 2 (ceil(k/stride) - 1) floats.  The slabs (cct_hip_conv_strided_backward_data_slab_floats()
+ * floats, 16-byte aligned) are rebuilt from the model [o][d][k][k] whenever it changes. */
+int cct_hip_conv_strided_backward_data_supported(int batch, int depth, int n, int k, int stride, int padding,
+                                                 int num_outputs);
+size_t cct_hip_conv_strided_backward_data_slab_floats(int num_outputs, int depth, int k, int stride);
+int cct_hip_conv_strided_backward_data_slabs(float *slabs, const float *model, int num_outputs, int depth,
+                                             int k, int stride);
+int cct_hip_conv_strided_backward_data(float *input_grad, const float *output_grad, const float *slabs,
+                                       int batch, int depth, int n, int k, int stride, int padding,
+                                       int num_outputs);
 /* DeviceDriver::sgemv (src/sched/DeviceDriver.h:214-215): row-major M x N, lda = N. */
 int cct_hip_sgemv(int TA, int M, int N, float alpha, const float *A, const float *x, float beta,
                   float *y);

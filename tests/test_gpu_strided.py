@@ -168,6 +168,84 @@ def test_strided_backward_weights_full_config3_vs_float64():
     assert ((db.double() - db_ref).abs().max() / db_ref.abs().max()).item() <= TOL
 
 
+# data gradient: depth * stride^2 maps must come as 1, 3 or 5 blocks of 16 (the 16-row kernel)
+# (and the output gradient must be large enough that a 128-pixel tile does not span dozens of images)
+DGRAD_SHAPES = [s for s in SHAPES if ((s[1] * s[4] * s[4] + 15) // 16) in (1, 3, 5) and (s[2] + 2 * s[5] - s[3]) // s[4] >= 2] + [
+    (3, 3, 61, 11, 4, 0, 20),      # 227-style geometry, smaller: rows left over by the floor division (61 = 4*12 + 13)
+    (2, 3, 40, 11, 4, 3, 9),       # padding 3
+    (2, 1, 29, 5, 2, 0, 7),        # one channel, stride 2
+]
+
+
+@pytest.mark.parametrize("shape", DGRAD_SHAPES, ids=_ids)
+def test_strided_backward_data_vs_oracle(oracle, shape):
+    """Input gradient against the oracle's remap + data-gradient GEMM + inverse_lower_cube
+    (src/bridges/ConvolutionBridge_impl.hxx:604-616)."""
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
+    drv = driver()
+    assert drv.conv_strided_backward_data_supported(*shape)
+    rng = np.random.default_rng(sum(shape) + 2)
+    x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+    w = (rng.standard_normal((o, d, k, k)) * 0.1).astype(np.float32)
+    og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+    _, lowered = oracle.conv_forward(x, w, None, k, s, p)
+    ref_dx, _, _ = oracle.conv_backward(x.shape, w, og, lowered, k, s, p)
+    slabs = empty((drv.conv_strided_backward_data_slab_floats(o, d, k, s),))
+    drv.conv_strided_backward_data_slabs(slabs, dev(w), o, d, k, s)
+    d_og = dev(og)
+    dx = empty((b, d, n, n))
+    drv.conv_strided_backward_data(dx, d_og, slabs, b, d, n, k, s, p, o)
+    assert rel_err(host(dx), ref_dx) <= TOL       # every element written (the buffer starts as NaN)
+    np.testing.assert_array_equal(host(d_og), og)  # the output gradient is read in place, not permuted
+    # small integers: exact in any order
+    wi = rng.integers(-3, 4, size=w.shape).astype(np.float32)
+    ogi = rng.integers(-3, 4, size=og.shape).astype(np.float32)
+    refi_dx, _, _ = oracle.conv_backward(x.shape, wi, ogi, lowered, k, s, p)
+    drv.conv_strided_backward_data_slabs(slabs, dev(wi), o, d, k, s)
+    drv.conv_strided_backward_data(dx, dev(ogi), slabs, b, d, n, k, s, p, o)
+    np.testing.assert_array_equal(host(dx), refi_dx)
+
+
+def test_strided_backward_data_reference_large_fixture():
+    """tests/test_parallelized_convolution_large_CPU.cpp:71-80, backward: input gradient for the output gradient 0.1 * i."""
+    shape = (4, 3, 127, 11, 4, 2, 8)
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
+    w = load_fixture("input", "conv_backward_model_large.txt").reshape(o, d, k, k)
+    og = (0.1 * np.arange(b * o * m * m, dtype=np.float64)).astype(np.float32).reshape(b, o, m, m)
+    drv = driver()
+    slabs = empty((drv.conv_strided_backward_data_slab_floats(o, d, k, s),))
+    drv.conv_strided_backward_data_slabs(slabs, dev(w), o, d, k, s)
+    dx = empty((b, d, n, n))
+    drv.conv_strided_backward_data(dx, dev(og), slabs, b, d, n, k, s, p, o)
+    want = load_fixture("output", "conv_backward_large.txt")
+    np.testing.assert_allclose(host(dx).reshape(-1)[:want.size], want, rtol=1e-4, atol=1e-3)
+
+
+def test_strided_backward_data_full_config3_vs_float64():
+    """benchmark configuration 3 at full size against float64 torch, in chunks of 32 images."""
+    import torch
+    shape = (256, 3, 227, 11, 4, 0, 96)
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
+    g = torch.Generator(device="cuda").manual_seed(1238)
+    w = torch.randn((o, d, k, k), device="cuda", generator=g) * 0.01
+    og = torch.randn((b, o, m, m), device="cuda", generator=g)
+    drv = driver()
+    slabs = empty((drv.conv_strided_backward_data_slab_floats(o, d, k, s),))
+    drv.conv_strided_backward_data_slabs(slabs, w, o, d, k, s)
+    dx = empty((b, d, n, n))
+    drv.conv_strided_backward_data(dx, og, slabs, b, d, n, k, s, p, o)
+    torch.cuda.synchronize()
+    worst = scale = 0.0
+    for i in range(0, b, 32):
+        ref = torch.nn.grad.conv2d_input((min(32, b - i), d, n, n), w.double(), og[i:i + 32].double(), stride=s, padding=p)
+        worst = max(worst, (dx[i:i + 32].double() - ref).abs().max().item())
+        scale = max(scale, ref.abs().max().item())
+    assert worst / scale <= TOL
+
+
 def test_unsupported_geometries_are_refused():
     from caffecontroll_amd import CctHipError
     drv = driver()
