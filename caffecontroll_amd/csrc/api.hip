@@ -32,6 +32,7 @@ static void read_tuning_from_env() {
   g_tuning.pool_plane = geti("CCT_HIP_POOL_PLANE", 0);
   g_tuning.gemm_nt = geti("CCT_HIP_GEMM_NT", 0);
   g_tuning.gemm_tile = geti("CCT_HIP_GEMM_TILE", -1);
+  g_tuning.gemm_nodma = geti("CCT_HIP_GEMM_NODMA", 0);
 }
 
 static char g_last_kernel[192] = "";
@@ -161,7 +162,7 @@ int cct_hip_set_tuning(const char *name, int value) {
   struct { const char *name; int *field; } const table[] = {
       {"direct_tile", &t.direct_tile}, {"direct_waves", &t.direct_waves}, {"direct_tb", &t.direct_tb},
       {"direct_nospec", &t.direct_nospec}, {"pool_plane", &t.pool_plane}, {"gemm_nt", &t.gemm_nt},
-      {"gemm_tile", &t.gemm_tile}};
+      {"gemm_tile", &t.gemm_tile}, {"gemm_nodma", &t.gemm_nodma}};
   for (const auto &e : table)
     if (!strcmp(e.name, name)) {
       *e.field = value;

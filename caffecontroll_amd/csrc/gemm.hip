@@ -21,12 +21,12 @@
 #include <cstdlib>
 
 #include "cct_common.h"
+#include "mfma_common.h"
 
 namespace cct {
 
-typedef float v16f __attribute__((ext_vector_type(16)));
-// native 4-float vector: stays in registers where HIP's f4 struct (a union) can end up in scratch
-typedef float f4 __attribute__((ext_vector_type(4)));
+// (v16f and f4 -- a native 4-float vector, which stays in registers where HIP's float4 struct can end
+// up in scratch -- come from mfma_common.h)
 // the same vector where only dword alignment may be assumed (global memory operands)
 typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
 
@@ -52,6 +52,7 @@ struct GemmArgs {
   int splits;        // K slices; grid = ntiles * splits workgroups
   uint32_t nblocks;
   int nt_store;      // stream the output with non-temporal stores (large outputs that are not re-read)
+  int dma;           // operands go global -> LDS without passing through registers (gemm_mainloop_dma)
 };
 
 __device__ __forceinline__ f4 ldg4(const float *__restrict__ base, int major, int minor,
@@ -314,6 +315,146 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs &g, float *smem, v1
 #undef CCT_FRAGS
 }
 
+// ---- operand tiles straight from global memory into LDS ------------------------------------------
+// Staging a tile through registers (global load, wait, ds_write) costs the wavefronts instruction
+// slots that the matrix pipe does not hide: with the MFMAs taken out, fetching and stashing alone
+// took 0.40 ms of the 1.98 ms forward GEMM of the AlexNet conv2 shape.  Here the tiles are moved by
+// 16-byte buffer loads that write LDS directly (one instruction moves 64 consecutive 16-byte
+// vectors of a stage; each lane supplies the global address of its vector).  LDS rows carry no
+// padding -- the transfer cannot insert any -- so a K-contiguous operand stores vector kq of row
+// `row` in slot kq ^ ((row >> 1) & 3) of its 4-slot row: eight consecutive rows of one fragment
+// read then cover all 32 banks.  Preconditions (checked on the host, else the register path runs):
+// operand bases 16-byte aligned, leading dimensions multiples of 4, a row-contiguous operand's row
+// count a multiple of 4, K a multiple of 16, operands below 2 GiB (32-bit buffer offsets).
+template <class T, bool KC, int ROWS>
+struct DmaLayout {
+  static constexpr int SIZE = ROWS * T::BK;       // floats per stage
+  static constexpr int TOTAL = ROWS * T::BK / 4;  // 16-byte vectors per stage
+  static constexpr int NWAVES = T::THREADS / 64;
+  static constexpr int NV = (TOTAL / 64 + NWAVES - 1) / NWAVES;  // transfers per wavefront per stage
+  // byte offset of the vector that lane `lane` of wavefront `wave` moves in transfer i, for K step 0
+  static __device__ __forceinline__ uint32_t source(int i, int wave, int lane, int row0, int rows_total, int ld) {
+    const int f = (i * NWAVES + wave) * 64 + lane;
+    if (KC) {
+      const int row = f >> 2, slot = f & 3, kq = slot ^ ((row >> 1) & 3);
+      return (uint32_t)(min(row0 + row, rows_total - 1) * (size_t)ld + kq * 4) * 4u;
+    }
+    const int kk = f / (ROWS / 4), rq = f - kk * (ROWS / 4);
+    return (uint32_t)((size_t)kk * ld + min(row0 + rq * 4, rows_total - 4)) * 4u;
+  }
+};
+
+template <class T, bool KC, int ROWS, int NT>
+struct DmaFrags {
+  // per-lane LDS offsets (floats) of the fragments of k-group 0 and 1 for the tile at wave row `wrow0`
+  int base[2];
+  __device__ __forceinline__ void init(int wrow0, int lane) {
+    const int r = lane & 31, h = lane >> 5;
+    if (KC) {
+      const int sw = (r >> 1) & 3;
+      base[0] = (wrow0 + r) * T::BK + ((h ^ sw) << 2);
+      base[1] = (wrow0 + r) * T::BK + (((2 + h) ^ sw) << 2);
+    } else {
+      base[0] = (h * 4) * ROWS + wrow0 + r;
+      base[1] = (8 + h * 4) * ROWS + wrow0 + r;
+    }
+  }
+  template <int KG>
+  __device__ __forceinline__ void load(f4 (&f)[NT], const float *__restrict__ lds) const {
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (KC) {
+        f[t] = *reinterpret_cast<const f4 *>(lds + base[KG] + t * 32 * T::BK);
+      } else {
+        const float *p = lds + base[KG] + t * 32;
+        f[t].x = p[0];
+        f[t].y = p[ROWS];
+        f[t].z = p[2 * ROWS];
+        f[t].w = p[3 * ROWS];
+      }
+    }
+  }
+};
+
+// Main K loop with direct transfers (K a multiple of BK = 16, two k-groups per step, two LDS
+// buffers, one barrier per step in the MIDDLE of the step):
+//   step t, first half : MFMAs of k-group 0 of stage t (both k-groups' fragments were read from LDS
+//                        during step t-1)
+//   wait + barrier     : stage t+1 (requested a whole step ago) has landed, and every wavefront's
+//                        reads of stage t have completed, so its buffer is free
+//   step t, second half: the transfers of stage t+2 are requested into that buffer, the fragments
+//                        of k-group 0 of stage t+1 are requested, MFMAs of k-group 1 of stage t run,
+//                        the fragments of k-group 1 of stage t+1 are requested
+template <class T, bool A_KC, bool B_KC>
+__device__ __forceinline__ void gemm_mainloop_dma(const GemmArgs &g, float *smem, v16f (&acc)[T::TM][T::TN], int m0,
+                                                  int n0, int kbeg, int nk, int lane, int wave, int wm0,
+                                                  int wn0) {
+  using DA = DmaLayout<T, A_KC, T::BM>;
+  using DB = DmaLayout<T, B_KC, T::BN>;
+  constexpr int STAGE = DA::SIZE + DB::SIZE;
+  constexpr int NW = T::THREADS / 64;
+  static_assert(T::BK == 16, "two k-groups per K step");
+  if (nk <= 0) return;
+  uint32_t aoff[DA::NV], boff[DB::NV];
+#pragma unroll
+  for (int i = 0; i < DA::NV; ++i) aoff[i] = DA::source(i, wave, lane, m0, g.M, g.lda);
+#pragma unroll
+  for (int i = 0; i < DB::NV; ++i) boff[i] = DB::source(i, wave, lane, n0, g.N, g.ldb);
+  const rsrc_t a_rsrc = make_rsrc(g.A), b_rsrc = make_rsrc(g.B);
+  const uint32_t a_step = A_KC ? (uint32_t)T::BK * 4u : (uint32_t)T::BK * (uint32_t)g.lda * 4u;
+  const uint32_t b_step = B_KC ? (uint32_t)T::BK * 4u : (uint32_t)T::BK * (uint32_t)g.ldb * 4u;
+  const uint32_t a_k0 = A_KC ? (uint32_t)kbeg * 4u : (uint32_t)kbeg * (uint32_t)g.lda * 4u;
+  const uint32_t b_k0 = B_KC ? (uint32_t)kbeg * 4u : (uint32_t)kbeg * (uint32_t)g.ldb * 4u;
+// transfers of K step t -> LDS buffer buf
+#define CCT_DMA_ISSUE(t, buf)                                                                      \
+  do {                                                                                             \
+    float *sa_ = smem + (buf) * STAGE, *sb_ = sa_ + DA::SIZE;                                      \
+    const uint32_t ga_ = a_k0 + (uint32_t)(t) * a_step, gb_ = b_k0 + (uint32_t)(t) * b_step;       \
+    _Pragma("unroll") for (int i = 0; i < DA::NV; ++i) {                                           \
+      if ((i * NW + wave) * 64 < DA::TOTAL) lds_dma16(a_rsrc, aoff[i], ga_, sa_ + (i * NW + wave) * 256); \
+    }                                                                                              \
+    _Pragma("unroll") for (int i = 0; i < DB::NV; ++i) {                                           \
+      if ((i * NW + wave) * 64 < DB::TOTAL) lds_dma16(b_rsrc, boff[i], gb_, sb_ + (i * NW + wave) * 256); \
+    }                                                                                              \
+  } while (0)
+  DmaFrags<T, A_KC, T::BM, T::TM> qa;
+  DmaFrags<T, B_KC, T::BN, T::TN> qb;
+  qa.init(wm0, lane);
+  qb.init(wn0, lane);
+
+  f4 fa0[T::TM], fb0[T::TN], fa1[T::TM], fb1[T::TN];
+  CCT_DMA_ISSUE(0, 0);
+  if (nk > 1) CCT_DMA_ISSUE(1, 1);
+  lds_dma_wait();
+  __syncthreads();
+  qa.template load<0>(fa0, smem);
+  qb.template load<0>(fb0, smem + DA::SIZE);
+  qa.template load<1>(fa1, smem);
+  qb.template load<1>(fb1, smem + DA::SIZE);
+  for (int t = 0; t < nk; ++t) {
+    const int cur = t & 1;
+    const bool more = (t + 1 < nk);
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_group<T::TM, T::TN>(acc, fa0, fb0);
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): stage t+1 landed; lgkmcnt(0): this wave's reads of stage t are done
+    __syncthreads();
+    if (t + 2 < nk) CCT_DMA_ISSUE(t + 2, cur);
+    const float *nxt = smem + (cur ^ 1) * STAGE;
+    if (more) {
+      qa.template load<0>(fa0, nxt);
+      qb.template load<0>(fb0, nxt + DA::SIZE);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    mfma_group<T::TM, T::TN>(acc, fa1, fb1);
+    if (more) {
+      qa.template load<1>(fa1, nxt);
+      qb.template load<1>(fb1, nxt + DA::SIZE);
+    }
+  }
+#undef CCT_DMA_ISSUE
+}
+
 // Epilogue of a tile whose columns lie wholly inside C and that reads nothing back: per lane one
 // row pointer advancing by a row stride and TN fixed column offsets.  ROWGUARD = false: the rows
 // lie inside C too, no bounds tests at all; true: rows past M are skipped (M not a multiple of the
@@ -365,7 +506,7 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
   }
 }
 
-template <class T, bool A_KC, bool B_KC>
+template <class T, bool A_KC, bool B_KC, bool DMA = false>
 __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
   using LA = OperandLayout<T, A_KC, T::BM>;
   using LB = OperandLayout<T, B_KC, T::BN>;
@@ -400,7 +541,8 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  gemm_mainloop<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
+  if (DMA) gemm_mainloop_dma<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, nk, lane, __builtin_amdgcn_readfirstlane(wave), wm0, wn0);
+  else gemm_mainloop<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
   const bool rows_inside = m0 + T::BM <= g.M, cols_inside = n0 + T::BN <= g.N;
 
   // epilogue: accumulator register v of lane (r,h) is C[8*(v/4) + 4*h + v%4][r] of its 32x32 tile
@@ -498,13 +640,20 @@ static int launch_cfg(GemmArgs &g, bool a_kc, bool b_kc, int splits, hipStream_t
   if (nblocks >= (1ull << 31)) return set_error(CCT_HIP_EINVAL, "sgemm: too many workgroups");
   g.nblocks = (uint32_t)nblocks;
   dim3 grid(g.nblocks), block(T::THREADS);
-  if (a_kc && b_kc) hipLaunchKernelGGL((gemm_kernel<T, true, true>), grid, block, 0, st, g);
-  else if (a_kc && !b_kc) hipLaunchKernelGGL((gemm_kernel<T, true, false>), grid, block, 0, st, g);
-  else if (!a_kc && b_kc) hipLaunchKernelGGL((gemm_kernel<T, false, true>), grid, block, 0, st, g);
-  else hipLaunchKernelGGL((gemm_kernel<T, false, false>), grid, block, 0, st, g);
+  if (g.dma) {
+    if (a_kc && b_kc) hipLaunchKernelGGL((gemm_kernel<T, true, true, true>), grid, block, 0, st, g);
+    else if (a_kc && !b_kc) hipLaunchKernelGGL((gemm_kernel<T, true, false, true>), grid, block, 0, st, g);
+    else if (!a_kc && b_kc) hipLaunchKernelGGL((gemm_kernel<T, false, true, true>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_kernel<T, false, false, true>), grid, block, 0, st, g);
+  } else {
+    if (a_kc && b_kc) hipLaunchKernelGGL((gemm_kernel<T, true, true>), grid, block, 0, st, g);
+    else if (a_kc && !b_kc) hipLaunchKernelGGL((gemm_kernel<T, true, false>), grid, block, 0, st, g);
+    else if (!a_kc && b_kc) hipLaunchKernelGGL((gemm_kernel<T, false, true>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((gemm_kernel<T, false, false>), grid, block, 0, st, g);
+  }
   CCT_LAUNCH_CHECK();
-  note_kernel("gemm_kernel<Tile<%d,%d,%d,%d,%d>,%s,%s> splits=%d", T::BM, T::BN, T::BK, T::WGM, T::WGN,
-              a_kc ? "true" : "false", b_kc ? "true" : "false", splits);
+  note_kernel("gemm_kernel<Tile<%d,%d,%d,%d,%d>,%s,%s%s> splits=%d", T::BM, T::BN, T::BK, T::WGM, T::WGN,
+              a_kc ? "true" : "false", b_kc ? "true" : "false", g.dma ? ",true" : "", splits);
   return 0;
 }
 
@@ -572,6 +721,13 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
     }
   }
   g.kchunk = kchunk;
+  {
+    // direct global -> LDS transfers need aligned, 4-float-granular operands below 2 GiB and whole K steps
+    const size_t a_floats = a_kc ? (size_t)M * lda : (size_t)g.K * lda, b_floats = b_kc ? (size_t)N * ldb : (size_t)g.K * ldb;
+    g.dma = g.K > 0 && g.K % bk == 0 && kchunk % bk == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)B % 16 == 0 &&
+            lda % 4 == 0 && ldb % 4 == 0 && (a_kc || M % 4 == 0) && (b_kc || N % 4 == 0) &&
+            a_floats < (1ull << 29) && b_floats < (1ull << 29) && !tuning().gemm_nodma;
+  }
   if (splits > 1) {
     void *ws = nullptr;
     int rc = get_workspace((size_t)splits * M * N * sizeof(float), &ws);

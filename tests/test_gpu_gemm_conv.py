@@ -67,6 +67,43 @@ def test_sgemm_all_layouts(oracle, case, TA, TB, order):
             assert rel_err(got, ref) <= TOL
 
 
+# shapes that meet the preconditions of the direct global -> LDS operand transfers (16-byte aligned bases,
+# leading dimensions and row-contiguous row counts multiples of 4, K a multiple of 16): every tile shape,
+# ragged tile edges, one split-K case
+DMA_CASES = [(64, 64, 16), (128, 128, 64), (256, 384, 96), (300, 200, 80), (500, 64, 800), (96, 4000, 368),
+             (192, 3004, 48), (256, 1000, 4096), (20, 576, 32), (260, 132, 1024)]
+
+
+@pytest.mark.parametrize("case", DMA_CASES, ids=lambda c: "M%d_N%d_K%d" % c)
+@pytest.mark.parametrize("TA", [N_, T_])
+@pytest.mark.parametrize("TB", [N_, T_])
+def test_sgemm_direct_transfer_path_matches_register_path(TA, TB, case):
+    """Operand tiles moved global -> LDS directly (the default where the operands allow it) against the same
+    kernel staging them through registers (tuning knob gemm_nodma): the k order of every accumulator is the same,
+    so the results must be identical bit for bit; and both within tolerance of float64."""
+    from gpu_util import tuning
+    M, N, K = case
+    rng = np.random.default_rng(M + 3 * N + 5 * K + TA + 2 * TB)
+    opA = rng.standard_normal((M, K)).astype(np.float32)
+    opB = rng.standard_normal((K, N)).astype(np.float32)
+    A = np.ascontiguousarray(opA.T if TA == T_ else opA)
+    B = np.ascontiguousarray(opB.T if TB == T_ else opB)
+    drv = driver()
+    dA, dB = dev(A), dev(B)
+    c_dma, c_reg = empty((M, N)), empty((M, N))
+    drv.sgemm_new(TA, TB, M, N, K, 1.0, dA, dB, 0.0, c_dma)
+    def flags():  # template arguments after the tile: <A k-contiguous>,<B k-contiguous>[,true for direct transfers]
+        name = drv.lib.cct_hip_last_kernel().decode()
+        return name[name.index(">,") + 2:name.rindex(">")].split(",")
+
+    assert len(flags()) == 3 and flags()[2] == "true"
+    with tuning("gemm_nodma", 1):
+        drv.sgemm_new(TA, TB, M, N, K, 1.0, dA, dB, 0.0, c_reg)
+        assert len(flags()) == 2
+    np.testing.assert_array_equal(host(c_dma), host(c_reg))
+    assert rel_err(host(c_dma), opA.astype(np.float64) @ opB.astype(np.float64)) <= TOL
+
+
 def test_sgemm_split_k_is_deterministic_and_correct(oracle):
     """Tiny output, long K: the weight-gradient shape class (goes through the split-K path)."""
     M, N, K = 40, 75, 40000
