@@ -36,13 +36,13 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_SOURCE = {"direct": "profiles/conv2_fwd_bwd_hbm_traffic_and_mfma.md",
                   "lowering": "profiles/conv2_lowering_path_hbm_traffic_and_mfma.md"}
 TRAFFIC_BYTES = {
-    ("GEMM", "conv_direct_kernel<5,1,2,1,32>"): ((230.1 + 223.7) * 1e6, "direct"),
-    ("GEMM Data", "conv_direct_kernel<5,1,2,1,32>"): ((322.3 + 75.7) * 1e6, "direct"),
+    ("GEMM", "conv_direct_kernel<5,1,2,1,32>"): ((238.5 + 230.6) * 1e6, "direct"),
+    ("GEMM Data", "conv_direct_kernel<5,1,2,1,32>"): ((320.6 + 76.2) * 1e6, "direct"),
     ("GEMM Wghts", "conv_direct_wgrad_spec_kernel<5,5,32,27,8>"): ((359.6 + 41.8) * 1e6, "direct"),
-    ("GEMM", "gemm_kernel<Tile<256,128,16,2,2>,true,true> splits=1"): ((1867.6 + 192.7) * 1e6, "lowering"),
-    ("GEMM Data", "gemm_kernel<Tile<128,128,16,2,2>,false,false> splits=1"): ((1209.0 + 1791.6) * 1e6, "lowering"),
-    ("GEMM Wghts", "gemm_kernel<Tile<256,128,16,2,2>,true,false> splits=26"): ((2203.8 + 63.9) * 1e6, "lowering"),
-    ("Lower Cube", "lower_kernel threads=320"): ((80.4 + 1791.6) * 1e6, "lowering"),
+    ("GEMM", "gemm_kernel<Tile<256,128,16,2,2>,true,true,true> splits=1"): ((1985.7 + 201.4) * 1e6, "lowering"),
+    ("GEMM Data", "gemm_kernel<Tile<128,128,16,2,2>,false,false,true> splits=1"): ((1172.9 + 1791.6) * 1e6, "lowering"),
+    ("GEMM Wghts", "gemm_kernel<Tile<256,128,16,2,2>,true,false,true> splits=26"): ((2384.4 + 63.9) * 1e6, "lowering"),
+    ("Lower Cube", "lower_kernel threads=512"): ((75.6 + 1791.6) * 1e6, "lowering"),
     ("Inverse Lwr", "lift_kernel<5,1> bias_blocks=256"): ((2190.6 + 71.7) * 1e6, "lowering"),
 }
 
