@@ -545,7 +545,6 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
       return true;
     }
   }
-  if (pw > 32) return false;  // the 32-row kernel has no instance for rows that wide
   // Candidate tiles: map tiles that divide the padded map count (the slab layout does not depend
   // on the choice), 128 or 256 pixels.  Estimated time, in units of one 32x128 block on a whole
   // compute unit: workgroups are handed out as residency slots free up, so the launch runs as
@@ -687,8 +686,11 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
     return pl.pw == 16 ? direct_launch16<3, 16>(g, pl, st)
                        : pl.pw == 32 ? direct_launch16<3, 32>(g, pl, st) : direct_launch16<3, 64>(g, pl, st);
   }
-  if (ks == 5) return pl.pw == 16 ? direct_launch_ks<5, 1, 16>(g, pl, st) : direct_launch_ks<5, 1, 32>(g, pl, st);
-  return pl.pw == 16 ? direct_launch_ks<3, 2, 16>(g, pl, st) : direct_launch_ks<3, 2, 32>(g, pl, st);
+  if (ks == 5)
+    return pl.pw == 16 ? direct_launch_ks<5, 1, 16>(g, pl, st)
+                       : pl.pw == 32 ? direct_launch_ks<5, 1, 32>(g, pl, st) : direct_launch_ks<5, 1, 64>(g, pl, st);
+  return pl.pw == 16 ? direct_launch_ks<3, 2, 16>(g, pl, st)
+                     : pl.pw == 32 ? direct_launch_ks<3, 2, 32>(g, pl, st) : direct_launch_ks<3, 2, 64>(g, pl, st);
 }
 
 
@@ -1275,8 +1277,12 @@ static int wgrad_launch(const WgradArgs &g, const WgradPlan &pl, hipStream_t st)
 static int conv_direct_wgrad(float *dw, float *db, const float *dout, const float *src, int batch, int d, int n,
                              int ks, int pad, int o, size_t src_img_stride, size_t dout_img_stride) {
   WgradPlan pl;
-  CCT_REQUIRE(wgrad_plan(batch, d, n, ks, pad, o, &pl),
-              "conv_direct wgrad: geometry not covered (k=%d pad=%d size=%d)", ks, pad, n);
+  if (!wgrad_plan(batch, d, n, ks, pad, o, &pl)) {
+    // rows too long for the image-pair kernels: the one-image-per-step kernel, if its patch holds them
+    CCT_REQUIRE(conv_strided_wgrad_covers(batch, d, n, ks, 1, pad, o),
+                "conv_direct wgrad: geometry not covered (k=%d pad=%d size=%d)", ks, pad, n);
+    return conv_strided_wgrad(dw, db, dout, src, batch, d, n, ks, 1, pad, o, src_img_stride, dout_img_stride);
+  }
   WgradArgs g;
   g.dout = dout; g.src = src;
   g.batch = batch; g.o = o; g.d = d; g.hs = n; g.pad = pad;
@@ -1403,7 +1409,8 @@ extern "C" int cct_hip_conv_direct_supported(int batch, int depth, int n, int k,
   WgradPlan wp;
   return direct_plan(batch, depth, num_outputs, n, k, padding, &pl) &&
                  direct_plan(batch, num_outputs, depth, m, k, k - 1 - padding, &pl) &&
-                 wgrad_plan(batch, depth, n, k, padding, num_outputs, &wp)
+                 (wgrad_plan(batch, depth, n, k, padding, num_outputs, &wp) ||
+                  conv_strided_wgrad_covers(batch, depth, n, k, 1, padding, num_outputs))
              ? 1
              : 0;
 }

@@ -36,4 +36,10 @@ __device__ __forceinline__ void lds_dma_wait() { __builtin_amdgcn_s_waitcnt(0x0F
 int reduce_partial_sums(float *dst, const float *ws, uint32_t n, float *dst2, const float *ws2, uint32_t n2,
                         int splits, hipStream_t st);
 
+// Weight (and bias) gradient kernel that stages one output row of ONE image per step (defined beside the strided
+// kernels): strided layers, and stride-1 layers whose rows are too long for the image-pair kernels.
+bool conv_strided_wgrad_covers(int batch, int d, int n, int ks, int stride, int pad, int o);
+int conv_strided_wgrad(float *dw, float *db, const float *dout, const float *src, int batch, int d, int n, int ks,
+                       int stride, int pad, int o, size_t src_img_stride, size_t dout_img_stride);
+
 }  // namespace cct

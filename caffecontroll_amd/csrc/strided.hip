@@ -635,11 +635,12 @@ struct StridedWgradArgs {
   int pws, pch;        // floats between patch rows / patch channels
   int nq2;             // groups of four pixels per output row: ceil(ho / 4)
   int steps_total, steps_per_split;  // a step = (image, output row)
+  uint32_t dout_img_stride, src_img_stride;  // floats between images (channel-slice views of wider tensors)
   uint32_t tiles_m, tiles_n, ntiles, nblocks;
   FastDiv div_ho, div_ast, div_pch, div_pws, div_wm;
 };
 
-constexpr int kSWgradSlabLoads = 12;   // per lane per step, at most
+constexpr int kSWgradSlabLoads = 16;   // per lane per step, at most
 constexpr int kSWgradPatchLoads = 20;
 
 template <int KS, int S, int TB>
@@ -695,12 +696,12 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
     const uint32_t img_ = fdiv((uint32_t)(s), g.div_ho);                                          \
     const int y_ = (s) - (int)img_ * g.ho;                                                        \
     float *sa_ = smem + (st) * stage + wave * 64;                                                 \
-    const uint32_t ga_ = (uint32_t)(((size_t)img_ * g.o * ho2 + (size_t)m0 * ho2 + y_ * g.ho) * 4); \
+    const uint32_t ga_ = (uint32_t)(((size_t)img_ * g.dout_img_stride + (size_t)m0 * ho2 + y_ * g.ho) * 4); \
     _Pragma("unroll") for (int k = 0; k < NAL; ++k) {                                             \
       if (k < g.nal) lds_dma4(a_rsrc, aoff[k], ga_, sa_ + k * nthreads);                          \
     }                                                                                             \
     float *sb_ = sa_ + g.a_floats;                                                                \
-    const uint32_t gb_ = (uint32_t)(((size_t)img_ * g.d * hs2 + (size_t)ch0 * hs2) * 4);          \
+    const uint32_t gb_ = (uint32_t)(((size_t)img_ * g.src_img_stride + (size_t)ch0 * hs2) * 4);   \
     /* the first patch row may lie above the image: that (negative) term goes into the lane     */ \
     /* offset, whose sum is non-negative for every lane that passes the row test                */ \
     const int top_ = S * y_ - g.pad;                                                              \
@@ -879,8 +880,8 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_spec_kernel(const Stri
 #define CCT_SWSPEC_STEP(s)                                                                        \
   const uint32_t img_ = fdiv((uint32_t)(s), g.div_ho);                                            \
   const int y_ = (s) - (int)img_ * g.ho;                                                          \
-  const uint32_t ga_ = (uint32_t)(((size_t)img_ * g.o * ho2 + (size_t)m0 * ho2 + y_ * g.ho) * 4); \
-  const uint32_t gb_ = (uint32_t)(((size_t)img_ * g.d * hs2 + (size_t)ch0 * hs2 + (size_t)S * y_ * g.hs) * 4)
+  const uint32_t ga_ = (uint32_t)(((size_t)img_ * g.dout_img_stride + (size_t)m0 * ho2 + y_ * g.ho) * 4); \
+  const uint32_t gb_ = (uint32_t)(((size_t)img_ * g.src_img_stride + (size_t)ch0 * hs2 + (size_t)S * y_ * g.hs) * 4)
 #define CCT_SWSPEC_SLOT(k, st)                                                                    \
   do {                                                                                            \
     if ((k) < NAL)                                                                                \
@@ -975,10 +976,15 @@ struct StridedWgradPlan {
 static bool strided_kernel_size(int ks, int stride) {
   return (ks == 11 && stride == 4) || (ks == 7 && stride == 2) || (ks == 5 && stride == 2) || (ks == 3 && stride == 2);
 }
+// the weight-gradient kernel also has stride-1 instances (3 x 3 and 5 x 5): the stride-1 kernels of their own
+// file stage image PAIRS and stop at padded rows of 32 floats, this one takes rows as long as its patch holds
+static bool strided_wgrad_kernel_size(int ks, int stride) {
+  return strided_kernel_size(ks, stride) || (stride == 1 && (ks == 3 || ks == 5));
+}
 
 // Chooses the workgroup shape for a geometry; false when the strided weight-gradient kernel does not cover it.
 static bool strided_wgrad_plan(int batch, int d, int n, int ks, int stride, int pad, int o, StridedWgradPlan *pl) {
-  if (!strided_kernel_size(ks, stride)) return false;
+  if (!strided_wgrad_kernel_size(ks, stride)) return false;
   if (batch <= 0 || d <= 0 || o <= 0 || pad < 0 || pad >= ks || n + 2 * pad < ks) return false;
   const int hp = n + 2 * pad, ho = (hp - ks) / stride + 1, kk = ks * ks;
   if ((double)batch * d * n * n >= 536870912.0 || (double)batch * o * ho * ho >= 536870912.0 ||
@@ -1045,8 +1051,13 @@ static int strided_wgrad_launch(const StridedWgradArgs &g, const StridedWgradPla
   return set_error(CCT_HIP_EINVAL, "conv_strided wgrad: no kernel instance for %d column blocks", pl.tb);
 }
 
-static int conv_strided_wgrad(float *dw, float *db, const float *dout, const float *src, int batch, int d, int n,
-                              int ks, int stride, int pad, int o) {
+bool conv_strided_wgrad_covers(int batch, int d, int n, int ks, int stride, int pad, int o) {
+  StridedWgradPlan pl;
+  return strided_wgrad_plan(batch, d, n, ks, stride, pad, o, &pl);
+}
+
+int conv_strided_wgrad(float *dw, float *db, const float *dout, const float *src, int batch, int d, int n, int ks,
+                       int stride, int pad, int o, size_t src_img_stride, size_t dout_img_stride) {
   StridedWgradPlan pl;
   CCT_REQUIRE(strided_wgrad_plan(batch, d, n, ks, stride, pad, o, &pl),
               "conv_strided wgrad: geometry not covered (k=%d stride=%d pad=%d size=%d)", ks, stride, pad, n);
@@ -1058,6 +1069,17 @@ static int conv_strided_wgrad(float *dw, float *db, const float *dout, const flo
   g.wm = pl.wm; g.wn = pl.wn; g.nch = pl.nch; g.ast = pl.ast; g.a_floats = pl.a_floats; g.b_floats = pl.b_floats;
   g.nal = pl.nal; g.nbl = pl.nbl; g.pws = pl.pws; g.pch = pl.pch; g.nq2 = pl.nq2;
   g.steps_total = batch * g.ho;
+  {
+    const size_t dense_src = (size_t)d * n * n, dense_dout = (size_t)o * g.ho * g.ho;
+    if (!src_img_stride) src_img_stride = dense_src;
+    if (!dout_img_stride) dout_img_stride = dense_dout;
+    CCT_REQUIRE(src_img_stride >= dense_src && dout_img_stride >= dense_dout,
+                "conv_strided wgrad: image stride smaller than an image");
+    CCT_REQUIRE((double)batch * src_img_stride < 536870912.0 && (double)batch * dout_img_stride < 536870912.0,
+                "conv_strided wgrad: strided tensor too large for 32-bit byte offsets");
+    g.src_img_stride = (uint32_t)src_img_stride;
+    g.dout_img_stride = (uint32_t)dout_img_stride;
+  }
   g.tiles_m = (uint32_t)((o + 32 * pl.wm - 1) / (32 * pl.wm));
   g.tiles_n = (uint32_t)((g.ncols + 32 * pl.tb * pl.wn - 1) / (32 * pl.tb * pl.wn));
   g.ntiles = g.tiles_m * g.tiles_n;
@@ -1100,8 +1122,8 @@ static int conv_strided_wgrad(float *dw, float *db, const float *dout, const flo
     rc = 0;
   } else if (ks == 11) rc = strided_wgrad_launch<11, 4>(g, pl, st);
   else if (ks == 7) rc = strided_wgrad_launch<7, 2>(g, pl, st);
-  else if (ks == 5) rc = strided_wgrad_launch<5, 2>(g, pl, st);
-  else rc = strided_wgrad_launch<3, 2>(g, pl, st);
+  else if (ks == 5) rc = stride == 2 ? strided_wgrad_launch<5, 2>(g, pl, st) : strided_wgrad_launch<5, 1>(g, pl, st);
+  else rc = stride == 2 ? strided_wgrad_launch<3, 2>(g, pl, st) : strided_wgrad_launch<3, 1>(g, pl, st);
   if (rc) return rc;
   if (splits > 1)
     return reduce_partial_sums(dw, g.out, (uint32_t)n_out, db, g.out_bias, db ? (uint32_t)o : 0u, splits, st);
@@ -1189,6 +1211,7 @@ extern "C" int cct_hip_conv_strided_backward_weights(float *model_grad, float *b
                                                      int stride, int padding, int num_outputs) {
   CCT_ENSURE_INIT();
   CCT_REQUIRE(model_grad && output_grad && input, "conv_strided_backward_weights: null argument");
+  CCT_REQUIRE(stride > 1, "conv_strided_backward_weights: stride-1 layers go through cct_hip_conv_direct_backward_weights");
   return conv_strided_wgrad(model_grad, bias_grad, output_grad, input, batch, depth, n, k, stride, padding,
-                            num_outputs);
+                            num_outputs, 0, 0);
 }

@@ -23,10 +23,14 @@ SHAPES = [
     (3, 5, 9, 5, 4, 6),       # full padding (p = k-1)
     (2, 6, 10, 3, 0, 40),     # no padding
     (1, 7, 5, 5, 2, 3),       # image as small as the filter
-    (5, 9, 30, 3, 1, 33),     # padded width 32: the widest the kernels take
+    (5, 9, 30, 3, 1, 33),     # padded width 32: the widest the image-pair weight-gradient kernels take
     (4, 5, 7, 3, 1, 4),       # 7x7 images: a 128-pixel tile spans four of them
     (3, 80, 13, 3, 1, 48),    # 48 maps forward, 80 maps in the data gradient: three and five 16-row blocks
     (2, 16, 27, 5, 2, 80),    # five 16-row blocks forward, one in the data gradient
+    (2, 8, 56, 3, 1, 16),     # padded rows of 33..64 floats: 64-float patch rows, one image per weight-gradient step
+    (2, 6, 40, 5, 2, 40),
+    (3, 20, 62, 3, 1, 33),    # padded width 64: the widest
+    (2, 3, 60, 5, 2, 8),
 ]
 
 
@@ -165,7 +169,7 @@ def test_direct_every_tile_instance(oracle, shape, tile):
         assert ran == 2  # single-block map tiles fit every map count
 
 
-@pytest.mark.parametrize("shape", [(4, 6, 13, 3, 1, 10), (3, 8, 27, 5, 2, 36)], ids=_ids)
+@pytest.mark.parametrize("shape", [(4, 6, 13, 3, 1, 10), (3, 8, 27, 5, 2, 36), (2, 5, 44, 3, 1, 12)], ids=_ids)
 def test_direct_kernels_on_channel_slices(oracle, shape):
     """Grouped convolution in place: each group reads its channel slice of the whole input and
     writes its slice of the whole output (image strides of the whole tensors); results equal the
@@ -279,11 +283,12 @@ def test_direct_support_matrix_and_errors():
     assert drv.conv_direct_supported(256, 256, 13, 3, 1, 1, 384)
     assert not drv.conv_direct_supported(256, 3, 227, 11, 4, 0, 96)   # k = 11, stride 4
     assert not drv.conv_direct_supported(4, 3, 20, 5, 4, 2, 10)       # stride 4
-    assert not drv.conv_direct_supported(4, 3, 40, 5, 1, 2, 10)       # padded image wider than 32
+    assert drv.conv_direct_supported(4, 3, 40, 5, 1, 2, 10)           # padded image 44 wide
+    assert not drv.conv_direct_supported(4, 3, 62, 5, 1, 2, 10)       # padded image wider than 64
     assert not drv.conv_direct_supported(4, 3, 20, 5, 1, 5, 10)       # padding above k-1
     assert not drv.conv_direct_supported(1, 2, 3, 3, 1, 0, 2)         # 1x1 output: a tile would span 128 images
     with pytest.raises(CctHipError):
-        drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 40, 5, 2, 10)
+        drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 62, 5, 2, 10)
     with pytest.raises(CctHipError):
         drv.conv_direct_backward_weights(empty((1,)), empty((1,)), empty((1,)), 4, 3, 20, 7, 3, 10)
     w = empty((drv.conv_direct_slab_floats(10, 3, 5, 0),), fill=1.0)
