@@ -433,6 +433,10 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_plane_kernel(float *__restric
 // contains it, so no range logic is needed beyond masking the clamped duplicates at the borders.
 // Additions stay in (ph, pw) order.  One 16-byte store per lane instead of four 4-byte ones, and
 // a quarter of the LDS reads and index arithmetic of the element-wise kernel.
+// K3S2 = true: 3 x 3 windows with stride 2 (the CaffeNet pooling layers).  Columns w0..w0+3 (w0 a multiple of 4)
+// can only lie in window columns c-1, c, c+1 with c = w0/2 -- w0 in c-1 and c, w0+1 in c, w0+2 in c and c+1,
+// w0+3 in c+1 -- so six (argmax, gradient) pairs are read and twelve tests made instead of eight and thirty-two.
+template <bool K3S2>
 __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict__ ig, const float *__restrict__ og,
                                                                const int *__restrict__ idx, cct_pool_args a,
                                                                uint32_t planes, int pp, int lpr_shift, FastDiv div_ir,
@@ -461,13 +465,14 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict
   if (w0 >= a.iC) return;
   const int nw = min(4, a.iC - w0);  // elements of this lane's quad inside the row
   // window columns pc0 .. pc0+3 (clamped; cv[j] false for the duplicates the clamp makes)
-  const int pc0 = w0 < k ? 0 : (int)fdiv((uint32_t)(w0 - k), div_s) + 1;
-  int pc[4];
-  bool cv[4];
+  const int pc0 = K3S2 ? (w0 >> 1) - 1 : w0 < k ? 0 : (int)fdiv((uint32_t)(w0 - k), div_s) + 1;
+  constexpr int NJ = K3S2 ? 3 : 4;
+  int pc[NJ];
+  bool cv[NJ];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    pc[j] = min(pc0 + j, a.oC - 1);
-    cv[j] = pc0 + j <= a.oC - 1;
+  for (int j = 0; j < NJ; ++j) {
+    pc[j] = min(max(pc0 + j, 0), a.oC - 1);
+    cv[j] = pc0 + j >= 0 && pc0 + j <= a.oC - 1;
   }
   float *dst = ig + (size_t)p0 * iplane + w0;
   const uint32_t nrows = np * (uint32_t)a.iR;
@@ -479,10 +484,10 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict
     const float *g = tog + pl * oplane;
     const int *x = tidx + pl * oplane;
     const int r0 = ph_lo * a.oC, r1 = min(ph_lo + 1, a.oR - 1) * a.oC;
-    int xi[2][4];
-    float gv[2][4];
+    int xi[2][NJ];
+    float gv[2][NJ];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NJ; ++j) {
       xi[0][j] = x[r0 + pc[j]]; gv[0][j] = g[r0 + pc[j]];
       xi[1][j] = x[r1 + pc[j]]; gv[1][j] = g[r1 + pc[j]];
     }
@@ -490,11 +495,14 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < NJ; ++j) {
         const bool ok = cv[j] && (i == 0 || row1);
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
+        for (int e = 0; e < 4; ++e) {
+          // K3S2: an even element e sits in window columns e/2 and e/2 + 1 of the three, an odd one in (e+1)/2 only
+          if (K3S2 && !((e & 1) ? j == (e + 1) / 2 : (j == e / 2 || j == e / 2 + 1))) continue;
           if (ok && xi[i][j] == me0 + e) acc[e] += gv[i][j];
+        }
       }
     float *o = dst + (size_t)row * a.iC;
     if (relu_data) {
@@ -1095,9 +1103,14 @@ static int maxpool_backward_impl(float *in_grad, const float *out_grad, const cc
     if (quad) {
       int lpr_shift = 0;
       while ((4 << lpr_shift) < a->iC) ++lpr_shift;
-      hipLaunchKernelGGL(maxpool_bwd_quad_kernel, grid, dim3(TPB), (size_t)2 * pp * oplane * sizeof(float),
-                         ctx().stream, in_grad, out_grad, a->max_index, *a, (uint32_t)planes, pp, lpr_shift,
-                         make_fastdiv(a->iR), make_fastdiv(a->stride), relu_data, pooled);
+      if (a->kernel_size == 3 && a->stride == 2)
+        hipLaunchKernelGGL(maxpool_bwd_quad_kernel<true>, grid, dim3(TPB), (size_t)2 * pp * oplane * sizeof(float),
+                           ctx().stream, in_grad, out_grad, a->max_index, *a, (uint32_t)planes, pp, lpr_shift,
+                           make_fastdiv(a->iR), make_fastdiv(a->stride), relu_data, pooled);
+      else
+        hipLaunchKernelGGL(maxpool_bwd_quad_kernel<false>, grid, dim3(TPB), (size_t)2 * pp * oplane * sizeof(float),
+                           ctx().stream, in_grad, out_grad, a->max_index, *a, (uint32_t)planes, pp, lpr_shift,
+                           make_fastdiv(a->iR), make_fastdiv(a->stride), relu_data, pooled);
       relu_data = nullptr;  // done inside the kernel
     } else if (a->kernel_size <= 2 * a->stride)
       hipLaunchKernelGGL(maxpool_bwd_plane_kernel<true>, grid, dim3(TPB), 0, ctx().stream, in_grad, out_grad,
