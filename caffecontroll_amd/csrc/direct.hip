@@ -533,7 +533,8 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   const int forced = tuning().direct_tile;
   pl->tm16 = 0;
   if (const int tm16 = direct_tm16(mtot); tm16 && (forced == 0 || forced == 161 || forced == 162)) {
-    for (int tnb = forced == 161 ? 1 : 2; tnb >= (forced == 162 ? 2 : 1); --tnb) {
+    // 128-pixel tiles first (one group of conv2's data gradient: 504 us against 581 with 256 pixels)
+    for (int tnb = forced == 162 ? 2 : 1; tnb <= (forced == 161 ? 1 : 2); ++tnb) {
       const int bn = 128 * tnb;
       const int rows = (ho - 1 + bn - 1) / ho + 1, imgs = (ho * ho - 1 + bn - 1) / (ho * ho) + 1;
       const int pr = rows - 1 + (imgs - 1) * (ks - 1) + ks;
