@@ -1168,10 +1168,51 @@ __global__ __launch_bounds__(256) void direct_reduce_kernel(float *__restrict__ 
   dst[e] = s;
 }
 
+// The same sums for small results with many partial sums (LeNet-sized layers: 500 gradients, hundreds of
+// step ranges), where one lane per element walks the ranges one after another and the launch is all
+// latency: a workgroup takes 16 elements, its 16 lane groups each add up every 16th range (z = g, g + 16, ...,
+// ascending), and lane group 0 adds the 16 group sums in ascending order.  A fixed order as well (run-to-run
+// identical results), but another one than direct_reduce_kernel's, so a layer always takes the same kernel.
+__global__ __launch_bounds__(256) void direct_reduce_small_kernel(float *__restrict__ dst, const float *__restrict__ ws,
+                                                                  uint32_t n, float *__restrict__ dst2,
+                                                                  const float *__restrict__ ws2, uint32_t n2,
+                                                                  int splits) {
+  __shared__ float part[16][17];
+  const int el = threadIdx.x & 15, grp = threadIdx.x >> 4;
+  uint32_t e = blockIdx.x * 16 + el;
+  const bool live = e < n + n2;
+  float s = 0.f;
+  if (live) {
+    const float *p;
+    uint32_t stride;
+    if (e >= n) { p = ws2 + (e - n); stride = n2; } else { p = ws + e; stride = n; }
+    p += (size_t)grp * stride;
+    int z = grp;
+    for (; z + 48 < splits; z += 64, p += (size_t)64 * stride) {
+      const float v0 = p[0], v1 = p[(size_t)16 * stride], v2 = p[(size_t)32 * stride], v3 = p[(size_t)48 * stride];
+      s += v0; s += v1; s += v2; s += v3;
+    }
+    for (; z < splits; z += 16, p += (size_t)16 * stride) s += *p;
+  }
+  part[grp][el] = s;
+  __syncthreads();
+  if (grp == 0 && live) {
+    float t = 0.f;
+#pragma unroll
+    for (int g2 = 0; g2 < 16; ++g2) t += part[g2][el];
+    if (e >= n) dst2[e - n] = t;
+    else dst[e] = t;
+  }
+}
+
 int reduce_partial_sums(float *dst, const float *ws, uint32_t n, float *dst2, const float *ws2, uint32_t n2,
                         int splits, hipStream_t st) {
-  hipLaunchKernelGGL(direct_reduce_kernel, dim3((n + n2 + 255) / 256), dim3(256), 0, st, dst, ws, n, dst2, ws2, n2,
-                     splits);
+  if (n + n2 <= 8192 && splits >= 64)
+    hipLaunchKernelGGL(direct_reduce_small_kernel, dim3((n + n2 + 15) / 16), dim3(256), 0, st, dst, ws, n, dst2, ws2,
+                       n2, splits);
+  else
+    hipLaunchKernelGGL(direct_reduce_kernel, dim3((n + n2 + 255) / 256), dim3(256), 0, st, dst, ws, n, dst2, ws2, n2,
+                       splits);
   CCT_LAUNCH_CHECK();
   return 0;
 }
