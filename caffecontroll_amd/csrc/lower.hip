@@ -25,13 +25,15 @@ struct LowerParams {
   int nbands, nslabs;
   uint32_t nblocks;
   int chunk_full;  // staged floats per channel for an interior band: ((RB-1)*s + k) * n
-  FastDiv div_kk, div_k, div_seg, div_n, div_chunk;
+  int flat;    // 1: whole rows (one slab) of a length that is not a multiple of 4: flat aligned stores
+  FastDiv div_kk, div_k, div_seg, div_n, div_chunk, div_m;
 };
 
 constexpr int LOWER_MAX_THREADS = 512;  // block size is chosen per launch (multiple of 64)
 
 // dynamic LDS: [DS*TH*TW floats tile][seglen uint16 offsets]
 typedef float lower_f4u __attribute__((ext_vector_type(4), aligned(4)));
+typedef float lower_f4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(LOWER_MAX_THREADS) void lower_kernel(float *__restrict__ dst,
                                                               const float *__restrict__ src,
@@ -109,11 +111,57 @@ __global__ __launch_bounds__(LOWER_MAX_THREADS) void lower_kernel(float *__restr
   }
   __syncthreads();
 
-  // (3) stream the lowered rows.  A lane owns a unit -- 4 consecutive positions of a lowered row
-  // (one 16-byte store; dword alignment is all such a store needs, so row lengths like 363 cost
-  // nothing) or one of the seg % 4 positions left over -- and a group of output columns, and walks
-  // over the band.  Short rows (few units) are spread over several column groups so that the
-  // whole workgroup stores.
+  // (3) stream the lowered rows.
+  if (P.flat) {
+    // Whole rows whose length is not a multiple of four floats: the band's output -- rb*m lowered
+    // rows -- is one contiguous range of HBM, written as a flat stream of 16-byte stores on 16-byte
+    // boundaries, consecutive lanes at consecutive addresses (a quad may end one lowered row and
+    // begin the next); the up to three floats before the first boundary and after the last go out
+    // singly.  Stores that straddle the boundaries (a lane per quad of a row, as below) measured
+    // 20 % slower on rows of 363 floats.
+    float *ob = dst + ((size_t)bi * P.m + r0) * P.m * P.rowlen;
+    const int L = rb * P.m * P.rowlen;
+    const int head = min((int)((4 - ((reinterpret_cast<uintptr_t>(ob) >> 2) & 3)) & 3), L);
+    const int nq = (L - head) >> 2;
+    // tile index of the flat element at row position rp = rl*m + c, column j of the lowered row
+    auto tix = [&](int rp, int j) -> int {
+      const int rl = P.RB > 1 ? (int)fdiv((uint32_t)rp, P.div_m) : 0;
+      return (rl * P.TW + (rp - rl * P.m)) * P.s + offs[j];
+    };
+    const uint32_t step = 4u * T;
+    const int drp = (int)fdiv(step, P.div_seg), dj = (int)(step - (uint32_t)drp * P.rowlen);
+    int rp = (int)fdiv((uint32_t)(head + 4 * tid), P.div_seg), j = head + 4 * tid - rp * P.rowlen;
+#pragma unroll 2
+    for (int q = tid; q < nq; q += T) {
+      float w[4];
+      if (j + 3 < P.rowlen) {
+        const int rl = P.RB > 1 ? (int)fdiv((uint32_t)rp, P.div_m) : 0;
+        const float *t = tile + (rl * P.TW + (rp - rl * P.m)) * P.s;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = t[offs[j + i]];
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int ji = j + i, wrap = ji >= P.rowlen;
+          w[i] = tile[tix(rp + wrap, ji - (wrap ? P.rowlen : 0))];
+        }
+      }
+      *reinterpret_cast<lower_f4 *>(ob + head + 4 * (size_t)q) = lower_f4{w[0], w[1], w[2], w[3]};
+      rp += drp; j += dj;
+      if (j >= P.rowlen) { j -= P.rowlen; ++rp; }
+    }
+    const int ntail = L - head - 4 * nq;
+    if (tid < head + ntail) {
+      const int f = tid < head ? tid : head + 4 * nq + (tid - head);
+      const int rpf = (int)fdiv((uint32_t)f, P.div_seg);
+      ob[f] = tile[tix(rpf, f - rpf * P.rowlen)];
+    }
+    return;
+  }
+  // Otherwise a lane owns a unit -- 4 consecutive positions of a lowered row (one 16-byte store;
+  // dword alignment is all such a store needs) or one of the seg % 4 positions left over -- and a
+  // group of output columns, and walks over the band.  Short rows (few units) are spread over
+  // several column groups so that the whole workgroup stores.
   float *out_band = dst + ((size_t)bi * P.m + r0) * P.m * P.rowlen + (size_t)dd0 * P.k * P.k;
   const int nq = seg >> 2, units = nq + (seg & 3);
   const int groups = units < T ? min(T / units, P.m) : 1;
@@ -203,29 +251,33 @@ extern "C" int cct_hip_lower_cube(float *dst, const float *src, const cct_pmap_h
   P.div_k = make_fastdiv(P.k);
   P.div_seg = make_fastdiv(P.seglen);
   P.div_n = make_fastdiv(P.n);
+  P.div_m = make_fastdiv(P.m);
+  P.flat = P.nslabs == 1 && (P.rowlen & 3) != 0;
   P.div_chunk = make_fastdiv(P.chunk_full);
 
   const size_t lds_bytes = lds_need(P.RB, P.DS);
-  // block size: a multiple of 64 close to a whole number of (unit, column group) work items; rows
-  // with many units take the size that wastes the fewest lanes of the last pass
+  // block size (a multiple of 64).  Flat stores balance any size: the largest workgroup unless the
+  // band is small.  Otherwise close to a whole number of (unit, column group) work items; rows
+  // with many units take the largest size (measured faster than the size that wastes the fewest
+  // lanes of the last pass: more stores in flight per compute unit).
   const long units = P.seglen / 4 + P.seglen % 4;
-  int threads = 256;
-  if (units < LOWER_MAX_THREADS) {
+  int threads = LOWER_MAX_THREADS;
+  if (P.flat) {
+    const long quads = (long)P.RB * P.m * P.rowlen / 4;
+    if (quads < 4 * LOWER_MAX_THREADS) threads = (int)((quads / 4 + 63) / 64 * 64);
+    if (threads < 128) threads = 128;
+  } else if (units < LOWER_MAX_THREADS) {
     // several column groups per workgroup: as many lanes as the groups use, rounded up to wavefronts
     const long groups = LOWER_MAX_THREADS / units < P.m ? LOWER_MAX_THREADS / units : P.m;
     threads = (int)((units * groups + 63) / 64 * 64);
     if (threads > LOWER_MAX_THREADS) threads = LOWER_MAX_THREADS;
     if (threads < 128) threads = 128;
-  } else {
-    // long rows: the largest workgroup (measured faster than the size that wastes the fewest lanes of the
-    // last pass: more stores in flight per compute unit)
-    threads = LOWER_MAX_THREADS;
   }
   hipStream_t st = ctx().stream;
   static LdsGrant grant;
   if (int rc = grant_dynamic_lds((const void *)lower_kernel, lds_bytes, grant)) return rc;
   hipLaunchKernelGGL(lower_kernel, dim3(P.nblocks), dim3(threads), lds_bytes, st, dst, src, P);
   CCT_LAUNCH_CHECK();
-  note_kernel("lower_kernel threads=%d", threads);
+  note_kernel("lower_kernel threads=%d%s", threads, P.flat ? " flat" : "");
   return 0;
 }
