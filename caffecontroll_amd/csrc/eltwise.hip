@@ -635,44 +635,66 @@ __global__ __launch_bounds__(TPB) void lrn_bwd_kernel(float *__restrict__ ig, co
   ig[e] = acc;
 }
 
-// Forward with one lane per (image, pixel, run of CH channels): the CH + 2*WN inputs under the run
-// are loaded once (all loads in flight together) and every channel's window is summed afresh from
-// them in ascending channel order -- the sums lrn_fwd_kernel forms (terms outside the depth enter
-// as +0, which leaves a sum of squares unchanged), a third of its loads and an eighth of its index
-// arithmetic.
+// Forward with one lane per (image, run of CH channels, four consecutive pixels of the plane): the
+// CH + 2*WN inputs under the run are loaded once (all loads in flight together) and every channel's
+// window is summed afresh from them in ascending channel order -- the sums lrn_fwd_kernel forms
+// (terms outside the depth enter as +0, which leaves a sum of squares unchanged), a third of its
+// loads and a fraction of its index arithmetic.  Every load and store moves 16 bytes (at dword
+// alignment: planes of 27 x 27 or 13 x 13 floats start anywhere), so a wavefront touches 1 KB of a
+// plane per instruction.  The last quad of a plane holds rc % 4 pixels and takes the scalar route.
+typedef float lrn_f4u __attribute__((ext_vector_type(4), aligned(4)));
 template <int WN, int CH, int MODE>
-__global__ __launch_bounds__(TPB) void lrn_fwd_run_kernel(float *__restrict__ out, float *__restrict__ denoms,
-                                                          const float *__restrict__ in, int rc, int D,
-                                                          uint32_t total, int nruns, float aos, float beta,
-                                                          FastDiv div_rc, FastDiv div_runs) {
+__global__ __launch_bounds__(TPB) void lrn_fwd_quad_kernel(float *__restrict__ out, float *__restrict__ denoms,
+                                                           const float *__restrict__ in, int rc, int D,
+                                                           uint32_t total, int nruns, int nqp, float aos,
+                                                           float beta, FastDiv div_qp, FastDiv div_runs) {
   const uint32_t e = blockIdx.x * TPB + threadIdx.x;
   if (e >= total) return;
-  // e = (ib*nruns + run)*rc + q
-  const uint32_t t1 = fdiv(e, div_rc);
-  const uint32_t q = e - t1 * rc;
+  // e = (ib*nruns + run)*nqp + quad
+  const uint32_t t1 = fdiv(e, div_qp);
+  const int q0 = 4 * (int)(e - t1 * nqp);
   const uint32_t ib = fdiv(t1, div_runs);
   const int c0 = (int)(t1 - ib * nruns) * CH;
-  const size_t base = (size_t)ib * D * rc + q;
+  const size_t base = (size_t)ib * D * rc + q0;
+  const int nv = min(4, rc - q0);  // pixels of this quad
   constexpr int NW = CH + 2 * WN;
-  float xw[NW];
+  lrn_f4u xw[NW];
 #pragma unroll
   for (int i = 0; i < NW; ++i) {
     const int c = c0 - WN + i;
     const int cc = min(max(c, 0), D - 1);           // clamped: the load needs no branch
-    const float v = in[base + (size_t)cc * rc];
-    xw[i] = (c >= 0 && c < D) ? v : 0.0f;
+    const float *p = in + base + (size_t)cc * rc;
+    lrn_f4u v;
+    if (nv == 4) {
+      v = *reinterpret_cast<const lrn_f4u *>(p);
+    } else {
+      v = lrn_f4u{p[0], nv > 1 ? p[1] : 0.0f, nv > 2 ? p[2] : 0.0f, 0.0f};
+    }
+    xw[i] = (c >= 0 && c < D) ? v : lrn_f4u{0.0f, 0.0f, 0.0f, 0.0f};
   }
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
     const int ch = c0 + c;
     if (ch >= D) break;
-    float sum = 0.0f;
+    lrn_f4u sum = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int j = 0; j <= 2 * WN; ++j) sum += xw[c + j] * xw[c + j];
-    const float scale = aos * sum + 1.0f;
+    lrn_f4u scale, y;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      scale[t] = aos * sum[t] + 1.0f;
+      y[t] = MODE == LRN_POW_LIBM ? xw[c + WN][t] / powf(scale[t], beta)
+                                  : xw[c + WN][t] * fast_rcp(lrn_pow(scale[t], beta, MODE));
+    }
     const size_t o = base + (size_t)ch * rc;
-    denoms[o] = scale;
-    out[o] = MODE == LRN_POW_LIBM ? xw[c + WN] / powf(scale, beta) : xw[c + WN] * fast_rcp(lrn_pow(scale, beta, MODE));
+    if (nv == 4) {
+      *reinterpret_cast<lrn_f4u *>(denoms + o) = scale;
+      *reinterpret_cast<lrn_f4u *>(out + o) = y;
+    } else {
+#pragma unroll
+      for (int t = 0; t < 3; ++t)
+        if (t < nv) { denoms[o + t] = scale[t]; out[o + t] = y[t]; }
+    }
   }
 }
 
@@ -1163,16 +1185,29 @@ int cct_hip_lrn_forward(float *out, const float *in, const cct_lrn_forward_args 
   if (total == 0) return 0;
   const int mode = lrn_pow_mode(a2->alpha_over_size, a2->beta);
   if (a->norm_window == 2) {
-    constexpr int CH = 16;  // twenty loads per sixteen outputs (runs of 8: 54 -> 49 us on norm1; the backward kernel, with four tensors' worth of registers per channel, is fastest at 8)
-    const int nruns = (a->iD + CH - 1) / CH, rc = a->iR * a->iC;
-    const size_t lanes = (size_t)a->iB * nruns * rc;
-#define CCT_LRN_FWD(MODE)                                                                                      \
-  hipLaunchKernelGGL((lrn_fwd_run_kernel<2, CH, MODE>), dim3(blocks_for(lanes)), dim3(TPB), 0, ctx().stream, out, \
-                     (float *)a->denoms, in, rc, a->iD, (uint32_t)lanes, nruns, a2->alpha_over_size, a2->beta,  \
-                     make_fastdiv(rc), make_fastdiv(nruns))
+    // Four pixels per lane and a run of CH channels: the longest run (fewest halo loads: CH + 4 loads
+    // per CH outputs) that still leaves some six workgroups per compute unit; the kernel runs for
+    // 25-50 us and is latency-bound below that (CaffeNet: norm1 runs of 8, norm2 runs of 4).
+    const int rc = a->iR * a->iC, nqp = (rc + 3) / 4;
+    const size_t want = (size_t)6 * TPB * (ctx().compute_units > 0 ? ctx().compute_units : 256);
+    int ch = 16;
+    while (ch > 4 && (size_t)a->iB * ((a->iD + ch - 1) / ch) * nqp < want) ch >>= 1;
+    const int nruns = (a->iD + ch - 1) / ch;
+    const size_t lanes = (size_t)a->iB * nruns * nqp;
+#define CCT_LRN_FWD_CH(MODE, CH)                                                                                \
+  hipLaunchKernelGGL((lrn_fwd_quad_kernel<2, CH, MODE>), dim3(blocks_for(lanes)), dim3(TPB), 0, ctx().stream, out, \
+                     (float *)a->denoms, in, rc, a->iD, (uint32_t)lanes, nruns, nqp, a2->alpha_over_size, a2->beta, \
+                     make_fastdiv(nqp), make_fastdiv(nruns))
+#define CCT_LRN_FWD(MODE)                      \
+  do {                                         \
+    if (ch == 16) CCT_LRN_FWD_CH(MODE, 16);    \
+    else if (ch == 8) CCT_LRN_FWD_CH(MODE, 8); \
+    else CCT_LRN_FWD_CH(MODE, 4);              \
+  } while (0)
     if (mode == LRN_POW_34) CCT_LRN_FWD(LRN_POW_34);
     else if (mode == LRN_POW_EXP2) CCT_LRN_FWD(LRN_POW_EXP2);
     else CCT_LRN_FWD(LRN_POW_LIBM);
+#undef CCT_LRN_FWD_CH
 #undef CCT_LRN_FWD
     CCT_LAUNCH_CHECK();
     return 0;
@@ -1193,6 +1228,8 @@ int cct_hip_lrn_backward(float *in_grad, const float *out_grad, const cct_lrn_ba
   if (total == 0) return 0;
   const int mode = lrn_pow_mode(a->alpha_over_size, a->beta);
   if (a->norm_window == 2) {
+    // one pixel per lane, runs of eight channels: with four tensors' worth of registers per window
+    // slot, two or four pixels per lane measured 10-40 % slower
     constexpr int CH = 8;
     const int nruns = (a->oD + CH - 1) / CH;
     const size_t lanes = (size_t)a->oB * nruns * a->oR * a->oC;
