@@ -528,15 +528,20 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict
 // tuning knob pool_plane = 1 takes the plane-tiled kernels at any size (used by the tests on small shapes)
 static bool force_pool_plane() { return tuning().pool_plane == 1; }
 
-// planes per workgroup: enough elements to keep 256 lanes busy for a few rounds, within the LDS tile
-static int pool_planes_per_block(size_t plane_words, size_t work_words, size_t planes) {
+// planes per workgroup, within the LDS tile.  `backward`: plane_words = the staged (gradient, arg-max)
+// pairs of a plane, work_words = the input-gradient elements it yields.
+static int pool_planes_per_block(size_t plane_words, size_t work_words, size_t planes, bool backward) {
   // small tensors are launch-bound; the one-lane-per-element kernels finish them sooner
   if (planes * (plane_words > work_words ? plane_words : work_words) < (1u << 20) && !force_pool_plane()) return 0;
   if (plane_words == 0 || plane_words > (size_t)kPoolLdsWords) return 0;
   // at most 20 KB of LDS per workgroup where a plane allows it: eight workgroups share a compute
   // unit and their load and store phases overlap
   size_t pp = plane_words > 5120 ? 1 : 5120 / plane_words;
-  const size_t want = (2048 + work_words - 1) / work_words;  // ~8 elements per lane
+  // Measured on the CaffeNet layers (planes of 55 x 55, 27 x 27, 13 x 13): the forward kernel is
+  // fastest with some 2300 staged inputs per workgroup (1 / 4 / 14 planes), the backward kernel
+  // with some 8000 gradient elements but no more than sixteen planes (3 / 12 / 16).
+  size_t want = backward ? (8192 + work_words - 1) / work_words : (2304 + plane_words - 1) / plane_words;
+  if (want > 16) want = 16;
   if (pp > want) pp = want;
   if (pp > planes) pp = planes;
   return (int)(pp < 1 ? 1 : pp);
@@ -1082,7 +1087,7 @@ int cct_hip_maxpool_forward(float *out, const float *in, const cct_pool_args *a)
   const size_t total = (size_t)a->D * a->B * a->oR * a->oC;
   if (total == 0) return 0;
   const size_t planes = (size_t)a->D * a->B, iplane = (size_t)a->iR * a->iC, oplane = (size_t)a->oR * a->oC;
-  if (const int pp = pool_planes_per_block(iplane, oplane, planes)) {
+  if (const int pp = pool_planes_per_block(iplane, oplane, planes, false)) {
     hipLaunchKernelGGL(maxpool_fwd_plane_kernel, dim3((uint32_t)((planes + pp - 1) / pp)), dim3(TPB),
                        (size_t)pp * iplane * sizeof(float), ctx().stream,
                        out, a->max_index, in, *a, (uint32_t)planes, pp, make_fastdiv(a->oC),
@@ -1106,7 +1111,7 @@ static int maxpool_backward_impl(float *in_grad, const float *out_grad, const cc
   const size_t total = (size_t)a->D * a->B * a->iR * a->iC;
   if (total == 0) return 0;
   const size_t planes = (size_t)a->D * a->B, iplane = (size_t)a->iR * a->iC, oplane = (size_t)a->oR * a->oC;
-  const int pp = pool_planes_per_block(2 * oplane, iplane, planes);
+  const int pp = pool_planes_per_block(2 * oplane, iplane, planes, true);
   const bool quad = pp && a->stride >= 2 && a->kernel_size <= 2 * a->stride && a->iC <= 256;
   if (pooled && !quad) {
     // the other kernels do not switch windows off while they stage: a pass over the (small) output
