@@ -27,14 +27,15 @@ CONFIGS = {
 }
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch (fetched + written) at the alexnet_conv2 shape, from rocprofv3 --pmc FETCH_SIZE
+# HBM bytes per launch (fetched + written) at the alexnet_conv2 and alexnet_conv1 shapes, from rocprofv3 --pmc FETCH_SIZE
 # and WRITE_SIZE runs of this file (one counter per run), each scaled by what the same counter
 # reads for a 1 GiB device copy (factors 2.000 and 1.000).  Not measured by this run: the record
 # names the summary under profiles/ the figure comes from.  Keyed by (stage, the kernel instance
 # the library reports it launched), so that a change of tile choice leaves `traffic` null instead
 # of attaching an old figure to another kernel.
 TRAFFIC_SOURCE = {"direct": "profiles/conv2_fwd_bwd_hbm_traffic_and_mfma.md",
-                  "lowering": "profiles/conv2_lowering_path_hbm_traffic_and_mfma.md"}
+                  "lowering": "profiles/conv2_lowering_path_hbm_traffic_and_mfma.md",
+                  "conv1": "profiles/conv1_fwd_bwd_trace_traffic_mfma.md"}
 TRAFFIC_BYTES = {
     ("GEMM", "conv_direct_kernel<5,1,2,1,32>"): ((238.5 + 230.6) * 1e6, "direct"),
     ("GEMM Data", "conv_direct_kernel<5,1,2,1,32>"): ((320.6 + 76.2) * 1e6, "direct"),
@@ -44,13 +45,17 @@ TRAFFIC_BYTES = {
     ("GEMM Wghts", "gemm_kernel<Tile<256,128,16,2,2>,true,false,true> splits=26"): ((2384.4 + 63.9) * 1e6, "lowering"),
     ("Lower Cube", "lower_kernel threads=512"): ((75.6 + 1791.6) * 1e6, "lowering"),
     ("Inverse Lwr", "lift_kernel<5,1> bias_blocks=256"): ((2190.6 + 71.7) * 1e6, "lowering"),
+    # alexnet_conv1 (the kernel instances differ from every conv2 one, so the keys cannot collide)
+    ("GEMM", "conv_strided_reg_kernel<11,4,3>"): ((160.8 + 302.6) * 1e6, "conv1"),
+    ("GEMM Data", "conv_direct16_kernel<3,3,1,64>"): ((301.2 + 158.6) * 1e6, "conv1"),
+    ("GEMM Wghts", "conv_strided_wgrad_spec_kernel<11,4,3,14,8,11> waves=3x4"): ((469.4 + 54.2) * 1e6, "conv1"),
 }
 
 
 def traffic_of(cfg, stage, kernel):
     """(bytes, source file) from the committed counter summaries, or (None, None) when the kernel
     instance that ran is not the one that was profiled."""
-    if cfg != "alexnet_conv2":
+    if cfg not in ("alexnet_conv2", "alexnet_conv1"):
         return None, None
     ent = TRAFFIC_BYTES.get((stage, kernel))
     return (ent[0], TRAFFIC_SOURCE[ent[1]]) if ent else (None, None)
