@@ -45,7 +45,8 @@ struct GemmArgs {
   int fmap;         // EPI_CONV_FORWARD: columns per image
   FastDiv div_fmap;
   const float *bias;
-  int relu;         // EPI_CONV_FORWARD: clamp at zero after the bias
+  int relu;         // clamp at zero after the bias (EPI_CONV_FORWARD; EPI_ALPHA_BETA with col_bias)
+  const float *col_bias;  // EPI_ALPHA_BETA: added to every row of C (one value per column), or null
   int tiles_m, tiles_n;
   uint32_t ntiles;
   int a_vec, b_vec;  // operand allows aligned 16-byte global loads
@@ -491,6 +492,11 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
     float *crow = ((MODE == EPI_SPLITK_PARTIAL) ? g.ws + (size_t)kslice * g.M * g.N : g.C) +
                   (size_t)row0 * rstride + col0;
     const float alpha = g.alpha;
+    // column bias and clamp of the plain epilogue (a fully connected layer's forward pass); uniform
+    const bool post = MODE == EPI_ALPHA_BETA && (g.col_bias || g.relu);
+    float cb[T::TN];
+#pragma unroll
+    for (int b = 0; b < T::TN; ++b) cb[b] = (post && g.col_bias) ? g.col_bias[col0 + b * 32] : 0.0f;
 #pragma unroll
     for (int a = 0; a < T::TM; ++a)
 #pragma unroll
@@ -500,8 +506,14 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
           if (ROWGUARD && row0 + a * 32 + 8 * j + i >= g.M) continue;
           float *c = crow + (size_t)(a * 32 + 8 * j + i) * rstride;
 #pragma unroll
-          for (int b = 0; b < T::TN; ++b)
-            c[b * 32] = (MODE == EPI_SPLITK_PARTIAL) ? acc[a][b][4 * j + i] : alpha * acc[a][b][4 * j + i];
+          for (int b = 0; b < T::TN; ++b) {
+            float y = (MODE == EPI_SPLITK_PARTIAL) ? acc[a][b][4 * j + i] : alpha * acc[a][b][4 * j + i];
+            if (post) {
+              if (g.col_bias) y += cb[b];
+              if (g.relu && !(y > 0.0f)) y = 0.0f;
+            }
+            c[b * 32] = y;
+          }
         }
   }
 }
@@ -580,7 +592,9 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
         const float x = acc[a][b][v];
         if (g.epi == EPI_ALPHA_BETA) {
           float *c = g.C + (size_t)row * g.ldc + col_off;
-          const float y = (g.beta == 0.0f) ? g.alpha * x : g.alpha * x + g.beta * (*c);
+          float y = (g.beta == 0.0f) ? g.alpha * x : g.alpha * x + g.beta * (*c);
+          if (g.col_bias) y += g.col_bias[col];
+          if (g.relu && !(y > 0.0f)) y = 0.0f;
           if (g.nt_store) __builtin_nontemporal_store(y, c);
           else *c = y;
         } else if (g.epi == EPI_SPLITK_PARTIAL) {
@@ -596,11 +610,12 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
   }
 }
 
-// C = alpha * sum_z ws[z] + beta * C, z ascending (fixed order)
+// C = alpha * sum_z ws[z] + beta * C, z ascending (fixed order); then the optional column bias and clamp
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *__restrict__ C,
                                                             const float *__restrict__ ws, int M, int N,
                                                             int ldc, int splits, float alpha, float beta,
-                                                            FastDiv div_n) {
+                                                            FastDiv div_n, const float *__restrict__ col_bias,
+                                                            int relu) {
   const uint32_t e = blockIdx.x * 256 + threadIdx.x;
   if (e >= (uint32_t)M * N) return;
   const uint32_t row = fdiv(e, div_n);
@@ -619,7 +634,10 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *__restrict__ 
   }
   for (; z < splits; ++z, p += mn) s += *p;
   float *c = C + (size_t)row * ldc + col;
-  *c = (beta == 0.0f) ? alpha * s : alpha * s + beta * (*c);
+  float y = (beta == 0.0f) ? alpha * s : alpha * s + beta * (*c);
+  if (col_bias) y += col_bias[col];
+  if (relu && !(y > 0.0f)) y = 0.0f;
+  *c = y;
 }
 
 typedef Tile<256, 128, 16, 2, 2> TileL;
@@ -661,13 +679,13 @@ static int launch_cfg(GemmArgs &g, bool a_kc, bool b_kc, int splits, hipStream_t
 // (cblas Trans).
 static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha, const float *A, int lda,
                          const float *B, int ldb, float beta, float *C, int ldc, int epi, int fmap,
-                         const float *bias, int relu = 0) {
+                         const float *bias, int relu = 0, const float *col_bias = nullptr) {
   if (M <= 0 || N <= 0) return 0;
   hipStream_t st = ctx().stream;
   GemmArgs g;
   g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
   g.alpha = alpha; g.beta = beta; g.epi = epi; g.fmap = fmap > 0 ? fmap : 1;
-  g.div_fmap = make_fastdiv((uint32_t)g.fmap); g.bias = bias; g.relu = relu; g.ws = nullptr;
+  g.div_fmap = make_fastdiv((uint32_t)g.fmap); g.bias = bias; g.relu = relu; g.col_bias = col_bias; g.ws = nullptr;
   // 16-byte global loads need dword alignment only
   g.a_vec = ((uintptr_t)A % 4 == 0);
   g.b_vec = ((uintptr_t)B % 4 == 0);
@@ -745,7 +763,7 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
     CCT_REQUIRE((size_t)M * N < (1ull << 31), "sgemm: split-K result too large");
     const uint32_t blocks = (uint32_t)(((size_t)M * N + 255) / 256);
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, st, C, g.ws, M, N, ldc, splits,
-                       alpha, beta, make_fastdiv((uint32_t)N));
+                       alpha, beta, make_fastdiv((uint32_t)N), col_bias, relu);
     CCT_LAUNCH_CHECK();
   }
   return 0;
@@ -784,6 +802,19 @@ extern "C" int cct_hip_sgemm_new(int TA, int TB, int M, int N, int K, float alph
   const int lda = (TA == CCT_NO_TRANS) ? K : M;
   const int ldb = (TB == CCT_NO_TRANS) ? N : K;
   return cct_hip_sgemm(CCT_ROW_MAJOR, TA, TB, M, N, K, alpha, A, lda, B, ldb, beta, C, N);
+}
+
+extern "C" int cct_hip_sgemm_new_bias(int TA, int TB, int M, int N, int K, float alpha, const float *A,
+                                      const float *B, float beta, float *C, const float *col_bias, int relu) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE((TA == CCT_NO_TRANS || TA == CCT_TRANS) && (TB == CCT_NO_TRANS || TB == CCT_TRANS),
+              "sgemm_new_bias: bad transpose flags %d %d", TA, TB);
+  CCT_REQUIRE(M >= 0 && N >= 0 && K >= 0, "sgemm_new_bias: negative dimension");
+  if (M == 0 || N == 0) return 0;
+  CCT_REQUIRE(A && B && C, "sgemm_new_bias: null matrix");
+  const int lda = (TA == CCT_NO_TRANS) ? K : M, ldb = (TB == CCT_NO_TRANS) ? N : K;
+  return gemm_rowmajor(TA == CCT_NO_TRANS, TB == CCT_TRANS, M, N, K, alpha, A, lda, B, ldb, beta, C, N,
+                       EPI_ALPHA_BETA, 0, nullptr, relu != 0, col_bias);
 }
 
 extern "C" int cct_hip_sgemm_conv_forward(int o, int batch, int fmap, int K, const float *model,

@@ -71,19 +71,18 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
   LogicalCubeType *get_model_grad_cube() override { return p_model_gradient_cube; }
   LogicalCubeType *get_bias_grad_cube() override { return p_bias_gradient_cube; }
 
-  // Y[B x O] = X[B x I] * W^T, then the bias through forward_bias with a 1x1 feature map
-  // (the non-CPU branch of the reference, :224-228)
+  // Y[B x O] = X[B x I] * W^T + bias: the reference's non-CPU branch runs sgemm_new and then
+  // forward_bias with a 1x1 feature map (:224-228); here the bias, and the clamp of an in-place ReLU
+  // that directly follows (set_fuse_relu), ride on the GEMM's output pass -- the same sums in the
+  // same order, two or three launches fewer per layer.
+  void set_fuse_relu(bool on) { fuse_relu_ = on; }
   void forward() override {
     this->report_forward_history.reset();
     LogicalCubeType *input_d_cube = p_input_layer->p_data_cube;
     LogicalCubeType *output_d_cube = p_output_layer->p_data_cube;
-    p_driver->sgemm_new(CblasNoTrans, CblasTrans, data_R, model_R, model_C, 1.f, input_d_cube->get_p_data(),
-                        p_model_cube->get_p_data(), 0.f, output_d_cube->get_p_data());
-    if (bias_term) {
-      DeviceMemoryPointer output = output_d_cube->get_device_pointer(p_driver);
-      DeviceMemoryPointer bias = p_bias_cube->get_device_pointer(p_driver);
-      p_driver->forward_bias(&bias, &output, 1, (int)oD, (int)iB);
-    }
+    p_driver->sgemm_new_bias(CblasNoTrans, CblasTrans, data_R, model_R, model_C, 1.f, input_d_cube->get_p_data(),
+                             p_model_cube->get_p_data(), 0.f, output_d_cube->get_p_data(),
+                             bias_term ? p_bias_cube->get_p_data() : nullptr, fuse_relu_);
     this->report_forward_history.end();
   }
 
@@ -112,6 +111,7 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
   LogicalCubeType *p_model_gradient_cube;
   LogicalCubeType *p_bias_gradient_cube;
   int data_R, data_C, model_R, model_C;
+  bool fuse_relu_ = false;
 
   void initialize_logical_cube(const LogicalCubeType *cube, const cnn::FillerParameter &filler_param) {
     DeviceMemoryPointer data = cube->get_device_pointer(p_driver);

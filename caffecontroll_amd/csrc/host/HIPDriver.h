@@ -221,6 +221,12 @@ class HIPDriver {
                  const float alpha, const float *pA, const float *pB, const float beta, float *pC) {
     ok(cct_hip_sgemm_new(TA, TB, M, N, K, alpha, pA, pB, beta, pC), "sgemm_new");
   }
+  // sgemm_new with a bias per column of C and, optionally, the clamp of a following ReLU in the same pass
+  void sgemm_new_bias(const CBLAS_TRANSPOSE TA, const CBLAS_TRANSPOSE TB, const int M, const int N, const int K,
+                      const float alpha, const float *pA, const float *pB, const float beta, float *pC,
+                      const float *col_bias, bool relu = false) {
+    ok(cct_hip_sgemm_new_bias(TA, TB, M, N, K, alpha, pA, pB, beta, pC, col_bias, relu ? 1 : 0), "sgemm_new_bias");
+  }
   void sgemm_conv_forward(int o, int batch, int fmap, int K, const float *model, const float *lowered,
                           const float *bias, float *out, bool relu = false) {
     ok(cct_hip_sgemm_conv_forward(o, batch, fmap, K, model, lowered, bias, out, relu ? 1 : 0), "sgemm_conv_forward");

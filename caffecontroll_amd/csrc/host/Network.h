@@ -265,6 +265,11 @@ class Network {
             for (BridgeT *cb : nodes_[producer_node].bridges)
               static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(cb)->sub_bridge()->set_fuse_relu(true);
             rb->forward_done_by_producer = true;
+          } else if (producer_node >= 0 && nodes_[producer_node].spec.type == CCT_LAYER_FC) {
+            // likewise after an inner-product layer: the clamp rides on the GEMM's output pass
+            for (BridgeT *fb : nodes_[producer_node].bridges)
+              static_cast<ParallelizedBridge<float, FullyConnectedBridge, HIPDriver> *>(fb)->sub_bridge()->set_fuse_relu(true);
+            rb->forward_done_by_producer = true;
           }
           nd.bridges.push_back(rb);
           break;

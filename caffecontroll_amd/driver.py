@@ -115,6 +115,11 @@ class HIPDriver:
         check(self.lib.cct_hip_sgemm(order, TA, TB, M, N, K, alpha, _p(A), lda, _p(B), ldb, beta,
                                      _p(Cm), ldc), "sgemm")
 
+    def sgemm_new_bias(self, TA, TB, M, N, K, alpha, A, B, beta, Cm, col_bias=None, relu=False):
+        """sgemm_new, then Cm[m][n] += col_bias[n] and, with relu, max(., 0), in the same pass."""
+        check(self.lib.cct_hip_sgemm_new_bias(TA, TB, M, N, K, alpha, _p(A), _p(B), beta, _p(Cm), _p(col_bias),
+                                              int(relu)), "sgemm_new_bias")
+
     def sgemm_new(self, TA, TB, M, N, K, alpha, A, B, beta, Cm):
         check(self.lib.cct_hip_sgemm_new(TA, TB, M, N, K, alpha, _p(A), _p(B), beta, _p(Cm)), "sgemm_new")
 

@@ -172,6 +172,14 @@ int cct_hip_sgemm(int order, int TA, int TB, int M, int N, int K, float alpha, c
  * lda = (TA==N ? K : M), ldb = (TB==N ? N : K), ldc = N. */
 int cct_hip_sgemm_new(int TA, int TB, int M, int N, int K, float alpha, const float *A,
                       const float *B, float beta, float *C);
+/* cct_hip_sgemm_new followed by the bias over a 1 x 1 feature map, in one pass: the non-CPU branch of
+ * FullyConnectedBridge::forward (src/bridges/FullyConnectedBridge_impl.hxx:224-228 -- sgemm_new, then
+ * forward_bias).  C[m][n] = alpha * op(A) op(B) + beta * C[m][n] + col_bias[n] (col_bias may be NULL);
+ * relu != 0 also applies the ReLU of a following in-place ReLUBridge (max(x, 0),
+ * src/kernels/relu.hxx:10-25) before the store.  The sums are those of the two separate calls, in
+ * the same order: identical results. */
+int cct_hip_sgemm_new_bias(int TA, int TB, int M, int N, int K, float alpha, const float *A,
+                           const float *B, float beta, float *C, const float *col_bias, int relu);
 /* Forward-convolution GEMM with the output permutation and bias of
  * ConvolutionBridge::forward (src/bridges/ConvolutionBridge_impl.hxx:328-364) folded into the
  * epilogue: out[b][o][fmap] = model[o x K] * lowered[b*fmap x K]^T + bias[o] (bias may be NULL).

@@ -142,6 +142,34 @@ def test_sgemm_new_fc_shapes(oracle):
     assert rel_err(host(dx), rdx) <= TOL and rel_err(host(dw), rdw) <= TOL and rel_err(host(db), rdb) <= TOL
 
 
+FC_FWD_SHAPES = [(64, 500, 800), (64, 10, 500), (256, 1000, 4096), (37, 53, 129), (130, 257, 64), (5, 3, 7)]
+
+
+@pytest.mark.parametrize("shape", FC_FWD_SHAPES)
+@pytest.mark.parametrize("bias,relu", [(True, False), (True, True), (False, True)])
+def test_sgemm_new_bias_equals_the_separate_calls(shape, bias, relu):
+    """The forward pass of FullyConnectedBridge in one call (sgemm_new + forward_bias over a 1x1
+    feature map, src/bridges/FullyConnectedBridge_impl.hxx:224-228, + the in-place ReLU that may
+    follow): bit-identical to the separate calls, whole tiles and ragged ones, with and without the
+    split over the contraction."""
+    M, N, K = shape
+    rng = np.random.default_rng(M * 7 + N)
+    drv = driver()
+    X = dev(rng.standard_normal((M, K)).astype(np.float32))
+    W = dev((rng.standard_normal((N, K)) * 0.1).astype(np.float32))
+    b = dev(rng.standard_normal(N).astype(np.float32)) if bias else None
+    sep, fused = empty((M, N)), empty((M, N))
+    drv.sgemm_new(N_, T_, M, N, K, 1.0, X, W, 0.0, sep)
+    if bias:
+        drv.forward_bias(b, sep, 1, N, M)
+    if relu:
+        drv.relu_forward(sep, sep, M * N)
+    drv.sgemm_new_bias(N_, T_, M, N, K, 1.0, X, W, 0.0, fused, b, relu)
+    np.testing.assert_array_equal(host(fused), host(sep))
+    if relu:
+        assert (host(fused) >= 0).all() and (M * N < 100 or (host(fused) == 0).any())
+
+
 def test_sgemv(oracle):
     rng = np.random.default_rng(7)
     M, N = 130, 70
