@@ -610,12 +610,14 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
   }
 }
 
-// C = alpha * sum_z ws[z] + beta * C, z ascending (fixed order); then the optional column bias and clamp
+// C = alpha * sum_z ws[z] + beta * C, z ascending (fixed order); then the optional column bias and clamp.
+// fmap > 0: the epilogue of the forward convolution instead (output permutation, bias per row, clamp).
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *__restrict__ C,
                                                             const float *__restrict__ ws, int M, int N,
                                                             int ldc, int splits, float alpha, float beta,
                                                             FastDiv div_n, const float *__restrict__ col_bias,
-                                                            int relu) {
+                                                            int relu, const float *__restrict__ row_bias, int fmap,
+                                                            FastDiv div_fmap) {
   const uint32_t e = blockIdx.x * 256 + threadIdx.x;
   if (e >= (uint32_t)M * N) return;
   const uint32_t row = fdiv(e, div_n);
@@ -633,6 +635,14 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *__restrict__ 
     for (int j = 0; j < 8; ++j) s += v[j];
   }
   for (; z < splits; ++z, p += mn) s += *p;
+  if (fmap > 0) {
+    // forward convolution: C is [image][row][fmap], column = image * fmap + position; bias per row
+    const uint32_t img = fdiv(col, div_fmap);
+    float y = row_bias ? s + row_bias[row] : s;
+    if (relu && !(y > 0.0f)) y = 0.0f;
+    C[((size_t)img * M + row) * fmap + (col - img * fmap)] = y;
+    return;
+  }
   float *c = C + (size_t)row * ldc + col;
   float y = (beta == 0.0f) ? alpha * s : alpha * s + beta * (*c);
   if (col_bias) y += col_bias[col];
@@ -716,11 +726,11 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
     for (int pass = 0; pass < 2; ++pass) {
       int sp = 1, kc = g.K > 0 ? g.K : bk;
       if (pass == 1) {
-        // split-K: plain epilogue only, when the tile grid alone cannot fill the device
+        // split-K, when the tile grid alone cannot fill the device (the reduction then carries the epilogue)
         // (K slices of at least 256, or 128 when the result is small enough for a cheap reduction:
         // those problems are bound by the latency of their few K steps, not by throughput)
-        const int min_chunk = (size_t)M * N <= 65536 ? 128 : 256;
-        if (epi != EPI_ALPHA_BETA || tiles >= slots || K < 2 * min_chunk) break;
+        const int min_chunk = (size_t)M * N <= 262144 ? 128 : 256;
+        if (tiles >= slots || K < 2 * min_chunk) break;
         sp = (int)(slots / tiles);
         if (sp > K / min_chunk) sp = K / min_chunk;
         if (sp < 2) break;
@@ -763,7 +773,8 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
     CCT_REQUIRE((size_t)M * N < (1ull << 31), "sgemm: split-K result too large");
     const uint32_t blocks = (uint32_t)(((size_t)M * N + 255) / 256);
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, st, C, g.ws, M, N, ldc, splits,
-                       alpha, beta, make_fastdiv((uint32_t)N), col_bias, relu);
+                       alpha, beta, make_fastdiv((uint32_t)N), col_bias, relu, bias,
+                       epi == EPI_CONV_FORWARD ? g.fmap : 0, g.div_fmap);
     CCT_LAUNCH_CHECK();
   }
   return 0;
