@@ -96,7 +96,7 @@ def test_noalloc_scratch_array_is_exported_by_the_device_code():
 
 
 def test_every_device_driver_member_is_bound_or_listed(tmp_path):
-    """The driver stub in INTEGRATION.md binds every member of the reference's DeviceDriver class
+    """The driver stub in the integration notes at the repository root binds every member of the reference's DeviceDriver class
     (src/sched/DeviceDriver.h:56-274), or the member is named in the table of members left
     unimplemented; every cct_hip_* call the stub makes is declared in include/cct_hip.h.  The
     member list is parsed from the reference header, so the test needs the reference checkout."""
