@@ -407,8 +407,8 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_plane_kernel(float *__restric
     float acc = 0.0f;
     if (TWO_BY_TWO) {
       // kernel <= 2*stride: at most two windows per direction; clamped positions keep the reads branch-free
-      const int r0 = ph_lo * a.oC, r1 = min(ph_lo + 1, a.oR - 1) * a.oC;
-      const int c0 = pw_lo, c1 = min(pw_lo + 1, a.oC - 1);
+      const int r0 = min(ph_lo, a.oR - 1) * a.oC, r1 = min(ph_lo + 1, a.oR - 1) * a.oC;
+      const int c0 = min(pw_lo, a.oC - 1), c1 = min(pw_lo + 1, a.oC - 1);
       const int x00 = x[r0 + c0], x01 = x[r0 + c1], x10 = x[r1 + c0], x11 = x[r1 + c1];
       const float g00 = g[r0 + c0], g01 = g[r0 + c1], g10 = g[r1 + c0], g11 = g[r1 + c1];
       const bool row1 = ph_lo + 1 <= ph_hi, col1 = pw_lo + 1 <= pw_hi, any = ph_lo <= ph_hi && pw_lo <= pw_hi;
@@ -480,10 +480,12 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict
     const uint32_t pl = fdiv(row, div_ir);
     const int h = (int)(row - pl * a.iR), me0 = h * a.iC + w0;
     const int ph_lo = h < k ? 0 : (int)fdiv((uint32_t)(h - k), div_s) + 1;
-    const bool row1 = ph_lo + 1 <= a.oR - 1;
+    // a row below the last window (floor-based output size: (iR - k) % s rows are covered by none)
+    // has ph_lo == oR: both window rows are switched off and the reads clamped into the plane
+    const bool row0 = ph_lo <= a.oR - 1, row1 = ph_lo + 1 <= a.oR - 1;
     const float *g = tog + pl * oplane;
     const int *x = tidx + pl * oplane;
-    const int r0 = ph_lo * a.oC, r1 = min(ph_lo + 1, a.oR - 1) * a.oC;
+    const int r0 = min(ph_lo, a.oR - 1) * a.oC, r1 = min(ph_lo + 1, a.oR - 1) * a.oC;
     int xi[2][NJ];
     float gv[2][NJ];
 #pragma unroll
@@ -496,7 +498,7 @@ __global__ __launch_bounds__(TPB) void maxpool_bwd_quad_kernel(float *__restrict
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j) {
-        const bool ok = cv[j] && (i == 0 || row1);
+        const bool ok = cv[j] && (i == 0 ? row0 : row1);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           // K3S2: an even element e sits in window columns e/2 and e/2 + 1 of the three, an odd one in (e+1)/2 only

@@ -37,7 +37,9 @@ def test_relu_fixture_and_oracle(oracle):
                                  # for the LDS-tiled kernels (forward only, both, window wider than 2 strides)
                                  (7, 11, 13, 3, 2), (1, 2, 100, 3, 2), (1, 1, 150, 2, 2), (1, 1, 140, 5, 2),
                                  # rows of 27, 64 and 65 elements: the lanes-over-rows backward kernel and its limit
-                                 (3, 5, 27, 3, 2), (2, 3, 64, 3, 2), (2, 3, 65, 2, 2)])
+                                 (3, 5, 27, 3, 2), (2, 3, 64, 3, 2), (2, 3, 65, 2, 2),
+                                 # a last row and column that no window covers ((n - k) % s != 0)
+                                 (5, 15, 31, 2, 2), (3, 8, 28, 3, 2), (2, 6, 30, 3, 2)])
 @pytest.mark.parametrize("plane_tiled", [False, True])
 def test_maxpool_bit_exact(oracle, cfg, plane_tiled):
     # small tensors take the one-lane-per-element kernels unless the plane-tiled ones are forced

@@ -1,0 +1,111 @@
+"""Seeded random geometries, beyond the hand-picked ones of the other files: the convolution bridge
+on its all-direct and its lowering path, max pooling (both kernel families, with and without the
+mask of a folded ReLU) and LRN, each against the CPU oracle.  The draws include what the fixed
+lists tend to miss: trailing rows and columns no pooling window covers, paddings up to k - 1, map
+and channel counts that are not multiples of any tile, planes whose size is not a multiple of four."""
+import numpy as np
+import pytest
+
+from gpu_util import driver, dev, empty, host, rel_err, tuning
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-4
+
+
+def _conv_geometries(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        k, s = [(3, 1), (5, 1), (3, 1), (5, 1), (11, 4), (7, 2), (5, 2), (3, 2)][rng.integers(0, 8)]
+        p = int(rng.integers(0, k)) if rng.random() < 0.7 else (k - 1) // 2
+        n = int(rng.integers(max(k - 2 * p, 1), 70 if s > 1 else 64))
+        if n + 2 * p < k:
+            continue
+        m = (n + 2 * p - k) // s + 1
+        b, d, o = int(rng.integers(1, 10)), int(rng.integers(1, 40)), int(rng.integers(1, 80))
+        if 2.0 * b * m * m * k * k * d * o > 6e8 or b * m * m * k * k * d > 3e7:
+            continue
+        out.append((b, d, n, k, s, p, o))
+    return out
+
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_convolution_bridge_random_geometries(oracle, seed):
+    from caffecontroll_amd.bridges import ConvolutionLayer
+    drv = driver()
+    rng = np.random.default_rng(seed + 100)
+    direct = 0
+    for shape in _conv_geometries(seed, 40):
+        b, d, n, k, s, p, o = shape
+        m = (n + 2 * p - k) // s + 1
+        x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+        w = (rng.standard_normal((o, d, k, k)) * 0.1).astype(np.float32)
+        bias = rng.standard_normal(o).astype(np.float32)
+        og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+        ref_out, lowered = oracle.conv_forward(x, w, bias, k, s, p)
+        ref_dx, ref_dw, ref_db = oracle.conv_backward(x.shape, w, og, lowered, k, s, p)
+        for level in (3, 1):   # all direct where the kernels cover the geometry; lowering + GEMM + lifting
+            in_grad, out_data = empty((b, d, n, n)), empty((b, o, m, m))
+            layer = ConvolutionLayer(b, d, n, k, s, p, o, dev(x), in_grad, out_data, dev(og))
+            layer.set_options(fused=level)
+            direct += layer.path() == 3
+            drv.memcpy(layer.model_ptr(), w.ctypes.data, w.nbytes, 0)
+            drv.memcpy(layer.bias_ptr(), bias.ctypes.data, bias.nbytes, 0)
+            layer.forward()
+            layer.backward(with_update=False)
+            dw, db = np.empty((o, d, k, k), np.float32), np.empty((o,), np.float32)
+            drv.memcpy(dw.ctypes.data, layer.model_grad_ptr(), dw.nbytes, 1)
+            drv.memcpy(db.ctypes.data, layer.bias_grad_ptr(), db.nbytes, 1)
+            what = (shape, level, layer.path())
+            assert rel_err(host(out_data), ref_out) <= TOL, what
+            assert rel_err(host(in_grad), ref_dx) <= TOL, what
+            assert rel_err(dw, np.asarray(ref_dw).reshape(dw.shape)) <= TOL, what
+            assert rel_err(db, ref_db) <= TOL, what
+            layer.close()
+    assert direct >= 20   # most draws are inside the direct kernels' reach
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_pooling_and_lrn_random_geometries(oracle, seed):
+    import torch
+    drv = driver()
+    rng = np.random.default_rng(seed)
+    uncovered = 0
+    for case in range(60):
+        B, D, n = int(rng.integers(1, 9)), int(rng.integers(1, 40)), int(rng.integers(2, 60))
+        k, s = int(rng.integers(2, 5)), int(rng.integers(1, 4))
+        if n >= k:
+            oR = (n - k) // s + 1
+            uncovered += (n - k) % s != 0
+            x = rng.standard_normal((B, D, n, n)).astype(np.float32)
+            x[rng.random(x.shape) < 0.3] = 0
+            with tuning("pool_plane", int(rng.integers(0, 2))):
+                idx, y = empty((B, D, oR, oR), dtype=torch.int32), empty((B, D, oR, oR))
+                args = drv.pool_args(k, s, n, n, D, B, idx)
+                drv.maxpool_forward(y, dev(x), args)
+                ry, ridx = oracle.maxpool_forward(x, k, s)
+                np.testing.assert_array_equal(host(y), ry)
+                np.testing.assert_array_equal(host(idx), ridx)
+                og = rng.standard_normal(ry.shape).astype(np.float32)
+                g, gm = empty(x.shape), empty(x.shape)
+                drv.maxpool_backward(g, dev(og), args)
+                np.testing.assert_array_equal(host(g), oracle.maxpool_backward(og, ridx, n, n), err_msg=str((B, D, n, k, s)))
+                # masked with (pooled > 0): windows whose maximum is not positive pass no gradient
+                drv.maxpool_backward(gm, dev(og), args, pooled=y)
+                want = oracle.maxpool_backward(np.where(ry > 0, og, 0).astype(np.float32), ridx, n, n)
+                np.testing.assert_array_equal(host(gm), want, err_msg=str((B, D, n, k, s)))
+        size = int(rng.choice([3, 5, 5, 5, 7]))
+        alpha, beta = float(rng.choice([1e-4, 1e-2, 0.3])), float(rng.choice([0.75, 0.75, 0.5, 1.25]))
+        n2 = int(rng.integers(1, 30))
+        x = (rng.standard_normal((B, D, n2, n2)) * 3).astype(np.float32)
+        og = rng.standard_normal((B, D, n2, n2)).astype(np.float32)
+        y, den, g = empty(x.shape), empty(x.shape), empty(x.shape)
+        dx = dev(x)
+        drv.lrn_forward(y, dx, n2, n2, D, B, size, alpha, beta, den)
+        ry, rden = oracle.lrn_forward(x, size, alpha, beta)
+        what = (B, D, n2, size, alpha, beta)
+        assert rel_err(host(den), rden) <= 1e-6, what
+        assert rel_err(host(y), ry) <= 1e-5, what
+        drv.lrn_backward(g, dev(og), dx, n2, n2, D, B, size, alpha, beta, den)
+        assert rel_err(host(g), oracle.lrn_backward(og, x, rden, size, alpha, beta)) <= 1e-5, what
+    assert uncovered >= 10
