@@ -252,7 +252,7 @@ extern "C" int cct_hip_lower_cube(float *dst, const float *src, const cct_pmap_h
   P.div_seg = make_fastdiv(P.seglen);
   P.div_n = make_fastdiv(P.n);
   P.div_m = make_fastdiv(P.m);
-  P.flat = P.nslabs == 1 && (P.rowlen & 3) != 0;
+  P.flat = P.nslabs == 1 && (P.rowlen & 3) != 0 && P.rowlen >= 4;  // a quad then spans at most two lowered rows
   P.div_chunk = make_fastdiv(P.chunk_full);
 
   const size_t lds_bytes = lds_need(P.RB, P.DS);

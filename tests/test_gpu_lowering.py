@@ -17,6 +17,7 @@ SHAPES = [
     (2, 20, 12, 5, 1, 0),     # LeNet conv2
     (2, 256, 13, 3, 1, 1),    # AlexNet conv3 geometry (channel slabs)
     (1, 7, 9, 3, 2, 1), (2, 5, 8, 1, 1, 0), (1, 2, 6, 6, 1, 0), (1, 9, 10, 3, 3, 2), (5, 4, 7, 4, 2, 3),
+    (5, 1, 7, 1, 1, 0), (3, 2, 9, 1, 2, 0), (2, 3, 6, 1, 1, 0),   # lowered rows of one, two and three floats
 ]
 
 

@@ -109,3 +109,66 @@ def test_pooling_and_lrn_random_geometries(oracle, seed):
         drv.lrn_backward(g, dev(og), dx, n2, n2, D, B, size, alpha, beta, den)
         assert rel_err(host(g), oracle.lrn_backward(og, x, rden, size, alpha, beta)) <= 1e-5, what
     assert uncovered >= 10
+
+
+@pytest.mark.parametrize("seed", [31, 32])
+def test_gemm_and_lowering_random_shapes(oracle, seed):
+    """sgemm in every layout with ragged sizes, unaligned leading dimensions and the split over the
+    contraction (against float64); lowering, lifting (+ bias gradient) bit for bit against the oracle,
+    kernel sizes from 1 to 11, any stride and padding."""
+    from caffecontroll_amd.driver import conv_pmap, lift_args
+    RM, CM, N_, T_ = 101, 102, 111, 112
+    drv = driver()
+    rng = np.random.default_rng(seed)
+
+    def store(mat, trans, order, pad):
+        src = mat.T if trans == T_ else mat
+        if order == CM:
+            src = src.T
+        buf = np.full((src.shape[0], src.shape[1] + pad), np.nan, np.float32)
+        buf[:, :src.shape[1]] = src
+        return buf, src.shape[1] + pad
+
+    for case in range(40):
+        kind = rng.integers(0, 4)
+        if kind == 0:
+            M, N, K = (int(rng.integers(1, 300)) for _ in range(3))
+        elif kind == 1:
+            M, N, K = int(rng.integers(1, 64)), int(rng.integers(1, 64)), int(rng.integers(256, 6000))
+        elif kind == 2:
+            M, N, K = int(rng.integers(1, 40)) * 16, int(rng.integers(1, 40)) * 4, int(rng.integers(1, 30)) * 16
+        else:
+            M, N, K = int(rng.integers(64, 700)), int(rng.integers(64, 2000)), int(rng.integers(1, 130))
+        pad = int(rng.choice([0, 0, 1, 3, 4]))
+        TA, TB, order = int(rng.choice([N_, T_])), int(rng.choice([N_, T_])), int(rng.choice([RM, CM]))
+        alpha, beta = [(1.0, 0.0), (1.5, -0.5), (0.7, 1.0)][rng.integers(0, 3)]
+        opA = rng.standard_normal((M, K)).astype(np.float32)
+        opB = rng.standard_normal((K, N)).astype(np.float32)
+        C0 = rng.standard_normal((M, N)).astype(np.float32)
+        (A, lda), (B, ldb), (Cb, ldc) = store(opA, TA, order, pad), store(opB, TB, order, pad), store(C0, N_, order, pad)
+        dC = dev(np.full_like(Cb, np.nan) if beta == 0.0 else Cb)
+        drv.sgemm(order, TA, TB, M, N, K, alpha, dev(A), lda, dev(B), ldb, beta, dC, ldc)
+        out = host(dC)
+        got = out[:, :N] if order == RM else out[:, :M].T
+        what = (M, N, K, pad, TA, TB, order, alpha, beta)
+        assert rel_err(got, alpha * opA.astype(np.float64) @ opB.astype(np.float64) + beta * C0) <= TOL, what
+        assert not pad or np.isnan(out[:, -pad:]).all(), what
+
+        k, s = [(3, 1), (5, 1), (1, 1), (2, 2), (11, 4), (7, 2), (5, 2), (3, 2), (4, 3), (6, 1)][rng.integers(0, 10)]
+        p, b, d = int(rng.integers(0, k)), int(rng.integers(1, 8)), int(rng.integers(1, 30))
+        n = int(rng.integers(max(k - 2 * p, 1), 50))
+        m = (n + 2 * p - k) // s + 1
+        if n + 2 * p < k or b * m * m * k * k * d > 2e7:
+            continue
+        what = (b, d, n, k, s, p)
+        x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+        low = empty((b * m * m, k * k * d))
+        drv.lower_cube(low, dev(x), conv_pmap(b, d, n, k, s, p))
+        np.testing.assert_array_equal(host(low), oracle.lower_cube(x, k, s, p), err_msg=str(what))
+        y = rng.standard_normal((k * k * d, b * m * m)).astype(np.float32)
+        o = int(rng.integers(1, 40))
+        og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+        dx, db = empty((b, d, n, n)), empty((o,))
+        drv.inverse_lower_cube_bias_backward(dx, dev(y), lift_args(b, d, n, k, s, p), db, dev(og), m * m, o, b)
+        np.testing.assert_array_equal(host(dx), oracle.inverse_lower_cube(y, b, d, n, k, s, p), err_msg=str(what))
+        assert rel_err(host(db), og.astype(np.float64).sum(axis=(0, 2, 3))) <= TOL, what
