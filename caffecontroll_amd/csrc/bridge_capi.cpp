@@ -216,6 +216,20 @@ int cct_net_set_train(cct_net *h, int train) {
   return 0;
 }
 
+int cct_net_set_conv_path(cct_net *h, int level) {
+  if (!h) return CCT_HIP_EINVAL;
+  for (int i = 0; i < h->net->num_layers(); ++i) {
+    Network::Node &nd = h->net->node(i);
+    if (nd.spec.type != CCT_LAYER_CONV) continue;
+    for (auto *b : nd.bridges) {
+      auto *cb = static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(b)->sub_bridge();
+      if (level < 0) cb->set_fused(true);
+      else cb->set_path(level);
+    }
+  }
+  return 0;
+}
+
 int cct_net_freeze_dropout_masks(cct_net *h, int freeze) {
   if (!h) return CCT_HIP_EINVAL;
   for (int i = 0; i < h->net->num_layers(); ++i) {

@@ -122,6 +122,7 @@ NET_PROTOTYPES = {
     "cct_net_tensor": ([_P, _I, _I, _I, C.POINTER(C.c_size_t)], _P),
     "cct_net_set_train": ([_P, _I], _I),
     "cct_net_freeze_dropout_masks": ([_P, _I], _I),
+    "cct_net_set_conv_path": ([_P, _I], _I),
     "cct_net_forward": ([_P], _I),
     "cct_net_backward": ([_P], _I),
     "cct_net_loss": ([_P, C.POINTER(C.c_float)], _I),
@@ -198,6 +199,10 @@ class Net:
 
     def set_train(self, train):
         check(self.lib.cct_net_set_train(self.h, int(train)), "net_set_train")
+
+    def set_conv_path(self, level):
+        """Path level of every convolution layer: 0 staged .. 3 all direct (where covered), -1 default."""
+        check(self.lib.cct_net_set_conv_path(self.h, int(level)), "net_set_conv_path")
 
     def freeze_dropout_masks(self, freeze=True):
         check(self.lib.cct_net_freeze_dropout_masks(self.h, int(freeze)), "net_freeze_dropout_masks")

@@ -158,6 +158,11 @@ void *cct_net_tensor(cct_net *net, int layer, int group, int which, size_t *n);
 int cct_net_set_train(cct_net *net, int train);
 /* Keep the dropout masks as they are instead of drawing new ones (for parity tests). */
 int cct_net_freeze_dropout_masks(cct_net *net, int freeze);
+/* Path level of every convolution layer (0 staged passes .. 3 all direct, as cct_conv_layer_set_options;
+ * a layer falls back where the direct kernels do not cover its geometry, and a grouped layer, which
+ * works on channel slices, stays on the direct kernels).  -1 puts every layer back on its default.
+ * Without a counterpart in the reference: it is how tests run one network on every path. */
+int cct_net_set_conv_path(cct_net *net, int level);
 int cct_net_forward(cct_net *net);
 int cct_net_backward(cct_net *net);   /* gradients + SGD update of every layer */
 int cct_net_loss(cct_net *net, float *loss_sum); /* batch-summed loss of the last forward (syncs) */

@@ -172,3 +172,84 @@ def test_gemm_and_lowering_random_shapes(oracle, seed):
         drv.inverse_lower_cube_bias_backward(dx, dev(y), lift_args(b, d, n, k, s, p), db, dev(og), m * m, o, b)
         np.testing.assert_array_equal(host(dx), oracle.inverse_lower_cube(y, b, d, n, k, s, p), err_msg=str(what))
         assert rel_err(host(db), og.astype(np.float64).sum(axis=(0, 2, 3))) <= TOL, what
+
+
+def _random_chain(rng):
+    """A random layer chain: one to three convolutions (kernel sizes 1..11, strides, paddings, two
+    groups) with ReLU / pooling / LRN between them, up to two inner-product layers with ReLU and
+    dropout, a classifier and the loss."""
+    from caffecontroll_amd import nets
+    B, D, S = int(rng.integers(1, 9)), int(rng.choice([1, 2, 3, 4, 6])), int(rng.integers(12, 40))
+    layers, d, n = [], D, S
+    for _ in range(int(rng.integers(1, 4))):
+        k, s = [(3, 1), (5, 1), (3, 1), (3, 2), (5, 2), (7, 2), (1, 1), (4, 1), (11, 4)][rng.integers(0, 9)]
+        p = int(rng.integers(0, min(k, 3)))
+        m = (n + 2 * p - k) // s + 1 if n + 2 * p >= k else 0
+        if m < 2:
+            break
+        group = int(rng.choice([1, 1, 2])) if d % 2 == 0 else 1
+        o = int(rng.integers(1, 24)) * group
+        layers.append(nets.conv(o, k, stride=s, pad=p, group=group, lr_mult=(1.0, 2.0),
+                                decay_mult=(1.0, float(rng.integers(0, 2)))))
+        d, n = o, m
+        if rng.random() < 0.8:
+            layers.append(nets.relu())
+        if rng.random() < 0.6:
+            pk, ps = [(2, 2), (3, 2), (2, 1), (3, 3)][rng.integers(0, 4)]
+            if n >= pk:
+                layers.append(nets.maxpool(pk, ps))
+                n = (n - pk) // ps + 1
+        if rng.random() < 0.4:
+            layers.append(nets.lrn(int(rng.choice([3, 5])), 1e-2, 0.75))
+    for _ in range(int(rng.integers(0, 3))):
+        layers.append(nets.fc(int(rng.integers(2, 70)), decay_mult=(1.0, 1.0)))
+        if rng.random() < 0.8:
+            layers.append(nets.relu())
+        if rng.random() < 0.4:
+            layers.append(nets.dropout(0.5))
+    classes = int(rng.integers(2, 12))
+    layers += [nets.fc(classes), nets.softmax_loss()]
+    return B, D, S, classes, layers
+
+
+@pytest.mark.parametrize("seed", [41, 42])
+def test_random_layer_chains_train_like_the_oracle(oracle, seed):
+    """Two training iterations of random layer chains, the convolution layers on a random path level
+    (default, all direct, direct data gradient, staged passes): every layer's output, the loss, every
+    gradient and every updated parameter against the oracle chain."""
+    from caffecontroll_amd import nets
+    from oracle_net import OracleNet
+    import test_gpu_nets as T
+    driver()
+    rng = np.random.default_rng(seed)
+    solver = dict(base_lr=0.01, momentum=0.9, weight_decay=0.0005)
+    done = 0
+    while done < 25:
+        B, D, S, classes, layers = _random_chain(rng)
+        if not any(L.type == nets.CONV for L in layers):
+            continue
+        net = nets.Net(B, D, S, layers, nets.solver_param(**solver))
+        net.set_conv_path(int(rng.choice([-1, 3, 3, 2, 0])))
+        ref = OracleNet(oracle, layers, B, D, S, solver)
+        T._init_and_sync_params(net, ref, rng)
+        net.freeze_dropout_masks(True)
+        for li, L in enumerate(layers):
+            if L.type == nets.DROPOUT:
+                ptr, n = net.tensor(li, nets.AUX)
+                mask = rng.integers(0, 2**32, n, dtype=np.uint64).astype(np.uint32)
+                T._up(ptr, mask)
+                ref.masks[li] = mask
+        for _ in range(2):
+            x = rng.standard_normal((B, D, S, S)).astype(np.float32)
+            labels = rng.integers(0, classes, B).astype(np.float32)
+            T._up(net.input_ptr(), x)
+            T._up(net.labels_ptr(), labels)
+            net.forward()
+            ref.forward(x, labels)
+            T._check_forward_and_align_switches(net, ref, layers, TOL)
+            assert abs(net.loss() - ref.loss) <= TOL * max(1.0, abs(ref.loss))
+            net.backward()
+            ref.backward()
+            T._compare_params(net, ref, TOL)
+        net.close()
+        done += 1
