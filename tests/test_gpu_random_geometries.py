@@ -253,3 +253,78 @@ def test_random_layer_chains_train_like_the_oracle(oracle, seed):
             T._compare_params(net, ref, TOL)
         net.close()
         done += 1
+
+
+@pytest.mark.parametrize("seed", [51, 52])
+def test_random_tower_graphs_train_like_the_oracle(oracle, seed):
+    """Random graphs of the two-tower kind (a stem whose output two or three towers read -- the
+    reference's Split --, grouped and plain convolutions of kernel size 1, 3 and 5 in the towers,
+    CONCAT, classifier): one training iteration on a random convolution path level against the
+    oracle graph.  Weights are scaled by their fan-in so that the loss gradient is well conditioned."""
+    from caffecontroll_amd import nets
+    from oracle_net import OracleGraph
+    import test_gpu_nets as T
+    driver()
+    rng = np.random.default_rng(seed)
+    solver = dict(base_lr=0.05, momentum=0.9, weight_decay=0.001)
+
+    def same_conv(o, group=1):
+        k = int(rng.choice([1, 3, 5]))
+        return nets.conv(o, k, pad=(k - 1) // 2, group=group)
+
+    for case in range(20):
+        B, D, S = int(rng.integers(1, 7)), int(rng.choice([1, 2, 3, 4])), int(rng.integers(8, 20))
+        layers = [same_conv(int(rng.integers(1, 8)) * 2)]
+        if rng.random() < 0.7:
+            layers.append(nets.relu())
+        if rng.random() < 0.5:
+            layers.append(nets.maxpool(2, 2))
+        if rng.random() < 0.4:
+            layers.append(nets.lrn(3, 1e-2, 0.75))
+        shared, ends, pool_towers = len(layers) - 1, [], rng.random() < 0.5
+        for _ in range(int(rng.integers(2, 4))):
+            g = int(rng.choice([1, 2]))
+            layers.append(same_conv(int(rng.integers(2, 8)) * g + (g == 1), g).read_from(shared))
+            if rng.random() < 0.7:
+                layers.append(nets.relu())
+            if rng.random() < 0.4:
+                layers.append(same_conv(int(rng.integers(3, 10))))
+                if rng.random() < 0.5:
+                    layers.append(nets.relu())
+            if pool_towers:
+                layers.append(nets.maxpool(2, 2))
+            ends.append(len(layers) - 1)
+        layers.append(nets.concat(*ends))
+        if rng.random() < 0.5:
+            layers += [nets.fc(int(rng.integers(2, 40))), nets.relu()]
+        classes = int(rng.integers(2, 8))
+        layers += [nets.fc(classes), nets.softmax_loss()]
+        net = nets.Net(B, D, S, layers, nets.solver_param(**solver))
+        net.set_conv_path(int(rng.choice([-1, 3, 0])))
+        ref = OracleGraph(oracle, layers, B, D, S, solver)
+        T._init_and_sync_params(net, ref, rng)
+        x = rng.standard_normal((B, D, S, S)).astype(np.float32)
+        labels = rng.integers(0, classes, B).astype(np.float32)
+        T._up(net.input_ptr(), x)
+        T._up(net.labels_ptr(), labels)
+        net.forward()
+        ref.forward(x, labels)
+        for li, L in enumerate(layers):
+            if L.type == nets.RELU:
+                continue
+            ptr, n = net.tensor(li, nets.OUTPUT)
+            want = ref.val[ref.blob[li]] if li != len(layers) - 1 else ref.out[li]
+            assert rel_err(T._down(ptr, n), want.reshape(-1)) <= TOL, (case, li)
+            if L.type == nets.MAXPOOL:   # route the gradients through the oracle's arg-max positions
+                ptr, n = net.tensor(li, nets.AUX)
+                T._up(ptr, ref.saved[(li, "idx")].reshape(-1).astype(np.int32))
+        assert abs(net.loss() - ref.loss) <= TOL * max(1.0, abs(ref.loss))
+        net.backward()
+        ref.backward()
+        for (li, gi), p in sorted(ref.params.items()):
+            for which, k, key, hist in ((nets.MODEL_GRAD, 0, "w", "hw"), (nets.BIAS_GRAD, 1, "b", "hb")):
+                ptr, n = net.tensor(li, which, gi)
+                lam = np.float32(solver["weight_decay"] * layers[li].decay_mult[k])
+                want = ref.grads[(li, gi)][k].reshape(-1) + lam * (p[key].reshape(-1) + p[hist])
+                assert rel_err(T._down(ptr, n), want) <= TOL, (case, li, gi, k)
+        net.close()
