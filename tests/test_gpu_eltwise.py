@@ -203,11 +203,11 @@ def test_sgd_and_blas1(oracle):
 
 
 def test_sgd_batch_matches_single_updates(oracle):
-    """Several tensors in one launch (more than one table of 16, sizes around the 2048-element
+    """Several tensors in one launch (more than one table of 16, sizes around the 512-element
     chunks, an empty one, every regulariser): the bits of the oracle's update for each."""
     drv = driver()
     rng = np.random.default_rng(77)
-    sizes = [1, 10, 256, 2047, 2048, 2049, 0, 4097, 500, 20, 50, 96, 384, 4096, 1000, 34848, 25000, 307200, 7, 800]
+    sizes = [1, 10, 256, 511, 512, 513, 2047, 2048, 2049, 0, 4097, 500, 20, 50, 96, 384, 4096, 1000, 34848, 25000, 307200, 7, 800]
     jobs, refs, devs = [], [], []
     for t, n in enumerate(sizes):
         w, g, h = (rng.standard_normal(n).astype(np.float32) for _ in range(3))
