@@ -817,14 +817,23 @@ __global__ __launch_bounds__(TPB) void softmax_fwd_kernel(float *__restrict__ pr
     loss_per_image[ib] = valid ? -logf(fmaxf(y[(int)lf], FLT_MIN)) : __int_as_float(0x7fc00000);
   }
 }
-// batch sum in ascending image order (the order the reference accumulates its scalar loss)
-__global__ void softmax_loss_sum_kernel(float *__restrict__ loss_sum, const float *__restrict__ per_image,
-                                        int batch) {
-  if (threadIdx.x == 0 && blockIdx.x == 0) {
-    float s = 0.0f;
-    for (int i = 0; i < batch; ++i) s += per_image[i];
-    *loss_sum = s;
+// batch sum in ascending image order (the order the reference accumulates its scalar loss): the
+// workgroup fetches the per-image losses TPB at a time, coalesced, and lane 0 adds them up in order
+__global__ __launch_bounds__(TPB) void softmax_loss_sum_kernel(float *__restrict__ loss_sum,
+                                                               const float *__restrict__ per_image, int batch) {
+  __shared__ float part[TPB];
+  float s = 0.0f;
+  for (int base = 0; base < batch; base += TPB) {
+    const int i = base + (int)threadIdx.x;
+    part[threadIdx.x] = i < batch ? per_image[i] : 0.0f;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const int n = min(TPB, batch - base);
+      for (int j = 0; j < n; ++j) s += part[j];
+    }
+    __syncthreads();
   }
+  if (threadIdx.x == 0) *loss_sum = s;
 }
 __global__ __launch_bounds__(TPB) void softmax_bwd_kernel(float *__restrict__ ig, const float *__restrict__ prob,
                                                           const float *__restrict__ labels, int len,
@@ -1303,7 +1312,7 @@ int cct_hip_softmax_loss_forward(float *prob, const float *in, const float *labe
                        (float *)ws, len_per_image);
     CCT_LAUNCH_CHECK();
   }
-  hipLaunchKernelGGL(softmax_loss_sum_kernel, dim3(1), dim3(64), 0, ctx().stream, loss_sum, (const float *)ws,
+  hipLaunchKernelGGL(softmax_loss_sum_kernel, dim3(1), dim3(TPB), 0, ctx().stream, loss_sum, (const float *)ws,
                      batch);
   CCT_LAUNCH_CHECK();
   return 0;
