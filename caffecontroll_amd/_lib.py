@@ -89,6 +89,12 @@ PROTOTYPES = {
     "cct_hip_conv_direct_backward_data": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z],
     "cct_hip_conv_direct_backward_data_relu": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z, _P],
     "cct_hip_conv_direct_backward_weights": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z],
+    "cct_hip_conv_direct_supported_grouped": [_I, _I, _I, _I, _I, _I, _I, _I],
+    "cct_hip_conv_direct_slab_floats_grouped": [_I, _I, _I, _I, _I],
+    "cct_hip_conv_direct_slabs_grouped": [_P, _P, _I, _I, _I, _I, _I],
+    "cct_hip_conv_direct_forward_grouped": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z, _I, _I],
+    "cct_hip_conv_direct_backward_data_grouped": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z, _P, _I],
+    "cct_hip_conv_direct_backward_weights_grouped": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _Z, _Z, _I],
     "cct_hip_conv_strided_supported": [_I, _I, _I, _I, _I, _I, _I],
     "cct_hip_conv_strided_slab_floats": [_I, _I, _I, _I, _I],
     "cct_hip_conv_strided_slabs": [_P, _P, _I, _I, _I, _I, _I],
@@ -135,6 +141,7 @@ PROTOTYPES = {
     "cct_hip_timer_elapsed_ms": [_P, C.POINTER(_F)],
 }
 _RESTYPE = {"cct_hip_last_error": C.c_char_p, "cct_hip_last_kernel": C.c_char_p, "cct_hip_conv_direct_slab_floats": C.c_size_t,
+            "cct_hip_conv_direct_slab_floats_grouped": C.c_size_t,
             "cct_hip_conv_strided_slab_floats": C.c_size_t,
             "cct_hip_conv_strided_backward_data_slab_floats": C.c_size_t}
 

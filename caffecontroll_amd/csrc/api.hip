@@ -29,13 +29,15 @@ static void read_tuning_from_env() {
   g_tuning.direct_waves = geti("CCT_HIP_DIRECT_WAVES", 0);
   g_tuning.direct_tb = geti("CCT_HIP_DIRECT_TB", 0);
   g_tuning.direct_nospec = geti("CCT_HIP_DIRECT_NOSPEC", 0);
+  g_tuning.direct_splits = geti("CCT_HIP_DIRECT_SPLITS", 0);
   g_tuning.pool_plane = geti("CCT_HIP_POOL_PLANE", 0);
   g_tuning.gemm_nt = geti("CCT_HIP_GEMM_NT", 0);
   g_tuning.gemm_tile = geti("CCT_HIP_GEMM_TILE", -1);
   g_tuning.gemm_nodma = geti("CCT_HIP_GEMM_NODMA", 0);
 }
 
-static char g_last_kernel[192] = "";
+// per host thread, like the error text: a launch on one thread never rewrites what another thread reads
+static thread_local char g_last_kernel[192] = "";
 
 void note_kernel(const char *fmt, ...) {
   va_list ap;
@@ -51,6 +53,7 @@ void mark_counters_dirty() {
 
 int grant_dynamic_lds(const void *kernel, size_t bytes, LdsGrant &st) {
   if (bytes <= 64 * 1024) return 0;
+  std::lock_guard<std::mutex> lk(g_mu);  // `st` is shared by every host thread that launches this instance
   if (st.device == g_ctx.device && st.bytes >= bytes) return 0;
   CCT_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
   st.device = g_ctx.device;
@@ -161,7 +164,7 @@ int cct_hip_set_tuning(const char *name, int value) {
   Tuning &t = tuning();
   struct { const char *name; int *field; } const table[] = {
       {"direct_tile", &t.direct_tile}, {"direct_waves", &t.direct_waves}, {"direct_tb", &t.direct_tb},
-      {"direct_nospec", &t.direct_nospec}, {"pool_plane", &t.pool_plane}, {"gemm_nt", &t.gemm_nt},
+      {"direct_nospec", &t.direct_nospec}, {"direct_splits", &t.direct_splits}, {"pool_plane", &t.pool_plane}, {"gemm_nt", &t.gemm_nt},
       {"gemm_tile", &t.gemm_tile}, {"gemm_nodma", &t.gemm_nodma}};
   for (const auto &e : table)
     if (!strcmp(e.name, name)) {
@@ -247,7 +250,12 @@ int cct_filler_draw_bernoulli(float *host, size_t n, float p, int random_seed) {
 
 int cct_filler_draw_gaussian(float *host, size_t n, float mean, float std_dev, int random_seed) {
   CCT_REQUIRE(host || n == 0, "filler_draw_gaussian: null array");
-  CCT_REQUIRE(std_dev > 0.0f, "filler_draw_gaussian: std must be positive");
+  CCT_REQUIRE(std_dev >= 0.0f && std::isfinite(std_dev) && std::isfinite(mean),
+              "filler_draw_gaussian: std must be finite and not negative");
+  if (std_dev == 0.0f) {  // what the reference's normal_distribution(mean, 0) yields: the mean everywhere
+    for (size_t i = 0; i < n; ++i) host[i] = mean;
+    return 0;
+  }
   std::mt19937 gen(filler_seed(random_seed));
   std::normal_distribution<float> gaussian(mean, std_dev);
   for (size_t i = 0; i < n; ++i) host[i] = gaussian(gen);

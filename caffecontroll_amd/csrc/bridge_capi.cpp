@@ -1,6 +1,7 @@
 // C entry points over the C++ host layer (see include/cct_bridge.h).
 #include <cmath>
 #include <exception>
+#include <memory>
 #include <string>
 
 #include "../../include/cct_bridge.h"
@@ -22,6 +23,21 @@ void fill_solver(cnn::SolverParameter &s, const cct_solver_param *p) {
   if (p->regularization_type) s.regularization_type_ = p->regularization_type;
 }
 
+// Runs `body` with the host layer's failures turned into exceptions (Fail.h) and returns what it returns, or
+// the error code with the message in cct_hip_last_error() if it throws: no failure inside a bridge ends
+// the caller's process or crosses the C boundary as an exception.
+template <typename F>
+int guarded(const char *what, F body) {
+  ErrorsAsExceptions scope;
+  try {
+    return body();
+  } catch (const std::exception &e) {
+    return cct::set_error(CCT_HIP_EINVAL, "%s: %s", what, e.what());
+  } catch (...) {
+    return cct::set_error(CCT_HIP_EINVAL, "%s: unknown failure", what);
+  }
+}
+
 }  // namespace
 
 struct cct_conv_bridge {
@@ -30,6 +46,11 @@ struct cct_conv_bridge {
   cnn::SolverParameter solver_param;
   Layer<float> *in_layer = nullptr, *out_layer = nullptr;
   ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *pbridge = nullptr;
+  ~cct_conv_bridge() {
+    delete pbridge;
+    delete in_layer;
+    delete out_layer;
+  }
 };
 
 extern "C" {
@@ -49,41 +70,42 @@ int cct_conv_bridge_create_shared(cct_conv_bridge **out, int b, int d, int n, co
     return cct::set_error(CCT_HIP_EINVAL, "conv_bridge_create: bad geometry or null tensor");
   if ((!share_pointer_with_prev_bridge && !in_grad) || (!share_pointer_with_next_bridge && !out_grad))
     return cct::set_error(CCT_HIP_EINVAL, "conv_bridge_create: a host-resident layer needs both of its cubes");
-  cct_conv_bridge *h = new cct_conv_bridge;
-  const int k = conv->kernel_size, s = conv->stride, p = conv->pad, o = conv->num_output;
-  const int m = (n + 2 * p - k) / s + 1;
-  cnn::ConvolutionParameter &cp = h->layer_param.convolution_param_;
-  cp.num_output_ = o; cp.kernel_size_ = k; cp.stride_ = s; cp.pad_ = p; cp.bias_term_ = conv->bias_term != 0;
-  h->layer_param.blobs_lr_[0] = conv->lr_mult_weights; h->layer_param.blobs_lr_[1] = conv->lr_mult_bias;
-  h->layer_param.weight_decay_[0] = conv->decay_mult_weights; h->layer_param.weight_decay_[1] = conv->decay_mult_bias;
-  fill_solver(h->solver_param, solver);
-  h->in_layer = new Layer<float>(new LogicalCube<float>(in_data, n, n, d, b),
-                                 new LogicalCube<float>(in_grad, n, n, d, b));
-  h->out_layer = new Layer<float>(new LogicalCube<float>(out_data, m, m, o, b),
-                                  new LogicalCube<float>(out_grad, m, m, o, b));
-  h->pbridge = new ParallelizedBridge<float, ConvolutionBridge, HIPDriver>(
-      h->in_layer, h->out_layer, &h->layer_param, &h->solver_param, &h->driver, 1, 1,
-      share_pointer_with_prev_bridge != 0, share_pointer_with_next_bridge != 0, false);
-  *out = h;
-  return 0;
+  *out = nullptr;
+  return guarded("conv_bridge_create", [&] {
+    std::unique_ptr<cct_conv_bridge> h(new cct_conv_bridge);  // its destructor frees what was built if a step throws
+    const int k = conv->kernel_size, s = conv->stride, p = conv->pad, o = conv->num_output;
+    const int m = (n + 2 * p - k) / s + 1;
+    cnn::ConvolutionParameter &cp = h->layer_param.convolution_param_;
+    cp.num_output_ = o; cp.kernel_size_ = k; cp.stride_ = s; cp.pad_ = p; cp.bias_term_ = conv->bias_term != 0;
+    h->layer_param.blobs_lr_[0] = conv->lr_mult_weights; h->layer_param.blobs_lr_[1] = conv->lr_mult_bias;
+    h->layer_param.weight_decay_[0] = conv->decay_mult_weights; h->layer_param.weight_decay_[1] = conv->decay_mult_bias;
+    fill_solver(h->solver_param, solver);
+    h->in_layer = new Layer<float>(new LogicalCube<float>(in_data, n, n, d, b),
+                                   new LogicalCube<float>(in_grad, n, n, d, b));
+    h->out_layer = new Layer<float>(new LogicalCube<float>(out_data, m, m, o, b),
+                                    new LogicalCube<float>(out_grad, m, m, o, b));
+    h->pbridge = new ParallelizedBridge<float, ConvolutionBridge, HIPDriver>(
+        h->in_layer, h->out_layer, &h->layer_param, &h->solver_param, &h->driver, 1, 1,
+        share_pointer_with_prev_bridge != 0, share_pointer_with_next_bridge != 0, false);
+    *out = h.release();
+    return 0;
+  });
 }
 
 int cct_conv_bridge_destroy(cct_conv_bridge *h) {
-  if (!h) return 0;
-  delete h->pbridge;
-  delete h->in_layer;
-  delete h->out_layer;
   delete h;
   return 0;
 }
 
 int cct_conv_bridge_set_options(cct_conv_bridge *h, int fused, int profile, int needs_backward_grad) {
   if (!h) return CCT_HIP_EINVAL;
-  if (fused >= 0) h->pbridge->sub_bridge()->set_path(fused);
-  h->pbridge->sub_bridge()->set_stage_profiling(profile != 0);
-  h->pbridge->needs_to_calc_backward_grad = needs_backward_grad != 0;
-  h->pbridge->sub_bridge()->needs_to_calc_backward_grad = needs_backward_grad != 0;
-  return 0;
+  return guarded("conv_bridge_set_options", [&] {
+    if (fused >= 0) h->pbridge->sub_bridge()->set_path(fused);
+    h->pbridge->sub_bridge()->set_stage_profiling(profile != 0);
+    h->pbridge->needs_to_calc_backward_grad = needs_backward_grad != 0;
+    h->pbridge->sub_bridge()->needs_to_calc_backward_grad = needs_backward_grad != 0;
+    return 0;
+  });
 }
 
 int cct_conv_bridge_path(cct_conv_bridge *h) { return h ? h->pbridge->sub_bridge()->path() : -1; }
@@ -97,7 +119,12 @@ float *cct_conv_bridge_bias_grad(cct_conv_bridge *h) {
   return h->pbridge->p_bias_grad ? h->pbridge->p_bias_grad->get_p_data() : nullptr;
 }
 float *cct_conv_bridge_lowered(cct_conv_bridge *h) {
-  return h->pbridge->sub_bridge()->get_lowered_cube()->get_p_data();
+  float *p = nullptr;  // the lowered cube is allocated on first use: NULL (and the error text) if that fails
+  guarded("conv_bridge_lowered", [&] {
+    p = h->pbridge->sub_bridge()->get_lowered_cube()->get_p_data();
+    return 0;
+  });
+  return p;
 }
 float *cct_conv_bridge_history(cct_conv_bridge *h) {
   return h->pbridge->get_grad_updater()->get_p_history_updates_cube()->get_p_data();
@@ -105,19 +132,23 @@ float *cct_conv_bridge_history(cct_conv_bridge *h) {
 
 int cct_conv_bridge_forward(cct_conv_bridge *h) {
   if (!h) return CCT_HIP_EINVAL;
-  h->pbridge->forward();
-  return 0;
+  return guarded("conv_bridge_forward", [&] {
+    h->pbridge->forward();
+    return 0;
+  });
 }
 
 int cct_conv_bridge_backward(cct_conv_bridge *h, int with_update) {
   if (!h) return CCT_HIP_EINVAL;
-  if (with_update) {
-    h->pbridge->backward();
-  } else {
-    h->pbridge->sub_bridge()->needs_to_calc_backward_grad = h->pbridge->needs_to_calc_backward_grad;
-    h->pbridge->sub_bridge()->backward();
-  }
-  return 0;
+  return guarded("conv_bridge_backward", [&] {
+    if (with_update) {
+      h->pbridge->backward();
+    } else {
+      h->pbridge->sub_bridge()->needs_to_calc_backward_grad = h->pbridge->needs_to_calc_backward_grad;
+      h->pbridge->sub_bridge()->backward();
+    }
+    return 0;
+  });
 }
 
 int cct_conv_bridge_stage_ms(cct_conv_bridge *h, float ms[CCT_CONV_STAGE_COUNT]) {
@@ -148,15 +179,13 @@ int cct_net_create(cct_net **out, int batch, int depth, int size, const cct_laye
   *out = nullptr;
   int rc = cct_net_validate(batch, depth, size, layers, n_layers, solver);
   if (rc) return rc;
-  try {
+  return guarded("net_create", [&] {
     Network *net = new Network(batch, depth, size, layers, n_layers, solver);
     cct_net *h = new cct_net;
     h->net = net;
     *out = h;
-  } catch (const std::exception &e) {
-    return cct::set_error(CCT_HIP_EINVAL, "net_create: %s", e.what());
-  }
-  return 0;
+    return 0;
+  });
 }
 
 int cct_net_destroy(cct_net *h) {
@@ -180,8 +209,12 @@ void *cct_net_tensor(cct_net *h, int layer, int group, int which, size_t *n) {
     if (n) *n = c->n_elements;
     return c->get_p_data();
   }
-  if (group < 0 || group >= (int)nd.bridges.size()) return nullptr;
-  Network::BridgeT *b = nd.bridges[group];
+  // a grouped convolution run by one bridge: `group` selects that group's slice of the layer's model,
+  // bias, gradients and momentum buffers ([o][d/g][k][k] and [o]: the groups lie one after another)
+  const int layer_groups = nd.spec.type == CCT_LAYER_CONV && nd.spec.group > 1 ? nd.spec.group : 1;
+  const bool sliced = layer_groups > 1 && nd.bridges.size() == 1 && which != 6;
+  if (group < 0 || group >= (sliced ? layer_groups : (int)nd.bridges.size())) return nullptr;
+  Network::BridgeT *b = nd.bridges[sliced ? 0 : group];
   switch (which) {
     case 0: c = b->get_model_cube(); break;
     case 1: c = b->get_bias_cube(); break;
@@ -206,6 +239,11 @@ void *cct_net_tensor(cct_net *h, int layer, int group, int which, size_t *n) {
     default: return nullptr;
   }
   if (!c) return nullptr;
+  if (sliced) {
+    const size_t per_group = c->n_elements / layer_groups;
+    if (n) *n = per_group;
+    return c->get_p_data() + (size_t)group * per_group;
+  }
   if (n) *n = c->n_elements;
   return c->get_p_data();
 }
@@ -218,16 +256,18 @@ int cct_net_set_train(cct_net *h, int train) {
 
 int cct_net_set_conv_path(cct_net *h, int level) {
   if (!h) return CCT_HIP_EINVAL;
-  for (int i = 0; i < h->net->num_layers(); ++i) {
-    Network::Node &nd = h->net->node(i);
-    if (nd.spec.type != CCT_LAYER_CONV) continue;
-    for (auto *b : nd.bridges) {
-      auto *cb = static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(b)->sub_bridge();
-      if (level < 0) cb->set_fused(true);
-      else cb->set_path(level);
+  return guarded("net_set_conv_path", [&] {
+    for (int i = 0; i < h->net->num_layers(); ++i) {
+      Network::Node &nd = h->net->node(i);
+      if (nd.spec.type != CCT_LAYER_CONV) continue;
+      for (auto *b : nd.bridges) {
+        auto *cb = static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(b)->sub_bridge();
+        if (level < 0) cb->set_fused(true);
+        else cb->set_path(level);
+      }
     }
-  }
-  return 0;
+    return 0;
+  });
 }
 
 int cct_net_freeze_dropout_masks(cct_net *h, int freeze) {
@@ -242,20 +282,75 @@ int cct_net_freeze_dropout_masks(cct_net *h, int freeze) {
 
 int cct_net_forward(cct_net *h) {
   if (!h) return CCT_HIP_EINVAL;
-  h->net->forward();
-  return 0;
+  return guarded("net_forward", [&] {
+    h->net->forward();
+    return 0;
+  });
 }
 
 int cct_net_backward(cct_net *h) {
   if (!h) return CCT_HIP_EINVAL;
-  h->net->backward();
-  return 0;
+  return guarded("net_backward", [&] {
+    h->net->backward();
+    return 0;
+  });
 }
 
 int cct_net_loss(cct_net *h, float *loss_sum) {
   if (!h || !loss_sum) return CCT_HIP_EINVAL;
-  *loss_sum = h->net->loss();
+  return guarded("net_loss", [&] {
+    *loss_sum = h->net->loss();
+    return 0;
+  });
+}
+
+int cct_net_set_profiling(cct_net *h, int on) {
+  if (!h) return CCT_HIP_EINVAL;
+  return guarded("net_set_profiling", [&] {
+    h->net->set_profiling(on != 0);
+    return 0;
+  });
+}
+
+int cct_net_layer_ms(cct_net *h, int layer, float *forward_ms, float *backward_ms) {
+  if (!h || layer < 0 || layer >= h->net->num_layers()) return CCT_HIP_EINVAL;
+  if (forward_ms) *forward_ms = h->net->layer_ms(layer, false);
+  if (backward_ms) *backward_ms = h->net->layer_ms(layer, true);
   return 0;
+}
+
+int cct_net_update_ms(cct_net *h, float *ms) {
+  if (!h || !ms) return CCT_HIP_EINVAL;
+  *ms = h->net->update_ms();
+  return 0;
+}
+
+namespace {
+ConvolutionBridge<float, HIPDriver> *conv_of(cct_net *h, int layer, int bridge) {
+  if (!h || layer < 0 || layer >= h->net->num_layers()) return nullptr;
+  Network::Node &nd = h->net->node(layer);
+  if (nd.spec.type != CCT_LAYER_CONV || bridge < 0 || bridge >= (int)nd.bridges.size()) return nullptr;
+  return static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(nd.bridges[bridge])->sub_bridge();
+}
+}  // namespace
+
+int cct_net_conv_bridges(cct_net *h, int layer) {
+  if (!h || layer < 0 || layer >= h->net->num_layers()) return 0;
+  Network::Node &nd = h->net->node(layer);
+  return nd.spec.type == CCT_LAYER_CONV ? (int)nd.bridges.size() : 0;
+}
+
+int cct_net_conv_stage_ms(cct_net *h, int layer, int bridge, float ms[CCT_CONV_STAGE_COUNT]) {
+  auto *cb = conv_of(h, layer, bridge);
+  if (!cb || !ms) return CCT_HIP_EINVAL;
+  for (int i = 0; i < STAGE_COUNT; ++i) ms[i] = cb->stage_ms(i);
+  return 0;
+}
+
+const char *cct_net_conv_stage_kernel(cct_net *h, int layer, int bridge, int stage) {
+  auto *cb = conv_of(h, layer, bridge);
+  if (!cb || stage < 0 || stage >= STAGE_COUNT) return "";
+  return cb->stage_kernel(stage).c_str();
 }
 
 namespace {
@@ -266,28 +361,30 @@ int io_result(cct_net *h, bool ok) {
 
 int cct_net_write_model(cct_net *h, const char *file) {
   if (!h || !file) return CCT_HIP_EINVAL;
-  return io_result(h, h->net->write_blobs(file, Network::BLOB_MODEL));
+  return guarded("net_write_model", [&] { return io_result(h, h->net->write_blobs(file, Network::BLOB_MODEL)); });
 }
 
 int cct_net_read_model(cct_net *h, const char *file) {
   if (!h || !file) return CCT_HIP_EINVAL;
-  return io_result(h, h->net->read_blobs(file, Network::BLOB_MODEL));
+  return guarded("net_read_model", [&] { return io_result(h, h->net->read_blobs(file, Network::BLOB_MODEL)); });
 }
 
 int cct_net_write_snapshot(cct_net *h, const char *base_filename, int iter) {
   if (!h || !base_filename || iter < 0) return CCT_HIP_EINVAL;
-  return io_result(h, h->net->write_snapshot(base_filename, iter));
+  return guarded("net_write_snapshot", [&] { return io_result(h, h->net->write_snapshot(base_filename, iter)); });
 }
 
 int cct_net_read_snapshot(cct_net *h, const char *stem, int *iter) {
   if (!h || !stem) return CCT_HIP_EINVAL;
-  return io_result(h, h->net->read_snapshot(stem, iter));
+  return guarded("net_read_snapshot", [&] { return io_result(h, h->net->read_snapshot(stem, iter)); });
 }
 
 int cct_net_set_iter(cct_net *h, int iter) {
   if (!h || iter < 0) return CCT_HIP_EINVAL;
-  h->net->set_current_iter(iter);
-  return 0;
+  return guarded("net_set_iter", [&] {
+    h->net->set_current_iter(iter);
+    return 0;
+  });
 }
 
 int cct_net_get_iter(cct_net *h) { return h ? h->net->current_iter() : -1; }

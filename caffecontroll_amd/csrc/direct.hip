@@ -56,6 +56,10 @@ struct DirectArgs {
   // phase) triples of the layer's input gradient, pixel (I, J) of map (c, pi, pj) is stored at
   // dst[img][c][S*I + pi - spad][S*J + pj - spad] of a [batch][sd][shs][shs] tensor (ss = S; 0 = plain output)
   int ss, shs, spad, sd;
+  // channel groups of a grouped convolution, all in this launch: group q reads channels q*kc .. of src and
+  // writes maps q*mtot .. of dst with the slab buffer at wt + q*wt_group_floats; tile ids run group by group
+  int groups;
+  uint32_t tiles_per_group, wt_group_floats;
 };
 
 constexpr int kDirect16PatchLoads = 10;  // the 16-row kernel stages four channels per step
@@ -91,7 +95,9 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
   const int psz = (NC * g.pr * PW + 63) & ~63;  // floats of patches per stage: whole 64-lane loads
   const int stage = ASZP + psz;
 
-  const uint32_t id = xcd_remap(blockIdx.x, g.ntiles);
+  uint32_t id = xcd_remap(blockIdx.x, g.ntiles);
+  const uint32_t grp = g.groups > 1 ? id / g.tiles_per_group : 0u;  // workgroup-uniform
+  id -= grp * g.tiles_per_group;
   const uint32_t tn = id / g.tiles_m, tm = id - tn * g.tiles_m;
   const int m0 = tm * BM;
   const uint32_t p0 = tn * BN;
@@ -135,7 +141,8 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     psrc_last[i] = (ok && (int)c < last_channels) ? psrc[i] : kOutOfRange;
   }
   const uint32_t a_step = (uint32_t)NC * g.slab_stride * 4u, b_step = (uint32_t)NC * g.hs * g.hs * 4u;  // bytes
-  const rsrc_t a_rsrc = make_rsrc(g.wt + (size_t)m0 * KK), b_rsrc = make_rsrc(g.src);
+  const rsrc_t a_rsrc = make_rsrc(g.wt + (size_t)grp * g.wt_group_floats + (size_t)m0 * KK),
+               b_rsrc = make_rsrc(g.src + (size_t)grp * g.kc * g.hs * g.hs);
   const int wave_elem0 = wave * 64;  // first element of this wave within a 256-element pass
 
 // global -> LDS stage s for step t (asynchronous; completion = vmcnt)
@@ -235,15 +242,16 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     const uint32_t p = p0 + wave * (32 * TNB) + b * 32 + r;
     if (p >= g.ptot) continue;
     const uint32_t img = fdiv(p, g.div_ho2);
-    const size_t pix = (size_t)img * g.dst_img_stride + (p - img * ho2);
+    const size_t pix = (size_t)img * g.dst_img_stride + (size_t)grp * g.mtot * ho2 + (p - img * ho2);
     float *out = g.dst + pix;
+    const float *gbias = g.bias ? g.bias + (size_t)grp * g.mtot : nullptr;
 #pragma unroll
     for (int a = 0; a < TMB; ++a)
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
         const int row = m0 + a * 32 + 8 * (v / 4) + 4 * h + (v % 4);
         if (row < g.mtot) {
-          float y = acc[a][b][v] + (g.bias ? g.bias[row] : 0.f);
+          float y = acc[a][b][v] + (gbias ? gbias[row] : 0.f);
           if (g.mask && !(g.mask[pix + (size_t)row * ho2] > 0.f)) y = 0.f;
           out[(size_t)row * ho2] = (g.relu && !(y > 0.f)) ? 0.f : y;
         }
@@ -291,7 +299,9 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
   const int psz = (NC * g.cs + 63) & ~63;
   const int stage = ASZP + psz;
 
-  const uint32_t tn = xcd_remap(blockIdx.x, g.ntiles);  // one map tile: the tile id is the pixel tile
+  uint32_t tn = xcd_remap(blockIdx.x, g.ntiles);  // one map tile: the tile id is (group, pixel tile)
+  const uint32_t grp = g.groups > 1 ? tn / g.tiles_per_group : 0u;  // workgroup-uniform
+  tn -= grp * g.tiles_per_group;
   const uint32_t p0 = tn * BN;
   const int ho2 = g.ho * g.ho;
   const uint32_t img0 = fdiv(p0, g.div_ho2);
@@ -321,7 +331,8 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
     psrc_last[i] = (ok && (int)c < last_channels) ? psrc[i] : kOutOfRange;
   }
   const uint32_t a_step = (uint32_t)NC * g.slab_stride * 4u, b_step = (uint32_t)NC * g.hs * g.hs * 4u;
-  const rsrc_t a_rsrc = make_rsrc(g.wt), b_rsrc = make_rsrc(g.src);
+  const rsrc_t a_rsrc = make_rsrc(g.wt + (size_t)grp * g.wt_group_floats),
+               b_rsrc = make_rsrc(g.src + (size_t)grp * g.kc * g.hs * g.hs);
   const int wave_elem0 = wave * 64;
 
 #define CCT_DIRECT16_ISSUE(t, s)                                                               \
@@ -452,15 +463,16 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
     const uint32_t p = p0 + wave * (32 * TNB) + b * 16 + r;
     if (p >= g.ptot) continue;
     const uint32_t img = fdiv(p, g.div_ho2);
-    const size_t pix = (size_t)img * g.dst_img_stride + (p - img * ho2);
+    const size_t pix = (size_t)img * g.dst_img_stride + (size_t)grp * g.mtot * ho2 + (p - img * ho2);
     float *out = g.dst + pix;
+    const float *gbias = g.bias ? g.bias + (size_t)grp * g.mtot : nullptr;
 #pragma unroll
     for (int a = 0; a < TM16; ++a)
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int row = a * 16 + 4 * q + v;
         if (row < g.mtot) {
-          float y = acc[a][b][v] + (g.bias ? g.bias[row] : 0.f);
+          float y = acc[a][b][v] + (gbias ? gbias[row] : 0.f);
           if (g.mask && !(g.mask[pix + (size_t)row * ho2] > 0.f)) y = 0.f;
           out[(size_t)row * ho2] = (g.relu && !(y > 0.f)) ? 0.f : y;
         }
@@ -493,6 +505,9 @@ __global__ __launch_bounds__(256) void direct_slab_kernel(float *__restrict__ wt
                                                           int reversed, FastDiv div_kk, FastDiv div_m) {
   const uint32_t e = blockIdx.x * 256 + threadIdx.x;
   if (e >= total) return;
+  // blockIdx.y = channel group: its own [n_m or n_c][..][kk] block of the model, its own slab buffer
+  wt += (size_t)blockIdx.y * total;
+  w += (size_t)blockIdx.y * n_c * n_m * kk;
   const uint32_t cm = fdiv(e, div_kk), j = e - cm * kk;
   const uint32_t c = fdiv(cm, div_m), m = cm - c * p_m;
   float v = 0.f;
@@ -515,16 +530,16 @@ static int direct_tm16(int mtot) {
 }
 
 // Chooses the kernel instance for a geometry; returns false when the direct path does not cover it.
-static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, DirectPlan *pl) {
+static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, DirectPlan *pl, int groups = 1) {
   if (ks != 3 && ks != 5) return false;
-  if (pad < 0 || pad > ks - 1 || batch <= 0 || kc <= 0 || mtot <= 0) return false;
+  if (pad < 0 || pad > ks - 1 || batch <= 0 || kc <= 0 || mtot <= 0 || groups <= 0) return false;
   const int ho = hs + 2 * pad - ks + 1, hp = ho + ks - 1;
   if (ho <= 0) return false;
   // padded rows of up to 32 floats; up to 64 on the 16-row kernel
   const int pw = hp <= 16 ? 16 : hp <= 32 ? 32 : 64;
   if (hp > pw) return false;
   // buffer loads address a tensor through 32-bit byte offsets
-  if ((double)batch * kc * hs * hs >= 1073741824.0 || (double)batch * ho * ho >= 2147483648.0) return false;
+  if ((double)batch * kc * groups * hs * hs >= 536870912.0 || (double)batch * ho * ho >= 2147483648.0) return false;
   const int cp = ks == 3 ? 2 : 1;
   const long ptot = (long)batch * ho * ho;
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
@@ -570,7 +585,7 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
       const size_t lds =
           2 * (size_t)((2 * cp * 32 * tmb * ks * ks + 255) / 256 * 256 + (patch + 63) / 64 * 64) * sizeof(float);
       if (patch > 256L * kDirectPatchLoads || lds > 64 * 1024) continue;
-      const long tiles = tiles_m * ((ptot + bn - 1) / bn);
+      const long tiles = groups * tiles_m * ((ptot + bn - 1) / bn);
       long slots = (long)(160 * 1024 / lds);
       if (slots > reg_slots[tmb][tnb]) slots = reg_slots[tmb][tnb];
       const long full = tiles / (cus * slots), rest = tiles - full * cus * slots;
@@ -637,13 +652,17 @@ struct DirectShuffle {
   int s, hs, pad, d;
 };
 
+// `kc` channels and `mtot` maps PER GROUP; with groups > 1 the tensors hold groups * kc channels and
+// groups * mtot maps per image and `wt` holds the groups' slab buffers one after another.
 static int conv_direct(const float *wt, const float *src, float *dst, const float *bias, int relu, int batch, int kc,
                        int mtot, int hs, int ks, int pad, size_t src_img_stride, size_t dst_img_stride,
-                       const float *mask = nullptr, const DirectShuffle *shuffle = nullptr) {
+                       const float *mask = nullptr, const DirectShuffle *shuffle = nullptr, int groups = 1) {
   DirectPlan pl;
-  CCT_REQUIRE(direct_plan(batch, kc, mtot, hs, ks, pad, &pl),
+  CCT_REQUIRE(groups >= 1, "conv_direct: groups must be positive");
+  CCT_REQUIRE(direct_plan(batch, kc, mtot, hs, ks, pad, &pl, groups),
               "conv_direct: geometry not covered (k=%d pad=%d size=%d)", ks, pad, hs);
   CCT_REQUIRE(!shuffle || pl.tm16, "conv_direct: the phase store needs the 16-row kernel");
+  CCT_REQUIRE(!shuffle || groups == 1, "conv_direct: the phase store takes one group");
   DirectArgs g;
   g.ss = g.shs = g.spad = g.sd = 0;
   if (shuffle) {
@@ -655,11 +674,11 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
   g.batch = batch; g.kc = kc; g.mtot = mtot; g.hs = hs; g.pad = pad;
   g.ho = hs + 2 * pad - ks + 1;
   {
-    const size_t dense_src = (size_t)kc * hs * hs, dense_dst = (size_t)mtot * g.ho * g.ho;
+    const size_t dense_src = (size_t)groups * kc * hs * hs, dense_dst = (size_t)groups * mtot * g.ho * g.ho;
     if (!src_img_stride) src_img_stride = dense_src;
     if (!dst_img_stride) dst_img_stride = dense_dst;
     CCT_REQUIRE(src_img_stride >= dense_src && dst_img_stride >= dense_dst, "conv_direct: image stride smaller than an image");
-    CCT_REQUIRE((double)batch * src_img_stride < 1073741824.0 && (double)batch * dst_img_stride < 2147483648.0,
+    CCT_REQUIRE((double)batch * src_img_stride < 536870912.0 && (double)batch * dst_img_stride < 2147483648.0,
                 "conv_direct: strided tensor too large for 32-bit byte offsets");
     g.src_img_stride = (uint32_t)src_img_stride;
     g.dst_img_stride = (uint32_t)dst_img_stride;
@@ -672,7 +691,10 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
   g.ptot = (uint32_t)((long)batch * g.ho * g.ho);
   g.tiles_m = pl.tm16 ? 1u : (uint32_t)((mtot + 32 * pl.tmb - 1) / (32 * pl.tmb));
   const uint32_t bn = 128 * pl.tnb;
-  g.ntiles = g.tiles_m * ((g.ptot + bn - 1) / bn);
+  g.groups = groups;
+  g.tiles_per_group = g.tiles_m * ((g.ptot + bn - 1) / bn);
+  g.ntiles = g.tiles_per_group * (uint32_t)groups;
+  g.wt_group_floats = (uint32_t)(direct_padded_channels(kc) * g.slab_stride);
   g.div_ho = make_fastdiv((uint32_t)g.ho);
   g.div_ho2 = make_fastdiv((uint32_t)(g.ho * g.ho));
   g.div_hp = make_fastdiv((uint32_t)g.hp);
@@ -731,6 +753,11 @@ struct WgradArgs {
   uint32_t dout_img_stride, src_img_stride;  // floats between images (channel-slice views)
   uint32_t tiles_m, tiles_n, ntiles, nblocks;
   FastDiv div_ho, div_ast;
+  // channel groups of a grouped convolution, all in this launch (o, d, ncols are PER GROUP): group q reads maps
+  // q*o .. of dout and channels q*d .. of src and writes block q of the [splits][groups][o][ncols] partial sums;
+  // ntiles = groups * tiles_per_group
+  int groups;
+  uint32_t tiles_per_group;
 };
 
 template <int KS, int PW>
@@ -757,7 +784,10 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
   const int nthreads = blockDim.x, nwaves = nthreads >> 6;
   const int r = lane & 31, h = lane >> 5;
   const uint32_t flat = xcd_remap(blockIdx.x, g.nblocks);
-  const uint32_t z = flat / g.ntiles, id = flat - z * g.ntiles;
+  const uint32_t z = flat / g.ntiles;
+  uint32_t id = flat - z * g.ntiles;
+  const uint32_t grp = g.groups > 1 ? id / g.tiles_per_group : 0u;  // workgroup-uniform
+  id -= grp * g.tiles_per_group;
   const uint32_t tm = id / g.tiles_n, tn = id - tm * g.tiles_n;  // column tiles of one row tile run together
   const int m0 = tm * g.bm, n0 = tn * BN, ch0 = n0 / KK;
   const int s_beg = z * g.steps_per_split, s_end = min(g.steps_total, s_beg + g.steps_per_split);
@@ -798,7 +828,7 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
     bmeta[k] = kr | (second << 4) | ((ok ? 1u : 0u) << 5);
   }
 
-  const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
+  const rsrc_t a_rsrc = make_rsrc(g.dout + (size_t)grp * g.o * ho2), b_rsrc = make_rsrc(g.src + (size_t)grp * g.d * hs2);
 
 // global -> LDS stage st for step s
 #define CCT_WGRAD_ISSUE(s, st)                                                                    \
@@ -920,9 +950,9 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
     // the two images of the pairs sit in the two lane halves; only the first column tile reports
     const float both = bsum + __shfl_xor(bsum, 32);
     const int row = m0 + wave * 32 + r;
-    if (h == 0 && row < g.o) g.out_bias[(size_t)z * g.o + row] = both;
+    if (h == 0 && row < g.o) g.out_bias[((size_t)z * g.groups + grp) * g.o + row] = both;
   }
-  float *out = g.out + (size_t)z * g.o * g.ncols;
+  float *out = g.out + ((size_t)z * g.groups + grp) * g.o * g.ncols;
 #pragma unroll
   for (int b = 0; b < TB; ++b) {
     const int col = n0 + b * 32 + r;
@@ -969,7 +999,10 @@ __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(con
   const int wn = WN == 1 ? 0 : wave_id / W, wave = wave_id - wn * W;  // column group, row block
   const int r = lane & 31, h = lane >> 5;
   const uint32_t flat = xcd_remap(blockIdx.x, g.nblocks);
-  const uint32_t z = flat / g.ntiles, id = flat - z * g.ntiles;
+  const uint32_t z = flat / g.ntiles;
+  uint32_t id = flat - z * g.ntiles;
+  const uint32_t grp = g.groups > 1 ? id / g.tiles_per_group : 0u;  // workgroup-uniform
+  id -= grp * g.tiles_per_group;
   const uint32_t tm = id / g.tiles_n, tn = id - tm * g.tiles_n;
   const int m0 = tm * (32 * W), n0 = tn * BN, ch0 = n0 / KK;
   const int s_beg = z * g.steps_per_split, s_end = min(g.steps_total, s_beg + g.steps_per_split);
@@ -992,7 +1025,7 @@ __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(con
     boff[k] = ok ? (second * g.src_img_stride + ch * hs2 + kr * g.hs + (uint32_t)scol) * 4u : 0u;
     bmeta[k] = kr | (second << 4) | ((ok ? 1u : 0u) << 5);
   }
-  const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
+  const rsrc_t a_rsrc = make_rsrc(g.dout + (size_t)grp * g.o * ho2), b_rsrc = make_rsrc(g.src + (size_t)grp * g.d * hs2);
 
   int bbase[TB];
 #pragma unroll
@@ -1128,9 +1161,9 @@ __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(con
     // the two images of the pairs sit in the two lane halves; only the first column tile reports
     const float both = bsum + __shfl_xor(bsum, 32);
     const int row = m0 + wave * 32 + r;
-    if (h == 0 && row < g.o) g.out_bias[(size_t)z * g.o + row] = both;
+    if (h == 0 && row < g.o) g.out_bias[((size_t)z * g.groups + grp) * g.o + row] = both;
   }
-  float *out = g.out + (size_t)z * g.o * g.ncols;
+  float *out = g.out + ((size_t)z * g.groups + grp) * g.o * g.ncols;
 #pragma unroll
   for (int b = 0; b < TB; ++b) {
     const int col = n0 + (wn * TB + b) * 32 + r;
@@ -1224,13 +1257,13 @@ struct WgradPlan {
   size_t lds;
 };
 
-static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPlan *pl) {
+static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPlan *pl, int groups = 1) {
   if (ks != 3 && ks != 5) return false;
   const int ho = n + 2 * pad - ks + 1, hp = ho + ks - 1;
   if (pad < 0 || pad > ks - 1 || ho <= 0 || hp > 32 || batch <= 0 || d <= 0 || o <= 0) return false;
   // buffer loads address a tensor through 32-bit byte offsets
-  if ((double)batch * o * ho * ho >= 1073741824.0 || (double)batch * d * n * n >= 1073741824.0 ||
-      (double)o * d * ks * ks >= 2147483648.0)
+  if ((double)batch * groups * o * ho * ho >= 536870912.0 || (double)batch * groups * d * n * n >= 536870912.0 ||
+      (double)groups * o * d * ks * ks >= 2147483648.0)
     return false;
   pl->pw = hp <= 16 ? 16 : 32;
   // wavefronts per workgroup (32 maps each): least padding of the map count, more wavefronts on ties
@@ -1323,14 +1356,27 @@ static int wgrad_launch(const WgradArgs &g, const WgradPlan &pl, hipStream_t st)
   return set_error(CCT_HIP_EINVAL, "conv_direct wgrad: no kernel instance for %d column blocks", pl.tb);
 }
 
+// `d` channels and `o` maps PER GROUP; with groups > 1 the tensors hold groups * d channels and groups * o maps
+// per image, dw is [groups][o][d][ks][ks] and db [groups][o].
 static int conv_direct_wgrad(float *dw, float *db, const float *dout, const float *src, int batch, int d, int n,
-                             int ks, int pad, int o, size_t src_img_stride, size_t dout_img_stride) {
+                             int ks, int pad, int o, size_t src_img_stride, size_t dout_img_stride, int groups = 1) {
   WgradPlan pl;
-  if (!wgrad_plan(batch, d, n, ks, pad, o, &pl)) {
-    // rows too long for the image-pair kernels: the one-image-per-step kernel, if its patch holds them
-    CCT_REQUIRE(conv_strided_wgrad_covers(batch, d, n, ks, 1, pad, o),
+  CCT_REQUIRE(groups >= 1, "conv_direct wgrad: groups must be positive");
+  if (!wgrad_plan(batch, d, n, ks, pad, o, &pl, groups)) {
+    // rows too long for the image-pair kernels: the one-image-per-step kernel, if its patch holds them,
+    // group by group on channel slices
+    CCT_REQUIRE(conv_strided_wgrad_covers(batch, d * groups, n, ks, 1, pad, o * groups) &&
+                    conv_strided_wgrad_covers(batch, d, n, ks, 1, pad, o),
                 "conv_direct wgrad: geometry not covered (k=%d pad=%d size=%d)", ks, pad, n);
-    return conv_strided_wgrad(dw, db, dout, src, batch, d, n, ks, 1, pad, o, src_img_stride, dout_img_stride);
+    const int ho = n + 2 * pad - ks + 1;
+    if (!src_img_stride) src_img_stride = (size_t)groups * d * n * n;
+    if (!dout_img_stride) dout_img_stride = (size_t)groups * o * ho * ho;
+    for (int q = 0; q < groups; ++q)
+      if (int rc = conv_strided_wgrad(dw + (size_t)q * o * d * ks * ks, db ? db + (size_t)q * o : nullptr,
+                                      dout + (size_t)q * o * ho * ho, src + (size_t)q * d * n * n, batch, d, n, ks, 1,
+                                      pad, o, src_img_stride, dout_img_stride))
+        return rc;
+    return 0;
   }
   WgradArgs g;
   g.dout = dout; g.src = src;
@@ -1338,12 +1384,12 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   g.ho = n + 2 * pad - ks + 1;
   g.ncols = d * ks * ks;
   {
-    const size_t dense_src = (size_t)d * n * n, dense_dout = (size_t)o * g.ho * g.ho;
+    const size_t dense_src = (size_t)groups * d * n * n, dense_dout = (size_t)groups * o * g.ho * g.ho;
     if (!src_img_stride) src_img_stride = dense_src;
     if (!dout_img_stride) dout_img_stride = dense_dout;
     CCT_REQUIRE(src_img_stride >= dense_src && dout_img_stride >= dense_dout,
                 "conv_direct wgrad: image stride smaller than an image");
-    CCT_REQUIRE((double)batch * src_img_stride < 1073741824.0 && (double)batch * dout_img_stride < 1073741824.0,
+    CCT_REQUIRE((double)batch * src_img_stride < 536870912.0 && (double)batch * dout_img_stride < 536870912.0,
                 "conv_direct wgrad: strided tensor too large for 32-bit byte offsets");
     g.src_img_stride = (uint32_t)src_img_stride;
     g.dout_img_stride = (uint32_t)dout_img_stride;
@@ -1352,13 +1398,16 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   g.steps_total = ((batch + 1) / 2) * g.ho;
   g.tiles_m = (uint32_t)((o + g.bm - 1) / g.bm);
   g.tiles_n = (uint32_t)((g.ncols + 32 * pl.tb * pl.wn - 1) / (32 * pl.tb * pl.wn));
-  g.ntiles = g.tiles_m * g.tiles_n;
+  g.groups = groups;
+  g.tiles_per_group = g.tiles_m * g.tiles_n;
+  g.ntiles = g.tiles_per_group * (uint32_t)groups;
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
   // workgroups resident per compute unit: LDS and wavefront slots (two per SIMD is plenty here)
   int per_cu = (int)((160 * 1024) / pl.lds);
   if (per_cu > 8 / (pl.waves * pl.wn)) per_cu = 8 / (pl.waves * pl.wn);
   if (per_cu < 1) per_cu = 1;
   int splits = (int)((long)per_cu * cus / g.ntiles);
+  if (tuning().direct_splits > 0) splits = tuning().direct_splits;  // tuning override
   if (splits < 1) splits = 1;
   if (splits > g.steps_total) splits = g.steps_total;
   g.steps_per_split = (g.steps_total + splits - 1) / splits;
@@ -1366,10 +1415,11 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   g.nblocks = g.ntiles * (uint32_t)splits;
   g.div_ho = make_fastdiv((uint32_t)g.ho);
   g.div_ast = make_fastdiv((uint32_t)g.ast);
-  const size_t n_out = (size_t)o * g.ncols;
+  const size_t n_out = (size_t)groups * o * g.ncols;  // all groups: dw is one contiguous [groups][o][ncols] block
+  const int o_all = groups * o;
   if (splits > 1) {
     void *ws = nullptr;
-    int rc = get_workspace((size_t)splits * (n_out + (db ? o : 0)) * sizeof(float), &ws);
+    int rc = get_workspace((size_t)splits * (n_out + (db ? o_all : 0)) * sizeof(float), &ws);
     if (rc) return rc;
     g.out = (float *)ws;
     g.out_bias = db ? g.out + (size_t)splits * n_out : nullptr;
@@ -1389,7 +1439,7 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   else rc = pl.pw == 16 ? wgrad_launch<3, 16>(g, pl, st) : wgrad_launch<3, 32>(g, pl, st);
   if (rc) return rc;
   if (splits > 1) {
-    const uint32_t n2 = db ? (uint32_t)o : 0u;
+    const uint32_t n2 = db ? (uint32_t)o_all : 0u;
     if (int rc2 = reduce_partial_sums(dw, g.out, (uint32_t)n_out, db, g.out_bias, n2, splits, st)) return rc2;
   }
   return 0;
@@ -1448,86 +1498,136 @@ static bool strided_dgrad_plan(int batch, int d, int n, int ks, int stride, int 
 
 using namespace cct;
 
-extern "C" int cct_hip_conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding,
-                                             int num_outputs) {
-  if (stride != 1 || ensure_init() != 0) return 0;
+static bool groups_divide(int groups, int depth, int num_outputs) {
+  return groups >= 1 && depth > 0 && num_outputs > 0 && depth % groups == 0 && num_outputs % groups == 0;
+}
+
+extern "C" int cct_hip_conv_direct_supported_grouped(int batch, int depth, int n, int k, int stride, int padding,
+                                                     int num_outputs, int groups) {
+  if (stride != 1 || !groups_divide(groups, depth, num_outputs) || ensure_init() != 0) return 0;
   DirectPlan pl;
   const int m = n + 2 * padding - k + 1;
+  const int dg = depth / groups, og = num_outputs / groups;
   // forward: channels = depth, maps = outputs, source n, pad p; data gradient: channels = outputs,
   // maps = depth, source m, pad k-1-p
   WgradPlan wp;
-  return direct_plan(batch, depth, num_outputs, n, k, padding, &pl) &&
-                 direct_plan(batch, num_outputs, depth, m, k, k - 1 - padding, &pl) &&
-                 (wgrad_plan(batch, depth, n, k, padding, num_outputs, &wp) ||
-                  conv_strided_wgrad_covers(batch, depth, n, k, 1, padding, num_outputs))
+  return direct_plan(batch, dg, og, n, k, padding, &pl, groups) &&
+                 direct_plan(batch, og, dg, m, k, k - 1 - padding, &pl, groups) &&
+                 (wgrad_plan(batch, dg, n, k, padding, og, &wp, groups) ||
+                  (conv_strided_wgrad_covers(batch, dg, n, k, 1, padding, og) &&
+                   conv_strided_wgrad_covers(batch, depth, n, k, 1, padding, num_outputs)))
              ? 1
              : 0;
 }
 
+extern "C" int cct_hip_conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding,
+                                             int num_outputs) {
+  return cct_hip_conv_direct_supported_grouped(batch, depth, n, k, stride, padding, num_outputs, 1);
+}
+
+extern "C" size_t cct_hip_conv_direct_slab_floats_grouped(int num_outputs, int depth, int k, int for_data_gradient,
+                                                          int groups) {
+  if (k <= 0 || !groups_divide(groups, depth, num_outputs)) return 0;
+  const int og = num_outputs / groups, dg = depth / groups;
+  const int n_c = for_data_gradient ? og : dg, n_m = for_data_gradient ? dg : og;
+  return (size_t)groups * direct_padded_channels(n_c) * direct_padded_maps(n_m) * k * k;
+}
+
 extern "C" size_t cct_hip_conv_direct_slab_floats(int num_outputs, int depth, int k, int for_data_gradient) {
-  if (num_outputs <= 0 || depth <= 0 || k <= 0) return 0;
-  const int n_c = for_data_gradient ? num_outputs : depth, n_m = for_data_gradient ? depth : num_outputs;
-  return (size_t)direct_padded_channels(n_c) * direct_padded_maps(n_m) * k * k;
+  return cct_hip_conv_direct_slab_floats_grouped(num_outputs, depth, k, for_data_gradient, 1);
+}
+
+extern "C" int cct_hip_conv_direct_slabs_grouped(float *slabs, const float *model, int num_outputs, int depth, int k,
+                                                 int for_data_gradient, int groups) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(k > 0 && groups_divide(groups, depth, num_outputs), "conv_direct_slabs: bad dimensions");
+  CCT_REQUIRE(slabs != model, "conv_direct_slabs: in-place use");
+  const int og = num_outputs / groups, dg = depth / groups;
+  const size_t total = cct_hip_conv_direct_slab_floats(og, dg, k, for_data_gradient);  // per group
+  CCT_REQUIRE(total * groups < (1ull << 31), "conv_direct_slabs: model too large");
+  // forward slabs: [depth][outputs][k*k]; data-gradient slabs: [outputs][depth][k*k] reversed; one such
+  // buffer per group, one after another
+  const int n_c = for_data_gradient ? og : dg, n_m = for_data_gradient ? dg : og;
+  const int p_m = direct_padded_maps(n_m);
+  hipLaunchKernelGGL(direct_slab_kernel, dim3((uint32_t)((total + 255) / 256), (uint32_t)groups), dim3(256), 0,
+                     ctx().stream, slabs, model, n_c, n_m, p_m, (uint32_t)total, k * k, for_data_gradient ? 1 : 0,
+                     make_fastdiv((uint32_t)(k * k)), make_fastdiv((uint32_t)p_m));
+  CCT_LAUNCH_CHECK();
+  return 0;
 }
 
 extern "C" int cct_hip_conv_direct_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
                                          int for_data_gradient) {
+  return cct_hip_conv_direct_slabs_grouped(slabs, model, num_outputs, depth, k, for_data_gradient, 1);
+}
+
+extern "C" int cct_hip_conv_direct_forward_grouped(float *output, const float *input, const float *slabs,
+                                                   const float *bias, int batch, int depth, int n, int k,
+                                                   int padding, int num_outputs, size_t input_image_stride,
+                                                   size_t output_image_stride, int relu, int groups) {
   CCT_ENSURE_INIT();
-  CCT_REQUIRE(num_outputs > 0 && depth > 0 && k > 0, "conv_direct_slabs: bad dimensions");
-  CCT_REQUIRE(slabs != model, "conv_direct_slabs: in-place use");
-  const size_t total = cct_hip_conv_direct_slab_floats(num_outputs, depth, k, for_data_gradient);
-  CCT_REQUIRE(total < (1ull << 31), "conv_direct_slabs: model too large");
-  // forward slabs: [depth][outputs][k*k]; data-gradient slabs: [outputs][depth][k*k] reversed
-  const int n_c = for_data_gradient ? num_outputs : depth, n_m = for_data_gradient ? depth : num_outputs;
-  const int p_m = direct_padded_maps(n_m);
-  hipLaunchKernelGGL(direct_slab_kernel, dim3((uint32_t)((total + 255) / 256)), dim3(256), 0, ctx().stream,
-                     slabs, model, n_c, n_m, p_m, (uint32_t)total, k * k, for_data_gradient ? 1 : 0,
-                     make_fastdiv((uint32_t)(k * k)), make_fastdiv((uint32_t)p_m));
-  CCT_LAUNCH_CHECK();
-  return 0;
+  CCT_REQUIRE(groups_divide(groups, depth, num_outputs), "conv_direct_forward: groups must divide both depths");
+  if (batch <= 0) return 0;
+  return conv_direct(slabs, input, output, bias, relu != 0, batch, depth / groups, num_outputs / groups, n, k,
+                     padding, input_image_stride, output_image_stride, nullptr, nullptr, groups);
 }
 
 extern "C" int cct_hip_conv_direct_forward(float *output, const float *input, const float *slabs,
                                            const float *bias, int batch, int depth, int n, int k, int padding,
                                            int num_outputs, size_t input_image_stride, size_t output_image_stride,
                                            int relu) {
+  return cct_hip_conv_direct_forward_grouped(output, input, slabs, bias, batch, depth, n, k, padding, num_outputs,
+                                             input_image_stride, output_image_stride, relu, 1);
+}
+
+extern "C" int cct_hip_conv_direct_backward_data_grouped(float *input_grad, const float *output_grad,
+                                                         const float *slabs, int batch, int depth, int n, int k,
+                                                         int padding, int num_outputs, size_t input_image_stride,
+                                                         size_t output_image_stride, const float *relu_data,
+                                                         int groups) {
   CCT_ENSURE_INIT();
+  CCT_REQUIRE(groups_divide(groups, depth, num_outputs), "conv_direct_backward_data: groups must divide both depths");
   if (batch <= 0) return 0;
-  return conv_direct(slabs, input, output, bias, relu != 0, batch, depth, num_outputs, n, k, padding,
-                     input_image_stride, output_image_stride);
+  const int m = n + 2 * padding - k + 1;
+  return conv_direct(slabs, output_grad, input_grad, nullptr, 0, batch, num_outputs / groups, depth / groups, m, k,
+                     k - 1 - padding, output_image_stride, input_image_stride, relu_data, nullptr, groups);
 }
 
 extern "C" int cct_hip_conv_direct_backward_data(float *input_grad, const float *output_grad,
                                                  const float *slabs, int batch, int depth, int n, int k,
                                                  int padding, int num_outputs, size_t input_image_stride,
                                                  size_t output_image_stride) {
-  CCT_ENSURE_INIT();
-  if (batch <= 0) return 0;
-  const int m = n + 2 * padding - k + 1;
-  return conv_direct(slabs, output_grad, input_grad, nullptr, 0, batch, num_outputs, depth, m, k,
-                     k - 1 - padding, output_image_stride, input_image_stride);
+  return cct_hip_conv_direct_backward_data_grouped(input_grad, output_grad, slabs, batch, depth, n, k, padding,
+                                                   num_outputs, input_image_stride, output_image_stride, nullptr, 1);
 }
 
 extern "C" int cct_hip_conv_direct_backward_data_relu(float *input_grad, const float *output_grad,
                                                       const float *slabs, int batch, int depth, int n, int k,
                                                       int padding, int num_outputs, size_t input_image_stride,
                                                       size_t output_image_stride, const float *relu_data) {
-  CCT_ENSURE_INIT();
   CCT_REQUIRE(relu_data, "conv_direct_backward_data_relu: null activation tensor");
-  if (batch <= 0) return 0;
-  const int m = n + 2 * padding - k + 1;
-  return conv_direct(slabs, output_grad, input_grad, nullptr, 0, batch, num_outputs, depth, m, k,
-                     k - 1 - padding, output_image_stride, input_image_stride, relu_data);
+  return cct_hip_conv_direct_backward_data_grouped(input_grad, output_grad, slabs, batch, depth, n, k, padding,
+                                                   num_outputs, input_image_stride, output_image_stride, relu_data, 1);
+}
+
+extern "C" int cct_hip_conv_direct_backward_weights_grouped(float *model_grad, float *bias_grad,
+                                                            const float *output_grad, const float *input, int batch,
+                                                            int depth, int n, int k, int padding, int num_outputs,
+                                                            size_t input_image_stride, size_t output_image_stride,
+                                                            int groups) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(batch > 0, "conv_direct_backward_weights: empty batch");
+  CCT_REQUIRE(groups_divide(groups, depth, num_outputs), "conv_direct_backward_weights: groups must divide both depths");
+  return conv_direct_wgrad(model_grad, bias_grad, output_grad, input, batch, depth / groups, n, k, padding,
+                           num_outputs / groups, input_image_stride, output_image_stride, groups);
 }
 
 extern "C" int cct_hip_conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                                     const float *input, int batch, int depth, int n, int k,
                                                     int padding, int num_outputs, size_t input_image_stride,
                                                     size_t output_image_stride) {
-  CCT_ENSURE_INIT();
-  CCT_REQUIRE(batch > 0, "conv_direct_backward_weights: empty batch");
-  return conv_direct_wgrad(model_grad, bias_grad, output_grad, input, batch, depth, n, k, padding, num_outputs,
-                           input_image_stride, output_image_stride);
+  return cct_hip_conv_direct_backward_weights_grouped(model_grad, bias_grad, output_grad, input, batch, depth, n, k,
+                                                      padding, num_outputs, input_image_stride, output_image_stride, 1);
 }
 
 extern "C" int cct_hip_conv_strided_backward_data_supported(int batch, int depth, int n, int k, int stride,

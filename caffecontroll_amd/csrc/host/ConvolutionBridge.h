@@ -21,7 +21,12 @@
 //     and weight-gradient kernels of their own; their data gradient (not needed for a first layer)
 //     comes from a direct kernel too where it covers the geometry (depth * stride^2 <= 80 in an odd
 //     number of 16-row blocks: AlexNet / CaffeNet conv1), else from the data-gradient GEMM and the
-//     lifting, which need no lowered input.
+//     lifting, which need no lowered input;
+//   * `group` > 1 (cnn.proto ConvolutionParameter.group, which the reference's bridge ignores and its
+//     network builder realises as towers between a Split and a Concat, src/DeepNet.h:1700-1757) is
+//     run by this one bridge: the model cube is [o][d/group][k][k] (the blob layout Caffe gives such
+//     a layer), group q maps its slice of the input channels to its slice of the output maps, and the
+//     direct kernels run all groups in one launch each.  Only the all-direct path covers it.
 #pragma once
 #include <cstdio>
 #include <cstdlib>
@@ -67,6 +72,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   typedef LogicalCube<DataType> LogicalCubeType;
 
   const size_t K;
+  const size_t group;  // channel groups (1: an ordinary convolution)
   const size_t num_output_features;
   const size_t stride;
   const size_t padding;
@@ -81,21 +87,22 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                     const cnn::LayerParameter *const _layer_param,
                     const cnn::SolverParameter *const _solver_param, DriverClass *const _p_driver)
       : Base(_p_input_layer, _p_output_layer, _layer_param, _solver_param, _p_driver),
-        K(_layer_param->convolution_param().kernel_size()), num_output_features(_p_output_layer->dD),
+        K(_layer_param->convolution_param().kernel_size()),
+        group(_layer_param->convolution_param().group() > 1 ? _layer_param->convolution_param().group() : 1),
+        num_output_features(_p_output_layer->dD),
         stride(_layer_param->convolution_param().stride()), padding(_layer_param->convolution_param().pad()),
         bias_term(_layer_param->convolution_param().bias_term()),
         weight_filler(_layer_param->convolution_param().weight_filler()),
         bias_filler(_layer_param->convolution_param().bias_filler()), p_model_cube(nullptr),
         p_bias_cube(nullptr), p_bias_gradient_cube(nullptr) {
     if (oR != (iR + 2 * padding - K) / stride + 1 || oC != (iC + 2 * padding - K) / stride + 1 || iB != oB ||
-        num_output_features != oD || iR != iC) {
-      std::fprintf(stderr, "ConvolutionBridge: inconsistent layer shapes\n");
-      std::abort();
+        num_output_features != oD || iR != iC || iD % group || num_output_features % group) {
+      host_fail("ConvolutionBridge: inconsistent layer shapes");
     }
     // cubes read outside the bridge (model / gradients), device resident
-    p_model_cube = new LogicalCubeType(K, K, iD, num_output_features, p_driver);
+    p_model_cube = new LogicalCubeType(K, K, iD / group, num_output_features, p_driver);
     initialize_logical_cube(p_model_cube, weight_filler);
-    p_model_gradient_cube = new LogicalCubeType(K, K, iD, num_output_features, p_driver);
+    p_model_gradient_cube = new LogicalCubeType(K, K, iD / group, num_output_features, p_driver);
     DeviceMemoryPointer mg = p_model_gradient_cube->get_device_pointer(p_driver);
     p_driver->sconstant_initialize(&mg, DataType(0.));
     if (bias_term) {
@@ -112,6 +119,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     p_forward_slabs = nullptr;
     p_backward_slabs = nullptr;
 
+    // shapes of the lowering path's GEMM operands (never run for a grouped layer)
     LogicalCubeType lowered_forward_model(nullptr, num_output_features, K * K * iD, 1, 1);
     LogicalCubeType lowered_forward_output(nullptr, num_output_features, oR * oC * iB, 1, 1);
     LogicalCubeType lowered_data(nullptr, K * K * iD, oR * oC * iB, 1, 1);
@@ -125,20 +133,23 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     p_backward_gemm_updategrad_kernel = new Kernel<DataType, KernelConfig_GEMM_TRANS_NOTRANS, DriverClass>(
         &lowered_forward_model, &lowered_forward_output, &lowered_data, p_driver);
     direct_ok_ = p_driver->conv_direct_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
-                                                 (int)num_output_features);
-    strided_ok_ = !direct_ok_ && p_driver->conv_strided_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride,
+                                                 (int)num_output_features, (int)group);
+    if (group > 1 && !direct_ok_)
+      host_fail("ConvolutionBridge: a grouped convolution runs on the direct kernels only, which do not cover this geometry");
+    strided_ok_ = !direct_ok_ && group == 1 && p_driver->conv_strided_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride,
                                                                   (int)padding, (int)num_output_features);
     strided_data_ok_ = strided_ok_ && p_driver->conv_strided_backward_data_supported(
                                           (int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
                                           (int)num_output_features);
     // Small layers (LeNet-sized) stay on the fused lowering path by default: the direct kernels'
     // fixed costs (slab re-layout, partial-sum reduction) outweigh what they save below a few GFLOP.
-    const double gemm_flop = 2.0 * num_output_features * (double)(oR * oC * iB) * (double)(K * K * iD);
+    const double gemm_flop = 2.0 * num_output_features * (double)(oR * oC * iB) * (double)(K * K * iD / group);
     // (a very short contraction -- LeNet conv1 has k*k*d = 25 -- makes the lowered GEMM all prologue and
     // epilogue; there the direct kernels win at any size)
     const bool short_contraction = K * K * iD <= 64;
     default_path_ = (direct_ok_ && (gemm_flop >= kConvDirectMinFlop || short_contraction)) ? PATH_DIRECT_ALL : PATH_FUSED;
     if (strided_ok_ && gemm_flop >= kConvDirectMinFlop) default_path_ = PATH_DIRECT_ALL;
+    if (group > 1) default_path_ = PATH_DIRECT_ALL;
     path_ = default_path_;
     for (int i = 0; i < STAGE_COUNT; ++i) { timers_[i] = nullptr; stage_ms_[i] = 0.f; }
   }
@@ -173,7 +184,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     if (level < PATH_STAGED) level = PATH_STAGED;
     if (level > PATH_DIRECT_ALL) level = PATH_DIRECT_ALL;
     if (level >= PATH_DIRECT_DATA && !direct_ok_) level = (strided_ok_ && level == PATH_DIRECT_ALL) ? PATH_DIRECT_ALL : PATH_FUSED;
-    if (views_) level = PATH_DIRECT_ALL;  // the lowering path cannot address channel-slice views
+    if (views_ || group > 1) level = PATH_DIRECT_ALL;  // the lowering path cannot address channel slices
     path_ = level;
   }
   int path() const { return path_; }
@@ -184,8 +195,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   // bridge then stays on it.
   void set_image_strides(size_t in_stride, size_t out_stride) {
     if (!direct_ok_) {
-      std::fprintf(stderr, "ConvolutionBridge: channel-slice views need the direct kernels\n");
-      std::abort();
+      host_fail("ConvolutionBridge: channel-slice views need the direct kernels");
     }
     in_image_stride_ = in_stride;
     out_image_stride_ = out_stride;
@@ -236,11 +246,11 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       // slabs are rebuilt every pass: the model changes between iterations
       begin(STAGE_GEMM);
       p_driver->conv_direct_slabs(forward_slabs()->get_p_data(), p_model_cube->get_p_data(),
-                                  (int)num_output_features, (int)iD, (int)K, 0);
+                                  (int)num_output_features, (int)iD, (int)K, 0, (int)group);
       p_driver->conv_direct_forward(output_d_cube->get_p_data(), input_d_cube->get_p_data(),
                                     forward_slabs()->get_p_data(), bias_term ? p_bias_cube->get_p_data() : nullptr,
                                     (int)iB, (int)iD, (int)iR, (int)K, (int)padding, (int)num_output_features,
-                                    in_image_stride_, out_image_stride_, fuse_relu_);
+                                    in_image_stride_, out_image_stride_, fuse_relu_, (int)group);
       end(STAGE_GEMM);
       report_forward_history.end();
       return;
@@ -335,7 +345,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                              bias_term ? p_bias_gradient_cube->get_p_data() : nullptr,
                                              output_g_cube->get_p_data(), p_input_layer->p_data_cube->get_p_data(),
                                              (int)iB, (int)iD, (int)iR, (int)K, (int)padding,
-                                             (int)num_output_features, in_image_stride_, out_image_stride_);
+                                             (int)num_output_features, in_image_stride_, out_image_stride_,
+                                             (int)group);
     } else {
       p_backward_gemm_updateweight_kernel->alpha = 1.0;
       p_backward_gemm_updateweight_kernel->beta = 0.0;
@@ -346,12 +357,13 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       // remap + data-gradient GEMM + lifting in one kernel, reading the output gradient in place
       begin(STAGE_GEMM_DATA);
       p_driver->conv_direct_slabs(backward_slabs()->get_p_data(), p_model_cube->get_p_data(),
-                                  (int)num_output_features, (int)iD, (int)K, 1);
+                                  (int)num_output_features, (int)iD, (int)K, 1, (int)group);
       p_driver->conv_direct_backward_data(input_g_cube->get_p_data(), output_g_cube->get_p_data(),
                                           backward_slabs()->get_p_data(), (int)iB, (int)iD, (int)iR, (int)K,
                                           (int)padding, (int)num_output_features, in_image_stride_,
                                           out_image_stride_,
-                                          input_is_relu_output ? p_input_layer->p_data_cube->get_p_data() : nullptr);
+                                          input_is_relu_output ? p_input_layer->p_data_cube->get_p_data() : nullptr,
+                                          (int)group);
       end(STAGE_GEMM_DATA);
     } else if (strided_direct_data) {
       // remap + data-gradient GEMM + lifting of a strided layer in one kernel (phase decomposition)
@@ -413,8 +425,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       p_driver->sgaussian_initialize(&data, (DataType)filler_param.mean(), (DataType)filler_param.std(),
                                      solver_param->random_seed());
     } else {
-      std::fprintf(stderr, "ERROR! INITIALIZATION TYPE NOT SUPPORTED: %s\n", type.c_str());
-      std::abort();
+      host_fail("ERROR! INITIALIZATION TYPE NOT SUPPORTED: " + type);
     }
   }
 
@@ -441,7 +452,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       p_forward_slabs = new LogicalCubeType(
           strided_ok_ ? p_driver->conv_strided_slab_floats((int)num_output_features, (int)iD, (int)K, (int)stride,
                                                            (int)padding)
-                      : p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 0),
+                      : p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 0, (int)group),
           1, 1, 1, p_driver);
     return p_forward_slabs;
   }
@@ -450,7 +461,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
       p_backward_slabs = new LogicalCubeType(
           strided_data_ok_ ? p_driver->conv_strided_backward_data_slab_floats((int)num_output_features, (int)iD,
                                                                               (int)K, (int)stride)
-                           : p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 1),
+                           : p_driver->conv_direct_slab_floats((int)num_output_features, (int)iD, (int)K, 1, (int)group),
           1, 1, 1, p_driver);
     return p_backward_slabs;
   }

@@ -37,8 +37,7 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
         bias_term(_layer_param->inner_product_param().bias_term()), p_model_cube(nullptr), p_bias_cube(nullptr),
         p_bias_gradient_cube(nullptr) {
     if (oR != 1 || oC != 1 || iB != oB || oD != num_output_features || iR != iC) {
-      std::fprintf(stderr, "FullyConnectedBridge: inconsistent layer shapes\n");
-      std::abort();
+      host_fail("FullyConnectedBridge: inconsistent layer shapes");
     }
     p_model_cube = new LogicalCubeType(K, K, iD, oD, p_driver);
     initialize_logical_cube(p_model_cube, _layer_param->inner_product_param().weight_filler());
@@ -126,8 +125,7 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
       p_driver->sgaussian_initialize(&data, (DataType)filler_param.mean(), (DataType)filler_param.std(),
                                      solver_param->random_seed());
     } else {
-      std::fprintf(stderr, "ERROR! INITIALIZATION TYPE NOT SUPPORTED: %s\n", type.c_str());
-      std::abort();
+      host_fail("ERROR! INITIALIZATION TYPE NOT SUPPORTED: " + type);
     }
   }
 };

@@ -3,7 +3,9 @@
 // and argument meaning; every member forwards to the C ABI in include/cct_hip.h.
 //
 // Error behaviour follows src/sched/DeviceDriver.h:48-51: members return void; on error the
-// message is printed and the process aborts (the reference asserts).
+// message is printed and the process aborts (the reference asserts) -- unless the calling thread
+// is inside an ErrorsAsExceptions scope (Fail.h), as the C entry points over the bridges are: then
+// the member throws HostError with the same message.
 //
 // The reference selects kernels with C function pointers as template arguments
 // (parallel_map<idx,func>).  The closed set of pairs it instantiates
@@ -15,9 +17,11 @@
 #include <cstdlib>
 #include <mutex>
 #include <random>
+#include <string>
 #include <vector>
 
 #include "../../../include/cct_hip.h"
+#include "Fail.h"
 #include "DeviceMemoryPointer.h"
 
 namespace cct {
@@ -47,7 +51,7 @@ class HIPDriver {
   // direction is taken from the two pointer types, as GPUDriver::memcpy does
   void memcpy(DeviceMemoryPointer *dst, DeviceMemoryPointer *src) {
     const bool dd = dst->type == DEVICEMEMORY_LOCAL_GPURAM, sd = src->type == DEVICEMEMORY_LOCAL_GPURAM;
-    if (!dd && !sd) { std::fprintf(stderr, "HIPDriver::memcpy: host to host copy\n"); std::abort(); }
+    if (!dd && !sd) { host_fail("HIPDriver::memcpy: host to host copy"); }
     const int kind = (dd && sd) ? 2 : dd ? 0 : 1;
     ok(cct_hip_memcpy(dst->ptr, src->ptr, dst->size_in_byte, kind), "memcpy");
   }
@@ -232,42 +236,40 @@ class HIPDriver {
     ok(cct_hip_sgemm_conv_forward(o, batch, fmap, K, model, lowered, bias, out, relu ? 1 : 0), "sgemm_conv_forward");
   }
   // ---- stride-1 convolution without the lowered matrix (no counterpart in DeviceDriver.h) ----
-  bool conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs) {
-    return cct_hip_conv_direct_supported(batch, depth, n, k, stride, padding, num_outputs) != 0;
+  // `groups` > 1: a grouped convolution (depth and num_outputs are the layer's totals), all groups in one launch
+  bool conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs,
+                             int groups = 1) {
+    return cct_hip_conv_direct_supported_grouped(batch, depth, n, k, stride, padding, num_outputs, groups) != 0;
   }
-  size_t conv_direct_slab_floats(int num_outputs, int depth, int k, int for_data_gradient) {
-    return cct_hip_conv_direct_slab_floats(num_outputs, depth, k, for_data_gradient);
+  size_t conv_direct_slab_floats(int num_outputs, int depth, int k, int for_data_gradient, int groups = 1) {
+    return cct_hip_conv_direct_slab_floats_grouped(num_outputs, depth, k, for_data_gradient, groups);
   }
   void conv_direct_slabs(float *slabs, const float *model, int num_outputs, int depth, int k,
-                         int for_data_gradient) {
-    ok(cct_hip_conv_direct_slabs(slabs, model, num_outputs, depth, k, for_data_gradient), "conv_direct_slabs");
+                         int for_data_gradient, int groups = 1) {
+    ok(cct_hip_conv_direct_slabs_grouped(slabs, model, num_outputs, depth, k, for_data_gradient, groups),
+       "conv_direct_slabs");
   }
   void conv_direct_forward(float *output, const float *input, const float *slabs, const float *bias, int batch,
                            int depth, int n, int k, int padding, int num_outputs, size_t in_stride = 0,
-                           size_t out_stride = 0, bool relu = false) {
-    ok(cct_hip_conv_direct_forward(output, input, slabs, bias, batch, depth, n, k, padding, num_outputs, in_stride,
-                                   out_stride, relu ? 1 : 0),
+                           size_t out_stride = 0, bool relu = false, int groups = 1) {
+    ok(cct_hip_conv_direct_forward_grouped(output, input, slabs, bias, batch, depth, n, k, padding, num_outputs,
+                                           in_stride, out_stride, relu ? 1 : 0, groups),
        "conv_direct_forward");
   }
   // relu_data (optional): the layer's input tensor when it is the output of an in-place ReLU -- the
   // gradient is then stored already masked with (relu_data > 0)
   void conv_direct_backward_data(float *input_grad, const float *output_grad, const float *slabs, int batch,
                                  int depth, int n, int k, int padding, int num_outputs, size_t in_stride = 0,
-                                 size_t out_stride = 0, const float *relu_data = nullptr) {
-    if (relu_data)
-      ok(cct_hip_conv_direct_backward_data_relu(input_grad, output_grad, slabs, batch, depth, n, k, padding,
-                                                num_outputs, in_stride, out_stride, relu_data),
-         "conv_direct_backward_data_relu");
-    else
-      ok(cct_hip_conv_direct_backward_data(input_grad, output_grad, slabs, batch, depth, n, k, padding,
-                                           num_outputs, in_stride, out_stride),
-         "conv_direct_backward_data");
+                                 size_t out_stride = 0, const float *relu_data = nullptr, int groups = 1) {
+    ok(cct_hip_conv_direct_backward_data_grouped(input_grad, output_grad, slabs, batch, depth, n, k, padding,
+                                                 num_outputs, in_stride, out_stride, relu_data, groups),
+       relu_data ? "conv_direct_backward_data_relu" : "conv_direct_backward_data");
   }
   void conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                     const float *input, int batch, int depth, int n, int k, int padding,
-                                    int num_outputs, size_t in_stride = 0, size_t out_stride = 0) {
-    ok(cct_hip_conv_direct_backward_weights(model_grad, bias_grad, output_grad, input, batch, depth, n, k, padding,
-                                            num_outputs, in_stride, out_stride),
+                                    int num_outputs, size_t in_stride = 0, size_t out_stride = 0, int groups = 1) {
+    ok(cct_hip_conv_direct_backward_weights_grouped(model_grad, bias_grad, output_grad, input, batch, depth, n, k,
+                                                    padding, num_outputs, in_stride, out_stride, groups),
        "conv_direct_backward_weights");
   }
   // ---- strided convolution without the lowered matrix (no counterpart in DeviceDriver.h) ----
@@ -351,10 +353,8 @@ class HIPDriver {
  private:
   int device_id_ = 0;
   static void ok(int rc, const char *what) {
-    if (rc != 0) {
-      std::fprintf(stderr, "HIPDriver::%s failed (%d): %s\n", what, rc, cct_hip_last_error());
-      std::abort();
-    }
+    if (rc != 0)
+      host_fail(std::string("HIPDriver::") + what + " failed (" + std::to_string(rc) + "): " + cct_hip_last_error());
   }
 
  private:

@@ -20,15 +20,17 @@
 //   * ReLU and dropout run in place on their input layer (the reference shares the layers on the
 //     GPU: ParallelizedBridge.h:183-198); an in-place ReLU directly after a convolution is applied
 //     by the convolution's output store (same values, one pass over the tensor less);
-//   * `group` > 1 is realised as `group` independent convolutions on channel slices whose outputs
-//     are concatenated along depth (the reference's two-tower Split/Concat arrangement,
-//     src/DeepNet.h:1700-1757); a group runs in place on its channel slices when the direct
-//     kernels take the layer, otherwise the slices are moved with a strided device copy.
+//   * `group` > 1 is `group` independent convolutions on channel slices whose outputs are
+//     concatenated along depth (the reference's two-tower Split/Concat arrangement,
+//     src/DeepNet.h:1700-1757): one bridge that runs all groups in each of its launches when the
+//     direct kernels take the layer, otherwise one bridge per group on contiguous copies of the
+//     slices, moved with a strided device copy.
 //
 // Model files and snapshots use the reference's format (src/DeepNet.h:268-422): raw fp32, for
 // every bridge in order its model cube and then its bias cube; a snapshot is three files
 // <base>.snapshot_iter<N>.{MODEL,HISTORY,ITER}.bin (weights, momentum buffers, one int).
 #pragma once
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <map>
@@ -57,10 +59,21 @@ class Network {
     LayerT *out = nullptr;
     std::vector<LayerT *> ins;                   // every bottom (CONCAT has several)
     bool run_backward = true;                    // false: no layer with weights upstream and none here
-    std::vector<BridgeT *> bridges;              // one per group (1 for everything but grouped conv)
+    std::vector<BridgeT *> bridges;              // 1; one per group for a grouped conv off the direct kernels
     std::vector<LayerT *> group_in, group_out;   // per-group contiguous layers (grouped conv only)
     std::vector<cnn::LayerParameter *> params;
   };
+
+  // What the filler draws (cct_hip_fill_*) would refuse, said before anything is built; NULL if fine.
+  static const char *bad_filler(const cct_filler &f) {
+    if (f.type < 0 || f.type > 3) return "unknown filler type";
+    if (f.type == CCT_FILLER_GAUSSIAN && !(f.std >= 0.f && std::isfinite(f.std) && std::isfinite(f.mean)))
+      return "gaussian std must be finite and not negative";
+    if (f.type == CCT_FILLER_BERNOULLI && !(f.value >= 0.f && f.value <= 1.f))
+      return "bernoulli probability must be in [0, 1]";
+    if (f.type == CCT_FILLER_CONSTANT && !std::isfinite(f.value)) return "constant value must be finite";
+    return nullptr;
+  }
 
   // Walks the chain with the reference's size rules (conv (R+2p-K)/s+1, src/DeepNet.h:112-115;
   // pooling (R-K)/s+1, :1374-1376) and returns "" if every layer can be built, else a message that
@@ -104,16 +117,16 @@ class Network {
                              std::to_string(R + 2L * s.pad) + ")");
           const int g = s.group > 1 ? s.group : 1;
           if (D % g || s.num_output % g) return at(i, "group must divide input depth and num_output");
-          if (s.weight_filler.type < 0 || s.weight_filler.type > 3 || s.bias_filler.type < 0 || s.bias_filler.type > 3)
-            return at(i, "unknown filler type");
+          if (const char *why = bad_filler(s.weight_filler)) return at(i, std::string("weight filler: ") + why);
+          if (const char *why = bad_filler(s.bias_filler)) return at(i, std::string("bias filler: ") + why);
           R = (R + 2L * s.pad - s.kernel_size) / s.stride + 1;
           D = s.num_output;
           break;
         }
         case CCT_LAYER_FC:
           if (s.num_output <= 0) return at(i, "inner product needs num_output >= 1");
-          if (s.weight_filler.type < 0 || s.weight_filler.type > 3 || s.bias_filler.type < 0 || s.bias_filler.type > 3)
-            return at(i, "unknown filler type");
+          if (const char *why = bad_filler(s.weight_filler)) return at(i, std::string("weight filler: ") + why);
+          if (const char *why = bad_filler(s.bias_filler)) return at(i, std::string("bias filler: ") + why);
           R = 1;
           D = s.num_output;
           break;
@@ -171,6 +184,17 @@ class Network {
 
   Network(int batch, int depth, int size, const cct_layer_spec *specs, int n_specs, const cct_solver_param *sp)
       : batch_(batch) {
+    try {
+      build(depth, size, specs, n_specs, sp);
+    } catch (...) {
+      release();  // a constructor that throws runs no destructor: free what was built so far
+      throw;
+    }
+  }
+
+ private:
+  void build(int depth, int size, const cct_layer_spec *specs, int n_specs, const cct_solver_param *sp) {
+    const int batch = batch_;
     {
       const std::string why = validate(batch, depth, size, specs, n_specs, sp);
       if (!why.empty()) throw std::invalid_argument(why);
@@ -186,7 +210,8 @@ class Network {
     LayerT *const input_layer = new_layer(size, size, depth);
     blobs_[input_layer] = TensorInfo();
     for (int i = 0; i < n_specs; ++i) {
-      Node nd;
+      nodes_.emplace_back();     // in place: what the node owns is freed by release() if a bridge below throws
+      Node &nd = nodes_.back();  // (nothing else is appended to nodes_ during this iteration)
       nd.spec = specs[i];
       const cct_layer_spec &s = specs[i];
       // the tensor(s) this layer reads: the producers' layers as they are; `cur` becomes this node's
@@ -210,9 +235,16 @@ class Network {
           if (D % g || s.num_output % g) fail("group must divide input depth and num_output");
           const size_t m = (R + 2 * s.pad - s.kernel_size) / s.stride + 1;
           nd.out = new_layer(m, m, s.num_output);
-          for (int gi = 0; gi < g; ++gi) {
+          // A grouped layer whose geometry the direct kernels take is ONE bridge over the whole
+          // tensors: the kernels run every group in the same launch.  Otherwise it is `g` bridges on
+          // contiguous per-group layers, the slices gathered before and scattered after.
+          const bool one_bridge = g > 1 && driver_.conv_direct_supported(batch_, (int)D, (int)R, s.kernel_size, s.stride,
+                                                                         s.pad, s.num_output, g);
+          const int n_bridges = one_bridge ? 1 : g;
+          for (int gi = 0; gi < n_bridges; ++gi) {
             cnn::LayerParameter *lp = new_param(s);
-            lp->convolution_param_.num_output_ = s.num_output / g;
+            lp->convolution_param_.num_output_ = one_bridge ? s.num_output : s.num_output / g;
+            lp->convolution_param_.group_ = one_bridge ? g : 1;
             lp->convolution_param_.kernel_size_ = s.kernel_size;
             lp->convolution_param_.stride_ = s.stride;
             lp->convolution_param_.pad_ = s.pad;
@@ -221,22 +253,13 @@ class Network {
             set_filler(lp->convolution_param_.bias_filler_, s.bias_filler);
             nd.params.push_back(lp);
             LayerT *gin = cur, *gout = nd.out;
-            // A group works in place on its channel slices of the whole tensors when the direct
-            // kernels take the layer (they accept an image stride); otherwise the slices are
-            // gathered into contiguous per-group layers and scattered back.
-            const bool slices_in_place = g > 1 && group_in_place(R, D / g, s, s.num_output / g, m);
-            if (g > 1 && slices_in_place) {
-              const size_t din = D / g, dout = s.num_output / g;
-              gin = view_layer(cur, gi * din * R * R, R, R, din);
-              gout = view_layer(nd.out, gi * dout * m * m, m, m, dout);
-            } else if (g > 1) {
+            if (n_bridges > 1) {
               gin = new_layer(R, R, D / g);
               gout = new_layer(m, m, s.num_output / g);
               nd.group_in.push_back(gin);
               nd.group_out.push_back(gout);
             }
             auto *b = new ParallelizedBridge<float, ConvolutionBridge, HIPDriver>(gin, gout, lp, &solver_, &driver_);
-            if (slices_in_place) b->sub_bridge()->set_image_strides(D * R * R, (size_t)s.num_output * m * m);
             b->needs_to_calc_backward_grad = !first_weight_layer;
             nd.bridges.push_back(b);
           }
@@ -324,7 +347,6 @@ class Network {
       ob.params_upstream = ob.params_upstream || params_upstream || has_params;
       ob.last_writer = i;
       ob.writers.push_back(i);
-      nodes_.push_back(nd);
     }
     // Fusions that depend on who reads a tensor, decided now that every reader is known.
     for (size_t i = 0; i < nodes_.size(); ++i) {
@@ -362,14 +384,24 @@ class Network {
     }
   }
 
-  ~Network() {
+  void release() {
+    for (void *t : fwd_timers_) if (t) cct_hip_timer_destroy(t);
+    for (void *t : bwd_timers_) if (t) cct_hip_timer_destroy(t);
+    if (update_timer_) cct_hip_timer_destroy(update_timer_);
+    fwd_timers_.clear(); bwd_timers_.clear(); update_timer_ = nullptr;
     for (Node &nd : nodes_) {
       for (BridgeT *b : nd.bridges) delete b;
       for (cnn::LayerParameter *p : nd.params) delete p;
     }
+    nodes_.clear();
     for (LayerT *l : layers_) delete l;
+    layers_.clear();
     delete labels_;
+    labels_ = nullptr;
   }
+
+ public:
+  ~Network() { release(); }
   Network(const Network &) = delete;
   Network &operator=(const Network &) = delete;
 
@@ -385,9 +417,43 @@ class Network {
         static_cast<DropoutBridge<float, HIPDriver> *>(nd.bridges[0])->train = train;
   }
 
+  // Per-layer times of the passes that follow, from events on the library's stream (what the
+  // reference prints per bridge from report_forward_history / report_backward_updateweight_history,
+  // src/DeepNet.h:2190-2215, measured on the device instead of the host clock), plus the stage
+  // timing of every convolution bridge.  Off by default: an event pair per layer costs launch slots.
+  void set_profiling(bool on) {
+    profile_ = on;
+    if (on && fwd_timers_.empty()) {
+      fwd_timers_.assign(nodes_.size(), nullptr);
+      bwd_timers_.assign(nodes_.size(), nullptr);
+      ran_fwd_.assign(nodes_.size(), false);
+      ran_bwd_.assign(nodes_.size(), false);
+    }
+    for (Node &nd : nodes_)
+      if (nd.spec.type == CCT_LAYER_CONV)
+        for (BridgeT *b : nd.bridges)
+          static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(b)->sub_bridge()->set_stage_profiling(on);
+  }
+  // milliseconds of layer i's last profiled forward / backward step (0 if it did not run); waits for the step
+  float layer_ms(int i, bool backward) {
+    std::vector<void *> &t = backward ? bwd_timers_ : fwd_timers_;
+    std::vector<bool> &ran = backward ? ran_bwd_ : ran_fwd_;
+    float ms = 0.f;
+    if (i >= 0 && i < (int)t.size() && t[i] && ran[i]) cct_hip_timer_elapsed_ms(t[i], &ms);
+    return ms;
+  }
+  // milliseconds of the deferred SGD updates at the end of the last profiled backward pass
+  float update_ms() {
+    float ms = 0.f;
+    if (update_timer_ && ran_update_) cct_hip_timer_elapsed_ms(update_timer_, &ms);
+    return ms;
+  }
+
   // DeepNet::run_forward_pass: every bridge in order
   void forward() {
-    for (Node &nd : nodes_) {
+    for (size_t i = 0; i < nodes_.size(); ++i) {
+      Node &nd = nodes_[i];
+      tick(fwd_timers_, ran_fwd_, i, true);
       const size_t g = nd.group_in.size();
       for (size_t gi = 0; gi < g; ++gi)
         slice_copy(nd.group_in[gi]->p_data_cube, nd.in->p_data_cube, gi, /*gather=*/true);
@@ -395,6 +461,7 @@ class Network {
       for (BridgeT *b : nd.bridges) b->forward();
       for (size_t gi = 0; gi < g; ++gi)
         slice_copy(nd.group_out[gi]->p_data_cube, nd.out->p_data_cube, gi, /*gather=*/false);
+      tick(fwd_timers_, ran_fwd_, i, false);
     }
   }
 
@@ -405,12 +472,15 @@ class Network {
     // tensors then share one launch
     driver_.begin_deferred_sgd();
     for (auto &kv : blobs_) kv.second.summed = false;
+    if (profile_) std::fill(ran_bwd_.begin(), ran_bwd_.end(), false);
     for (int i = (int)nodes_.size() - 1; i >= 0; --i) {
       Node &nd = nodes_[i];
       if (!nd.run_backward) continue;
+      tick(bwd_timers_, ran_bwd_, i, true);
       sum_reader_gradients(nd.out);
       if (nd.spec.type == CCT_LAYER_CONCAT) {
         concat_copy(nd, /*data=*/false);
+        tick(bwd_timers_, ran_bwd_, i, false);
         continue;
       }
       const size_t g = nd.group_in.size();
@@ -420,8 +490,17 @@ class Network {
       if (nd.bridges[0]->needs_to_calc_backward_grad)
         for (size_t gi = 0; gi < g; ++gi)
           slice_copy(nd.group_in[gi]->p_gradient_cube, nd.in->p_gradient_cube, gi, /*gather=*/false);
+      tick(bwd_timers_, ran_bwd_, i, false);
+    }
+    if (profile_) {
+      if (!update_timer_) cct_hip_timer_create(&update_timer_);
+      cct_hip_timer_start(update_timer_);
     }
     driver_.flush_deferred_sgd();
+    if (profile_) {
+      cct_hip_timer_stop(update_timer_);
+      ran_update_ = true;
+    }
   }
 
   float loss() { return softmax_ ? softmax_->get_loss() : 0.f; }
@@ -512,7 +591,7 @@ class Network {
   HIPDriver driver_;
   cnn::SolverParameter solver_;
   int batch_;
-  CubeT *labels_;
+  CubeT *labels_ = nullptr;
   std::vector<LayerT *> layers_;
   std::vector<Node> nodes_;
   SoftmaxLossBridge<float, HIPDriver> *softmax_ = nullptr;
@@ -564,6 +643,21 @@ class Network {
     }
   }
 
+  bool profile_ = false, ran_update_ = false;
+  std::vector<void *> fwd_timers_, bwd_timers_;
+  std::vector<bool> ran_fwd_, ran_bwd_;
+  void *update_timer_ = nullptr;
+  void tick(std::vector<void *> &timers, std::vector<bool> &ran, size_t i, bool start) {
+    if (!profile_) return;
+    if (!timers[i]) cct_hip_timer_create(&timers[i]);
+    if (start) {
+      cct_hip_timer_start(timers[i]);
+    } else {
+      cct_hip_timer_stop(timers[i]);
+      ran[i] = true;
+    }
+  }
+
   std::string io_error_;
   bool io_fail(const std::string &msg) {
     io_error_ = msg;
@@ -593,18 +687,6 @@ class Network {
     LayerT *l = new LayerT(new CubeT(R, C, D, batch_, &driver_), new CubeT(R, C, D, batch_, &driver_));
     layers_.push_back(l);
     return l;
-  }
-  // non-owning layer over a channel slice (first element at `offset` floats) of `whole`
-  LayerT *view_layer(LayerT *whole, size_t offset, size_t R, size_t C, size_t D) {
-    LayerT *l = new LayerT(new CubeT(whole->p_data_cube->get_p_data() + offset, R, C, D, batch_),
-                           new CubeT(whole->p_gradient_cube->get_p_data() + offset, R, C, D, batch_));
-    layers_.push_back(l);
-    return l;
-  }
-  // the condition under which ConvolutionBridge picks the all-direct path on its own
-  bool group_in_place(size_t R, size_t d, const cct_layer_spec &s, size_t o, size_t m) {
-    if (!driver_.conv_direct_supported(batch_, (int)d, (int)R, s.kernel_size, s.stride, s.pad, (int)o)) return false;
-    return 2.0 * o * (double)(m * m * batch_) * (double)(s.kernel_size * s.kernel_size * d) >= kConvDirectMinFlop;
   }
   static cnn::LayerParameter *new_param(const cct_layer_spec &s) {
     cnn::LayerParameter *lp = new cnn::LayerParameter;

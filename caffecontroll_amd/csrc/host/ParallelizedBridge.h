@@ -59,9 +59,7 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
         p_grad_updater_bias(nullptr) {
     (void)_n_thread_per_partition;
     if (_n_partition != 1 || _layer_param->gpu_0_batch_proportion() != 1.0f) {
-      std::fprintf(stderr, "ParallelizedBridge: this build runs one device partition "
-                           "(n_partition=1, gpu_0_batch_proportion=1.0)\n");
-      std::abort();
+      host_fail("ParallelizedBridge: this build runs one device partition (n_partition=1, gpu_0_batch_proportion=1.0)");
     }
     // device-side layers of the sub-bridge: the caller's own, or copies this bridge owns
     LayerType *sub_in = _input_layer, *sub_out = _output_layer;
@@ -112,9 +110,7 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
     if (p_device_output_layer || share_input_output_layer || !share) {
       // going from shared to host-resident output after construction would need new device cubes
       // under a sub-bridge that already holds the old ones
-      std::fprintf(stderr, "ParallelizedBridge: share_pointer_with_next_bridge can only be raised, and only "
-                           "before the bridge owns device output cubes\n");
-      std::abort();
+      host_fail("ParallelizedBridge: share_pointer_with_next_bridge can only be raised, and only before the bridge owns device output cubes");
     }
     share_pointer_with_next_bridge = share;
   }

@@ -34,8 +34,7 @@ class ReLUBridge : public AbstractBridge<DataType, DriverClass> {
              const cnn::SolverParameter *const sp, DriverClass *const drv)
       : Base(in, out, lp, sp, drv) {
     if (oR != iR || oC != iC || oD != iD || oB != iB) {
-      std::fprintf(stderr, "ReLUBridge: input and output shapes differ\n");
-      std::abort();
+      host_fail("ReLUBridge: input and output shapes differ");
     }
   }
   // set when the producing bridge clamps at zero while it stores (in-place ReLU after a convolution)
@@ -72,8 +71,7 @@ class MaxPoolingBridge : public AbstractBridge<DataType, DriverClass> {
         stride(lp->pooling_param().stride()) {
     const size_t ph = (iR - kernel_size) / stride + 1, pw = (iC - kernel_size) / stride + 1;
     if (oR != ph || oC != pw || oD != iD || oB != iB) {
-      std::fprintf(stderr, "MaxPoolingBridge: inconsistent layer shapes\n");
-      std::abort();
+      host_fail("MaxPoolingBridge: inconsistent layer shapes");
     }
     max_index = new LogicalCube<int>(oR, oC, iD, iB, p_driver);
   }
@@ -127,8 +125,7 @@ class LRNBridge : public AbstractBridge<DataType, DriverClass> {
       : Base(in, out, lp, sp, drv), alpha(lp->lrn_param().alpha()), beta(lp->lrn_param().beta()),
         local_size(lp->lrn_param().local_size()) {
     if (oR != iR || oC != iC || oD != iD || oB != iB || local_size % 2 != 1 || alpha < 0 || beta < 0) {
-      std::fprintf(stderr, "LRNBridge: bad shapes or parameters\n");
-      std::abort();
+      host_fail("LRNBridge: bad shapes or parameters");
     }
     denoms = new LogicalCubeType(iR, iC, iD, iB, p_driver);
   }
@@ -175,8 +172,7 @@ class DropoutBridge : public AbstractBridge<DataType, DriverClass> {
                 const cnn::SolverParameter *const sp, DriverClass *const drv)
       : Base(in, out, lp, sp, drv), dropout_ratio(lp->dropout_param().dropout_ratio()), train(true) {
     if (oR != iR || oC != iC || oD != iD || oB != iB || !(dropout_ratio < 1.f) || dropout_ratio < 0.f) {
-      std::fprintf(stderr, "DropoutBridge: bad shapes or ratio\n");
-      std::abort();
+      host_fail("DropoutBridge: bad shapes or ratio");
     }
     scale = (float)(1. / (1. - dropout_ratio));
     uint_thres_ = static_cast<unsigned int>(UINT_MAX * dropout_ratio);
@@ -223,8 +219,7 @@ class SoftmaxLossBridge : public AbstractBridge<DataType, DriverClass> {
                     LogicalCubeType *const _p_data_labels)
       : Base(in, out, lp, sp, drv), p_data_labels(_p_data_labels) {
     if (oR != iR || oC != iC || oD != iD || oB != iB || _p_data_labels->n_elements != iB) {
-      std::fprintf(stderr, "SoftmaxLossBridge: bad shapes\n");
-      std::abort();
+      host_fail("SoftmaxLossBridge: bad shapes");
     }
     loss_device = new LogicalCubeType(1, 1, 1, 1, p_driver);
   }

@@ -6,6 +6,8 @@
 #include <cstdlib>
 #include <string>
 
+#include "Fail.h"
+
 namespace cct {
 
 struct Util {
@@ -39,8 +41,7 @@ struct Util {
                                         float caffe_stepsize, float power, float max_iter) {
     float rate = 0.f;
     if (!try_get_learning_rate(lr_policy, base_lr, gamma, iter, caffe_stepsize, power, max_iter, &rate)) {
-      std::fprintf(stderr, "Unknown or unsupported learning rate policy: %s\n", lr_policy.c_str());
-      std::abort();
+      host_fail("Unknown or unsupported learning rate policy: " + lr_policy);
     }
     return rate;
   }

@@ -516,7 +516,7 @@ static bool strided_plan(int batch, int d, int n, int ks, int stride, int pad, i
   if (batch <= 0 || d <= 0 || o <= 0 || pad < 0 || pad >= ks || n + 2 * pad < ks) return false;
   const int hp = n + 2 * pad, ho = (hp - ks) / stride + 1;
   // buffer loads address the tensors through 32-bit byte offsets
-  if ((double)batch * d * n * n >= 1073741824.0 || (double)batch * o * ho * ho >= 1073741824.0) return false;
+  if ((double)batch * d * n * n >= 536870912.0 || (double)batch * o * ho * ho >= 536870912.0) return false;
   pl->ks = ks; pl->s = stride;
   pl->vp = (ks + 1) / 2;
   pl->ast = (2 * pl->vp) | 1;

@@ -127,15 +127,16 @@ class HIPDriver:
         check(self.lib.cct_hip_sgemm_conv_forward(o, batch, fmap, K, _p(model), _p(lowered), _p(bias),
                                                   _p(out), int(relu)), "sgemm_conv_forward")
 
-    def conv_direct_supported(self, b, d, n, k, s, p, o):
-        return bool(self.lib.cct_hip_conv_direct_supported(b, d, n, k, s, p, o))
+    # `groups` > 1: a grouped convolution (d and o are the layer's totals), all groups in one launch
+    def conv_direct_supported(self, b, d, n, k, s, p, o, groups=1):
+        return bool(self.lib.cct_hip_conv_direct_supported_grouped(b, d, n, k, s, p, o, groups))
 
-    def conv_direct_slab_floats(self, o, d, k, for_data_gradient):
-        return int(self.lib.cct_hip_conv_direct_slab_floats(o, d, k, int(for_data_gradient)))
+    def conv_direct_slab_floats(self, o, d, k, for_data_gradient, groups=1):
+        return int(self.lib.cct_hip_conv_direct_slab_floats_grouped(o, d, k, int(for_data_gradient), groups))
 
-    def conv_direct_slabs(self, slabs, model, o, d, k, for_data_gradient):
-        check(self.lib.cct_hip_conv_direct_slabs(_p(slabs), _p(model), o, d, k, int(for_data_gradient)),
-              "conv_direct_slabs")
+    def conv_direct_slabs(self, slabs, model, o, d, k, for_data_gradient, groups=1):
+        check(self.lib.cct_hip_conv_direct_slabs_grouped(_p(slabs), _p(model), o, d, k, int(for_data_gradient),
+                                                         groups), "conv_direct_slabs")
 
     # -- strided convolution without the lowered matrix ------------------------------------------
     def conv_strided_supported(self, b, d, n, k, s, p, o):
@@ -169,25 +170,24 @@ class HIPDriver:
         check(self.lib.cct_hip_conv_strided_backward_data(_p(in_grad), _p(out_grad), _p(slabs), b, d, n, k, s, p, o),
               "conv_strided_backward_data")
 
-    def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o, in_stride=0, out_stride=0, relu=False):
-        check(self.lib.cct_hip_conv_direct_forward(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o,
-                                                   in_stride, out_stride, int(relu)), "conv_direct_forward")
+    def conv_direct_forward(self, out, inp, slabs, bias, b, d, n, k, p, o, in_stride=0, out_stride=0, relu=False,
+                            groups=1):
+        check(self.lib.cct_hip_conv_direct_forward_grouped(_p(out), _p(inp), _p(slabs), _p(bias), b, d, n, k, p, o,
+                                                           in_stride, out_stride, int(relu), groups),
+              "conv_direct_forward")
 
     def conv_direct_backward_data(self, din, dout, slabs, b, d, n, k, p, o, in_stride=0, out_stride=0,
-                                  relu_data=None):
+                                  relu_data=None, groups=1):
         """relu_data: the layer's input tensor when it is the output of an in-place ReLU; the gradient
-        then comes out already masked with (relu_data > 0)."""
-        if relu_data is not None:
-            check(self.lib.cct_hip_conv_direct_backward_data_relu(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o,
-                                                                  in_stride, out_stride, _p(relu_data)),
-                  "conv_direct_backward_data_relu")
-            return
-        check(self.lib.cct_hip_conv_direct_backward_data(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o,
-                                                         in_stride, out_stride), "conv_direct_backward_data")
+        is then stored already masked with (relu_data > 0)."""
+        check(self.lib.cct_hip_conv_direct_backward_data_grouped(_p(din), _p(dout), _p(slabs), b, d, n, k, p, o,
+                                                                 in_stride, out_stride, _p(relu_data), groups),
+              "conv_direct_backward_data")
 
-    def conv_direct_backward_weights(self, dw, dout, inp, b, d, n, k, p, o, db=None, in_stride=0, out_stride=0):
-        check(self.lib.cct_hip_conv_direct_backward_weights(_p(dw), _p(db), _p(dout), _p(inp), b, d, n, k, p, o,
-                                                            in_stride, out_stride),
+    def conv_direct_backward_weights(self, dw, dout, inp, b, d, n, k, p, o, db=None, in_stride=0, out_stride=0,
+                                     groups=1):
+        check(self.lib.cct_hip_conv_direct_backward_weights_grouped(_p(dw), _p(db), _p(dout), _p(inp), b, d, n, k,
+                                                                    p, o, in_stride, out_stride, groups),
               "conv_direct_backward_weights")
 
     def sgemv(self, TA, M, N, alpha, A, x, beta, y):

@@ -126,6 +126,12 @@ NET_PROTOTYPES = {
     "cct_net_forward": ([_P], _I),
     "cct_net_backward": ([_P], _I),
     "cct_net_loss": ([_P, C.POINTER(C.c_float)], _I),
+    "cct_net_set_profiling": ([_P, _I], _I),
+    "cct_net_layer_ms": ([_P, _I, C.POINTER(C.c_float), C.POINTER(C.c_float)], _I),
+    "cct_net_update_ms": ([_P, C.POINTER(C.c_float)], _I),
+    "cct_net_conv_bridges": ([_P, _I], _I),
+    "cct_net_conv_stage_ms": ([_P, _I, _I, C.POINTER(C.c_float)], _I),
+    "cct_net_conv_stage_kernel": ([_P, _I, _I, _I], C.c_char_p),
     "cct_net_write_model": ([_P, C.c_char_p], _I),
     "cct_net_read_model": ([_P, C.c_char_p], _I),
     "cct_net_write_snapshot": ([_P, C.c_char_p, _I], _I),
@@ -217,6 +223,36 @@ class Net:
         v = C.c_float()
         check(self.lib.cct_net_loss(self.h, C.byref(v)), "net_loss")
         return v.value
+
+    # ---- per-layer device times (the breakdown the reference prints per bridge) ----
+    def set_profiling(self, on=True):
+        check(self.lib.cct_net_set_profiling(self.h, int(on)), "net_set_profiling")
+
+    def layer_ms(self, layer):
+        """(forward ms, backward ms) of the layer's last profiled steps; waits for them."""
+        f, b = C.c_float(), C.c_float()
+        check(self.lib.cct_net_layer_ms(self.h, layer, C.byref(f), C.byref(b)), "net_layer_ms")
+        return f.value, b.value
+
+    def update_ms(self):
+        v = C.c_float()
+        check(self.lib.cct_net_update_ms(self.h, C.byref(v)), "net_update_ms")
+        return v.value
+
+    def conv_stages(self, layer):
+        """Per bridge of a convolution layer: {stage label: (ms, kernel instance)} of the last profiled pass."""
+        from .bridges import STAGE_NAMES
+        out = []
+        for bi in range(self.lib.cct_net_conv_bridges(self.h, layer)):
+            ms = (C.c_float * len(STAGE_NAMES))()
+            check(self.lib.cct_net_conv_stage_ms(self.h, layer, bi, ms), "net_conv_stage_ms")
+            ent = {}
+            for si, name in enumerate(STAGE_NAMES):
+                if ms[si] > 0:
+                    key = name if name not in ent else name + " (backward)"
+                    ent[key] = (ms[si], self.lib.cct_net_conv_stage_kernel(self.h, layer, bi, si).decode())
+            out.append(ent)
+        return out
 
     # ---- model files and snapshots in the reference's format (src/DeepNet.h:268-422) ----
     def write_model(self, path):

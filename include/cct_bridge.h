@@ -10,8 +10,9 @@
  *   gradient update on the device)   src/bridges/ParallelizedBridge_impl.hxx:508-753, 761-1141
  *   SGDGradientUpdater::update        src/algorithms/GradientUpdater.h:154-193
  * All data pointers are device pointers.  Return value: 0 on success, non-zero otherwise
- * (cct_hip_last_error() has the text).  Errors inside the C++ layer abort, as the reference's
- * asserts do.
+ * (cct_hip_last_error() has the text).  That includes failures inside the C++ layer (a HIP error
+ * in the middle of an iteration, an inconsistent layer): a C++ caller of the bridges gets the
+ * reference's abort-on-error, these entry points never end the caller's process.
  */
 #ifndef CCT_BRIDGE_H
 #define CCT_BRIDGE_H
@@ -152,7 +153,8 @@ int cct_net_num_layers(cct_net *net);
 /* Device pointer + element count of a tensor of layer `layer`, channel group `group`:
  * which = 0 model, 1 bias, 2 model gradient, 3 bias gradient, 4 output data of the layer,
  * 5 gradient w.r.t. the layer's input, 6 dropout mask (uint32) / max-pool argmax (int32),
- * 7 momentum buffer of the model, 8 momentum buffer of the bias.
+ * 7 momentum buffer of the model, 8 momentum buffer of the bias.  For a grouped convolution 0-3, 7
+ * and 8 are the group's own [o/g][d/g][k][k] / [o/g] slices.
  * Returns NULL (and *n = 0) when the layer has no such tensor. */
 void *cct_net_tensor(cct_net *net, int layer, int group, int which, size_t *n);
 int cct_net_set_train(cct_net *net, int train);
@@ -166,6 +168,21 @@ int cct_net_set_conv_path(cct_net *net, int level);
 int cct_net_forward(cct_net *net);
 int cct_net_backward(cct_net *net);   /* gradients + SGD update of every layer */
 int cct_net_loss(cct_net *net, float *loss_sum); /* batch-summed loss of the last forward (syncs) */
+/* Per-layer device times of the forward / backward passes that follow (events on the library's stream
+ * around every layer; the reference prints the same breakdown from its per-bridge reports,
+ * src/DeepNet.h:2190-2215, src/bridges/ConvolutionBridge_impl.hxx:325-366) and stage timing of every
+ * convolution bridge.  Off by default.  cct_net_layer_ms waits for the layer's step and returns the
+ * milliseconds of its last profiled forward and backward step (0 for a step that did not run; either
+ * pointer may be NULL); cct_net_update_ms the deferred SGD updates at the end of the backward pass. */
+int cct_net_set_profiling(cct_net *net, int on);
+int cct_net_layer_ms(cct_net *net, int layer, float *forward_ms, float *backward_ms);
+int cct_net_update_ms(cct_net *net, float *ms);
+/* Convolution layers: number of bridges the layer runs as (1; `group` of them for a grouped layer whose
+ * geometry the direct kernels do not take; 0 for other layer types), and per bridge what
+ * cct_conv_bridge_stage_ms / _stage_kernel return for a single bridge. */
+int cct_net_conv_bridges(cct_net *net, int layer);
+int cct_net_conv_stage_ms(cct_net *net, int layer, int bridge, float ms[CCT_CONV_STAGE_COUNT]);
+const char *cct_net_conv_stage_kernel(cct_net *net, int layer, int bridge, int stage);
 
 /* Model files and snapshots in the reference's format: raw fp32, per bridge its model then its
  * bias (DeepNet::write_model_to_file / read_model_from_file, src/DeepNet.h:328-374; the

@@ -103,7 +103,7 @@ int cct_hip_set_stream(void *hip_stream);
 /* Tuning knobs, for experiments and for tests that pin a kernel instance.  Names: "direct_tile"
  * (<map blocks><pixel blocks> of the direct convolution tile, 161 / 162 = its 16-row variant with 128 / 256
  * pixels, 0 = automatic), "direct_waves",
- * "direct_tb", "direct_nospec", "pool_plane", "gemm_nt", "gemm_tile" (-1 = automatic), "gemm_nodma" (1 = GEMM
+ * "direct_tb", "direct_nospec", "direct_splits" (step ranges of the direct weight-gradient launch, 0 = automatic), "pool_plane", "gemm_nt", "gemm_tile" (-1 = automatic), "gemm_nodma" (1 = GEMM
  * operand tiles always staged through registers).  The
  * environment variables CCT_HIP_<NAME IN CAPITALS> give the initial values; they are read once,
  * when the library initialises, never on a launch path.  No counterpart in the reference. */
@@ -114,7 +114,9 @@ const char *cct_hip_last_error(void);
 /* The kernel instance the library chose for the most recent lowering, lifting, GEMM or direct
  * convolution call: kernel name with its template arguments as a kernel trace prints them, then
  * launch-time choices (e.g. "gemm_kernel<Tile<256,128,16,2,2>,true,false> splits=26").  For
- * harnesses that label measurements with what actually ran.  No counterpart in the reference. */
+ * harnesses that label measurements with what actually ran.  Kept per host thread: the text is
+ * that of the calling thread's own last launch and stays valid until that thread's next one.  No
+ * counterpart in the reference. */
 const char *cct_hip_last_kernel(void);
 /* Number of compute units of the selected device (0 before init). */
 int cct_hip_compute_units(void);
@@ -238,6 +240,35 @@ int cct_hip_conv_direct_backward_data_relu(float *input_grad, const float *outpu
 int cct_hip_conv_direct_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
                                          const float *input, int batch, int depth, int n, int k, int padding,
                                          int num_outputs, size_t input_image_stride, size_t output_image_stride);
+/* The same five calls for a grouped convolution (`group` of cnn.proto's ConvolutionParameter; the
+ * reference builds such a layer as towers between a Split and a Concat, src/DeepNet.h:1700-1757),
+ * all groups in ONE launch: `depth` and `num_outputs` are the layer's totals, both divisible by
+ * `groups`; group q convolves channels [q*depth/groups, (q+1)*depth/groups) of the input with
+ * filters [q*num_outputs/groups, ...) of the model [num_outputs][depth/groups][k][k] (the blob
+ * layout Caffe gives a grouped layer) into the same range of output maps.  The slab buffer holds
+ * the groups' slabs one after another (cct_hip_conv_direct_slab_floats_grouped() floats in all);
+ * model_grad / bias_grad have the model's / bias's layout.  Image strides as above, for the whole
+ * tensors (0 = dense).  relu_data may be NULL (no ReLU mask).  With groups == 1 these ARE the
+ * calls above.  Per element the sums run in the same order as in one call per group on channel
+ * slices, so results are identical whenever both pick the same kernel instance and step ranges. */
+int cct_hip_conv_direct_supported_grouped(int batch, int depth, int n, int k, int stride, int padding,
+                                          int num_outputs, int groups);
+size_t cct_hip_conv_direct_slab_floats_grouped(int num_outputs, int depth, int k, int for_data_gradient,
+                                               int groups);
+int cct_hip_conv_direct_slabs_grouped(float *slabs, const float *model, int num_outputs, int depth, int k,
+                                      int for_data_gradient, int groups);
+int cct_hip_conv_direct_forward_grouped(float *output, const float *input, const float *slabs,
+                                        const float *bias, int batch, int depth, int n, int k, int padding,
+                                        int num_outputs, size_t input_image_stride, size_t output_image_stride,
+                                        int relu, int groups);
+int cct_hip_conv_direct_backward_data_grouped(float *input_grad, const float *output_grad, const float *slabs,
+                                              int batch, int depth, int n, int k, int padding, int num_outputs,
+                                              size_t input_image_stride, size_t output_image_stride,
+                                              const float *relu_data, int groups);
+int cct_hip_conv_direct_backward_weights_grouped(float *model_grad, float *bias_grad, const float *output_grad,
+                                                 const float *input, int batch, int depth, int n, int k,
+                                                 int padding, int num_outputs, size_t input_image_stride,
+                                                 size_t output_image_stride, int groups);
 /* ---- strided convolution without the lowered matrix ---------------------------------------- */
 /* The same replacement of ConvolutionBridge's lowering pipeline for strided layers: stride 4 with an
  * 11 x 11 kernel (AlexNet / CaffeNet conv1, benchmark configuration 3; the reference's "large" golden

@@ -97,4 +97,14 @@ def test_rejected_arguments():
     p = buf.ctypes.data_as(C.c_void_p)
     assert lib.cct_filler_draw_xavier(p, 4, 0, 1) != 0
     assert lib.cct_filler_draw_bernoulli(p, 4, 1.5, 1) != 0
-    assert lib.cct_filler_draw_gaussian(p, 4, 0.0, 0.0, 1) != 0
+    assert lib.cct_filler_draw_gaussian(p, 4, 0.0, -1.0, 1) != 0
+    assert lib.cct_filler_draw_gaussian(p, 4, 0.0, float("nan"), 1) != 0
+
+
+def test_gaussian_with_zero_std_is_the_mean():
+    """The reference's normal_distribution(mean, 0) yields mean + 0 * draw (src/sched/DeviceDriver_CPU.cpp:690-699):
+    a prototxt with `std: 0` gives constant weights, it does not end the process."""
+    lib = _lib.load()
+    buf = np.full(9, np.nan, np.float32)
+    assert lib.cct_filler_draw_gaussian(buf.ctypes.data_as(C.c_void_p), 9, 0.25, 0.0, 3) == 0
+    np.testing.assert_array_equal(buf, np.full(9, 0.25, np.float32))

@@ -214,6 +214,90 @@ def test_direct_kernels_on_channel_slices(oracle, shape):
     np.testing.assert_array_equal(host(d_og), og)
 
 
+GROUPED = [
+    # b, d (all groups), n, k, p, o (all groups), groups, pinned tile
+    (4, 12, 13, 3, 1, 20, 2, 11),
+    (3, 16, 27, 5, 2, 72, 2, 21),
+    (2, 15, 44, 3, 1, 36, 3, 11),     # padded rows of 46 floats: the one-image-per-step weight gradient, group by group
+    (3, 96, 27, 5, 2, 32, 2, 161),    # 48 channels per group: the data gradient runs on 16-row tiles
+    (2, 12, 9, 5, 4, 160, 4, 161),    # 40 maps per group forward (three 16-row blocks), 3 channels per group
+]
+
+
+@pytest.mark.parametrize("cfg", GROUPED, ids=lambda c: "b%d_d%d_n%d_k%d_p%d_o%d_g%d_t%d" % c)
+def test_grouped_launch_equals_per_group_launches(oracle, cfg):
+    """A grouped convolution as ONE launch per product (group index inside the grid) against one launch per
+    group on channel slices of the same tensors: with the tile and the step ranges pinned to the same
+    choice both ways, every output element sees the same sums in the same order, so the results are
+    identical bit for bit; unpinned, the one-launch form is held to the oracle run group by group."""
+    b, d, n, k, p, o, groups, tile = cfg
+    dg, og = d // groups, o // groups
+    m = n + 2 * p - k + 1
+    rng = np.random.default_rng(321 + sum(cfg))
+    x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+    og_t = rng.standard_normal((b, o, m, m)).astype(np.float32)
+    w = (rng.standard_normal((o, dg, k, k)) * 0.1).astype(np.float32)     # Caffe's blob of a grouped layer
+    bias = rng.standard_normal(o).astype(np.float32)
+    drv = driver()
+    assert drv.conv_direct_supported(b, d, n, k, 1, p, o, groups)
+    d_x, d_og, d_w, d_bias = dev(x), dev(og_t), dev(w), dev(bias)
+    in_stride, out_stride = d * n * n, o * m * m
+
+    def run_grouped():
+        sf = empty((drv.conv_direct_slab_floats(o, d, k, 0, groups),))
+        sb = empty((drv.conv_direct_slab_floats(o, d, k, 1, groups),))
+        drv.conv_direct_slabs(sf, d_w, o, d, k, 0, groups)
+        drv.conv_direct_slabs(sb, d_w, o, d, k, 1, groups)
+        out, dx, dw, db = empty((b, o, m, m)), empty((b, d, n, n)), empty((o, dg, k, k)), empty((o,))
+        out_relu, dx_relu = empty((b, o, m, m)), empty((b, d, n, n))
+        drv.conv_direct_forward(out, d_x, sf, d_bias, b, d, n, k, p, o, groups=groups)
+        drv.conv_direct_forward(out_relu, d_x, sf, d_bias, b, d, n, k, p, o, relu=True, groups=groups)
+        drv.conv_direct_backward_data(dx, d_og, sb, b, d, n, k, p, o, groups=groups)
+        drv.conv_direct_backward_data(dx_relu, d_og, sb, b, d, n, k, p, o, relu_data=d_x, groups=groups)
+        drv.conv_direct_backward_weights(dw, d_og, d_x, b, d, n, k, p, o, db=db, groups=groups)
+        return [host(t) for t in (out, dx, dw, db, out_relu, dx_relu)], host(sf), host(sb)
+
+    def run_per_group():
+        out, dx, dw, db = empty((b, o, m, m)), empty((b, d, n, n)), empty((o, dg, k, k)), empty((o,))
+        slabs_f, slabs_b = [], []
+        for gi in range(groups):
+            wg = d_w[gi * og:(gi + 1) * og].contiguous()
+            sf, sb = _slabs(wg, og, dg, k)
+            slabs_f.append(host(sf))
+            slabs_b.append(host(sb))
+            xs, ogs = d_x[:, gi * dg:(gi + 1) * dg], d_og[:, gi * og:(gi + 1) * og]
+            drv.conv_direct_forward(out[:, gi * og:(gi + 1) * og], xs, sf, d_bias[gi * og:(gi + 1) * og], b, dg, n, k, p,
+                                    og, in_stride, out_stride)
+            drv.conv_direct_backward_data(dx[:, gi * dg:(gi + 1) * dg], ogs, sb, b, dg, n, k, p, og, in_stride, out_stride)
+            drv.conv_direct_backward_weights(dw[gi * og:(gi + 1) * og], ogs, xs, b, dg, n, k, p, og,
+                                             db=db[gi * og:(gi + 1) * og], in_stride=in_stride, out_stride=out_stride)
+        return [host(t) for t in (out, dx, dw, db)], np.concatenate(slabs_f), np.concatenate(slabs_b)
+
+    with tuning("direct_tile", tile), tuning("direct_splits", 3):
+        one, sf1, sb1 = run_grouped()
+        per, sfg, sbg = run_per_group()
+    np.testing.assert_array_equal(sf1, sfg)
+    np.testing.assert_array_equal(sb1, sbg)
+    for got, want, name in zip(one[:4], per, ("output", "input gradient", "weight gradient", "bias gradient")):
+        np.testing.assert_array_equal(got, want, err_msg=name)
+    np.testing.assert_array_equal(one[4], oracle.relu_forward(one[0]))
+    np.testing.assert_array_equal(one[5], oracle.relu_backward(one[1], x))
+    # unpinned (the library's own choice of tile and step ranges for the whole launch) against the oracle
+    free, _, _ = run_grouped()
+    for gi in range(groups):
+        xs = np.ascontiguousarray(x[:, gi * dg:(gi + 1) * dg])
+        ogs = np.ascontiguousarray(og_t[:, gi * og:(gi + 1) * og])
+        wg, bg = w[gi * og:(gi + 1) * og], bias[gi * og:(gi + 1) * og]
+        ref_out, lowered = oracle.conv_forward(xs, wg, bg, k, 1, p)
+        ref_dx, ref_dw, ref_db = oracle.conv_backward(xs.shape, wg, ogs, lowered, k, 1, p)
+        assert rel_err(free[0][:, gi * og:(gi + 1) * og], ref_out) <= TOL
+        assert rel_err(free[1][:, gi * dg:(gi + 1) * dg], ref_dx) <= TOL
+        assert rel_err(free[2][gi * og:(gi + 1) * og], np.asarray(ref_dw).reshape(og, dg, k, k)) <= TOL
+        assert rel_err(free[3][gi * og:(gi + 1) * og], ref_db) <= TOL
+    np.testing.assert_array_equal(host(d_x), x)
+    np.testing.assert_array_equal(host(d_og), og_t)
+
+
 def test_direct_exact_on_small_integers(oracle):
     """Small-integer tensors make every sum exact in fp32, so the direct kernels must reproduce the
     lowering pipeline bit for bit whatever the summation order."""
@@ -287,6 +371,18 @@ def test_direct_support_matrix_and_errors():
     assert not drv.conv_direct_supported(4, 3, 62, 5, 1, 2, 10)       # padded image wider than 64
     assert not drv.conv_direct_supported(4, 3, 20, 5, 1, 5, 10)       # padding above k-1
     assert not drv.conv_direct_supported(1, 2, 3, 3, 1, 0, 2)         # 1x1 output: a tile would span 128 images
+    # tensors read through buffer descriptors (2 GiB of addressable bytes each) must stay below 2^29 floats
+    assert drv.conv_direct_supported(4660, 128, 30, 3, 1, 1, 16)
+    assert not drv.conv_direct_supported(4661, 128, 30, 3, 1, 1, 16)      # input just above 2 GiB
+    assert drv.conv_direct_supported(2330, 256, 30, 3, 1, 1, 16, 2)
+    assert not drv.conv_direct_supported(2331, 256, 30, 3, 1, 1, 16, 2)   # the same as two groups
+    assert drv.conv_strided_supported(1848, 3, 227, 11, 4, 0, 96)
+    assert not drv.conv_strided_supported(1849, 3, 227, 11, 4, 0, 96)     # output gradient of 2 GiB and more
+    assert not drv.conv_strided_backward_data_supported(1849, 3, 227, 11, 4, 0, 96)
+    # groups must divide both depths
+    assert drv.conv_direct_supported(4, 6, 13, 3, 1, 1, 8, 2)
+    assert not drv.conv_direct_supported(4, 6, 13, 3, 1, 1, 9, 2)
+    assert not drv.conv_direct_supported(4, 7, 13, 3, 1, 1, 8, 2)
     with pytest.raises(CctHipError):
         drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 62, 5, 2, 10)
     with pytest.raises(CctHipError):
@@ -349,6 +445,52 @@ def test_bridge_falls_back_where_direct_does_not_apply():
 # (8, 4 and 6 wavefronts)
 FULL_SIZE = [(256, 96, 27, 5, 2, 256), (256, 48, 27, 5, 2, 128), (256, 256, 13, 3, 1, 384),
              (256, 192, 13, 3, 1, 192), (255, 192, 13, 3, 1, 128)]
+
+
+# the grouped layers of the CaffeNet iteration at batch 256, both groups in one launch: conv2, conv4, conv5
+FULL_SIZE_GROUPED = [(256, 96, 27, 5, 2, 256, 2), (256, 384, 13, 3, 1, 384, 2), (256, 384, 13, 3, 1, 256, 2)]
+
+
+@pytest.mark.parametrize("cfg", FULL_SIZE_GROUPED, ids=lambda c: "b%d_d%d_n%d_k%d_p%d_o%d_g%d" % c)
+def test_full_size_grouped_vs_float64(cfg):
+    """CaffeNet's grouped layers at full size, every group in the same launch, against torch's float64
+    grouped convolution and its gradients."""
+    import torch
+    import torch.nn.functional as F
+    b, d, n, k, p, o, groups = cfg
+    m = n + 2 * p - k + 1
+    drv = driver()
+    g = torch.Generator(device="cuda").manual_seed(4321)
+    x = torch.randn((b, d, n, n), device="cuda", generator=g)
+    w = torch.randn((o, d // groups, k, k), device="cuda", generator=g) * 0.01
+    bias = torch.full((o,), 0.1, device="cuda")
+    og = torch.randn((b, o, m, m), device="cuda", generator=g)
+    sf = empty((drv.conv_direct_slab_floats(o, d, k, 0, groups),))
+    sb = empty((drv.conv_direct_slab_floats(o, d, k, 1, groups),))
+    drv.conv_direct_slabs(sf, w, o, d, k, 0, groups)
+    drv.conv_direct_slabs(sb, w, o, d, k, 1, groups)
+    out, dx, dw, db = empty((b, o, m, m)), empty((b, d, n, n)), empty((o, d // groups, k, k)), empty((o,))
+    drv.conv_direct_forward(out, x, sf, bias, b, d, n, k, p, o, groups=groups)
+    drv.conv_direct_backward_data(dx, og, sb, b, d, n, k, p, o, groups=groups)
+    drv.conv_direct_backward_weights(dw, og, x, b, d, n, k, p, o, db=db, groups=groups)
+    torch.cuda.synchronize()
+    db_ref = og.double().sum(dim=(0, 2, 3))
+    assert ((db.double() - db_ref).abs().max() / db_ref.abs().max()).item() <= TOL
+    worst_out = worst_dx = scale_out = scale_dx = 0.0
+    dw_ref = torch.zeros((o, d // groups, k, k), dtype=torch.float64, device="cuda")
+    wd = w.double()
+    for i in range(0, b, 32):
+        xs, gs = x[i:i + 32].double(), og[i:i + 32].double()
+        ro = F.conv2d(xs, wd, bias.double(), padding=p, groups=groups)
+        rdx = torch.nn.grad.conv2d_input(xs.shape, wd, gs, padding=p, groups=groups)
+        dw_ref += torch.nn.grad.conv2d_weight(xs, wd.shape, gs, padding=p, groups=groups)
+        worst_out = max(worst_out, (out[i:i + 32].double() - ro).abs().max().item())
+        worst_dx = max(worst_dx, (dx[i:i + 32].double() - rdx).abs().max().item())
+        scale_out = max(scale_out, ro.abs().max().item())
+        scale_dx = max(scale_dx, rdx.abs().max().item())
+    assert worst_out / scale_out <= TOL
+    assert worst_dx / scale_dx <= TOL
+    assert ((dw.double() - dw_ref).abs().max() / dw_ref.abs().max()).item() <= TOL
 
 
 @pytest.mark.parametrize("cfg", FULL_SIZE, ids=_ids)

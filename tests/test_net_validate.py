@@ -71,6 +71,24 @@ def test_bad_sizes():
         nets.validate(4, 1, 28, [])
 
 
+def test_bad_filler_parameters_are_refused_not_fatal():
+    """What the filler draws would refuse is said by the validation walk, with the layer's index: a negative or
+    non-finite gaussian std, a bernoulli probability outside [0, 1]; std 0 (constant weights in the reference) passes."""
+    def chain(**kw):
+        return [nets.conv(4, 3, **kw), nets.fc(3), nets.softmax_loss()]
+    nets.validate(2, 1, 8, chain(weight_filler=nets.filler("gaussian", std=0.0)))
+    for kw, fragment in ((dict(weight_filler=nets.filler("gaussian", std=-1.0)), "layer 0: weight filler: gaussian std"),
+                         (dict(bias_filler=nets.filler("gaussian", std=float("nan"))), "layer 0: bias filler: gaussian std"),
+                         (dict(weight_filler=nets.filler("bernoulli", value=1.5)), "bernoulli probability"),
+                         (dict(bias_filler=nets.filler("constant", value=float("inf"))), "constant value")):
+        with pytest.raises(CctHipError) as e:
+            nets.validate(2, 1, 8, chain(**kw))
+        assert fragment in str(e.value)
+    with pytest.raises(CctHipError, match="layer 1: weight filler"):
+        nets.validate(2, 1, 8, [nets.conv(4, 3), nets.fc(3, weight_filler=nets.filler("bernoulli", value=-0.1)),
+                                nets.softmax_loss()])
+
+
 def test_net_create_refuses_before_touching_a_device():
     """cct_net_create runs the same check first: on this path nothing device-side is reached, so
     the call is safe (and meaningful) on a machine without a GPU."""
