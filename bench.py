@@ -8,6 +8,12 @@ out-grad remap, data-gradient GEMM, lift + bias gradient, weight-gradient GEMM) 
 are already resident in HBM.  Prints ONE JSON line.
 
     python bench.py --gpus 1 --steps 20 --warmup 5
+
+`value` is the images/sec of that layer.  The same line carries, outside `value`, the other half of
+the headline metric -- `iterations`: ms per LeNet (batch 64) and per AlexNet-shaped CaffeNet (batch 256)
+training iteration, each with a whole-iteration roofline, its per-layer times and a CPU baseline of the
+same chain -- and `configs`: the stage lines of the LeNet conv1 and AlexNet conv1 layers
+(`--headline-only` leaves both out).  `--workload <name>` prints any one of them as a line of its own.
 """
 import argparse
 import json
@@ -27,38 +33,68 @@ CONFIGS = {
 }
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch (fetched + written) at the alexnet_conv2 and alexnet_conv1 shapes, from rocprofv3 --pmc FETCH_SIZE
-# and WRITE_SIZE runs of this file (one counter per run), each scaled by what the same counter
-# reads for a 1 GiB device copy (factors 2.000 and 1.000).  Not measured by this run: the record
-# names the summary under profiles/ the figure comes from.  Keyed by (stage, the kernel instance
-# the library reports it launched), so that a change of tile choice leaves `traffic` null instead
-# of attaching an old figure to another kernel.
-TRAFFIC_SOURCE = {"direct": "profiles/conv2_fwd_bwd_hbm_traffic_and_mfma.md",
-                  "lowering": "profiles/conv2_lowering_path_hbm_traffic_and_mfma.md",
-                  "conv1": "profiles/conv1_fwd_bwd_trace_traffic_mfma.md"}
-TRAFFIC_BYTES = {
-    ("GEMM", "conv_direct_kernel<5,1,2,1,32>"): ((238.5 + 230.6) * 1e6, "direct"),
-    ("GEMM Data", "conv_direct_kernel<5,1,2,1,32>"): ((320.6 + 76.2) * 1e6, "direct"),
-    ("GEMM Wghts", "conv_direct_wgrad_spec_kernel<5,5,32,27,8>"): ((359.6 + 41.8) * 1e6, "direct"),
-    ("GEMM", "gemm_kernel<Tile<256,128,16,2,2>,true,true,true> splits=1"): ((1985.7 + 201.4) * 1e6, "lowering"),
-    ("GEMM Data", "gemm_kernel<Tile<128,128,16,2,2>,false,false,true> splits=1"): ((1172.9 + 1791.6) * 1e6, "lowering"),
-    ("GEMM Wghts", "gemm_kernel<Tile<256,128,16,2,2>,true,false,true> splits=26"): ((2384.4 + 63.9) * 1e6, "lowering"),
-    ("Lower Cube", "lower_kernel threads=512"): ((75.6 + 1791.6) * 1e6, "lowering"),
-    ("Inverse Lwr", "lift_kernel<5,1> bias_blocks=256"): ((2190.6 + 71.7) * 1e6, "lowering"),
-    # alexnet_conv1 (the kernel instances differ from every conv2 one, so the keys cannot collide)
-    ("GEMM", "conv_strided_reg_kernel<11,4,3>"): ((160.8 + 302.6) * 1e6, "conv1"),
-    ("GEMM Data", "conv_direct16_kernel<3,3,1,64>"): ((301.2 + 158.6) * 1e6, "conv1"),
-    ("GEMM Wghts", "conv_strided_wgrad_spec_kernel<11,4,3,14,8,11> waves=3x4"): ((469.4 + 54.2) * 1e6, "conv1"),
-}
+# HBM bytes per launch (fetched + written) come from the committed counter summaries under profiles/
+# (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this file, one counter per run, each scaled by what
+# the same counter reads for a 1 GiB device copy): the tables are parsed, not copied.  Not measured by
+# this run: the record names the summary the figure comes from.  A row is looked up by the kernel
+# instance the library reports it launched, so a change of tile choice leaves `traffic` null instead of
+# attaching an old figure to another kernel.
+TRAFFIC_SOURCE = {("alexnet_conv2", "direct"): "profiles/conv2_fwd_bwd_hbm_traffic_and_mfma.md",
+                  ("alexnet_conv2", "lowering"): "profiles/conv2_lowering_path_hbm_traffic_and_mfma.md",
+                  ("alexnet_conv1", "direct"): "profiles/conv1_fwd_bwd_trace_traffic_mfma.md",
+                  ("caffenet", "direct"): "profiles/caffenet_iteration_kernel_trace.md",
+                  ("lenet", "direct"): "profiles/lenet_iteration_kernel_trace.md"}
+# which launches of a kernel a stage means, where a summary lists one kernel's launches by role
+STAGE_ROLE = {"GEMM": "forward", "GEMM Data": "data-gradient", "GEMM Wghts": "weight-gradient"}
 
 
-def traffic_of(cfg, stage, kernel):
-    """(bytes, source file) from the committed counter summaries, or (None, None) when the kernel
-    instance that ran is not the one that was profiled."""
-    if cfg not in ("alexnet_conv2", "alexnet_conv1"):
+def _squash(name):
+    return "".join(name.split())
+
+
+def parse_traffic_table(path):
+    """{(kernel instance without blanks, role or ""): fetched + written bytes per dispatch} from the markdown
+    tables of a counter summary (columns `kernel`, `fetched MB`, `written MB`)."""
+    out = {}
+    try:
+        lines = open(os.path.join(ROOT, path)).read().splitlines()
+    except OSError:
+        return out
+    cols = None
+    for line in lines:
+        if not line.startswith("|"):
+            cols = None
+            continue
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if cols is None:
+            cols = cells if "kernel" in cells and "fetched MB" in cells and "written MB" in cells else None
+            continue
+        if set(cells[0]) <= set("-: "):
+            continue
+        name = cells[0].strip("`")
+        role = ""
+        if name.endswith(")") and " (" in name:
+            name, role = name[:name.rindex(" (")], name[name.rindex(" (") + 2:-1].split()[0]
+        try:
+            nbytes = (float(cells[cols.index("fetched MB")]) + float(cells[cols.index("written MB")])) * 1e6
+        except ValueError:
+            continue
+        out[(_squash(name), role)] = nbytes
+    return out
+
+
+def traffic_of(workload, path_kind, stage, kernel):
+    """(bytes, source file) for the kernel instance that ran, or (None, None) when the committed summary of this
+    workload has no row for it."""
+    source = TRAFFIC_SOURCE.get((workload, path_kind))
+    if not source or not kernel:
         return None, None
-    ent = TRAFFIC_BYTES.get((stage, kernel))
-    return (ent[0], TRAFFIC_SOURCE[ent[1]]) if ent else (None, None)
+    table = parse_traffic_table(source)
+    name = _squash(kernel.split(" ")[0])
+    for key in ((name, STAGE_ROLE.get(stage, "")), (name, "")):
+        if key in table:
+            return table[key], source
+    return None, None
 
 
 def synth(cfg, seed, torch):
@@ -82,6 +118,24 @@ def synth(cfg, seed, torch):
     return x, w, bias, og
 
 
+def host_cores():
+    """Host cores this process may use (the box's share, not what the machine has)."""
+    cores = os.cpu_count() or 1
+    try:
+        cores = min(cores, len(os.sched_getaffinity(0)))
+    except Exception:
+        pass
+    if os.environ.get("OMP_NUM_THREADS", "").isdigit():
+        cores = min(cores, int(os.environ["OMP_NUM_THREADS"]))
+    return max(cores, 1)
+
+
+def cct_partitions(cores, batch):
+    """DeepNet::get_hw_concurrency (src/DeepNet.h:716-725): the largest power of two not above the hardware
+    threads, capped by the batch (src/DeepNet.h:1102-1105)."""
+    return min(2 ** int(math.floor(math.log2(max(cores, 1)))), batch)
+
+
 def cpu_baseline(cfg, seed):
     """The CPU oracle (a port of CcT's CPUDriver path, GEMMs through OpenBLAS when found) timed on
     this host with CcT's own threading policy: P = min(2^floor(log2 cores), b) batch partitions,
@@ -90,14 +144,8 @@ def cpu_baseline(cfg, seed):
     import numpy as np
     from oracle import cct_oracle as O
     b, d, n, k, s, p, o = CONFIGS[cfg]
-    cores = os.cpu_count() or 1
-    try:
-        cores = min(cores, len(os.sched_getaffinity(0)))
-    except Exception:
-        pass
-    if os.environ.get("OMP_NUM_THREADS", "").isdigit():
-        cores = min(cores, int(os.environ["OMP_NUM_THREADS"]))
-    P = min(2 ** int(math.floor(math.log2(max(cores, 1)))), b)
+    cores = host_cores()
+    P = cct_partitions(cores, b)
     blas = O.bind_openblas(1)
     x, w, bias, og = synth(cfg, seed, None)
     bounds = [(i * b // P, (i + 1) * b // P) for i in range(P)]
@@ -191,13 +239,89 @@ def net_workload(workload):
 FIRST_LOSS_PER_IMAGE = {"caffenet": 6.914681, "lenet": 2.291778}
 
 
-def net_iteration(args, torch, np):
+def net_flop(wl):
+    """Algorithmic FLOP of one training iteration: 2 * outputs * contraction per GEMM-shaped product, three
+    products per weight layer (forward, data gradient, weight gradient), two for the first weight layer, which
+    computes no data gradient (src/DeepNet.h:1108-1110).  Returns (total, {layer index: FLOP per product})."""
+    from caffecontroll_amd import nets
+    d, n, first, total, per_layer = wl["D"], wl["S"], True, 0.0, {}
+    for li, L in enumerate(wl["layers"]):
+        if L.type == nets.CONV:
+            m = (n + 2 * L.pad - L.kernel_size) // L.stride + 1
+            f = 2.0 * L.num_output * wl["B"] * m * m * L.kernel_size ** 2 * (d // max(L.group, 1))
+            d, n = L.num_output, m
+        elif L.type == nets.FC:
+            f = 2.0 * L.num_output * wl["B"] * d * n * n
+            d, n = L.num_output, 1
+        elif L.type == nets.MAXPOOL:
+            n = (n - L.kernel_size) // L.stride + 1
+            continue
+        else:
+            continue
+        per_layer[li] = f
+        total += f * (2 if first else 3)
+        first = False
+    return total, per_layer
+
+
+LAYER_TYPE_NAMES = {1: "conv", 2: "fc", 3: "relu", 4: "maxpool", 5: "lrn", 6: "dropout", 7: "softmax_loss", 8: "concat"}
+
+
+def net_cpu_baseline(workload):
+    """One training iteration of the same chain on the CPU oracle with CcT's threading policy (src/DeepNet.h:716-725,
+    1102-1105, 1165-1167, 1397): convolution, pooling, LRN, ReLU and dropout cut into P = min(2^floor(log2 cores),
+    batch) batch partitions with one BLAS thread each, inner-product layers as one partition on P/2 BLAS threads."""
+    import numpy as np
+    from oracle import cct_oracle as O
+    from oracle.oracle_net import OracleNet
+    from caffecontroll_amd import nets
+    wl = net_workload(workload)
+    B, layers = wl["B"], wl["layers"]
+    cores = host_cores()
+    P = cct_partitions(cores, B)
+    blas = O.bind_openblas(1)
+    sv = wl["solver"]
+    ref = OracleNet(O, layers, B, wl["D"], wl["S"],
+                    dict(base_lr=sv["base_lr"], momentum=sv["momentum"], weight_decay=sv["weight_decay"]),
+                    partitions=P, fc_blas_threads=max(P // 2, 1) if blas else 0)
+    for key, (w, bias) in wl["params"].items():
+        ref.params[key]["w"][...] = w.reshape(ref.params[key]["w"].shape)
+        ref.params[key]["b"][...] = bias
+    rng = np.random.default_rng(5)
+    d, n = wl["D"], wl["S"]
+    for li, (dd, nn) in enumerate(ref.shapes):
+        if layers[li].type == nets.DROPOUT:
+            ref.masks[li] = rng.integers(0, 2 ** 32, B * dd * nn * nn, dtype=np.uint64).astype(np.uint32)
+
+    def run():
+        t0 = time.perf_counter()
+        ref.forward(wl["x"], wl["labels"])
+        ref.backward()
+        return time.perf_counter() - t0
+
+    warm = run()   # also pays the first touch of the lowered matrices
+    reps = max(1, min(10 if workload == "lenet" else 2, int(15.0 / max(warm, 1e-3))))
+    times = sorted(run() for _ in range(reps))
+    med = times[len(times) // 2]
+    if blas:
+        O.unbind_openblas()
+    return {"value": med * 1e3, "unit": "ms", "images_per_sec": B / med, "cores": P, "kind": "port",
+            "sample": "one full %s training iteration (batch %d): 1 warm-up + %d timed, median; %d batch partitions x 1 "
+                      "BLAS thread for convolution / pooling / LRN / ReLU / dropout, inner-product layers on %d BLAS "
+                      "threads; sgemm=%s" % (workload, B, reps, P, max(P // 2, 1),
+                                             "OpenBLAS (scipy bundle)" if blas else "plain loops")}
+
+
+def net_iteration(args, torch, np, workload=None, steps=None, warmup=None, with_cpu=True):
     """benchmark configurations 4 and 5: one step = forward + backward + SGD update of every layer,
     synthetic images and labels already on the device."""
     from caffecontroll_amd import HIPDriver, nets
+    workload = workload or args.workload
+    steps = steps or args.steps
+    warmup = args.warmup if warmup is None else warmup
     drv = HIPDriver(0)
     drv.set_stream(torch.cuda.current_stream().cuda_stream)
-    wl = net_workload(args.workload)
+    wl = net_workload(workload)
     B, D, S, classes, layers, x, labels = (wl[k] for k in ("B", "D", "S", "classes", "layers", "x", "labels"))
     rng = np.random.default_rng(99)
     net = nets.Net(B, D, S, layers, nets.solver_param(**wl["solver"]))
@@ -214,21 +338,21 @@ def net_iteration(args, torch, np):
     net.forward()
     first_loss = net.loss() / B
     net.set_train(True)
-    want = FIRST_LOSS_PER_IMAGE[args.workload]
+    want = FIRST_LOSS_PER_IMAGE[workload]
     if not abs(first_loss - want) <= 1e-3 * want:
         raise SystemExit("bench.py: first-pass loss per image %.5f differs from the oracle's %.5f" % (first_loss, want))
 
     pipeline = None
-    if args.input_pipeline:
+    if args.input_pipeline and workload == args.workload:
         # Raw 256x256 byte images in host memory stand in for the LMDB records; every step the
         # loader copies one batch into pinned staging, uploads it on its copy stream while the
         # previous iteration computes, and the transform kernel (mean, random crop, mirror, scale)
         # writes the network's input.
         from caffecontroll_amd import corpus
-        H = 256 if args.workload == "caffenet" else S
+        H = 256 if workload == "caffenet" else S
         crop = S if H != S else 0
-        mean = rng.uniform(100, 125, (D, H, H)).astype(np.float32) if args.workload == "caffenet" else None
-        scale = 1.0 if args.workload == "caffenet" else 0.00390625
+        mean = rng.uniform(100, 125, (D, H, H)).astype(np.float32) if workload == "caffenet" else None
+        scale = 1.0 if workload == "caffenet" else 0.00390625
         cp = corpus.Corpus.create(B, D, H, H, crop_size=crop, scale=scale, mirror=crop > 0, phase=0, mean=mean, seed=1)
         pool = [(rng.integers(0, 256, (B, D, H, H), dtype=np.uint8), rng.integers(0, classes, B).astype(np.float32))
                 for _ in range(2)]
@@ -270,81 +394,95 @@ def net_iteration(args, torch, np):
         if pipeline is not None:
             feed()
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     loss = net.loss() / B
-    ms = elapsed * 1e3 / args.steps
-    return {
-        "metric": "ms per %s train iteration (1 GPU)" % ("LeNet" if args.workload == "lenet" else "AlexNet-shaped"),
-        "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+    ms = elapsed * 1e3 / steps
+
+    # A few more iterations with per-layer events on the library's stream (outside the timed region): where
+    # the iteration's time goes, and the product kernel the iteration waits for longest.
+    total_flop, layer_flop = net_flop(wl)
+    prof_steps = 5 if workload == "caffenet" else 20
+    net.set_profiling(True)
+    layer_ms = [[0.0, 0.0] for _ in layers]
+    stage_ms, stage_kernel, update_ms = {}, {}, 0.0
+    for it in range(prof_steps + 1):
+        net.forward()
+        net.backward()
+        if it == 0:
+            continue   # the first profiled pass creates the events
+        for li in range(len(layers)):
+            f, b_ = net.layer_ms(li)
+            layer_ms[li][0] += f
+            layer_ms[li][1] += b_
+            if layers[li].type == nets.CONV:
+                for bi, ent in enumerate(net.conv_stages(li)):
+                    for name, (t, kern) in ent.items():
+                        stage_ms[(li, bi, name)] = stage_ms.get((li, bi, name), 0.0) + t
+                        stage_kernel[(li, bi, name)] = kern
+        update_ms += net.update_ms()
+    net.set_profiling(False)
+    per_layer = []
+    for li, L in enumerate(layers):
+        f, b_ = layer_ms[li][0] / prof_steps, layer_ms[li][1] / prof_steps
+        if f <= 0 and b_ <= 0:
+            continue   # in-place layers folded into their neighbours' stores
+        ent = {"layer": li, "type": LAYER_TYPE_NAMES.get(L.type, str(L.type)), "forward_ms": round(f, 4),
+               "backward_ms": round(b_, 4)}
+        if li in layer_flop:
+            ent["flop_per_product"] = layer_flop[li]
+        per_layer.append(ent)
+    products = []
+    for (li, bi, name), t in stage_ms.items():
+        if name not in STAGE_ROLE:
+            continue
+        t /= prof_steps
+        flop = layer_flop[li] / max(len([k for k in stage_ms if k[0] == li and k[2] == name]), 1)
+        products.append({"layer": li, "stage": name, "kernel": stage_kernel[(li, bi, name)], "ms": round(t, 4),
+                         "tflops": round(flop / t / 1e9, 2), "frac": round(flop / t / 1e9 / PEAK_FP32_MFMA_TFLOPS, 4),
+                         "flop_per_launch": flop})
+    products.sort(key=lambda e: -e["ms"])
+    dom = products[0] if products else None
+    traffic, source = traffic_of(workload, "direct", dom["stage"], dom["kernel"]) if dom else (None, None)
+    achieved = total_flop / ms / 1e9
+    result = {
+        "metric": "ms per %s train iteration (1 GPU)" % ("LeNet" if workload == "lenet" else "AlexNet-shaped"),
+        "value": round(ms, 4), "unit": "ms", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic", "images_per_sec": round(B * 1e3 / ms, 1),
         "config": {"workload": "%s: fwd+bwd+SGD, batch %d, %dx%dx%d inputs, %d classes%s" % (
-            args.workload, B, D, S, S, classes, ", conv2/4/5 in 2 groups" if args.workload == "caffenet" else "")},
+            workload, B, D, S, S, classes, ", conv2/4/5 in 2 groups" if workload == "caffenet" else "")},
         "first_loss_per_image": round(float(first_loss), 5), "oracle_first_loss_per_image": want,
         "final_loss_per_image": round(float(loss), 5),
+        # whole iteration against the fp32 matrix peak: every FLOP of the iteration's GEMM-shaped products over the
+        # wall time of the iteration (element-wise layers, SGD and launch gaps count as lost time); `dominant` is the
+        # product kernel with the longest average launch, priced on its own algorithmic FLOP
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "flop_per_iteration": total_flop,
+                     "traffic": traffic, "traffic_source": source,
+                     "dominant": dom, "scope": "whole iteration"},
+        "layers": per_layer, "sgd_update_ms": round(update_ms / prof_steps, 4),
+        "conv_products": products,
         **({"input_pipeline": pipeline} if pipeline is not None else {}),
     }
+    net.close()
+    del net
+    if with_cpu and not args.no_cpu_baseline:
+        result["cpu_baseline"] = net_cpu_baseline(workload)
+    return result
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="alexnet_conv2", choices=sorted(CONFIGS) + ["lenet", "caffenet"],
-                    help="a single conv layer (default: AlexNet conv2, the headline config) or a whole training "
-                         "iteration of LeNet (b=64) / CaffeNet (b=256, grouped conv2/4/5)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--input-pipeline", action="store_true",
-                    help="lenet/caffenet: feed every iteration through the input pipeline (raw bytes in host memory "
-                         "-> pinned staging -> asynchronous upload -> transform kernel)")
-    ap.add_argument("--unfused", action="store_true", help="staged forward (GEMM, remap, bias) and separate bias gradient")
-    ap.add_argument("--path", type=int, default=-1, choices=[-1, 0, 1, 2, 3],
-                    help="conv path level: 0 separate passes, 1 fused epilogues, 2 direct data gradient, 3 all "
-                         "direct kernels (no lowered matrix); -1 = the bridge's default")
-    ap.add_argument("--no-lowering-path", action="store_true",
-                    help="skip the extra passes at path level 1 that report the lowering / lifting stages")
-    ap.add_argument("--no-data-grad", action="store_true", help="first-layer mode: skip data-gradient GEMM and lift")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="only run 5 device-to-device copies of 1 GiB (a plain copy kernel of known size, used "
-                         "to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters) and exit")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on ONE GPU (batch sharding over several GPUs is a design note, "
-              "not built); run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
-
-    import numpy as np
-    import torch
-    from caffecontroll_amd import HIPDriver, load
+def conv_layer(args, cfg, torch, np, steps, warmup, with_lowering=True, with_cpu=True):
+    """One of the single-layer configurations: `steps` timed passes of ConvolutionBridge forward + backward on tensors
+    resident in HBM; returns the record (headline fields, per-stage times, rooflines, CPU baseline)."""
+    from caffecontroll_amd import HIPDriver
     from caffecontroll_amd.bridges import ConvolutionLayer
-
-    load()
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(3)
-    if args.copy_calibration:
-        drv = HIPDriver(0)
-        nbytes = 1 << 30
-        src = torch.ones(nbytes // 4, device="cuda")
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            drv.memcpy(dst, src, nbytes, 2)
-        drv.device_sync()
-        print(json.dumps({"copy_calibration_bytes_read": nbytes, "copy_calibration_bytes_written": nbytes,
-                          "copies": 5}))
-        return
-    if args.workload in ("lenet", "caffenet"):
-        print(json.dumps(net_iteration(args, torch, np)))
-        return
-    cfg = args.workload
     b, d, n, k, s, p, o = CONFIGS[cfg]
     m = (n + 2 * p - k) // s + 1
     seed = 1234 + sorted(CONFIGS).index(cfg)
@@ -407,15 +545,14 @@ def main():
             per_stage[name] = ent
         return path, elapsed, per_stage
 
-    path, elapsed, per_stage = run_path(0 if args.unfused else (None if args.path < 0 else args.path),
-                                        args.steps, args.warmup)
-    ms_per_step = elapsed * 1e3 / args.steps
+    path, elapsed, per_stage = run_path(0 if args.unfused else (None if args.path < 0 else args.path), steps, warmup)
+    ms_per_step = elapsed * 1e3 / steps
 
     def mfma_roofline(stages):
         # dominant kernel = the product kernel with the longest average launch
         dom = max((g for g in ("GEMM", "GEMM Data", "GEMM Wghts") if g in stages), key=lambda g: stages[g]["ms"])
         ent = stages[dom]
-        traffic, source = traffic_of(cfg, dom, ent["kernel"])
+        traffic, source = traffic_of(cfg, "direct" if path >= 2 and stages is per_stage else "lowering", dom, ent["kernel"])
         return {"bound": "mfma", "achieved": ent["tflops"], "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": ent["frac_fp32_mfma_peak"], "traffic": traffic, "traffic_source": source,
                 "kernel": ent["kernel"], "stage": dom, "flop_per_launch": gemm_flop, "avg_launch_ms": ent["ms"]}
@@ -427,14 +564,14 @@ def main():
             return None
         worst = min(names, key=lambda g: stages[g]["frac_hbm_peak"])
         ent = stages[worst]
-        traffic, source = traffic_of(cfg, worst, ent["kernel"])
+        traffic, source = traffic_of(cfg, "lowering", worst, ent["kernel"])
         return {"bound": "hbm", "achieved": ent["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": ent["frac_hbm_peak"], "traffic": traffic, "traffic_source": source, "kernel": ent["kernel"],
                 "stage": worst, "bytes_per_launch": ent["algorithmic_bytes"], "avg_launch_ms": ent["ms"]}
 
     result = {
-        "metric": "images/sec conv fwd+bwd (1 GPU)", "value": round(b * args.steps / elapsed, 1),
-        "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "metric": "images/sec conv fwd+bwd (1 GPU)", "value": round(b * steps / elapsed, 1),
+        "unit": "images/sec", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: conv fwd+bwd b=%d d=%d n=%d k=%d s=%d p=%d o=%d%s%s" % (
@@ -444,18 +581,87 @@ def main():
     }
     if hbm_roofline(per_stage):
         result["roofline_hbm"] = hbm_roofline(per_stage)
-    elif not args.no_lowering_path:
+    elif with_lowering:
         # The same layer once more through the reference's stage sequence (lower, GEMM, remap, GEMM,
         # lift, GEMM; path level 1), outside `value`: per-stage times of the lowering path and the
         # HBM-bound lowering / lifting kernels against the 8 TB/s roofline.
-        _, low_elapsed, low_stages = run_path(1, max(3, min(args.steps, 10)), 2)
+        _, low_elapsed, low_stages = run_path(1, max(3, min(steps, 10)), 2)
         result["stages_lowering_path"] = low_stages
-        result["lowering_path_ms_per_step"] = round(low_elapsed * 1e3 / max(3, min(args.steps, 10)), 4)
+        result["lowering_path_ms_per_step"] = round(low_elapsed * 1e3 / max(3, min(steps, 10)), 4)
         result["roofline_hbm"] = hbm_roofline(low_stages)
         result["roofline_mfma_lowering_path"] = mfma_roofline(low_stages)
-    if not args.no_cpu_baseline:
-        del in_data, in_grad, out_data, out_grad
+    if with_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg, seed)
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="alexnet_conv2", choices=sorted(CONFIGS) + ["lenet", "caffenet"],
+                    help="a single conv layer (default: AlexNet conv2, the headline config) or a whole training "
+                         "iteration of LeNet (b=64) / CaffeNet (b=256, grouped conv2/4/5)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="alexnet_conv2 only: leave out the `iterations` (LeNet, CaffeNet) and `configs` (LeNet conv1, "
+                         "AlexNet conv1) records that the default line carries beside the headline")
+    ap.add_argument("--input-pipeline", action="store_true",
+                    help="lenet/caffenet: feed every iteration through the input pipeline (raw bytes in host memory "
+                         "-> pinned staging -> asynchronous upload -> transform kernel)")
+    ap.add_argument("--unfused", action="store_true", help="staged forward (GEMM, remap, bias) and separate bias gradient")
+    ap.add_argument("--path", type=int, default=-1, choices=[-1, 0, 1, 2, 3],
+                    help="conv path level: 0 separate passes, 1 fused epilogues, 2 direct data gradient, 3 all "
+                         "direct kernels (no lowered matrix); -1 = the bridge's default")
+    ap.add_argument("--no-lowering-path", action="store_true",
+                    help="skip the extra passes at path level 1 that report the lowering / lifting stages")
+    ap.add_argument("--no-data-grad", action="store_true", help="first-layer mode: skip data-gradient GEMM and lift")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run 5 device-to-device copies of 1 GiB (a plain copy kernel of known size, used "
+                         "to scale rocprofv3's FETCH_SIZE / WRITE_SIZE counters) and exit")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on ONE GPU (batch sharding over several GPUs is a design note, "
+              "not built); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from caffecontroll_amd import HIPDriver, load
+    from caffecontroll_amd.bridges import ConvolutionLayer
+
+    load()
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    if args.copy_calibration:
+        drv = HIPDriver(0)
+        nbytes = 1 << 30
+        src = torch.ones(nbytes // 4, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            drv.memcpy(dst, src, nbytes, 2)
+        drv.device_sync()
+        print(json.dumps({"copy_calibration_bytes_read": nbytes, "copy_calibration_bytes_written": nbytes,
+                          "copies": 5}))
+        return
+    if args.workload in ("lenet", "caffenet"):
+        print(json.dumps(net_iteration(args, torch, np)))
+        return
+    result = conv_layer(args, args.workload, torch, np, args.steps, args.warmup,
+                        with_lowering=not args.no_lowering_path, with_cpu=not args.no_cpu_baseline)
+    extras = args.workload == "alexnet_conv2" and not args.headline_only and args.path < 0 and not args.unfused \
+        and not args.no_data_grad
+    if extras:
+        # the other half of the headline metric and the remaining single-layer configurations, outside `value`
+        result["configs"] = {
+            cfg: conv_layer(args, cfg, torch, np, 50 if cfg == "lenet_conv1" else args.steps, args.warmup,
+                            with_lowering=not args.no_lowering_path, with_cpu=not args.no_cpu_baseline)
+            for cfg in ("lenet_conv1", "alexnet_conv1")}
+        result["iterations"] = {
+            "lenet": net_iteration(args, torch, np, workload="lenet", steps=200, warmup=20),
+            "caffenet": net_iteration(args, torch, np, workload="caffenet", steps=max(args.steps, 10), warmup=5)}
     print(json.dumps(result))
 
 

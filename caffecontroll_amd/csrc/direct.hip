@@ -1333,8 +1333,7 @@ static int wgrad_launch_spec(const WgradArgs &g, const WgradPlan &pl, hipStream_
   if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;
   hipLaunchKernelGGL(kern, dim3(g.nblocks), dim3(64 * W * WN), pl.lds, st, g);
   CCT_LAUNCH_CHECK();
-  if (WN == 1) note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d>", KS, TB, PW, HO, W);
-  else note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d,%d>", KS, TB, PW, HO, W, WN);
+  note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d,%d>", KS, TB, PW, HO, W, WN);
   return 0;
 }
 

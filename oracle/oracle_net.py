@@ -1,7 +1,10 @@
 """CPU reference of a layer chain, composed from the oracle's per-layer functions in the order
 DeepNet::run_forward_pass / run_backward_pass visit the bridges (src/DeepNet.h:171-266): ReLU and
 dropout in place, the first weight layer without a data gradient, grouped convolutions as
-independent convolutions on channel slices, one SGD update per weight layer per iteration."""
+independent convolutions on channel slices, one SGD update per weight layer per iteration.
+
+TEST INFRASTRUCTURE ONLY, like the rest of this folder: the parity tests compare the device against
+it, and the `cpu_baseline` leg of bench.py times it."""
 from concurrent.futures import ThreadPoolExecutor
 
 import numpy as np
@@ -10,13 +13,19 @@ CONV, FC, RELU, MAXPOOL, LRN, DROPOUT, SOFTMAXLOSS, CONCAT = 1, 2, 3, 4, 5, 6, 7
 
 
 class OracleNet:
-    def __init__(self, O, layers, batch, depth, size, solver, partitions=1):
+    def __init__(self, O, layers, batch, depth, size, solver, partitions=1, fc_blas_threads=0):
         """solver: dict(base_lr, momentum, weight_decay); fixed learning-rate policy.
         partitions > 1: convolutions run the way the reference's ParallelizedBridge runs them on a
         CPU, the batch cut into that many contiguous partitions, one thread each, the partitions'
         weight and bias gradients added up in partition order
-        (src/bridges/ParallelizedBridge_impl.hxx:888-955)."""
+        (src/bridges/ParallelizedBridge_impl.hxx:888-955); pooling, LRN, ReLU and dropout are cut the
+        same way (src/DeepNet.h:1397, 1455, 1516, 1842: per-image work, so the values do not depend on
+        the cut).
+        fc_blas_threads > 0 (needs OpenBLAS bound): the reference's policy for inner-product layers,
+        ONE partition whose GEMMs use that many BLAS threads (src/DeepNet.h:1165-1167, half the
+        hardware threads), while every partitioned layer runs one BLAS thread per partition."""
         self.O, self.layers, self.solver = O, layers, solver
+        self.fc_blas_threads = fc_blas_threads
         self.partitions = max(1, min(partitions, batch))
         self.bounds = [(i * batch // self.partitions, (i + 1) * batch // self.partitions)
                        for i in range(self.partitions)]
@@ -51,6 +60,23 @@ class OracleNet:
         self.masks = {}
         self.train = True   # False: dropout layers pass their input through (TEST phase)
 
+    def _blas(self, for_fc):
+        if self.fc_blas_threads > 0:
+            self.O.bind_openblas(self.fc_blas_threads if for_fc else 1)
+
+    def _cut(self, fn, *arrays):
+        """fn(*slices) per batch partition, one thread each; returns the list of results (one entry when
+        the net is not partitioned).  Every array has the batch as its first axis."""
+        if self.partitions == 1:
+            return [fn(*arrays)]
+        with ThreadPoolExecutor(self.partitions) as ex:
+            return list(ex.map(lambda lh: fn(*[a[lh[0]:lh[1]] for a in arrays]), self.bounds))
+
+    @staticmethod
+    def _join(parts, k=None):
+        parts = [q if k is None else q[k] for q in parts]
+        return parts[0] if len(parts) == 1 else np.concatenate(parts, axis=0)
+
     def forward(self, x, labels):
         O = self.O
         self.acts = [x]
@@ -58,6 +84,7 @@ class OracleNet:
         cur = x
         for i, L in enumerate(self.layers):
             if L.type == CONV:
+                self._blas(False)
                 g = max(L.group, 1)
                 dg = cur.shape[1] // g
                 outs = []
@@ -76,23 +103,30 @@ class OracleNet:
                     outs.append(out)
                 cur = np.concatenate(outs, axis=1) if g > 1 else outs[0]
             elif L.type == FC:
+                self._blas(True)
                 p = self.params[(i, 0)]
                 self.saved[(i, 0)] = cur.reshape(cur.shape[0], -1).copy()
                 cur = O.fc_forward(self.saved[(i, 0)], p["w"], p["b"]).reshape(cur.shape[0], L.num_output, 1, 1)
             elif L.type == RELU:
-                cur = O.relu_forward(cur)
+                cur = self._join(self._cut(O.relu_forward, cur))
                 self.acts[-1] = cur  # in place: the layer below now holds the rectified values
             elif L.type == MAXPOOL:
                 self.saved[i] = cur.shape
-                cur, idx = O.maxpool_forward(cur, L.kernel_size, L.stride)
+                parts = self._cut(lambda a: O.maxpool_forward(np.ascontiguousarray(a), L.kernel_size, L.stride), cur)
+                cur, idx = self._join(parts, 0), self._join(parts, 1)
                 self.saved[(i, "idx")] = idx
             elif L.type == LRN:
                 self.saved[i] = cur
-                cur, den = O.lrn_forward(cur, L.lrn_local_size, L.lrn_alpha, L.lrn_beta)
+                parts = self._cut(lambda a: O.lrn_forward(np.ascontiguousarray(a), L.lrn_local_size, L.lrn_alpha,
+                                                          L.lrn_beta), cur)
+                cur, den = self._join(parts, 0), self._join(parts, 1)
                 self.saved[(i, "den")] = den
             elif L.type == DROPOUT:
                 if self.train:
-                    cur = O.dropout_forward(cur, self.masks[i], L.dropout_ratio, threshold=True)
+                    mask = np.asarray(self.masks[i]).reshape(cur.shape)
+                    cur = self._join(self._cut(
+                        lambda a, mk: O.dropout_forward(np.ascontiguousarray(a), np.ascontiguousarray(mk).reshape(-1),
+                                                        L.dropout_ratio, threshold=True).reshape(a.shape), cur, mask))
                 self.acts[-1] = cur
             elif L.type == SOFTMAXLOSS:
                 cur, self.loss = O.softmax_loss_forward(cur, labels)
@@ -115,18 +149,27 @@ class OracleNet:
                 grad = O.softmax_loss_backward(self.acts[ai], self.labels)
                 ai -= 1
             elif L.type == RELU:
-                grad = O.relu_backward(grad, self.acts[ai])
+                grad = self._join(self._cut(lambda gq, a: O.relu_backward(np.ascontiguousarray(gq), np.ascontiguousarray(a)),
+                                            grad, self.acts[ai].reshape(grad.shape)))
             elif L.type == DROPOUT:
-                grad = O.dropout_forward(grad, self.masks[i], L.dropout_ratio, threshold=True)
+                mask = np.asarray(self.masks[i]).reshape(grad.shape)
+                grad = self._join(self._cut(
+                    lambda a, mk: O.dropout_forward(np.ascontiguousarray(a), np.ascontiguousarray(mk).reshape(-1),
+                                                    L.dropout_ratio, threshold=True).reshape(a.shape), grad, mask))
             elif L.type == MAXPOOL:
                 shp = self.saved[i]
-                grad = O.maxpool_backward(grad, self.saved[(i, "idx")], shp[2], shp[3])
+                grad = self._join(self._cut(
+                    lambda gq, ix: O.maxpool_backward(np.ascontiguousarray(gq), np.ascontiguousarray(ix), shp[2], shp[3]),
+                    grad, self.saved[(i, "idx")]))
                 ai -= 1
             elif L.type == LRN:
-                grad = O.lrn_backward(grad, self.saved[i], self.saved[(i, "den")], L.lrn_local_size,
-                                      L.lrn_alpha, L.lrn_beta)
+                grad = self._join(self._cut(
+                    lambda gq, a, dn: O.lrn_backward(np.ascontiguousarray(gq), np.ascontiguousarray(a),
+                                                     np.ascontiguousarray(dn), L.lrn_local_size, L.lrn_alpha, L.lrn_beta),
+                    grad, self.saved[i], self.saved[(i, "den")]))
                 ai -= 1
             elif L.type == FC:
+                self._blas(True)
                 p = self.params[(i, 0)]
                 need = i != self.first_weight
                 xin = self.saved[(i, 0)]
@@ -136,6 +179,7 @@ class OracleNet:
                 grad = dx.reshape(self.acts[ai - 1].shape) if need else None
                 ai -= 1
             elif L.type == CONV:
+                self._blas(False)
                 g = max(L.group, 1)
                 need = i != self.first_weight
                 og_d = grad.shape[1] // g

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from gpu_util import driver, rel_err
-from oracle_net import OracleGraph
+from oracle.oracle_net import OracleGraph
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 from gpu_util import driver, rel_err
-from oracle_net import OracleNet
+from oracle.oracle_net import OracleNet
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4

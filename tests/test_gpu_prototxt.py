@@ -237,7 +237,7 @@ def test_prototxt_network_trains_like_the_oracle(oracle, text, solver_text, dept
     layer's output, every gradient and every updated weight agree within 1e-4."""
     from caffecontroll_amd import nets, prototxt as P
     from gpu_util import rel_err
-    from oracle_net import OracleGraph
+    from oracle.oracle_net import OracleGraph
     sp, _ = P.solver_from_prototxt(solver_text)
     nd = P.network_from_prototxt(text)
     driver()

@@ -218,7 +218,7 @@ def test_random_layer_chains_train_like_the_oracle(oracle, seed):
     (default, all direct, direct data gradient, staged passes): every layer's output, the loss, every
     gradient and every updated parameter against the oracle chain."""
     from caffecontroll_amd import nets
-    from oracle_net import OracleNet
+    from oracle.oracle_net import OracleNet
     import test_gpu_nets as T
     driver()
     rng = np.random.default_rng(seed)
@@ -262,7 +262,7 @@ def test_random_tower_graphs_train_like_the_oracle(oracle, seed):
     CONCAT, classifier): one training iteration on a random convolution path level against the
     oracle graph.  Weights are scaled by their fan-in so that the loss gradient is well conditioned."""
     from caffecontroll_amd import nets
-    from oracle_net import OracleGraph
+    from oracle.oracle_net import OracleGraph
     import test_gpu_nets as T
     driver()
     rng = np.random.default_rng(seed)
