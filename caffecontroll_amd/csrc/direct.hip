@@ -570,6 +570,12 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   // blocks x 128 pixels; 6, 4, 3, 2 for 256 pixels); a wrong figure costs speed, not correctness.
   static const int reg_slots[5][3] = {{0, 0, 0}, {0, 8, 6}, {0, 7, 4}, {0, 5, 3}, {0, 4, 2}};
   static const double fill[4] = {1.0, 0.7, 0.93, 0.97};  // MFMA rate with 1, 2, 3 workgroups on a unit
+  // MFMA rate of an instance on a launch of many balanced rounds, relative to the best instance of its
+  // kernel size (measured on the CaffeNet layers at batch 256: conv3 / conv4 for k = 3, conv2 for k = 5).
+  // 64 x 128 and 32 x 256 tiles lead; 64 x 256 and the three- and four-block map tiles hold fewer
+  // wavefronts per SIMD and lose 6-15 %.
+  static const double rate3[5][3] = {{0, 0, 0}, {0, 0.965, 0.985}, {0, 1.0, 0.94}, {0, 0.895, 0.85}, {0, 0.91, 0.935}};
+  static const double rate5[5][3] = {{0, 0, 0}, {0, 0.977, 1.0}, {0, 0.987, 0.925}, {0, 0.98, 0.96}, {0, 0.85, 0.913}};
   struct Candidate { DirectPlan plan; double cost; } cand[8];
   int ncand = 0;
   double best = -1;
@@ -591,8 +597,9 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
       const long full = tiles / (cus * slots), rest = tiles - full * cus * slots;
       const long last = (rest + cus - 1) / cus;
       const double work = tmb * tnb;
-      const double cost = full * slots * work / (slots < 4 ? fill[slots] : 1.0) +
-                          last * work / (last < 4 ? fill[last] : 1.0);
+      const double cost = (full * slots * work / (slots < 4 ? fill[slots] : 1.0) +
+                           last * work / (last < 4 ? fill[last] : 1.0)) /
+                          (ks == 3 ? rate3[tmb][tnb] : rate5[tmb][tnb]);
       Candidate &c = cand[ncand++];
       c.plan.ks = ks; c.plan.tmb = tmb; c.plan.tnb = tnb; c.plan.cp = cp; c.plan.pw = pw; c.plan.pr = pr;
       c.plan.lds = lds;
@@ -601,15 +608,10 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
     }
   }
   if (ncand == 0) return false;
-  // the estimate is good to a few percent: among the candidates that close to the best, the wider
-  // pixel tile (measured a little faster at equal balance), then the lower estimate
   const Candidate *pick = nullptr;
-  for (int i = 0; i < ncand; ++i) {
-    if (cand[i].cost > best * 1.025) continue;
-    if (!pick || cand[i].plan.tnb > pick->plan.tnb ||
-        (cand[i].plan.tnb == pick->plan.tnb && cand[i].cost < pick->cost))
-      pick = &cand[i];
-  }
+  for (int i = 0; i < ncand; ++i)
+    if (!pick || cand[i].cost < pick->cost) pick = &cand[i];
+  (void)best;
   *pl = pick->plan;
   pl->tm16 = 0;
   return true;
