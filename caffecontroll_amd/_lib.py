@@ -82,6 +82,9 @@ PROTOTYPES = {
     "cct_hip_sgemm_new": [_I, _I, _I, _I, _I, _F, _P, _P, _F, _P],
     "cct_hip_sgemm_new_bias": [_I, _I, _I, _I, _I, _F, _P, _P, _F, _P, _P, _I],
     "cct_hip_sgemm_conv_forward": [_I, _I, _I, _I, _P, _P, _P, _P, _I],
+    "cct_hip_fc_small_supported": [_I, _I, _I],
+    "cct_hip_fc_small_forward": [_P, _P, _P, _P, _I, _I, _I, _I],
+    "cct_hip_fc_small_backward": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
     "cct_hip_conv_direct_supported": [_I, _I, _I, _I, _I, _I, _I],
     "cct_hip_conv_direct_slab_floats": [_I, _I, _I, _I],
     "cct_hip_conv_direct_slabs": [_P, _P, _I, _I, _I, _I],
@@ -134,6 +137,7 @@ PROTOTYPES = {
     "cct_hip_dropout_forward_train": [_P, _P, _P, _F, _U, _Z],
     "cct_hip_softmax_loss_forward": [_P, _P, _P, _P, _I, _I],
     "cct_hip_softmax_loss_backward": [_P, _P, _P, _I, _I, _I],
+    "cct_hip_softmax_loss_forward_backward": [_P, _P, _P, _P, _P, _I, _I, _I],
     "cct_hip_timer_create": [C.POINTER(_P)],
     "cct_hip_timer_destroy": [_P],
     "cct_hip_timer_start": [_P],

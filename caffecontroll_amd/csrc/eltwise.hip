@@ -795,9 +795,12 @@ __global__ __launch_bounds__(TPB) void rand_uint_kernel(unsigned int *__restrict
 }
 
 // ---- softmax loss: one workgroup per image ----------------------------------------------------------
+// Probabilities, the image's loss and, if asked, the input gradient (prob - onehot) * factor of the backward
+// pass in the same launch; the batch sum of the losses follows in softmax_loss_sum_kernel.
 __global__ __launch_bounds__(TPB) void softmax_fwd_kernel(float *__restrict__ prob, const float *__restrict__ in,
                                                           const float *__restrict__ labels,
-                                                          float *__restrict__ loss_per_image, int len) {
+                                                          float *__restrict__ loss_per_image, int len,
+                                                          float *__restrict__ in_grad, double factor) {
   __shared__ float scratch[8];
   const int ib = blockIdx.x, tid = threadIdx.x;
   const float *x = in + (size_t)ib * len;
@@ -808,14 +811,18 @@ __global__ __launch_bounds__(TPB) void softmax_fwd_kernel(float *__restrict__ pr
   float s = 0.0f;
   for (int i = tid; i < len; i += TPB) s += expf(x[i] - mx);
   s = block_reduce<false>(s, scratch);
-  for (int i = tid; i < len; i += TPB) y[i] = expf(x[i] - mx) / s;
-  __syncthreads();
-  if (tid == 0) {
-    // a label outside [0, len) (NaN included) is never used as an index: the image's loss is NaN
-    const float lf = labels[ib];
-    const bool valid = lf >= 0.0f && lf < (float)len;
-    loss_per_image[ib] = valid ? -logf(fmaxf(y[(int)lf], FLT_MIN)) : __int_as_float(0x7fc00000);
+  // a label outside [0, len) (NaN included) is never used as an index: the image's loss is NaN and the
+  // gradient subtracts no 1
+  const float lf = labels[ib];
+  const bool valid = lf >= 0.0f && lf < (float)len;
+  const int label = valid ? (int)lf : -1;
+  for (int i = tid; i < len; i += TPB) {
+    const float pv = expf(x[i] - mx) / s;
+    y[i] = pv;
+    if (in_grad) in_grad[(size_t)ib * len + i] = (float)((double)(i == label ? pv - 1.0f : pv) * factor);
+    if (i == label) loss_per_image[ib] = -logf(fmaxf(pv, FLT_MIN));
   }
+  if (!valid && tid == 0) loss_per_image[ib] = __int_as_float(0x7fc00000);
 }
 // batch sum in ascending image order (the order the reference accumulates its scalar loss): the
 // workgroup fetches the per-image losses TPB at a time, coalesced, and lane 0 adds them up in order
@@ -834,6 +841,50 @@ __global__ __launch_bounds__(TPB) void softmax_loss_sum_kernel(float *__restrict
     __syncthreads();
   }
   if (threadIdx.x == 0) *loss_sum = s;
+}
+// The whole batch in ONE workgroup of sixteen wavefronts, for problems of a few thousand scores (LeNet: 64
+// images x 10 classes), where the launches cost more than the arithmetic: wavefront w takes images w, w + 16, ...; a lane takes
+// classes lane, lane + 64, ... of the scores staged in LDS; maximum and sum by shuffle trees; the per-image losses meet in LDS and
+// lane 0 adds them in ascending image order, as softmax_loss_sum_kernel does.  Same values as the
+// two-launch form for at most 64 classes (one class per lane: the sum of exponentials is the same shuffle
+// tree over the same lanes), equal to rounding beyond.
+constexpr int kSoftmaxSmallBatch = 1024, kSoftmaxSmallScores = 8192, kSoftmaxSmallThreads = 1024;
+__global__ __launch_bounds__(kSoftmaxSmallThreads) void softmax_loss_small_kernel(
+    float *__restrict__ prob, const float *__restrict__ in, const float *__restrict__ labels, int len, int batch,
+    float *__restrict__ in_grad, double factor, float *__restrict__ loss_sum) {
+  __shared__ float xs[kSoftmaxSmallScores];   // all scores, fetched once, coalesced: the per-image passes read LDS
+  __shared__ float loss_of[kSoftmaxSmallBatch];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < batch * len; i += kSoftmaxSmallThreads) xs[i] = in[i];
+  __syncthreads();
+  for (int ib = wave; ib < batch; ib += kSoftmaxSmallThreads / 64) {
+    const float *x = xs + ib * len;
+    float *y = prob + (size_t)ib * len;
+    float mx = -FLT_MAX;
+    for (int i = lane; i < len; i += 64) mx = fmaxf(mx, x[i]);
+    mx = wave_max_f(mx);
+    mx = __shfl(mx, 0, 64);
+    float s = 0.0f;
+    for (int i = lane; i < len; i += 64) s += expf(x[i] - mx);
+    s = wave_sum_f(s);
+    s = __shfl(s, 0, 64);
+    const float lf = labels[ib];
+    const bool valid = lf >= 0.0f && lf < (float)len;
+    const int label = valid ? (int)lf : -1;
+    for (int i = lane; i < len; i += 64) {
+      const float pv = expf(x[i] - mx) / s;
+      y[i] = pv;
+      if (in_grad) in_grad[(size_t)ib * len + i] = (float)((double)(i == label ? pv - 1.0f : pv) * factor);
+      if (i == label) loss_of[ib] = -logf(fmaxf(pv, FLT_MIN));
+    }
+    if (!valid && lane == 0) loss_of[ib] = __int_as_float(0x7fc00000);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float total = 0.0f;
+    for (int j = 0; j < batch; ++j) total += loss_of[j];
+    *loss_sum = total;
+  }
 }
 __global__ __launch_bounds__(TPB) void softmax_bwd_kernel(float *__restrict__ ig, const float *__restrict__ prob,
                                                           const float *__restrict__ labels, int len,
@@ -1299,23 +1350,43 @@ int cct_hip_rand_uint_initialize(unsigned int *buf, int n) {
   return 0;
 }
 
-int cct_hip_softmax_loss_forward(float *prob, const float *in, const float *labels, float *loss_sum,
-                                 int len_per_image, int batch) {
-  CCT_ENSURE_INIT();
-  CCT_REQUIRE(prob && in && labels && loss_sum, "softmax_loss_forward: null argument");
-  CCT_REQUIRE(len_per_image > 0 && batch >= 0, "softmax_loss_forward: bad sizes");
+static int softmax_loss_launch(float *prob, const float *in, const float *labels, float *loss_sum, float *in_grad,
+                               int len_per_image, int batch, int spatial, const char *what) {
+  CCT_REQUIRE(prob && in && labels && loss_sum, "%s: null argument", what);
+  CCT_REQUIRE(len_per_image > 0 && batch >= 0 && spatial > 0, "%s: bad sizes", what);
+  CCT_REQUIRE((size_t)len_per_image * (size_t)(batch > 0 ? batch : 1) < (1ull << 31), "%s: tensor too large", what);
+  const double factor = 1. / (double)(batch > 0 ? batch : 1) / (double)spatial;
+  if (batch > 0 && batch <= kSoftmaxSmallBatch && (size_t)batch * len_per_image <= (size_t)kSoftmaxSmallScores) {
+    hipLaunchKernelGGL(softmax_loss_small_kernel, dim3(1), dim3(kSoftmaxSmallThreads), 0, ctx().stream, prob, in, labels, len_per_image,
+                       batch, in_grad, factor, loss_sum);
+    CCT_LAUNCH_CHECK();
+    return 0;
+  }
   void *ws = nullptr;
   int rc = get_workspace((size_t)(batch > 0 ? batch : 1) * sizeof(float), &ws);
   if (rc) return rc;
   if (batch > 0) {
-    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(batch), dim3(TPB), 0, ctx().stream, prob, in, labels,
-                       (float *)ws, len_per_image);
+    hipLaunchKernelGGL(softmax_fwd_kernel, dim3(batch), dim3(TPB), 0, ctx().stream, prob, in, labels, (float *)ws,
+                       len_per_image, in_grad, factor);
     CCT_LAUNCH_CHECK();
   }
-  hipLaunchKernelGGL(softmax_loss_sum_kernel, dim3(1), dim3(TPB), 0, ctx().stream, loss_sum, (const float *)ws,
-                     batch);
+  hipLaunchKernelGGL(softmax_loss_sum_kernel, dim3(1), dim3(TPB), 0, ctx().stream, loss_sum, (const float *)ws, batch);
   CCT_LAUNCH_CHECK();
   return 0;
+}
+
+int cct_hip_softmax_loss_forward(float *prob, const float *in, const float *labels, float *loss_sum,
+                                 int len_per_image, int batch) {
+  CCT_ENSURE_INIT();
+  return softmax_loss_launch(prob, in, labels, loss_sum, nullptr, len_per_image, batch, 1, "softmax_loss_forward");
+}
+
+int cct_hip_softmax_loss_forward_backward(float *prob, float *in_grad, const float *in, const float *labels,
+                                          float *loss_sum, int len_per_image, int batch, int spatial) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(in_grad, "softmax_loss_forward_backward: null gradient");
+  return softmax_loss_launch(prob, in, labels, loss_sum, in_grad, len_per_image, batch, spatial,
+                             "softmax_loss_forward_backward");
 }
 
 int cct_hip_softmax_loss_backward(float *in_grad, const float *prob, const float *labels, int len_per_image,

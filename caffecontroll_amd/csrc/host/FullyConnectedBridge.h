@@ -56,6 +56,8 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
     data_C = (int)(iR * iC * iD);     // its columns (features in)
     model_R = (int)oD;                // rows of the model matrix (features out)
     model_C = data_C;
+    // a handful of outputs: one launch per pass instead of GEMM + split-K reduction + bias passes
+    small_ = p_driver->fc_small_supported(data_R, data_C, model_R);
   }
 
   ~FullyConnectedBridge() {
@@ -75,10 +77,23 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
   // that directly follows (set_fuse_relu), ride on the GEMM's output pass -- the same sums in the
   // same order, two or three launches fewer per layer.
   void set_fuse_relu(bool on) { fuse_relu_ = on; }
+  // The input layer is the output of an in-place ReLU whose backward this bridge performs on the input
+  // gradient it produces (the ReLU bridge then skips its own): masked in the store of the small-layer
+  // kernel, else by a pass after the data-gradient GEMM.  Only meaningful with needs_to_calc_backward_grad.
+  bool input_is_relu_output = false;
+  // false: always the three GEMMs (what tests compare the one-launch kernels with)
+  void set_small_kernels(bool on) { small_ = on && p_driver->fc_small_supported(data_R, data_C, model_R); }
+  bool small_kernels() const { return small_; }
   void forward() override {
     this->report_forward_history.reset();
     LogicalCubeType *input_d_cube = p_input_layer->p_data_cube;
     LogicalCubeType *output_d_cube = p_output_layer->p_data_cube;
+    if (small_) {
+      p_driver->fc_small_forward(output_d_cube->get_p_data(), input_d_cube->get_p_data(), p_model_cube->get_p_data(),
+                                 bias_term ? p_bias_cube->get_p_data() : nullptr, data_R, data_C, model_R, fuse_relu_);
+      this->report_forward_history.end();
+      return;
+    }
     p_driver->sgemm_new_bias(CblasNoTrans, CblasTrans, data_R, model_R, model_C, 1.f, input_d_cube->get_p_data(),
                              p_model_cube->get_p_data(), 0.f, output_d_cube->get_p_data(),
                              bias_term ? p_bias_cube->get_p_data() : nullptr, fuse_relu_);
@@ -91,6 +106,16 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
     LogicalCubeType *output_g_cube = p_output_layer->p_gradient_cube;
     LogicalCubeType *input_g_cube = p_input_layer->p_gradient_cube;
     LogicalCubeType *input_d_cube = p_input_layer->p_data_cube;
+    if (small_) {
+      p_driver->fc_small_backward(needs_to_calc_backward_grad ? input_g_cube->get_p_data() : nullptr,
+                                  p_model_gradient_cube->get_p_data(),
+                                  bias_term ? p_bias_gradient_cube->get_p_data() : nullptr, output_g_cube->get_p_data(),
+                                  input_d_cube->get_p_data(), p_model_cube->get_p_data(), data_R, data_C, model_R,
+                                  needs_to_calc_backward_grad && input_is_relu_output ? input_d_cube->get_p_data()
+                                                                                      : nullptr);
+      this->report_backward_updateweight_history.end();
+      return;
+    }
     if (bias_term) {
       DeviceMemoryPointer output = output_g_cube->get_device_pointer(p_driver);
       DeviceMemoryPointer bias = p_bias_gradient_cube->get_device_pointer(p_driver);
@@ -98,9 +123,14 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
     }
     // the reference always computes the data gradient here (:306-308); it is skipped when the
     // caller says the layer below does not need it
-    if (needs_to_calc_backward_grad)
+    if (needs_to_calc_backward_grad) {
       p_driver->sgemm_new(CblasNoTrans, CblasNoTrans, data_R, model_C, model_R, 1.f, output_g_cube->get_p_data(),
                           p_model_cube->get_p_data(), 0.f, input_g_cube->get_p_data());
+      if (input_is_relu_output) {  // the GEMM has no store to fold the mask into
+        DeviceMemoryPointer in_grad = input_g_cube->get_device_pointer(p_driver);
+        p_driver->relu_backward(&in_grad, &in_grad, input_d_cube->get_p_data());
+      }
+    }
     p_driver->sgemm_new(CblasTrans, CblasNoTrans, model_R, model_C, data_R, 1.f, output_g_cube->get_p_data(),
                         input_d_cube->get_p_data(), 0.f, p_model_gradient_cube->get_p_data());
     this->report_backward_updateweight_history.end();
@@ -110,7 +140,7 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
   LogicalCubeType *p_model_gradient_cube;
   LogicalCubeType *p_bias_gradient_cube;
   int data_R, data_C, model_R, model_C;
-  bool fuse_relu_ = false;
+  bool fuse_relu_ = false, small_ = false;
 
   void initialize_logical_cube(const LogicalCubeType *cube, const cnn::FillerParameter &filler_param) {
     DeviceMemoryPointer data = cube->get_device_pointer(p_driver);

@@ -155,6 +155,12 @@ class HIPDriver {
                             int len_per_image, int batch) {
     ok(cct_hip_softmax_loss_forward(prob, in, labels, loss_sum, len_per_image, batch), "softmax_loss_forward");
   }
+  // forward and backward in one launch (a training iteration asks for both)
+  void softmax_loss_forward_backward(float *prob, float *in_grad, const float *in, const float *labels,
+                                     float *loss_sum, int len_per_image, int batch, int spatial) {
+    ok(cct_hip_softmax_loss_forward_backward(prob, in_grad, in, labels, loss_sum, len_per_image, batch, spatial),
+       "softmax_loss_forward_backward");
+  }
   void softmax_loss_backward(float *in_grad, const float *prob, const float *labels, int len_per_image,
                              int batch, int spatial) {
     ok(cct_hip_softmax_loss_backward(in_grad, prob, labels, len_per_image, batch, spatial),
@@ -236,6 +242,19 @@ class HIPDriver {
     ok(cct_hip_sgemm_conv_forward(o, batch, fmap, K, model, lowered, bias, out, relu ? 1 : 0), "sgemm_conv_forward");
   }
   // ---- stride-1 convolution without the lowered matrix (no counterpart in DeviceDriver.h) ----
+  // ---- inner-product layers with few outputs (no counterpart in DeviceDriver.h) ----
+  bool fc_small_supported(int batch, int in_features, int out_features) {
+    return cct_hip_fc_small_supported(batch, in_features, out_features) != 0;
+  }
+  void fc_small_forward(float *y, const float *x, const float *w, const float *bias, int batch, int in_features,
+                        int out_features, bool relu) {
+    ok(cct_hip_fc_small_forward(y, x, w, bias, batch, in_features, out_features, relu ? 1 : 0), "fc_small_forward");
+  }
+  void fc_small_backward(float *dx, float *dw, float *db, const float *dy, const float *x, const float *w, int batch,
+                         int in_features, int out_features, const float *relu_data) {
+    ok(cct_hip_fc_small_backward(dx, dw, db, dy, x, w, batch, in_features, out_features, relu_data),
+       "fc_small_backward");
+  }
   // `groups` > 1: a grouped convolution (depth and num_outputs are the layer's totals), all groups in one launch
   bool conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs,
                              int groups = 1) {

@@ -329,6 +329,8 @@ class Network {
           nd.out = new_layer(R, R, D);
           nd.params.push_back(new_param(s));
           softmax_ = new SoftmaxLossBridge<float, HIPDriver>(cur, nd.out, nd.params[0], &solver_, &driver_, labels_);
+          softmax_node_runs_backward_ = params_upstream;
+          softmax_->gradient_with_forward = params_upstream;  // chains start in the TRAIN phase
           nd.bridges.push_back(softmax_);
           break;
         }
@@ -351,7 +353,13 @@ class Network {
     // Fusions that depend on who reads a tensor, decided now that every reader is known.
     for (size_t i = 0; i < nodes_.size(); ++i) {
       Node &nd = nodes_[i];
-      if (nd.spec.type != CCT_LAYER_CONV && nd.spec.type != CCT_LAYER_MAXPOOL) continue;
+      if (nd.spec.type == CCT_LAYER_FC) {
+        // an inner-product layer of few outputs masks its input gradient in its one backward launch
+        auto *fb = static_cast<ParallelizedBridge<float, FullyConnectedBridge, HIPDriver> *>(nd.bridges[0])->sub_bridge();
+        if (!fb->small_kernels()) continue;
+      } else if (nd.spec.type != CCT_LAYER_CONV && nd.spec.type != CCT_LAYER_MAXPOOL) {
+        continue;
+      }
       const cct_layer_spec &s = nd.spec;
       LayerT *bottom = s.n_bottoms ? (s.bottoms[0] < 0 ? layers_[0] : nodes_[s.bottoms[0]].out)
                                    : (i == 0 ? layers_[0] : nodes_[i - 1].out);
@@ -369,6 +377,8 @@ class Network {
         if (nd.spec.type == CCT_LAYER_CONV)
           for (BridgeT *cb : nd.bridges)
             static_cast<ParallelizedBridge<float, ConvolutionBridge, HIPDriver> *>(cb)->sub_bridge()->input_is_relu_output = true;
+        else if (nd.spec.type == CCT_LAYER_FC)
+          static_cast<ParallelizedBridge<float, FullyConnectedBridge, HIPDriver> *>(nd.bridges[0])->sub_bridge()->input_is_relu_output = true;
         else
           static_cast<MaxPoolingBridge<float, HIPDriver> *>(nd.bridges[0])->input_is_relu_output = true;
         static_cast<ReLUBridge<float, HIPDriver> *>(nodes_[writer].bridges[0])->backward_done_by_consumer = true;
@@ -415,6 +425,9 @@ class Network {
     for (Node &nd : nodes_)
       if (nd.spec.type == CCT_LAYER_DROPOUT)
         static_cast<DropoutBridge<float, HIPDriver> *>(nd.bridges[0])->train = train;
+    // TRAIN phase: every forward pass is followed by a backward pass, so the loss layer writes its
+    // gradient in the launch that computes the probabilities (if anything upstream wants one)
+    if (softmax_) softmax_->gradient_with_forward = train && softmax_node_runs_backward_;
   }
 
   // Per-layer times of the passes that follow, from events on the library's stream (what the
@@ -595,6 +608,7 @@ class Network {
   std::vector<LayerT *> layers_;
   std::vector<Node> nodes_;
   SoftmaxLossBridge<float, HIPDriver> *softmax_ = nullptr;
+  bool softmax_node_runs_backward_ = false;
 
   // What the network knows about a tensor (a Layer that some node produced, or the input).
   struct TensorInfo {

@@ -224,14 +224,32 @@ class SoftmaxLossBridge : public AbstractBridge<DataType, DriverClass> {
     loss_device = new LogicalCubeType(1, 1, 1, 1, p_driver);
   }
   ~SoftmaxLossBridge() { delete loss_device; }
+  // Training: forward() also writes the input gradient (the launch that computes the probabilities holds
+  // everything the gradient needs), and the backward() that follows it has nothing left to do.  Set by the
+  // owner of the chain when every forward pass is followed by a backward pass; a backward() without a
+  // forward() since the last one computes the gradient from the stored probabilities as usual.
+  bool gradient_with_forward = false;
   // probabilities go to the output layer's data cube; the batch-summed loss stays on the device
   void forward() override {
+    if (gradient_with_forward) {
+      p_driver->softmax_loss_forward_backward(p_output_layer->p_data_cube->get_p_data(),
+                                              p_input_layer->p_gradient_cube->get_p_data(),
+                                              p_input_layer->p_data_cube->get_p_data(), p_data_labels->get_p_data(),
+                                              loss_device->get_p_data(), (int)(iR * iC * iD), (int)iB, (int)(iR * iC));
+      gradient_is_current_ = true;
+      return;
+    }
     p_driver->softmax_loss_forward(p_output_layer->p_data_cube->get_p_data(), p_input_layer->p_data_cube->get_p_data(),
                                    p_data_labels->get_p_data(), loss_device->get_p_data(), (int)(iR * iC * iD),
                                    (int)iB);
+    gradient_is_current_ = false;
   }
   // input gradient = (prob - onehot) / B / (R*C), from the probabilities stored by forward()
   void backward() override {
+    if (gradient_is_current_) {
+      gradient_is_current_ = false;
+      return;
+    }
     p_driver->softmax_loss_backward(p_input_layer->p_gradient_cube->get_p_data(),
                                     p_output_layer->p_data_cube->get_p_data(), p_data_labels->get_p_data(),
                                     (int)(iR * iC * iD), (int)iB, (int)(iR * iC));
@@ -247,6 +265,7 @@ class SoftmaxLossBridge : public AbstractBridge<DataType, DriverClass> {
 
  private:
   LogicalCubeType *loss_device;
+  bool gradient_is_current_ = false;
 };
 
 #undef CCT_BRIDGE_USINGS

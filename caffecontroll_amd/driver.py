@@ -127,6 +127,18 @@ class HIPDriver:
         check(self.lib.cct_hip_sgemm_conv_forward(o, batch, fmap, K, _p(model), _p(lowered), _p(bias),
                                                   _p(out), int(relu)), "sgemm_conv_forward")
 
+    # -- inner-product layers with few outputs: one launch per pass -----------------------------
+    def fc_small_supported(self, batch, in_features, out_features):
+        return bool(self.lib.cct_hip_fc_small_supported(batch, in_features, out_features))
+
+    def fc_small_forward(self, y, x, w, bias, batch, in_features, out_features, relu=False):
+        check(self.lib.cct_hip_fc_small_forward(_p(y), _p(x), _p(w), _p(bias), batch, in_features, out_features,
+                                                int(relu)), "fc_small_forward")
+
+    def fc_small_backward(self, dx, dw, db, dy, x, w, batch, in_features, out_features, relu_data=None):
+        check(self.lib.cct_hip_fc_small_backward(_p(dx), _p(dw), _p(db), _p(dy), _p(x), _p(w), batch, in_features,
+                                                 out_features, _p(relu_data)), "fc_small_backward")
+
     # `groups` > 1: a grouped convolution (d and o are the layer's totals), all groups in one launch
     def conv_direct_supported(self, b, d, n, k, s, p, o, groups=1):
         return bool(self.lib.cct_hip_conv_direct_supported_grouped(b, d, n, k, s, p, o, groups))
@@ -304,6 +316,12 @@ class HIPDriver:
     def softmax_loss_forward(self, prob, inp, labels, loss_sum, len_per_image, batch):
         check(self.lib.cct_hip_softmax_loss_forward(_p(prob), _p(inp), _p(labels), _p(loss_sum),
                                                     len_per_image, batch), "softmax_loss_forward")
+
+    def softmax_loss_forward_backward(self, prob, in_grad, inp, labels, loss_sum, len_per_image, batch, spatial=1):
+        """The forward pass and the gradient of the backward pass in one launch."""
+        check(self.lib.cct_hip_softmax_loss_forward_backward(_p(prob), _p(in_grad), _p(inp), _p(labels), _p(loss_sum),
+                                                             len_per_image, batch, spatial),
+              "softmax_loss_forward_backward")
 
     def softmax_loss_backward(self, in_grad, prob, labels, len_per_image, batch, spatial=1):
         check(self.lib.cct_hip_softmax_loss_backward(_p(in_grad), _p(prob), _p(labels), len_per_image,

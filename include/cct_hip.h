@@ -189,6 +189,22 @@ int cct_hip_sgemm_new_bias(int TA, int TB, int M, int N, int K, float alpha, con
  * src/kernels/relu.hxx:10-25) before the store. */
 int cct_hip_sgemm_conv_forward(int o, int batch, int fmap, int K, const float *model,
                                const float *lowered, const float *bias, float *out, int relu);
+/* ---- inner-product layers with few outputs -------------------------------------------------- */
+/* FullyConnectedBridge::forward / ::backward (src/bridges/FullyConnectedBridge_impl.hxx:169-234,
+ * 255-326) for layers of at most 32 outputs at batches of at most 1024 (LeNet's 500 -> 10 classifier):
+ * the sgemm_new + forward_bias of the forward pass as one launch, and the backward_bias_fc + two
+ * sgemm_new of the backward pass as one launch, in plain fp32 multiply-adds (a 64 x 64 matrix-core
+ * tile would be nearly all padding; the layer's time is launch latency).  x [batch][in], w [out][in],
+ * y / dy [batch][out], all dense.
+ * forward: y = x w^T + bias (bias may be NULL); relu != 0 clamps at zero (a following in-place ReLU).
+ * backward: dw = dy^T x; db = column sums of dy (db may be NULL); dx = dy w unless dx is NULL, stored
+ * as 0 wherever relu_data (same shape as dx: the layer's input, output of an in-place ReLU before the
+ * layer) is not positive, if relu_data is given.  Fixed summation orders: run-to-run identical. */
+int cct_hip_fc_small_supported(int batch, int in_features, int out_features);
+int cct_hip_fc_small_forward(float *y, const float *x, const float *w, const float *bias, int batch,
+                             int in_features, int out_features, int relu);
+int cct_hip_fc_small_backward(float *dx, float *dw, float *db, const float *dy, const float *x, const float *w,
+                              int batch, int in_features, int out_features, const float *relu_data);
 /* ---- stride-1 convolution without the lowered matrix ------------------------------------ */
 /* Fused replacements for chains of ConvolutionBridge's lowering pipeline when stride == 1 and
  * k is 3 or 5 (padded image at most 32 wide).  Results agree with the lowering path to fp32
@@ -418,6 +434,13 @@ int cct_hip_dropout_forward_train(float *out, const float *in, const unsigned in
  * sum) becomes NaN, and the backward pass subtracts no 1 for it. */
 int cct_hip_softmax_loss_forward(float *prob, const float *in, const float *labels,
                                  float *loss_sum, int len_per_image, int batch);
+/* The forward pass above and the backward pass below in the same launch, for a training iteration that
+ * will ask for the gradient anyway (SoftmaxLossBridge::forward then ::backward,
+ * src/bridges/SoftmaxLossBridge_impl.hxx:36-84, 90-143): prob and loss_sum as cct_hip_softmax_loss_forward
+ * writes them, in_grad as cct_hip_softmax_loss_backward would compute it from that prob.  Batches of a few
+ * thousand scores in all (LeNet: 64 x 10) take one single-workgroup launch for everything. */
+int cct_hip_softmax_loss_forward_backward(float *prob, float *in_grad, const float *in, const float *labels,
+                                          float *loss_sum, int len_per_image, int batch, int spatial);
 /* parallel_map<_f_src_to_dst_softmax_backward,_f_softmax_backward>, src/kernels/softmax.hxx:62-81:
  * in_grad = (prob - onehot(label)) / batch / spatial. */
 int cct_hip_softmax_loss_backward(float *in_grad, const float *prob, const float *labels,

@@ -167,6 +167,22 @@ def test_softmax_loss(oracle):
         drv.softmax_loss_backward(g, prob, dl, D, B, 1)
         rg = oracle.softmax_loss_backward(rprob, labels)
         assert rel_err(host(g), rg) <= 1e-5
+        # both passes in one launch: the same probabilities, loss and gradient bit for bit, call after call
+        # (the launch's arrival counter must come back to zero each time)
+        for _ in range(3):
+            prob2, loss2, g2 = empty(x.shape), empty((1,)), empty(x.shape)
+            drv.softmax_loss_forward_backward(prob2, g2, dev(x), dl, loss2, D, B, 1)
+            np.testing.assert_array_equal(host(prob2), host(prob))
+            np.testing.assert_array_equal(host(loss2), host(loss))
+            np.testing.assert_array_equal(host(g2), host(g))
+    # a label that is no class index: that image's loss (and the sum) is NaN, its gradient subtracts no 1
+    x = np.zeros((3, 4, 1, 1), np.float32)
+    bad = np.array([1.0, 7.0, 2.0], np.float32)
+    prob, loss, g = empty(x.shape), empty((1,)), empty(x.shape)
+    drv.softmax_loss_forward_backward(prob, g, dev(x), dev(bad), loss, 4, 3, 1)
+    assert np.isnan(host(loss)[0])
+    np.testing.assert_allclose(host(g).reshape(3, 4)[1], np.full(4, 0.25 / 3, np.float32), rtol=1e-6)
+    np.testing.assert_allclose(host(g).reshape(3, 4)[0], np.array([0.25, -0.75, 0.25, 0.25], np.float32) / 3, rtol=1e-6)
     pin = load_fixture("input", "softmax_backward_in.txt")
     labels = load_fixture("input", "softmax_label.txt")
     g = empty(pin.shape)

@@ -121,6 +121,53 @@ def test_sgemm_split_k_is_deterministic_and_correct(oracle):
     assert rel_err(outs[0], ref64) <= TOL
 
 
+FC_SMALL = [(64, 500, 10), (64, 800, 32), (1, 7, 1), (37, 129, 17), (256, 4096, 16), (1024, 33, 3)]
+
+
+@pytest.mark.parametrize("shape", FC_SMALL, ids=lambda c: "b%d_i%d_o%d" % c)
+def test_fc_small_kernels_match_oracle_and_gemm_path(oracle, shape):
+    """Inner-product layers of few outputs (LeNet's 500 -> 10): forward and backward as one launch each,
+    against the oracle's FullyConnectedBridge and against the library's own three-GEMM path; the ReLU clamp
+    (forward) and the ReLU mask on the input gradient (backward) are exactly those of the separate passes."""
+    B_, I, O = shape
+    rng = np.random.default_rng(B_ + I + O)
+    x = rng.standard_normal((B_, I)).astype(np.float32)
+    w = (rng.standard_normal((O, I)) * 0.05).astype(np.float32)
+    dy = rng.standard_normal((B_, O)).astype(np.float32)
+    bias = rng.standard_normal(O).astype(np.float32)
+    drv = driver()
+    assert drv.fc_small_supported(B_, I, O)
+    dx_, dw_, db_ = dev(x), dev(w), dev(bias)
+    y = empty((B_, O))
+    drv.fc_small_forward(y, dx_, dw_, db_, B_, I, O)
+    ref_y = oracle.fc_forward(x, w, bias)
+    assert rel_err(host(y), ref_y) <= TOL
+    y_nb, y_relu = empty((B_, O)), empty((B_, O))
+    drv.fc_small_forward(y_nb, dx_, dw_, None, B_, I, O)
+    assert rel_err(host(y_nb), ref_y - bias[None, :]) <= TOL
+    drv.fc_small_forward(y_relu, dx_, dw_, db_, B_, I, O, relu=True)
+    np.testing.assert_array_equal(host(y_relu), oracle.relu_forward(host(y)))
+    y_gemm = empty((B_, O))
+    drv.sgemm_new_bias(N_, T_, B_, O, I, 1.0, dx_, dw_, 0.0, y_gemm, db_, False)
+    assert rel_err(host(y), host(y_gemm)) <= 1e-5
+    # backward
+    gx, gw, gb = empty((B_, I)), empty((O, I)), empty((O,))
+    drv.fc_small_backward(gx, gw, gb, dev(dy), dx_, dw_, B_, I, O)
+    rdx, rdw, rdb = oracle.fc_backward(x, w, dy)
+    assert rel_err(host(gx), rdx) <= TOL and rel_err(host(gw), rdw) <= TOL and rel_err(host(gb), rdb) <= TOL
+    gx2, gw2 = empty((B_, I)), empty((O, I))
+    drv.fc_small_backward(gx2, gw2, None, dev(dy), dx_, dw_, B_, I, O, relu_data=dx_)
+    np.testing.assert_array_equal(host(gx2), oracle.relu_backward(host(gx), x))
+    np.testing.assert_array_equal(host(gw2), host(gw))       # run-to-run identical
+    gw3 = empty((O, I))
+    drv.fc_small_backward(None, gw3, None, dev(dy), dx_, dw_, B_, I, O)   # a first layer: no input gradient
+    np.testing.assert_array_equal(host(gw3), host(gw))
+    assert not drv.fc_small_supported(B_, I, 33) and not drv.fc_small_supported(1025, I, O)
+    from caffecontroll_amd import CctHipError
+    with pytest.raises(CctHipError):
+        drv.fc_small_forward(y, dx_, dw_, db_, B_, I, 33)
+
+
 def test_sgemm_new_fc_shapes(oracle):
     """The three sgemm_new calls of FullyConnectedBridge (LeNet ip1: 64 x 800 -> 500)."""
     B_, I, O = 64, 800, 500
