@@ -62,7 +62,7 @@ struct DirectArgs {
   uint32_t tiles_per_group, wt_group_floats;
 };
 
-constexpr int kDirect16PatchLoads = 10;  // the 16-row kernel stages four channels per step
+constexpr int kDirect16PatchLoads = 11;  // the 16-row kernel stages four channels per step
 
 constexpr int kDirectPatchLoads = 8;  // source elements per lane per step, at most
 
@@ -548,8 +548,13 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   const int forced = tuning().direct_tile;
   pl->tm16 = 0;
   if (const int tm16 = direct_tm16(mtot); tm16 && (forced == 0 || forced == 161 || forced == 162)) {
-    // 128-pixel tiles first (one group of conv2's data gradient: 504 us against 581 with 256 pixels)
-    for (int tnb = forced == 162 ? 2 : 1; tnb <= (forced == 161 ? 1 : 2); ++tnb) {
+    // 256-pixel tiles (seven LDS reads per twelve MFMAs of a tap instead of five per six) where the launch still
+    // has some four of them per compute unit -- measured 1.5-3 % faster on the data gradients of CaffeNet's conv1
+    // (sixteen phases) and grouped conv2 -- else 128-pixel tiles
+    const bool wide_first = forced == 162 || (forced == 0 && (long)groups * ((ptot + 255) / 256) >= 4L * cus);
+    for (int trial = 0; trial < 2; ++trial) {
+      const int tnb = (trial == 0) == wide_first ? 2 : 1;
+      if ((forced == 161 && tnb == 2) || (forced == 162 && tnb == 1)) continue;
       const int bn = 128 * tnb;
       const int rows = (ho - 1 + bn - 1) / ho + 1, imgs = (ho * ho - 1 + bn - 1) / (ho * ho) + 1;
       const int pr = rows - 1 + (imgs - 1) * (ks - 1) + ks;
