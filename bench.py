@@ -478,6 +478,48 @@ def net_iteration(args, torch, np, workload=None, steps=None, warmup=None, with_
     return result
 
 
+def host_layers(args, cfg, torch, np, steps=10, warmup=3):
+    """The same layer with its input and output layers in (page-locked) HOST memory, the placement
+    ParallelizedBridge handles with share_pointer_with_prev/next_bridge = false
+    (src/bridges/ParallelizedBridge_impl.hxx:595-621, 686-705): every forward uploads the input and downloads the
+    output, every backward uploads the output gradient and downloads the input gradient.  Measured both ways:
+    the batch in pieces with copies and kernels overlapped, and the reference's blocking copy - pass - copy
+    sequence.  PCIe-inclusive, so never `value`."""
+    from caffecontroll_amd import HIPDriver
+    from caffecontroll_amd.bridges import ConvolutionLayer, solver_param
+    b, d, n, k, s, p, o = CONFIGS[cfg]
+    m = (n + 2 * p - k) // s + 1
+    drv = HIPDriver(0)
+    drv.set_stream(torch.cuda.current_stream().cuda_stream)
+    x, w, bias, og = synth(cfg, 1234 + sorted(CONFIGS).index(cfg), torch)
+    pin = lambda a: torch.from_numpy(a).pin_memory()
+    h_in, h_ig = pin(x), torch.empty((b, d, n, n)).pin_memory()
+    h_out, h_og = torch.empty((b, o, m, m)).pin_memory(), pin(og)
+    moved = 4.0 * 2 * (b * d * n * n + b * o * m * m)
+    out = {"bytes_over_the_link_per_step": moved, "host_memory": "page-locked"}
+    for mode in ("overlapped", "blocking"):
+        # ParallelizedBridge::backward (copies, gradients, SGD update); a zero learning rate keeps the weights put
+        layer = ConvolutionLayer(b, d, n, k, s, p, o, h_in.numpy(), h_ig.numpy(), h_out.numpy(), h_og.numpy(),
+                                 share_prev=False, share_next=False, solver=solver_param(base_lr=0.0))
+        drv.memcpy(layer.model_ptr(), w.ctypes.data, w.nbytes, 0)
+        drv.memcpy(layer.bias_ptr(), bias.ctypes.data, bias.nbytes, 0)
+        layer.set_staging(mode == "overlapped")
+        for _ in range(warmup):
+            layer.forward()
+            layer.backward(with_update=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            layer.forward()
+            layer.backward(with_update=True)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        out[mode] = {"ms_per_step": round(ms, 4), "images_per_sec": round(b * 1e3 / ms, 1),
+                     "link_GBps": round(moved / ms / 1e6, 1), "in_pieces": layer.staging_overlapped()}
+        layer.close()
+    return out
+
+
 def conv_layer(args, cfg, torch, np, steps, warmup, with_lowering=True, with_cpu=True):
     """One of the single-layer configurations: `steps` timed passes of ConvolutionBridge forward + backward on tensors
     resident in HBM; returns the record (headline fields, per-stage times, rooflines, CPU baseline)."""
@@ -607,6 +649,9 @@ def main():
     ap.add_argument("--headline-only", action="store_true",
                     help="alexnet_conv2 only: leave out the `iterations` (LeNet, CaffeNet) and `configs` (LeNet conv1, "
                          "AlexNet conv1) records that the default line carries beside the headline")
+    ap.add_argument("--host-layers", action="store_true",
+                    help="single conv layers: also time the layer with its input and output layers in page-locked host "
+                         "memory (copies overlapped with the kernels, and the blocking sequence beside it)")
     ap.add_argument("--input-pipeline", action="store_true",
                     help="lenet/caffenet: feed every iteration through the input pipeline (raw bytes in host memory "
                          "-> pinned staging -> asynchronous upload -> transform kernel)")
@@ -653,6 +698,8 @@ def main():
                         with_lowering=not args.no_lowering_path, with_cpu=not args.no_cpu_baseline)
     extras = args.workload == "alexnet_conv2" and not args.headline_only and args.path < 0 and not args.unfused \
         and not args.no_data_grad
+    if args.host_layers or extras:
+        result["host_resident_layers"] = host_layers(args, args.workload, torch, np)
     if extras:
         # the other half of the headline metric and the remaining single-layer configurations, outside `value`
         result["configs"] = {

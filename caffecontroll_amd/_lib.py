@@ -72,6 +72,13 @@ PROTOTYPES = {
     "cct_hip_free": [_P],
     "cct_hip_memcpy": [_P, _P, _Z, _I],
     "cct_hip_memset": [_P, _I, _Z],
+    "cct_hip_pipe_create": [C.POINTER(_P)],
+    "cct_hip_pipe_destroy": [_P],
+    "cct_hip_pipe_begin": [_P],
+    "cct_hip_pipe_upload": [_P, _P, _P, _Z, C.POINTER(_I)],
+    "cct_hip_pipe_wait_upload": [_P, _I],
+    "cct_hip_pipe_download": [_P, _P, _P, _Z],
+    "cct_hip_pipe_finish": [_P],
     "cct_hip_lower_cube": [_P, _P, C.POINTER(PMapHelper)],
     "cct_hip_inverse_lower_cube": [_P, _P, C.POINTER(InverseLowerCubeArgs)],
     "cct_hip_inverse_lower_cube_bias_backward": [_P, _P, C.POINTER(InverseLowerCubeArgs), _P, _P, _I, _I, _I],

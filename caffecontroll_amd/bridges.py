@@ -39,6 +39,8 @@ BRIDGE_PROTOTYPES = {
     "cct_conv_bridge_history": ([_P], _P),
     "cct_conv_bridge_forward": ([_P], _I),
     "cct_conv_bridge_backward": ([_P, _I], _I),
+    "cct_conv_bridge_set_staging": ([_P, _I], _I),
+    "cct_conv_bridge_staging": ([_P], _I),
     "cct_conv_bridge_stage_ms": ([_P, C.POINTER(C.c_float)], _I),
     "cct_conv_bridge_stage_kernel": ([_P, _I], C.c_char_p),
 }
@@ -106,6 +108,14 @@ class ConvolutionLayer:
     def path(self):
         """Path level in effect (0..3)."""
         return self.lib.cct_conv_bridge_path(self.h)
+
+    def set_staging(self, overlapped=True):
+        """Host-resident layers: move the batch in pieces with copies and kernels overlapped (default), or as
+        one blocking copy in, the pass, one blocking copy out."""
+        check(self.lib.cct_conv_bridge_set_staging(self.h, int(overlapped)), "conv_bridge_set_staging")
+
+    def staging_overlapped(self):
+        return bool(self.lib.cct_conv_bridge_staging(self.h))
 
     # device addresses of the cubes the reference exposes on the bridge
     def model_ptr(self):

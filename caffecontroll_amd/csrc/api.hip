@@ -218,6 +218,100 @@ int cct_hip_memcpy(void *dst, const void *src, size_t size_in_byte, int kind) {
   return 0;
 }
 
+// ---- overlapped host <-> device staging ------------------------------------------------------------
+// Two side streams at the default priority, one per direction (the link is full duplex), and a pool of
+// events that order them against the library's compute stream.
+struct cct_hip_pipe {
+  hipStream_t up = nullptr, down = nullptr;
+  std::vector<hipEvent_t> events;
+  size_t next_event = 0;
+  int take(hipEvent_t *ev) {
+    if (next_event == events.size()) {
+      hipEvent_t e;
+      CCT_HIP_CHECK(hipEventCreateWithFlags(&e, hipEventDisableTiming));
+      events.push_back(e);
+    }
+    *ev = events[next_event++];
+    return 0;
+  }
+};
+
+int cct_hip_pipe_create(cct_hip_pipe **out) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(out != nullptr, "pipe_create: null result pointer");
+  cct_hip_pipe *p = new cct_hip_pipe;
+  hipError_t e = hipStreamCreateWithFlags(&p->up, hipStreamNonBlocking);
+  if (e == hipSuccess) e = hipStreamCreateWithFlags(&p->down, hipStreamNonBlocking);
+  if (e != hipSuccess) {
+    if (p->up) (void)hipStreamDestroy(p->up);
+    delete p;
+    return set_error((int)e, "pipe_create: %s", hipGetErrorString(e));
+  }
+  *out = p;
+  return 0;
+}
+
+int cct_hip_pipe_destroy(cct_hip_pipe *p) {
+  if (!p) return 0;
+  (void)hipStreamSynchronize(p->up);
+  (void)hipStreamSynchronize(p->down);
+  for (hipEvent_t e : p->events) (void)hipEventDestroy(e);
+  (void)hipStreamDestroy(p->up);
+  (void)hipStreamDestroy(p->down);
+  delete p;
+  return 0;
+}
+
+int cct_hip_pipe_begin(cct_hip_pipe *p) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(p != nullptr, "pipe_begin: null pipe");
+  // uploads must not overtake kernels already enqueued that still read the buffers they will overwrite
+  hipEvent_t ev;
+  if (int rc = p->take(&ev)) return rc;
+  CCT_HIP_CHECK(hipEventRecord(ev, ctx().stream));
+  CCT_HIP_CHECK(hipStreamWaitEvent(p->up, ev, 0));
+  return 0;
+}
+
+int cct_hip_pipe_upload(cct_hip_pipe *p, void *dst_device, const void *src_host, size_t bytes, int *ticket) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(p && ticket && (bytes == 0 || (dst_device && src_host)), "pipe_upload: null argument");
+  if (bytes) CCT_HIP_CHECK(hipMemcpyAsync(dst_device, src_host, bytes, hipMemcpyHostToDevice, p->up));
+  hipEvent_t ev;
+  if (int rc = p->take(&ev)) return rc;
+  CCT_HIP_CHECK(hipEventRecord(ev, p->up));
+  *ticket = (int)(p->next_event - 1);
+  return 0;
+}
+
+int cct_hip_pipe_wait_upload(cct_hip_pipe *p, int ticket) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(p && ticket >= 0 && (size_t)ticket < p->next_event, "pipe_wait_upload: no such upload");
+  CCT_HIP_CHECK(hipStreamWaitEvent(ctx().stream, p->events[ticket], 0));
+  return 0;
+}
+
+int cct_hip_pipe_download(cct_hip_pipe *p, void *dst_host, const void *src_device, size_t bytes) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(p && (bytes == 0 || (dst_host && src_device)), "pipe_download: null argument");
+  hipEvent_t ev;
+  if (int rc = p->take(&ev)) return rc;
+  CCT_HIP_CHECK(hipEventRecord(ev, ctx().stream));
+  CCT_HIP_CHECK(hipStreamWaitEvent(p->down, ev, 0));
+  if (bytes) CCT_HIP_CHECK(hipMemcpyAsync(dst_host, src_device, bytes, hipMemcpyDeviceToHost, p->down));
+  return 0;
+}
+
+int cct_hip_pipe_finish(cct_hip_pipe *p) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(p != nullptr, "pipe_finish: null pipe");
+  CCT_HIP_CHECK(hipStreamSynchronize(p->up));
+  CCT_HIP_CHECK(hipStreamSynchronize(ctx().stream));
+  CCT_HIP_CHECK(hipStreamSynchronize(p->down));
+  p->next_event = 0;
+  return 0;
+}
+
 // ---- random fillers: drawn on the host exactly as CPUDriver does, then copied to the device ------
 // std::mt19937 seeded with random_seed (std::random_device when -1) and the standard library's
 // distribution objects, one draw per element in index order (src/sched/DeviceDriver_CPU.cpp:661-699).

@@ -110,6 +110,14 @@ int cct_conv_bridge_set_options(cct_conv_bridge *h, int fused, int profile, int 
 
 int cct_conv_bridge_path(cct_conv_bridge *h) { return h ? h->pbridge->sub_bridge()->path() : -1; }
 
+int cct_conv_bridge_set_staging(cct_conv_bridge *h, int overlapped) {
+  if (!h) return CCT_HIP_EINVAL;
+  h->pbridge->set_overlapped_staging(overlapped != 0);
+  return 0;
+}
+
+int cct_conv_bridge_staging(cct_conv_bridge *h) { return h && h->pbridge->overlapped_staging() ? 1 : 0; }
+
 float *cct_conv_bridge_model(cct_conv_bridge *h) { return h->pbridge->p_model_cube->get_p_data(); }
 float *cct_conv_bridge_bias(cct_conv_bridge *h) {
   return h->pbridge->p_bias_cube ? h->pbridge->p_bias_cube->get_p_data() : nullptr;

@@ -222,6 +222,75 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   // stage profiling on ("" if it has not)
   const std::string &stage_kernel(int stage) const { return stage_kernel_[stage]; }
 
+  // ---- the passes on a range of images (for a scheduler that moves the batch in pieces) ----
+  // True when forward and data gradient can run on images [b0, b0 + nb) alone: the all-direct path, whose
+  // kernels take a batch count and tensor pointers (every image's result is independent of the others; the
+  // weight gradient sums over the batch and stays one call over all of it).
+  bool supports_batch_ranges() const { return path_ == PATH_DIRECT_ALL && !views_; }
+  // once per pass, before the first range: the weight slabs (the model changes between iterations)
+  void forward_prepare() {
+    if (strided_ok_)
+      p_driver->conv_strided_slabs(forward_slabs()->get_p_data(), p_model_cube->get_p_data(),
+                                   (int)num_output_features, (int)iD, (int)K, (int)stride, (int)padding);
+    else
+      p_driver->conv_direct_slabs(forward_slabs()->get_p_data(), p_model_cube->get_p_data(),
+                                  (int)num_output_features, (int)iD, (int)K, 0, (int)group);
+  }
+  void forward_range(size_t b0, size_t nb) {
+    const size_t in_img = iR * iC * iD, out_img = oR * oC * oD;
+    float *out = p_output_layer->p_data_cube->get_p_data() + b0 * out_img;
+    const float *in = p_input_layer->p_data_cube->get_p_data() + b0 * in_img;
+    const float *bias = bias_term ? p_bias_cube->get_p_data() : nullptr;
+    if (strided_ok_)
+      p_driver->conv_strided_forward(out, in, forward_slabs()->get_p_data(), bias, (int)nb, (int)iD, (int)iR, (int)K,
+                                     (int)stride, (int)padding, (int)num_output_features, fuse_relu_);
+    else
+      p_driver->conv_direct_forward(out, in, forward_slabs()->get_p_data(), bias, (int)nb, (int)iD, (int)iR, (int)K,
+                                    (int)padding, (int)num_output_features, 0, 0, fuse_relu_, (int)group);
+  }
+  // data gradient of a range; false if this layer's data gradient is not a per-range kernel (a strided layer
+  // without the phase-decomposed kernel): the caller then runs backward() on the whole batch
+  bool backward_data_ranges_supported() const { return supports_batch_ranges() && (direct_ok_ || strided_data_ok_); }
+  void backward_data_prepare() {
+    if (direct_ok_)
+      p_driver->conv_direct_slabs(backward_slabs()->get_p_data(), p_model_cube->get_p_data(),
+                                  (int)num_output_features, (int)iD, (int)K, 1, (int)group);
+    else
+      p_driver->conv_strided_backward_data_slabs(backward_slabs()->get_p_data(), p_model_cube->get_p_data(),
+                                                 (int)num_output_features, (int)iD, (int)K, (int)stride);
+  }
+  void backward_data_range(size_t b0, size_t nb) {
+    const size_t in_img = iR * iC * iD, out_img = oR * oC * oD;
+    float *ig = p_input_layer->p_gradient_cube->get_p_data() + b0 * in_img;
+    const float *og = p_output_layer->p_gradient_cube->get_p_data() + b0 * out_img;
+    const float *in = p_input_layer->p_data_cube->get_p_data() + b0 * in_img;
+    if (direct_ok_) {
+      p_driver->conv_direct_backward_data(ig, og, backward_slabs()->get_p_data(), (int)nb, (int)iD, (int)iR, (int)K,
+                                          (int)padding, (int)num_output_features, 0, 0,
+                                          input_is_relu_output ? in : nullptr, (int)group);
+    } else {
+      p_driver->conv_strided_backward_data(ig, og, backward_slabs()->get_p_data(), (int)nb, (int)iD, (int)iR, (int)K,
+                                           (int)stride, (int)padding, (int)num_output_features);
+      if (input_is_relu_output) {
+        DeviceMemoryPointer g = p_driver->get_device_pointer(ig, nb * in_img * sizeof(DataType));
+        p_driver->relu_backward(&g, &g, in);
+      }
+    }
+  }
+  // weight and bias gradient over the whole batch (all-direct path)
+  void backward_weights_all() {
+    float *dw = p_model_gradient_cube->get_p_data();
+    float *db = bias_term ? p_bias_gradient_cube->get_p_data() : nullptr;
+    const float *og = p_output_layer->p_gradient_cube->get_p_data();
+    const float *in = p_input_layer->p_data_cube->get_p_data();
+    if (strided_ok_)
+      p_driver->conv_strided_backward_weights(dw, db, og, in, (int)iB, (int)iD, (int)iR, (int)K, (int)stride,
+                                              (int)padding, (int)num_output_features);
+    else
+      p_driver->conv_direct_backward_weights(dw, db, og, in, (int)iB, (int)iD, (int)iR, (int)K, (int)padding,
+                                             (int)num_output_features, 0, 0, (int)group);
+  }
+
   // (1) input --lowering--> lowered  (2) model x lowered^T --> output  (3) remap + bias
   void forward() override {
     report_forward_history.reset();

@@ -58,6 +58,24 @@ class HIPDriver {
   void memset(DeviceMemoryPointer *dst, const char value) {
     ok(cct_hip_memset(dst->ptr, value, dst->size_in_byte), "memset");
   }
+  // ---- overlapped staging of host-resident layers (no counterpart in DeviceDriver.h) ----
+  cct_hip_pipe *pipe_create() {
+    cct_hip_pipe *p = nullptr;
+    ok(cct_hip_pipe_create(&p), "pipe_create");
+    return p;
+  }
+  void pipe_destroy(cct_hip_pipe *p) { ok(cct_hip_pipe_destroy(p), "pipe_destroy"); }
+  void pipe_begin(cct_hip_pipe *p) { ok(cct_hip_pipe_begin(p), "pipe_begin"); }
+  int pipe_upload(cct_hip_pipe *p, void *dst_device, const void *src_host, size_t bytes) {
+    int ticket = -1;
+    ok(cct_hip_pipe_upload(p, dst_device, src_host, bytes, &ticket), "pipe_upload");
+    return ticket;
+  }
+  void pipe_wait_upload(cct_hip_pipe *p, int ticket) { ok(cct_hip_pipe_wait_upload(p, ticket), "pipe_wait_upload"); }
+  void pipe_download(cct_hip_pipe *p, void *dst_host, const void *src_device, size_t bytes) {
+    ok(cct_hip_pipe_download(p, dst_host, src_device, bytes), "pipe_download");
+  }
+  void pipe_finish(cct_hip_pipe *p) { ok(cct_hip_pipe_finish(p), "pipe_finish"); }
 
   // ---- lowering / lifting (DeviceDriver.h:100-122) ----
   void lower_cube(DeviceMemoryPointer *dst, DeviceMemoryPointer *src, const PMapHelper args) {

@@ -19,6 +19,15 @@
 // the mode the reference's own bridge tests run in (tests/test_parallelized_convolution.cpp).
 // share_input_output_layer (ReLU, dropout: top == bottom) tells the bridge that its output layer
 // is its input layer, so no output cubes exist.
+//
+// Where the reference issues one blocking copy before and one after the sub-bridge, a sub-bridge that
+// can run on a range of images (ConvolutionBridge on its all-direct path) gets the batch in pieces
+// through a staging pipe: piece i+1 uploads and piece i-1 downloads while piece i computes, the two
+// directions of the link in use at once.  Every image's forward result and data gradient is independent
+// of the other images, and the weight gradient is still ONE call over the whole batch once the last piece
+// has arrived, so the results are those of the blocking sequence bit for bit (set_overlapped_staging(false)
+// runs that sequence).  The overlap needs page-locked host cubes; with pageable ones the copies are
+// correct but serialise.
 #pragma once
 #include "AbstractBridge.h"
 #include "GradientUpdater.h"
@@ -93,6 +102,7 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
   }
 
   ~ParallelizedBridge() {
+    if (pipe_) this->p_driver->pipe_destroy(pipe_);
     delete p_grad_updater;
     delete p_grad_updater_bias;
     delete p_sub_bridge;
@@ -138,8 +148,17 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
     return p_grad_updater ? p_grad_updater->current_iter : p_grad_updater_bias ? p_grad_updater_bias->current_iter : -1;
   }
 
+  // pieces the batch moves in when the layers are host resident and the sub-bridge can run on ranges
+  // (false: the reference's blocking copy - compute - copy sequence)
+  void set_overlapped_staging(bool on) { overlapped_ = on; }
+  bool overlapped_staging() const { return overlapped_ && staged_ranges<SubBridgeType>(nullptr); }
+
   void forward() override {
     this->report_forward_history.reset();
+    if ((p_device_input_layer || p_device_output_layer) && overlapped_ && forward_in_pieces<SubBridgeType>(nullptr)) {
+      this->report_forward_history.end();
+      return;
+    }
     if (p_device_input_layer) copy_cube(p_device_input_layer->p_data_cube, this->p_input_layer->p_data_cube, true);
     p_sub_bridge->forward();
     if (p_device_output_layer) copy_cube(this->p_output_layer->p_data_cube, p_device_output_layer->p_data_cube, false);
@@ -149,12 +168,14 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
   // sub-bridge backward, then the model and bias updates on the device
   void backward() override {
     this->report_backward_updateweight_history.reset();
-    if (p_device_output_layer)
-      copy_cube(p_device_output_layer->p_gradient_cube, this->p_output_layer->p_gradient_cube, true);
     p_sub_bridge->needs_to_calc_backward_grad = needs_to_calc_backward_grad;
-    p_sub_bridge->backward();
-    if (p_device_input_layer && needs_to_calc_backward_grad)
-      copy_cube(this->p_input_layer->p_gradient_cube, p_device_input_layer->p_gradient_cube, false);
+    if (!((p_device_input_layer || p_device_output_layer) && overlapped_ && backward_in_pieces<SubBridgeType>(nullptr))) {
+      if (p_device_output_layer)
+        copy_cube(p_device_output_layer->p_gradient_cube, this->p_output_layer->p_gradient_cube, true);
+      p_sub_bridge->backward();
+      if (p_device_input_layer && needs_to_calc_backward_grad)
+        copy_cube(this->p_input_layer->p_gradient_cube, p_device_input_layer->p_gradient_cube, false);
+    }
     if (p_grad_updater) p_grad_updater->update(p_model_grad->get_p_data());
     if (p_grad_updater_bias) p_grad_updater_bias->update(p_bias_grad->get_p_data());
     this->report_backward_updateweight_history.end();
@@ -163,6 +184,90 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
  private:
   bool share_pointer_with_prev_bridge, share_pointer_with_next_bridge, share_input_output_layer;
   LayerType *p_device_input_layer = nullptr, *p_device_output_layer = nullptr;
+  bool overlapped_ = true;
+  cct_hip_pipe *pipe_ = nullptr;
+  static constexpr size_t kPieces = 4;
+
+  // Sub-bridges with forward_range / backward_data_range members take the batch in pieces; for every other
+  // bridge type these overloads are chosen and report "not done" (SFINAE on the member's presence).
+  template <typename S>
+  bool staged_ranges(decltype(&S::forward_range)) const { return p_sub_bridge->supports_batch_ranges(); }
+  template <typename S>
+  bool staged_ranges(...) const { return false; }
+
+  template <typename S>
+  bool forward_in_pieces(decltype(&S::forward_range)) {
+    S *sb = p_sub_bridge;
+    if (!sb->supports_batch_ranges()) return false;
+    if (!pipe_) pipe_ = this->p_driver->pipe_create();
+    const size_t B = this->iB, pieces = B < kPieces ? B : kPieces;
+    LogicalCubeType *h_in = this->p_input_layer->p_data_cube, *h_out = this->p_output_layer->p_data_cube;
+    const size_t in_img = h_in->n_elements / B, out_img = h_out->n_elements / B;
+    float *d_in = p_device_input_layer ? p_device_input_layer->p_data_cube->get_p_data() : nullptr;
+    float *d_out = p_device_output_layer ? p_device_output_layer->p_data_cube->get_p_data() : nullptr;
+    int tickets[kPieces];
+    this->p_driver->pipe_begin(pipe_);
+    for (size_t i = 0; i < pieces; ++i) {
+      const size_t b0 = i * B / pieces, b1 = (i + 1) * B / pieces;
+      tickets[i] = d_in ? this->p_driver->pipe_upload(pipe_, d_in + b0 * in_img, h_in->get_p_data() + b0 * in_img,
+                                                      (b1 - b0) * in_img * sizeof(DataType))
+                        : -1;
+    }
+    sb->forward_prepare();
+    for (size_t i = 0; i < pieces; ++i) {
+      const size_t b0 = i * B / pieces, b1 = (i + 1) * B / pieces;
+      if (tickets[i] >= 0) this->p_driver->pipe_wait_upload(pipe_, tickets[i]);
+      sb->forward_range(b0, b1 - b0);
+      if (d_out)
+        this->p_driver->pipe_download(pipe_, h_out->get_p_data() + b0 * out_img, d_out + b0 * out_img,
+                                      (b1 - b0) * out_img * sizeof(DataType));
+    }
+    this->p_driver->pipe_finish(pipe_);
+    return true;
+  }
+  template <typename S>
+  bool forward_in_pieces(...) { return false; }
+
+  template <typename S>
+  bool backward_in_pieces(decltype(&S::backward_data_range)) {
+    S *sb = p_sub_bridge;
+    if (!sb->supports_batch_ranges() || (needs_to_calc_backward_grad && !sb->backward_data_ranges_supported())) return false;
+    if (!pipe_) pipe_ = this->p_driver->pipe_create();
+    const size_t B = this->iB, pieces = B < kPieces ? B : kPieces;
+    LogicalCubeType *h_ig = this->p_input_layer->p_gradient_cube, *h_og = this->p_output_layer->p_gradient_cube;
+    const size_t in_img = this->p_input_layer->p_data_cube->n_elements / B, out_img = h_og->n_elements / B;
+    float *d_ig = p_device_input_layer ? p_device_input_layer->p_gradient_cube->get_p_data() : nullptr;
+    float *d_og = p_device_output_layer ? p_device_output_layer->p_gradient_cube->get_p_data() : nullptr;
+    int tickets[kPieces];
+    this->p_driver->pipe_begin(pipe_);
+    for (size_t i = 0; i < pieces; ++i) {
+      const size_t b0 = i * B / pieces, b1 = (i + 1) * B / pieces;
+      tickets[i] = d_og ? this->p_driver->pipe_upload(pipe_, d_og + b0 * out_img, h_og->get_p_data() + b0 * out_img,
+                                                      (b1 - b0) * out_img * sizeof(DataType))
+                        : -1;
+    }
+    if (needs_to_calc_backward_grad) {
+      sb->backward_data_prepare();
+      for (size_t i = 0; i < pieces; ++i) {
+        const size_t b0 = i * B / pieces, b1 = (i + 1) * B / pieces;
+        if (tickets[i] >= 0) this->p_driver->pipe_wait_upload(pipe_, tickets[i]);
+        sb->backward_data_range(b0, b1 - b0);
+        if (d_ig)
+          this->p_driver->pipe_download(pipe_, h_ig->get_p_data() + b0 * in_img, d_ig + b0 * in_img,
+                                        (b1 - b0) * in_img * sizeof(DataType));
+      }
+    } else {
+      for (size_t i = 0; i < pieces; ++i)
+        if (tickets[i] >= 0) this->p_driver->pipe_wait_upload(pipe_, tickets[i]);
+    }
+    // the whole output gradient is on the device by now: the weight (and bias) gradient in one call, as unpieced
+    sb->backward_weights_all();
+    this->p_driver->pipe_finish(pipe_);
+    return true;
+  }
+  template <typename S>
+  bool backward_in_pieces(...) { return false; }
+
   // host <-> device copy of a whole cube (synchronous, like the reference's driver memcpy)
   void copy_cube(LogicalCubeType *dst, LogicalCubeType *src, bool to_device) {
     DeviceMemoryPointer d = to_device ? dst->get_device_pointer(this->p_driver)

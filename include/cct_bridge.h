@@ -74,6 +74,13 @@ int cct_conv_bridge_destroy(cct_conv_bridge *h);
 int cct_conv_bridge_set_options(cct_conv_bridge *h, int fused, int profile, int needs_backward_grad);
 /* The level in effect (0..3, see above). */
 int cct_conv_bridge_path(cct_conv_bridge *h);
+/* Host-resident layers (cct_conv_bridge_create_shared with a share flag 0): overlapped != 0 (the default)
+ * moves the batch in four pieces through two copy streams, piece i+1 uploading and piece i-1 downloading
+ * while piece i computes, when the layer runs on its all-direct path; 0 is the reference's sequence of
+ * one blocking copy in, the pass, one blocking copy out (src/bridges/ParallelizedBridge_impl.hxx:595-621,
+ * 686-705).  Same results bit for bit.  cct_conv_bridge_staging: 1 if forward/backward will run in pieces. */
+int cct_conv_bridge_set_staging(cct_conv_bridge *h, int overlapped);
+int cct_conv_bridge_staging(cct_conv_bridge *h);
 float *cct_conv_bridge_model(cct_conv_bridge *h);      /* [o][d][k][k] */
 float *cct_conv_bridge_bias(cct_conv_bridge *h);       /* [o] or NULL */
 float *cct_conv_bridge_model_grad(cct_conv_bridge *h);

@@ -128,6 +128,28 @@ int cct_hip_free(void *dev_ptr);
 int cct_hip_memcpy(void *dst, const void *src, size_t size_in_byte, int kind);
 int cct_hip_memset(void *dev_ptr, int value, size_t size_in_byte);
 
+/* ---- overlapped host <-> device staging ---------------------------------------------------- */
+/* For a bridge whose layers live in host memory (ParallelizedBridge with share_pointer_with_prev_bridge /
+ * share_pointer_with_next_bridge false, src/bridges/ParallelizedBridge_impl.hxx:595-621, 686-705, where
+ * the reference issues blocking DeviceDriver::memcpy calls around the sub-bridge): a pipe is two side
+ * streams, one per direction of the link, ordered against the library's compute stream by events, so that
+ * the batch can move in pieces -- piece i+1 uploading and piece i-1 downloading while piece i computes.
+ *   begin     uploads enqueued from here on start only after the kernels enqueued so far;
+ *   upload    asynchronous host -> device copy on the upload stream; *ticket names it;
+ *   wait_upload  kernels enqueued from here on start only after that upload has landed;
+ *   download  asynchronous device -> host copy on the download stream, after the kernels enqueued so far;
+ *   finish    the host waits for both side streams and the compute stream (tickets end here).
+ * The copies overlap with kernels (and with each other) only from / to page-locked host memory
+ * (hipHostMalloc, a pinned torch tensor); from pageable memory they are correct but serialise. */
+typedef struct cct_hip_pipe cct_hip_pipe;
+int cct_hip_pipe_create(cct_hip_pipe **pipe);
+int cct_hip_pipe_destroy(cct_hip_pipe *pipe);
+int cct_hip_pipe_begin(cct_hip_pipe *pipe);
+int cct_hip_pipe_upload(cct_hip_pipe *pipe, void *dst_device, const void *src_host, size_t bytes, int *ticket);
+int cct_hip_pipe_wait_upload(cct_hip_pipe *pipe, int ticket);
+int cct_hip_pipe_download(cct_hip_pipe *pipe, void *dst_host, const void *src_device, size_t bytes);
+int cct_hip_pipe_finish(cct_hip_pipe *pipe);
+
 /* ---- lowering / lifting / remap ------------------------------------------------------ */
 /* DeviceDriver::lower_cube<_fpmap_id,_fmap_lower> (src/sched/DeviceDriver.h:108-112; CPU
  * semantics src/sched/DeviceDriver_CPU.cpp:124-301).  src [sB][sD][sR][sC] ->

@@ -230,3 +230,57 @@ def test_pbridge_on_host_layers_like_the_reference_tests(share):
                                rtol=1e-4, atol=1e-3)
     np.testing.assert_allclose(_read(layer.bias_ptr(), (o,)), load_fixture("output", "conv_bias.txt"), rtol=1e-4, atol=1e-3)
     layer.close()
+
+
+@pytest.mark.parametrize("shape", [(32, 48, 27, 5, 1, 2, 64), (10, 3, 67, 11, 4, 0, 32), (7, 16, 13, 3, 1, 1, 48), (3, 8, 20, 5, 1, 0, 16)],
+                         ids=lambda s: "b%d_d%d_n%d_k%d_s%d_p%d_o%d" % s)
+@pytest.mark.parametrize("first_layer", [False, True])
+def test_pbridge_overlapped_staging_equals_blocking_copies(shape, first_layer):
+    """Host-resident layers on both sides: the batch moved in four pieces through the copy streams (upload of
+    piece i+1 and download of piece i-1 beside the kernels of piece i; weight gradient in one call once the whole
+    output gradient has arrived) against one blocking copy in, the pass, one blocking copy out
+    (src/bridges/ParallelizedBridge_impl.hxx:595-621, 686-705): output, input gradient, weight and bias gradients
+    and the updated weights bit for bit, on pinned and on pageable host arrays, two iterations in a row; batches
+    that do not divide by four, stride-1 and strided layers."""
+    import torch
+    from caffecontroll_amd.bridges import ConvolutionLayer, solver_param
+    b, d, n, k, s, p, o = shape
+    m = (n + 2 * p - k) // s + 1
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+    og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+    w = (rng.standard_normal((o, d, k, k)) * 0.05).astype(np.float32)
+    bias = rng.standard_normal(o).astype(np.float32)
+    driver()
+    results = {}
+    for mode in ("blocking", "pieces-pinned", "pieces-pageable"):
+        if mode == "pieces-pinned":
+            mk = lambda a: torch.from_numpy(a.copy()).pin_memory().numpy()
+        else:
+            mk = lambda a: a.copy()
+        h_in, h_ig = mk(x), mk(np.full(x.shape, np.nan, np.float32))
+        h_out, h_og = mk(np.full(og.shape, np.nan, np.float32)), mk(og)
+        layer = ConvolutionLayer(b, d, n, k, s, p, o, h_in, h_ig, h_out, h_og, share_prev=False, share_next=False,
+                                 solver=solver_param(base_lr=0.01, momentum=0.9, weight_decay=0.0005))
+        layer.set_options(fused=3, needs_backward_grad=not first_layer)
+        assert layer.path() == 3
+        layer.set_staging(mode != "blocking")
+        assert layer.staging_overlapped() == (mode != "blocking")
+        _copy_to(layer.model_ptr(), w)
+        _copy_to(layer.bias_ptr(), bias)
+        snap = []
+        for it in range(2):
+            layer.forward()
+            layer.backward(with_update=True)
+            snap.append([h_out.copy(), None if first_layer else h_ig.copy(), _read(layer.model_grad_ptr(), (w.size,)),
+                         _read(layer.bias_grad_ptr(), (o,)), _read(layer.model_ptr(), (w.size,)), _read(layer.bias_ptr(), (o,))])
+        results[mode] = snap
+        layer.close()
+    assert not np.isnan(results["blocking"][1][0]).any()
+    for mode in ("pieces-pinned", "pieces-pageable"):
+        for it in range(2):
+            for got, want, name in zip(results[mode][it], results["blocking"][it],
+                                       ("output", "input gradient", "weight gradient", "bias gradient", "weights", "bias")):
+                if want is None:
+                    continue
+                np.testing.assert_array_equal(got, want, err_msg="%s, iteration %d, %s" % (mode, it, name))
