@@ -41,6 +41,7 @@ BRIDGE_PROTOTYPES = {
     "cct_conv_bridge_backward": ([_P, _I], _I),
     "cct_conv_bridge_set_staging": ([_P, _I], _I),
     "cct_conv_bridge_staging": ([_P], _I),
+    "cct_conv_bridge_share_with_next": ([_P, _P, _P], _I),
     "cct_conv_bridge_stage_ms": ([_P, C.POINTER(C.c_float)], _I),
     "cct_conv_bridge_stage_kernel": ([_P, _I], C.c_char_p),
 }
@@ -113,6 +114,13 @@ class ConvolutionLayer:
         """Host-resident layers: move the batch in pieces with copies and kernels overlapped (default), or as
         one blocking copy in, the pass, one blocking copy out."""
         check(self.lib.cct_conv_bridge_set_staging(self.h, int(overlapped)), "conv_bridge_set_staging")
+
+    def share_with_next(self, out_data, out_grad):
+        """Raise share_pointer_with_next_bridge on a bridge created with a host-resident output layer: its output
+        layer becomes these DEVICE tensors ([b][o][m][m]) and the copies to / from the host stop."""
+        self._keep = self._keep + (out_data, out_grad)
+        check(self.lib.cct_conv_bridge_share_with_next(self.h, out_data.data_ptr(), out_grad.data_ptr()),
+              "conv_bridge_share_with_next")
 
     def staging_overlapped(self):
         return bool(self.lib.cct_conv_bridge_staging(self.h))

@@ -116,6 +116,17 @@ int cct_conv_bridge_set_staging(cct_conv_bridge *h, int overlapped) {
   return 0;
 }
 
+int cct_conv_bridge_share_with_next(cct_conv_bridge *h, float *out_data_device, float *out_grad_device) {
+  if (!h || !out_data_device || !out_grad_device) return CCT_HIP_EINVAL;
+  return guarded("conv_bridge_share_with_next", [&] {
+    // the output layer's cubes now name the device memory of the next bridge's input layer
+    h->out_layer->p_data_cube->set_p_data(out_data_device);
+    h->out_layer->p_gradient_cube->set_p_data(out_grad_device);
+    h->pbridge->set_share_pointer_with_next_bridge(true);
+    return 0;
+  });
+}
+
 int cct_conv_bridge_staging(cct_conv_bridge *h) { return h && h->pbridge->overlapped_staging() ? 1 : 0; }
 
 float *cct_conv_bridge_model(cct_conv_bridge *h) { return h->pbridge->p_model_cube->get_p_data(); }

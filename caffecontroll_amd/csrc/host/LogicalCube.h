@@ -49,6 +49,17 @@ class LogicalCube {
     p_data = data;
   }
 
+  // Becomes a non-owning view of `data` (same shape), releasing the memory the cube owned, if any: how a
+  // bridge's own device cube turns into an alias of its neighbour's once the two are told to share.
+  void adopt(T *const data) {
+    if (own_data && p_data) {
+      DeviceMemoryPointer_Local_GPURAM mem(p_data, n_elements * sizeof(T));
+      p_driver->free(&mem);
+    }
+    own_data = false;
+    p_data = data;
+  }
+
   // The reference returns a heap wrapper that is never freed (src/LogicalCube.h:64-66); this
   // returns the wrapper by value.
   DeviceMemoryPointer get_device_pointer(HIPDriver *driver) const {

@@ -115,14 +115,22 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
   bool get_share_pointer_with_prev_bridge() const { return share_pointer_with_prev_bridge; }
   bool get_share_pointer_with_next_bridge() const { return share_pointer_with_next_bridge; }
   bool get_share_input_output_layer() const { return share_input_output_layer; }
+  // The builder of the next bridge raises the flag once it knows that bridge lives on the same device
+  // (src/DeepNet.h:1116-1120): the output layer's cubes are then device memory the two bridges share.  The
+  // device cubes this bridge allocated for a host-resident output become views of them (the sub-bridge keeps
+  // its layer object) and the copies after forward() / before backward() stop.  Lowering the flag again would
+  // need device cubes under a sub-bridge that was built on the caller's own layer: refused.
   void set_share_pointer_with_next_bridge(bool share) {
     if (share == share_pointer_with_next_bridge) return;
-    if (p_device_output_layer || share_input_output_layer || !share) {
-      // going from shared to host-resident output after construction would need new device cubes
-      // under a sub-bridge that already holds the old ones
-      host_fail("ParallelizedBridge: share_pointer_with_next_bridge can only be raised, and only before the bridge owns device output cubes");
+    if (!share || share_input_output_layer)
+      host_fail("ParallelizedBridge: share_pointer_with_next_bridge can only be raised, and not on a bridge whose "
+                "output layer is its input layer");
+    if (p_device_output_layer) {
+      p_device_output_layer->p_data_cube->adopt(this->p_output_layer->p_data_cube->get_p_data());
+      p_device_output_layer->p_gradient_cube->adopt(this->p_output_layer->p_gradient_cube->get_p_data());
+      output_is_view_ = true;
     }
-    share_pointer_with_next_bridge = share;
+    share_pointer_with_next_bridge = true;
   }
 
   SubBridgeType *sub_bridge() { return p_sub_bridge; }
@@ -155,13 +163,13 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
 
   void forward() override {
     this->report_forward_history.reset();
-    if ((p_device_input_layer || p_device_output_layer) && overlapped_ && forward_in_pieces<SubBridgeType>(nullptr)) {
+    if ((p_device_input_layer || staged_output()) && overlapped_ && forward_in_pieces<SubBridgeType>(nullptr)) {
       this->report_forward_history.end();
       return;
     }
     if (p_device_input_layer) copy_cube(p_device_input_layer->p_data_cube, this->p_input_layer->p_data_cube, true);
     p_sub_bridge->forward();
-    if (p_device_output_layer) copy_cube(this->p_output_layer->p_data_cube, p_device_output_layer->p_data_cube, false);
+    if (staged_output()) copy_cube(this->p_output_layer->p_data_cube, p_device_output_layer->p_data_cube, false);
     this->report_forward_history.end();
   }
 
@@ -169,8 +177,8 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
   void backward() override {
     this->report_backward_updateweight_history.reset();
     p_sub_bridge->needs_to_calc_backward_grad = needs_to_calc_backward_grad;
-    if (!((p_device_input_layer || p_device_output_layer) && overlapped_ && backward_in_pieces<SubBridgeType>(nullptr))) {
-      if (p_device_output_layer)
+    if (!((p_device_input_layer || staged_output()) && overlapped_ && backward_in_pieces<SubBridgeType>(nullptr))) {
+      if (staged_output())
         copy_cube(p_device_output_layer->p_gradient_cube, this->p_output_layer->p_gradient_cube, true);
       p_sub_bridge->backward();
       if (p_device_input_layer && needs_to_calc_backward_grad)
@@ -184,8 +192,10 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
  private:
   bool share_pointer_with_prev_bridge, share_pointer_with_next_bridge, share_input_output_layer;
   LayerType *p_device_input_layer = nullptr, *p_device_output_layer = nullptr;
-  bool overlapped_ = true;
+  bool overlapped_ = true, output_is_view_ = false;
   cct_hip_pipe *pipe_ = nullptr;
+  // the device copy of a host-resident output layer (null once the output is shared with the next bridge)
+  LayerType *staged_output() const { return output_is_view_ ? nullptr : p_device_output_layer; }
   static constexpr size_t kPieces = 4;
 
   // Sub-bridges with forward_range / backward_data_range members take the batch in pieces; for every other
@@ -204,7 +214,7 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
     LogicalCubeType *h_in = this->p_input_layer->p_data_cube, *h_out = this->p_output_layer->p_data_cube;
     const size_t in_img = h_in->n_elements / B, out_img = h_out->n_elements / B;
     float *d_in = p_device_input_layer ? p_device_input_layer->p_data_cube->get_p_data() : nullptr;
-    float *d_out = p_device_output_layer ? p_device_output_layer->p_data_cube->get_p_data() : nullptr;
+    float *d_out = staged_output() ? p_device_output_layer->p_data_cube->get_p_data() : nullptr;
     int tickets[kPieces];
     this->p_driver->pipe_begin(pipe_);
     for (size_t i = 0; i < pieces; ++i) {
@@ -237,7 +247,7 @@ class ParallelizedBridge : public AbstractBridge<DataType, DriverClass> {
     LogicalCubeType *h_ig = this->p_input_layer->p_gradient_cube, *h_og = this->p_output_layer->p_gradient_cube;
     const size_t in_img = this->p_input_layer->p_data_cube->n_elements / B, out_img = h_og->n_elements / B;
     float *d_ig = p_device_input_layer ? p_device_input_layer->p_gradient_cube->get_p_data() : nullptr;
-    float *d_og = p_device_output_layer ? p_device_output_layer->p_gradient_cube->get_p_data() : nullptr;
+    float *d_og = staged_output() ? p_device_output_layer->p_gradient_cube->get_p_data() : nullptr;
     int tickets[kPieces];
     this->p_driver->pipe_begin(pipe_);
     for (size_t i = 0; i < pieces; ++i) {

@@ -80,6 +80,12 @@ int cct_conv_bridge_path(cct_conv_bridge *h);
  * one blocking copy in, the pass, one blocking copy out (src/bridges/ParallelizedBridge_impl.hxx:595-621,
  * 686-705).  Same results bit for bit.  cct_conv_bridge_staging: 1 if forward/backward will run in pieces. */
 int cct_conv_bridge_set_staging(cct_conv_bridge *h, int overlapped);
+/* ParallelizedBridge::set_share_pointer_with_next_bridge(true) (src/bridges/ParallelizedBridge.h:190-194), which
+ * the builder of the NEXT bridge calls once it knows that bridge lives on the same device (src/DeepNet.h:1116-1120):
+ * a bridge created with share_pointer_with_next_bridge == 0 stops copying its output to the host; its output layer
+ * becomes the given DEVICE tensors (out_data / out_grad [b][o][m][m]), shared with the next bridge.  The flag
+ * cannot be lowered again. */
+int cct_conv_bridge_share_with_next(cct_conv_bridge *h, float *out_data_device, float *out_grad_device);
 int cct_conv_bridge_staging(cct_conv_bridge *h);
 float *cct_conv_bridge_model(cct_conv_bridge *h);      /* [o][d][k][k] */
 float *cct_conv_bridge_bias(cct_conv_bridge *h);       /* [o] or NULL */

@@ -284,3 +284,38 @@ def test_pbridge_overlapped_staging_equals_blocking_copies(shape, first_layer):
                 if want is None:
                     continue
                 np.testing.assert_array_equal(got, want, err_msg="%s, iteration %d, %s" % (mode, it, name))
+
+
+def test_pbridge_share_with_next_can_be_raised_after_construction(oracle):
+    """The reference builds a bridge with share_pointer_with_next_bridge false and lets the builder of the next
+    bridge raise it (src/DeepNet.h:1116-1120).  Here: a bridge created over a host output layer first copies its
+    output to the host; once told to share, it writes into the next bridge's device tensors, reads its output
+    gradient from there, and leaves the host arrays alone."""
+    from caffecontroll_amd.bridges import ConvolutionLayer, solver_param
+    b, d, n, k, s, p, o = 4, 6, 13, 3, 1, 1, 10
+    m = n
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+    og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+    w = (rng.standard_normal((o, d, k, k)) * 0.1).astype(np.float32)
+    bias = rng.standard_normal(o).astype(np.float32)
+    ref_out, low = oracle.conv_forward(x, w, bias, k, s, p)
+    ref_dx, _, _ = oracle.conv_backward(x.shape, w, og, low, k, s, p)
+    driver()
+    in_data, in_grad = dev(x), empty((b, d, n, n))
+    h_out, h_og = np.full((b, o, m, m), np.nan, np.float32), np.zeros((b, o, m, m), np.float32)
+    layer = ConvolutionLayer(b, d, n, k, s, p, o, in_data, in_grad, h_out, h_og, share_prev=True, share_next=False,
+                             solver=solver_param(base_lr=0.0))
+    _copy_to(layer.model_ptr(), w)
+    _copy_to(layer.bias_ptr(), bias)
+    layer.forward()
+    assert rel_err(h_out, ref_out) <= 1e-4
+    d_out, d_og = empty((b, o, m, m)), dev(og)
+    layer.share_with_next(d_out, d_og)
+    h_out[...] = np.nan
+    layer.forward()
+    assert rel_err(host(d_out), ref_out) <= 1e-4
+    assert np.isnan(h_out).all()                  # nothing is copied to the host any more
+    layer.backward(with_update=True)              # ParallelizedBridge::backward reads the device gradient in place
+    assert rel_err(host(in_grad), ref_dx) <= 1e-4
+    layer.close()
