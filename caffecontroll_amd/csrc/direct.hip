@@ -28,6 +28,7 @@
 //
 // Bound: fp32 MFMA rate.  Algorithmic work 2 * mtot * batch*ho*ho * kc*KS*KS FLOP per call.
 #include <cstdlib>
+#include <type_traits>
 
 #include "cct_common.h"
 #include "mfma_common.h"
@@ -982,7 +983,14 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
 // With WN > 1 the workgroup is a W x WN grid of wavefronts: W row blocks times WN column groups of TB
 // blocks each (192 maps = six row blocks then run as twelve wavefronts, three on every SIMD, instead
 // of six wavefronts that leave two SIMDs half idle).
-template <int KS, int TB, int PW, int HO, int W, int WN = 1>
+//
+// ALDS: the dout rows go through LDS after all, fetched the way the patches are (4 bytes per lane straight into
+// LDS, consecutive lanes on consecutive words of a row, rows packed HO words apart -- an odd stride, so the
+// 32 maps of a wavefront fall on 32 banks).  A lane that fetches its own row touches a cache line of its own
+// with every 16-byte load (64 lines per instruction); with few MFMAs per row -- three column blocks a
+// wavefront, and both column groups fetching the same rows -- the address path of the texture unit is then
+// busy for longer than the MFMAs of the step take.
+template <int KS, int TB, int PW, int HO, int W, int WN = 1, bool ALDS = false>
 __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(const WgradArgs g) {
   constexpr int KK = KS * KS, BN = 32 * TB * WN, NT = 64 * W * WN;
   constexpr int PWS = WgradStrides<KS, PW>::PWS, PCH = WgradStrides<KS, PW>::PCH;
@@ -996,8 +1004,11 @@ __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(con
   // workgroups share a compute unit: their barriers fall at different times and the MFMA pipes
   // stay fed across them.
   constexpr int NQD = (HO + 3) / 4;
-  constexpr int NAW = NQD;                       // dout loads (16 bytes per lane) per lane per step
-  constexpr int STAGE = BSZ;
+  // ALDS: one image's 32 * W rows of HO words take NAI loads of 4 bytes per lane (whole passes), image 0 then
+  // image 1, behind the patches of the stage
+  constexpr int NAI = (32 * W * HO + NT - 1) / NT, AIMG = NAI * NT;
+  constexpr int NAW = ALDS ? 2 * NAI : NQD;      // dout loads per lane per step
+  constexpr int STAGE = BSZ + (ALDS ? 2 * AIMG : 0);
   constexpr int NQ = (HO + 1) / 2;                // x pairs per step
   extern __shared__ __attribute__((aligned(16))) float smem[];
 
@@ -1019,6 +1030,16 @@ __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(con
   // byte offset of this lane's dout row within (image pair, first map of the tile, row y)
   const uint32_t avoff =
       ((min((uint32_t)(m0 + wave * 32 + r), (uint32_t)g.o - 1) - m0) * ho2 + h * g.dout_img_stride) * 4u;
+  // ALDS: byte offset of word k * NT + tid of an image's rows within (image, first map of the tile, row y)
+  uint32_t aoff[ALDS ? NAI : 1];
+  if constexpr (ALDS) {
+#pragma unroll
+    for (int k = 0; k < NAI; ++k) {
+      const uint32_t e = (uint32_t)(k * NT + tid), m = e / HO, x = e - m * HO;
+      aoff[k] = (m < 32u * W && m0 + (int)m < g.o) ? (m * ho2 + x) * 4u : kOutOfRange;
+    }
+  }
+  const int abase = h * AIMG + (wave * 32 + r) * HO;  // this lane's row within the staged dout rows
   uint32_t boff[NBW], bmeta[NBW];
 #pragma unroll
   for (int k = 0; k < NBW; ++k) {
@@ -1029,10 +1050,13 @@ __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(con
     const int scol = (int)pcol - g.pad;
     const bool ok = e < (uint32_t)(NCH * PCH) && prow < 2u * KS && ch0 + (int)ch < g.d &&
                     (unsigned)scol < (unsigned)g.hs;
-    boff[k] = ok ? (second * g.src_img_stride + ch * hs2 + kr * g.hs + (uint32_t)scol) * 4u : 0u;
-    bmeta[k] = kr | (second << 4) | ((ok ? 1u : 0u) << 5);
+    boff[k] = ok ? (second * g.src_img_stride + ch * hs2 + kr * g.hs + (uint32_t)scol) * 4u : kOutOfRange;
+    bmeta[k] = kr + 8u * second;
   }
-  const rsrc_t a_rsrc = make_rsrc(g.dout + (size_t)grp * g.o * ho2), b_rsrc = make_rsrc(g.src + (size_t)grp * g.d * hs2);
+  // the patch descriptor starts `pad` rows ahead of the tensor (never read there: those rows fail the row test)
+  const rsrc_t a_rsrc = make_rsrc(g.dout + (size_t)grp * g.o * ho2),
+               b_rsrc = make_rsrc(g.src + (size_t)grp * g.d * hs2 - (ptrdiff_t)g.pad * g.hs);
+  const rsrc_t a_none = make_rsrc_empty(g.dout);  // every load through it is out of range: zeros
 
   int bbase[TB];
 #pragma unroll
@@ -1050,60 +1074,100 @@ __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(con
   // bias gradient: lane (r, h) adds up dout[map r][image h of every pair][every row][every x]
   float bsum = 0.0f;
 
-// per-step scalars of step s
-#define CCT_WSPEC_STEP(s)                                                                         \
-  const uint32_t pair_ = fdiv((uint32_t)(s), g.div_ho);                                           \
-  const int y_ = (s) - (int)pair_ * HO;                                                           \
-  const int img0_ = 2 * (int)pair_;                                                               \
-  const bool two_ = img0_ + 1 < g.batch;                                                          \
-  const uint32_t ga_ = (uint32_t)(((size_t)img0_ * g.dout_img_stride + m0 * ho2 + y_ * HO) * 4);  \
-  const uint32_t av_ = (h && !two_) ? kOutOfRange : avoff;                                        \
-  const uint32_t gb_ = (uint32_t)(((size_t)img0_ * g.src_img_stride + ch0 * hs2) * 4);            \
-  const uint32_t row0_ = (uint32_t)((y_ - g.pad) * g.hs * 4)
-#define CCT_WSPEC_A(k)                                                                            \
-  an[k] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(                           \
-      a_rsrc, av_ + ((k) + 1 < NQD ? 16u * (k) : 4u * (HO - 4)), ga_, 0))
-#define CCT_WSPEC_B(k, st)                                                                        \
+  // The step loop is unrolled by two: the stage a step reads, P, and the stage its loads fill, P ^ 1, are
+  // compile-time constants, so LDS addresses are fixed registers plus immediates and the lane-fetched dout rows
+  // of the two stages are two register sets, never copied.  Whatever moves with the step (image pair, row) is
+  // in the SCALAR offset of a load; a lane's own offset never changes, and what is left per patch load is the
+  // test whether its source row exists (compare + select).  Vector ALU instructions and MFMAs of one SIMD do not
+  // overlap, so every one of them taken out of the loop is four cycles returned to the MFMA pipe.
+  struct StepScalars {
+    uint32_t ga, gb, norows;
+    bool two;
+  };
+  auto scalars_of = [&](int s) {
+    StepScalars c;
+    const uint32_t pair = fdiv((uint32_t)s, g.div_ho);
+    const int y = s - (int)pair * HO;
+    const int img0 = 2 * (int)pair;
+    c.two = img0 + 1 < g.batch;
+    c.ga = (uint32_t)(((size_t)img0 * g.dout_img_stride + m0 * ho2 + y * HO) * 4);
+    // (the patch descriptor starts `pad` rows ahead of the tensor: row y + kr of it is source row y - pad + kr)
+    c.gb = (uint32_t)(((size_t)img0 * g.src_img_stride + ch0 * hs2 + y * g.hs) * 4);
+    // kernel rows kr whose source row y - pad + kr exists
+    const int lo = max(0, g.pad - y), hi = min(KS - 1, g.hs - 1 + g.pad - y);
+    const uint32_t one = hi >= lo ? ((2u << hi) - (1u << lo)) : 0u;
+    c.norows = ~(one | (c.two ? one << 8 : 0u));
+    return c;
+  };
+  f4 abuf[2][NQD];  // the dout row this lane fetched itself, per stage
+#pragma unroll
+  for (int k = 0; k < NQD; ++k) abuf[0][k] = abuf[1][k] = f4{0.f, 0.f, 0.f, 0.f};
+  // dout loads of the step described by c, into stage st (IN: the step is an interior one)
+#define CCT_WSPEC_A(k, st, c)                                                                     \
   do {                                                                                            \
-    const uint32_t mt_ = bmeta[k];                                                                \
-    const int srow_ = y_ - g.pad + (int)(mt_ & 15u);                                              \
-    const bool ok_ = (mt_ & 32u) && (unsigned)srow_ < (unsigned)g.hs && (two_ || !(mt_ & 16u));   \
-    lds_dma4(b_rsrc, ok_ ? boff[k] + row0_ : kOutOfRange, gb_,                                    \
-             smem + (st) * STAGE + (k) * NT + wave_id * 64);                                     \
+    if constexpr (ALDS) {                                                                         \
+      /* loads NAI .. 2 NAI - 1 are the second image's: all zeros when the pair has only one */   \
+      if ((k) < NAI)                                                                              \
+        lds_dma4(a_rsrc, aoff[(k) % NAI], c.ga, smem + (st) * STAGE + BSZ + (k) * NT + wave_id * 64); \
+      else                                                                                        \
+        lds_dma4(c.two ? a_rsrc : a_none, aoff[(k) % NAI], c.ga + g.dout_img_stride * 4u,         \
+                 smem + (st) * STAGE + BSZ + (k) * NT + wave_id * 64);                            \
+    } else {                                                                                      \
+      abuf[st][(k) % NQD] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(         \
+          a_rsrc, (!h || c.two) ? avoff : kOutOfRange,                                            \
+          c.ga + ((k) + 1 < NQD ? 16u * (k) : 4u * (HO - 4)), 0));                                \
+    }                                                                                             \
+  } while (0)
+#define CCT_WSPEC_B(k, st, c)                                                                     \
+  do {                                                                                            \
+    /* bmeta[k]: kernel row of a first-image lane, 8 + kernel row of a second-image lane; bit  */  \
+    /* bmeta[k] of c.norows says that this row does not exist in the step, which moves the     */  \
+    /* offset out of range (two vector instructions: bit-field extract, shift-or)              */  \
+    lds_dma4(b_rsrc, boff[k] | (((c.norows >> bmeta[k]) & 1u) << 31), c.gb,                       \
+             smem + (st) * STAGE + (k) * NT + wave_id * 64);                                      \
   } while (0)
 
   const bool do_bias = g.out_bias && tn == 0 && wn == 0;  // wave-uniform
-  f4 an[NQD];  // this lane's dout row of the coming step
-#pragma unroll
-  for (int k = 0; k < NQD; ++k) an[k] = f4{0.f, 0.f, 0.f, 0.f};
   if (s_beg < s_end) {
-    CCT_WSPEC_STEP(s_beg);
+    const StepScalars c0 = scalars_of(s_beg);
 #pragma unroll
-    for (int k = 0; k < NAW; ++k) CCT_WSPEC_A(k);
+    for (int k = 0; k < NAW; ++k) CCT_WSPEC_A(k, 0, c0);
 #pragma unroll
-    for (int k = 0; k < NBW; ++k) CCT_WSPEC_B(k, 0);
+    for (int k = 0; k < NBW; ++k) CCT_WSPEC_B(k, 0, c0);
     lds_dma_wait();
   }
   __syncthreads();
 
-  for (int s = s_beg; s < s_end; ++s) {
-    const int cur = (s - s_beg) & 1, nxt = cur ^ 1;
-    CCT_WSPEC_STEP(min(s + 1, s_end - 1));
-    const float *sb = smem + cur * STAGE;
-    // this lane's dout row, fetched during the previous step: pixel x is component x % 4 of run
-    // x / 4, or of the overlapping last run
-    f4 aq[NQD];
+  // fragment addresses per stage: patch columns of this lane's TB blocks, and its staged dout row
+  int bb[2][TB], ab[2];
 #pragma unroll
-    for (int j = 0; j < NQD; ++j) aq[j] = an[j];
+  for (int b = 0; b < TB; ++b) {
+    bb[0][b] = bbase[b];
+    bb[1][b] = bbase[b] + STAGE;
+    // (kept as a register of its own: seen as bb[0][b] + constant, it would be re-added before every read --
+    // the paired LDS read reaches only 255 words beyond its address register)
+    asm volatile("" : "+v"(bb[1][b]));
+  }
+  ab[0] = BSZ + abase;
+  ab[1] = STAGE + BSZ + abase;
+  asm volatile("" : "+v"(ab[1]));
+
+  // one step: MFMAs on stage P, loads of the step described by c into stage P ^ 1
+  auto step = [&](auto stage_c, const StepScalars &c) {
+    constexpr int P = decltype(stage_c)::value, N = P ^ 1;
     float fa[2][2], fb[2][2][TB];
-#define CCT_WSPEC_AVAL(x) ((x) < 4 * (NQD - 1) ? aq[(x) / 4][(x) % 4] : aq[NQD - 1][((x) - (HO - 4)) & 3])
+    // this lane's dout row: staged, or fetched by the lane during the previous step (pixel x is component
+    // x % 4 of run x / 4, or of the overlapping last run)
+#define CCT_WSPEC_AVAL(x)                                                                         \
+  (ALDS ? smem[ab[P] + (x)]                                                                       \
+        : ((x) < 4 * (NQD - 1) ? abuf[P][(x) / 4][(x) % 4] : abuf[P][NQD - 1][((x) - (HO - 4)) & 3]))
 #define CCT_WSPEC_FRAGS(buf, x)                                                                   \
   do {                                                                                            \
     fa[buf][0] = CCT_WSPEC_AVAL(x);                                                               \
     fa[buf][1] = (x) + 1 < HO ? CCT_WSPEC_AVAL((x) + 1) : 0.0f;                                   \
     _Pragma("unroll") for (int b = 0; b < TB; ++b) {                                              \
-      fb[buf][0][b] = sb[bbase[b] + (x)];                                                         \
-      fb[buf][1][b] = sb[bbase[b] + (x) + 1];                                                     \
+      fb[buf][0][b] = smem[bb[P][b] + (x)];                                                       \
+      fb[buf][1][b] = smem[bb[P][b] + (x) + 1];                                                   \
     }                                                                                             \
   } while (0)
     // bias gradient: only the wavefronts that report it add up their dout row (in pixel order), in one
@@ -1126,24 +1190,22 @@ __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(con
             acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[cb][e], fb[cb][e][b], acc[b], 0, 0, 0);
         }
       }
-      // this pair's share of the next step's loads
-      constexpr int A0 = 0;
-      (void)A0;
-      // (all of them within the first NQI pairs, so that the last ones have landed by the barrier)
+      // this pair's share of the next step's loads (all of them within the first NQI pairs, so that the
+      // last ones have landed by the barrier)
       constexpr int NQI = (NQ * 5 + 7) / 8;
       const int qi = q < NQI ? q : NQI, qj = q + 1 < NQI ? q + 1 : NQI;
       const int a_lo = qi * NAW / NQI, a_hi = qj * NAW / NQI;
       const int b_lo = qi * NBW / NQI, b_hi = qj * NBW / NQI;
 #pragma unroll
       for (int k = 0; k < NAW; ++k)
-        if (k >= a_lo && k < a_hi) CCT_WSPEC_A(k);
+        if (k >= a_lo && k < a_hi) CCT_WSPEC_A(k, N, c);
 #pragma unroll
       for (int k = 0; k < NBW; ++k)
-        if (k >= b_lo && k < b_hi) CCT_WSPEC_B(k, nxt);
+        if (k >= b_lo && k < b_hi) CCT_WSPEC_B(k, N, c);
       // issue order: LDS reads of the next pair first, one per MFMA, then the global loads
       {
         constexpr int NM = 2 * TB;
-        const int nr = (q + 1 < NQ) ? TB : 0;
+        const int nr = (q + 1 < NQ) ? TB + (ALDS ? 1 : 0) : 0;
         const int nv = (a_hi - a_lo) + (b_hi - b_lo);
         const int nm = (2 * q + 1 < HO) ? NM : TB;
 #pragma unroll
@@ -1159,8 +1221,17 @@ __global__ __launch_bounds__(64 * W * WN) void conv_direct_wgrad_spec_kernel(con
 #undef CCT_WSPEC_AVAL
     lds_dma_wait();
     __syncthreads();
+  };
+  // the loads of the last step of a range re-fetch that step into the idle stage
+  auto run = [&](auto stage_c, int s) { step(stage_c, scalars_of(min(s + 1, s_end - 1))); };
+  {
+    int s = s_beg;
+    for (; s + 1 < s_end; s += 2) {
+      run(std::integral_constant<int, 0>{}, s);
+      run(std::integral_constant<int, 1>{}, s + 1);
+    }
+    if (s < s_end) run(std::integral_constant<int, 0>{}, s);
   }
-#undef CCT_WSPEC_STEP
 #undef CCT_WSPEC_A
 #undef CCT_WSPEC_B
 
@@ -1260,6 +1331,7 @@ int reduce_partial_sums(float *dst, const float *ws, uint32_t n, float *dst2, co
 struct WgradPlan {
   int waves, tb, pw, ast, a_floats, stage;
   int wn;  // column groups of the workgroup's wavefront grid (specialised instances only, else 1)
+  bool alds;  // specialised instances: the dout rows are staged in LDS
   bool spec;  // a compile-time specialised instance exists for this shape
   size_t lds;
 };
@@ -1313,6 +1385,7 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
               (pl->waves == 4 || pl->waves == 6 || pl->waves == 8));
   if (tuning().direct_nospec) pl->spec = false;  // tuning override
   pl->wn = 1;
+  pl->alds = false;
   int nch_spec = nch;
   if (pl->spec) {
     // six row blocks: twelve wavefronts (six row blocks x two column groups of three blocks)
@@ -1325,6 +1398,10 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
     const int nt = 64 * pl->waves * pl->wn;
     pl->a_floats = 0;
     pl->stage = (nch_spec * pch + nt - 1) / nt * nt;
+    // 13-pixel rows: few MFMAs per row fetched, and a lane fetching its own row touches a cache line per load --
+    // measured faster staged in LDS for every 3 x 3 instance, slower for the 5 x 5 one (27-pixel rows)
+    pl->alds = tuning().direct_alds == 1 || (tuning().direct_alds == 0 && ks == 3);
+    if (pl->alds) pl->stage += 2 * ((32 * pl->waves * ho + nt - 1) / nt * nt);
   }
   // fragment loads may run a few words past the last patch row: the padding of the patch region
   // absorbs that, else a little slack is added
@@ -1333,15 +1410,20 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
   return pl->lds <= 160 * 1024;
 }
 
-template <int KS, int TB, int PW, int HO, int W, int WN = 1>
-static int wgrad_launch_spec(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
-  auto kern = conv_direct_wgrad_spec_kernel<KS, TB, PW, HO, W, WN>;
+template <int KS, int TB, int PW, int HO, int W, int WN, bool ALDS>
+static int wgrad_launch_spec_as(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
+  auto kern = conv_direct_wgrad_spec_kernel<KS, TB, PW, HO, W, WN, ALDS>;
   static LdsGrant grant;
   if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;
   hipLaunchKernelGGL(kern, dim3(g.nblocks), dim3(64 * W * WN), pl.lds, st, g);
   CCT_LAUNCH_CHECK();
-  note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d,%d>", KS, TB, PW, HO, W, WN);
+  note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d,%d,%d>", KS, TB, PW, HO, W, WN, ALDS ? 1 : 0);
   return 0;
+}
+template <int KS, int TB, int PW, int HO, int W, int WN = 1>
+static int wgrad_launch_spec(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
+  return pl.alds ? wgrad_launch_spec_as<KS, TB, PW, HO, W, WN, true>(g, pl, st)
+                 : wgrad_launch_spec_as<KS, TB, PW, HO, W, WN, false>(g, pl, st);
 }
 
 template <int KS, int PW>

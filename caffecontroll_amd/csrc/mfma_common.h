@@ -21,6 +21,10 @@ constexpr uint32_t kOutOfRange = 0x80000000u;
 __device__ __forceinline__ rsrc_t make_rsrc(const void *base) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)kOutOfRange, 0x00020000);
 }
+// a descriptor of size zero: every lane is out of range whatever its offset
+__device__ __forceinline__ rsrc_t make_rsrc_empty(const void *base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0, 0x00020000);
+}
 __device__ __forceinline__ void lds_dma16(rsrc_t r, uint32_t lane_bytes, uint32_t wave_bytes, float *lds_wave_base) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_void *)(uintptr_t)lds_wave_base, 16, lane_bytes, wave_bytes, 0, 0);
 }

@@ -103,7 +103,9 @@ int cct_hip_set_stream(void *hip_stream);
 /* Tuning knobs, for experiments and for tests that pin a kernel instance.  Names: "direct_tile"
  * (<map blocks><pixel blocks> of the direct convolution tile, 161 / 162 = its 16-row variant with 128 / 256
  * pixels, 0 = automatic), "direct_waves",
- * "direct_tb", "direct_nospec", "direct_splits" (step ranges of the direct weight-gradient launch, 0 = automatic), "pool_plane", "gemm_nt", "gemm_tile" (-1 = automatic), "gemm_nodma" (1 = GEMM
+ * "direct_tb", "direct_nospec", "direct_splits" (step ranges of the direct weight-gradient launch, 0 = automatic),
+ * "direct_alds" (shape-specialised weight-gradient kernels: 1 = output-gradient rows staged in LDS, 2 = fetched by
+ * their lanes, 0 = automatic), "pool_plane", "gemm_nt", "gemm_tile" (-1 = automatic), "gemm_nodma" (1 = GEMM
  * operand tiles always staged through registers).  The
  * environment variables CCT_HIP_<NAME IN CAPITALS> give the initial values; they are read once,
  * when the library initialises, never on a launch path.  No counterpart in the reference. */

@@ -538,3 +538,37 @@ def test_full_size_direct_vs_float64(cfg):
     assert worst_out / scale_out <= TOL
     assert worst_dx / scale_dx <= TOL
     assert err(dw, dw_ref) <= TOL
+
+
+# every specialised weight-gradient instance (8, 4, 6 x 2 wavefronts; 5x5 on 27 rows, 3x3 on 13), with map counts
+# that leave rows of the last tile empty, an odd batch (the last step holds one image) and two groups
+STAGED_ROWS = [(256, 96, 27, 5, 2, 256, 1), (64, 48, 27, 5, 2, 100, 1), (33, 48, 27, 5, 2, 128, 2),
+               (256, 256, 13, 3, 1, 384, 1), (255, 192, 13, 3, 1, 192, 1), (64, 64, 13, 3, 1, 250, 1),
+               (63, 128, 13, 3, 1, 170, 2), (256, 192, 13, 3, 1, 192, 2)]
+
+
+@pytest.mark.parametrize("cfg", STAGED_ROWS, ids=lambda c: "b%d_d%d_n%d_k%d_p%d_o%d_g%d" % c)
+def test_wgrad_rows_staged_in_lds_equal_rows_fetched_by_lanes(cfg):
+    """The shape-specialised weight-gradient kernels feed the MFMAs' output-gradient operand either from rows each
+    lane fetched itself or from rows staged in LDS: the same values in the same order of additions, so weight and
+    bias gradients agree bit for bit."""
+    import torch
+    b, d, n, k, p, o, groups = cfg
+    m = n + 2 * p - k + 1
+    drv = driver()
+    g = torch.Generator(device="cuda").manual_seed(99)
+    x = torch.randn((b, d * groups, n, n), device="cuda", generator=g)
+    og = torch.randn((b, o * groups, m, m), device="cuda", generator=g)
+    got = {}
+    for mode in (1, 2):
+        dw, db = empty((o * groups, d, k, k), fill=float("nan")), empty((o * groups,), fill=float("nan"))
+        with tuning("direct_alds", mode):
+            drv.conv_direct_backward_weights(dw, og, x, b, d * groups, n, k, p, o * groups, db=db, groups=groups)
+            names = drv.lib.cct_hip_last_kernel().decode()
+        torch.cuda.synchronize()
+        got[mode] = (host(dw), host(db), names)
+    assert "wgrad_spec_kernel" in got[1][2] and got[1][2].rstrip(">").endswith(",1"), got[1][2]
+    assert got[2][2].rstrip(">").endswith(",0"), got[2][2]
+    assert not np.isnan(got[1][0]).any() and not np.isnan(got[1][1]).any()
+    assert np.array_equal(got[1][0], got[2][0])
+    assert np.array_equal(got[1][1], got[2][1])
