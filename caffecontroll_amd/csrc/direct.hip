@@ -69,19 +69,28 @@ constexpr int kDirectPatchLoads = 8;  // source elements per lane per step, at m
 
 // Fragments of contraction index idx = cp*KS*KS + j (idx is a constant after unrolling): weights of
 // tap j of channel pair cp for TMB row blocks, source elements under tap j for TNB pixel blocks.
-template <int KS, int TMB, int TNB, int PW>
+// wa[cp][a] / pb[cp][b]: LDS word of this lane's first weight of row block a / first source element of pixel
+// block b, for channel pair cp, within the stage being read.
+template <int KS, int TMB, int TNB, int CP, int PW>
 __device__ __forceinline__ void direct_frags(float (&fa)[TMB], float (&fb)[TNB], const float *__restrict__ sm,
-                                             int abase, const int (&bbase)[TNB], int pair_stride, int idx) {
-  constexpr int KK = KS * KS, BM = 32 * TMB;
+                                             const int (&wa)[CP][TMB], const int (&pb)[CP][TNB], int idx) {
+  constexpr int KK = KS * KS;
   const int cp = idx / KK, j = idx % KK, u = j / KS, v = j % KS;
 #pragma unroll
-  for (int a = 0; a < TMB; ++a) fa[a] = sm[abase + cp * (2 * BM * KK) + a * (32 * KK) + j];
+  for (int a = 0; a < TMB; ++a) fa[a] = sm[wa[cp][a] + j];
 #pragma unroll
-  for (int b = 0; b < TNB; ++b) fb[b] = sm[bbase[b] + cp * pair_stride + u * PW + v];
+  for (int b = 0; b < TNB; ++b) fb[b] = sm[pb[cp][b] + u * PW + v];
+}
+
+// Wavefronts per SIMD the register allocation must leave room for, by accumulator blocks of the tile: the
+// workgroups resident on a compute unit are what hides the barrier of every step (and the tail of the grid),
+// so a tile must not lose a resident workgroup to a handful of address registers.
+constexpr int direct_waves_per_simd(int blocks) {
+  return blocks <= 1 ? 8 : blocks == 2 ? 7 : blocks == 3 ? 5 : blocks == 4 ? 4 : blocks <= 6 ? 3 : 2;
 }
 
 template <int KS, int TMB, int TNB, int CP, int PW>
-__global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g) {
+__global__ __launch_bounds__(256, direct_waves_per_simd(TMB * TNB)) void conv_direct_kernel(const DirectArgs g) {
   constexpr int KK = KS * KS, BM = 32 * TMB, BN = 128 * TNB, NC = 2 * CP;
   constexpr int ASZ = NC * BM * KK;           // floats of weight slabs per stage
   constexpr int ASZP = (ASZ + 255) / 256 * 256;  // LDS room for them: whole 64-lane 16-byte loads
@@ -124,9 +133,12 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
   for (int i = 0; i < NA4; ++i) {
     const int e4 = tid + i * 256;
     const int c = e4 / SLAB4, f = (e4 - c * SLAB4) * 4;
-    aoff[i] = (uint32_t)(c * g.slab_stride + f) * 4u;  // bytes
+    // bytes; the lanes past the slabs' end fill the padding of the LDS region with zeros
+    aoff[i] = e4 < ASZ / 4 ? (uint32_t)(c * g.slab_stride + f) * 4u : kOutOfRange;
   }
-  uint32_t psrc[NPL], psrc_last[NPL];  // byte offsets for any step / for the final step
+  // byte offsets; in the final step the lanes of channels past the last one fetch nothing (that test is redone
+  // where it is needed, in the final step's loads, rather than kept in a second set of registers)
+  uint32_t psrc[NPL];
   const int last_channels = g.kc - (g.nsteps - 1) * NC;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
@@ -139,7 +151,6 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     const bool ok = c < (uint32_t)NC && img < (uint32_t)g.batch && (unsigned)srow < (unsigned)g.hs &&
                     (unsigned)scol < (unsigned)g.hs;
     psrc[i] = ok ? (img * g.src_img_stride + (c * g.hs + srow) * g.hs + scol) * 4u : kOutOfRange;
-    psrc_last[i] = (ok && (int)c < last_channels) ? psrc[i] : kOutOfRange;
   }
   const uint32_t a_step = (uint32_t)NC * g.slab_stride * 4u, b_step = (uint32_t)NC * g.hs * g.hs * 4u;  // bytes
   const rsrc_t a_rsrc = make_rsrc(g.wt + (size_t)grp * g.wt_group_floats + (size_t)m0 * KK),
@@ -153,13 +164,15 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     const uint32_t ga_ = (uint32_t)(t) * a_step, gb_ = (uint32_t)(t) * b_step;                 \
     _Pragma("unroll") for (int i = 0; i < NA4; ++i) {                                          \
       if (i * 256 + wave_elem0 < ASZP / 4)                                                     \
-        lds_dma16(a_rsrc, (i * 256 + tid < ASZ / 4) ? aoff[i] : kOutOfRange, ga_,              \
-                  st_ + (i * 256 + wave_elem0) * 4);                                           \
+        lds_dma16(a_rsrc, aoff[i], ga_, st_ + (i * 256 + wave_elem0) * 4);                     \
     }                                                                                          \
     const bool last_ = (t) == g.nsteps - 1;                                                    \
     _Pragma("unroll") for (int i = 0; i < NPL; ++i) {                                          \
       if (i * 256 + wave_elem0 < psz)                                                          \
-        lds_dma4(b_rsrc, last_ ? psrc_last[i] : psrc[i], gb_, st_ + ASZP + i * 256 + wave_elem0); \
+        lds_dma4(b_rsrc,                                                                       \
+                 (last_ && (int)fdiv((uint32_t)(tid + i * 256) / PW, g.div_pr) >= last_channels) ? kOutOfRange \
+                                                                                                : psrc[i], \
+                 gb_, st_ + ASZP + i * 256 + wave_elem0);                                      \
     }                                                                                          \
   } while (0)
 
@@ -189,24 +202,74 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
   lds_dma_wait();
   __syncthreads();
 
-  for (int t = 0; t < g.nsteps; ++t) {
-    const float *sm = smem + (t & 1) * stage;
+  // Fragment addresses of both stages as registers of their own (seen as one base plus constants, they would be
+  // re-added before every read: the paired LDS read reaches 255 words beyond its address register).  Vector ALU
+  // instructions and MFMAs of one SIMD do not overlap, so address arithmetic in the loop is MFMA time lost.
+  int wa2[2][CP][TMB], pb2[2][CP][TNB];
+#pragma unroll
+  for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+    for (int cp = 0; cp < CP; ++cp) {
+#pragma unroll
+      for (int a = 0; a < TMB; ++a) {
+        wa2[s2][cp][a] = s2 * stage + abase + cp * (2 * BM * KK) + a * (32 * KK);
+        asm volatile("" : "+v"(wa2[s2][cp][a]));
+      }
+#pragma unroll
+      for (int b = 0; b < TNB; ++b) {
+        pb2[s2][cp][b] = s2 * stage + bbase[b] + cp * pair_stride;
+        asm volatile("" : "+v"(pb2[s2][cp][b]));
+      }
+    }
+
+  // One step.  FAST: the stage read is the compile-time constant P and the step fetched, t + 1, exists and is not
+  // the final one (its loads need no choice between the two offset sets); else the stage is t & 1 and the loads
+  // are chosen at run time.  The loop runs FAST steps in pairs and leaves the last two or three to the other form.
+  auto step = [&](auto fast_c, auto stage_c, int t) {
+    constexpr bool FAST = decltype(fast_c)::value;
+    constexpr int P = decltype(stage_c)::value;
     // every wave finished reading the other stage before the barrier that ended step t-1
-    if (t + 1 < g.nsteps) CCT_DIRECT_ISSUE(t + 1, (t & 1) ^ 1);
+    if constexpr (FAST) {
+      float *st_ = smem + (P ^ 1) * stage;
+      const uint32_t ga_ = (uint32_t)(t + 1) * a_step, gb_ = (uint32_t)(t + 1) * b_step;
+      // loads this wavefront makes per step (counts as scalar registers read afresh every step: a loop-invariant
+      // "does load i exist" flag would be kept as a lane mask and turned back into a branch with vector
+      // instructions)
+      int na_ = (ASZP / 4 - wave_elem0 + 255) / 256, np_ = (psz - wave_elem0 + 255) / 256;
+      asm volatile("" : "+s"(na_), "+s"(np_));
+#pragma unroll
+      for (int i = 0; i < NA4; ++i) {
+        if (__builtin_expect(i < na_, 1)) lds_dma16(a_rsrc, aoff[i], ga_, st_ + (i * 256 + wave_elem0) * 4);
+      }
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) {
+        if (__builtin_expect(i < np_, 1)) lds_dma4(b_rsrc, psrc[i], gb_, st_ + ASZP + i * 256 + wave_elem0);
+      }
+    } else {
+      if (t + 1 < g.nsteps) CCT_DIRECT_ISSUE(t + 1, (t & 1) ^ 1);
+    }
+    const float *sm = smem;
+    int wa[CP][TMB], pb[CP][TNB];
+#pragma unroll
+    for (int cp = 0; cp < CP; ++cp) {
+#pragma unroll
+      for (int a = 0; a < TMB; ++a)
+        wa[cp][a] = FAST ? wa2[P][cp][a] : (t & 1) * stage + abase + cp * (2 * BM * KK) + a * (32 * KK);
+#pragma unroll
+      for (int b = 0; b < TNB; ++b) pb[cp][b] = FAST ? pb2[P][cp][b] : (t & 1) * stage + bbase[b] + cp * pair_stride;
+    }
     // Contraction indices are taken two at a time (neighbouring taps sit in neighbouring LDS words,
     // which lets the compiler fetch both with one ds_read2); the fragments of pair q+1 are
     // requested before the MFMAs of pair q.
     constexpr int NI = CP * KK, NQ = (NI + 1) / 2;
     float fa[2][2][TMB], fb[2][2][TNB];
-    direct_frags<KS, TMB, TNB, PW>(fa[0][0], fb[0][0], sm, abase, bbase, pair_stride, 0);
-    if (NI > 1) direct_frags<KS, TMB, TNB, PW>(fa[0][1], fb[0][1], sm, abase, bbase, pair_stride, 1);
+    direct_frags<KS, TMB, TNB, CP, PW>(fa[0][0], fb[0][0], sm, wa, pb, 0);
+    if (NI > 1) direct_frags<KS, TMB, TNB, CP, PW>(fa[0][1], fb[0][1], sm, wa, pb, 1);
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
       const int nb = (q + 1) & 1, cb = q & 1;
-      if (2 * q + 2 < NI)
-        direct_frags<KS, TMB, TNB, PW>(fa[nb][0], fb[nb][0], sm, abase, bbase, pair_stride, 2 * q + 2);
-      if (2 * q + 3 < NI)
-        direct_frags<KS, TMB, TNB, PW>(fa[nb][1], fb[nb][1], sm, abase, bbase, pair_stride, 2 * q + 3);
+      if (2 * q + 2 < NI) direct_frags<KS, TMB, TNB, CP, PW>(fa[nb][0], fb[nb][0], sm, wa, pb, 2 * q + 2);
+      if (2 * q + 3 < NI) direct_frags<KS, TMB, TNB, CP, PW>(fa[nb][1], fb[nb][1], sm, wa, pb, 2 * q + 3);
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
         if (2 * q + e < NI) {
@@ -234,6 +297,14 @@ __global__ __launch_bounds__(256, 2) void conv_direct_kernel(const DirectArgs g)
     }
     lds_dma_wait();
     __syncthreads();
+  };
+  {
+    int t = 0;
+    for (; t + 3 < g.nsteps; t += 2) {
+      step(std::true_type{}, std::integral_constant<int, 0>{}, t);
+      step(std::true_type{}, std::integral_constant<int, 1>{}, t + 1);
+    }
+    for (; t < g.nsteps; ++t) step(std::false_type{}, std::integral_constant<int, 0>{}, t);
   }
 #undef CCT_DIRECT_ISSUE
 
@@ -576,12 +647,12 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   // blocks x 128 pixels; 6, 4, 3, 2 for 256 pixels); a wrong figure costs speed, not correctness.
   static const int reg_slots[5][3] = {{0, 0, 0}, {0, 8, 6}, {0, 7, 4}, {0, 5, 3}, {0, 4, 2}};
   static const double fill[4] = {1.0, 0.7, 0.93, 0.97};  // MFMA rate with 1, 2, 3 workgroups on a unit
-  // MFMA rate of an instance on a launch of many balanced rounds, relative to the best instance of its
-  // kernel size (measured on the CaffeNet layers at batch 256: conv3 / conv4 for k = 3, conv2 for k = 5).
-  // 64 x 128 and 32 x 256 tiles lead; 64 x 256 and the three- and four-block map tiles hold fewer
-  // wavefronts per SIMD and lose 6-15 %.
-  static const double rate3[5][3] = {{0, 0, 0}, {0, 0.965, 0.985}, {0, 1.0, 0.94}, {0, 0.895, 0.85}, {0, 0.91, 0.935}};
-  static const double rate5[5][3] = {{0, 0, 0}, {0, 0.977, 1.0}, {0, 0.987, 0.925}, {0, 0.98, 0.96}, {0, 0.85, 0.913}};
+  // MFMA rate of an instance relative to what the round count alone predicts: measured time of every instance
+  // against this estimate on the CaffeNet layers at batch 256 (conv3 / conv4 / conv5 forward and data gradient
+  // for k = 3, conv2 whole and in two groups for k = 5), averaged per instance.  The 32 x 128 tile leads for
+  // k = 3 (no vector ALU work is left in its step loop and eight workgroups share a compute unit).
+  static const double rate3[5][3] = {{0, 0, 0}, {0, 1.023, 0.983}, {0, 0.985, 0.982}, {0, 0.967, 1.043}, {0, 1.0, 1.042}};
+  static const double rate5[5][3] = {{0, 0, 0}, {0, 1.009, 1.017}, {0, 1.008, 0.975}, {0, 0.912, 1.022}, {0, 0.977, 1.03}};
   struct Candidate { DirectPlan plan; double cost; } cand[8];
   int ncand = 0;
   double best = -1;
