@@ -87,8 +87,12 @@ PROTOTYPES = {
     "cct_hip_copy_depth_slice": [_P, _P, _I, _I, _I, _I, _Z, _I],
     "cct_hip_sgemm": [_I, _I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I],
     "cct_hip_sgemm_new": [_I, _I, _I, _I, _I, _F, _P, _P, _F, _P],
+    "cct_hip_sgemm_new_colsum": [_I, _I, _I, _I, _I, _F, _P, _P, _F, _P, _P, _P, _I, _I],
     "cct_hip_sgemm_new_bias": [_I, _I, _I, _I, _I, _F, _P, _P, _F, _P, _P, _I],
     "cct_hip_sgemm_conv_forward": [_I, _I, _I, _I, _P, _P, _P, _P, _I],
+    "cct_hip_conv_small_supported": [_I, _I, _I, _I, _I, _I, _I],
+    "cct_hip_conv_small_forward": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I],
+    "cct_hip_conv_small_backward_weights": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I],
     "cct_hip_fc_small_supported": [_I, _I, _I],
     "cct_hip_fc_small_forward": [_P, _P, _P, _P, _I, _I, _I, _I],
     "cct_hip_fc_small_backward": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],

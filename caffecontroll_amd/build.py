@@ -12,7 +12,7 @@ from concurrent.futures import ThreadPoolExecutor
 PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(PKG, "csrc")
 LIB = os.path.join(PKG, "libcct_hip.so")
-SOURCES = ["api.hip", "lower.hip", "lift.hip", "gemm.hip", "fc_small.hip", "direct.hip", "strided.hip", "eltwise.hip", "corpus.hip", "bridge_capi.cpp"]
+SOURCES = ["api.hip", "lower.hip", "lift.hip", "gemm.hip", "fc_small.hip", "conv_small.hip", "direct.hip", "strided.hip", "eltwise.hip", "corpus.hip", "bridge_capi.cpp"]
 
 HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
 FLAGS = [

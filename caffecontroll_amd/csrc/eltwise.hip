@@ -5,6 +5,7 @@
 #include <cstring>
 
 #include "cct_common.h"
+#include "colsum.h"
 
 namespace cct {
 
@@ -169,25 +170,7 @@ __global__ __launch_bounds__(TPB) void bias_forward_flat_kernel(float *__restric
 __global__ __launch_bounds__(TPB) void bias_backward_fc_kernel(float *__restrict__ bias,
                                                                const float *__restrict__ og, int D, int B) {
   __shared__ float part[4][64];
-  const int lane = threadIdx.x & 63, q = threadIdx.x >> 6;
-  const int d = blockIdx.x * 64 + lane;
-  const int per = (B + 3) / 4, b0 = q * per, b1 = min(B, b0 + per);
-  float s = 0.0f;
-  if (d < D) {
-    const float *p = og + (size_t)b0 * D + d;
-    int b = b0;
-    for (; b + 8 <= b1; b += 8, p += (size_t)8 * D) {
-      float v[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) v[j] = p[(size_t)j * D];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) s += v[j];
-    }
-    for (; b < b1; ++b, p += D) s += *p;
-  }
-  part[q][lane] = s;
-  __syncthreads();
-  if (q == 0 && d < D) bias[d] = ((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane];
+  colsum_block(bias, og, D, B, blockIdx.x, part);
 }
 
 // ---- ReLU ----------------------------------------------------------------------------------

@@ -21,6 +21,7 @@
 #include <cstdlib>
 
 #include "cct_common.h"
+#include "colsum.h"
 #include "mfma_common.h"
 
 namespace cct {
@@ -612,12 +613,25 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
 
 // C = alpha * sum_z ws[z] + beta * C, z ascending (fixed order); then the optional column bias and clamp.
 // fmap > 0: the epilogue of the forward convolution instead (output permutation, bias per row, clamp).
+// Workgroups from `cs_first` on do an unrelated small job that rides along in this launch: the column sums of
+// cs.src (colsum.h).
+struct ColSumJob {
+  float *dst;
+  const float *src;
+  int rows, cols;
+};
+
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(float *__restrict__ C,
                                                             const float *__restrict__ ws, int M, int N,
                                                             int ldc, int splits, float alpha, float beta,
                                                             FastDiv div_n, const float *__restrict__ col_bias,
                                                             int relu, const float *__restrict__ row_bias, int fmap,
-                                                            FastDiv div_fmap) {
+                                                            FastDiv div_fmap, uint32_t cs_first, ColSumJob cs) {
+  __shared__ float cs_part[4][64];
+  if (blockIdx.x >= cs_first) {  // workgroup-uniform
+    colsum_block(cs.dst, cs.src, cs.cols, cs.rows, blockIdx.x - cs_first, cs_part);
+    return;
+  }
   const uint32_t e = blockIdx.x * 256 + threadIdx.x;
   if (e >= (uint32_t)M * N) return;
   const uint32_t row = fdiv(e, div_n);
@@ -687,10 +701,24 @@ static int launch_cfg(GemmArgs &g, bool a_kc, bool b_kc, int splits, hipStream_t
 
 // Row-major GEMM driver.  a_kc: A(m,k) = A[m*lda + k] (cblas NoTrans); b_kc: B(k,n) = B[n*ldb + k]
 // (cblas Trans).
+__global__ __launch_bounds__(256) void colsum_kernel(ColSumJob cs) {
+  __shared__ float part[4][64];
+  colsum_block(cs.dst, cs.src, cs.cols, cs.rows, blockIdx.x, part);
+}
+
+// `colsum`: column sums to compute beside the product, in the spare workgroups of the split-K reduction when
+// there is one, else in a launch of their own.
 static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha, const float *A, int lda,
                          const float *B, int ldb, float beta, float *C, int ldc, int epi, int fmap,
-                         const float *bias, int relu = 0, const float *col_bias = nullptr) {
-  if (M <= 0 || N <= 0) return 0;
+                         const float *bias, int relu = 0, const float *col_bias = nullptr,
+                         const ColSumJob *colsum = nullptr) {
+  if (M <= 0 || N <= 0) {
+    if (colsum && colsum->cols > 0) {
+      hipLaunchKernelGGL(colsum_kernel, dim3((uint32_t)((colsum->cols + 63) / 64)), dim3(256), 0, ctx().stream, *colsum);
+      CCT_LAUNCH_CHECK();
+    }
+    return 0;
+  }
   hipStream_t st = ctx().stream;
   GemmArgs g;
   g.A = A; g.B = B; g.C = C; g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb; g.ldc = ldc;
@@ -744,7 +772,7 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
       const long rem = n % sh.occ;
       double t = (double)(n / sh.occ) * sh.occ * w;
       if (rem) t += rem * w / (rem * 0.55 < 1.0 ? rem * 0.55 : 1.0);
-      if (sp > 1) t += 3e-6 + 8.0 * sp * (double)M * N / hbm_rate;  // partial sums out and back in
+      if (sp > 1) t += 5e-6 + 8.0 * sp * (double)M * N / hbm_rate;  // partial sums out and back in
       if (t < best) { best = t; cfg = c; splits = sp; kchunk = kc; }
     }
   }
@@ -772,9 +800,14 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   if (splits > 1) {
     CCT_REQUIRE((size_t)M * N < (1ull << 31), "sgemm: split-K result too large");
     const uint32_t blocks = (uint32_t)(((size_t)M * N + 255) / 256);
-    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, st, C, g.ws, M, N, ldc, splits,
+    const uint32_t extra = colsum && colsum->cols > 0 ? (uint32_t)((colsum->cols + 63) / 64) : 0u;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks + extra), dim3(256), 0, st, C, g.ws, M, N, ldc, splits,
                        alpha, beta, make_fastdiv((uint32_t)N), col_bias, relu, bias,
-                       epi == EPI_CONV_FORWARD ? g.fmap : 0, g.div_fmap);
+                       epi == EPI_CONV_FORWARD ? g.fmap : 0, g.div_fmap, blocks,
+                       colsum ? *colsum : ColSumJob{nullptr, nullptr, 0, 0});
+    CCT_LAUNCH_CHECK();
+  } else if (colsum && colsum->cols > 0) {
+    hipLaunchKernelGGL(colsum_kernel, dim3((uint32_t)((colsum->cols + 63) / 64)), dim3(256), 0, st, *colsum);
     CCT_LAUNCH_CHECK();
   }
   return 0;
@@ -813,6 +846,22 @@ extern "C" int cct_hip_sgemm_new(int TA, int TB, int M, int N, int K, float alph
   const int lda = (TA == CCT_NO_TRANS) ? K : M;
   const int ldb = (TB == CCT_NO_TRANS) ? N : K;
   return cct_hip_sgemm(CCT_ROW_MAJOR, TA, TB, M, N, K, alpha, A, lda, B, ldb, beta, C, N);
+}
+
+extern "C" int cct_hip_sgemm_new_colsum(int TA, int TB, int M, int N, int K, float alpha, const float *A,
+                                        const float *B, float beta, float *C, float *colsum, const float *colsum_src,
+                                        int rows, int cols) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE((TA == CCT_NO_TRANS || TA == CCT_TRANS) && (TB == CCT_NO_TRANS || TB == CCT_TRANS),
+              "sgemm_new_colsum: bad transpose flags %d %d", TA, TB);
+  CCT_REQUIRE(M >= 0 && N >= 0 && K >= 0 && rows >= 0 && cols >= 0, "sgemm_new_colsum: negative dimension");
+  CCT_REQUIRE((M == 0 || N == 0) || (A && B && C), "sgemm_new_colsum: null matrix");
+  CCT_REQUIRE(cols == 0 || (colsum && colsum_src), "sgemm_new_colsum: null column-sum argument");
+  const int lda = (TA == CCT_NO_TRANS) ? K : M;
+  const int ldb = (TB == CCT_NO_TRANS) ? N : K;
+  const ColSumJob job{colsum, colsum_src, rows, cols};
+  return gemm_rowmajor(TA == CCT_NO_TRANS, TB == CCT_TRANS, M, N, K, alpha, A, lda, B, ldb, beta, C, N,
+                       EPI_ALPHA_BETA, 0, nullptr, 0, nullptr, &job);
 }
 
 extern "C" int cct_hip_sgemm_new_bias(int TA, int TB, int M, int N, int K, float alpha, const float *A,

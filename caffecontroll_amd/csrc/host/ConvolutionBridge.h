@@ -136,6 +136,11 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                                  (int)num_output_features, (int)group);
     if (group > 1 && !direct_ok_)
       host_fail("ConvolutionBridge: a grouped convolution runs on the direct kernels only, which do not cover this geometry");
+    // one or three channels and a few maps (LeNet's first layer): plain multiply-add kernels for the forward pass and
+    // the weight gradient that read the model cube as it is (no slabs); they run where the all-direct path does
+    small_ok_ = direct_ok_ && group == 1 &&
+                p_driver->conv_small_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
+                                               (int)num_output_features);
     strided_ok_ = !direct_ok_ && group == 1 && p_driver->conv_strided_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride,
                                                                   (int)padding, (int)num_output_features);
     strided_data_ok_ = strided_ok_ && p_driver->conv_strided_backward_data_supported(
@@ -203,6 +208,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     views_ = true;
   }
   void set_fused(bool on) { set_path(on ? default_path_ : PATH_STAGED); }
+  // The plain multiply-add kernels for layers of one or three channels and few maps, on by default where they
+  // apply (on the all-direct path, on dense tensors); off: the MFMA direct kernels run such a layer too.
+  void set_small_kernels(bool on) { use_small_ = on; }
+  bool small_kernels() const { return small_ok_ && use_small_ && !views_; }
   // Apply the ReLU of a following in-place ReLUBridge (y = max(x, 0)) while the output is stored,
   // instead of in a pass of its own; the ReLU bridge then skips its forward.
   void set_fuse_relu(bool on) { fuse_relu_ = on; }
@@ -229,6 +238,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   bool supports_batch_ranges() const { return path_ == PATH_DIRECT_ALL && !views_; }
   // once per pass, before the first range: the weight slabs (the model changes between iterations)
   void forward_prepare() {
+    if (small_kernels())
+      return;  // reads the model cube itself
     if (strided_ok_)
       p_driver->conv_strided_slabs(forward_slabs()->get_p_data(), p_model_cube->get_p_data(),
                                    (int)num_output_features, (int)iD, (int)K, (int)stride, (int)padding);
@@ -241,7 +252,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     float *out = p_output_layer->p_data_cube->get_p_data() + b0 * out_img;
     const float *in = p_input_layer->p_data_cube->get_p_data() + b0 * in_img;
     const float *bias = bias_term ? p_bias_cube->get_p_data() : nullptr;
-    if (strided_ok_)
+    if (small_kernels())
+      p_driver->conv_small_forward(out, in, p_model_cube->get_p_data(), bias, (int)nb, (int)iD, (int)iR, (int)K,
+                                   (int)padding, (int)num_output_features, fuse_relu_);
+    else if (strided_ok_)
       p_driver->conv_strided_forward(out, in, forward_slabs()->get_p_data(), bias, (int)nb, (int)iD, (int)iR, (int)K,
                                      (int)stride, (int)padding, (int)num_output_features, fuse_relu_);
     else
@@ -283,7 +297,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     float *db = bias_term ? p_bias_gradient_cube->get_p_data() : nullptr;
     const float *og = p_output_layer->p_gradient_cube->get_p_data();
     const float *in = p_input_layer->p_data_cube->get_p_data();
-    if (strided_ok_)
+    if (small_kernels())
+      p_driver->conv_small_backward_weights(dw, db, og, in, (int)iB, (int)iD, (int)iR, (int)K, (int)padding,
+                                            (int)num_output_features);
+    else if (strided_ok_)
       p_driver->conv_strided_backward_weights(dw, db, og, in, (int)iB, (int)iD, (int)iR, (int)K, (int)stride,
                                               (int)padding, (int)num_output_features);
     else
@@ -307,6 +324,15 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                      forward_slabs()->get_p_data(), bias_term ? p_bias_cube->get_p_data() : nullptr,
                                      (int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
                                      (int)num_output_features, fuse_relu_);
+      end(STAGE_GEMM);
+      report_forward_history.end();
+      return;
+    }
+    if (path_ == PATH_DIRECT_ALL && small_kernels()) {
+      begin(STAGE_GEMM);
+      p_driver->conv_small_forward(output_d_cube->get_p_data(), input_d_cube->get_p_data(), p_model_cube->get_p_data(),
+                                   bias_term ? p_bias_cube->get_p_data() : nullptr, (int)iB, (int)iD, (int)iR, (int)K,
+                                   (int)padding, (int)num_output_features, fuse_relu_);
       end(STAGE_GEMM);
       report_forward_history.end();
       return;
@@ -409,6 +435,12 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                               output_g_cube->get_p_data(), p_input_layer->p_data_cube->get_p_data(),
                                               (int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
                                               (int)num_output_features);
+    } else if (direct_weights && small_kernels()) {
+      p_driver->conv_small_backward_weights(p_model_gradient_cube->get_p_data(),
+                                            bias_term ? p_bias_gradient_cube->get_p_data() : nullptr,
+                                            output_g_cube->get_p_data(), p_input_layer->p_data_cube->get_p_data(),
+                                            (int)iB, (int)iD, (int)iR, (int)K, (int)padding,
+                                            (int)num_output_features);
     } else if (direct_weights) {
       p_driver->conv_direct_backward_weights(p_model_gradient_cube->get_p_data(),
                                              bias_term ? p_bias_gradient_cube->get_p_data() : nullptr,
@@ -504,6 +536,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   bool views_ = false;
   bool fuse_relu_ = false;
   bool direct_ok_ = false, strided_ok_ = false, strided_data_ok_ = false, profile_ = false;
+  bool small_ok_ = false, use_small_ = true;
   LogicalCubeType *lowered() {
     if (!p_forward_lowered_data) p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
     return p_forward_lowered_data;

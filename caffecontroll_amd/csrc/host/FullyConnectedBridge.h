@@ -116,16 +116,19 @@ class FullyConnectedBridge : public AbstractBridge<DataType, DriverClass> {
       this->report_backward_updateweight_history.end();
       return;
     }
-    if (bias_term) {
+    if (bias_term && !needs_to_calc_backward_grad) {
       DeviceMemoryPointer output = output_g_cube->get_device_pointer(p_driver);
       DeviceMemoryPointer bias = p_bias_gradient_cube->get_device_pointer(p_driver);
       p_driver->backward_bias_fc(&bias, &output, (int)oD, (int)iB);
     }
     // the reference always computes the data gradient here (:306-308); it is skipped when the
-    // caller says the layer below does not need it
+    // caller says the layer below does not need it.  The bias gradient (the same bits as backward_bias_fc's) goes
+    // with it: both read the output gradient, and the product's reduction launch has workgroups to spare.
     if (needs_to_calc_backward_grad) {
-      p_driver->sgemm_new(CblasNoTrans, CblasNoTrans, data_R, model_C, model_R, 1.f, output_g_cube->get_p_data(),
-                          p_model_cube->get_p_data(), 0.f, input_g_cube->get_p_data());
+      p_driver->sgemm_new_colsum(CblasNoTrans, CblasNoTrans, data_R, model_C, model_R, 1.f, output_g_cube->get_p_data(),
+                                 p_model_cube->get_p_data(), 0.f, input_g_cube->get_p_data(),
+                                 bias_term ? p_bias_gradient_cube->get_p_data() : nullptr, output_g_cube->get_p_data(),
+                                 bias_term ? (int)iB : 0, bias_term ? (int)oD : 0);
       if (input_is_relu_output) {  // the GEMM has no store to fold the mask into
         DeviceMemoryPointer in_grad = input_g_cube->get_device_pointer(p_driver);
         p_driver->relu_backward(&in_grad, &in_grad, input_d_cube->get_p_data());

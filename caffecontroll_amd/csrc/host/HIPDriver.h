@@ -249,6 +249,13 @@ class HIPDriver {
                  const float alpha, const float *pA, const float *pB, const float beta, float *pC) {
     ok(cct_hip_sgemm_new(TA, TB, M, N, K, alpha, pA, pB, beta, pC), "sgemm_new");
   }
+  // sgemm_new, and beside it the column sums of a rows x cols matrix (an inner-product layer's bias gradient)
+  void sgemm_new_colsum(const CBLAS_TRANSPOSE TA, const CBLAS_TRANSPOSE TB, const int M, const int N, const int K,
+                        const float alpha, const float *pA, const float *pB, const float beta, float *pC,
+                        float *colsum, const float *colsum_src, int rows, int cols) {
+    ok(cct_hip_sgemm_new_colsum(TA, TB, M, N, K, alpha, pA, pB, beta, pC, colsum, colsum_src, rows, cols),
+       "sgemm_new_colsum");
+  }
   // sgemm_new with a bias per column of C and, optionally, the clamp of a following ReLU in the same pass
   void sgemm_new_bias(const CBLAS_TRANSPOSE TA, const CBLAS_TRANSPOSE TB, const int M, const int N, const int K,
                       const float alpha, const float *pA, const float *pB, const float beta, float *pC,
@@ -272,6 +279,20 @@ class HIPDriver {
                          int in_features, int out_features, const float *relu_data) {
     ok(cct_hip_fc_small_backward(dx, dw, db, dy, x, w, batch, in_features, out_features, relu_data),
        "fc_small_backward");
+  }
+  // ---- convolutions with a very short contraction and few maps (no counterpart in DeviceDriver.h) ----
+  bool conv_small_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs) {
+    return cct_hip_conv_small_supported(batch, depth, n, k, stride, padding, num_outputs) != 0;
+  }
+  void conv_small_forward(float *out, const float *in, const float *model, const float *bias, int batch, int depth,
+                          int n, int k, int padding, int num_outputs, bool relu) {
+    ok(cct_hip_conv_small_forward(out, in, model, bias, batch, depth, n, k, padding, num_outputs, relu ? 1 : 0),
+       "conv_small_forward");
+  }
+  void conv_small_backward_weights(float *dw, float *db, const float *dout, const float *in, int batch, int depth,
+                                   int n, int k, int padding, int num_outputs) {
+    ok(cct_hip_conv_small_backward_weights(dw, db, dout, in, batch, depth, n, k, padding, num_outputs),
+       "conv_small_backward_weights");
   }
   // `groups` > 1: a grouped convolution (depth and num_outputs are the layer's totals), all groups in one launch
   bool conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs,

@@ -120,6 +120,11 @@ class HIPDriver:
         check(self.lib.cct_hip_sgemm_new_bias(TA, TB, M, N, K, alpha, _p(A), _p(B), beta, _p(Cm), _p(col_bias),
                                               int(relu)), "sgemm_new_bias")
 
+    def sgemm_new_colsum(self, TA, TB, M, N, K, alpha, A, B, beta, Cm, colsum, colsum_src, rows, cols):
+        """sgemm_new, and beside it colsum[c] = sum over r of colsum_src[r][c] (rows x cols, dense)."""
+        check(self.lib.cct_hip_sgemm_new_colsum(TA, TB, M, N, K, alpha, _p(A), _p(B), beta, _p(Cm), _p(colsum),
+                                                _p(colsum_src), rows, cols), "sgemm_new_colsum")
+
     def sgemm_new(self, TA, TB, M, N, K, alpha, A, B, beta, Cm):
         check(self.lib.cct_hip_sgemm_new(TA, TB, M, N, K, alpha, _p(A), _p(B), beta, _p(Cm)), "sgemm_new")
 
@@ -138,6 +143,18 @@ class HIPDriver:
     def fc_small_backward(self, dx, dw, db, dy, x, w, batch, in_features, out_features, relu_data=None):
         check(self.lib.cct_hip_fc_small_backward(_p(dx), _p(dw), _p(db), _p(dy), _p(x), _p(w), batch, in_features,
                                                  out_features, _p(relu_data)), "fc_small_backward")
+
+    # -- convolutions with a very short contraction and few maps (LeNet conv1) -------------------
+    def conv_small_supported(self, b, d, n, k, s, p, o):
+        return bool(self.lib.cct_hip_conv_small_supported(b, d, n, k, s, p, o))
+
+    def conv_small_forward(self, out, x, w, bias, b, d, n, k, p, o, relu=False):
+        check(self.lib.cct_hip_conv_small_forward(_p(out), _p(x), _p(w), _p(bias), b, d, n, k, p, o, int(relu)),
+              "conv_small_forward")
+
+    def conv_small_backward_weights(self, dw, dout, x, b, d, n, k, p, o, db=None):
+        check(self.lib.cct_hip_conv_small_backward_weights(_p(dw), _p(db), _p(dout), _p(x), b, d, n, k, p, o),
+              "conv_small_backward_weights")
 
     # `groups` > 1: a grouped convolution (d and o are the layer's totals), all groups in one launch
     def conv_direct_supported(self, b, d, n, k, s, p, o, groups=1):

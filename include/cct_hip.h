@@ -204,6 +204,13 @@ int cct_hip_sgemm_new(int TA, int TB, int M, int N, int K, float alpha, const fl
  * relu != 0 also applies the ReLU of a following in-place ReLUBridge (max(x, 0),
  * src/kernels/relu.hxx:10-25) before the store.  The sums are those of the two separate calls, in
  * the same order: identical results. */
+/* sgemm_new, and beside it colsum[c] = sum over r of colsum_src[r][c] (rows x cols, dense row-major; rows ascending
+ * within four quarters that are added in order: the same bits as cct_hip_backward_bias_fc).  The two
+ * results are independent; the sums ride in spare workgroups of the product's reduction launch when it has one.
+ * For FullyConnectedBridge::backward, which computes the bias gradient and the data gradient from the same
+ * output gradient (src/bridges/FullyConnectedBridge_impl.hxx:268-308). */
+int cct_hip_sgemm_new_colsum(int TA, int TB, int M, int N, int K, float alpha, const float *A, const float *B,
+                             float beta, float *C, float *colsum, const float *colsum_src, int rows, int cols);
 int cct_hip_sgemm_new_bias(int TA, int TB, int M, int N, int K, float alpha, const float *A,
                            const float *B, float beta, float *C, const float *col_bias, int relu);
 /* Forward-convolution GEMM with the output permutation and bias of
@@ -229,6 +236,20 @@ int cct_hip_fc_small_forward(float *y, const float *x, const float *w, const flo
                              int in_features, int out_features, int relu);
 int cct_hip_fc_small_backward(float *dx, float *dw, float *db, const float *dy, const float *x, const float *w,
                               int batch, int in_features, int out_features, const float *relu_data);
+/* ---- convolutions with a very short contraction and few maps --------------------------------- */
+/* ConvolutionBridge::forward / ::backward (src/bridges/ConvolutionBridge_impl.hxx:294-373, 551-628) for stride-1
+ * layers with one or three input channels, k = 3 or 5 and at most 32 output maps (LeNet's first layer): lowering,
+ * GEMM, remap and bias of the forward pass as ONE launch that reads the model cube [o][d][k][k] as it is, and the
+ * weight and bias gradient as one launch plus the fixed-order sum of its per-image-group partial sums, in plain
+ * fp32 multiply-adds (k*k*d of 25 leaves a matrix-core tile mostly padding).  in [batch][d][n][n], out / dout
+ * [batch][o][m][m], all dense; bias / db may be NULL; relu != 0 clamps the output at zero.  Results agree with
+ * the other paths to fp32 rounding; run-to-run identical.  No data gradient (a first layer needs none; the
+ * other kernels provide it otherwise). */
+int cct_hip_conv_small_supported(int batch, int d, int n, int k, int stride, int pad, int o);
+int cct_hip_conv_small_forward(float *out, const float *in, const float *w, const float *bias, int batch, int d, int n,
+                               int k, int pad, int o, int relu);
+int cct_hip_conv_small_backward_weights(float *dw, float *db, const float *dout, const float *in, int batch, int d,
+                                        int n, int k, int pad, int o);
 /* ---- stride-1 convolution without the lowered matrix ------------------------------------ */
 /* Fused replacements for chains of ConvolutionBridge's lowering pipeline when stride == 1 and
  * k is 3 or 5 (padded image at most 32 wide).  Results agree with the lowering path to fp32

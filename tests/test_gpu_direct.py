@@ -572,3 +572,59 @@ def test_wgrad_rows_staged_in_lds_equal_rows_fetched_by_lanes(cfg):
     assert not np.isnan(got[1][0]).any() and not np.isnan(got[1][1]).any()
     assert np.array_equal(got[1][0], got[2][0])
     assert np.array_equal(got[1][1], got[2][1])
+
+
+# (batch, channels, size, kernel, pad, maps): LeNet's first layer, RGB inputs, every pad of a 3 x 3 and a 5 x 5 filter,
+# one map, the most maps, batches that do not divide into the image groups of the weight-gradient launch
+SMALL = [(64, 1, 28, 5, 0, 20), (7, 3, 17, 3, 1, 32), (5, 3, 12, 5, 2, 9), (3, 1, 9, 3, 2, 1), (33, 1, 8, 5, 4, 5),
+         (1, 3, 5, 5, 0, 2), (600, 1, 6, 3, 0, 3)]
+
+
+@pytest.mark.parametrize("shape", SMALL, ids=lambda c: "b%d_d%d_n%d_k%d_p%d_o%d" % c)
+def test_small_convolution_kernels_match_oracle(oracle, shape):
+    """The multiply-add kernels for layers of one or three channels and few maps: forward (with and without bias
+    and ReLU) and weight / bias gradient against the oracle's lowering + GEMM; two runs bit-identical."""
+    b, d, n, k, p, o = shape
+    drv = driver()
+    assert drv.conv_small_supported(b, d, n, k, 1, p, o)
+    m = n + 2 * p - k + 1
+    rng = np.random.default_rng(sum(shape))
+    x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+    w = (rng.standard_normal((o, d, k, k)) * 0.2).astype(np.float32)
+    bias = rng.standard_normal(o).astype(np.float32)
+    og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+    ref_out, low = oracle.conv_forward(x, w, bias, k, 1, p)
+    _, ref_dw, ref_db = oracle.conv_backward(x.shape, w, og, low, k, 1, p, need_in_grad=False)
+    dx_, dw_, dog = dev(x), dev(w), dev(og)
+    out = empty((b, o, m, m), fill=float("nan"))
+    drv.conv_small_forward(out, dx_, dw_, dev(bias), b, d, n, k, p, o)
+    assert rel_err(host(out), ref_out) <= TOL
+    drv.conv_small_forward(out, dx_, dw_, dev(bias), b, d, n, k, p, o, relu=True)
+    assert rel_err(host(out), np.maximum(ref_out, 0)) <= TOL
+    ref_nobias, _ = oracle.conv_forward(x, w, None, k, 1, p)
+    drv.conv_small_forward(out, dx_, dw_, None, b, d, n, k, p, o)
+    assert rel_err(host(out), ref_nobias) <= TOL
+    runs = []
+    for _ in range(2):
+        gw, gb = empty((o, d, k, k), fill=float("nan")), empty((o,), fill=float("nan"))
+        drv.conv_small_backward_weights(gw, dog, dx_, b, d, n, k, p, o, db=gb)
+        runs.append((host(gw), host(gb)))
+    assert rel_err(runs[0][0], ref_dw.reshape(o, d, k, k)) <= TOL
+    assert rel_err(runs[0][1], ref_db.reshape(o)) <= TOL
+    assert np.array_equal(runs[0][0], runs[1][0]) and np.array_equal(runs[0][1], runs[1][1])
+    gw = empty((o, d, k, k), fill=float("nan"))
+    drv.conv_small_backward_weights(gw, dog, dx_, b, d, n, k, p, o)    # no bias gradient wanted
+    assert np.array_equal(host(gw), runs[0][0])
+
+
+def test_small_convolution_support_and_errors():
+    drv = driver()
+    assert not drv.conv_small_supported(4, 2, 12, 5, 1, 0, 8)      # two channels
+    assert not drv.conv_small_supported(4, 1, 12, 5, 2, 0, 8)      # strided
+    assert not drv.conv_small_supported(4, 1, 12, 7, 1, 0, 8)      # 7 x 7
+    assert not drv.conv_small_supported(4, 1, 12, 5, 1, 0, 33)     # too many maps
+    assert not drv.conv_small_supported(4, 1, 3, 5, 1, 0, 8)       # filter larger than the padded image
+    assert not drv.conv_small_supported(4, 1, 12, 5, 1, 5, 8)      # pad >= k
+    from caffecontroll_amd import CctHipError
+    with pytest.raises(CctHipError, match="not covered"):
+        drv.conv_small_forward(empty((4, 8, 8, 8)), empty((4, 2, 12, 12)), empty((8, 2, 5, 5)), None, 4, 2, 12, 5, 0, 8)

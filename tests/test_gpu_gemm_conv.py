@@ -411,3 +411,28 @@ def test_full_size_conv_against_torch_fp64(shape):
     assert err(dx, x64.grad) <= TOL
     assert err(dw.reshape(o, d, k, k), w64.grad) <= TOL
     assert err(db, b64.grad) <= TOL
+
+
+@pytest.mark.parametrize("shape", [(64, 800, 500, 64, 500), (256, 4096, 4096, 256, 4096), (3, 5, 7, 9, 70),
+                                   (128, 128, 64, 33, 129), (0, 5, 7, 4, 3)],
+                         ids=lambda s: "m%d_n%d_k%d_rows%d_cols%d" % s)
+def test_sgemm_new_with_column_sums(shape):
+    """The product with the column sums of another matrix beside it (an inner-product layer's data gradient with its
+    bias gradient): the product equals sgemm_new's and the sums equal backward_bias_fc's, bit for bit, whether the
+    product's launch has a reduction to carry them or not."""
+    M, N, K, rows, cols = shape
+    drv = driver()
+    rng = np.random.default_rng(sum(shape))
+    a = rng.standard_normal((M, K)).astype(np.float32)
+    b = rng.standard_normal((K, N)).astype(np.float32)
+    src = rng.standard_normal((rows, cols)).astype(np.float32)
+    da, db, dsrc = dev(a), dev(b), dev(src)
+    c0, c1 = empty((M, N), fill=float("nan")), empty((M, N), fill=float("nan"))
+    s0, s1 = empty((cols,), fill=float("nan")), empty((cols,), fill=float("nan"))
+    if M:
+        drv.sgemm_new(111, 111, M, N, K, 1.0, da, db, 0.0, c0)
+    drv.backward_bias_fc(s0, dsrc, cols, rows)
+    drv.sgemm_new_colsum(111, 111, M, N, K, 1.0, da, db, 0.0, c1, s1, dsrc, rows, cols)
+    assert np.array_equal(host(c0), host(c1), equal_nan=True)
+    assert np.array_equal(host(s0), host(s1))
+    assert rel_err(host(s1), src.astype(np.float64).sum(axis=0)) <= 1e-5
