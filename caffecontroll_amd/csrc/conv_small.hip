@@ -23,10 +23,6 @@ namespace cct {
 
 constexpr int kConvSmallMaxMaps = 32;
 constexpr int CS_THREADS = 256;
-#ifndef CCT_CS_MG
-#define CCT_CS_MG 1
-#define CCT_CS_U 3
-#endif
 
 // Sum over the 64 lanes of a wavefront, valid in lane 63, as data-parallel-primitive moves (no LDS traffic):
 // neighbours within quads, quads within rows of 16 (half-row and row mirrors), then row 0 -> 1, 2 -> 3 and
@@ -212,7 +208,9 @@ static int conv_small_wgrad_launch(float *dw, float *db, const float *dout, cons
   constexpr int DKK = D * KS * KS;
   // maps per workgroup and pixels per lane and trip: what the register file holds (MG * (DKK + 1) sums,
   // U * (DKK + MG) loaded values)
-  constexpr int MG = DKK <= 27 ? CCT_CS_MG : 1, U = DKK <= 27 ? CCT_CS_U : 1;
+  // (measured on LeNet's first layer: more maps per workgroup save loads but serialise more lane sums per
+  // wavefront -- four maps cost 15 us against 12 us for one)
+  constexpr int MG = 1, U = DKK <= 27 ? 3 : 1;
   static_assert(MG * (DKK + 1) <= CS_THREADS, "one lane per sum of the workgroup");
   const int m = n + 2 * pad - KS + 1;
   // groups of whole images
@@ -231,7 +229,7 @@ static int conv_small_wgrad_launch(float *dw, float *db, const float *dout, cons
                      ctx().stream, part, part_bias, dout, in, batch, n, pad, o, m, per, make_fastdiv((uint32_t)(m * m)),
                      make_fastdiv((uint32_t)m));
   CCT_LAUNCH_CHECK();
-  note_kernel("conv_small_wgrad_kernel<%d,%d> groups=%d", KS, D, groups);
+  note_kernel("conv_small_wgrad_kernel<%d,%d,%d,%d> groups=%d", KS, D, MG, U, groups);
   return reduce_partial_sums(dw, part, (uint32_t)(o * DKK), db, part_bias, db ? (uint32_t)o : 0u, groups, ctx().stream);
 }
 

@@ -1488,7 +1488,7 @@ static int wgrad_launch_spec_as(const WgradArgs &g, const WgradPlan &pl, hipStre
   if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;
   hipLaunchKernelGGL(kern, dim3(g.nblocks), dim3(64 * W * WN), pl.lds, st, g);
   CCT_LAUNCH_CHECK();
-  note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d,%d,%d>", KS, TB, PW, HO, W, WN, ALDS ? 1 : 0);
+  note_kernel("conv_direct_wgrad_spec_kernel<%d,%d,%d,%d,%d,%d,%s>", KS, TB, PW, HO, W, WN, ALDS ? "true" : "false");
   return 0;
 }
 template <int KS, int TB, int PW, int HO, int W, int WN = 1>

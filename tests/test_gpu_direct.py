@@ -567,8 +567,8 @@ def test_wgrad_rows_staged_in_lds_equal_rows_fetched_by_lanes(cfg):
             names = drv.lib.cct_hip_last_kernel().decode()
         torch.cuda.synchronize()
         got[mode] = (host(dw), host(db), names)
-    assert "wgrad_spec_kernel" in got[1][2] and got[1][2].rstrip(">").endswith(",1"), got[1][2]
-    assert got[2][2].rstrip(">").endswith(",0"), got[2][2]
+    assert "wgrad_spec_kernel" in got[1][2] and got[1][2].endswith(",true>"), got[1][2]
+    assert got[2][2].endswith(",false>"), got[2][2]
     assert not np.isnan(got[1][0]).any() and not np.isnan(got[1][1]).any()
     assert np.array_equal(got[1][0], got[2][0])
     assert np.array_equal(got[1][1], got[2][1])
