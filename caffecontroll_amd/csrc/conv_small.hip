@@ -165,7 +165,7 @@ __global__ __launch_bounds__(CS_THREADS) void conv_small_wgrad_kernel(float *__r
   for (int g = 0; g < MG; ++g)
 #pragma unroll
     for (int j = 0; j <= DKK; ++j) {
-      const float v = conv_small_wave_sum(j < DKK ? acc[g][j < DKK ? j : 0] : bsum[g]);
+      const float v = conv_small_wave_sum(j < DKK ? acc[g][j % DKK] : bsum[g]);
       if ((tid & 63) == 63) red[tid >> 6][g][j] = v;
     }
   __syncthreads();

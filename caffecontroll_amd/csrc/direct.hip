@@ -655,7 +655,6 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   static const double rate5[5][3] = {{0, 0, 0}, {0, 1.009, 1.017}, {0, 1.008, 0.975}, {0, 0.912, 1.022}, {0, 0.977, 1.03}};
   struct Candidate { DirectPlan plan; double cost; } cand[8];
   int ncand = 0;
-  double best = -1;
   for (int tmb = 4; tmb >= 1; --tmb) {
     if (padded % (32 * tmb)) continue;
     const long tiles_m = padded / (32 * tmb);
@@ -681,14 +680,12 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
       c.plan.ks = ks; c.plan.tmb = tmb; c.plan.tnb = tnb; c.plan.cp = cp; c.plan.pw = pw; c.plan.pr = pr;
       c.plan.lds = lds;
       c.cost = cost;
-      if (best < 0 || cost < best) best = cost;
     }
   }
   if (ncand == 0) return false;
   const Candidate *pick = nullptr;
   for (int i = 0; i < ncand; ++i)
     if (!pick || cand[i].cost < pick->cost) pick = &cand[i];
-  (void)best;
   *pl = pick->plan;
   pl->tm16 = 0;
   return true;

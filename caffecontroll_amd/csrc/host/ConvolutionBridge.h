@@ -26,7 +26,11 @@
 //     network builder realises as towers between a Split and a Concat, src/DeepNet.h:1700-1757) is
 //     run by this one bridge: the model cube is [o][d/group][k][k] (the blob layout Caffe gives such
 //     a layer), group q maps its slice of the input channels to its slice of the output maps, and the
-//     direct kernels run all groups in one launch each.  Only the all-direct path covers it.
+//     direct kernels run all groups in one launch each.  Only the all-direct path covers it;
+//   * stride-1 layers with one or three input channels, k = 3 or 5 and at most 32 maps (LeNet's first
+//     layer) take plain multiply-add kernels for the forward pass and the weight gradient where they
+//     would take the all-direct path (set_small_kernels): the forward launch reads the model cube as it
+//     is, so no slabs are built for it.
 #pragma once
 #include <cstdio>
 #include <cstdlib>
