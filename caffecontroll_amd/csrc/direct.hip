@@ -341,19 +341,27 @@ __global__ __launch_bounds__(256, direct_waves_per_simd(TMB * TNB)) void conv_di
 // wavefront owns 2*TNB blocks of 16 consecutive pixels.
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// wavefronts per SIMD the register allocation must leave room for, by accumulator registers of the tile (what the
+// instances held before their fragment addresses became registers)
+constexpr int direct16_waves_per_simd(int acc_regs) {
+  return acc_regs <= 8 ? 8 : acc_regs <= 16 ? 6 : acc_regs <= 24 ? 5 : acc_regs <= 48 ? 4 : acc_regs <= 80 ? 3 : 2;
+}
+
+// wa[a] / pb[b]: LDS word of this lane's first weight of row block a / first source element of pixel block b within
+// the stage being read.
 template <int KS, int TM16, int NB, int PW>
 __device__ __forceinline__ void direct16_frags(float (&fa)[TM16], float (&fb)[NB], const float *__restrict__ sm,
-                                               int abase, const int (&bbase)[NB], int j) {
-  constexpr int KK = KS * KS;
+                                               const int (&wa)[TM16], const int (&pb)[NB], int j) {
   const int u = j / KS, v = j % KS;
 #pragma unroll
-  for (int a = 0; a < TM16; ++a) fa[a] = sm[abase + a * (16 * KK) + j];
+  for (int a = 0; a < TM16; ++a) fa[a] = sm[wa[a] + j];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) fb[b] = sm[bbase[b] + u * PW + v];
+  for (int b = 0; b < NB; ++b) fb[b] = sm[pb[b] + u * PW + v];
 }
 
 template <int KS, int TM16, int TNB, int PW>
-__global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs g) {
+__global__ __launch_bounds__(256, direct16_waves_per_simd(TM16 * 2 * TNB * 4)) void conv_direct16_kernel(
+    const DirectArgs g) {
   constexpr int KK = KS * KS, BM = 16 * TM16, BN = 128 * TNB, NC = 4, NB = 2 * TNB;
   constexpr int ASZ = NC * BM * KK;
   constexpr int ASZP = (ASZ + 255) / 256 * 256;
@@ -385,9 +393,12 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
   for (int i = 0; i < NA4; ++i) {
     const int e4 = tid + i * 256;
     const int c = e4 / SLAB4, f = (e4 - c * SLAB4) * 4;
-    aoff[i] = (uint32_t)(c * g.slab_stride + f) * 4u;
+    // bytes; the lanes past the slabs' end fill the padding of the LDS region with zeros
+    aoff[i] = e4 < ASZ / 4 ? (uint32_t)(c * g.slab_stride + f) * 4u : kOutOfRange;
   }
-  uint32_t psrc[NPL], psrc_last[NPL];
+  // byte offsets; in the final step the lanes of channels past the last one fetch nothing (tested where it is
+  // needed, in the final step's loads)
+  uint32_t psrc[NPL];
   const int last_channels = g.kc - (g.nsteps - 1) * NC;
 #pragma unroll
   for (int i = 0; i < NPL; ++i) {
@@ -400,7 +411,6 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
     const bool ok = c < (uint32_t)NC && prow < (uint32_t)g.pr && img < (uint32_t)g.batch && (unsigned)srow < (unsigned)g.hs &&
                     (unsigned)scol < (unsigned)g.hs;
     psrc[i] = ok ? (img * g.src_img_stride + (c * g.hs + srow) * g.hs + scol) * 4u : kOutOfRange;
-    psrc_last[i] = (ok && (int)c < last_channels) ? psrc[i] : kOutOfRange;
   }
   const uint32_t a_step = (uint32_t)NC * g.slab_stride * 4u, b_step = (uint32_t)NC * g.hs * g.hs * 4u;
   const rsrc_t a_rsrc = make_rsrc(g.wt + (size_t)grp * g.wt_group_floats),
@@ -413,13 +423,14 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
     const uint32_t ga_ = (uint32_t)(t) * a_step, gb_ = (uint32_t)(t) * b_step;                 \
     _Pragma("unroll") for (int i = 0; i < NA4; ++i) {                                          \
       if (i * 256 + wave_elem0 < ASZP / 4)                                                     \
-        lds_dma16(a_rsrc, (i * 256 + tid < ASZ / 4) ? aoff[i] : kOutOfRange, ga_,              \
-                  st_ + (i * 256 + wave_elem0) * 4);                                           \
+        lds_dma16(a_rsrc, aoff[i], ga_, st_ + (i * 256 + wave_elem0) * 4);                     \
     }                                                                                          \
     const bool last_ = (t) == g.nsteps - 1;                                                    \
     _Pragma("unroll") for (int i = 0; i < NPL; ++i) {                                          \
       if (i * 256 + wave_elem0 < psz)                                                          \
-        lds_dma4(b_rsrc, last_ ? psrc_last[i] : psrc[i], gb_, st_ + ASZP + i * 256 + wave_elem0); \
+        lds_dma4(b_rsrc,                                                                       \
+                 (last_ && (int)fdiv((uint32_t)(tid + i * 256), g.div_cs) >= last_channels) ? kOutOfRange : psrc[i], \
+                 gb_, st_ + ASZP + i * 256 + wave_elem0);                                      \
     }                                                                                          \
   } while (0)
 
@@ -447,20 +458,59 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
   lds_dma_wait();
   __syncthreads();
 
-  for (int t = 0; t < g.nsteps; ++t) {
-    const float *sm = smem + (t & 1) * stage;
-    if (t + 1 < g.nsteps) CCT_DIRECT16_ISSUE(t + 1, (t & 1) ^ 1);
+  // Fragment addresses of both stages as registers of their own, the step loop in pairs with the stage a
+  // compile-time constant, scalar load counts: as in conv_direct_kernel, no vector ALU instruction is left in the loop.
+  int wa2[2][TM16], pb2[2][NB];
+#pragma unroll
+  for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+    for (int a = 0; a < TM16; ++a) {
+      wa2[s2][a] = s2 * stage + abase + a * (16 * KK);
+      asm volatile("" : "+v"(wa2[s2][a]));
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      pb2[s2][b] = s2 * stage + bbase[b];
+      asm volatile("" : "+v"(pb2[s2][b]));
+    }
+  }
+
+  auto step = [&](auto fast_c, auto stage_c, int t) {
+    constexpr bool FAST = decltype(fast_c)::value;
+    constexpr int P = decltype(stage_c)::value;
+    if constexpr (FAST) {
+      float *st_ = smem + (P ^ 1) * stage;
+      const uint32_t ga_ = (uint32_t)(t + 1) * a_step, gb_ = (uint32_t)(t + 1) * b_step;
+      int na_ = (ASZP / 4 - wave_elem0 + 255) / 256, np_ = (psz - wave_elem0 + 255) / 256;
+      asm volatile("" : "+s"(na_), "+s"(np_));
+#pragma unroll
+      for (int i = 0; i < NA4; ++i) {
+        if (__builtin_expect(i < na_, 1)) lds_dma16(a_rsrc, aoff[i], ga_, st_ + (i * 256 + wave_elem0) * 4);
+      }
+#pragma unroll
+      for (int i = 0; i < NPL; ++i) {
+        if (__builtin_expect(i < np_, 1)) lds_dma4(b_rsrc, psrc[i], gb_, st_ + ASZP + i * 256 + wave_elem0);
+      }
+    } else {
+      if (t + 1 < g.nsteps) CCT_DIRECT16_ISSUE(t + 1, (t & 1) ^ 1);
+    }
+    const float *sm = smem;
+    int wa[TM16], pb[NB];
+#pragma unroll
+    for (int a = 0; a < TM16; ++a) wa[a] = FAST ? wa2[P][a] : (t & 1) * stage + abase + a * (16 * KK);
+#pragma unroll
+    for (int b = 0; b < NB; ++b) pb[b] = FAST ? pb2[P][b] : (t & 1) * stage + bbase[b];
     // taps two at a time (neighbouring taps sit in neighbouring LDS words); the fragments of pair
     // n+1 are requested before the MFMAs of pair n
     constexpr int NI = KK, NQ = (NI + 1) / 2;
     float fa[2][2][TM16], fb[2][2][NB];
-    direct16_frags<KS, TM16, NB, PW>(fa[0][0], fb[0][0], sm, abase, bbase, 0);
-    direct16_frags<KS, TM16, NB, PW>(fa[0][1], fb[0][1], sm, abase, bbase, 1);
+    direct16_frags<KS, TM16, NB, PW>(fa[0][0], fb[0][0], sm, wa, pb, 0);
+    direct16_frags<KS, TM16, NB, PW>(fa[0][1], fb[0][1], sm, wa, pb, 1);
 #pragma unroll
     for (int n = 0; n < NQ; ++n) {
       const int nb = (n + 1) & 1, cb = n & 1;
-      if (2 * n + 2 < NI) direct16_frags<KS, TM16, NB, PW>(fa[nb][0], fb[nb][0], sm, abase, bbase, 2 * n + 2);
-      if (2 * n + 3 < NI) direct16_frags<KS, TM16, NB, PW>(fa[nb][1], fb[nb][1], sm, abase, bbase, 2 * n + 3);
+      if (2 * n + 2 < NI) direct16_frags<KS, TM16, NB, PW>(fa[nb][0], fb[nb][0], sm, wa, pb, 2 * n + 2);
+      if (2 * n + 3 < NI) direct16_frags<KS, TM16, NB, PW>(fa[nb][1], fb[nb][1], sm, wa, pb, 2 * n + 3);
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
         if (2 * n + e < NI) {
@@ -484,6 +534,14 @@ __global__ __launch_bounds__(256, 2) void conv_direct16_kernel(const DirectArgs 
     }
     lds_dma_wait();
     __syncthreads();
+  };
+  {
+    int t = 0;
+    for (; t + 3 < g.nsteps; t += 2) {
+      step(std::true_type{}, std::integral_constant<int, 0>{}, t);
+      step(std::true_type{}, std::integral_constant<int, 1>{}, t + 1);
+    }
+    for (; t < g.nsteps; ++t) step(std::false_type{}, std::integral_constant<int, 0>{}, t);
   }
 #undef CCT_DIRECT16_ISSUE
 
