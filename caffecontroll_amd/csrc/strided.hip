@@ -444,6 +444,37 @@ __global__ __launch_bounds__(256, 4) void conv_strided_reg_kernel(const StridedR
   // ---- epilogue: accumulator register v of lane (r,h) is row 8*(v/4) + 4*h + v%4, column r ----
   const uint32_t pe = p0 + wave * 32 + r;
   if (pe >= g.ptot) return;
+  if (m0 + BM <= g.mtot) {
+    // Every row of the tile exists (always, when the map count is a multiple of the tile: conv1's 96).  With a
+    // contraction of only k*k*d = 363 the tile runs 183 MFMAs per channel, so the address arithmetic of 16 * TMB
+    // stores per lane is a visible share of the kernel: here each store is one buffer store whose lane offset is
+    // the same for all of them (row m0 + 4h at the lane's pixel) and whose row offset is a scalar; the bias comes in
+    // as 16-byte loads of the four consecutive rows a lane holds per accumulator quarter.
+    const rsrc_t o_rsrc = make_rsrc(g.dst);
+    const uint32_t voff = (uint32_t)((((size_t)img * g.mtot + m0 + 4 * h) * ho2 + pix) * 4u);
+    const uint32_t plane = (uint32_t)ho2 * 4u;
+    f4 bq[TMB][4];
+    if (g.bias) {
+      const rsrc_t bias_rsrc = make_rsrc(g.bias);
+#pragma unroll
+      for (int a = 0; a < TMB; ++a)
+#pragma unroll
+        for (int qv = 0; qv < 4; ++qv)
+          bq[a][qv] = __builtin_bit_cast(f4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                 bias_rsrc, 16u * h, (uint32_t)(m0 + a * 32 + 8 * qv) * 4u, 0));
+    }
+#pragma unroll
+    for (int a = 0; a < TMB; ++a)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        float yv = acc[a][v];
+        if (g.bias) yv += bq[a][v / 4][v % 4];
+        if (g.relu) yv = (yv > 0.f) ? yv : 0.f;
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, yv), o_rsrc, voff,
+                                              (uint32_t)(a * 32 + 8 * (v / 4) + (v % 4)) * plane, 0);
+      }
+    return;
+  }
   float *out = g.dst + (size_t)img * g.mtot * ho2 + pix;
   float bv[TMB][16];
 #pragma unroll
