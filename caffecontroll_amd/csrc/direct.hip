@@ -65,7 +65,10 @@ struct DirectArgs {
 
 constexpr int kDirect16PatchLoads = 11;  // the 16-row kernel stages four channels per step
 
-constexpr int kDirectPatchLoads = 8;  // source elements per lane per step, at most
+// source elements per lane per step, at most, by patch row length: eight for rows of up to 64 floats; rows of 128
+// and 256 floats (images wider than 64) hold as many source rows in more loads
+constexpr int kDirectPatchLoads = 8;
+constexpr int direct_patch_loads(int pw) { return pw <= 64 ? kDirectPatchLoads : pw == 128 ? 16 : 24; }
 
 // Fragments of contraction index idx = cp*KS*KS + j (idx is a constant after unrolling): weights of
 // tap j of channel pair cp for TMB row blocks, source elements under tap j for TNB pixel blocks.
@@ -96,7 +99,7 @@ __global__ __launch_bounds__(256, direct_waves_per_simd(TMB * TNB)) void conv_di
   constexpr int ASZP = (ASZ + 255) / 256 * 256;  // LDS room for them: whole 64-lane 16-byte loads
   constexpr int SLAB4 = BM * KK / 4;          // 16-byte vectors per slab
   constexpr int NA4 = (ASZP / 4 + 255) / 256;  // 16-byte vectors per lane per stage
-  constexpr int NPL = kDirectPatchLoads;
+  constexpr int NPL = direct_patch_loads(PW);
   extern __shared__ __attribute__((aligned(16))) float smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -665,8 +668,8 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   if (pad < 0 || pad > ks - 1 || batch <= 0 || kc <= 0 || mtot <= 0 || groups <= 0) return false;
   const int ho = hs + 2 * pad - ks + 1, hp = ho + ks - 1;
   if (ho <= 0) return false;
-  // padded rows of up to 32 floats; up to 64 on the 16-row kernel
-  const int pw = hp <= 16 ? 16 : hp <= 32 ? 32 : 64;
+  // padded rows of up to 256 floats on the 32-row kernel, up to 64 on the 16-row kernel
+  const int pw = hp <= 16 ? 16 : hp <= 32 ? 32 : hp <= 64 ? 64 : hp <= 128 ? 128 : 256;
   if (hp > pw) return false;
   // buffer loads address a tensor through 32-bit byte offsets
   if ((double)batch * kc * groups * hs * hs >= 536870912.0 || (double)batch * ho * ho >= 2147483648.0) return false;
@@ -677,7 +680,7 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   // tuning override "<map blocks><pixel blocks>", e.g. 22; 161 / 162 = the 16-row kernel with 128 / 256 pixels
   const int forced = tuning().direct_tile;
   pl->tm16 = 0;
-  if (const int tm16 = direct_tm16(mtot); tm16 && (forced == 0 || forced == 161 || forced == 162)) {
+  if (const int tm16 = direct_tm16(mtot); tm16 && pw <= 64 && (forced == 0 || forced == 161 || forced == 162)) {
     // 256-pixel tiles (seven LDS reads per twelve MFMAs of a tap instead of five per six) where the launch still
     // has some four of them per compute unit -- measured 1.5-3 % faster on the data gradients of CaffeNet's conv1
     // (sixteen phases) and grouped conv2 -- else 128-pixel tiles
@@ -724,7 +727,7 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
       const long patch = 2L * cp * pr * pw;
       const size_t lds =
           2 * (size_t)((2 * cp * 32 * tmb * ks * ks + 255) / 256 * 256 + (patch + 63) / 64 * 64) * sizeof(float);
-      if (patch > 256L * kDirectPatchLoads || lds > 64 * 1024) continue;
+      if (patch > 256L * direct_patch_loads(pw) || lds > 64 * 1024) continue;
       const long tiles = groups * tiles_m * ((ptot + bn - 1) / bn);
       long slots = (long)(160 * 1024 / lds);
       if (slots > reg_slots[tmb][tnb]) slots = reg_slots[tmb][tnb];
@@ -844,10 +847,16 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
                        : pl.pw == 32 ? direct_launch16<3, 32>(g, pl, st) : direct_launch16<3, 64>(g, pl, st);
   }
   if (ks == 5)
-    return pl.pw == 16 ? direct_launch_ks<5, 1, 16>(g, pl, st)
-                       : pl.pw == 32 ? direct_launch_ks<5, 1, 32>(g, pl, st) : direct_launch_ks<5, 1, 64>(g, pl, st);
-  return pl.pw == 16 ? direct_launch_ks<3, 2, 16>(g, pl, st)
-                     : pl.pw == 32 ? direct_launch_ks<3, 2, 32>(g, pl, st) : direct_launch_ks<3, 2, 64>(g, pl, st);
+    return pl.pw == 16    ? direct_launch_ks<5, 1, 16>(g, pl, st)
+           : pl.pw == 32  ? direct_launch_ks<5, 1, 32>(g, pl, st)
+           : pl.pw == 64  ? direct_launch_ks<5, 1, 64>(g, pl, st)
+           : pl.pw == 128 ? direct_launch_ks<5, 1, 128>(g, pl, st)
+                          : direct_launch_ks<5, 1, 256>(g, pl, st);
+  return pl.pw == 16    ? direct_launch_ks<3, 2, 16>(g, pl, st)
+         : pl.pw == 32  ? direct_launch_ks<3, 2, 32>(g, pl, st)
+         : pl.pw == 64  ? direct_launch_ks<3, 2, 64>(g, pl, st)
+         : pl.pw == 128 ? direct_launch_ks<3, 2, 128>(g, pl, st)
+                        : direct_launch_ks<3, 2, 256>(g, pl, st);
 }
 
 

@@ -649,6 +649,11 @@ static int strided_launch(const StridedArgs &g, const StridedPlan &pl, hipStream
 // Partial sums of the step ranges go to a workspace and are added in a fixed order
 // (run-to-run identical results).  The bias gradient rides along: the dout fragments a wavefront
 // of column group 0 feeds to the matrix cores are also summed per lane.
+// Output rows too long for one step's slab and patch (images wider than some 60 pixels at stride 1) are taken in
+// pieces of cw pixels: a step is then (image, row, piece), the piece's first pixel x0 moves both operands' scalar
+// offsets, and what lies outside the image -- left of it in the first piece, right of it and past the row's end in
+// the last -- is masked per lane by bit sets fixed at the start (the patch descriptor starts `pad` floats ahead
+// of the tensor, so that every lane offset is non-negative).
 //
 // Bound: fp32 MFMA rate.  Algorithmic work 2 * o * batch*ho*ho * d*KS*KS FLOP per call.
 struct StridedWgradArgs {
@@ -664,11 +669,12 @@ struct StridedWgradArgs {
   int a_floats, b_floats;  // slab / patch floats per stage, whole passes of the workgroup
   int nal, nbl;        // loads per lane per step: slab, patch
   int pws, pch;        // floats between patch rows / patch channels
-  int nq2;             // groups of four pixels per output row: ceil(ho / 4)
-  int steps_total, steps_per_split;  // a step = (image, output row)
+  int nq2;             // groups of four pixels per step: ceil(cw / 4)
+  int cw, nchunks;     // a long output row is taken in nchunks pieces of cw pixels (the last may be shorter); ho, 1 otherwise
+  int steps_total, steps_per_split;  // a step = (image, output row, piece of the row)
   uint32_t dout_img_stride, src_img_stride;  // floats between images (channel-slice views of wider tensors)
   uint32_t tiles_m, tiles_n, ntiles, nblocks;
-  FastDiv div_ho, div_ast, div_pch, div_pws, div_wm;
+  FastDiv div_ho, div_ast, div_pch, div_pws, div_wm, div_nchunks;
 };
 
 constexpr int kSWgradSlabLoads = 16;   // per lane per step, at most
@@ -695,16 +701,20 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
   const int stage = g.a_floats + g.b_floats;
 
   // ---- dout slab: pass k of the workgroup covers slab words k*nthreads + tid ----
-  uint32_t aoff[NAL];  // byte offset from (image, map m0, row y); kOutOfRange = a zero word
+  const int x_last = (g.nchunks - 1) * g.cw;  // first pixel of a row's last piece
+  const int tw = S * (g.cw - 1) + KS;         // source columns a piece touches
+  uint32_t aoff[NAL];  // byte offset from (image, map m0, row y, pixel x0); kOutOfRange = a zero word
+  uint32_t a_last = 0u, b_first = 0u, b_last = 0u;  // per load: the word exists in the last / first / last piece
 #pragma unroll
   for (int k = 0; k < NAL; ++k) {
     const uint32_t e = (uint32_t)(k * nthreads + tid);
     const uint32_t m = fdiv(e, g.div_ast), i = e - m * g.ast;
-    const bool ok = k < g.nal && m < (uint32_t)bm && m0 + (int)m < g.o && i < (uint32_t)g.ho;
+    const bool ok = k < g.nal && m < (uint32_t)bm && m0 + (int)m < g.o && i < (uint32_t)g.cw;
     aoff[k] = ok ? (m * ho2 + i) * 4u : kOutOfRange;
+    if (x_last + (int)i < g.ho) a_last |= 1u << k;  // the pixel exists in the last piece of a row
   }
   // ---- source patch: element e = k*nthreads + tid of the [nch][pch] array (rows of pws floats) ----
-  uint32_t boff[NBL];               // byte offset from (image, channel ch0, row S*y - pad); kOutOfRange = never valid
+  uint32_t boff[NBL];               // byte offset from (image, channel ch0, row S*y - pad, column S*x0 - pad); kOutOfRange = never valid
   uint32_t brow[(NBL + 4) / 5];     // tap row of each element, six bits apiece
 #pragma unroll
   for (int k = 0; k < (NBL + 4) / 5; ++k) brow[k] = 0u;
@@ -713,33 +723,40 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
     const uint32_t e = (uint32_t)(k * nthreads + tid);
     const uint32_t ch = fdiv(e, g.div_pch), rem = e - ch * g.pch;
     const uint32_t prow = fdiv(rem, g.div_pws), pcol = rem - prow * g.pws;
-    const int scol = (int)pcol - g.pad;
     const bool ok = k < g.nbl && ch < (uint32_t)g.nch && prow < (uint32_t)KS && ch0 + (int)ch < g.d &&
-                    (unsigned)scol < (unsigned)g.hs;
-    boff[k] = ok ? (ch * hs2 + prow * g.hs + (uint32_t)scol) * 4u : kOutOfRange;
+                    pcol < (uint32_t)tw;
+    boff[k] = ok ? (ch * hs2 + prow * g.hs + pcol) * 4u : kOutOfRange;
     brow[k / 5] |= (ok ? prow : 0u) << (6 * (k % 5));
+    if ((int)pcol >= g.pad) b_first |= 1u << k;                       // not left of the image in the first piece
+    if (S * x_last + (int)pcol - g.pad < g.hs) b_last |= 1u << k;     // not right of it in the last piece
   }
-  const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src);
+  const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src - g.pad);
 
 // global -> LDS stage st for step s
 #define CCT_SWGRAD_ISSUE(s, st)                                                                   \
   do {                                                                                            \
-    const uint32_t img_ = fdiv((uint32_t)(s), g.div_ho);                                          \
-    const int y_ = (s) - (int)img_ * g.ho;                                                        \
+    const uint32_t rowid_ = fdiv((uint32_t)(s), g.div_nchunks);                                   \
+    const int piece_ = (s) - (int)rowid_ * g.nchunks, x0_ = piece_ * g.cw;                        \
+    const uint32_t img_ = fdiv(rowid_, g.div_ho);                                                 \
+    const int y_ = (int)rowid_ - (int)img_ * g.ho;                                                \
+    const uint32_t ma_ = piece_ == g.nchunks - 1 ? a_last : ~0u;                                  \
+    const uint32_t mb_ = (piece_ == 0 ? b_first : ~0u) & (piece_ == g.nchunks - 1 ? b_last : ~0u); \
     float *sa_ = smem + (st) * stage + wave * 64;                                                 \
-    const uint32_t ga_ = (uint32_t)(((size_t)img_ * g.dout_img_stride + (size_t)m0 * ho2 + y_ * g.ho) * 4); \
+    const uint32_t ga_ =                                                                          \
+        (uint32_t)(((size_t)img_ * g.dout_img_stride + (size_t)m0 * ho2 + y_ * g.ho + x0_) * 4);  \
     _Pragma("unroll") for (int k = 0; k < NAL; ++k) {                                             \
-      if (k < g.nal) lds_dma4(a_rsrc, aoff[k], ga_, sa_ + k * nthreads);                          \
+      if (k < g.nal) lds_dma4(a_rsrc, ((ma_ >> k) & 1u) ? aoff[k] : kOutOfRange, ga_, sa_ + k * nthreads); \
     }                                                                                             \
     float *sb_ = sa_ + g.a_floats;                                                                \
-    const uint32_t gb_ = (uint32_t)(((size_t)img_ * g.src_img_stride + (size_t)ch0 * hs2) * 4);   \
+    const uint32_t gb_ =                                                                          \
+        (uint32_t)(((size_t)img_ * g.src_img_stride + (size_t)ch0 * hs2 + (size_t)S * x0_) * 4);  \
     /* the first patch row may lie above the image: that (negative) term goes into the lane     */ \
     /* offset, whose sum is non-negative for every lane that passes the row test                */ \
     const int top_ = S * y_ - g.pad;                                                              \
     const uint32_t row0_ = (uint32_t)(top_ * g.hs * 4);                                           \
     _Pragma("unroll") for (int k = 0; k < NBL; ++k) {                                             \
       const int srow_ = top_ + (int)((brow[k / 5] >> (6 * (k % 5))) & 63u);                       \
-      const bool ok_ = (int)boff[k] >= 0 && (unsigned)srow_ < (unsigned)g.hs;                     \
+      const bool ok_ = (int)boff[k] >= 0 && ((mb_ >> k) & 1u) && (unsigned)srow_ < (unsigned)g.hs; \
       if (k < g.nbl) lds_dma4(b_rsrc, ok_ ? boff[k] + row0_ : kOutOfRange, gb_, sb_ + k * nthreads); \
     }                                                                                             \
   } while (0)
@@ -1000,6 +1017,7 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_spec_kernel(const Stri
 
 struct StridedWgradPlan {
   int tb, wm, wn, nch, ast, a_floats, b_floats, nal, nbl, pws, pch, nq2;
+  int cw, nchunks;  // pieces an output row is taken in: nchunks of cw pixels (ho, 1 where a row fits a step)
   bool spec;  // a compile-time specialised instance exists for this shape
   size_t lds;
 };
@@ -1022,11 +1040,16 @@ static bool strided_wgrad_plan(int batch, int d, int n, int ks, int stride, int 
       (double)o * d * kk >= 536870912.0)
     return false;  // 32-bit byte offsets
   const int ncols = d * kk, cb = (ncols + 31) / 32, mb = (o + 31) / 32;
-  const int nq2 = (ho + 3) / 4, ast = 4 * nq2 + 1;
-  const int tw = stride * (ho - 1) + ks;                      // source columns an output row touches
+  long best_cost = -1;
+  // an output row in as few pieces as the slab and patch loads of a step allow (balanced; the last piece wide enough
+  // that only it can reach past the image's right edge)
+  for (int nchunks = 1; nchunks <= 16 && best_cost < 0; ++nchunks) {
+  const int cw = (ho + nchunks - 1) / nchunks, last_w = ho - (nchunks - 1) * cw;
+  if (nchunks > 1 && (last_w < 1 || last_w * stride < ks || cw < ks)) continue;
+  const int nq2 = (cw + 3) / 4, ast = 4 * nq2 + 1;
+  const int tw = stride * (cw - 1) + ks;                      // source columns a piece of an output row touches
   const int pws = tw + (((ks - tw) % 32) + 32) % 32;          // >= tw, == ks (mod 32)
   const int raw = ks * pws, pch = raw + (((kk - raw) % 32) + 32) % 32;  // >= raw, == ks*ks (mod 32)
-  long best_cost = -1;
   // candidates: column blocks per wavefront x column groups x row blocks; cost = MFMAs issued per step
   for (int tb = 3; tb >= 1; --tb)
     for (int wn = 4; wn >= 1; --wn)
@@ -1053,13 +1076,15 @@ static bool strided_wgrad_plan(int batch, int d, int n, int ks, int stride, int 
           best_cost = cost;
           pl->tb = tb; pl->wm = wm; pl->wn = wn; pl->nch = nch; pl->ast = ast; pl->a_floats = a_floats;
           pl->b_floats = b_floats; pl->nal = nal; pl->nbl = nbl; pl->pws = pws; pl->pch = pch; pl->nq2 = nq2;
+          pl->cw = cw; pl->nchunks = nchunks;
           pl->lds = lds;
         }
       }
+  }
   if (best_cost < 0) return false;
   // conv1 of AlexNet / CaffeNet: 11 x 11, stride 4, no padding, 53..56 pixels per output row, a spare column
   pl->spec = ks == 11 && stride == 4 && pad == 0 && pl->tb == 3 && pl->nq2 == 14 && pl->nal == 8 && pl->nbl == 11 &&
-             ncols % 32 != 0 && !tuning().direct_nospec;
+             pl->nchunks == 1 && ncols % 32 != 0 && !tuning().direct_nospec;
   if (pl->spec) pl->lds += kSWgradOnes * sizeof(float);
   return pl->lds <= 160 * 1024;
 }
@@ -1099,7 +1124,8 @@ int conv_strided_wgrad(float *dw, float *db, const float *dout, const float *src
   g.ncols = d * ks * ks;
   g.wm = pl.wm; g.wn = pl.wn; g.nch = pl.nch; g.ast = pl.ast; g.a_floats = pl.a_floats; g.b_floats = pl.b_floats;
   g.nal = pl.nal; g.nbl = pl.nbl; g.pws = pl.pws; g.pch = pl.pch; g.nq2 = pl.nq2;
-  g.steps_total = batch * g.ho;
+  g.cw = pl.cw; g.nchunks = pl.nchunks;
+  g.steps_total = batch * g.ho * pl.nchunks;
   {
     const size_t dense_src = (size_t)d * n * n, dense_dout = (size_t)o * g.ho * g.ho;
     if (!src_img_stride) src_img_stride = dense_src;
@@ -1130,6 +1156,7 @@ int conv_strided_wgrad(float *dw, float *db, const float *dout, const float *src
   g.div_pch = make_fastdiv((uint32_t)g.pch);
   g.div_pws = make_fastdiv((uint32_t)g.pws);
   g.div_wm = make_fastdiv((uint32_t)g.wm);
+  g.div_nchunks = make_fastdiv((uint32_t)g.nchunks);
   const size_t n_out = (size_t)o * g.ncols;
   if (splits > 1) {
     void *ws = nullptr;

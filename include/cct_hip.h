@@ -252,8 +252,9 @@ int cct_hip_conv_small_backward_weights(float *dw, float *db, const float *dout,
                                         int n, int k, int pad, int o);
 /* ---- stride-1 convolution without the lowered matrix ------------------------------------ */
 /* Fused replacements for chains of ConvolutionBridge's lowering pipeline when stride == 1 and
- * k is 3 or 5 (padded image at most 32 wide).  Results agree with the lowering path to fp32
- * rounding (the sums run in another order), not bit for bit.
+ * k is 3 or 5 and the padded image is at most 256 wide (up to 32: image-pair weight-gradient kernels; wider:
+ * the weight gradient takes one image per step and long output rows in pieces).  Results agree with the
+ * lowering path to fp32 rounding (the sums run in another order), not bit for bit.
  * cct_hip_conv_direct_supported: 1 if both directions cover the geometry, else 0. */
 int cct_hip_conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding,
                                   int num_outputs);

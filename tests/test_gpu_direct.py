@@ -29,8 +29,14 @@ SHAPES = [
     (2, 16, 27, 5, 2, 80),    # five 16-row blocks forward, one in the data gradient
     (2, 8, 56, 3, 1, 16),     # padded rows of 33..64 floats: 64-float patch rows, one image per weight-gradient step
     (2, 6, 40, 5, 2, 40),
-    (3, 20, 62, 3, 1, 33),    # padded width 64: the widest
+    (3, 20, 62, 3, 1, 33),    # padded width 64: the widest the 16-row kernel takes
     (2, 3, 60, 5, 2, 8),
+    (2, 6, 100, 3, 1, 24),    # padded rows of 65..128 floats: 128-float patch rows (32-row kernel only)
+    (1, 4, 126, 3, 1, 33),    # padded width 128
+    (2, 3, 96, 5, 2, 9),
+    (1, 5, 224, 3, 1, 8),     # padded rows of up to 256 floats (VGG-sized planes)
+    (1, 3, 150, 5, 0, 4),
+    (1, 2, 254, 3, 1, 3),     # padded width 256: the widest
 ]
 
 
@@ -368,7 +374,10 @@ def test_direct_support_matrix_and_errors():
     assert not drv.conv_direct_supported(256, 3, 227, 11, 4, 0, 96)   # k = 11, stride 4
     assert not drv.conv_direct_supported(4, 3, 20, 5, 4, 2, 10)       # stride 4
     assert drv.conv_direct_supported(4, 3, 40, 5, 1, 2, 10)           # padded image 44 wide
-    assert not drv.conv_direct_supported(4, 3, 62, 5, 1, 2, 10)       # padded image wider than 64
+    assert drv.conv_direct_supported(4, 3, 62, 5, 1, 2, 10)           # padded image 66 wide: 128-float patch rows
+    assert drv.conv_direct_supported(2, 8, 224, 3, 1, 1, 16)          # VGG-sized planes
+    assert drv.conv_direct_supported(1, 3, 254, 3, 1, 1, 4)           # padded image 256 wide: the widest
+    assert not drv.conv_direct_supported(1, 3, 255, 3, 1, 1, 4)       # wider
     assert not drv.conv_direct_supported(4, 3, 20, 5, 1, 5, 10)       # padding above k-1
     assert not drv.conv_direct_supported(1, 2, 3, 3, 1, 0, 2)         # 1x1 output: a tile would span 128 images
     # tensors read through buffer descriptors (2 GiB of addressable bytes each) must stay below 2^29 floats
@@ -384,7 +393,7 @@ def test_direct_support_matrix_and_errors():
     assert not drv.conv_direct_supported(4, 6, 13, 3, 1, 1, 9, 2)
     assert not drv.conv_direct_supported(4, 7, 13, 3, 1, 1, 8, 2)
     with pytest.raises(CctHipError):
-        drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 62, 5, 2, 10)
+        drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 300, 5, 2, 10)   # padded width above 256
     with pytest.raises(CctHipError):
         drv.conv_direct_backward_weights(empty((1,)), empty((1,)), empty((1,)), 4, 3, 20, 7, 3, 10)
     w = empty((drv.conv_direct_slab_floats(10, 3, 5, 0),), fill=1.0)

@@ -65,6 +65,52 @@ def test_convolution_bridge_random_geometries(oracle, seed):
     assert direct >= 20   # most draws are inside the direct kernels' reach
 
 
+@pytest.mark.parametrize("seed", [31, 32])
+def test_wide_image_convolutions_stay_on_the_direct_kernels(oracle, seed):
+    """Stride-1 layers with k = 3 or 5 on images 65 to 254 pixels wide (padded rows of up to 256 floats): forward
+    and data gradient on 128- and 256-float patch rows, the weight gradient with its output rows taken in pieces;
+    all three against the oracle, and never the lowering path."""
+    from caffecontroll_amd.bridges import ConvolutionLayer
+    drv = driver()
+    rng = np.random.default_rng(seed)
+    done = 0
+    while done < 8:
+        k = int(rng.choice([3, 5]))
+        p = int(rng.integers(0, k))
+        n = int(rng.integers(65, 257 - 2 * p))
+        if n + 2 * p > 256:
+            continue
+        m = n + 2 * p - k + 1
+        b, d, o = int(rng.integers(1, 4)), int(rng.integers(1, 9)), int(rng.integers(1, 40))
+        if 2.0 * b * m * m * k * k * d * o > 8e8:
+            continue
+        x = rng.standard_normal((b, d, n, n)).astype(np.float32)
+        w = (rng.standard_normal((o, d, k, k)) * 0.1).astype(np.float32)
+        bias = rng.standard_normal(o).astype(np.float32)
+        og = rng.standard_normal((b, o, m, m)).astype(np.float32)
+        ref_out, lowered = oracle.conv_forward(x, w, bias, k, 1, p)
+        ref_dx, ref_dw, ref_db = oracle.conv_backward(x.shape, w, og, lowered, k, 1, p)
+        assert drv.conv_direct_supported(b, d, n, k, 1, p, o), (b, d, n, k, p, o)
+        in_grad, out_data = empty((b, d, n, n)), empty((b, o, m, m))
+        layer = ConvolutionLayer(b, d, n, k, 1, p, o, dev(x), in_grad, out_data, dev(og))
+        layer.set_options(fused=3)
+        assert layer.path() == 3
+        drv.memcpy(layer.model_ptr(), w.ctypes.data, w.nbytes, 0)
+        drv.memcpy(layer.bias_ptr(), bias.ctypes.data, bias.nbytes, 0)
+        layer.forward()
+        layer.backward(with_update=False)
+        dw, db = np.empty((o, d, k, k), np.float32), np.empty((o,), np.float32)
+        drv.memcpy(dw.ctypes.data, layer.model_grad_ptr(), dw.nbytes, 1)
+        drv.memcpy(db.ctypes.data, layer.bias_grad_ptr(), db.nbytes, 1)
+        what = (b, d, n, k, p, o)
+        assert rel_err(host(out_data), ref_out) <= TOL, what
+        assert rel_err(host(in_grad), ref_dx) <= TOL, what
+        assert rel_err(dw, np.asarray(ref_dw).reshape(dw.shape)) <= TOL, what
+        assert rel_err(db, ref_db) <= TOL, what
+        layer.close()
+        done += 1
+
+
 @pytest.mark.parametrize("seed", [21, 22])
 def test_pooling_and_lrn_random_geometries(oracle, seed):
     import torch

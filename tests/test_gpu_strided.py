@@ -28,6 +28,15 @@ SHAPES = [
     (4, 6, 13, 3, 2, 0, 70),
     (2, 1, 43, 11, 4, 0, 97),      # one channel, four map blocks
 ]
+# long output rows: the weight gradient takes a row in pieces (the data-gradient kernel does not cover these)
+LONG_ROWS = [
+    (1, 3, 500, 11, 4, 0, 8),
+    (2, 2, 300, 7, 2, 0, 12),
+    (1, 2, 401, 5, 2, 0, 9),
+    (1, 2, 600, 3, 2, 0, 5),
+    (1, 2, 300, 7, 2, 3, 12),      # padded
+    (1, 1, 2000, 11, 4, 0, 4),     # the longest rows the kernels take (498 pixels in 16 pieces)
+]
 _ids = lambda s: "b%d_d%d_n%d_k%d_s%d_p%d_o%d" % s
 
 
@@ -41,7 +50,7 @@ def _forward(drv, x, w, bias, shape, relu=False):
     return host(out)
 
 
-@pytest.mark.parametrize("shape", SHAPES, ids=_ids)
+@pytest.mark.parametrize("shape", SHAPES + LONG_ROWS, ids=_ids)
 def test_strided_forward_vs_oracle(oracle, shape):
     b, d, n, k, s, p, o = shape
     drv = driver()
@@ -93,7 +102,7 @@ def test_strided_forward_full_config3_vs_float64():
     assert rel_err(got, ref) <= TOL
 
 
-@pytest.mark.parametrize("shape", SHAPES, ids=_ids)
+@pytest.mark.parametrize("shape", SHAPES + LONG_ROWS, ids=_ids)
 def test_strided_backward_weights_vs_oracle(oracle, shape):
     """Weight and bias gradient against the oracle's remap + weight-gradient GEMM on the lowered matrix
     (src/bridges/ConvolutionBridge_impl.hxx:575-604, 619-621)."""
@@ -252,6 +261,6 @@ def test_unsupported_geometries_are_refused():
     assert not drv.conv_strided_supported(2, 3, 30, 11, 3, 0, 8)     # stride 3
     assert not drv.conv_strided_supported(2, 3, 30, 9, 4, 0, 8)      # no 9x9 instance
     assert not drv.conv_strided_supported(2, 3, 2000, 11, 4, 2, 8)   # padded rows too long for the LDS patch
-    assert not drv.conv_strided_supported(2, 3, 2000, 11, 4, 0, 8)   # source rows too long for the weight gradient's patch
+    assert not drv.conv_strided_supported(2, 3, 3000, 11, 4, 0, 8)   # output rows longer than the weight gradient's 16 pieces
     with pytest.raises(CctHipError, match="not covered"):
         drv.conv_strided_forward(empty((4,)), empty((4,)), empty((4,)), None, 2, 3, 30, 11, 3, 0, 8)
