@@ -61,14 +61,19 @@ struct DirectArgs {
   // writes maps q*mtot .. of dst with the slab buffer at wt + q*wt_group_floats; tile ids run group by group
   int groups;
   uint32_t tiles_per_group, wt_group_floats;
+  // 32-row kernel, images wider than a patch row: every image is cut into `nbands` column bands of `wv` output
+  // columns (the last one may reach past the right edge), and a band is numbered like an image of its own --
+  // tile pixel p = ((img * nbands + band) * ho + y) * wv + x -- so a tile's patch holds wv + KS - 1 columns of
+  // the source rows it touches instead of whole rows.  One band of wv = ho columns otherwise.
+  int wv, nbands;
+  uint32_t vpix;      // wv * ho: pixels of a band
+  FastDiv div_wv, div_vpix, div_nbands;
 };
 
 constexpr int kDirect16PatchLoads = 11;  // the 16-row kernel stages four channels per step
 
-// source elements per lane per step, at most, by patch row length: eight for rows of up to 64 floats; rows of 128
-// and 256 floats (images wider than 64) hold as many source rows in more loads
+// source elements per lane per step, at most
 constexpr int kDirectPatchLoads = 8;
-constexpr int direct_patch_loads(int pw) { return pw <= 64 ? kDirectPatchLoads : pw == 128 ? 16 : 24; }
 
 // Fragments of contraction index idx = cp*KS*KS + j (idx is a constant after unrolling): weights of
 // tap j of channel pair cp for TMB row blocks, source elements under tap j for TNB pixel blocks.
@@ -99,7 +104,7 @@ __global__ __launch_bounds__(256, direct_waves_per_simd(TMB * TNB)) void conv_di
   constexpr int ASZP = (ASZ + 255) / 256 * 256;  // LDS room for them: whole 64-lane 16-byte loads
   constexpr int SLAB4 = BM * KK / 4;          // 16-byte vectors per slab
   constexpr int NA4 = (ASZP / 4 + 255) / 256;  // 16-byte vectors per lane per stage
-  constexpr int NPL = direct_patch_loads(PW);
+  constexpr int NPL = kDirectPatchLoads;
   extern __shared__ __attribute__((aligned(16))) float smem[];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -116,9 +121,9 @@ __global__ __launch_bounds__(256, direct_waves_per_simd(TMB * TNB)) void conv_di
   const uint32_t p0 = tn * BN;
   const int ho2 = g.ho * g.ho;
 
-  // first patch row: the virtual row of the tile's first pixel
-  const uint32_t img0 = fdiv(p0, g.div_ho2);
-  const uint32_t y0 = fdiv(p0 - img0 * ho2, g.div_ho);
+  // first patch row: the virtual row of the tile's first pixel (bands stacked like images, hp rows each)
+  const uint32_t img0 = fdiv(p0, g.div_vpix);
+  const uint32_t y0 = fdiv(p0 - img0 * g.vpix, g.div_wv);
   const int v_lo = img0 * g.hp + y0;
 
   // ---- per-lane loader state -------------------------------------------------------------
@@ -149,10 +154,10 @@ __global__ __launch_bounds__(256, direct_waves_per_simd(TMB * TNB)) void conv_di
     const uint32_t pc = e % PW, rest = e / PW;
     const uint32_t c = fdiv(rest, g.div_pr), prow = rest - c * g.pr;
     const uint32_t v = v_lo + prow;
-    const uint32_t img = fdiv(v, g.div_hp);
-    const int srow = (int)(v - img * g.hp) - g.pad, scol = (int)pc - g.pad;
-    const bool ok = c < (uint32_t)NC && img < (uint32_t)g.batch && (unsigned)srow < (unsigned)g.hs &&
-                    (unsigned)scol < (unsigned)g.hs;
+    const uint32_t vi = fdiv(v, g.div_hp), img = fdiv(vi, g.div_nbands), band = vi - img * g.nbands;
+    const int srow = (int)(v - vi * g.hp) - g.pad, scol = (int)(band * g.wv + pc) - g.pad;
+    const bool ok = c < (uint32_t)NC && img < (uint32_t)g.batch && pc < (uint32_t)(g.wv + KS - 1) &&
+                    (unsigned)srow < (unsigned)g.hs && (unsigned)scol < (unsigned)g.hs;
     psrc[i] = ok ? (img * g.src_img_stride + (c * g.hs + srow) * g.hs + scol) * 4u : kOutOfRange;
   }
   const uint32_t a_step = (uint32_t)NC * g.slab_stride * 4u, b_step = (uint32_t)NC * g.hs * g.hs * 4u;  // bytes
@@ -186,10 +191,10 @@ __global__ __launch_bounds__(256, direct_waves_per_simd(TMB * TNB)) void conv_di
   for (int b = 0; b < TNB; ++b) {
     uint32_t p = p0 + wave * (32 * TNB) + b * 32 + r;
     p = min(p, g.ptot - 1);
-    const uint32_t img = fdiv(p, g.div_ho2);
-    const uint32_t pix = p - img * ho2;
-    const uint32_t y = fdiv(pix, g.div_ho), x = pix - y * g.ho;
-    bbase[b] = ASZP + h * (g.pr * PW) + (int)(img * g.hp + y - v_lo) * PW + (int)x;
+    const uint32_t vi = fdiv(p, g.div_vpix);
+    const uint32_t pix = p - vi * g.vpix;
+    const uint32_t y = fdiv(pix, g.div_wv), x = pix - y * g.wv;
+    bbase[b] = ASZP + h * (g.pr * PW) + (int)(vi * g.hp + y - v_lo) * PW + (int)x;
   }
   const int pair_stride = 2 * g.pr * PW;  // patch floats per channel pair
 
@@ -316,8 +321,10 @@ __global__ __launch_bounds__(256, direct_waves_per_simd(TMB * TNB)) void conv_di
   for (int b = 0; b < TNB; ++b) {
     const uint32_t p = p0 + wave * (32 * TNB) + b * 32 + r;
     if (p >= g.ptot) continue;
-    const uint32_t img = fdiv(p, g.div_ho2);
-    const size_t pix = (size_t)img * g.dst_img_stride + (size_t)grp * g.mtot * ho2 + (p - img * ho2);
+    const uint32_t vi = fdiv(p, g.div_vpix), img = fdiv(vi, g.div_nbands), band = vi - img * g.nbands;
+    const uint32_t bpix = p - vi * g.vpix, by = fdiv(bpix, g.div_wv), xr = band * g.wv + (bpix - by * g.wv);
+    if (xr >= (uint32_t)g.ho) continue;  // the last band's columns past the right edge
+    const size_t pix = (size_t)img * g.dst_img_stride + (size_t)grp * g.mtot * ho2 + (by * g.ho + xr);
     float *out = g.dst + pix;
     const float *gbias = g.bias ? g.bias + (size_t)grp * g.mtot : nullptr;
 #pragma unroll
@@ -651,6 +658,7 @@ __global__ __launch_bounds__(256) void direct_slab_kernel(float *__restrict__ wt
 
 struct DirectPlan {
   int ks, tmb, tnb, cp, pw, pr;
+  int wv, nbands;  // column bands of a wide image (DirectArgs); wv = output width and one band otherwise
   int tm16;  // > 0: the 16-row kernel with this many row blocks (one map tile); tmb is unused then
   size_t lds;
 };
@@ -668,19 +676,32 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   if (pad < 0 || pad > ks - 1 || batch <= 0 || kc <= 0 || mtot <= 0 || groups <= 0) return false;
   const int ho = hs + 2 * pad - ks + 1, hp = ho + ks - 1;
   if (ho <= 0) return false;
-  // padded rows of up to 256 floats on the 32-row kernel, up to 64 on the 16-row kernel
-  const int pw = hp <= 16 ? 16 : hp <= 32 ? 32 : hp <= 64 ? 64 : hp <= 128 ? 128 : 256;
-  if (hp > pw) return false;
+  // Patch rows hold 16, 32 or 64 floats.  A wider padded image is cut into column bands (32-row kernel only),
+  // each numbered like an image of `wv` columns: the fewest bands that fit 64-float rows, or 32-float rows (more
+  // patch rows per load, which is what lets a tile of narrow bands fit); the tile estimate below chooses.
+  struct Bands { int nbands, wv, pw; } layouts[2];
+  int nlayouts = 0;
+  if (hp <= 64) {
+    layouts[nlayouts++] = {1, ho, hp <= 16 ? 16 : hp <= 32 ? 32 : 64};
+  } else {
+    for (int row = 64; row >= 32; row /= 2) {
+      const int widest = row - (ks - 1), nb = (ho + widest - 1) / widest;
+      layouts[nlayouts++] = {nb, (ho + nb - 1) / nb, row};
+    }
+  }
   // buffer loads address a tensor through 32-bit byte offsets
-  if ((double)batch * kc * groups * hs * hs >= 536870912.0 || (double)batch * ho * ho >= 2147483648.0) return false;
+  if ((double)batch * kc * groups * hs * hs >= 536870912.0) return false;
   const int cp = ks == 3 ? 2 : 1;
-  const long ptot = (long)batch * ho * ho;
+  pl->wv = ho; pl->nbands = 1;
   const int cus = ctx().compute_units > 0 ? ctx().compute_units : 256;
   const int padded = direct_padded_maps(mtot);
   // tuning override "<map blocks><pixel blocks>", e.g. 22; 161 / 162 = the 16-row kernel with 128 / 256 pixels
   const int forced = tuning().direct_tile;
   pl->tm16 = 0;
-  if (const int tm16 = direct_tm16(mtot); tm16 && pw <= 64 && (forced == 0 || forced == 161 || forced == 162)) {
+  if (const int tm16 = direct_tm16(mtot); tm16 && hp <= 64 && (forced == 0 || forced == 161 || forced == 162)) {
+    const int pw = layouts[0].pw;
+    const long ptot = (long)batch * ho * ho;
+    if (ptot >= 2147483648L) return false;
     // 256-pixel tiles (seven LDS reads per twelve MFMAs of a tap instead of five per six) where the launch still
     // has some four of them per compute unit -- measured 1.5-3 % faster on the data gradients of CaffeNet's conv1
     // (sixteen phases) and grouped conv2 -- else 128-pixel tiles
@@ -714,20 +735,24 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   // k = 3 (no vector ALU work is left in its step loop and eight workgroups share a compute unit).
   static const double rate3[5][3] = {{0, 0, 0}, {0, 1.023, 0.983}, {0, 0.985, 0.982}, {0, 0.967, 1.043}, {0, 1.0, 1.042}};
   static const double rate5[5][3] = {{0, 0, 0}, {0, 1.009, 1.017}, {0, 1.008, 0.975}, {0, 0.912, 1.022}, {0, 0.977, 1.03}};
-  struct Candidate { DirectPlan plan; double cost; } cand[8];
+  struct Candidate { DirectPlan plan; double cost; } cand[16];
   int ncand = 0;
+  for (int l = 0; l < nlayouts; ++l) {
+  const int nbands = layouts[l].nbands, wv = layouts[l].wv, pw = layouts[l].pw;
+  const long ptot = (long)batch * nbands * wv * ho;  // the last band's columns past the right edge included
+  if (ptot >= 2147483648L) continue;
   for (int tmb = 4; tmb >= 1; --tmb) {
     if (padded % (32 * tmb)) continue;
     const long tiles_m = padded / (32 * tmb);
     for (int tnb = 2; tnb >= 1; --tnb) {
       if (forced && forced != 10 * tmb + tnb) continue;
       const int bn = 128 * tnb;
-      const int rows = (ho - 1 + bn - 1) / ho + 1, imgs = (ho * ho - 1 + bn - 1) / (ho * ho) + 1;
+      const int rows = (wv - 1 + bn - 1) / wv + 1, imgs = (wv * ho - 1 + bn - 1) / (wv * ho) + 1;
       const int pr = rows - 1 + (imgs - 1) * (ks - 1) + ks;
       const long patch = 2L * cp * pr * pw;
       const size_t lds =
           2 * (size_t)((2 * cp * 32 * tmb * ks * ks + 255) / 256 * 256 + (patch + 63) / 64 * 64) * sizeof(float);
-      if (patch > 256L * direct_patch_loads(pw) || lds > 64 * 1024) continue;
+      if (patch > 256L * kDirectPatchLoads || lds > 64 * 1024) continue;
       const long tiles = groups * tiles_m * ((ptot + bn - 1) / bn);
       long slots = (long)(160 * 1024 / lds);
       if (slots > reg_slots[tmb][tnb]) slots = reg_slots[tmb][tnb];
@@ -739,9 +764,10 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
                           (ks == 3 ? rate3[tmb][tnb] : rate5[tmb][tnb]);
       Candidate &c = cand[ncand++];
       c.plan.ks = ks; c.plan.tmb = tmb; c.plan.tnb = tnb; c.plan.cp = cp; c.plan.pw = pw; c.plan.pr = pr;
-      c.plan.lds = lds;
+      c.plan.lds = lds; c.plan.wv = wv; c.plan.nbands = nbands;
       c.cost = cost;
     }
+  }
   }
   if (ncand == 0) return false;
   const Candidate *pick = nullptr;
@@ -825,7 +851,8 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
   g.nsteps = pl.tm16 ? (kc + 3) / 4 : (kc + 2 * pl.cp - 1) / (2 * pl.cp);
   CCT_REQUIRE((uintptr_t)wt % 16 == 0, "conv_direct: slab buffer must be 16-byte aligned");
   g.slab_stride = direct_padded_maps(mtot) * ks * ks;
-  g.ptot = (uint32_t)((long)batch * g.ho * g.ho);
+  g.wv = pl.wv; g.nbands = pl.nbands; g.vpix = (uint32_t)(pl.wv * g.ho);
+  g.ptot = (uint32_t)((long)batch * pl.nbands * g.vpix);
   g.tiles_m = pl.tm16 ? 1u : (uint32_t)((mtot + 32 * pl.tmb - 1) / (32 * pl.tmb));
   const uint32_t bn = 128 * pl.tnb;
   g.groups = groups;
@@ -836,6 +863,9 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
   g.div_ho2 = make_fastdiv((uint32_t)(g.ho * g.ho));
   g.div_hp = make_fastdiv((uint32_t)g.hp);
   g.div_pr = make_fastdiv((uint32_t)g.pr);
+  g.div_wv = make_fastdiv((uint32_t)g.wv);
+  g.div_vpix = make_fastdiv(g.vpix);
+  g.div_nbands = make_fastdiv((uint32_t)g.nbands);
   g.cs = g.pr * pl.pw + 16;
   g.div_cs = make_fastdiv((uint32_t)g.cs);
   hipStream_t st = ctx().stream;
@@ -847,16 +877,12 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
                        : pl.pw == 32 ? direct_launch16<3, 32>(g, pl, st) : direct_launch16<3, 64>(g, pl, st);
   }
   if (ks == 5)
-    return pl.pw == 16    ? direct_launch_ks<5, 1, 16>(g, pl, st)
-           : pl.pw == 32  ? direct_launch_ks<5, 1, 32>(g, pl, st)
-           : pl.pw == 64  ? direct_launch_ks<5, 1, 64>(g, pl, st)
-           : pl.pw == 128 ? direct_launch_ks<5, 1, 128>(g, pl, st)
-                          : direct_launch_ks<5, 1, 256>(g, pl, st);
-  return pl.pw == 16    ? direct_launch_ks<3, 2, 16>(g, pl, st)
-         : pl.pw == 32  ? direct_launch_ks<3, 2, 32>(g, pl, st)
-         : pl.pw == 64  ? direct_launch_ks<3, 2, 64>(g, pl, st)
-         : pl.pw == 128 ? direct_launch_ks<3, 2, 128>(g, pl, st)
-                        : direct_launch_ks<3, 2, 256>(g, pl, st);
+    return pl.pw == 16   ? direct_launch_ks<5, 1, 16>(g, pl, st)
+           : pl.pw == 32 ? direct_launch_ks<5, 1, 32>(g, pl, st)
+                         : direct_launch_ks<5, 1, 64>(g, pl, st);
+  return pl.pw == 16   ? direct_launch_ks<3, 2, 16>(g, pl, st)
+         : pl.pw == 32 ? direct_launch_ks<3, 2, 32>(g, pl, st)
+                       : direct_launch_ks<3, 2, 64>(g, pl, st);
 }
 
 

@@ -1040,10 +1040,13 @@ static bool strided_wgrad_plan(int batch, int d, int n, int ks, int stride, int 
       (double)o * d * kk >= 536870912.0)
     return false;  // 32-bit byte offsets
   const int ncols = d * kk, cb = (ncols + 31) / 32, mb = (o + 31) / 32;
-  long best_cost = -1;
-  // an output row in as few pieces as the slab and patch loads of a step allow (balanced; the last piece wide enough
-  // that only it can reach past the image's right edge)
-  for (int nchunks = 1; nchunks <= 16 && best_cost < 0; ++nchunks) {
+  double best_cost = -1;
+  // An output row is taken whole or in up to 64 balanced pieces (the last piece wide enough that only it can reach
+  // past the image's right edge): as few as the slab and patch loads of a step allow for the tile, since every step
+  // costs a barrier and a pipeline refill -- about what 13 more pixels would.
+  const int forced = tuning().strided_wgrad;
+  for (int nchunks = 1; nchunks <= 64; ++nchunks) {
+  if (forced && nchunks != forced / 1000) continue;
   const int cw = (ho + nchunks - 1) / nchunks, last_w = ho - (nchunks - 1) * cw;
   if (nchunks > 1 && (last_w < 1 || last_w * stride < ks || cw < ks)) continue;
   const int nq2 = (cw + 3) / 4, ast = 4 * nq2 + 1;
@@ -1056,6 +1059,7 @@ static bool strided_wgrad_plan(int batch, int d, int n, int ks, int stride, int 
       for (int wm = 4; wm >= 1; --wm) {
         const int w = wm * wn;
         if (w > 12) continue;
+        if (forced && forced % 1000 != tb * 100 + wn * 10 + wm) continue;
         if (wm > mb || (wn - 1) * tb >= cb) continue;  // wavefronts with nothing to do
         const int nth = 64 * w;
         const int tiles_n = (cb + tb * wn - 1) / (tb * wn), tiles_m = (mb + wm - 1) / wm;
@@ -1069,9 +1073,16 @@ static bool strided_wgrad_plan(int batch, int d, int n, int ks, int stride, int 
         if (nal > kSWgradSlabLoads || nbl > kSWgradPatchLoads) continue;
         const size_t lds = (size_t)2 * (a_floats + b_floats) * sizeof(float);
         if (lds > 160 * 1024) continue;
-        // padded work; on ties: wider per-wavefront tiles, then a wavefront count that loads the four SIMDs evenly
-        long cost = (long)tiles_n * tb * wn * tiles_m * wm * 1000;
-        cost += (3 - tb) * 40 + (w % 4 ? 20 : 0) + (12 - w);
+        // Padded MFMA work, step overhead included, over the rate of the tile relative to one column block per
+        // wavefront: with three blocks a wavefront reads four LDS fragments per three MFMAs instead of two per
+        // one (measured 1.26 and 1.33 for two and three blocks on 96 -> 96 maps of 5 x 5 at 96 x 96 and on
+        // 128 -> 128 maps of 3 x 3 at 112 x 112); twelve wavefronts hide a step's barrier better than eight or four
+        // (1.0 : 0.92 : 0.9 there); a wavefront count that loads the four SIMDs unevenly loses more than its padding
+        // saves (six wavefronts against four on 64 -> 64 maps of 7 x 7, stride 2: 0.24 against 0.17 ms).
+        static const double tb_rate[4] = {0, 1.0, 1.26, 1.33};
+        double cost = (double)tiles_n * tb * wn * tiles_m * wm * nchunks * (4 * nq2 + 13) / tb_rate[tb];
+        cost /= w >= 12 ? 1.0 : w >= 8 ? 0.92 : w >= 4 ? 0.9 : 0.85;
+        if (w % 4) cost *= 1.15;
         if (best_cost < 0 || cost < best_cost) {
           best_cost = cost;
           pl->tb = tb; pl->wm = wm; pl->wn = wn; pl->nch = nch; pl->ast = ast; pl->a_floats = a_floats;
@@ -1099,7 +1110,7 @@ static int strided_wgrad_launch(const StridedWgradArgs &g, const StridedWgradPla
     if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;                 \
     hipLaunchKernelGGL(kern, grid, block, pl.lds, st, g);                                         \
     CCT_LAUNCH_CHECK();                                                                           \
-    note_kernel("conv_strided_wgrad_kernel<%d,%d,%d> waves=%dx%d", KS, S, TB, pl.wm, pl.wn);      \
+    note_kernel("conv_strided_wgrad_kernel<%d,%d,%d> waves=%dx%d pieces=%d", KS, S, TB, pl.wm, pl.wn, pl.nchunks); \
     return 0;                                                                                     \
   }
   CCT_SWGRAD_CASE(1) CCT_SWGRAD_CASE(2) CCT_SWGRAD_CASE(3)

@@ -105,7 +105,8 @@ int cct_hip_set_stream(void *hip_stream);
  * pixels, 0 = automatic), "direct_waves",
  * "direct_tb", "direct_nospec", "direct_splits" (step ranges of the direct weight-gradient launch, 0 = automatic),
  * "direct_alds" (shape-specialised weight-gradient kernels: 1 = output-gradient rows staged in LDS, 2 = fetched by
- * their lanes, 0 = automatic), "pool_plane", "gemm_nt", "gemm_tile" (-1 = automatic), "gemm_nodma" (1 = GEMM
+ * their lanes, 0 = automatic), "strided_wgrad" (tile of the strided weight-gradient kernel: pieces of an output row
+ * x 1000 + column blocks x 100 + column groups x 10 + row blocks, 0 = automatic), "pool_plane", "gemm_nt", "gemm_tile" (-1 = automatic), "gemm_nodma" (1 = GEMM
  * operand tiles always staged through registers).  The
  * environment variables CCT_HIP_<NAME IN CAPITALS> give the initial values; they are read once,
  * when the library initialises, never on a launch path.  No counterpart in the reference. */
@@ -252,8 +253,10 @@ int cct_hip_conv_small_backward_weights(float *dw, float *db, const float *dout,
                                         int n, int k, int pad, int o);
 /* ---- stride-1 convolution without the lowered matrix ------------------------------------ */
 /* Fused replacements for chains of ConvolutionBridge's lowering pipeline when stride == 1 and
- * k is 3 or 5 and the padded image is at most 256 wide (up to 32: image-pair weight-gradient kernels; wider:
- * the weight gradient takes one image per step and long output rows in pieces).  Results agree with the
+ * k is 3 or 5.  Forward and data gradient take an image whose padded rows exceed 64 floats in column bands;
+ * the weight gradient has image-pair kernels for padded rows of up to 32 floats and otherwise takes one image
+ * per step and long output rows in up to 64 pieces (what bounds the width: a few thousand columns, fewer for a
+ * layer with under 32 maps).  Results agree with the
  * lowering path to fp32 rounding (the sums run in another order), not bit for bit.
  * cct_hip_conv_direct_supported: 1 if both directions cover the geometry, else 0. */
 int cct_hip_conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding,

@@ -374,10 +374,11 @@ def test_direct_support_matrix_and_errors():
     assert not drv.conv_direct_supported(256, 3, 227, 11, 4, 0, 96)   # k = 11, stride 4
     assert not drv.conv_direct_supported(4, 3, 20, 5, 4, 2, 10)       # stride 4
     assert drv.conv_direct_supported(4, 3, 40, 5, 1, 2, 10)           # padded image 44 wide
-    assert drv.conv_direct_supported(4, 3, 62, 5, 1, 2, 10)           # padded image 66 wide: 128-float patch rows
+    assert drv.conv_direct_supported(4, 3, 62, 5, 1, 2, 10)           # padded image 66 wide: two column bands
     assert drv.conv_direct_supported(2, 8, 224, 3, 1, 1, 16)          # VGG-sized planes
-    assert drv.conv_direct_supported(1, 3, 254, 3, 1, 1, 4)           # padded image 256 wide: the widest
-    assert not drv.conv_direct_supported(1, 3, 255, 3, 1, 1, 4)       # wider
+    assert all(drv.conv_direct_supported(1, 3, n, 3, 1, 1, 4) for n in range(8, 1700))   # every width in between
+    assert drv.conv_direct_supported(1, 8, 4000, 5, 1, 2, 8)
+    assert not drv.conv_direct_supported(1, 3, 9000, 3, 1, 1, 4)      # output rows beyond the weight gradient's 64 pieces
     assert not drv.conv_direct_supported(4, 3, 20, 5, 1, 5, 10)       # padding above k-1
     assert not drv.conv_direct_supported(1, 2, 3, 3, 1, 0, 2)         # 1x1 output: a tile would span 128 images
     # tensors read through buffer descriptors (2 GiB of addressable bytes each) must stay below 2^29 floats
@@ -393,7 +394,7 @@ def test_direct_support_matrix_and_errors():
     assert not drv.conv_direct_supported(4, 6, 13, 3, 1, 1, 9, 2)
     assert not drv.conv_direct_supported(4, 7, 13, 3, 1, 1, 8, 2)
     with pytest.raises(CctHipError):
-        drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 300, 5, 2, 10)   # padded width above 256
+        drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 30, 7, 3, 10)   # no 7 x 7 instance
     with pytest.raises(CctHipError):
         drv.conv_direct_backward_weights(empty((1,)), empty((1,)), empty((1,)), 4, 3, 20, 7, 3, 10)
     w = empty((drv.conv_direct_slab_floats(10, 3, 5, 0),), fill=1.0)

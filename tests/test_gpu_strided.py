@@ -35,7 +35,7 @@ LONG_ROWS = [
     (1, 2, 401, 5, 2, 0, 9),
     (1, 2, 600, 3, 2, 0, 5),
     (1, 2, 300, 7, 2, 3, 12),      # padded
-    (1, 1, 2000, 11, 4, 0, 4),     # the longest rows the kernels take (498 pixels in 16 pieces)
+    (1, 1, 2000, 11, 4, 0, 4),     # 498-pixel output rows
 ]
 _ids = lambda s: "b%d_d%d_n%d_k%d_s%d_p%d_o%d" % s
 
@@ -261,6 +261,7 @@ def test_unsupported_geometries_are_refused():
     assert not drv.conv_strided_supported(2, 3, 30, 11, 3, 0, 8)     # stride 3
     assert not drv.conv_strided_supported(2, 3, 30, 9, 4, 0, 8)      # no 9x9 instance
     assert not drv.conv_strided_supported(2, 3, 2000, 11, 4, 2, 8)   # padded rows too long for the LDS patch
-    assert not drv.conv_strided_supported(2, 3, 3000, 11, 4, 0, 8)   # output rows longer than the weight gradient's 16 pieces
+    assert drv.conv_strided_supported(2, 3, 9000, 11, 4, 0, 8)       # long rows: the weight gradient takes them in pieces
+    assert not drv.conv_strided_supported(2, 3, 12000, 11, 4, 0, 8)  # more than its 64 pieces
     with pytest.raises(CctHipError, match="not covered"):
         drv.conv_strided_forward(empty((4,)), empty((4,)), empty((4,)), None, 2, 3, 30, 11, 3, 0, 8)
