@@ -672,17 +672,23 @@ static int direct_tm16(int mtot) {
 
 // Chooses the kernel instance for a geometry; returns false when the direct path does not cover it.
 static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, DirectPlan *pl, int groups = 1) {
-  if (ks != 3 && ks != 5) return false;
+  if (ks != 3 && ks != 5 && ks != 7) return false;
   if (pad < 0 || pad > ks - 1 || batch <= 0 || kc <= 0 || mtot <= 0 || groups <= 0) return false;
   const int ho = hs + 2 * pad - ks + 1, hp = ho + ks - 1;
   if (ho <= 0) return false;
   // Patch rows hold 16, 32 or 64 floats.  A wider padded image is cut into column bands (32-row kernel only),
   // each numbered like an image of `wv` columns: the fewest bands that fit 64-float rows, or 32-float rows (more
-  // patch rows per load, which is what lets a tile of narrow bands fit); the tile estimate below chooses.
+  // patch rows per load, which is what lets a tile of narrow bands fit); the tile estimate below chooses.  An
+  // image of 33..64 padded columns whose rows are too many for one patch (7 x 7 filters) falls back to bands of
+  // 32-float rows as well.
   struct Bands { int nbands, wv, pw; } layouts[2];
   int nlayouts = 0;
   if (hp <= 64) {
     layouts[nlayouts++] = {1, ho, hp <= 16 ? 16 : hp <= 32 ? 32 : 64};
+    if (hp > 32) {
+      const int widest = 32 - (ks - 1), nb = (ho + widest - 1) / widest;
+      layouts[nlayouts++] = {nb, (ho + nb - 1) / nb, 32};
+    }
   } else {
     for (int row = 64; row >= 32; row /= 2) {
       const int widest = row - (ks - 1), nb = (ho + widest - 1) / widest;
@@ -698,7 +704,7 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
   // tuning override "<map blocks><pixel blocks>", e.g. 22; 161 / 162 = the 16-row kernel with 128 / 256 pixels
   const int forced = tuning().direct_tile;
   pl->tm16 = 0;
-  if (const int tm16 = direct_tm16(mtot); tm16 && hp <= 64 && (forced == 0 || forced == 161 || forced == 162)) {
+  if (const int tm16 = direct_tm16(mtot); tm16 && ks <= 5 && hp <= 64 && (forced == 0 || forced == 161 || forced == 162)) {
     const int pw = layouts[0].pw;
     const long ptot = (long)batch * ho * ho;
     if (ptot >= 2147483648L) return false;
@@ -752,7 +758,8 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
       const long patch = 2L * cp * pr * pw;
       const size_t lds =
           2 * (size_t)((2 * cp * 32 * tmb * ks * ks + 255) / 256 * 256 + (patch + 63) / 64 * 64) * sizeof(float);
-      if (patch > 256L * kDirectPatchLoads || lds > 64 * 1024) continue;
+      // the 7 x 7 instances ask for their LDS size (two map blocks of 49-tap slabs pass the default 64 KB)
+      if (patch > 256L * kDirectPatchLoads || lds > (ks == 7 ? 80 : 64) * 1024 || (ks == 7 && tmb > 2)) continue;
       const long tiles = groups * tiles_m * ((ptot + bn - 1) / bn);
       long slots = (long)(160 * 1024 / lds);
       if (slots > reg_slots[tmb][tnb]) slots = reg_slots[tmb][tnb];
@@ -768,6 +775,7 @@ static bool direct_plan(int batch, int kc, int mtot, int hs, int ks, int pad, Di
       c.cost = cost;
     }
   }
+  if (hp <= 64 && ncand) break;  // whole rows fit: no bands
   }
   if (ncand == 0) return false;
   const Candidate *pick = nullptr;
@@ -783,13 +791,20 @@ static int direct_launch_ks(const DirectArgs &g, const DirectPlan &pl, hipStream
   dim3 grid(g.ntiles), block(256);
 #define CCT_DIRECT_CASE(TMB, TNB)                                                                      \
   if (pl.tmb == TMB && pl.tnb == TNB) {                                                                \
-    hipLaunchKernelGGL((conv_direct_kernel<KS, TMB, TNB, CP, PW>), grid, block, pl.lds, st, g);        \
+    auto kern = conv_direct_kernel<KS, TMB, TNB, CP, PW>;                                              \
+    if (pl.lds > 64 * 1024) {                                                                          \
+      static LdsGrant grant;                                                                           \
+      if (int rc = grant_dynamic_lds((const void *)kern, pl.lds, grant)) return rc;                    \
+    }                                                                                                  \
+    hipLaunchKernelGGL(kern, grid, block, pl.lds, st, g);                                              \
     CCT_LAUNCH_CHECK();                                                                                \
     note_kernel("conv_direct_kernel<%d,%d,%d,%d,%d>", KS, TMB, TNB, CP, PW);                           \
     return 0;                                                                                          \
   }
-  CCT_DIRECT_CASE(1, 1) CCT_DIRECT_CASE(2, 1) CCT_DIRECT_CASE(3, 1) CCT_DIRECT_CASE(4, 1)
-  CCT_DIRECT_CASE(1, 2) CCT_DIRECT_CASE(2, 2) CCT_DIRECT_CASE(3, 2) CCT_DIRECT_CASE(4, 2)
+  CCT_DIRECT_CASE(1, 1) CCT_DIRECT_CASE(2, 1) CCT_DIRECT_CASE(1, 2) CCT_DIRECT_CASE(2, 2)
+  if constexpr (KS < 7) {  // 7 x 7: at most two map blocks (the slabs of more do not fit beside the patch)
+    CCT_DIRECT_CASE(3, 1) CCT_DIRECT_CASE(4, 1) CCT_DIRECT_CASE(3, 2) CCT_DIRECT_CASE(4, 2)
+  }
 #undef CCT_DIRECT_CASE
   return set_error(CCT_HIP_EINVAL, "conv_direct: no kernel instance for tile %dx%d", pl.tmb, pl.tnb);
 }
@@ -876,6 +891,10 @@ static int conv_direct(const float *wt, const float *src, float *dst, const floa
     return pl.pw == 16 ? direct_launch16<3, 16>(g, pl, st)
                        : pl.pw == 32 ? direct_launch16<3, 32>(g, pl, st) : direct_launch16<3, 64>(g, pl, st);
   }
+  if (ks == 7)
+    return pl.pw == 16   ? direct_launch_ks<7, 1, 16>(g, pl, st)
+           : pl.pw == 32 ? direct_launch_ks<7, 1, 32>(g, pl, st)
+                         : direct_launch_ks<7, 1, 64>(g, pl, st);
   if (ks == 5)
     return pl.pw == 16   ? direct_launch_ks<5, 1, 16>(g, pl, st)
            : pl.pw == 32 ? direct_launch_ks<5, 1, 32>(g, pl, st)

@@ -1028,7 +1028,7 @@ static bool strided_kernel_size(int ks, int stride) {
 // the weight-gradient kernel also has stride-1 instances (3 x 3 and 5 x 5): the stride-1 kernels of their own
 // file stage image PAIRS and stop at padded rows of 32 floats, this one takes rows as long as its patch holds
 static bool strided_wgrad_kernel_size(int ks, int stride) {
-  return strided_kernel_size(ks, stride) || (stride == 1 && (ks == 3 || ks == 5));
+  return strided_kernel_size(ks, stride) || (stride == 1 && (ks == 3 || ks == 5 || ks == 7));
 }
 
 // Chooses the workgroup shape for a geometry; false when the strided weight-gradient kernel does not cover it.
@@ -1190,7 +1190,7 @@ int conv_strided_wgrad(float *dw, float *db, const float *dout, const float *src
     note_kernel("conv_strided_wgrad_spec_kernel<11,4,3,14,8,11> waves=%dx%d", pl.wm, pl.wn);
     rc = 0;
   } else if (ks == 11) rc = strided_wgrad_launch<11, 4>(g, pl, st);
-  else if (ks == 7) rc = strided_wgrad_launch<7, 2>(g, pl, st);
+  else if (ks == 7) rc = stride == 2 ? strided_wgrad_launch<7, 2>(g, pl, st) : strided_wgrad_launch<7, 1>(g, pl, st);
   else if (ks == 5) rc = stride == 2 ? strided_wgrad_launch<5, 2>(g, pl, st) : strided_wgrad_launch<5, 1>(g, pl, st);
   else rc = stride == 2 ? strided_wgrad_launch<3, 2>(g, pl, st) : strided_wgrad_launch<3, 1>(g, pl, st);
   if (rc) return rc;

@@ -31,12 +31,18 @@ SHAPES = [
     (2, 6, 40, 5, 2, 40),
     (3, 20, 62, 3, 1, 33),    # padded width 64: the widest the 16-row kernel takes
     (2, 3, 60, 5, 2, 8),
-    (2, 6, 100, 3, 1, 24),    # padded rows of 65..128 floats: 128-float patch rows (32-row kernel only)
-    (1, 4, 126, 3, 1, 33),    # padded width 128
+    (2, 6, 100, 3, 1, 24),    # padded rows above 64 floats: column bands (32-row kernel only); two bands of 50
+    (1, 4, 126, 3, 1, 33),    # three bands
     (2, 3, 96, 5, 2, 9),
-    (1, 5, 224, 3, 1, 8),     # padded rows of up to 256 floats (VGG-sized planes)
+    (1, 5, 224, 3, 1, 8),     # VGG-sized planes: four bands of 56
     (1, 3, 150, 5, 0, 4),
-    (1, 2, 254, 3, 1, 3),     # padded width 256: the widest
+    (1, 2, 254, 3, 1, 3),     # five bands of 51, the last one a column short
+    (1, 40, 63, 3, 1, 2),     # 63 = 2 x 32: bands of 32-float patch rows (64-float rows would not fit a tile's patch)
+    (1, 2, 330, 5, 3, 5),
+    (3, 5, 20, 7, 3, 12),     # 7 x 7
+    (2, 3, 33, 7, 0, 40),
+    (2, 4, 9, 7, 6, 33),      # full padding
+    (1, 3, 80, 7, 3, 70),     # 7 x 7 in column bands, two map blocks
 ]
 
 
@@ -394,9 +400,9 @@ def test_direct_support_matrix_and_errors():
     assert not drv.conv_direct_supported(4, 6, 13, 3, 1, 1, 9, 2)
     assert not drv.conv_direct_supported(4, 7, 13, 3, 1, 1, 8, 2)
     with pytest.raises(CctHipError):
-        drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 30, 7, 3, 10)   # no 7 x 7 instance
+        drv.conv_direct_forward(empty((4,)), empty((4,)), empty((4,)), None, 4, 3, 30, 9, 4, 10)   # no 9 x 9 instance
     with pytest.raises(CctHipError):
-        drv.conv_direct_backward_weights(empty((1,)), empty((1,)), empty((1,)), 4, 3, 20, 7, 3, 10)
+        drv.conv_direct_backward_weights(empty((1,)), empty((1,)), empty((1,)), 4, 3, 20, 9, 4, 10)
     w = empty((drv.conv_direct_slab_floats(10, 3, 5, 0),), fill=1.0)
     with pytest.raises(CctHipError):
         drv.conv_direct_slabs(w, w, 10, 3, 5, 0)
