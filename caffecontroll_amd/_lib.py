@@ -90,6 +90,10 @@ PROTOTYPES = {
     "cct_hip_sgemm_new_colsum": [_I, _I, _I, _I, _I, _F, _P, _P, _F, _P, _P, _P, _I, _I],
     "cct_hip_sgemm_new_bias": [_I, _I, _I, _I, _I, _F, _P, _P, _F, _P, _P, _I],
     "cct_hip_sgemm_conv_forward": [_I, _I, _I, _I, _P, _P, _P, _P, _I],
+    "cct_hip_conv1x1_supported": [_I, _I, _I, _I, _I, _I, _I],
+    "cct_hip_conv1x1_forward": [_P, _P, _P, _P, _I, _I, _I, _I, _I],
+    "cct_hip_conv1x1_backward_data": [_P, _P, _P, _I, _I, _I, _I],
+    "cct_hip_conv1x1_backward_weights": [_P, _P, _P, _P, _I, _I, _I, _I],
     "cct_hip_conv_small_supported": [_I, _I, _I, _I, _I, _I, _I],
     "cct_hip_conv_small_forward": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I],
     "cct_hip_conv_small_backward_weights": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I],

@@ -55,6 +55,14 @@ struct GemmArgs {
   uint32_t nblocks;
   int nt_store;      // stream the output with non-temporal stores (large outputs that are not re-read)
   int dma;           // operands go global -> LDS without passing through registers (gemm_mainloop_dma)
+  // A batch of products in one launch (1 x 1 convolution on [image][channel][pixel] tensors).  The grid's slice
+  // index (what selects a K range otherwise) selects images; a slice covers the whole K.
+  //   bmode 1: one product per image, image i with A + i*a_bstride, B + i*b_bstride, C + i*c_bstride;
+  //   bmode 2: ONE product summed over the images, slice z = (image group, K range): it adds K range
+  //            z % bksplit (kchunk wide) of images (z / bksplit)*bgroup .. +bgroup-1 (of nbatch) and stores like
+  //            a K slice does (partial sums for the reduction when there are several slices).
+  int bmode, nbatch, bgroup, bksplit;
+  size_t a_bstride, b_bstride, c_bstride;  // floats
 };
 
 __device__ __forceinline__ f4 ldg4(const float *__restrict__ base, int major, int minor,
@@ -520,7 +528,8 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
 }
 
 template <class T, bool A_KC, bool B_KC, bool DMA = false>
-__global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
+__global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g_in) {
+  GemmArgs g = g_in;  // the batched modes move the matrix pointers (workgroup-uniform)
   using LA = OperandLayout<T, A_KC, T::BM>;
   using LB = OperandLayout<T, B_KC, T::BN>;
   __shared__ __attribute__((aligned(16))) float smem[2 * (LA::SIZE + LB::SIZE)];
@@ -542,7 +551,17 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
     tn = id % g.tiles_n; tm = id / g.tiles_n;
   }
   const int m0 = tm * T::BM, n0 = tn * T::BN;
-  const int kbeg = kslice * g.kchunk;
+  int kbeg = kslice * g.kchunk;
+  int more_images = 0;  // bmode 2: images of this slice after the first
+  if (g.bmode) {
+    const uint32_t igroup = g.bmode == 1 ? kslice : kslice / (uint32_t)g.bksplit;
+    kbeg = g.bmode == 1 ? 0 : (int)(kslice - igroup * g.bksplit) * g.kchunk;
+    const uint32_t img = g.bmode == 1 ? igroup : igroup * (uint32_t)g.bgroup;
+    g.A += (size_t)img * g.a_bstride;
+    g.B += (size_t)img * g.b_bstride;
+    if (g.bmode == 1) g.C += (size_t)img * g.c_bstride;
+    else more_images = min(g.bgroup, g.nbatch - (int)img) - 1;
+  }
   const int kend = min(g.K, kbeg + g.kchunk);
   const int nk = (kend - kbeg + T::BK - 1) / T::BK;
 
@@ -554,8 +573,15 @@ __global__ __launch_bounds__(T::THREADS, 2) void gemm_kernel(const GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-  if (DMA) gemm_mainloop_dma<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, nk, lane, __builtin_amdgcn_readfirstlane(wave), wm0, wn0);
-  else gemm_mainloop<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
+  for (;;) {
+    if (DMA) gemm_mainloop_dma<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, nk, lane, __builtin_amdgcn_readfirstlane(wave), wm0, wn0);
+    else gemm_mainloop<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
+    if (--more_images < 0) break;
+    // the next image of the sum: same tile, same accumulators; the LDS stages are refilled from scratch
+    g.A += g.a_bstride;
+    g.B += g.b_bstride;
+    __syncthreads();
+  }
   const bool rows_inside = m0 + T::BM <= g.M, cols_inside = n0 + T::BN <= g.N;
 
   // epilogue: accumulator register v of lane (r,h) is C[8*(v/4) + 4*h + v%4][r] of its 32x32 tile
@@ -706,12 +732,18 @@ __global__ __launch_bounds__(256) void colsum_kernel(ColSumJob cs) {
   colsum_block(cs.dst, cs.src, cs.cols, cs.rows, blockIdx.x, part);
 }
 
+// A batch of products in one launch (GemmArgs::bmode): `count` images, strides in floats between them.
+struct GemmBatch {
+  int mode, count;
+  size_t a_stride, b_stride, c_stride;
+};
+
 // `colsum`: column sums to compute beside the product, in the spare workgroups of the split-K reduction when
-// there is one, else in a launch of their own.
+// there is one, else in a launch of their own.  `batch`: M, N, K and the matrices describe one image.
 static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha, const float *A, int lda,
                          const float *B, int ldb, float beta, float *C, int ldc, int epi, int fmap,
                          const float *bias, int relu = 0, const float *col_bias = nullptr,
-                         const ColSumJob *colsum = nullptr) {
+                         const ColSumJob *colsum = nullptr, const GemmBatch *batch = nullptr) {
   if (M <= 0 || N <= 0) {
     if (colsum && colsum->cols > 0) {
       hipLaunchKernelGGL(colsum_kernel, dim3((uint32_t)((colsum->cols + 63) / 64)), dim3(256), 0, ctx().stream, *colsum);
@@ -729,6 +761,10 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   g.b_vec = ((uintptr_t)B % 4 == 0);
   g.nt_store = tuning().gemm_nt;
   if (K <= 0) g.K = 0;  // degenerate: C = beta*C through the normal epilogue with zero accumulators
+  const int bmode = batch ? batch->mode : 0, nbatch = batch ? batch->count : 1;
+  g.bmode = bmode; g.nbatch = nbatch; g.bgroup = 1; g.bksplit = 1;
+  g.a_bstride = batch ? batch->a_stride : 0; g.b_bstride = batch ? batch->b_stride : 0;
+  g.c_bstride = batch ? batch->c_stride : 0;
 
   // Tile shape and split-K factor come from a small occupancy model.  A compute unit holds `occ`
   // workgroups of a shape; the busiest unit gets n = ceil(blocks / units) of them and works them off
@@ -749,11 +785,37 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
   for (int c = 0; c < 5; ++c) {
     if (forced >= 0 && forced <= 4 && c != forced) continue;  // tuning override
     const Shape &sh = shapes[c];
-    const long tiles = (long)((M + sh.bm - 1) / sh.bm) * ((N + sh.bn - 1) / sh.bn);
+    const long tiles = (long)((M + sh.bm - 1) / sh.bm) * ((N + sh.bn - 1) / sh.bn) * (bmode == 1 ? nbatch : 1);
     const long slots = (long)sh.occ * cus;
+    if (bmode == 2) {
+      // one product summed over the images: the slices are groups of images or, when there are fewer images than
+      // slices wanted, K ranges of single images -- as many as fill the device while a slice keeps some 256 of
+      // K; every image refills the pipeline (about four K steps' worth)
+      long sp = tiles >= slots ? 1 : slots / tiles;
+      const long most = ((long)nbatch * K + 255) / 256;
+      if (sp > most) sp = most;
+      if (sp < 1) sp = 1;
+      int group = 1, ksplit = 1, kc = K > 0 ? K : bk;
+      if (sp <= nbatch) {
+        group = (int)((nbatch + sp - 1) / sp);
+      } else {
+        ksplit = (int)(sp / nbatch);
+        kc = (((K + ksplit - 1) / ksplit) + bk - 1) / bk * bk;
+        ksplit = (K + kc - 1) / kc;
+      }
+      sp = (long)((nbatch + group - 1) / group) * ksplit;
+      const long blocks = tiles * sp, n = (blocks + cus - 1) / cus, rem = n % sh.occ;
+      const double w = 2.0 * sh.bm * sh.bn * ((double)group * (kc + 4 * bk) + sh.k0) / (cu_rate * sh.eff);
+      double t = (double)(n / sh.occ) * sh.occ * w;
+      if (rem) t += rem * w / (rem * 0.55 < 1.0 ? rem * 0.55 : 1.0);
+      if (sp > 1) t += 5e-6 + 8.0 * sp * (double)M * N / hbm_rate;
+      if (t < best) { best = t; cfg = c; splits = (int)sp; kchunk = kc; g.bgroup = group; g.bksplit = ksplit; }
+      continue;
+    }
     for (int pass = 0; pass < 2; ++pass) {
       int sp = 1, kc = g.K > 0 ? g.K : bk;
       if (pass == 1) {
+        if (bmode) break;
         // split-K, when the tile grid alone cannot fill the device (the reduction then carries the epilogue)
         // (K slices of at least 256, or 128 when the result is small enough for a cheap reduction:
         // those problems are bound by the latency of their few K steps, not by throughput)
@@ -782,8 +844,10 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
     const size_t a_floats = a_kc ? (size_t)M * lda : (size_t)g.K * lda, b_floats = b_kc ? (size_t)N * ldb : (size_t)g.K * ldb;
     g.dma = g.K > 0 && g.K % bk == 0 && kchunk % bk == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)B % 16 == 0 &&
             lda % 4 == 0 && ldb % 4 == 0 && (a_kc || M % 4 == 0) && (b_kc || N % 4 == 0) &&
-            a_floats < (1ull << 29) && b_floats < (1ull << 29) && !tuning().gemm_nodma;
+            a_floats < (1ull << 29) && b_floats < (1ull << 29) && !tuning().gemm_nodma &&
+            g.a_bstride % 4 == 0 && g.b_bstride % 4 == 0;
   }
+  const int slices = bmode == 1 ? nbatch : splits;  // what the grid multiplies the tiles by
   if (splits > 1) {
     void *ws = nullptr;
     int rc = get_workspace((size_t)splits * M * N * sizeof(float), &ws);
@@ -791,11 +855,11 @@ static int gemm_rowmajor(bool a_kc, bool b_kc, int M, int N, int K, float alpha,
     g.ws = (float *)ws;
     g.epi = EPI_SPLITK_PARTIAL;
   }
-  int rc = cfg == 0   ? launch_cfg<TileL>(g, a_kc, b_kc, splits, st)
-           : cfg == 1 ? launch_cfg<TileM>(g, a_kc, b_kc, splits, st)
-           : cfg == 2 ? launch_cfg<TileS>(g, a_kc, b_kc, splits, st)
-           : cfg == 3 ? launch_cfg<TileLT>(g, a_kc, b_kc, splits, st)
-                      : launch_cfg<TileR>(g, a_kc, b_kc, splits, st);
+  int rc = cfg == 0   ? launch_cfg<TileL>(g, a_kc, b_kc, slices, st)
+           : cfg == 1 ? launch_cfg<TileM>(g, a_kc, b_kc, slices, st)
+           : cfg == 2 ? launch_cfg<TileS>(g, a_kc, b_kc, slices, st)
+           : cfg == 3 ? launch_cfg<TileLT>(g, a_kc, b_kc, slices, st)
+                      : launch_cfg<TileR>(g, a_kc, b_kc, slices, st);
   if (rc) return rc;
   if (splits > 1) {
     CCT_REQUIRE((size_t)M * N < (1ull << 31), "sgemm: split-K result too large");
@@ -885,4 +949,64 @@ extern "C" int cct_hip_sgemm_conv_forward(int o, int batch, int fmap, int K, con
   CCT_REQUIRE((size_t)batch * fmap < (1ull << 31), "sgemm_conv_forward: too many output positions");
   return gemm_rowmajor(true, true, o, batch * fmap, K, 1.0f, model, K, lowered, K, 0.0f, out, batch * fmap,
                        EPI_CONV_FORWARD, fmap, bias, relu != 0);
+}
+
+// ---- 1 x 1 convolution (stride 1, no padding): products on the tensors as they lie ---------------------------
+// A 1 x 1 filter needs no lowering: with `plane` = n*n pixels per map, image i of the input IS the d x plane
+// matrix of its lowered form.  Forward and data gradient are one product per image, all in one launch; the
+// weight gradient is one product summed over the images.
+static bool conv1x1_dims_ok(int batch, int depth, int plane, int num_outputs) {
+  return batch > 0 && depth > 0 && plane > 0 && num_outputs > 0 && (double)depth * plane < 2147483648.0 &&
+         (double)num_outputs * plane < 2147483648.0 && (double)depth * num_outputs < 2147483648.0;
+}
+
+extern "C" int cct_hip_conv1x1_supported(int batch, int depth, int n, int k, int stride, int padding,
+                                         int num_outputs) {
+  return k == 1 && stride == 1 && padding == 0 && n > 0 && (double)n * n < 2147483648.0 &&
+                 conv1x1_dims_ok(batch, depth, n * n, num_outputs)
+             ? 1
+             : 0;
+}
+
+extern "C" int cct_hip_conv1x1_forward(float *output, const float *input, const float *model, const float *bias,
+                                       int batch, int depth, int plane, int num_outputs, int relu) {
+  CCT_ENSURE_INIT();
+  if (batch == 0) return 0;
+  CCT_REQUIRE(conv1x1_dims_ok(batch, depth, plane, num_outputs), "conv1x1_forward: bad dimensions");
+  CCT_REQUIRE(output && input && model, "conv1x1_forward: null argument");
+  // out_i [o x plane] = model [o x d] * in_i [d x plane] + bias per row
+  const GemmBatch gb{1, batch, 0, (size_t)depth * plane, (size_t)num_outputs * plane};
+  return gemm_rowmajor(true, false, num_outputs, plane, depth, 1.0f, model, depth, input, plane, 0.0f, output, plane,
+                       EPI_CONV_FORWARD, plane, bias, relu != 0, nullptr, nullptr, &gb);
+}
+
+extern "C" int cct_hip_conv1x1_backward_data(float *input_grad, const float *output_grad, const float *model,
+                                             int batch, int depth, int plane, int num_outputs) {
+  CCT_ENSURE_INIT();
+  if (batch == 0) return 0;
+  CCT_REQUIRE(conv1x1_dims_ok(batch, depth, plane, num_outputs), "conv1x1_backward_data: bad dimensions");
+  CCT_REQUIRE(input_grad && output_grad && model, "conv1x1_backward_data: null argument");
+  // din_i [d x plane] = model^T [d x o] * dout_i [o x plane]
+  const GemmBatch gb{1, batch, 0, (size_t)num_outputs * plane, (size_t)depth * plane};
+  return gemm_rowmajor(false, false, depth, plane, num_outputs, 1.0f, model, depth, output_grad, plane, 0.0f,
+                       input_grad, plane, EPI_ALPHA_BETA, 0, nullptr, 0, nullptr, nullptr, &gb);
+}
+
+extern "C" int cct_hip_conv1x1_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
+                                                const float *input, int batch, int depth, int plane,
+                                                int num_outputs) {
+  CCT_ENSURE_INIT();
+  CCT_REQUIRE(batch >= 0 && (batch == 0 || conv1x1_dims_ok(batch, depth, plane, num_outputs)),
+              "conv1x1_backward_weights: bad dimensions");
+  CCT_REQUIRE(model_grad && (batch == 0 || (output_grad && input)), "conv1x1_backward_weights: null argument");
+  if (batch == 0) {
+    if (int rc = cct_hip_memset(model_grad, 0, (size_t)num_outputs * depth * sizeof(float))) return rc;
+    return bias_grad ? cct_hip_memset(bias_grad, 0, (size_t)num_outputs * sizeof(float)) : 0;
+  }
+  // dW [o x d] = sum_i dout_i [o x plane] * in_i^T [plane x d]
+  const GemmBatch gb{2, batch, (size_t)num_outputs * plane, (size_t)depth * plane, 0};
+  if (int rc = gemm_rowmajor(true, true, num_outputs, depth, plane, 1.0f, output_grad, plane, input, plane, 0.0f,
+                             model_grad, depth, EPI_ALPHA_BETA, 0, nullptr, 0, nullptr, nullptr, &gb))
+    return rc;
+  return bias_grad ? cct_hip_backward_bias(bias_grad, output_grad, plane, num_outputs, batch) : 0;
 }

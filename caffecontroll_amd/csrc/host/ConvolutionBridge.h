@@ -30,7 +30,9 @@
 //   * stride-1 layers with one or three input channels, k = 3 or 5 and at most 32 maps (LeNet's first
 //     layer) take plain multiply-add kernels for the forward pass and the weight gradient where they
 //     would take the all-direct path (set_small_kernels): the forward launch reads the model cube as it
-//     is, so no slabs are built for it.
+//     is, so no slabs are built for it;
+//   * 1 x 1 layers (stride 1, no padding) take level 3 as products on the tensors as they lie: lowering such a
+//     layer is a permuting copy, and so are the remap and the lifting.
 #pragma once
 #include <cstdio>
 #include <cstdlib>
@@ -147,6 +149,9 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                                (int)num_output_features);
     strided_ok_ = !direct_ok_ && group == 1 && p_driver->conv_strided_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride,
                                                                   (int)padding, (int)num_output_features);
+    pointwise_ok_ = !direct_ok_ && !strided_ok_ && group == 1 &&
+                    p_driver->conv1x1_supported((int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
+                                                (int)num_output_features);
     strided_data_ok_ = strided_ok_ && p_driver->conv_strided_backward_data_supported(
                                           (int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
                                           (int)num_output_features);
@@ -158,6 +163,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     const bool short_contraction = K * K * iD <= 64;
     default_path_ = (direct_ok_ && (gemm_flop >= kConvDirectMinFlop || short_contraction)) ? PATH_DIRECT_ALL : PATH_FUSED;
     if (strided_ok_ && gemm_flop >= kConvDirectMinFlop) default_path_ = PATH_DIRECT_ALL;
+    if (pointwise_ok_) default_path_ = PATH_DIRECT_ALL;  // fewer launches and no copies at any size
     if (group > 1) default_path_ = PATH_DIRECT_ALL;
     path_ = default_path_;
     for (int i = 0; i < STAGE_COUNT; ++i) { timers_[i] = nullptr; stage_ms_[i] = 0.f; }
@@ -192,7 +198,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   void set_path(int level) {
     if (level < PATH_STAGED) level = PATH_STAGED;
     if (level > PATH_DIRECT_ALL) level = PATH_DIRECT_ALL;
-    if (level >= PATH_DIRECT_DATA && !direct_ok_) level = (strided_ok_ && level == PATH_DIRECT_ALL) ? PATH_DIRECT_ALL : PATH_FUSED;
+    if (level >= PATH_DIRECT_DATA && !direct_ok_)
+      level = ((strided_ok_ || pointwise_ok_) && level == PATH_DIRECT_ALL) ? PATH_DIRECT_ALL : PATH_FUSED;
     if (views_ || group > 1) level = PATH_DIRECT_ALL;  // the lowering path cannot address channel slices
     path_ = level;
   }
@@ -242,8 +249,8 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   bool supports_batch_ranges() const { return path_ == PATH_DIRECT_ALL && !views_; }
   // once per pass, before the first range: the weight slabs (the model changes between iterations)
   void forward_prepare() {
-    if (small_kernels())
-      return;  // reads the model cube itself
+    if (small_kernels() || pointwise_ok_)
+      return;  // these read the model cube itself
     if (strided_ok_)
       p_driver->conv_strided_slabs(forward_slabs()->get_p_data(), p_model_cube->get_p_data(),
                                    (int)num_output_features, (int)iD, (int)K, (int)stride, (int)padding);
@@ -256,7 +263,10 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     float *out = p_output_layer->p_data_cube->get_p_data() + b0 * out_img;
     const float *in = p_input_layer->p_data_cube->get_p_data() + b0 * in_img;
     const float *bias = bias_term ? p_bias_cube->get_p_data() : nullptr;
-    if (small_kernels())
+    if (pointwise_ok_)
+      p_driver->conv1x1_forward(out, in, p_model_cube->get_p_data(), bias, (int)nb, (int)iD, (int)(iR * iC),
+                                (int)num_output_features, fuse_relu_);
+    else if (small_kernels())
       p_driver->conv_small_forward(out, in, p_model_cube->get_p_data(), bias, (int)nb, (int)iD, (int)iR, (int)K,
                                    (int)padding, (int)num_output_features, fuse_relu_);
     else if (strided_ok_)
@@ -268,8 +278,11 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   }
   // data gradient of a range; false if this layer's data gradient is not a per-range kernel (a strided layer
   // without the phase-decomposed kernel): the caller then runs backward() on the whole batch
-  bool backward_data_ranges_supported() const { return supports_batch_ranges() && (direct_ok_ || strided_data_ok_); }
+  bool backward_data_ranges_supported() const {
+    return supports_batch_ranges() && (direct_ok_ || strided_data_ok_ || pointwise_ok_);
+  }
   void backward_data_prepare() {
+    if (pointwise_ok_) return;
     if (direct_ok_)
       p_driver->conv_direct_slabs(backward_slabs()->get_p_data(), p_model_cube->get_p_data(),
                                   (int)num_output_features, (int)iD, (int)K, 1, (int)group);
@@ -282,7 +295,14 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     float *ig = p_input_layer->p_gradient_cube->get_p_data() + b0 * in_img;
     const float *og = p_output_layer->p_gradient_cube->get_p_data() + b0 * out_img;
     const float *in = p_input_layer->p_data_cube->get_p_data() + b0 * in_img;
-    if (direct_ok_) {
+    if (pointwise_ok_) {
+      p_driver->conv1x1_backward_data(ig, og, p_model_cube->get_p_data(), (int)nb, (int)iD, (int)(iR * iC),
+                                      (int)num_output_features);
+      if (input_is_relu_output) {
+        DeviceMemoryPointer g = p_driver->get_device_pointer(ig, nb * in_img * sizeof(DataType));
+        p_driver->relu_backward(&g, &g, in);
+      }
+    } else if (direct_ok_) {
       p_driver->conv_direct_backward_data(ig, og, backward_slabs()->get_p_data(), (int)nb, (int)iD, (int)iR, (int)K,
                                           (int)padding, (int)num_output_features, 0, 0,
                                           input_is_relu_output ? in : nullptr, (int)group);
@@ -301,7 +321,9 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     float *db = bias_term ? p_bias_gradient_cube->get_p_data() : nullptr;
     const float *og = p_output_layer->p_gradient_cube->get_p_data();
     const float *in = p_input_layer->p_data_cube->get_p_data();
-    if (small_kernels())
+    if (pointwise_ok_)
+      p_driver->conv1x1_backward_weights(dw, db, og, in, (int)iB, (int)iD, (int)(iR * iC), (int)num_output_features);
+    else if (small_kernels())
       p_driver->conv_small_backward_weights(dw, db, og, in, (int)iB, (int)iD, (int)iR, (int)K, (int)padding,
                                             (int)num_output_features);
     else if (strided_ok_)
@@ -328,6 +350,15 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
                                      forward_slabs()->get_p_data(), bias_term ? p_bias_cube->get_p_data() : nullptr,
                                      (int)iB, (int)iD, (int)iR, (int)K, (int)stride, (int)padding,
                                      (int)num_output_features, fuse_relu_);
+      end(STAGE_GEMM);
+      report_forward_history.end();
+      return;
+    }
+    if (path_ == PATH_DIRECT_ALL && pointwise_ok_) {
+      begin(STAGE_GEMM);
+      p_driver->conv1x1_forward(output_d_cube->get_p_data(), input_d_cube->get_p_data(), p_model_cube->get_p_data(),
+                                bias_term ? p_bias_cube->get_p_data() : nullptr, (int)iB, (int)iD, (int)(iR * iC),
+                                (int)num_output_features, fuse_relu_);
       end(STAGE_GEMM);
       report_forward_history.end();
       return;
@@ -397,6 +428,18 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
     LogicalCubeType lowered_model(p_model_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
     LogicalCubeType lowered_model_grad(p_model_gradient_cube->get_p_data(), num_output_features, K * K * iD, 1, 1);
     DeviceMemoryPointer og = output_g_cube->get_device_pointer(p_driver);
+    if (path_ == PATH_DIRECT_ALL && pointwise_ok_) {
+      begin(STAGE_GEMM_WEIGHTS);
+      backward_weights_all();
+      end(STAGE_GEMM_WEIGHTS);
+      if (needs_to_calc_backward_grad) {
+        begin(STAGE_GEMM_DATA);
+        backward_data_range(0, iB);
+        end(STAGE_GEMM_DATA);
+      }
+      report_backward_updateweight_history.end();
+      return;
+    }
     const bool direct_data = path_ >= PATH_DIRECT_DATA && needs_to_calc_backward_grad && direct_ok_;
     const bool direct_weights = path_ == PATH_DIRECT_ALL;
     // a strided layer on the all-direct path that must hand back an input gradient: the permuted output
@@ -541,6 +584,7 @@ class ConvolutionBridge : public AbstractBridge<DataType, DriverClass> {
   bool fuse_relu_ = false;
   bool direct_ok_ = false, strided_ok_ = false, strided_data_ok_ = false, profile_ = false;
   bool small_ok_ = false, use_small_ = true;
+  bool pointwise_ok_ = false;  // 1 x 1, stride 1, no padding: products on the tensors as they lie
   LogicalCubeType *lowered() {
     if (!p_forward_lowered_data) p_forward_lowered_data = new LogicalCubeType(K * K * iD, oR * oC * iB, 1, 1, p_driver);
     return p_forward_lowered_data;

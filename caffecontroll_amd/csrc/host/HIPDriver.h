@@ -294,6 +294,22 @@ class HIPDriver {
     ok(cct_hip_conv_small_backward_weights(dw, db, dout, in, batch, depth, n, k, padding, num_outputs),
        "conv_small_backward_weights");
   }
+  // ---- 1 x 1 convolutions: products on the tensors as they lie (no counterpart in DeviceDriver.h) ----
+  bool conv1x1_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs) {
+    return cct_hip_conv1x1_supported(batch, depth, n, k, stride, padding, num_outputs) != 0;
+  }
+  void conv1x1_forward(float *out, const float *in, const float *model, const float *bias, int batch, int depth,
+                       int plane, int num_outputs, bool relu) {
+    ok(cct_hip_conv1x1_forward(out, in, model, bias, batch, depth, plane, num_outputs, relu ? 1 : 0), "conv1x1_forward");
+  }
+  void conv1x1_backward_data(float *din, const float *dout, const float *model, int batch, int depth, int plane,
+                             int num_outputs) {
+    ok(cct_hip_conv1x1_backward_data(din, dout, model, batch, depth, plane, num_outputs), "conv1x1_backward_data");
+  }
+  void conv1x1_backward_weights(float *dw, float *db, const float *dout, const float *in, int batch, int depth,
+                                int plane, int num_outputs) {
+    ok(cct_hip_conv1x1_backward_weights(dw, db, dout, in, batch, depth, plane, num_outputs), "conv1x1_backward_weights");
+  }
   // `groups` > 1: a grouped convolution (depth and num_outputs are the layer's totals), all groups in one launch
   bool conv_direct_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs,
                              int groups = 1) {

@@ -145,6 +145,21 @@ class HIPDriver:
                                                  out_features, _p(relu_data)), "fc_small_backward")
 
     # -- convolutions with a very short contraction and few maps (LeNet conv1) -------------------
+    # 1 x 1 convolutions (stride 1, no padding) as products on the tensors as they lie; plane = n * n
+    def conv1x1_supported(self, b, d, n, k, s, p, o):
+        return bool(self.lib.cct_hip_conv1x1_supported(b, d, n, k, s, p, o))
+
+    def conv1x1_forward(self, out, x, w, bias, b, d, plane, o, relu=False):
+        check(self.lib.cct_hip_conv1x1_forward(_p(out), _p(x), _p(w), _p(bias), b, d, plane, o, int(relu)),
+              "conv1x1_forward")
+
+    def conv1x1_backward_data(self, dx, dout, w, b, d, plane, o):
+        check(self.lib.cct_hip_conv1x1_backward_data(_p(dx), _p(dout), _p(w), b, d, plane, o), "conv1x1_backward_data")
+
+    def conv1x1_backward_weights(self, dw, dout, x, b, d, plane, o, db=None):
+        check(self.lib.cct_hip_conv1x1_backward_weights(_p(dw), _p(db), _p(dout), _p(x), b, d, plane, o),
+              "conv1x1_backward_weights")
+
     def conv_small_supported(self, b, d, n, k, s, p, o):
         return bool(self.lib.cct_hip_conv_small_supported(b, d, n, k, s, p, o))
 

@@ -251,6 +251,22 @@ int cct_hip_conv_small_forward(float *out, const float *in, const float *w, cons
                                int k, int pad, int o, int relu);
 int cct_hip_conv_small_backward_weights(float *dw, float *db, const float *dout, const float *in, int batch, int d,
                                         int n, int k, int pad, int o);
+/* ---- 1 x 1 convolution without lowering --------------------------------------------------- */
+/* A 1 x 1 filter at stride 1 without padding makes lower_cube a permuting copy: image i of the input
+ * [batch][depth][plane] (plane = n*n) is already the depth x plane operand of its product.  These three replace
+ * lower_cube + GEMM + remap_output + bias of ConvolutionBridge::forward (src/bridges/ConvolutionBridge_impl.hxx:294-373)
+ * and remap + the two GEMMs + inverse_lower_cube + bias gradient of ::backward (:551-628) with products on the
+ * tensors as they lie: forward and data gradient one product per image (all images in one launch), the weight
+ * gradient one product summed over the images in a fixed order.  model [num_outputs][depth]; bias / bias_grad may
+ * be NULL; relu != 0 clamps the output at zero.  Results agree with the lowering path to fp32 rounding.
+ * cct_hip_conv1x1_supported: 1 for k == 1, stride == 1, padding == 0 (else 0: the lowering path takes the layer). */
+int cct_hip_conv1x1_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs);
+int cct_hip_conv1x1_forward(float *output, const float *input, const float *model, const float *bias, int batch,
+                            int depth, int plane, int num_outputs, int relu);
+int cct_hip_conv1x1_backward_data(float *input_grad, const float *output_grad, const float *model, int batch,
+                                  int depth, int plane, int num_outputs);
+int cct_hip_conv1x1_backward_weights(float *model_grad, float *bias_grad, const float *output_grad,
+                                     const float *input, int batch, int depth, int plane, int num_outputs);
 /* ---- stride-1 convolution without the lowered matrix ------------------------------------ */
 /* Fused replacements for chains of ConvolutionBridge's lowering pipeline when stride == 1 and
  * k is 3 or 5.  Forward and data gradient take an image whose padded rows exceed 64 floats in column bands;
