@@ -232,7 +232,8 @@ def test_pbridge_on_host_layers_like_the_reference_tests(share):
     layer.close()
 
 
-@pytest.mark.parametrize("shape", [(32, 48, 27, 5, 1, 2, 64), (10, 3, 67, 11, 4, 0, 32), (7, 16, 13, 3, 1, 1, 48), (3, 8, 20, 5, 1, 0, 16)],
+@pytest.mark.parametrize("shape", [(32, 48, 27, 5, 1, 2, 64), (10, 3, 67, 11, 4, 0, 32), (7, 16, 13, 3, 1, 1, 48), (3, 8, 20, 5, 1, 0, 16),
+                                   (9, 24, 14, 1, 1, 0, 40), (5, 6, 20, 7, 1, 3, 12), (6, 4, 100, 3, 1, 1, 8)],
                          ids=lambda s: "b%d_d%d_n%d_k%d_s%d_p%d_o%d" % s)
 @pytest.mark.parametrize("first_layer", [False, True])
 def test_pbridge_overlapped_staging_equals_blocking_copies(shape, first_layer):
@@ -241,7 +242,7 @@ def test_pbridge_overlapped_staging_equals_blocking_copies(shape, first_layer):
     output gradient has arrived) against one blocking copy in, the pass, one blocking copy out
     (src/bridges/ParallelizedBridge_impl.hxx:595-621, 686-705): output, input gradient, weight and bias gradients
     and the updated weights bit for bit, on pinned and on pageable host arrays, two iterations in a row; batches
-    that do not divide by four, stride-1 and strided layers."""
+    that do not divide by four, stride-1 and strided layers, a 1 x 1 layer, a 7 x 7 layer and a 100-wide image."""
     import torch
     from caffecontroll_amd.bridges import ConvolutionLayer, solver_param
     b, d, n, k, s, p, o = shape

@@ -16,7 +16,7 @@ def _conv_geometries(seed, count):
     rng = np.random.default_rng(seed)
     out = []
     while len(out) < count:
-        k, s = [(3, 1), (5, 1), (3, 1), (7, 1), (11, 4), (7, 2), (5, 2), (3, 2)][rng.integers(0, 8)]
+        k, s = [(3, 1), (5, 1), (1, 1), (7, 1), (11, 4), (7, 2), (5, 2), (3, 2)][rng.integers(0, 8)]
         p = int(rng.integers(0, k)) if rng.random() < 0.7 else (k - 1) // 2
         n = int(rng.integers(max(k - 2 * p, 1), 70 if s > 1 else 64))
         if n + 2 * p < k:
