@@ -30,7 +30,14 @@ CONFIGS = {
     "lenet_conv1": (64, 1, 28, 5, 1, 0, 20),
     "alexnet_conv2": (256, 96, 27, 5, 1, 2, 256),
     "alexnet_conv1": (256, 3, 227, 11, 4, 0, 96),
+    # geometries beyond the reference's benchmark files, for the direct paths that cover them: a VGG-sized 3 x 3
+    # layer (images in column bands), a 7 x 7 stride-1 layer, a 1 x 1 layer (products on the tensors as they lie)
+    "vgg_conv1_2": (32, 64, 224, 3, 1, 1, 64),
+    "conv7x7_56": (32, 64, 56, 7, 1, 3, 64),
+    "pointwise_28": (64, 256, 28, 1, 1, 0, 256),
 }
+SEEDS = {"alexnet_conv1": 1234, "alexnet_conv2": 1235, "lenet_conv1": 1236, "vgg_conv1_2": 1237, "conv7x7_56": 1238,
+         "pointwise_28": 1239}
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch (fetched + written) come from the committed counter summaries under profiles/
@@ -42,6 +49,9 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_SOURCE = {("alexnet_conv2", "direct"): "profiles/conv2_fwd_bwd_hbm_traffic_and_mfma.md",
                   ("alexnet_conv2", "lowering"): "profiles/conv2_lowering_path_hbm_traffic_and_mfma.md",
                   ("alexnet_conv1", "direct"): "profiles/conv1_fwd_bwd_trace_traffic_mfma.md",
+                  ("vgg_conv1_2", "direct"): "profiles/wide_3x3_layer_trace_traffic_mfma.md",
+                  ("conv7x7_56", "direct"): "profiles/conv7x7_stride1_layer_trace_traffic_mfma.md",
+                  ("pointwise_28", "direct"): "profiles/pointwise_layer_trace_traffic_mfma.md",
                   ("caffenet", "direct"): "profiles/caffenet_iteration_kernel_trace.md",
                   ("lenet", "direct"): "profiles/lenet_iteration_kernel_trace.md"}
 # which launches of a kernel a stage means, where a summary lists one kernel's launches by role
@@ -491,7 +501,7 @@ def host_layers(args, cfg, torch, np, steps=10, warmup=3):
     m = (n + 2 * p - k) // s + 1
     drv = HIPDriver(0)
     drv.set_stream(torch.cuda.current_stream().cuda_stream)
-    x, w, bias, og = synth(cfg, 1234 + sorted(CONFIGS).index(cfg), torch)
+    x, w, bias, og = synth(cfg, SEEDS[cfg], torch)
     pin = lambda a: torch.from_numpy(a).pin_memory()
     h_in, h_ig = pin(x), torch.empty((b, d, n, n)).pin_memory()
     h_out, h_og = torch.empty((b, o, m, m)).pin_memory(), pin(og)
@@ -527,7 +537,7 @@ def conv_layer(args, cfg, torch, np, steps, warmup, with_lowering=True, with_cpu
     from caffecontroll_amd.bridges import ConvolutionLayer
     b, d, n, k, s, p, o = CONFIGS[cfg]
     m = (n + 2 * p - k) // s + 1
-    seed = 1234 + sorted(CONFIGS).index(cfg)
+    seed = SEEDS[cfg]
     drv = HIPDriver(0)
     drv.set_stream(torch.cuda.current_stream().cuda_stream)
 
