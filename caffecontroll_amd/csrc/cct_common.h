@@ -27,7 +27,7 @@ struct Context {
 
 // Tuning overrides, for experiments and for tests that pin a kernel instance.  Read ONCE from the
 // environment when the library initialises (CCT_HIP_DIRECT_TILE, _DIRECT_WAVES, _DIRECT_TB,
-// _DIRECT_NOSPEC, _DIRECT_SPLITS, _DIRECT_ALDS, _STRIDED_WGRAD, _POOL_PLANE, _GEMM_NT, _GEMM_TILE, _GEMM_NODMA), changed afterwards only through
+// _DIRECT_NOSPEC, _DIRECT_SPLITS, _DIRECT_ALDS, _DIRECT_WGRAD_ROWS, _STRIDED_WGRAD, _POOL_PLANE, _GEMM_NT, _GEMM_TILE, _GEMM_NODMA), changed afterwards only through
 // cct_hip_set_tuning(); the launch paths read this struct, never the environment.
 struct Tuning {
   int direct_tile = 0;    // "<map blocks><pixel blocks>" of conv_direct_kernel, 0 = model's choice
@@ -36,6 +36,7 @@ struct Tuning {
   int direct_nospec = 0;  // 1: never take the shape-specialised weight-gradient instances
   int direct_splits = 0;  // step ranges of the weight-gradient launch (its partial sums), 0 = model's choice
   int direct_alds = 0;    // specialised weight-gradient instances: 1 = dout rows through LDS, 2 = never, 0 = model's choice
+  int direct_wgrad_rows = 0;  // stride-1 weight gradient: 1 = image-pair kernels wherever they apply, 2 = one image per step always, 0 = model's choice
   int strided_wgrad = 0;  // strided weight-gradient tile: row pieces * 1000 + column blocks * 100 + column groups * 10 + row blocks, 0 = model's choice
   int pool_plane = 0;     // 1: plane-tiled pooling kernels at any size
   int gemm_nt = 0;        // 1: non-temporal stores in the GEMM epilogue

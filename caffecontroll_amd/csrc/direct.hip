@@ -1630,7 +1630,17 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
                              int ks, int pad, int o, size_t src_img_stride, size_t dout_img_stride, int groups = 1) {
   WgradPlan pl;
   CCT_REQUIRE(groups >= 1, "conv_direct wgrad: groups must be positive");
-  if (!wgrad_plan(batch, d, n, ks, pad, o, &pl, groups)) {
+  bool pairs = wgrad_plan(batch, d, n, ks, pad, o, &pl, groups);
+  if (pairs && tuning().direct_wgrad_rows != 1) {
+    // Image pairs pay off on short rows (a step of the one-image kernel is half as many MFMAs deep) and where a
+    // compile-time instance exists.  Measured at 3 x 3: 13-14 pixel rows 80-129 against 53-58 TFLOP/s, 16 pixels
+    // equal, 20-30 pixels 25-80 against 50-80 (the generic image-pair kernel wants 128 maps per workgroup).
+    const bool rows = tuning().direct_wgrad_rows == 2 || (!pl.spec && n + 2 * pad > 18);
+    if (rows && conv_strided_wgrad_covers(batch, d * groups, n, ks, 1, pad, o * groups) &&
+        conv_strided_wgrad_covers(batch, d, n, ks, 1, pad, o))
+      pairs = false;
+  }
+  if (!pairs) {
     // rows too long for the image-pair kernels: the one-image-per-step kernel, if its patch holds them,
     // group by group on channel slices
     CCT_REQUIRE(conv_strided_wgrad_covers(batch, d * groups, n, ks, 1, pad, o * groups) &&

@@ -105,7 +105,8 @@ int cct_hip_set_stream(void *hip_stream);
  * pixels, 0 = automatic), "direct_waves",
  * "direct_tb", "direct_nospec", "direct_splits" (step ranges of the direct weight-gradient launch, 0 = automatic),
  * "direct_alds" (shape-specialised weight-gradient kernels: 1 = output-gradient rows staged in LDS, 2 = fetched by
- * their lanes, 0 = automatic), "strided_wgrad" (tile of the strided weight-gradient kernel: pieces of an output row
+ * their lanes, 0 = automatic), "direct_wgrad_rows" (stride-1 weight gradient: 1 = the image-pair kernels wherever they
+ * apply, 2 = the one-image-per-step kernel always, 0 = automatic), "strided_wgrad" (tile of the strided weight-gradient kernel: pieces of an output row
  * x 1000 + column blocks x 100 + column groups x 10 + row blocks, 0 = automatic), "pool_plane", "gemm_nt", "gemm_tile" (-1 = automatic), "gemm_nodma" (1 = GEMM
  * operand tiles always staged through registers).  The
  * environment variables CCT_HIP_<NAME IN CAPITALS> give the initial values; they are read once,
