@@ -1633,9 +1633,10 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   bool pairs = wgrad_plan(batch, d, n, ks, pad, o, &pl, groups);
   if (pairs && tuning().direct_wgrad_rows != 1) {
     // Image pairs pay off on short rows (a step of the one-image kernel is half as many MFMAs deep) and where a
-    // compile-time instance exists.  Measured at 3 x 3: 13-14 pixel rows 80-129 against 53-58 TFLOP/s, 16 pixels
-    // equal, 20-30 pixels 25-80 against 50-80 (the generic image-pair kernel wants 128 maps per workgroup).
-    const bool rows = tuning().direct_wgrad_rows == 2 || (!pl.spec && n + 2 * pad > 18);
+    // compile-time instance exists.  Measured at 3 x 3, pairs against rows: 7-14 pixel rows 65-91 against 53-81
+    // TFLOP/s (129 against 70 with a compile-time instance), 16 pixels 61 against 78, 20-30 pixels 25-81 against
+    // 61-101 (the generic image-pair kernel wants 128 maps per workgroup).
+    const bool rows = tuning().direct_wgrad_rows == 2 || (!pl.spec && n + 2 * pad > 17);
     if (rows && conv_strided_wgrad_covers(batch, d * groups, n, ks, 1, pad, o * groups) &&
         conv_strided_wgrad_covers(batch, d, n, ks, 1, pad, o))
       pairs = false;

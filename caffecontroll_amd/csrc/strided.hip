@@ -26,6 +26,7 @@
 //
 // Bound: fp32 MFMA rate.  Algorithmic work 2 * mtot * batch*ho*ho * kc*KS*KS FLOP per call.
 #include <cstdlib>
+#include <type_traits>
 
 #include "cct_common.h"
 #include "mfma_common.h"
@@ -731,14 +732,70 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
     if (S * x_last + (int)pcol - g.pad < g.hs) b_last |= 1u << k;     // not right of it in the last piece
   }
   const rsrc_t a_rsrc = make_rsrc(g.dout), b_rsrc = make_rsrc(g.src - g.pad);
+  if (g.nchunks == 1) {
+    // a row in one piece: what the first and the last piece leave out is left out of every step
+#pragma unroll
+    for (int k = 0; k < NAL; ++k)
+      if (!((a_last >> k) & 1u)) aoff[k] = kOutOfRange;
+#pragma unroll
+    for (int k = 0; k < NBL; ++k)
+      if (!((b_first & b_last) >> k & 1u)) boff[k] = kOutOfRange;
+  }
+  // (image, output row, piece) of the next step to fetch, kept as counters (steps are fetched in order)
+  int nx_img, nx_y, nx_piece;
+  {
+    const uint32_t rowid = fdiv((uint32_t)s_beg, g.div_nchunks);
+    nx_piece = s_beg - (int)rowid * g.nchunks;
+    nx_img = (int)fdiv(rowid, g.div_ho);
+    nx_y = (int)rowid - nx_img * g.ho;
+  }
 
-// global -> LDS stage st for step s
+// global -> LDS stage st for the next step.  A step whose k source rows lie inside the image -- nearly every one --
+// needs next to no per-lane work: every load is a fixed lane offset plus a scalar offset, and only the first and
+// the last piece of a row in several pieces mark the words they lack (two instructions per load).  (Issuing these
+// loads in batches between the MFMAs of the current step instead of all at its start measured 3-10 % slower.)
 #define CCT_SWGRAD_ISSUE(s, st)                                                                   \
   do {                                                                                            \
-    const uint32_t rowid_ = fdiv((uint32_t)(s), g.div_nchunks);                                   \
-    const int piece_ = (s) - (int)rowid_ * g.nchunks, x0_ = piece_ * g.cw;                        \
-    const uint32_t img_ = fdiv(rowid_, g.div_ho);                                                 \
-    const int y_ = (int)rowid_ - (int)img_ * g.ho;                                                \
+    const int piece_ = nx_piece, x0_ = piece_ * g.cw, y_ = nx_y;                                  \
+    const uint32_t img_ = (uint32_t)nx_img;                                                       \
+    if (++nx_piece == g.nchunks) {                                                                \
+      nx_piece = 0;                                                                               \
+      if (++nx_y == g.ho) { nx_y = 0; ++nx_img; }                                                 \
+    }                                                                                             \
+    const int top_ = S * y_ - g.pad;                                                              \
+    if (top_ >= 0 && top_ + KS <= g.hs) {                                                         \
+      float *sa_ = smem + (st) * stage + wave * 64;                                               \
+      const uint32_t ga_ =                                                                        \
+          (uint32_t)(((size_t)img_ * g.dout_img_stride + (size_t)m0 * ho2 + y_ * g.ho + x0_) * 4); \
+      float *sb_ = sa_ + g.a_floats;                                                              \
+      const uint32_t gb_ = (uint32_t)(((size_t)img_ * g.src_img_stride + (size_t)ch0 * hs2 +      \
+                                       (size_t)top_ * g.hs + (size_t)S * x0_) * 4);               \
+      /* counts and strides read afresh: kept across the loop they (and every multiple the loads use) would be */ \
+      /* scalar registers spilled to lanes and read back with a vector instruction apiece            */ \
+      int nal_ = g.nal, nbl_ = g.nbl, nth_ = nthreads;                                            \
+      asm volatile("" : "+s"(nal_), "+s"(nbl_), "+s"(nth_));                                      \
+      if (g.nchunks == 1 || (piece_ > 0 && piece_ < g.nchunks - 1)) {                             \
+        _Pragma("unroll") for (int k = 0; k < NAL; ++k) {                                         \
+          if (__builtin_expect(k < nal_, 1)) lds_dma4(a_rsrc, aoff[k], ga_, sa_ + k * nth_);     \
+        }                                                                                         \
+        _Pragma("unroll") for (int k = 0; k < NBL; ++k) {                                         \
+          if (__builtin_expect(k < nbl_, 1)) lds_dma4(b_rsrc, boff[k], gb_, sb_ + k * nth_);     \
+        }                                                                                         \
+      } else {                                                                                    \
+        /* first or last piece of a row: the words it lacks get the top offset bit (out of range) */ \
+        const uint32_t na_ = piece_ == g.nchunks - 1 ? ~a_last : 0u;                              \
+        const uint32_t nb_ = (piece_ == 0 ? ~b_first : 0u) | (piece_ == g.nchunks - 1 ? ~b_last : 0u); \
+        _Pragma("unroll") for (int k = 0; k < NAL; ++k) {                                         \
+          if (__builtin_expect(k < nal_, 1))                                                      \
+            lds_dma4(a_rsrc, aoff[k] | (((na_ >> k) & 1u) << 31), ga_, sa_ + k * nth_);           \
+        }                                                                                         \
+        _Pragma("unroll") for (int k = 0; k < NBL; ++k) {                                         \
+          if (__builtin_expect(k < nbl_, 1))                                                      \
+            lds_dma4(b_rsrc, boff[k] | (((nb_ >> k) & 1u) << 31), gb_, sb_ + k * nth_);           \
+        }                                                                                         \
+      }                                                                                           \
+      break;                                                                                      \
+    }                                                                                             \
     const uint32_t ma_ = piece_ == g.nchunks - 1 ? a_last : ~0u;                                  \
     const uint32_t mb_ = (piece_ == 0 ? b_first : ~0u) & (piece_ == g.nchunks - 1 ? b_last : ~0u); \
     float *sa_ = smem + (st) * stage + wave * 64;                                                 \
@@ -752,7 +809,6 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
         (uint32_t)(((size_t)img_ * g.src_img_stride + (size_t)ch0 * hs2 + (size_t)S * x0_) * 4);  \
     /* the first patch row may lie above the image: that (negative) term goes into the lane     */ \
     /* offset, whose sum is non-negative for every lane that passes the row test                */ \
-    const int top_ = S * y_ - g.pad;                                                              \
     const uint32_t row0_ = (uint32_t)(top_ * g.hs * 4);                                           \
     _Pragma("unroll") for (int k = 0; k < NBL; ++k) {                                             \
       const int srow_ = top_ + (int)((brow[k / 5] >> (6 * (k % 5))) & 63u);                       \
@@ -777,6 +833,7 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
 #pragma unroll
     for (int e = 0; e < 16; ++e) acc[b][e] = 0.0f;
   float bsum = 0.0f;  // lane (r, h) adds up dout[map r][every image][every row][x = h (mod 2)]
+  const bool want_bias = g.out_bias && tn == 0 && wni == 0;  // wavefront-uniform
 
   if (s_beg < s_end) {
     CCT_SWGRAD_ISSUE(s_beg, 0);
@@ -787,20 +844,26 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
   for (int s = s_beg; s < s_end; ++s) {
     const int cur = (s - s_beg) & 1;
     if (s + 1 < s_end) CCT_SWGRAD_ISSUE(s + 1, cur ^ 1);
-    const float *sa = smem + cur * stage + abase;
-    const float *sb[TB];
+    // LDS addresses of this lane's fragments at pixel 0 of the step, as registers of their own that advance once per
+    // trip of the pixel loop (left to itself the compiler re-adds the stage to every one of them every trip:
+    // vector ALU instructions take MFMA issue slots)
+    typedef __attribute__((address_space(3))) const float lds_cfloat;
+    lds_cfloat *ia = (lds_cfloat *)smem + (cur * stage + abase), *ib[TB];
+    asm volatile("" : "+v"(ia));
 #pragma unroll
-    for (int b = 0; b < TB; ++b) sb[b] = smem + cur * stage + bbase[b];
+    for (int b = 0; b < TB; ++b) {
+      ib[b] = (lds_cfloat *)smem + (cur * stage + bbase[b]);
+      asm volatile("" : "+v"(ib[b]));
+    }
     // fragment buffers; reads past ho stay inside the stage and meet zero dout words
     float fa[2], fb[2][TB];
 #define CCT_SWGRAD_FRAGS(buf, x)                                                                  \
   do {                                                                                            \
-    fa[buf] = sa[(x)];                                                                            \
-    _Pragma("unroll") for (int b = 0; b < TB; ++b) fb[buf][b] = sb[b][S * (x)];                   \
+    fa[buf] = ia[(x)];                                                                            \
+    _Pragma("unroll") for (int b = 0; b < TB; ++b) fb[buf][b] = ib[b][S * (x)];                   \
   } while (0)
 #define CCT_SWGRAD_MFMA(buf)                                                                      \
   do {                                                                                            \
-    bsum += fa[buf];                                                                              \
     _Pragma("unroll") for (int b = 0; b < TB; ++b)                                                \
         acc[b] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[buf], fb[buf][b], acc[b], 0, 0, 0);      \
   } while (0)
@@ -815,16 +878,37 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
     }                                                                                             \
     __builtin_amdgcn_sched_barrier(0);                                                            \
   } while (0)
-    CCT_SWGRAD_FRAGS(0, 0);
-    for (int qd = 0; qd < g.nq2; ++qd) {
-      const int x = 4 * qd;
-      CCT_SWGRAD_FRAGS(1, x + 2);
-      CCT_SWGRAD_MFMA(0);
-      CCT_SWGRAD_ORDER();
-      CCT_SWGRAD_FRAGS(0, x + 4);
-      CCT_SWGRAD_MFMA(1);
-      CCT_SWGRAD_ORDER();
+// four pixels from offset x of the address registers; the wavefronts that own a part of the bias gradient (few)
+// add up their dout fragments, behind a scalar branch
+#define CCT_SWGRAD_QUAD(x)                                                                        \
+  do {                                                                                            \
+    CCT_SWGRAD_FRAGS(1, (x) + 2);                                                                 \
+    CCT_SWGRAD_MFMA(0);                                                                           \
+    CCT_SWGRAD_ORDER();                                                                           \
+    if (__builtin_expect(bias_flag != 0, 0)) bsum += fa[0] + fa[1];                               \
+    CCT_SWGRAD_FRAGS(0, (x) + 4);                                                                 \
+    CCT_SWGRAD_MFMA(1);                                                                           \
+    CCT_SWGRAD_ORDER();                                                                           \
+  } while (0)
+    {
+      int bias_flag = __builtin_amdgcn_readfirstlane(want_bias ? 1 : 0);
+      asm volatile("" : "+s"(bias_flag));  // a scalar test every time, not a lane mask and a select
+      CCT_SWGRAD_FRAGS(0, 0);
+      int qd = 0;
+      for (; qd + 2 <= g.nq2; qd += 2) {
+        CCT_SWGRAD_QUAD(0);
+        CCT_SWGRAD_QUAD(4);
+        ia += 8;
+        asm volatile("" : "+v"(ia));
+#pragma unroll
+        for (int b = 0; b < TB; ++b) {
+          ib[b] += 8 * S;
+          asm volatile("" : "+v"(ib[b]));
+        }
+      }
+      if (qd < g.nq2) CCT_SWGRAD_QUAD(0);
     }
+#undef CCT_SWGRAD_QUAD
 #undef CCT_SWGRAD_FRAGS
 #undef CCT_SWGRAD_MFMA
 #undef CCT_SWGRAD_ORDER
@@ -833,7 +917,7 @@ __global__ __launch_bounds__(768) void conv_strided_wgrad_kernel(const StridedWg
   }
 #undef CCT_SWGRAD_ISSUE
 
-  if (g.out_bias && tn == 0 && wni == 0) {
+  if (want_bias) {
     const float both = bsum + __shfl_xor(bsum, 32);
     const int row = m0 + wmi * 32 + r;
     if (h == 0 && row < g.o) g.out_bias[(size_t)z * g.o + row] = both;
