@@ -233,6 +233,8 @@ GROUPED = [
     (2, 15, 44, 3, 1, 36, 3, 11),     # padded rows of 46 floats: the one-image-per-step weight gradient, group by group
     (3, 96, 27, 5, 2, 32, 2, 161),    # 48 channels per group: the data gradient runs on 16-row tiles
     (2, 12, 9, 5, 4, 160, 4, 161),    # 40 maps per group forward (three 16-row blocks), 3 channels per group
+    (2, 6, 100, 3, 1, 10, 2, 11),     # images in two column bands, weight-gradient rows in pieces, on channel slices
+    (2, 8, 21, 7, 3, 12, 2, 21),      # 7 x 7
 ]
 
 
