@@ -13,8 +13,9 @@
 // the lowering path to fp32 rounding, not bit for bit.
 //
 // One workgroup (4 wavefronts) computes BM = 32*TMB output maps x BN = 128*TNB consecutive output
-// pixels (pixels are numbered across the whole batch, so a tile may straddle images).  The
-// contraction index is consumed two*CP channels per step:
+// pixels (pixels are numbered across the whole batch, so a tile may straddle images; an image whose
+// padded rows exceed a patch row is cut into column bands that are numbered like images, see
+// DirectArgs::wv).  KS is 3, 5 or 7.  The contraction index is consumed two*CP channels per step:
 //   * the weight slab of a channel, wt[c][m0..m0+BM)[KS*KS], is one contiguous run in memory and is
 //     copied to LDS as is (16-byte loads);
 //   * the source rows that the tile's pixels touch are copied to a zero-bordered LDS patch of

@@ -12,7 +12,7 @@
 //     of running remap_output and the bias map as separate passes (set_fused(false) restores
 //     the staged sequence);
 //   * the bias gradient is reduced in the same launch as the lifting kernel;
-//   * for stride-1 layers with k = 3 or 5 the data gradient (path level 2) or all three products
+//   * for stride-1 layers with k = 3, 5 or 7 the data gradient (path level 2) or all three products
 //     (level 3, the default where the geometry allows it) come from direct-convolution kernels
 //     that never materialise the lowered matrices; results then agree with the lowering path to
 //     fp32 rounding instead of bit for bit.  The lowered buffers are allocated on first use, so

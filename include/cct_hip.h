@@ -270,7 +270,7 @@ int cct_hip_conv1x1_backward_weights(float *model_grad, float *bias_grad, const 
                                      const float *input, int batch, int depth, int plane, int num_outputs);
 /* ---- stride-1 convolution without the lowered matrix ------------------------------------ */
 /* Fused replacements for chains of ConvolutionBridge's lowering pipeline when stride == 1 and
- * k is 3 or 5.  Forward and data gradient take an image whose padded rows exceed 64 floats in column bands;
+ * k is 3, 5 or 7.  Forward and data gradient take an image whose padded rows exceed 64 floats in column bands;
  * the weight gradient has image-pair kernels for padded rows of up to 32 floats and otherwise takes one image
  * per step and long output rows in up to 64 pieces (what bounds the width: a few thousand columns, fewer for a
  * layer with under 32 maps).  Results agree with the

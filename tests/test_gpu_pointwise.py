@@ -163,7 +163,7 @@ def test_bridge_runs_pointwise_layers_without_lowering(oracle, shape):
         kernels = layer.stage_kernels()
         if level is None:
             assert kernels["Lower Cube"] == "" and kernels["Inverse Lwr"] == "" and kernels["Bw Remap"] == ""
-            assert kernels["GEMM"].startswith("gemm_kernel") and kernels["GEMM Wghts"] != ""
+            assert kernels["GEMM"].startswith("gemm_batched_kernel") and kernels["GEMM Wghts"] != ""
         else:
             assert kernels["Lower Cube"] != ""
         assert rel_err(host(out_data), ref_out) <= TOL, level
