@@ -462,7 +462,10 @@ def test_bridge_falls_back_where_direct_does_not_apply():
 # one group of conv4; between them they run every compile-time specialised weight-gradient instance
 # (8, 4 and 6 wavefronts)
 FULL_SIZE = [(256, 96, 27, 5, 2, 256), (256, 48, 27, 5, 2, 128), (256, 256, 13, 3, 1, 384),
-             (256, 192, 13, 3, 1, 192), (255, 192, 13, 3, 1, 128)]
+             (256, 192, 13, 3, 1, 192), (255, 192, 13, 3, 1, 128),
+             # beyond CaffeNet: a VGG-sized 3 x 3 layer (four column bands, weight-gradient rows in four pieces), a
+             # 112-wide one with an odd batch, a 7 x 7 stride-1 layer
+             (32, 64, 224, 3, 1, 64), (17, 128, 112, 3, 1, 128), (32, 64, 56, 7, 3, 64)]
 
 
 # the grouped layers of the CaffeNet iteration at batch 256, both groups in one launch: conv2, conv4, conv5

@@ -324,6 +324,39 @@ def test_caffenet_full_batch_iteration_untouched(oracle):
     net.close()
 
 
+@pytest.mark.parametrize("level", [3, -1])
+def test_wide_network_in_network_style_iterations(oracle, level):
+    """A chain with the geometries beyond CaffeNet's and LeNet's: 3x72x72 inputs, a 7 x 7 stride-1 layer (images in
+    column bands on the all-direct path), 1 x 1 layers (products on the tensors as they lie at any level), a 3 x 3 layer
+    on 36-pixel rows (weight gradient one image per step); two training iterations with momentum and weight decay,
+    every layer's output, the loss and every updated parameter against the oracle chain."""
+    from caffecontroll_amd import nets
+    rng = np.random.default_rng(77 + level)
+    B, D, S, classes = 6, 3, 72, 7
+    layers = [nets.conv(16, 7, 1, 3), nets.relu(), nets.conv(24, 1), nets.relu(), nets.maxpool(2, 2),
+              nets.conv(32, 3, 1, 1), nets.relu(), nets.maxpool(2, 2), nets.conv(16, 1), nets.relu(),
+              nets.fc(classes), nets.softmax_loss()]
+    solver = dict(base_lr=0.01, momentum=0.9, weight_decay=0.0005)
+    driver()
+    net = nets.Net(B, D, S, layers, nets.solver_param(**solver))
+    net.set_conv_path(level)
+    ref = OracleNet(oracle, layers, B, D, S, solver)
+    _init_and_sync_params(net, ref, rng)
+    for _ in range(2):
+        x = rng.standard_normal((B, D, S, S)).astype(np.float32)
+        labels = rng.integers(0, classes, B).astype(np.float32)
+        _up(net.input_ptr(), x)
+        _up(net.labels_ptr(), labels)
+        net.forward()
+        ref.forward(x, labels)
+        _check_forward_and_align_switches(net, ref, layers, TOL)
+        assert abs(net.loss() - ref.loss) <= TOL * max(1.0, abs(ref.loss))
+        net.backward()
+        ref.backward()
+        _compare_params(net, ref, TOL)
+    net.close()
+
+
 def test_dropout_masks_change_and_test_phase_is_identity():
     from caffecontroll_amd import nets
     driver()
