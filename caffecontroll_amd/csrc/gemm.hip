@@ -258,7 +258,8 @@ struct FastLoader {
 //                        of stage t run, then the fragments of k-group 1 of stage t+1 are requested
 // so LDS and HBM latencies are covered by 32 MFMAs (2048 matrix-pipe cycles) each.
 template <class T, bool A_KC, bool B_KC>
-__device__ __forceinline__ void gemm_mainloop(const GemmArgs &g, float *smem, v16f (&acc)[T::TM][T::TN], int m0,
+__device__ __forceinline__ void gemm_mainloop(const GemmArgs &g, const float *__restrict__ Ap,
+                                              const float *__restrict__ Bp, float *smem, v16f (&acc)[T::TM][T::TN], int m0,
                                               int n0, int kbeg, int kend, int nk, int tid, int lane, int wm0,
                                               int wn0) {
   using LA = OperandLayout<T, A_KC, T::BM>;
@@ -268,16 +269,16 @@ __device__ __forceinline__ void gemm_mainloop(const GemmArgs &g, float *smem, v1
   f4 ra[LA::NV], rb[LB::NV];
   FastLoader<T, A_KC, T::BM> la;
   FastLoader<T, B_KC, T::BN> lb;
-  la.init(g.A, g.lda, m0, kbeg, g.M, tid);
-  lb.init(g.B, g.ldb, n0, kbeg, g.N, tid);
+  la.init(Ap, g.lda, m0, kbeg, g.M, tid);
+  lb.init(Bp, g.ldb, n0, kbeg, g.N, tid);
   const int nk_full = (kend - kbeg) / T::BK;
 // global -> registers for K step t
 #define CCT_FETCH(t)                                                                         \
   do {                                                                                       \
     if ((t) >= nk_full) {                                                                    \
       const int k0_ = kbeg + (t) * T::BK;                                                    \
-      load_tile<T, A_KC, T::BM>(ra, g.A, g.lda, m0, k0_, g.M, kend, 0, tid);                 \
-      load_tile<T, B_KC, T::BN>(rb, g.B, g.ldb, n0, k0_, g.N, kend, 0, tid);                 \
+      load_tile<T, A_KC, T::BM>(ra, Ap, g.lda, m0, k0_, g.M, kend, 0, tid);                  \
+      load_tile<T, B_KC, T::BN>(rb, Bp, g.ldb, n0, k0_, g.N, kend, 0, tid);                  \
     } else {                                                                                 \
       la.load(ra, g.a_vec);                                                                  \
       lb.load(rb, g.b_vec);                                                                  \
@@ -396,7 +397,8 @@ struct DmaFrags {
 //                        of k-group 0 of stage t+1 are requested, MFMAs of k-group 1 of stage t run,
 //                        the fragments of k-group 1 of stage t+1 are requested
 template <class T, bool A_KC, bool B_KC>
-__device__ __forceinline__ void gemm_mainloop_dma(const GemmArgs &g, float *smem, v16f (&acc)[T::TM][T::TN], int m0,
+__device__ __forceinline__ void gemm_mainloop_dma(const GemmArgs &g, const float *Ap, const float *Bp, float *smem,
+                                                  v16f (&acc)[T::TM][T::TN], int m0,
                                                   int n0, int kbeg, int nk, int lane, int wave, int wm0,
                                                   int wn0) {
   using DA = DmaLayout<T, A_KC, T::BM>;
@@ -410,7 +412,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmArgs &g, float *smem
   for (int i = 0; i < DA::NV; ++i) aoff[i] = DA::source(i, wave, lane, m0, g.M, g.lda);
 #pragma unroll
   for (int i = 0; i < DB::NV; ++i) boff[i] = DB::source(i, wave, lane, n0, g.N, g.ldb);
-  const rsrc_t a_rsrc = make_rsrc(g.A), b_rsrc = make_rsrc(g.B);
+  const rsrc_t a_rsrc = make_rsrc(Ap), b_rsrc = make_rsrc(Bp);
   const uint32_t a_step = A_KC ? (uint32_t)T::BK * 4u : (uint32_t)T::BK * (uint32_t)g.lda * 4u;
   const uint32_t b_step = B_KC ? (uint32_t)T::BK * 4u : (uint32_t)T::BK * (uint32_t)g.ldb * 4u;
   const uint32_t a_k0 = A_KC ? (uint32_t)kbeg * 4u : (uint32_t)kbeg * (uint32_t)g.lda * 4u;
@@ -470,7 +472,7 @@ __device__ __forceinline__ void gemm_mainloop_dma(const GemmArgs &g, float *smem
 // lie inside C too, no bounds tests at all; true: rows past M are skipped (M not a multiple of the
 // tile height, e.g. 96 output maps).  row0/col0 are the lane's first row and column.
 template <class T, int MODE, bool ROWGUARD>
-__device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&acc)[T::TM][T::TN], int row0,
+__device__ __forceinline__ void fast_epilogue(const GemmArgs &g, float *Cp, const v16f (&acc)[T::TM][T::TN], int row0,
                                               int col0, uint32_t kslice) {
   if (MODE == EPI_CONV_FORWARD) {
     size_t coff[T::TN];
@@ -488,7 +490,7 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
         for (int i = 0; i < 4; ++i) {
           const int row = row0 + a * 32 + 8 * j + i;
           if (ROWGUARD && row >= g.M) continue;
-          float *c = g.C + (size_t)row * g.fmap;
+          float *c = Cp + (size_t)row * g.fmap;
           const float add = g.bias ? g.bias[row] : 0.0f;
 #pragma unroll
           for (int b = 0; b < T::TN; ++b) {
@@ -498,7 +500,7 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
         }
   } else {
     const size_t rstride = (MODE == EPI_SPLITK_PARTIAL) ? (size_t)g.N : (size_t)g.ldc;
-    float *crow = ((MODE == EPI_SPLITK_PARTIAL) ? g.ws + (size_t)kslice * g.M * g.N : g.C) +
+    float *crow = ((MODE == EPI_SPLITK_PARTIAL) ? g.ws + (size_t)kslice * g.M * g.N : Cp) +
                   (size_t)row0 * rstride + col0;
     const float alpha = g.alpha;
     // column bias and clamp of the plain epilogue (a fully connected layer's forward pass); uniform
@@ -527,23 +529,14 @@ __device__ __forceinline__ void fast_epilogue(const GemmArgs &g, const v16f (&ac
   }
 }
 
-// The kernel's arguments as they are, or (batched modes, which move the matrix pointers) a copy of them.  The plain
-// kernel must not take the copy: with it the 128 x 128 instances hold 137-144 instead of 108-110 registers and
-// the inner-product GEMMs of CaffeNet run 13 % slower.
-template <bool BATCHED> struct GemmArgHolder;
-template <> struct GemmArgHolder<false> {
-  const GemmArgs &g;
-  __device__ __forceinline__ explicit GemmArgHolder(const GemmArgs &a) : g(a) {}
-};
-template <> struct GemmArgHolder<true> {
-  GemmArgs g;
-  __device__ __forceinline__ explicit GemmArgHolder(const GemmArgs &a) : g(a) {}
-};
-
+// One workgroup's tile.  BATCHED: a batch of products in one launch (GemmArgs::bmode) -- the matrix pointers move
+// with the slice and the main loop sits in a loop over images.  That costs the 128 x 128 instances 30 registers
+// (and cost the inner-product GEMMs of CaffeNet 13 % while the plain kernel carried it), so the batched form is a
+// template parameter and has kernels of its own.
 template <class T, bool A_KC, bool B_KC, bool DMA, bool BATCHED>
-__device__ __forceinline__ void gemm_workgroup(const GemmArgs &g_in, float *smem) {
-  GemmArgHolder<BATCHED> holder(g_in);
-  auto &g = holder.g;
+__device__ __forceinline__ void gemm_workgroup(const GemmArgs &g, float *smem) {
+  const float *Ap = g.A, *Bp = g.B;
+  float *Cp = g.C;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -568,9 +561,9 @@ __device__ __forceinline__ void gemm_workgroup(const GemmArgs &g_in, float *smem
     const uint32_t igroup = g.bmode == 1 ? kslice : kslice / (uint32_t)g.bksplit;
     kbeg = g.bmode == 1 ? 0 : (int)(kslice - igroup * g.bksplit) * g.kchunk;
     const uint32_t img = g.bmode == 1 ? igroup : igroup * (uint32_t)g.bgroup;
-    g.A += (size_t)img * g.a_bstride;
-    g.B += (size_t)img * g.b_bstride;
-    if (g.bmode == 1) g.C += (size_t)img * g.c_bstride;
+    Ap += (size_t)img * g.a_bstride;
+    Bp += (size_t)img * g.b_bstride;
+    if (g.bmode == 1) Cp += (size_t)img * g.c_bstride;
     else more_images = min(g.bgroup, g.nbatch - (int)img) - 1;
   }
   const int kend = min(g.K, kbeg + g.kchunk);
@@ -586,17 +579,17 @@ __device__ __forceinline__ void gemm_workgroup(const GemmArgs &g_in, float *smem
 
   if constexpr (BATCHED) {
     for (;;) {
-      if (DMA) gemm_mainloop_dma<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, nk, lane, __builtin_amdgcn_readfirstlane(wave), wm0, wn0);
-      else gemm_mainloop<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
+      if (DMA) gemm_mainloop_dma<T, A_KC, B_KC>(g, Ap, Bp, smem, acc, m0, n0, kbeg, nk, lane, __builtin_amdgcn_readfirstlane(wave), wm0, wn0);
+      else gemm_mainloop<T, A_KC, B_KC>(g, Ap, Bp, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
       if (--more_images < 0) break;
       // the next image of the sum: same tile, same accumulators; the LDS stages are refilled from scratch
-      g.A += g.a_bstride;
-      g.B += g.b_bstride;
+      Ap += g.a_bstride;
+      Bp += g.b_bstride;
       __syncthreads();
     }
   } else {
-    if (DMA) gemm_mainloop_dma<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, nk, lane, __builtin_amdgcn_readfirstlane(wave), wm0, wn0);
-    else gemm_mainloop<T, A_KC, B_KC>(g, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
+    if (DMA) gemm_mainloop_dma<T, A_KC, B_KC>(g, Ap, Bp, smem, acc, m0, n0, kbeg, nk, lane, __builtin_amdgcn_readfirstlane(wave), wm0, wn0);
+    else gemm_mainloop<T, A_KC, B_KC>(g, Ap, Bp, smem, acc, m0, n0, kbeg, kend, nk, tid, lane, wm0, wn0);
   }
   const bool rows_inside = m0 + T::BM <= g.M, cols_inside = n0 + T::BN <= g.N;
 
@@ -605,13 +598,13 @@ __device__ __forceinline__ void gemm_workgroup(const GemmArgs &g_in, float *smem
   if (cols_inside && !(g.epi == EPI_ALPHA_BETA && g.beta != 0.0f)) {
     const int er = m0 + wm0 + 4 * h, ec = n0 + wn0 + r;
     if (rows_inside) {
-      if (g.epi == EPI_ALPHA_BETA) fast_epilogue<T, EPI_ALPHA_BETA, false>(g, acc, er, ec, kslice);
-      else if (g.epi == EPI_SPLITK_PARTIAL) fast_epilogue<T, EPI_SPLITK_PARTIAL, false>(g, acc, er, ec, kslice);
-      else fast_epilogue<T, EPI_CONV_FORWARD, false>(g, acc, er, ec, kslice);
+      if (g.epi == EPI_ALPHA_BETA) fast_epilogue<T, EPI_ALPHA_BETA, false>(g, Cp, acc, er, ec, kslice);
+      else if (g.epi == EPI_SPLITK_PARTIAL) fast_epilogue<T, EPI_SPLITK_PARTIAL, false>(g, Cp, acc, er, ec, kslice);
+      else fast_epilogue<T, EPI_CONV_FORWARD, false>(g, Cp, acc, er, ec, kslice);
     } else {
-      if (g.epi == EPI_ALPHA_BETA) fast_epilogue<T, EPI_ALPHA_BETA, true>(g, acc, er, ec, kslice);
-      else if (g.epi == EPI_SPLITK_PARTIAL) fast_epilogue<T, EPI_SPLITK_PARTIAL, true>(g, acc, er, ec, kslice);
-      else fast_epilogue<T, EPI_CONV_FORWARD, true>(g, acc, er, ec, kslice);
+      if (g.epi == EPI_ALPHA_BETA) fast_epilogue<T, EPI_ALPHA_BETA, true>(g, Cp, acc, er, ec, kslice);
+      else if (g.epi == EPI_SPLITK_PARTIAL) fast_epilogue<T, EPI_SPLITK_PARTIAL, true>(g, Cp, acc, er, ec, kslice);
+      else fast_epilogue<T, EPI_CONV_FORWARD, true>(g, Cp, acc, er, ec, kslice);
     }
     return;
   }
@@ -634,7 +627,7 @@ __device__ __forceinline__ void gemm_workgroup(const GemmArgs &g_in, float *smem
         if (row >= g.M) continue;
         const float x = acc[a][b][v];
         if (g.epi == EPI_ALPHA_BETA) {
-          float *c = g.C + (size_t)row * g.ldc + col_off;
+          float *c = Cp + (size_t)row * g.ldc + col_off;
           float y = (g.beta == 0.0f) ? g.alpha * x : g.alpha * x + g.beta * (*c);
           if (g.col_bias) y += g.col_bias[col];
           if (g.relu && !(y > 0.0f)) y = 0.0f;
@@ -645,8 +638,8 @@ __device__ __forceinline__ void gemm_workgroup(const GemmArgs &g_in, float *smem
         } else {
           float y = g.bias ? x + g.bias[row] : x;
           if (g.relu && !(y > 0.0f)) y = 0.0f;
-          if (g.nt_store) __builtin_nontemporal_store(y, g.C + (size_t)row * g.fmap + col_off);
-          else g.C[(size_t)row * g.fmap + col_off] = y;
+          if (g.nt_store) __builtin_nontemporal_store(y, Cp + (size_t)row * g.fmap + col_off);
+          else Cp[(size_t)row * g.fmap + col_off] = y;
         }
       }
     }
