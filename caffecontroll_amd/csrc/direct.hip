@@ -1156,7 +1156,8 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
 
 
 // The same computation with the output size, the wavefront count and hence every trip count known
-// at compile time (the AlexNet/CaffeNet shapes): the whole step is one straight line of code, so
+// at compile time (the AlexNet/CaffeNet shapes, and 3 x 3 layers with 7-, 14- and 28-pixel outputs): the whole step
+// is one straight line of code, so
 // the loads of the next step are spread between the MFMAs of this one instead of forming a phase
 // of their own.  Differences from the generic kernel: each wavefront stages its own 32 rows of the
 // dout slab (private, padded to whole 64-word loads), and the prefetch is unconditional -- the
@@ -1562,7 +1563,7 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
   const int bsz = (nch * pch + 63) / 64 * 64;
   pl->stage = pl->a_floats + bsz;
   pl->spec = (ks == 5 && ho == 27 && pl->pw == 32 && pl->tb == 5 && (pl->waves == 4 || pl->waves == 8)) ||
-             (ks == 3 && ho == 13 && pl->pw == 16 && pl->tb == 6 &&
+             (ks == 3 && (ho == 13 || ho == 14 || ho == 7 || ho == 28) && pl->tb == 6 &&
               (pl->waves == 4 || pl->waves == 6 || pl->waves == 8));
   if (tuning().direct_nospec) pl->spec = false;  // tuning override
   pl->wn = 1;
@@ -1579,9 +1580,9 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
     const int nt = 64 * pl->waves * pl->wn;
     pl->a_floats = 0;
     pl->stage = (nch_spec * pch + nt - 1) / nt * nt;
-    // 13-pixel rows: few MFMAs per row fetched, and a lane fetching its own row touches a cache line per load --
-    // measured faster staged in LDS for every 3 x 3 instance, slower for the 5 x 5 one (27-pixel rows)
-    pl->alds = tuning().direct_alds == 1 || (tuning().direct_alds == 0 && ks == 3);
+    // short rows: few MFMAs per row fetched, and a lane fetching its own row touches a cache line per load --
+    // measured faster staged in LDS for the 3 x 3 instances on 7 to 14 pixel rows, slower on 27 and 28 pixel rows
+    pl->alds = tuning().direct_alds == 1 || (tuning().direct_alds == 0 && ks == 3 && ho <= 14);
     if (pl->alds) pl->stage += 2 * ((32 * pl->waves * ho + nt - 1) / nt * nt);
   }
   // fragment loads may run a few words past the last patch row: the padding of the patch region
@@ -1605,6 +1606,14 @@ template <int KS, int TB, int PW, int HO, int W, int WN = 1>
 static int wgrad_launch_spec(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
   return pl.alds ? wgrad_launch_spec_as<KS, TB, PW, HO, W, WN, true>(g, pl, st)
                  : wgrad_launch_spec_as<KS, TB, PW, HO, W, WN, false>(g, pl, st);
+}
+
+// the 3 x 3 instances of one output size: 8, 6 (as twelve wavefronts) or 4 row blocks
+template <int HO, int PW = 16>
+static int wgrad_launch_spec3(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
+  return pl.waves == 8   ? wgrad_launch_spec<3, 6, PW, HO, 8>(g, pl, st)
+         : pl.waves == 6 ? wgrad_launch_spec<3, 3, PW, HO, 6, 2>(g, pl, st)
+                         : wgrad_launch_spec<3, 6, PW, HO, 4>(g, pl, st);
 }
 
 template <int KS, int PW>
@@ -1636,7 +1645,8 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
     // Image pairs pay off on short rows (a step of the one-image kernel is half as many MFMAs deep) and where a
     // compile-time instance exists.  Measured at 3 x 3, pairs against rows: 7-14 pixel rows 65-91 against 53-81
     // TFLOP/s (129 against 70 with a compile-time instance), 16 pixels 61 against 78, 20-30 pixels 25-81 against
-    // 61-101 (the generic image-pair kernel wants 128 maps per workgroup).
+    // 61-101 (the generic image-pair kernel wants 128 maps per workgroup); compile-time instances at 28 pixels
+    // 105-136 against 97-113, at 14 pixels 111-134 against 77-82, at 7 pixels 99-118 against 50-56.
     const bool rows = tuning().direct_wgrad_rows == 2 || (!pl.spec && n + 2 * pad > 17);
     if (rows && conv_strided_wgrad_covers(batch, d * groups, n, ks, 1, pad, o * groups) &&
         conv_strided_wgrad_covers(batch, d, n, ks, 1, pad, o))
@@ -1712,9 +1722,10 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   if (pl.spec && ks == 5)
     rc = pl.waves == 8 ? wgrad_launch_spec<5, 5, 32, 27, 8>(g, pl, st) : wgrad_launch_spec<5, 5, 32, 27, 4>(g, pl, st);
   else if (pl.spec)
-    rc = pl.waves == 8   ? wgrad_launch_spec<3, 6, 16, 13, 8>(g, pl, st)
-         : pl.waves == 6 ? wgrad_launch_spec<3, 3, 16, 13, 6, 2>(g, pl, st)
-                         : wgrad_launch_spec<3, 6, 16, 13, 4>(g, pl, st);
+    rc = g.ho == 13 ? wgrad_launch_spec3<13>(g, pl, st)
+         : g.ho == 14 ? wgrad_launch_spec3<14>(g, pl, st)
+         : g.ho == 28 ? wgrad_launch_spec3<28, 32>(g, pl, st)
+                      : wgrad_launch_spec3<7>(g, pl, st);
   else if (ks == 5) rc = pl.pw == 16 ? wgrad_launch<5, 16>(g, pl, st) : wgrad_launch<5, 32>(g, pl, st);
   else rc = pl.pw == 16 ? wgrad_launch<3, 16>(g, pl, st) : wgrad_launch<3, 32>(g, pl, st);
   if (rc) return rc;

@@ -43,6 +43,10 @@ SHAPES = [
     (2, 3, 33, 7, 0, 40),
     (2, 4, 9, 7, 6, 33),      # full padding
     (1, 3, 80, 7, 3, 70),     # 7 x 7 in column bands, two map blocks
+    (3, 20, 14, 3, 1, 40),    # 14-, 7- and 28-pixel outputs of 3 x 3 layers: compile-time weight-gradient instances
+    (3, 21, 7, 3, 1, 192),    # (four, twelve and eight wavefronts; an odd batch: the last step holds one image)
+    (2, 64, 28, 3, 1, 250),
+    (5, 64, 16, 3, 0, 33),    # 14-pixel outputs without padding
 ]
 
 
@@ -465,7 +469,9 @@ FULL_SIZE = [(256, 96, 27, 5, 2, 256), (256, 48, 27, 5, 2, 128), (256, 256, 13, 
              (256, 192, 13, 3, 1, 192), (255, 192, 13, 3, 1, 128),
              # beyond CaffeNet: a VGG-sized 3 x 3 layer (four column bands, weight-gradient rows in four pieces), a
              # 112-wide one with an odd batch, a 7 x 7 stride-1 layer
-             (32, 64, 224, 3, 1, 64), (17, 128, 112, 3, 1, 128), (32, 64, 56, 7, 3, 64)]
+             (32, 64, 224, 3, 1, 64), (17, 128, 112, 3, 1, 128), (32, 64, 56, 7, 3, 64),
+             # 3 x 3 layers on 28-, 14- and 7-pixel maps (weight gradients by compile-time instances of their own)
+             (64, 128, 28, 3, 1, 256), (255, 256, 14, 3, 1, 256), (256, 512, 7, 3, 1, 512)]
 
 
 # the grouped layers of the CaffeNet iteration at batch 256, both groups in one launch: conv2, conv4, conv5
@@ -561,18 +567,22 @@ def test_full_size_direct_vs_float64(cfg):
     assert err(dw, dw_ref) <= TOL
 
 
-# every specialised weight-gradient instance (8, 4, 6 x 2 wavefronts; 5x5 on 27 rows, 3x3 on 13), with map counts
-# that leave rows of the last tile empty, an odd batch (the last step holds one image) and two groups
+# every specialised weight-gradient instance (8, 4, 6 x 2 wavefronts; 5x5 on 27 rows, 3x3 on 13, 14, 7 and 28), with
+# map counts that leave rows of the last tile empty, an odd batch (the last step holds one image) and two groups
 STAGED_ROWS = [(256, 96, 27, 5, 2, 256, 1), (64, 48, 27, 5, 2, 100, 1), (33, 48, 27, 5, 2, 128, 2),
                (256, 256, 13, 3, 1, 384, 1), (255, 192, 13, 3, 1, 192, 1), (64, 64, 13, 3, 1, 250, 1),
-               (63, 128, 13, 3, 1, 170, 2), (256, 192, 13, 3, 1, 192, 2)]
+               (63, 128, 13, 3, 1, 170, 2), (256, 192, 13, 3, 1, 192, 2),
+               (128, 128, 14, 3, 1, 256, 1), (65, 192, 14, 3, 1, 192, 1), (31, 64, 16, 3, 0, 100, 2),
+               (128, 128, 7, 3, 1, 250, 1), (64, 192, 7, 3, 1, 170, 2), (33, 64, 9, 3, 0, 128, 1),
+               (32, 64, 28, 3, 1, 256, 1), (17, 128, 28, 3, 1, 192, 1), (9, 64, 30, 3, 0, 100, 2)]
 
 
 @pytest.mark.parametrize("cfg", STAGED_ROWS, ids=lambda c: "b%d_d%d_n%d_k%d_p%d_o%d_g%d" % c)
 def test_wgrad_rows_staged_in_lds_equal_rows_fetched_by_lanes(cfg):
     """The shape-specialised weight-gradient kernels feed the MFMAs' output-gradient operand either from rows each
     lane fetched itself or from rows staged in LDS: the same values in the same order of additions, so weight and
-    bias gradients agree bit for bit."""
+    bias gradients agree bit for bit (with the count of step ranges pinned: the default follows the LDS a workgroup
+    takes, and another split of the steps is another order of additions)."""
     import torch
     b, d, n, k, p, o, groups = cfg
     m = n + 2 * p - k + 1
@@ -583,7 +593,7 @@ def test_wgrad_rows_staged_in_lds_equal_rows_fetched_by_lanes(cfg):
     got = {}
     for mode in (1, 2):
         dw, db = empty((o * groups, d, k, k), fill=float("nan")), empty((o * groups,), fill=float("nan"))
-        with tuning("direct_alds", mode):
+        with tuning("direct_alds", mode), tuning("direct_splits", 5):
             drv.conv_direct_backward_weights(dw, og, x, b, d * groups, n, k, p, o * groups, db=db, groups=groups)
             names = drv.lib.cct_hip_last_kernel().decode()
         torch.cuda.synchronize()
