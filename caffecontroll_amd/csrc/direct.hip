@@ -1156,7 +1156,8 @@ __global__ __launch_bounds__(512) void conv_direct_wgrad_kernel(const WgradArgs 
 
 
 // The same computation with the output size, the wavefront count and hence every trip count known
-// at compile time (the AlexNet/CaffeNet shapes, and 3 x 3 layers with 7-, 14- and 28-pixel outputs): the whole step
+// at compile time (the AlexNet/CaffeNet shapes; 3 x 3 layers with 7-, 14- and 28-pixel outputs, 5 x 5 layers with
+// 14- and 28-pixel outputs): the whole step
 // is one straight line of code, so
 // the loads of the next step are spread between the MFMAs of this one instead of forming a phase
 // of their own.  Differences from the generic kernel: each wavefront stages its own 32 rows of the
@@ -1562,7 +1563,8 @@ static bool wgrad_plan(int batch, int d, int n, int ks, int pad, int o, WgradPla
   const int nch = (32 * pl->tb - 1) / (ks * ks) + 2;
   const int bsz = (nch * pch + 63) / 64 * 64;
   pl->stage = pl->a_floats + bsz;
-  pl->spec = (ks == 5 && ho == 27 && pl->pw == 32 && pl->tb == 5 && (pl->waves == 4 || pl->waves == 8)) ||
+  pl->spec = (ks == 5 && (ho == 27 || ho == 28 || ho == 14) && pl->pw == 32 && pl->tb == 5 &&
+              (pl->waves == 4 || pl->waves == 8)) ||
              (ks == 3 && (ho == 13 || ho == 14 || ho == 7 || ho == 28) && pl->tb == 6 &&
               (pl->waves == 4 || pl->waves == 6 || pl->waves == 8));
   if (tuning().direct_nospec) pl->spec = false;  // tuning override
@@ -1608,6 +1610,12 @@ static int wgrad_launch_spec(const WgradArgs &g, const WgradPlan &pl, hipStream_
                  : wgrad_launch_spec_as<KS, TB, PW, HO, W, WN, false>(g, pl, st);
 }
 
+// the 5 x 5 instances of one output size: 8 or 4 row blocks
+template <int HO>
+static int wgrad_launch_spec5(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
+  return pl.waves == 8 ? wgrad_launch_spec<5, 5, 32, HO, 8>(g, pl, st) : wgrad_launch_spec<5, 5, 32, HO, 4>(g, pl, st);
+}
+
 // the 3 x 3 instances of one output size: 8, 6 (as twelve wavefronts) or 4 row blocks
 template <int HO, int PW = 16>
 static int wgrad_launch_spec3(const WgradArgs &g, const WgradPlan &pl, hipStream_t st) {
@@ -1647,7 +1655,12 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
     // TFLOP/s (129 against 70 with a compile-time instance), 16 pixels 61 against 78, 20-30 pixels 25-81 against
     // 61-101 (the generic image-pair kernel wants 128 maps per workgroup); compile-time instances at 28 pixels
     // 105-136 against 97-113, at 14 pixels 111-134 against 77-82, at 7 pixels 99-118 against 50-56.
-    const bool rows = tuning().direct_wgrad_rows == 2 || (!pl.spec && n + 2 * pad > 17);
+    // At 5 x 5 a step holds 25 MFMAs per column block instead of 9 and pairs stay ahead for longer: 14-pixel
+    // outputs 65-88 against 56-67, 16-20 pixels 72-86 against 68-82, 24-28 pixels 39-80 against 67-95 -- except
+    // with 256 maps (eight wavefronts, 107 against 95); compile-time instances 96-125 at 14 pixels and 81-144 at 28.
+    const int longest_pair_row = ks == 5 ? 24 : 17;
+    const bool rows = tuning().direct_wgrad_rows == 2 ||
+                      (!pl.spec && n + 2 * pad > longest_pair_row && !(ks == 5 && o >= 256));
     if (rows && conv_strided_wgrad_covers(batch, d * groups, n, ks, 1, pad, o * groups) &&
         conv_strided_wgrad_covers(batch, d, n, ks, 1, pad, o))
       pairs = false;
@@ -1720,7 +1733,9 @@ static int conv_direct_wgrad(float *dw, float *db, const float *dout, const floa
   hipStream_t st = ctx().stream;
   int rc;
   if (pl.spec && ks == 5)
-    rc = pl.waves == 8 ? wgrad_launch_spec<5, 5, 32, 27, 8>(g, pl, st) : wgrad_launch_spec<5, 5, 32, 27, 4>(g, pl, st);
+    rc = g.ho == 27 ? wgrad_launch_spec5<27>(g, pl, st)
+         : g.ho == 28 ? wgrad_launch_spec5<28>(g, pl, st)
+                      : wgrad_launch_spec5<14>(g, pl, st);
   else if (pl.spec)
     rc = g.ho == 13 ? wgrad_launch_spec3<13>(g, pl, st)
          : g.ho == 14 ? wgrad_launch_spec3<14>(g, pl, st)

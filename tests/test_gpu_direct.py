@@ -47,6 +47,12 @@ SHAPES = [
     (3, 21, 7, 3, 1, 192),    # (four, twelve and eight wavefronts; an odd batch: the last step holds one image)
     (2, 64, 28, 3, 1, 250),
     (5, 64, 16, 3, 0, 33),    # 14-pixel outputs without padding
+    (3, 16, 28, 5, 2, 40),    # 5 x 5 with 28- and 14-pixel outputs: compile-time weight-gradient instances
+    (3, 32, 14, 5, 2, 250),
+    (3, 12, 14, 5, 2, 40),    # 5 x 5 on padded rows of 18 and 24 floats: image-pair weight-gradient kernel
+    (2, 7, 20, 5, 2, 130),
+    (2, 6, 22, 5, 2, 260),    # 26 floats: image pairs with 256 maps or more, one image per step below
+    (2, 6, 22, 5, 2, 70),
 ]
 
 
@@ -471,7 +477,9 @@ FULL_SIZE = [(256, 96, 27, 5, 2, 256), (256, 48, 27, 5, 2, 128), (256, 256, 13, 
              # 112-wide one with an odd batch, a 7 x 7 stride-1 layer
              (32, 64, 224, 3, 1, 64), (17, 128, 112, 3, 1, 128), (32, 64, 56, 7, 3, 64),
              # 3 x 3 layers on 28-, 14- and 7-pixel maps (weight gradients by compile-time instances of their own)
-             (64, 128, 28, 3, 1, 256), (255, 256, 14, 3, 1, 256), (256, 512, 7, 3, 1, 512)]
+             (64, 128, 28, 3, 1, 256), (255, 256, 14, 3, 1, 256), (256, 512, 7, 3, 1, 512),
+             # 5 x 5 layers on 28- and 14-pixel maps (likewise)
+             (128, 96, 28, 5, 2, 256), (127, 128, 14, 5, 2, 256)]
 
 
 # the grouped layers of the CaffeNet iteration at batch 256, both groups in one launch: conv2, conv4, conv5
@@ -567,14 +575,17 @@ def test_full_size_direct_vs_float64(cfg):
     assert err(dw, dw_ref) <= TOL
 
 
-# every specialised weight-gradient instance (8, 4, 6 x 2 wavefronts; 5x5 on 27 rows, 3x3 on 13, 14, 7 and 28), with
+# every specialised weight-gradient instance (8, 4, 6 x 2 wavefronts; 5x5 on 27, 28 and 14 rows, 3x3 on 13, 14, 7 and
+# 28), with
 # map counts that leave rows of the last tile empty, an odd batch (the last step holds one image) and two groups
 STAGED_ROWS = [(256, 96, 27, 5, 2, 256, 1), (64, 48, 27, 5, 2, 100, 1), (33, 48, 27, 5, 2, 128, 2),
                (256, 256, 13, 3, 1, 384, 1), (255, 192, 13, 3, 1, 192, 1), (64, 64, 13, 3, 1, 250, 1),
                (63, 128, 13, 3, 1, 170, 2), (256, 192, 13, 3, 1, 192, 2),
                (128, 128, 14, 3, 1, 256, 1), (65, 192, 14, 3, 1, 192, 1), (31, 64, 16, 3, 0, 100, 2),
                (128, 128, 7, 3, 1, 250, 1), (64, 192, 7, 3, 1, 170, 2), (33, 64, 9, 3, 0, 128, 1),
-               (32, 64, 28, 3, 1, 256, 1), (17, 128, 28, 3, 1, 192, 1), (9, 64, 30, 3, 0, 100, 2)]
+               (32, 64, 28, 3, 1, 256, 1), (17, 128, 28, 3, 1, 192, 1), (9, 64, 30, 3, 0, 100, 2),
+               (64, 32, 28, 5, 2, 100, 1), (33, 64, 28, 5, 2, 256, 1), (65, 32, 14, 5, 2, 128, 2),
+               (32, 64, 18, 5, 0, 250, 1)]
 
 
 @pytest.mark.parametrize("cfg", STAGED_ROWS, ids=lambda c: "b%d_d%d_n%d_k%d_p%d_o%d_g%d" % c)
