@@ -1034,7 +1034,7 @@ extern "C" int cct_hip_conv1x1_backward_weights(float *model_grad, float *bias_g
                                                 const float *input, int batch, int depth, int plane,
                                                 int num_outputs) {
   CCT_ENSURE_INIT();
-  CCT_REQUIRE(batch >= 0 && (batch == 0 || conv1x1_dims_ok(batch, depth, plane, num_outputs)),
+  CCT_REQUIRE(batch >= 0 && conv1x1_dims_ok(batch > 0 ? batch : 1, depth, plane, num_outputs),
               "conv1x1_backward_weights: bad dimensions");
   CCT_REQUIRE(model_grad && (batch == 0 || (output_grad && input)), "conv1x1_backward_weights: null argument");
   if (batch == 0) {

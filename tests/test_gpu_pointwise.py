@@ -135,6 +135,8 @@ def test_pointwise_support_and_errors():
     drv.conv1x1_forward(empty((4,)), empty((4,)), empty((6,)), None, 0, 2, 4, 3)
     drv.conv1x1_backward_weights(dw, empty((4,)), empty((4,)), 0, 2, 4, 3, db=db)
     assert not host(dw).any() and not host(db).any()
+    with pytest.raises(CctHipError):   # an empty batch does not excuse a bad layer shape
+        drv.conv1x1_backward_weights(dw, empty((4,)), empty((4,)), 0, -2, 4, 3)
 
 
 @pytest.mark.parametrize("shape", [(4, 64, 13, 96), (3, 16, 8, 32), (9, 20, 30, 7)], ids=_ids)
