@@ -35,9 +35,12 @@ CONFIGS = {
     "vgg_conv1_2": (32, 64, 224, 3, 1, 1, 64),
     "conv7x7_56": (32, 64, 56, 7, 1, 3, 64),
     "pointwise_28": (64, 256, 28, 1, 1, 0, 256),
+    # 3 x 3 on 14 x 14 maps and 5 x 5 on 28 x 28 maps: output sizes the weight gradient has compile-time instances for
+    "conv3x3_14": (256, 256, 14, 3, 1, 1, 256),
+    "conv5x5_28": (128, 96, 28, 5, 1, 2, 256),
 }
 SEEDS = {"alexnet_conv1": 1234, "alexnet_conv2": 1235, "lenet_conv1": 1236, "vgg_conv1_2": 1237, "conv7x7_56": 1238,
-         "pointwise_28": 1239}
+         "pointwise_28": 1239, "conv3x3_14": 1240, "conv5x5_28": 1241}
 PEAK_FP32_MFMA_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
 # HBM bytes per launch (fetched + written) come from the committed counter summaries under profiles/
@@ -52,6 +55,8 @@ TRAFFIC_SOURCE = {("alexnet_conv2", "direct"): "profiles/conv2_fwd_bwd_hbm_traff
                   ("vgg_conv1_2", "direct"): "profiles/wide_3x3_layer_trace_traffic_mfma.md",
                   ("conv7x7_56", "direct"): "profiles/conv7x7_stride1_layer_trace_traffic_mfma.md",
                   ("pointwise_28", "direct"): "profiles/pointwise_layer_trace_traffic_mfma.md",
+                  ("conv3x3_14", "direct"): "profiles/conv3x3_on_14x14_layer_trace_traffic_mfma.md",
+                  ("conv5x5_28", "direct"): "profiles/conv5x5_on_28x28_layer_trace_traffic_mfma.md",
                   ("caffenet", "direct"): "profiles/caffenet_iteration_kernel_trace.md",
                   ("lenet", "direct"): "profiles/lenet_iteration_kernel_trace.md"}
 # which launches of a kernel a stage means, where a summary lists one kernel's launches by role
