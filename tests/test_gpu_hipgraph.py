@@ -90,10 +90,12 @@ def test_lowering_path_in_a_graph():
     _check_replays(graph, outputs, eager_work)
 
 
-@pytest.mark.parametrize("shape", [(16, 16, 13, 3, 1, 32), (8, 8, 27, 5, 2, 48)])
+@pytest.mark.parametrize("shape", [(16, 16, 13, 3, 1, 32), (8, 8, 27, 5, 2, 48), (16, 64, 14, 3, 1, 128),
+                                   (6, 32, 28, 5, 2, 64), (4, 4, 100, 3, 1, 8), (4, 8, 20, 7, 3, 16)])
 def test_direct_kernels_in_a_graph(shape):
     """Weight re-layout, forward (bias and ReLU in the epilogue), data gradient and weight gradient (partial
-    sums over step ranges in the workspace, fixed-order reduction) of the direct path."""
+    sums over step ranges in the workspace, fixed-order reduction) of the direct path: the generic kernels, two
+    compile-time weight-gradient instances, an image in column bands, a 7 x 7 layer."""
     drv = driver()
     b, d, n, k, p, o = shape
     if not drv.conv_direct_supported(b, d, n, k, 1, p, o):
@@ -120,6 +122,33 @@ def test_direct_kernels_in_a_graph(shape):
 
     def eager_work():
         drv.conv_direct_backward_weights(empty((o, d, k, k)), og, x, b, d, n, k, p, o, db=empty((o,)))
+
+    _check_replays(graph, [out, dx, dw, db], eager_work)
+
+
+@pytest.mark.parametrize("shape", [(8, 32, 13, 48), (5, 64, 8, 64)])
+def test_pointwise_products_in_a_graph(shape):
+    """1 x 1 layers: one product per image forward and for the data gradient, one product summed over the images
+    (partial sums in the workspace, fixed-order reduction) plus the bias gradient for the weights."""
+    drv = driver()
+    b, d, n, o = shape
+    rng = np.random.default_rng(74)
+    x = dev(rng.standard_normal((b, d, n, n)).astype(np.float32))
+    w = dev((rng.standard_normal((o, d)) * 0.1).astype(np.float32))
+    bias = dev(rng.standard_normal(o).astype(np.float32))
+    og = dev(rng.standard_normal((b, o, n, n)).astype(np.float32))
+    out, dx, dw, db = empty((b, o, n, n)), empty((b, d, n, n)), empty((o, d)), empty((o,))
+
+    def seq():
+        drv.conv1x1_forward(out, x, w, bias, b, d, n * n, o, relu=True)
+        drv.conv1x1_backward_data(dx, og, w, b, d, n * n, o)
+        drv.conv1x1_backward_weights(dw, og, x, b, d, n * n, o, db=db)
+
+    seq()
+    graph = _record(seq)
+
+    def eager_work():
+        drv.conv1x1_backward_weights(empty((o, d)), og, x, b, d, n * n, o, db=empty((o,)))
 
     _check_replays(graph, [out, dx, dw, db], eager_work)
 
