@@ -32,6 +32,7 @@ static void read_tuning_from_env() {
   g_tuning.direct_splits = geti("CCT_HIP_DIRECT_SPLITS", 0);
   g_tuning.direct_alds = geti("CCT_HIP_DIRECT_ALDS", 0);
   g_tuning.direct_wgrad_rows = geti("CCT_HIP_DIRECT_WGRAD_ROWS", 0);
+  g_tuning.conv1x1_per_image = geti("CCT_HIP_CONV1X1_PER_IMAGE", 0);
   g_tuning.strided_wgrad = geti("CCT_HIP_STRIDED_WGRAD", 0);
   g_tuning.pool_plane = geti("CCT_HIP_POOL_PLANE", 0);
   g_tuning.gemm_nt = geti("CCT_HIP_GEMM_NT", 0);
@@ -168,7 +169,7 @@ int cct_hip_set_tuning(const char *name, int value) {
   struct { const char *name; int *field; } const table[] = {
       {"direct_tile", &t.direct_tile}, {"direct_waves", &t.direct_waves}, {"direct_tb", &t.direct_tb},
       {"direct_nospec", &t.direct_nospec}, {"direct_splits", &t.direct_splits}, {"direct_alds", &t.direct_alds},
-      {"direct_wgrad_rows", &t.direct_wgrad_rows}, {"strided_wgrad", &t.strided_wgrad}, {"pool_plane", &t.pool_plane}, {"gemm_nt", &t.gemm_nt},
+      {"direct_wgrad_rows", &t.direct_wgrad_rows}, {"conv1x1_per_image", &t.conv1x1_per_image}, {"strided_wgrad", &t.strided_wgrad}, {"pool_plane", &t.pool_plane}, {"gemm_nt", &t.gemm_nt},
       {"gemm_tile", &t.gemm_tile}, {"gemm_nodma", &t.gemm_nodma}};
   for (const auto &e : table)
     if (!strcmp(e.name, name)) {

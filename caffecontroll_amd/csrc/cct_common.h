@@ -36,6 +36,7 @@ struct Tuning {
   int direct_nospec = 0;  // 1: never take the shape-specialised weight-gradient instances
   int direct_splits = 0;  // step ranges of the weight-gradient launch (its partial sums), 0 = model's choice
   int direct_alds = 0;    // specialised weight-gradient instances: 1 = dout rows through LDS, 2 = never, 0 = model's choice
+  int conv1x1_per_image = 0;  // 1 x 1 layers, forward and data gradient: 1 = one product per image, 2 = one product over the pixels of all images, 0 = by plane size
   int direct_wgrad_rows = 0;  // stride-1 weight gradient: 1 = image-pair kernels wherever they apply, 2 = one image per step always, 0 = model's choice
   int strided_wgrad = 0;  // strided weight-gradient tile: row pieces * 1000 + column blocks * 100 + column groups * 10 + row blocks, 0 = model's choice
   int pool_plane = 0;     // 1: plane-tiled pooling kernels at any size

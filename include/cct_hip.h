@@ -108,7 +108,8 @@ int cct_hip_set_stream(void *hip_stream);
  * their lanes, 0 = automatic), "direct_wgrad_rows" (stride-1 weight gradient: 1 = the image-pair kernels wherever they
  * apply, 2 = the one-image-per-step kernel always, 0 = automatic), "strided_wgrad" (tile of the strided weight-gradient kernel: pieces of an output row
  * x 1000 + column blocks x 100 + column groups x 10 + row blocks, 0 = automatic), "pool_plane", "gemm_nt", "gemm_tile" (-1 = automatic), "gemm_nodma" (1 = GEMM
- * operand tiles always staged through registers).  The
+ * operand tiles always staged through registers), "conv1x1_per_image" (1 x 1 layers, forward and data gradient: 1 = one
+ * product per image, 2 = one product over the pixels of all images, 0 = automatic).  The
  * environment variables CCT_HIP_<NAME IN CAPITALS> give the initial values; they are read once,
  * when the library initialises, never on a launch path.  No counterpart in the reference. */
 int cct_hip_set_tuning(const char *name, int value);
@@ -257,8 +258,9 @@ int cct_hip_conv_small_backward_weights(float *dw, float *db, const float *dout,
  * [batch][depth][plane] (plane = n*n) is already the depth x plane operand of its product.  These three replace
  * lower_cube + GEMM + remap_output + bias of ConvolutionBridge::forward (src/bridges/ConvolutionBridge_impl.hxx:294-373)
  * and remap + the two GEMMs + inverse_lower_cube + bias gradient of ::backward (:551-628) with products on the
- * tensors as they lie: forward and data gradient one product per image (all images in one launch), the weight
- * gradient one product summed over the images in a fixed order.  model [num_outputs][depth]; bias / bias_grad may
+ * tensors as they lie: forward and data gradient one product whose columns run over the pixels of all images (one
+ * product per image, all in one launch, for planes above 2048 pixels or below 4), the weight gradient one product
+ * summed over the images in a fixed order.  model [num_outputs][depth]; bias / bias_grad may
  * be NULL; relu != 0 clamps the output at zero.  Results agree with the lowering path to fp32 rounding.
  * cct_hip_conv1x1_supported: 1 for k == 1, stride == 1, padding == 0 (else 0: the lowering path takes the layer). */
 int cct_hip_conv1x1_supported(int batch, int depth, int n, int k, int stride, int padding, int num_outputs);

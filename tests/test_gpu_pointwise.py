@@ -5,7 +5,7 @@ src/bridges/ConvolutionBridge_impl.hxx:294-373, 551-628), through the C ABI and 
 import numpy as np
 import pytest
 
-from gpu_util import driver, dev, empty, host, rel_err
+from gpu_util import driver, dev, empty, host, rel_err, tuning
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-4
@@ -32,6 +32,25 @@ def _tensors(shape, seed):
     bias = rng.standard_normal(o).astype(np.float32)
     og = rng.standard_normal((b, o, n, n)).astype(np.float32)
     return x, w, bias, og
+
+
+@pytest.mark.parametrize("per_image", [1, 2], ids=["per_image", "across_images"])
+@pytest.mark.parametrize("shape", SHAPES + [(3, 5, 1, 7), (9, 16, 2, 32)], ids=_ids)
+def test_forward_and_data_gradient_in_both_forms(oracle, shape, per_image):
+    """Forward and data gradient as one product per image and as one product whose columns run over the pixels of
+    all images (planes that are not a multiple of four floats: vectors that straddle two images; planes shorter than
+    a vector keep one product per image whatever the knob says)."""
+    b, d, n, o = shape
+    x, w, bias, og = _tensors(shape, 7 + sum(shape))
+    drv = driver()
+    ref_out, lowered = oracle.conv_forward(x, w, bias, 1, 1, 0)
+    ref_dx, _, _ = oracle.conv_backward(x.shape, w, og, lowered, 1, 1, 0)
+    out, dx = empty((b, o, n, n), fill=float("nan")), empty((b, d, n, n), fill=float("nan"))
+    with tuning("conv1x1_per_image", per_image):
+        drv.conv1x1_forward(out, dev(x), dev(w), dev(bias), b, d, n * n, o)
+        drv.conv1x1_backward_data(dx, dev(og), dev(w), b, d, n * n, o)
+    assert rel_err(host(out), ref_out) <= TOL
+    assert rel_err(host(dx), ref_dx) <= TOL
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=_ids)
