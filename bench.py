@@ -52,6 +52,7 @@ PEAK_HBM_GBS = 8000.0
 TRAFFIC_SOURCE = {("alexnet_conv2", "direct"): "profiles/conv2_fwd_bwd_hbm_traffic_and_mfma.md",
                   ("alexnet_conv2", "lowering"): "profiles/conv2_lowering_path_hbm_traffic_and_mfma.md",
                   ("alexnet_conv1", "direct"): "profiles/conv1_fwd_bwd_trace_traffic_mfma.md",
+                  ("lenet_conv1", "direct"): "profiles/lenet_conv1_layer_trace_traffic.md",
                   ("vgg_conv1_2", "direct"): "profiles/wide_3x3_layer_trace_traffic_mfma.md",
                   ("conv7x7_56", "direct"): "profiles/conv7x7_stride1_layer_trace_traffic_mfma.md",
                   ("pointwise_28", "direct"): "profiles/pointwise_layer_trace_traffic_mfma.md",
